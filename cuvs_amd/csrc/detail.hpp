@@ -1,0 +1,243 @@
+/*
+ * Internal declarations shared by the host driver and the HIP kernels of the IVF-PQ search path.
+ */
+#pragma once
+
+#include <cuvs/core/resources.hpp>
+#include <cuvs/neighbors/ivf_pq.hpp>
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+namespace cuvs {
+
+[[noreturn]] inline void fail(const char* fmt, ...)
+{
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  throw logic_error(buf);
+}
+
+#define CUVS_EXPECTS(cond, ...) \
+  do {                          \
+    if (!(cond)) { ::cuvs::fail(__VA_ARGS__); } \
+  } while (0)
+
+#define CUVS_HIP_TRY(call)                                                                  \
+  do {                                                                                      \
+    hipError_t status_ = (call);                                                            \
+    if (status_ != hipSuccess) {                                                            \
+      ::cuvs::fail("HIP error at %s:%d: %s (%s)", __FILE__, __LINE__, hipGetErrorName(status_), \
+                   hipGetErrorString(status_));                                             \
+    }                                                                                       \
+  } while (0)
+
+/** Owning device allocation. */
+struct device_buffer {
+  void* ptr    = nullptr;
+  size_t bytes = 0;
+  device_buffer() = default;
+  explicit device_buffer(size_t n) { allocate(n); }
+  ~device_buffer() { release(); }
+  device_buffer(const device_buffer&)            = delete;
+  device_buffer& operator=(const device_buffer&) = delete;
+  device_buffer(device_buffer&& o) noexcept : ptr(o.ptr), bytes(o.bytes)
+  {
+    o.ptr   = nullptr;
+    o.bytes = 0;
+  }
+  device_buffer& operator=(device_buffer&& o) noexcept
+  {
+    if (this != &o) {
+      release();
+      ptr     = o.ptr;
+      bytes   = o.bytes;
+      o.ptr   = nullptr;
+      o.bytes = 0;
+    }
+    return *this;
+  }
+  void allocate(size_t n)
+  {
+    release();
+    if (n > 0) {
+      CUVS_HIP_TRY(hipMalloc(&ptr, n));
+      bytes = n;
+    }
+  }
+  void release()
+  {
+    if (ptr != nullptr) { (void)hipFree(ptr); }
+    ptr   = nullptr;
+    bytes = 0;
+  }
+  template <typename T>
+  T* as() const
+  {
+    return static_cast<T*>(ptr);
+  }
+};
+
+inline uint32_t round_up_u32(uint32_t v, uint32_t m) { return ((v + m - 1) / m) * m; }
+inline uint64_t round_up_u64(uint64_t v, uint64_t m) { return ((v + m - 1) / m) * m; }
+inline uint32_t next_pow2(uint32_t v)
+{
+  uint32_t p = 1;
+  while (p < v) { p <<= 1; }
+  return p;
+}
+
+}  // namespace cuvs
+
+namespace cuvs::neighbors::ivf_pq::detail {
+
+using cuvs::distance::DistanceType;
+
+/** Index contents.  Lists live in two arenas (codes, ids); list `l` starts at row `row_offset[l]`
+ *  (a multiple of 32) and owns round_up(size, 32) rows. */
+struct index_impl {
+  DistanceType metric        = DistanceType::L2Expanded;
+  codebook_gen codebook_kind = codebook_gen::PER_SUBSPACE;
+  bool conservative_memory_allocation = false;
+  uint32_t n_lists = 0, dim = 0, pq_bits = 0, pq_dim = 0;
+  uint32_t dim_ext = 0, pq_len = 0, rot_dim = 0, book_size = 0;
+  uint32_t n_chunks = 0;  // 16-byte chunks per encoded row
+
+  device_buffer centers, centers_rot, rotation, rotation_t, pq_centers;
+  bool rotation_is_identity = false;
+
+  device_buffer codes_arena, ids_arena;
+  std::vector<uint32_t> h_list_sizes;
+  std::vector<uint64_t> h_row_offsets;  // [n_lists + 1], in rows, multiples of 32
+  device_buffer list_sizes, data_ptrs, inds_ptrs;
+  std::vector<int64_t> accum_sorted_sizes;  // [n_lists + 1]
+  int64_t size = 0;
+
+  uint64_t group_bytes() const { return uint64_t(n_chunks) * kIndexGroupSize * kIndexGroupVecLen; }
+  /** Recompute pointer tables, device sizes and the sorted prefix sums from the host vectors
+   *  (role of ivf::detail::recompute_internal_state, cpp/src/neighbors/ivf_common.cuh:255-290). */
+  void recompute_internal_state(hipStream_t stream);
+};
+
+void init_index(index_impl& ix, const index_params& params, uint32_t dim);
+
+/* ------------------------------------------------------------------------------------------ */
+/* kernel launchers (kernels.hip)                                                              */
+/* ------------------------------------------------------------------------------------------ */
+
+void launch_fill_u32(uint32_t* dst, uint32_t value, uint64_t n, hipStream_t stream);
+
+/** qf[q, d] = mapping<float>(queries[q, d])  (detail/ann_utils.cuh:168-201) */
+void launch_map_queries(const void* queries, elem_type type, uint64_t n_elems, float* out,
+                        hipStream_t stream);
+
+/** scores[q, l] = alpha * (sum_d centers[l, d] * qf[q, d] + centers[l, dim] * qnorm), fp32 FMA in
+ *  ascending d.  half_inputs rounds both operands to binary16 first and the result to binary16. */
+void launch_coarse_scores(const float* qf, const float* centers, uint32_t n_queries,
+                          uint32_t n_lists, uint32_t dim, uint32_t dim_ext, bool ip_like,
+                          bool half_inputs, float* scores, hipStream_t stream);
+
+/** probes[q, 0..P) = lists with the P smallest (score, list id), ascending. */
+void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_lists,
+                          uint32_t n_probes, uint32_t* probes, hipStream_t stream);
+
+/** rot_q = rotation * qf (+ row normalisation for cosine); rotation_t is [dim, rot_dim]. */
+void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries, uint32_t dim,
+                   uint32_t rot_dim, bool identity, bool normalize, float* rot_q,
+                   hipStream_t stream);
+
+/** chunk_indices[q, p] = inclusive prefix sum of list_sizes[probes[q, p]]; n_samples[q] = total.
+ *  When `stats` is non-null, adds the scanned bytes and rows to stats[0], stats[1]. */
+void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
+                          uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
+                          uint32_t* n_samples, unsigned long long* stats, hipStream_t stream);
+
+/** pair_order = ids of the (query, probe) pairs grouped by probed list. `counters` is scratch of
+ *  2 * n_lists + 2 words. */
+void launch_order_pairs(const uint32_t* probes, uint32_t n_pairs, uint32_t n_lists,
+                        uint32_t* counters, uint32_t* pair_order, hipStream_t stream);
+
+struct scan_args {
+  uint32_t n_queries, n_probes, k, max_samples;
+  uint32_t rot_dim, pq_dim, pq_len, pq_bits;
+  int metric;          // DistanceType
+  int per_cluster;     // codebook kind
+  int lut_dtype;       // CUDA_R_32F / 16F / 8U
+  int out_half;        // internal distance dtype is fp16
+  int fused;           // per-pair top-k in the kernel
+  const float* rot_q;           // [n_queries, rot_dim]
+  const float* centers_rot;     // [n_lists, rot_dim]
+  const float* pq_centers;
+  const uint8_t* const* data_ptrs;
+  const int64_t* const* inds_ptrs;
+  const uint32_t* list_sizes;
+  const uint32_t* probes;         // [n_queries, n_probes]
+  const uint32_t* chunk_indices;  // [n_queries, n_probes]
+  const uint32_t* pair_order;     // [n_queries * n_probes] or null
+  const uint32_t* filter_bits;    // or null
+  int64_t filter_nbits;
+  uint32_t* query_kth;            // [n_queries] ordered-score upper bounds (fused)
+  unsigned long long* out_keys;   // fused: [n_queries, n_probes, k]
+  float* out_scores;              // non-fused: [n_queries, max_samples]
+};
+/** LDS bytes the scan kernel needs for these arguments. */
+size_t scan_lds_bytes(const scan_args& a);
+void launch_scan(const scan_args& a, hipStream_t stream);
+
+struct merge_args {
+  uint32_t n_queries, n_probes, k, max_samples;
+  int fused;
+  int metric;
+  float scaling;
+  const unsigned long long* in_keys;  // fused
+  const float* in_scores;             // non-fused
+  const uint32_t* n_samples;
+  const uint32_t* probes;
+  const uint32_t* chunk_indices;
+  const int64_t* const* inds_ptrs;
+  int64_t* neighbors;  // [n_queries, k]
+  float* distances;    // [n_queries, k]
+};
+void launch_merge(const merge_args& a, hipStream_t stream);
+
+/* list maintenance and encoding */
+void launch_normalize_rows(float* x, uint64_t n_rows, uint32_t dim, hipStream_t stream);
+void launch_histogram(const uint32_t* labels, uint64_t n, uint32_t* counts, hipStream_t stream);
+void launch_relocate_lists(const uint8_t* old_codes, const int64_t* old_ids, uint8_t* new_codes,
+                           int64_t* new_ids, const uint64_t* old_row_offsets,
+                           const uint64_t* new_row_offsets, const uint32_t* old_sizes,
+                           uint32_t n_lists, uint32_t n_chunks, hipStream_t stream);
+struct encode_args {
+  const float* xf;  // mapped rows [n, dim]
+  uint64_t n_rows;
+  uint32_t dim, dim_ext, rot_dim, pq_dim, pq_len, pq_bits, n_chunks;
+  int per_cluster;
+  const uint32_t* labels;
+  const float* centers;
+  const float* rotation_t;
+  int identity_rotation;
+  const float* pq_centers;
+  /* mode A: append into lists */
+  uint32_t* cursors;          // [n_lists] next free slot per list
+  uint8_t* const* data_ptrs;  // per-list code base
+  int64_t* const* inds_ptrs;  // per-list id base
+  const int64_t* ids;         // [n] or null
+  int64_t first_id;           // used when ids is null
+  /* mode B: bit-contiguous output rows */
+  uint8_t* flat_codes;  // [n, ceil(pq_dim * pq_bits / 8)] or null
+  float* scratch;       // [rot_dim, n] rotated residuals
+};
+void launch_encode(const encode_args& a, hipStream_t stream);
+
+void launch_unpack_contiguous(const uint8_t* list_data, uint32_t n_rows, uint32_t offset,
+                              uint32_t pq_dim, uint32_t pq_bits, uint8_t* out, hipStream_t stream);
+
+}  // namespace cuvs::neighbors::ivf_pq::detail

@@ -1,0 +1,201 @@
+/*
+ * IVF-PQ index object: derived dimensions, model storage, list arenas and the dependent state
+ * (pointer tables, sorted size prefix sums).  Contents and derived quantities follow cuVS
+ * cpp/src/neighbors/ivf_pq_index.cu:78-111,223-235,599-622 and
+ * cpp/include/cuvs/neighbors/ivf_pq.hpp:222-296.
+ */
+#include "detail.hpp"
+
+#include <algorithm>
+#include <functional>
+
+namespace cuvs::neighbors::ivf_pq {
+
+namespace detail {
+
+void init_index(index_impl& ix, const index_params& params, uint32_t dim)
+{
+  CUVS_EXPECTS(params.pq_bits >= 4 && params.pq_bits <= 8,
+               "pq_bits must be within [4, 8], got %u", params.pq_bits);
+  CUVS_EXPECTS(dim > 0, "dim must be positive");
+  CUVS_EXPECTS(params.n_lists > 0, "n_lists must be positive");
+  uint32_t pq_dim = params.pq_dim;
+  if (pq_dim == 0) {
+    // calculate_pq_dim (ivf_pq_index.cu:612-622): half the dimension from 128 up, rounded down
+    // to a multiple of 32, or to a power of two below 32
+    uint32_t d = dim >= 128 ? dim / 2 : dim;
+    pq_dim     = (d / 32) * 32;
+    if (pq_dim == 0) {
+      pq_dim = 1;
+      while ((pq_dim << 1) <= d) { pq_dim <<= 1; }
+    }
+  }
+  CUVS_EXPECTS((params.pq_bits * pq_dim) % 8 == 0,
+               "pq_bits * pq_dim must be a multiple of 8 (pq_bits = %u, pq_dim = %u)",
+               params.pq_bits, pq_dim);
+  switch (params.metric) {
+    case DistanceType::L2Expanded:
+    case DistanceType::L2SqrtExpanded:
+    case DistanceType::InnerProduct:
+    case DistanceType::CosineExpanded: break;
+    default: fail("Unsupported distance type %d.", int(params.metric));
+  }
+  ix.metric                         = params.metric;
+  ix.codebook_kind                  = params.codebook_kind;
+  ix.conservative_memory_allocation = params.conservative_memory_allocation;
+  ix.n_lists                        = params.n_lists;
+  ix.dim                            = dim;
+  ix.pq_bits                        = params.pq_bits;
+  ix.pq_dim                         = pq_dim;
+  ix.dim_ext                        = round_up_u32(dim + 1, 8);
+  ix.pq_len                         = (dim + pq_dim - 1) / pq_dim;
+  ix.rot_dim                        = ix.pq_len * pq_dim;
+  ix.book_size                      = 1u << params.pq_bits;
+  const uint32_t cpc                = (kIndexGroupVecLen * 8u) / params.pq_bits;
+  ix.n_chunks                       = (pq_dim + cpc - 1) / cpc;
+  ix.h_list_sizes.assign(ix.n_lists, 0);
+  ix.h_row_offsets.assign(ix.n_lists + 1, 0);
+  ix.accum_sorted_sizes.assign(ix.n_lists + 1, 0);
+  ix.list_sizes.allocate(sizeof(uint32_t) * ix.n_lists);
+  ix.data_ptrs.allocate(sizeof(void*) * ix.n_lists);
+  ix.inds_ptrs.allocate(sizeof(void*) * ix.n_lists);
+  ix.size = 0;
+}
+
+void index_impl::recompute_internal_state(hipStream_t stream)
+{
+  std::vector<uint8_t*> dptr(n_lists);
+  std::vector<int64_t*> iptr(n_lists);
+  const uint64_t gb = group_bytes();
+  for (uint32_t l = 0; l < n_lists; l++) {
+    dptr[l] = codes_arena.as<uint8_t>() + (h_row_offsets[l] / kIndexGroupSize) * gb;
+    iptr[l] = ids_arena.as<int64_t>() + h_row_offsets[l];
+  }
+  CUVS_HIP_TRY(hipMemcpyAsync(data_ptrs.ptr, dptr.data(), sizeof(void*) * n_lists,
+                              hipMemcpyHostToDevice, stream));
+  CUVS_HIP_TRY(hipMemcpyAsync(inds_ptrs.ptr, iptr.data(), sizeof(void*) * n_lists,
+                              hipMemcpyHostToDevice, stream));
+  CUVS_HIP_TRY(hipMemcpyAsync(list_sizes.ptr, h_list_sizes.data(), sizeof(uint32_t) * n_lists,
+                              hipMemcpyHostToDevice, stream));
+  CUVS_HIP_TRY(hipStreamSynchronize(stream));  // the host vectors above go out of scope
+  std::vector<uint32_t> sorted(h_list_sizes);
+  std::sort(sorted.begin(), sorted.end(), std::greater<uint32_t>());
+  accum_sorted_sizes.assign(n_lists + 1, 0);
+  for (uint32_t l = 0; l < n_lists; l++) {
+    accum_sorted_sizes[l + 1] = accum_sorted_sizes[l] + sorted[l];
+  }
+  size = accum_sorted_sizes[n_lists];
+}
+
+}  // namespace detail
+
+template <typename IdxT>
+index<IdxT>::index() : impl_(new detail::index_impl())
+{
+}
+template <typename IdxT>
+index<IdxT>::~index() = default;
+template <typename IdxT>
+index<IdxT>::index(index&&) noexcept = default;
+template <typename IdxT>
+index<IdxT>& index<IdxT>::operator=(index&&) noexcept = default;
+
+#define IMPL_GETTER(type, name, expr)    \
+  template <typename IdxT>               \
+  type index<IdxT>::name() const         \
+  {                                      \
+    return expr;                         \
+  }
+
+IMPL_GETTER(int64_t, size, impl_->size)
+IMPL_GETTER(uint32_t, dim, impl_->dim)
+IMPL_GETTER(uint32_t, dim_ext, impl_->dim_ext)
+IMPL_GETTER(uint32_t, rot_dim, impl_->rot_dim)
+IMPL_GETTER(uint32_t, pq_bits, impl_->pq_bits)
+IMPL_GETTER(uint32_t, pq_dim, impl_->pq_dim)
+IMPL_GETTER(uint32_t, pq_len, impl_->pq_len)
+IMPL_GETTER(uint32_t, pq_book_size, impl_->book_size)
+IMPL_GETTER(uint32_t, n_lists, impl_->n_lists)
+IMPL_GETTER(cuvs::distance::DistanceType, metric, impl_->metric)
+IMPL_GETTER(codebook_gen, codebook_kind, impl_->codebook_kind)
+IMPL_GETTER(list_layout, codes_layout, list_layout::INTERLEAVED)
+IMPL_GETTER(bool, conservative_memory_allocation, impl_->conservative_memory_allocation)
+IMPL_GETTER(const float*, centers, impl_->centers.template as<float>())
+IMPL_GETTER(const float*, centers_rot, impl_->centers_rot.template as<float>())
+IMPL_GETTER(const float*, rotation_matrix, impl_->rotation.template as<float>())
+IMPL_GETTER(const float*, pq_centers, impl_->pq_centers.template as<float>())
+IMPL_GETTER(const uint32_t*, list_sizes, impl_->list_sizes.template as<uint32_t>())
+IMPL_GETTER(const uint8_t* const*, data_ptrs, impl_->data_ptrs.template as<const uint8_t*>())
+IMPL_GETTER(const IdxT* const*, inds_ptrs, impl_->inds_ptrs.template as<const IdxT*>())
+IMPL_GETTER(const int64_t*, accum_sorted_sizes, impl_->accum_sorted_sizes.data())
+
+template class index<int64_t>;
+
+index<int64_t> build(cuvs::resources const& res,
+                     const index_params& params,
+                     uint32_t dim,
+                     const float* pq_centers,
+                     const float* centers,
+                     const float* centers_rot,
+                     const float* rotation_matrix)
+{
+  CUVS_EXPECTS(params.codes_layout == list_layout::INTERLEAVED,
+               "only the INTERLEAVED codes layout is supported");
+  CUVS_EXPECTS(pq_centers != nullptr && centers != nullptr && centers_rot != nullptr &&
+                 rotation_matrix != nullptr,
+               "model tensors must not be null");
+  index<int64_t> idx;
+  auto& ix = *idx.impl();
+  detail::init_index(ix, params, dim);
+  hipStream_t stream = res.stream();
+  const size_t n_books =
+    ix.codebook_kind == codebook_gen::PER_SUBSPACE ? ix.pq_dim : ix.n_lists;
+  auto copy_in = [&](device_buffer& dst, const float* src, size_t n) {
+    dst.allocate(n * sizeof(float));
+    CUVS_HIP_TRY(hipMemcpyAsync(dst.ptr, src, n * sizeof(float), hipMemcpyDeviceToDevice, stream));
+  };
+  copy_in(ix.pq_centers, pq_centers, n_books * ix.pq_len * ix.book_size);
+  copy_in(ix.centers, centers, size_t(ix.n_lists) * ix.dim_ext);
+  copy_in(ix.centers_rot, centers_rot, size_t(ix.n_lists) * ix.rot_dim);
+  copy_in(ix.rotation, rotation_matrix, size_t(ix.rot_dim) * ix.dim);
+
+  // transposed copy [dim, rot_dim] for coalesced reads, and the identity check
+  std::vector<float> rot(size_t(ix.rot_dim) * ix.dim), rot_t(size_t(ix.rot_dim) * ix.dim);
+  CUVS_HIP_TRY(hipMemcpyAsync(rot.data(), rotation_matrix, rot.size() * sizeof(float),
+                              hipMemcpyDeviceToHost, stream));
+  CUVS_HIP_TRY(hipStreamSynchronize(stream));
+  bool identity = ix.rot_dim == ix.dim;
+  for (uint32_t r = 0; r < ix.rot_dim; r++) {
+    for (uint32_t d = 0; d < ix.dim; d++) {
+      const float v               = rot[size_t(r) * ix.dim + d];
+      rot_t[size_t(d) * ix.rot_dim + r] = v;
+      if (v != (r == d ? 1.0f : 0.0f)) { identity = false; }
+    }
+  }
+  ix.rotation_is_identity = identity;
+  ix.rotation_t.allocate(rot_t.size() * sizeof(float));
+  CUVS_HIP_TRY(hipMemcpyAsync(ix.rotation_t.ptr, rot_t.data(), rot_t.size() * sizeof(float),
+                              hipMemcpyHostToDevice, stream));
+  ix.recompute_internal_state(stream);
+  return idx;
+}
+
+void unpack_contiguous_list_data(cuvs::resources const& res,
+                                 const index<int64_t>& idx,
+                                 uint8_t* out_codes,
+                                 uint32_t n_rows,
+                                 uint32_t label,
+                                 uint32_t offset)
+{
+  const auto& ix = *idx.impl();
+  CUVS_EXPECTS(label < ix.n_lists, "label (%u) must be smaller than n_lists (%u)", label, ix.n_lists);
+  CUVS_EXPECTS(uint64_t(offset) + n_rows <= ix.h_list_sizes[label],
+               "offset + n_rows (%u + %u) must not exceed the list size (%u)", offset, n_rows,
+               ix.h_list_sizes[label]);
+  const uint8_t* data = ix.codes_arena.as<uint8_t>() +
+                        (ix.h_row_offsets[label] / kIndexGroupSize) * ix.group_bytes();
+  detail::launch_unpack_contiguous(data, n_rows, offset, ix.pq_dim, ix.pq_bits, out_codes,
+                                   res.stream());
+}
+
+}  // namespace cuvs::neighbors::ivf_pq

@@ -1,0 +1,1232 @@
+/*
+ * HIP kernels of the IVF-PQ search path for gfx950 (wave64, 160 KB LDS per CU).
+ *
+ * Stage order of one search batch (host driver: search.cpp):
+ *   map_queries -> coarse_scores -> select_probes -> rotate -> chunk_indices -> order_pairs
+ *   -> scan (LUT in LDS + code scan + per-pair top-k) -> merge (+ distance / id post-processing)
+ * List maintenance: histogram, relocate_lists, encode, unpack_contiguous.
+ *
+ * Arithmetic that decides results is written with explicit fmaf / explicit rounding so that it is
+ * reproducible against a scalar CPU implementation: dot products accumulate with one FMA per
+ * element in ascending index order; lookup-table entries are built in fp32 and rounded once.
+ */
+#include "detail.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <cfloat>
+#include <type_traits>
+
+namespace cuvs::neighbors::ivf_pq::detail {
+
+namespace {
+
+constexpr int kBlock              = 256;
+constexpr unsigned long long kInvalidKey = 0xFFFFFFFFFFFFFFFFull;
+
+/* ---------------------------------------------------------------------------------------- */
+/* small device helpers                                                                      */
+/* ---------------------------------------------------------------------------------------- */
+
+/** Monotone map float -> uint32 (ascending); -0 and +0 map to the same key. */
+__device__ __forceinline__ uint32_t order_f32(float f)
+{
+  f          = (f == 0.0f) ? 0.0f : f;
+  uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float unorder_f32(uint32_t k)
+{
+  uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+  return __uint_as_float(u);
+}
+
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v)
+{
+  const uint32_t lane = threadIdx.x & 63u;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    uint32_t o = __shfl_up(v, d, 64);
+    if (lane >= uint32_t(d)) { v += o; }
+  }
+  return v;
+}
+
+/** In-place ascending bitonic sort of n (power of two) keys in LDS by the whole block. */
+__device__ void block_bitonic_sort(unsigned long long* a, uint32_t n)
+{
+  for (uint32_t size = 2; size <= n; size <<= 1) {
+    for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+      for (uint32_t t = threadIdx.x; t < (n >> 1); t += blockDim.x) {
+        const uint32_t pos     = 2 * t - (t & (stride - 1));
+        const uint32_t partner = pos + stride;
+        const bool ascending   = (pos & size) == 0;
+        const unsigned long long x = a[pos];
+        const unsigned long long y = a[partner];
+        if ((x > y) == ascending) {
+          a[pos]     = y;
+          a[partner] = x;
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+/* ---------------------------------------------------------------------------------------- */
+/* exact k-smallest selection of 64-bit keys by one block: MSB-first radix passes over an     */
+/* 11-bit digit that stop as soon as a digit boundary coincides with the k-th element, then    */
+/* one collection pass and a bitonic sort of the k survivors.                                  */
+/* ---------------------------------------------------------------------------------------- */
+
+constexpr int kRadixBits = 11;
+constexpr int kBins      = 1 << kRadixBits;
+
+struct select_smem {
+  uint32_t hist[kBins];
+  uint32_t wave_sums[kBlock / 64];
+  uint32_t bin, before, upto, count;
+};
+
+/**
+ * key_of(i), i < n, returns the key of element i or kInvalidKey.  Writes the min(k, #valid)
+ * smallest keys ascending into out[0..), pads the rest of out[0..out_cap) with kInvalidKey and
+ * returns their number.  out_cap is a power of two >= k.  All threads of the block must call.
+ */
+template <typename KeyFn>
+__device__ uint32_t block_select_sorted(KeyFn key_of, uint32_t n, uint32_t k,
+                                        unsigned long long* out, uint32_t out_cap, select_smem& sm)
+{
+  const uint32_t tid = threadIdx.x;
+  unsigned long long prefix = 0;
+  uint32_t pb   = 0;  // number of leading key bits already fixed in `prefix`
+  uint32_t need = k;
+  bool none     = false;
+  for (;;) {
+    const uint32_t digit_bits = (64u - pb) < uint32_t(kRadixBits) ? (64u - pb) : uint32_t(kRadixBits);
+    const uint32_t shift      = 64u - pb - digit_bits;
+    const uint32_t dmask      = (1u << digit_bits) - 1u;
+    for (uint32_t i = tid; i < uint32_t(kBins); i += kBlock) { sm.hist[i] = 0; }
+    __syncthreads();
+    for (uint32_t i = tid; i < n; i += kBlock) {
+      const unsigned long long key = key_of(i);
+      if (key != kInvalidKey && (pb == 0 || (key >> (64u - pb)) == prefix)) {
+        atomicAdd(&sm.hist[uint32_t(key >> shift) & dmask], 1u);
+      }
+    }
+    __syncthreads();
+    constexpr uint32_t per = kBins / kBlock;
+    uint32_t s = 0;
+#pragma unroll
+    for (uint32_t j = 0; j < per; j++) { s += sm.hist[tid * per + j]; }
+    uint32_t incl = wave_inclusive_scan(s);
+    if ((tid & 63u) == 63u) { sm.wave_sums[tid >> 6] = incl; }
+    __syncthreads();
+    uint32_t base = 0, total = 0;
+#pragma unroll
+    for (uint32_t w = 0; w < kBlock / 64; w++) {
+      const uint32_t ws = sm.wave_sums[w];
+      if (w < (tid >> 6)) { base += ws; }
+      total += ws;
+    }
+    incl += base;
+    const uint32_t excl = incl - s;
+    if (pb == 0 && need > total) { need = total; }
+    if (need == 0) {
+      none = true;
+      break;
+    }
+    if (excl < need && need <= incl) {
+      uint32_t c = excl;
+      for (uint32_t j = 0; j < per; j++) {
+        const uint32_t h = sm.hist[tid * per + j];
+        if (c + h >= need) {
+          sm.bin    = tid * per + j;
+          sm.before = c;
+          sm.upto   = c + h;
+          break;
+        }
+        c += h;
+      }
+    }
+    __syncthreads();
+    const uint32_t b      = sm.bin;
+    const uint32_t before = sm.before;
+    const uint32_t upto   = sm.upto;
+    prefix                = (prefix << digit_bits) | b;
+    pb += digit_bits;
+    __syncthreads();
+    if (upto == need || pb >= 64u) { break; }
+    need -= before;
+  }
+
+  if (tid == 0) { sm.count = 0; }
+  __syncthreads();
+  if (!none) {
+    for (uint32_t i = tid; i < n; i += kBlock) {
+      const unsigned long long key = key_of(i);
+      if (key != kInvalidKey && (key >> (64u - pb)) <= prefix) {
+        const uint32_t pos = atomicAdd(&sm.count, 1u);
+        if (pos < out_cap) { out[pos] = key; }
+      }
+    }
+  }
+  __syncthreads();
+  uint32_t cnt = sm.count;
+  if (cnt > out_cap) { cnt = out_cap; }
+  for (uint32_t i = cnt + tid; i < out_cap; i += kBlock) { out[i] = kInvalidKey; }
+  __syncthreads();
+  block_bitonic_sort(out, out_cap);
+  return cnt < k ? cnt : k;
+}
+
+/* ---------------------------------------------------------------------------------------- */
+/* element mapping, coarse scores, probe selection                                           */
+/* ---------------------------------------------------------------------------------------- */
+
+__global__ void fill_u32_kernel(uint32_t* dst, uint32_t value, uint64_t n)
+{
+  const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) { dst[i] = value; }
+}
+
+template <typename T>
+__device__ __forceinline__ float map_elem(T v);
+template <>
+__device__ __forceinline__ float map_elem<float>(float v)
+{
+  return v;
+}
+template <>
+__device__ __forceinline__ float map_elem<_Float16>(_Float16 v)
+{
+  return float(v);
+}
+template <>
+__device__ __forceinline__ float map_elem<int8_t>(int8_t v)
+{
+  return float(v) * (1.0f / 128.0f);
+}
+template <>
+__device__ __forceinline__ float map_elem<uint8_t>(uint8_t v)
+{
+  return float(v) * (1.0f / 256.0f);
+}
+
+template <typename T>
+__global__ void map_queries_kernel(const T* in, uint64_t n, float* out)
+{
+  const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) { out[i] = map_elem<T>(in[i]); }
+}
+
+__device__ __forceinline__ float round_to_half(float v) { return float(_Float16(v)); }
+
+/**
+ * 64 queries x 64 lists per block, 4 x 4 outputs per thread, K staged through LDS in slabs of 16.
+ * Every output is one FMA chain over d = 0..dim-1 followed by the norm term, so the value does
+ * not depend on the tiling.
+ */
+constexpr int kCoarseTile = 64;
+constexpr int kCoarseK    = 16;
+
+template <bool HALF>
+__global__ __launch_bounds__(kBlock) void coarse_scores_kernel(const float* __restrict__ qf,
+                                                                const float* __restrict__ centers,
+                                                                uint32_t n_queries,
+                                                                uint32_t n_lists, uint32_t dim,
+                                                                uint32_t dim_ext, float qnorm,
+                                                                float alpha,
+                                                                float* __restrict__ scores)
+{
+  __shared__ float sq[kCoarseK][kCoarseTile + 4];
+  __shared__ float sc[kCoarseK][kCoarseTile + 4];
+  const uint32_t tid = threadIdx.x;
+  const uint32_t tx  = tid & 15u;  // list direction
+  const uint32_t ty  = tid >> 4;   // query direction
+  const uint32_t q0  = blockIdx.y * kCoarseTile;
+  const uint32_t l0  = blockIdx.x * kCoarseTile;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) { acc[i][j] = 0.0f; }
+  }
+  const uint32_t lr = tid >> 4;   // 0..15: row within a load pass
+  const uint32_t lc = tid & 15u;  // 0..15: column (k) within the slab
+  for (uint32_t d0 = 0; d0 < dim; d0 += kCoarseK) {
+#pragma unroll
+    for (int pass = 0; pass < 4; pass++) {
+      const uint32_t r = lr + 16u * pass;
+      const uint32_t d = d0 + lc;
+      float vq = 0.0f, vc = 0.0f;
+      if (d < dim) {
+        if (q0 + r < n_queries) { vq = qf[uint64_t(q0 + r) * dim + d]; }
+        if (l0 + r < n_lists) { vc = centers[uint64_t(l0 + r) * dim_ext + d]; }
+      }
+      if (HALF) {
+        vq = round_to_half(vq);
+        vc = round_to_half(vc);
+      }
+      sq[lc][r] = vq;
+      sc[lc][r] = vc;
+    }
+    __syncthreads();
+    const uint32_t kmax = (dim - d0) < uint32_t(kCoarseK) ? (dim - d0) : uint32_t(kCoarseK);
+    for (uint32_t kk = 0; kk < kmax; kk++) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) { a[i] = sq[kk][ty * 4 + i]; }
+#pragma unroll
+      for (int j = 0; j < 4; j++) { b[j] = sc[kk][tx * 4 + j]; }
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) { acc[i][j] = fmaf(b[j], a[i], acc[i][j]); }
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const uint32_t l = l0 + tx * 4 + j;
+    if (l >= n_lists) { continue; }
+    float nrm = centers[uint64_t(l) * dim_ext + dim];
+    if (HALF) { nrm = round_to_half(nrm); }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t q = q0 + ty * 4 + i;
+      if (q >= n_queries) { continue; }
+      float v = alpha * fmaf(nrm, qnorm, acc[i][j]);
+      if (HALF) { v = round_to_half(v); }
+      scores[uint64_t(q) * n_lists + l] = v;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void select_probes_kernel(const float* __restrict__ scores,
+                                                                uint32_t n_lists,
+                                                                uint32_t n_probes,
+                                                                uint32_t out_cap,
+                                                                uint32_t* __restrict__ probes)
+{
+  extern __shared__ __align__(16) unsigned char dyn_smem[];
+  __shared__ select_smem sm;
+  unsigned long long* out = reinterpret_cast<unsigned long long*>(dyn_smem);
+  const uint32_t q        = blockIdx.x;
+  const float* row        = scores + uint64_t(q) * n_lists;
+  auto key_of             = [row](uint32_t i) -> unsigned long long {
+    const float v = row[i];
+    if (v != v) { return kInvalidKey; }
+    return (static_cast<unsigned long long>(order_f32(v)) << 32) | i;
+  };
+  block_select_sorted(key_of, n_lists, n_probes, out, out_cap, sm);
+  for (uint32_t r = threadIdx.x; r < n_probes; r += kBlock) {
+    const unsigned long long key = out[r];
+    // fewer than n_probes comparable scores (NaN input): fall back to the slot number
+    probes[uint64_t(q) * n_probes + r] = key == kInvalidKey ? (r % n_lists) : uint32_t(key);
+  }
+}
+
+/* ---------------------------------------------------------------------------------------- */
+/* rotation, chunk indices, pair ordering                                                    */
+/* ---------------------------------------------------------------------------------------- */
+
+constexpr int kRotQueries = 4;
+
+__global__ __launch_bounds__(kBlock) void rotate_kernel(const float* __restrict__ qf,
+                                                         const float* __restrict__ rotation_t,
+                                                         uint32_t n_queries, uint32_t dim,
+                                                         uint32_t rot_dim, int identity,
+                                                         int normalize, float* __restrict__ rot_q)
+{
+  extern __shared__ __align__(16) unsigned char dyn_smem[];
+  float* sq           = reinterpret_cast<float*>(dyn_smem);  // [kRotQueries][dim]
+  float* sr           = sq + kRotQueries * dim;              // [kRotQueries][rot_dim]
+  __shared__ float s_norm[kRotQueries];
+  const uint32_t q0   = blockIdx.x * kRotQueries;
+  const uint32_t nq   = (n_queries - q0) < uint32_t(kRotQueries) ? (n_queries - q0) : kRotQueries;
+  for (uint32_t i = threadIdx.x; i < nq * dim; i += kBlock) { sq[i] = qf[uint64_t(q0) * dim + i]; }
+  __syncthreads();
+  for (uint32_t r = threadIdx.x; r < rot_dim; r += kBlock) {
+    float acc[kRotQueries];
+#pragma unroll
+    for (int i = 0; i < kRotQueries; i++) { acc[i] = 0.0f; }
+    if (identity) {
+#pragma unroll
+      for (int i = 0; i < kRotQueries; i++) { acc[i] = (uint32_t(i) < nq) ? sq[i * dim + r] : 0.0f; }
+    } else {
+      for (uint32_t d = 0; d < dim; d++) {
+        const float w = rotation_t[uint64_t(d) * rot_dim + r];
+#pragma unroll
+        for (int i = 0; i < kRotQueries; i++) {
+          if (uint32_t(i) < nq) { acc[i] = fmaf(w, sq[i * dim + d], acc[i]); }
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kRotQueries; i++) {
+      if (uint32_t(i) < nq) { sr[i * rot_dim + r] = acc[i]; }
+    }
+  }
+  __syncthreads();
+  if (normalize) {
+    // cosine: divide by the L2 norm; the sum of squares is one FMA chain in ascending order
+    if (threadIdx.x < nq) {
+      float ss = 0.0f;
+      for (uint32_t r = 0; r < rot_dim; r++) {
+        const float v = sr[threadIdx.x * rot_dim + r];
+        ss            = fmaf(v, v, ss);
+      }
+      s_norm[threadIdx.x] = sqrtf(ss);
+    }
+    __syncthreads();
+  }
+  for (uint32_t i = threadIdx.x; i < nq * rot_dim; i += kBlock) {
+    float v = sr[i];
+    if (normalize) {
+      const float nrm = s_norm[i / rot_dim];
+      if (nrm > 0.0f) { v = v / nrm; }
+    }
+    rot_q[uint64_t(q0) * rot_dim + i] = v;
+  }
+}
+
+/** One wave per query: inclusive prefix sums of the probed list sizes in probe order. */
+__global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __restrict__ list_sizes,
+                                                            const uint32_t* __restrict__ probes,
+                                                            uint32_t n_probes,
+                                                            uint32_t row_chunk_bytes,
+                                                            uint32_t* __restrict__ chunk_indices,
+                                                            uint32_t* __restrict__ n_samples,
+                                                            unsigned long long* stats)
+{
+  const uint32_t q    = blockIdx.x;
+  const uint32_t lane = threadIdx.x;
+  uint32_t carry      = 0;
+  unsigned long long padded_rows = 0;
+  for (uint32_t p0 = 0; p0 < n_probes; p0 += 64) {
+    const uint32_t p = p0 + lane;
+    uint32_t sz      = 0;
+    if (p < n_probes) { sz = list_sizes[probes[uint64_t(q) * n_probes + p]]; }
+    padded_rows += (sz + 31u) & ~31u;
+    const uint32_t incl = wave_inclusive_scan(sz) + carry;
+    if (p < n_probes) { chunk_indices[uint64_t(q) * n_probes + p] = incl; }
+    carry = __shfl(incl, 63, 64);
+  }
+  if (lane == 0) { n_samples[q] = carry; }
+  if (stats != nullptr) {
+    // wave reduction of the padded row count
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) { padded_rows += __shfl_down(padded_rows, d, 64); }
+    if (lane == 0) {
+      atomicAdd(&stats[0], padded_rows * row_chunk_bytes);
+      atomicAdd(&stats[1], static_cast<unsigned long long>(carry));
+    }
+  }
+}
+
+__global__ void pair_histogram_kernel(const uint32_t* __restrict__ probes, uint32_t n_pairs,
+                                      uint32_t* __restrict__ counts)
+{
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n_pairs) { atomicAdd(&counts[probes[i]], 1u); }
+}
+
+/** Single block: cursors[l] = exclusive prefix sum of counts[l]. */
+__global__ __launch_bounds__(kBlock) void exclusive_scan_kernel(const uint32_t* __restrict__ counts,
+                                                                 uint32_t n,
+                                                                 uint32_t* __restrict__ cursors)
+{
+  __shared__ uint32_t wave_sums[kBlock / 64];
+  __shared__ uint32_t s_carry;
+  if (threadIdx.x == 0) { s_carry = 0; }
+  __syncthreads();
+  for (uint32_t i0 = 0; i0 < n; i0 += kBlock) {
+    const uint32_t i = i0 + threadIdx.x;
+    const uint32_t v = i < n ? counts[i] : 0u;
+    uint32_t incl    = wave_inclusive_scan(v);
+    if ((threadIdx.x & 63u) == 63u) { wave_sums[threadIdx.x >> 6] = incl; }
+    __syncthreads();
+    uint32_t base = s_carry;
+    for (uint32_t w = 0; w < (threadIdx.x >> 6); w++) { base += wave_sums[w]; }
+    incl += base;
+    if (i < n) { cursors[i] = incl - v; }
+    __syncthreads();
+    if (threadIdx.x == kBlock - 1) { s_carry = incl; }
+    __syncthreads();
+  }
+}
+
+__global__ void pair_scatter_kernel(const uint32_t* __restrict__ probes, uint32_t n_pairs,
+                                    uint32_t* __restrict__ cursors,
+                                    uint32_t* __restrict__ pair_order)
+{
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n_pairs) {
+    const uint32_t pos = atomicAdd(&cursors[probes[i]], 1u);
+    pair_order[pos]    = i;
+  }
+}
+
+/* ---------------------------------------------------------------------------------------- */
+/* lookup-table element types                                                                */
+/* ---------------------------------------------------------------------------------------- */
+
+enum { LUT_F32 = 0, LUT_F16 = 1, LUT_FP8U = 2, LUT_FP8S = 3 };
+
+/* 8-bit float with 5 exponent bits, bias 15, 3 (unsigned) or 2 (signed, sign in the LSB) value
+ * bits: encode truncates, decode adds half a unit (cuVS ivf_pq_fp_8bit.cuh:31-100). */
+__device__ __forceinline__ uint8_t fp8_encode_unsigned(float v)
+{
+  if (v < 3.0517578125e-05f) { return 0; }  // 2^-15
+  if (v >= 122880.0f) { return 0xffu; }     // 2^16 * (2 - 1/8)
+  return uint8_t((__float_as_uint(v) + (15u << 23) - 0x3f800000u) >> 20);
+}
+__device__ __forceinline__ uint8_t fp8_encode_signed(float v)
+{
+  const uint8_t u = fp8_encode_unsigned(fabsf(v));
+  return uint8_t((u & 0xfeu) | (v < 0.0f ? 1u : 0u));
+}
+
+template <int LUT>
+struct lut_traits;
+template <>
+struct lut_traits<LUT_F32> {
+  using storage = float;
+  static __device__ __forceinline__ storage encode(float v) { return v; }
+  static __device__ __forceinline__ float to_float(storage s) { return s; }
+  static __device__ __forceinline__ _Float16 to_half(storage s) { return _Float16(s); }
+};
+template <>
+struct lut_traits<LUT_F16> {
+  using storage = _Float16;
+  static __device__ __forceinline__ storage encode(float v) { return _Float16(v); }
+  static __device__ __forceinline__ float to_float(storage s) { return float(s); }
+  static __device__ __forceinline__ _Float16 to_half(storage s) { return s; }
+};
+template <>
+struct lut_traits<LUT_FP8U> {
+  using storage = uint8_t;
+  static __device__ __forceinline__ storage encode(float v) { return fp8_encode_unsigned(v); }
+  static __device__ __forceinline__ float to_float(storage s)
+  {
+    return __uint_as_float(0x38080000u + (uint32_t(s) << 20));
+  }
+  static __device__ __forceinline__ _Float16 to_half(storage s)
+  {
+    const uint16_t bits = uint16_t(0x0040u + (uint32_t(s) << 7));
+    return __builtin_bit_cast(_Float16, bits);
+  }
+};
+template <>
+struct lut_traits<LUT_FP8S> {
+  using storage = uint8_t;
+  static __device__ __forceinline__ storage encode(float v) { return fp8_encode_signed(v); }
+  static __device__ __forceinline__ float to_float(storage s)
+  {
+    const uint32_t bits = 0x38080000u + (uint32_t(s & 0xfeu) << 20);
+    return __uint_as_float(bits | (uint32_t(s & 1u) << 31));
+  }
+  static __device__ __forceinline__ _Float16 to_half(storage s)
+  {
+    const uint16_t bits = uint16_t((0x0040u + (uint32_t(s & 0xfeu) << 7)) | (uint32_t(s & 1u) << 15));
+    return __builtin_bit_cast(_Float16, bits);
+  }
+};
+
+/* ---------------------------------------------------------------------------------------- */
+/* the scan kernel: one block per (query, probed list) pair                                   */
+/* ---------------------------------------------------------------------------------------- */
+
+constexpr uint32_t kCandCap = 1024;  // per-block candidate buffer (keys), >= k + kBlock
+
+struct scan_smem_tail {
+  uint32_t count;
+  uint32_t thr;
+};
+
+__device__ __forceinline__ bool is_ip_metric(int metric)
+{
+  return metric == int(DistanceType::InnerProduct) || metric == int(DistanceType::CosineExpanded);
+}
+
+template <int LUT, bool OUT_HALF, int BITS, bool FUSED>
+__global__ __launch_bounds__(kBlock) void scan_kernel(scan_args a)
+{
+  using traits  = lut_traits<LUT>;
+  using lut_t   = typename traits::storage;
+  using acc_t   = typename std::conditional<OUT_HALF, _Float16, float>::type;
+  constexpr uint32_t B   = 1u << BITS;
+  constexpr uint32_t CPC = 128u / BITS;  // codes per 16-byte chunk
+
+  extern __shared__ __align__(16) unsigned char dyn_smem[];
+  const uint32_t lut_entries = a.pq_dim << BITS;
+  lut_t* lut                 = reinterpret_cast<lut_t*>(dyn_smem);
+  const uint32_t lut_bytes   = (lut_entries * uint32_t(sizeof(lut_t)) + 15u) & ~15u;
+  float* base_diff           = reinterpret_cast<float*>(dyn_smem + lut_bytes);
+  const bool ip              = is_ip_metric(a.metric);
+  const uint32_t diff_floats = a.rot_dim * (ip ? 2u : 1u);
+  unsigned long long* cand =
+    reinterpret_cast<unsigned long long*>(dyn_smem + lut_bytes + ((diff_floats * 4u + 15u) & ~15u));
+  scan_smem_tail* tail = reinterpret_cast<scan_smem_tail*>(cand + (FUSED ? kCandCap : 0));
+
+  const uint32_t tid  = threadIdx.x;
+  const uint32_t pair = a.pair_order != nullptr ? a.pair_order[blockIdx.x] : blockIdx.x;
+  const uint32_t q    = pair / a.n_probes;
+  const uint32_t p    = pair - q * a.n_probes;
+  const uint32_t label = a.probes[uint64_t(q) * a.n_probes + p];
+  const uint32_t* chunk_row = a.chunk_indices + uint64_t(q) * a.n_probes;
+  const uint32_t sample_off = p > 0 ? chunk_row[p - 1] : 0u;
+  const uint32_t n_rows     = chunk_row[p] - sample_off;
+
+  /* ---- stage the per-dimension query/centre terms ---- */
+  const float* rq = a.rot_q + uint64_t(q) * a.rot_dim;
+  const float* cr = a.centers_rot + uint64_t(label) * a.rot_dim;
+  for (uint32_t i = tid; i < a.rot_dim; i += kBlock) {
+    if (!ip) {
+      base_diff[i] = rq[i] - cr[i];
+    } else {
+      const float qv       = rq[i];
+      base_diff[2 * i]     = qv;
+      base_diff[2 * i + 1] = cr[i] * qv;
+    }
+  }
+  if (FUSED && tid == 0) {
+    tail->count = 0;
+    tail->thr   = 0xFFFFFFFFu;
+  }
+  __syncthreads();
+
+  /* ---- lookup table: LUT[j][code] = LutT(score of codebook entry `code` in subspace j) ---- */
+  {
+    const float* books = a.pq_centers +
+                         (a.per_cluster ? uint64_t(label) * a.pq_len * B : uint64_t(0));
+    for (uint32_t i = tid; i < lut_entries; i += kBlock) {
+      const uint32_t j    = i >> BITS;
+      const uint32_t code = i & (B - 1u);
+      const float* book   = books + (a.per_cluster ? uint64_t(0) : uint64_t(j) * a.pq_len * B) + code;
+      float score         = 0.0f;
+      for (uint32_t t = 0; t < a.pq_len; t++) {
+        const float pqc  = book[uint64_t(t) * B];
+        const uint32_t d = j * a.pq_len + t;
+        if (!ip) {
+          float diff = base_diff[d];
+          diff -= pqc;
+          score = fmaf(diff, diff, score);
+        } else {
+          const float qv = base_diff[2 * d];
+          score -= base_diff[2 * d + 1];
+          score = fmaf(-qv, pqc, score);
+        }
+      }
+      lut[i] = traits::encode(score);
+    }
+  }
+  __syncthreads();
+
+  /* ---- scan the list ---- */
+  const uint8_t* list_data = a.data_ptrs[label];
+  const int64_t* list_ids  = a.filter_bits != nullptr ? a.inds_ptrs[label] : nullptr;
+  const uint32_t n_chunks  = (a.pq_dim + CPC - 1u) / CPC;
+  const uint32_t n_full    = a.pq_dim / CPC;
+  const uint32_t n_padded  = (n_rows + 31u) & ~31u;
+  uint32_t thr             = 0xFFFFFFFFu;
+  if (FUSED) { thr = a.query_kth[q]; }
+
+  for (uint32_t i0 = 0; i0 < n_padded; i0 += kBlock) {
+    const uint32_t i = i0 + tid;
+    bool valid       = i < n_rows;
+    if (valid && list_ids != nullptr) {
+      const int64_t id = list_ids[i];
+      valid = id >= 0 && id < a.filter_nbits && ((a.filter_bits[id >> 5] >> (id & 31)) & 1u) != 0;
+    }
+    float score_f = 0.0f;
+    if (valid) {
+      const uint8_t* ptr =
+        list_data + uint64_t(i >> 5) * n_chunks * 512u + uint64_t(i & 31u) * 16u;
+      acc_t acc        = acc_t(0);
+      const lut_t* lh  = lut;
+      for (uint32_t m = 0; m < n_full; m++) {
+        const uint4 v       = *reinterpret_cast<const uint4*>(ptr + uint64_t(m) * 512u);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (uint32_t kk = 0; kk < CPC; kk++) {
+          constexpr uint32_t mask = B - 1u;
+          const uint32_t bit      = kk * BITS;
+          const uint32_t word     = bit >> 5;
+          const uint32_t off      = bit & 31u;
+          uint32_t c              = w[word] >> off;
+          if (off + BITS > 32u) { c |= w[(word + 1u) & 3u] << (32u - off); }
+          c &= mask;
+          if (OUT_HALF) {
+            acc = acc_t(acc + traits::to_half(lh[(kk << BITS) + c]));
+          } else {
+            acc = acc_t(acc + traits::to_float(lh[(kk << BITS) + c]));
+          }
+        }
+        lh += CPC << BITS;
+      }
+      if (n_full < n_chunks) {
+        const uint4 v       = *reinterpret_cast<const uint4*>(ptr + uint64_t(n_full) * 512u);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        const uint32_t rem  = a.pq_dim - n_full * CPC;
+#pragma unroll
+        for (uint32_t kk = 0; kk < CPC; kk++) {
+          if (kk < rem) {
+            constexpr uint32_t mask = B - 1u;
+            const uint32_t bit      = kk * BITS;
+            const uint32_t word     = bit >> 5;
+            const uint32_t off      = bit & 31u;
+            uint32_t c              = w[word] >> off;
+            if (off + BITS > 32u) { c |= w[(word + 1u) & 3u] << (32u - off); }
+            c &= mask;
+            if (OUT_HALF) {
+              acc = acc_t(acc + traits::to_half(lh[(kk << BITS) + c]));
+            } else {
+              acc = acc_t(acc + traits::to_float(lh[(kk << BITS) + c]));
+            }
+          }
+        }
+      }
+      if (a.metric == int(DistanceType::CosineExpanded)) { acc = acc_t(acc + acc_t(1)); }
+      score_f = float(acc);
+    }
+    if (score_f != score_f) { valid = false; }  // NaN never enters a result
+
+    if (FUSED) {
+      if (valid) {
+        const uint32_t okey = order_f32(score_f);
+        if (okey <= thr) {
+          const uint32_t pos = atomicAdd(&tail->count, 1u);
+          cand[pos] = (static_cast<unsigned long long>(okey) << 32) | (sample_off + i);
+        }
+      }
+      __syncthreads();
+      const uint32_t cnt = tail->count;
+      __syncthreads();  // every thread has read the count before anyone appends again
+      if (cnt > kCandCap - kBlock) {
+        // prune: keep the k smallest candidates, tighten the threshold
+        for (uint32_t t = cnt + tid; t < kCandCap; t += kBlock) { cand[t] = kInvalidKey; }
+        __syncthreads();
+        block_bitonic_sort(cand, kCandCap);
+        if (tid == 0) {
+          tail->count = cnt < a.k ? cnt : a.k;
+          if (cnt >= a.k) { tail->thr = uint32_t(cand[a.k - 1] >> 32); }
+        }
+        __syncthreads();
+        const uint32_t t2 = tail->thr;
+        thr               = t2 < thr ? t2 : thr;
+      }
+    } else {
+      if (i < n_rows) {
+        a.out_scores[uint64_t(q) * a.max_samples + sample_off + i] =
+          valid ? score_f : __uint_as_float(0x7fc00000u);
+      }
+    }
+  }
+
+  if (FUSED) {
+    __syncthreads();
+    uint32_t cnt = tail->count;
+    if (cnt >= a.k) {
+      uint32_t n2 = 1;
+      while (n2 < cnt) { n2 <<= 1; }
+      for (uint32_t t = cnt + tid; t < n2; t += kBlock) { cand[t] = kInvalidKey; }
+      __syncthreads();
+      block_bitonic_sort(cand, n2);
+      cnt = a.k;
+      if (tid == 0) { atomicMin(&a.query_kth[q], uint32_t(cand[a.k - 1] >> 32)); }
+    }
+    unsigned long long* out = a.out_keys + (uint64_t(q) * a.n_probes + p) * a.k;
+    for (uint32_t r = tid; r < a.k; r += kBlock) { out[r] = r < cnt ? cand[r] : kInvalidKey; }
+  }
+}
+
+/* ---------------------------------------------------------------------------------------- */
+/* per-query merge + post-processing                                                          */
+/* ---------------------------------------------------------------------------------------- */
+
+__device__ __forceinline__ float postprocess_distance(float d, int metric, float s)
+{
+  // cuVS postprocess_distances (cpp/src/neighbors/ivf_common.cuh:175-252)
+  switch (metric) {
+    case int(DistanceType::L2Expanded): return s != 1.0f ? d * (s * s) : d;
+    case int(DistanceType::L2SqrtExpanded): return s != 1.0f ? sqrtf(d) * s : sqrtf(d);
+    case int(DistanceType::InnerProduct): return d * (-1.0f * s * s);
+    case int(DistanceType::CosineExpanded): return s != 1.0f ? d * (s * s) : d;
+    default: return d;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void merge_kernel(merge_args a, uint32_t out_cap)
+{
+  extern __shared__ __align__(16) unsigned char dyn_smem[];
+  __shared__ select_smem sm;
+  unsigned long long* out = reinterpret_cast<unsigned long long*>(dyn_smem);
+  const uint32_t q        = blockIdx.x;
+  uint32_t n;
+  if (a.fused) {
+    n                              = a.n_probes * a.k;
+    const unsigned long long* keys = a.in_keys + uint64_t(q) * n;
+    block_select_sorted([keys](uint32_t i) { return keys[i]; }, n, a.k, out, out_cap, sm);
+  } else {
+    n                = a.n_samples[q];
+    const float* row = a.in_scores + uint64_t(q) * a.max_samples;
+    block_select_sorted(
+      [row](uint32_t i) -> unsigned long long {
+        const float v = row[i];
+        if (v != v) { return kInvalidKey; }
+        return (static_cast<unsigned long long>(order_f32(v)) << 32) | i;
+      },
+      n, a.k, out, out_cap, sm);
+  }
+  const uint32_t* chunk  = a.chunk_indices + uint64_t(q) * a.n_probes;
+  const uint32_t* probes = a.probes + uint64_t(q) * a.n_probes;
+  for (uint32_t r = threadIdx.x; r < a.k; r += kBlock) {
+    const unsigned long long key = out[r];
+    int64_t id                   = INT64_MAX;  // kOutOfBoundsRecord
+    float d                      = FLT_MAX;
+    if (key != kInvalidKey) {
+      uint32_t sample = uint32_t(key);
+      d               = unorder_f32(uint32_t(key >> 32));
+      // find_chunk_ix (cpp/src/neighbors/ivf_common.cuh:94-110)
+      uint32_t lo = 0, hi = a.n_probes;
+      do {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (chunk[mid] <= sample) {
+          lo = mid + 1;
+        } else {
+          hi = mid;
+        }
+      } while (lo < hi);
+      if (lo < a.n_probes) {
+        if (lo > 0) { sample -= chunk[lo - 1]; }
+        id = a.inds_ptrs[probes[lo]][sample];
+      }
+    }
+    a.neighbors[uint64_t(q) * a.k + r] = id;
+    a.distances[uint64_t(q) * a.k + r] = postprocess_distance(d, a.metric, a.scaling);
+  }
+}
+
+/* ---------------------------------------------------------------------------------------- */
+/* list maintenance and encoding                                                              */
+/* ---------------------------------------------------------------------------------------- */
+
+/** One thread per row: x /= ||x||_2, the sum of squares being one FMA chain in ascending order. */
+__global__ void normalize_rows_kernel(float* __restrict__ x, uint64_t n_rows, uint32_t dim)
+{
+  const uint64_t r = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (r >= n_rows) { return; }
+  float* row = x + r * dim;
+  float ss   = 0.0f;
+  for (uint32_t d = 0; d < dim; d++) { ss = fmaf(row[d], row[d], ss); }
+  const float nrm = sqrtf(ss);
+  if (nrm > 0.0f) {
+    for (uint32_t d = 0; d < dim; d++) { row[d] = row[d] / nrm; }
+  }
+}
+
+__global__ void histogram_kernel(const uint32_t* __restrict__ labels, uint64_t n,
+                                 uint32_t* __restrict__ counts)
+{
+  const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) { atomicAdd(&counts[labels[i]], 1u); }
+}
+
+/** One block per list: move the occupied 32-row groups and ids to their new arena position. */
+__global__ __launch_bounds__(kBlock) void relocate_lists_kernel(
+  const uint8_t* __restrict__ old_codes, const int64_t* __restrict__ old_ids,
+  uint8_t* __restrict__ new_codes, int64_t* __restrict__ new_ids,
+  const uint64_t* __restrict__ old_row_offsets, const uint64_t* __restrict__ new_row_offsets,
+  const uint32_t* __restrict__ old_sizes, uint32_t n_chunks)
+{
+  const uint32_t l  = blockIdx.x;
+  const uint32_t sz = old_sizes[l];
+  if (sz == 0) { return; }
+  const uint64_t group_bytes = uint64_t(n_chunks) * 512u;
+  const uint64_t n_vec       = uint64_t((sz + 31u) >> 5) * group_bytes / 16u;
+  const uint4* src = reinterpret_cast<const uint4*>(old_codes + (old_row_offsets[l] >> 5) * group_bytes);
+  uint4* dst       = reinterpret_cast<uint4*>(new_codes + (new_row_offsets[l] >> 5) * group_bytes);
+  for (uint64_t i = threadIdx.x; i < n_vec; i += kBlock) { dst[i] = src[i]; }
+  const int64_t* si = old_ids + old_row_offsets[l];
+  int64_t* di       = new_ids + new_row_offsets[l];
+  for (uint32_t i = threadIdx.x; i < sz; i += kBlock) { di[i] = si[i]; }
+}
+
+/**
+ * One thread per row.  residual = rotation * (x - centre[label]) with FMA chains in ascending
+ * order; code_j = argmin over the codebook of the squared distance, lowest code wins ties
+ * (cuVS ivf_pq_build.cuh:140-206, ivf_pq_process_and_fill_codes.cuh:84-126).
+ * The rotated residual of a row is kept in column r of `a.scratch` ([rot_dim, n], so that the
+ * threads of a wave touch consecutive addresses).  With per-subspace codebooks every thread of
+ * the block reads the same codebook element at the same time, which the compiler turns into
+ * scalar loads.
+ */
+template <int BITS, bool PER_CLUSTER>
+__global__ __launch_bounds__(kBlock) void encode_kernel(encode_args a)
+{
+  constexpr uint32_t B   = 1u << BITS;
+  constexpr uint32_t CPC = 128u / BITS;
+  const uint64_t r       = uint64_t(blockIdx.x) * kBlock + threadIdx.x;
+  if (r >= a.n_rows) { return; }
+  const uint32_t label = a.labels[r];
+  const float* x       = a.xf + r * a.dim;
+  const float* c       = a.centers + uint64_t(label) * a.dim_ext;
+  float* res           = a.scratch + r;  // element d at res[d * n_rows]
+  const uint64_t rs    = a.n_rows;
+  auto xval = [&](uint32_t d) -> float { return x[d]; };
+  if (a.identity_rotation) {
+    for (uint32_t d = 0; d < a.rot_dim; d++) { res[d * rs] = d < a.dim ? xval(d) - c[d] : 0.0f; }
+  } else {
+    for (uint32_t o = 0; o < a.rot_dim; o++) {
+      float acc = 0.0f;
+      for (uint32_t d = 0; d < a.dim; d++) {
+        acc = fmaf(a.rotation_t[uint64_t(d) * a.rot_dim + o], xval(d) - c[d], acc);
+      }
+      res[o * rs] = acc;
+    }
+  }
+
+  uint32_t slot        = 0;
+  uint8_t* list_base   = nullptr;
+  uint8_t* flat_row    = nullptr;
+  const uint32_t row_bytes = (a.pq_dim * BITS + 7u) / 8u;
+  if (a.flat_codes != nullptr) {
+    flat_row = a.flat_codes + r * row_bytes;
+    for (uint32_t b = 0; b < row_bytes; b++) { flat_row[b] = 0; }
+  } else {
+    slot      = atomicAdd(&a.cursors[label], 1u);
+    list_base = a.data_ptrs[label] + uint64_t(slot >> 5) * a.n_chunks * 512u + uint64_t(slot & 31u) * 16u;
+    a.inds_ptrs[label][slot] = a.ids != nullptr ? a.ids[r] : a.first_id + int64_t(r);
+  }
+
+  uint32_t w[4] = {0, 0, 0, 0};
+  for (uint32_t j = 0; j < a.pq_dim; j++) {
+    const float* book =
+      a.pq_centers + (PER_CLUSTER ? uint64_t(label) : uint64_t(j)) * a.pq_len * B;
+    float best        = __uint_as_float(0x7f800000u);
+    uint32_t code     = 0;
+    for (uint32_t l = 0; l < B; l++) {
+      float d = 0.0f;
+      for (uint32_t t = 0; t < a.pq_len; t++) {
+        const float v = res[uint64_t(j * a.pq_len + t) * rs] - book[uint64_t(t) * B + l];
+        d             = fmaf(v, v, d);
+      }
+      if (d < best) {
+        best = d;
+        code = l;
+      }
+    }
+    if (flat_row != nullptr) {
+      const uint32_t bit = j * BITS;
+      flat_row[bit >> 3] |= uint8_t(code << (bit & 7u));
+      if ((bit & 7u) + BITS > 8u) { flat_row[(bit >> 3) + 1] |= uint8_t(code >> (8u - (bit & 7u))); }
+    } else {
+      const uint32_t kk   = j % CPC;
+      const uint32_t bit  = kk * BITS;
+      const uint32_t word = bit >> 5;
+      const uint32_t off  = bit & 31u;
+      // dynamic register-array indexing is avoided with a small select chain
+#pragma unroll
+      for (uint32_t ww = 0; ww < 4; ww++) {
+        if (ww == word) { w[ww] |= code << off; }
+        if (ww == word + 1u && off + BITS > 32u) { w[ww] |= code >> (32u - off); }
+      }
+      if (kk == CPC - 1u || j == a.pq_dim - 1u) {
+        *reinterpret_cast<uint4*>(list_base + uint64_t(j / CPC) * 512u) = make_uint4(w[0], w[1], w[2], w[3]);
+        w[0] = w[1] = w[2] = w[3] = 0;
+      }
+    }
+  }
+}
+
+__global__ void unpack_contiguous_kernel(const uint8_t* __restrict__ list_data, uint32_t n_rows,
+                                         uint32_t offset, uint32_t pq_dim, uint32_t pq_bits,
+                                         uint8_t* __restrict__ out)
+{
+  const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= n_rows) { return; }
+  const uint32_t cpc       = 128u / pq_bits;
+  const uint32_t n_chunks  = (pq_dim + cpc - 1u) / cpc;
+  const uint32_t row_bytes = (pq_dim * pq_bits + 7u) / 8u;
+  const uint32_t i         = offset + r;
+  const uint8_t* ptr = list_data + uint64_t(i >> 5) * n_chunks * 512u + uint64_t(i & 31u) * 16u;
+  uint8_t* dst       = out + uint64_t(r) * row_bytes;
+  for (uint32_t b = 0; b < row_bytes; b++) { dst[b] = 0; }
+  const uint32_t mask = (1u << pq_bits) - 1u;
+  for (uint32_t j = 0; j < pq_dim; j++) {
+    const uint8_t* chunk = ptr + uint64_t(j / cpc) * 512u;
+    const uint32_t bit   = (j % cpc) * pq_bits;
+    uint32_t pairv       = chunk[bit >> 3];
+    if ((bit & 7u) + pq_bits > 8u) { pairv |= uint32_t(chunk[(bit >> 3) + 1]) << 8; }
+    const uint32_t code = (pairv >> (bit & 7u)) & mask;
+    const uint32_t ob   = j * pq_bits;
+    dst[ob >> 3] |= uint8_t(code << (ob & 7u));
+    if ((ob & 7u) + pq_bits > 8u) { dst[(ob >> 3) + 1] |= uint8_t(code >> (8u - (ob & 7u))); }
+  }
+}
+
+inline uint32_t blocks_for(uint64_t n, uint32_t block) { return uint32_t((n + block - 1) / block); }
+
+}  // namespace
+
+/* ---------------------------------------------------------------------------------------- */
+/* launchers                                                                                  */
+/* ---------------------------------------------------------------------------------------- */
+
+#define CUVS_LAUNCH_CHECK() CUVS_HIP_TRY(hipGetLastError())
+
+void launch_fill_u32(uint32_t* dst, uint32_t value, uint64_t n, hipStream_t stream)
+{
+  if (n == 0) { return; }
+  fill_u32_kernel<<<blocks_for(n, 256), 256, 0, stream>>>(dst, value, n);
+  CUVS_LAUNCH_CHECK();
+}
+
+void launch_map_queries(const void* queries, elem_type type, uint64_t n_elems, float* out,
+                        hipStream_t stream)
+{
+  if (n_elems == 0) { return; }
+  const uint32_t grid = blocks_for(n_elems, 256);
+  switch (type) {
+    case elem_type::f32:
+      map_queries_kernel<float><<<grid, 256, 0, stream>>>(static_cast<const float*>(queries), n_elems, out);
+      break;
+    case elem_type::f16:
+      map_queries_kernel<_Float16><<<grid, 256, 0, stream>>>(static_cast<const _Float16*>(queries), n_elems, out);
+      break;
+    case elem_type::i8:
+      map_queries_kernel<int8_t><<<grid, 256, 0, stream>>>(static_cast<const int8_t*>(queries), n_elems, out);
+      break;
+    case elem_type::u8:
+      map_queries_kernel<uint8_t><<<grid, 256, 0, stream>>>(static_cast<const uint8_t*>(queries), n_elems, out);
+      break;
+  }
+  CUVS_LAUNCH_CHECK();
+}
+
+void launch_coarse_scores(const float* qf, const float* centers, uint32_t n_queries,
+                          uint32_t n_lists, uint32_t dim, uint32_t dim_ext, bool ip_like,
+                          bool half_inputs, float* scores, hipStream_t stream)
+{
+  if (n_queries == 0 || n_lists == 0) { return; }
+  const float qnorm = ip_like ? 0.0f : -0.5f;
+  const float alpha = ip_like ? -1.0f : -2.0f;
+  dim3 grid(blocks_for(n_lists, kCoarseTile), blocks_for(n_queries, kCoarseTile));
+  if (half_inputs) {
+    coarse_scores_kernel<true><<<grid, kBlock, 0, stream>>>(qf, centers, n_queries, n_lists, dim, dim_ext, qnorm, alpha, scores);
+  } else {
+    coarse_scores_kernel<false><<<grid, kBlock, 0, stream>>>(qf, centers, n_queries, n_lists, dim, dim_ext, qnorm, alpha, scores);
+  }
+  CUVS_LAUNCH_CHECK();
+}
+
+void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_lists,
+                          uint32_t n_probes, uint32_t* probes, hipStream_t stream)
+{
+  if (n_queries == 0) { return; }
+  const uint32_t out_cap = next_pow2(n_probes);
+  const size_t smem      = size_t(out_cap) * 8;
+  CUVS_EXPECTS(smem <= 96 * 1024, "n_probes (%u) is too large for the probe selection kernel", n_probes);
+  if (smem > 32 * 1024) {
+    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(select_probes_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+  }
+  select_probes_kernel<<<n_queries, kBlock, smem, stream>>>(scores, n_lists, n_probes, out_cap, probes);
+  CUVS_LAUNCH_CHECK();
+}
+
+void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries, uint32_t dim,
+                   uint32_t rot_dim, bool identity, bool normalize, float* rot_q,
+                   hipStream_t stream)
+{
+  if (n_queries == 0) { return; }
+  const size_t smem = size_t(kRotQueries) * (dim + rot_dim) * sizeof(float);
+  CUVS_EXPECTS(smem <= 150 * 1024, "dim (%u) is too large for the rotation kernel", dim);
+  if (smem > 32 * 1024) {
+    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(rotate_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+  }
+  rotate_kernel<<<blocks_for(n_queries, kRotQueries), kBlock, smem, stream>>>(
+    qf, rotation_t, n_queries, dim, rot_dim, identity ? 1 : 0, normalize ? 1 : 0, rot_q);
+  CUVS_LAUNCH_CHECK();
+}
+
+void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
+                          uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
+                          uint32_t* n_samples, unsigned long long* stats, hipStream_t stream)
+{
+  if (n_queries == 0) { return; }
+  chunk_indices_kernel<<<n_queries, 64, 0, stream>>>(list_sizes, probes, n_probes, row_chunk_bytes,
+                                                     chunk_indices, n_samples, stats);
+  CUVS_LAUNCH_CHECK();
+}
+
+void launch_order_pairs(const uint32_t* probes, uint32_t n_pairs, uint32_t n_lists,
+                        uint32_t* counters, uint32_t* pair_order, hipStream_t stream)
+{
+  if (n_pairs == 0) { return; }
+  uint32_t* counts  = counters;
+  uint32_t* cursors = counters + n_lists;
+  launch_fill_u32(counts, 0, n_lists, stream);
+  pair_histogram_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(probes, n_pairs, counts);
+  CUVS_LAUNCH_CHECK();
+  exclusive_scan_kernel<<<1, kBlock, 0, stream>>>(counts, n_lists, cursors);
+  CUVS_LAUNCH_CHECK();
+  pair_scatter_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(probes, n_pairs, cursors, pair_order);
+  CUVS_LAUNCH_CHECK();
+}
+
+size_t scan_lds_bytes(const scan_args& a)
+{
+  const size_t elem = a.lut_dtype == CUDA_R_32F ? 4 : (a.lut_dtype == CUDA_R_16F ? 2 : 1);
+  const size_t lut  = ((size_t(a.pq_dim) << a.pq_bits) * elem + 15) & ~size_t(15);
+  const bool ip     = a.metric == int(DistanceType::InnerProduct) || a.metric == int(DistanceType::CosineExpanded);
+  const size_t diff = (size_t(a.rot_dim) * (ip ? 2 : 1) * 4 + 15) & ~size_t(15);
+  return lut + diff + (a.fused ? size_t(kCandCap) * 8 : 0) + 16;
+}
+
+namespace {
+
+template <int LUT, bool OUT_HALF, int BITS, bool FUSED>
+void launch_scan_instance(const scan_args& a, hipStream_t stream)
+{
+  const size_t smem = scan_lds_bytes(a);
+  auto kernel       = scan_kernel<LUT, OUT_HALF, BITS, FUSED>;
+  if (smem > 32 * 1024) {
+    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+  }
+  kernel<<<a.n_queries * a.n_probes, kBlock, smem, stream>>>(a);
+  CUVS_LAUNCH_CHECK();
+}
+
+template <int LUT, bool OUT_HALF, int BITS>
+void launch_scan_fused(const scan_args& a, hipStream_t stream)
+{
+  if (a.fused) {
+    launch_scan_instance<LUT, OUT_HALF, BITS, true>(a, stream);
+  } else {
+    launch_scan_instance<LUT, OUT_HALF, BITS, false>(a, stream);
+  }
+}
+
+template <int LUT, bool OUT_HALF>
+void launch_scan_bits(const scan_args& a, hipStream_t stream)
+{
+  switch (a.pq_bits) {
+    case 4: launch_scan_fused<LUT, OUT_HALF, 4>(a, stream); break;
+    case 5: launch_scan_fused<LUT, OUT_HALF, 5>(a, stream); break;
+    case 6: launch_scan_fused<LUT, OUT_HALF, 6>(a, stream); break;
+    case 7: launch_scan_fused<LUT, OUT_HALF, 7>(a, stream); break;
+    case 8: launch_scan_fused<LUT, OUT_HALF, 8>(a, stream); break;
+    default: fail("pq_bits must be within [4, 8]");
+  }
+}
+
+}  // namespace
+
+void launch_scan(const scan_args& a, hipStream_t stream)
+{
+  if (a.n_queries == 0) { return; }
+  CUVS_EXPECTS(!a.fused || a.k + kBlock <= kCandCap, "k (%u) is too large for the fused scan", a.k);
+  const bool ip = a.metric == int(DistanceType::InnerProduct) || a.metric == int(DistanceType::CosineExpanded);
+  int lut       = LUT_F32;
+  if (a.lut_dtype == CUDA_R_16F) { lut = LUT_F16; }
+  if (a.lut_dtype == CUDA_R_8U) { lut = ip ? LUT_FP8S : LUT_FP8U; }
+  if (a.out_half) {
+    switch (lut) {
+      case LUT_F16: launch_scan_bits<LUT_F16, true>(a, stream); break;
+      case LUT_FP8U: launch_scan_bits<LUT_FP8U, true>(a, stream); break;
+      case LUT_FP8S: launch_scan_bits<LUT_FP8S, true>(a, stream); break;
+      default: fail("fp16 internal distances need an fp16 or 8-bit lookup table");
+    }
+  } else {
+    switch (lut) {
+      case LUT_F32: launch_scan_bits<LUT_F32, false>(a, stream); break;
+      case LUT_F16: launch_scan_bits<LUT_F16, false>(a, stream); break;
+      case LUT_FP8U: launch_scan_bits<LUT_FP8U, false>(a, stream); break;
+      case LUT_FP8S: launch_scan_bits<LUT_FP8S, false>(a, stream); break;
+    }
+  }
+}
+
+void launch_merge(const merge_args& a, hipStream_t stream)
+{
+  if (a.n_queries == 0) { return; }
+  const uint32_t out_cap = next_pow2(a.k);
+  const size_t smem      = size_t(out_cap) * 8;
+  CUVS_EXPECTS(smem <= 96 * 1024, "k (%u) is too large for the merge kernel", a.k);
+  if (smem > 32 * 1024) {
+    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(merge_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+  }
+  merge_kernel<<<a.n_queries, kBlock, smem, stream>>>(a, out_cap);
+  CUVS_LAUNCH_CHECK();
+}
+
+void launch_normalize_rows(float* x, uint64_t n_rows, uint32_t dim, hipStream_t stream)
+{
+  if (n_rows == 0) { return; }
+  normalize_rows_kernel<<<blocks_for(n_rows, 256), 256, 0, stream>>>(x, n_rows, dim);
+  CUVS_LAUNCH_CHECK();
+}
+
+void launch_histogram(const uint32_t* labels, uint64_t n, uint32_t* counts, hipStream_t stream)
+{
+  if (n == 0) { return; }
+  histogram_kernel<<<blocks_for(n, 256), 256, 0, stream>>>(labels, n, counts);
+  CUVS_LAUNCH_CHECK();
+}
+
+void launch_relocate_lists(const uint8_t* old_codes, const int64_t* old_ids, uint8_t* new_codes,
+                           int64_t* new_ids, const uint64_t* old_row_offsets,
+                           const uint64_t* new_row_offsets, const uint32_t* old_sizes,
+                           uint32_t n_lists, uint32_t n_chunks, hipStream_t stream)
+{
+  if (n_lists == 0) { return; }
+  relocate_lists_kernel<<<n_lists, kBlock, 0, stream>>>(old_codes, old_ids, new_codes, new_ids,
+                                                        old_row_offsets, new_row_offsets, old_sizes,
+                                                        n_chunks);
+  CUVS_LAUNCH_CHECK();
+}
+
+namespace {
+template <int BITS>
+void launch_encode_bits(const encode_args& a, uint32_t grid, hipStream_t stream)
+{
+  if (a.per_cluster) {
+    encode_kernel<BITS, true><<<grid, kBlock, 0, stream>>>(a);
+  } else {
+    encode_kernel<BITS, false><<<grid, kBlock, 0, stream>>>(a);
+  }
+}
+}  // namespace
+
+void launch_encode(const encode_args& a, hipStream_t stream)
+{
+  if (a.n_rows == 0) { return; }
+  const uint32_t grid = blocks_for(a.n_rows, kBlock);
+  switch (a.pq_bits) {
+    case 4: launch_encode_bits<4>(a, grid, stream); break;
+    case 5: launch_encode_bits<5>(a, grid, stream); break;
+    case 6: launch_encode_bits<6>(a, grid, stream); break;
+    case 7: launch_encode_bits<7>(a, grid, stream); break;
+    case 8: launch_encode_bits<8>(a, grid, stream); break;
+    default: fail("pq_bits must be within [4, 8]");
+  }
+  CUVS_LAUNCH_CHECK();
+}
+
+void launch_unpack_contiguous(const uint8_t* list_data, uint32_t n_rows, uint32_t offset,
+                              uint32_t pq_dim, uint32_t pq_bits, uint8_t* out, hipStream_t stream)
+{
+  if (n_rows == 0) { return; }
+  unpack_contiguous_kernel<<<blocks_for(n_rows, 256), 256, 0, stream>>>(list_data, n_rows, offset,
+                                                                        pq_dim, pq_bits, out);
+  CUVS_LAUNCH_CHECK();
+}
+
+}  // namespace cuvs::neighbors::ivf_pq::detail

@@ -1,0 +1,426 @@
+/*
+ * Host driver of IVF-PQ search.  Validation, probe-count clamping, the max_samples bound and the
+ * score / lookup-table type rules follow cuVS detail::search and ivfpq_search::fun
+ * (cpp/src/neighbors/ivf_pq/ivf_pq_search.cuh:878-1048, :681-743); batching and the kernel
+ * plan are this library's own (results do not depend on how queries are batched).
+ */
+#include "detail.hpp"
+
+#include <algorithm>
+#include <limits>
+
+namespace cuvs {
+
+struct resources::profile_state {
+  hipEvent_t ev[5]            = {};
+  unsigned long long* d_stats = nullptr;
+};
+
+void destroy_profile_state(resources::profile_state* p)
+{
+  if (p == nullptr) { return; }
+  for (auto& e : p->ev) {
+    if (e != nullptr) { (void)hipEventDestroy(e); }
+  }
+  if (p->d_stats != nullptr) { (void)hipFree(p->d_stats); }
+  delete p;
+}
+
+}  // namespace cuvs
+
+namespace cuvs::neighbors::ivf_pq {
+
+namespace {
+
+using detail::index_impl;
+
+constexpr uint32_t kMaxFusedK = 256;   // larger k dumps all scores and selects afterwards
+constexpr uint32_t kMaxK      = 8192;  // bound of the per-query selection buffer in LDS
+constexpr size_t kMaxLds      = 160 * 1024;
+
+/** A pointer is usable by kernels when HIP knows it as device, managed or pinned host memory
+ *  (role of utils::check_pointer_residency, detail/ann_utils.cuh). */
+bool device_accessible(const void* p)
+{
+  hipPointerAttribute_t attr;
+  const hipError_t st = hipPointerGetAttributes(&attr, p);
+  if (st != hipSuccess) {
+    (void)hipGetLastError();  // clear the sticky error left by an unregistered host pointer
+    return false;
+  }
+  return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged ||
+         attr.type == hipMemoryTypeHost || attr.type == hipMemoryTypeArray;
+}
+
+size_t workspace_budget(const cuvs::resources& res)
+{
+  size_t free_b = 0, total_b = 0;
+  CUVS_HIP_TRY(hipMemGetInfo(&free_b, &total_b));
+  // what is already cached in the workspace counts as available
+  size_t budget = (free_b + res.workspace_capacity()) / 10 * 4;
+  if (res.workspace_limit() != 0) { budget = std::min(budget, res.workspace_limit()); }
+  return std::max(budget, size_t(64) << 20);
+}
+
+struct plan {
+  uint32_t n_probes;
+  uint32_t max_samples;
+  bool fused;
+  uint32_t batch;
+  size_t per_query_bytes;
+  size_t fixed_bytes;
+};
+
+size_t a256(size_t v) { return (v + 255) & ~size_t(255); }
+
+plan make_plan(const cuvs::resources& res, const search_params& params, const index_impl& ix,
+               uint32_t n_queries, uint32_t k)
+{
+  plan p{};
+  p.n_probes = std::min<uint32_t>(params.n_probes, ix.n_lists);
+  {
+    // ivf_pq_search.cuh:934-940
+    const int64_t ms = ((ix.accum_sorted_sizes[p.n_probes] + 127) / 128) * 128;
+    CUVS_EXPECTS(ms <= int64_t(std::numeric_limits<uint32_t>::max()),
+                 "The maximum sample size is too big.");
+    p.max_samples = uint32_t(ms);
+  }
+  p.fused = k <= kMaxFusedK;
+  const size_t P = p.n_probes;
+  p.per_query_bytes = size_t(ix.dim) * 4 + size_t(ix.n_lists) * 4 + size_t(ix.rot_dim) * 4 +
+                      P * 4 * 3 + 16 +
+                      (p.fused ? P * k * 8 : size_t(p.max_samples) * 4);
+  p.fixed_bytes = a256(size_t(ix.n_lists) * 8 + 16) + 16 * 256;
+  const size_t budget = workspace_budget(res);
+  size_t b = budget > p.fixed_bytes ? (budget - p.fixed_bytes) / (p.per_query_bytes + 64) : 1;
+  b        = std::max<size_t>(b, 1);
+  b        = std::min<size_t>(b, std::max<uint32_t>(params.max_internal_batch_size, 1u));
+  b        = std::min<size_t>(b, n_queries);
+  // keep the pair count of a batch within uint32 indexing
+  while (b > 1 && b * P >= (size_t(1) << 31)) { b /= 2; }
+  p.batch = uint32_t(b);
+  return p;
+}
+
+void validate(const search_params& params, const index_impl& ix, int64_t k)
+{
+  // ivf_pq_search.cuh:901-923
+  CUVS_EXPECTS(params.internal_distance_dtype == CUDA_R_16F ||
+                 params.internal_distance_dtype == CUDA_R_32F,
+               "internal_distance_dtype must be either CUDA_R_16F or CUDA_R_32F");
+  CUVS_EXPECTS(params.lut_dtype == CUDA_R_16F || params.lut_dtype == CUDA_R_32F ||
+                 params.lut_dtype == CUDA_R_8U,
+               "lut_dtype must be CUDA_R_16F, CUDA_R_32F or CUDA_R_8U");
+  CUVS_EXPECTS(k > 0, "parameter `k` in top-k must be positive.");
+  CUVS_EXPECTS(k <= ix.size,
+               "parameter `k` (%lld) in top-k must not be larger that the total size of the index "
+               "(%lld)",
+               static_cast<long long>(k), static_cast<long long>(ix.size));
+  CUVS_EXPECTS(params.n_probes > 0,
+               "n_probes (number of clusters to probe in the search) must be positive.");
+  // ivf_pq_search.cuh:699-707
+  CUVS_EXPECTS(!(params.internal_distance_dtype == CUDA_R_16F && params.lut_dtype == CUDA_R_32F),
+               "Unexpected lut_dtype / internal_distance_dtype combination (%d, %d). Size of the "
+               "internal_distance_dtype should be not smaller than the size of the lut_dtype.",
+               int(params.lut_dtype), int(params.internal_distance_dtype));
+  CUVS_EXPECTS(params.coarse_search_dtype == CUDA_R_32F || params.coarse_search_dtype == CUDA_R_16F,
+               "Unsupported coarse_search_dtype (only CUDA_R_32F and CUDA_R_16F are supported)");
+  CUVS_EXPECTS(k <= kMaxK, "parameter `k` (%lld) must not exceed %u", static_cast<long long>(k),
+               kMaxK);
+}
+
+float scaling_factor(elem_type t)
+{
+  // utils::config<T>::kDivisor / utils::config<float>::kDivisor (ivf_pq_search.cuh:1043)
+  return t == elem_type::u8 ? 256.0f : (t == elem_type::i8 ? 128.0f : 1.0f);
+}
+
+size_t elem_size(elem_type t) { return t == elem_type::f32 ? 4 : (t == elem_type::f16 ? 2 : 1); }
+
+struct coarse_buffers {
+  float* qf;
+  float* scores;
+  uint32_t* probes;
+};
+
+/** mapping + centre scores + probe selection for one batch */
+void run_coarse(const cuvs::resources& res, const search_params& params, const index_impl& ix,
+                const void* queries, elem_type type, uint32_t nq, uint32_t n_probes,
+                const coarse_buffers& b)
+{
+  hipStream_t s     = res.stream();
+  const bool ip     = ix.metric == detail::DistanceType::InnerProduct ||
+                  ix.metric == detail::DistanceType::CosineExpanded;
+  detail::launch_map_queries(queries, type, uint64_t(nq) * ix.dim, b.qf, s);
+  detail::launch_coarse_scores(b.qf, ix.centers.as<float>(), nq, ix.n_lists, ix.dim, ix.dim_ext,
+                               ip, params.coarse_search_dtype == CUDA_R_16F, b.scores, s);
+  detail::launch_select_probes(b.scores, nq, ix.n_lists, n_probes, b.probes, s);
+}
+
+}  // namespace
+
+void select_clusters(cuvs::resources const& res_c,
+                     const search_params& params,
+                     const index<int64_t>& idx,
+                     const void* queries,
+                     elem_type type,
+                     int64_t n_queries,
+                     uint32_t* clusters_to_probe)
+{
+  auto& res      = const_cast<cuvs::resources&>(res_c);
+  const auto& ix = *idx.impl();
+  CUVS_EXPECTS(params.n_probes > 0,
+               "n_probes (number of clusters to probe in the search) must be positive.");
+  CUVS_EXPECTS(params.coarse_search_dtype == CUDA_R_32F || params.coarse_search_dtype == CUDA_R_16F,
+               "Unsupported coarse_search_dtype (only CUDA_R_32F and CUDA_R_16F are supported)");
+  CUVS_EXPECTS(device_accessible(queries) && device_accessible(clusters_to_probe),
+               "all pointers must be accessible from the device.");
+  const uint32_t P       = std::min<uint32_t>(params.n_probes, ix.n_lists);
+  const size_t per_query = size_t(ix.dim) * 4 + size_t(ix.n_lists) * 4 + 64;
+  size_t batch           = std::max<size_t>(1, workspace_budget(res) / per_query);
+  batch                  = std::min<size_t>(batch, size_t(n_queries));
+  batch                  = std::min<size_t>(batch, 65535u * 64u);
+  res.reset_workspace();
+  res.reserve_workspace(a256(batch * ix.dim * 4) + a256(batch * size_t(ix.n_lists) * 4) + 1024);
+  coarse_buffers b;
+  b.qf     = static_cast<float*>(res.workspace_alloc(batch * ix.dim * 4));
+  b.scores = static_cast<float*>(res.workspace_alloc(batch * size_t(ix.n_lists) * 4));
+  for (int64_t q0 = 0; q0 < n_queries; q0 += int64_t(batch)) {
+    const uint32_t nq = uint32_t(std::min<int64_t>(int64_t(batch), n_queries - q0));
+    b.probes          = clusters_to_probe + q0 * P;
+    run_coarse(res, params, ix,
+               static_cast<const char*>(queries) + size_t(q0) * ix.dim * elem_size(type), type, nq,
+               P, b);
+  }
+  res.reset_workspace();
+}
+
+void search(cuvs::resources const& res_c,
+            const search_params& params,
+            const index<int64_t>& idx,
+            const void* queries,
+            elem_type type,
+            int64_t n_queries,
+            int64_t query_dim,
+            int64_t* neighbors,
+            float* distances,
+            int64_t k64,
+            const cuvs::neighbors::filtering::base_filter& sample_filter)
+{
+  auto& res      = const_cast<cuvs::resources&>(res_c);
+  const auto& ix = *idx.impl();
+
+  const uint32_t* filter_bits = nullptr;
+  int64_t filter_nbits        = 0;
+  if (dynamic_cast<const filtering::none_sample_filter*>(&sample_filter) == nullptr) {
+    auto* bf = dynamic_cast<const filtering::bitset_filter*>(&sample_filter);
+    CUVS_EXPECTS(bf != nullptr, "Unsupported sample filter type");  // ivf_pq_search.cuh:1126-1133
+    filter_bits  = bf->bits;
+    filter_nbits = bf->n_bits;
+    CUVS_EXPECTS(filter_bits != nullptr && device_accessible(filter_bits),
+                 "the filter bitset must be accessible from the device.");
+  }
+
+  // ivf_pq_search.cuh:1088-1096
+  CUVS_EXPECTS(query_dim == int64_t(ix.dim),
+               "Number of query dimensions should equal number of dimensions in the index.");
+  validate(params, ix, k64);
+  if (n_queries == 0) { return; }
+  CUVS_EXPECTS(n_queries <= int64_t(std::numeric_limits<uint32_t>::max()), "too many queries");
+  CUVS_EXPECTS(device_accessible(queries) && device_accessible(neighbors) &&
+                 device_accessible(distances),
+               "all pointers must be accessible from the device.");
+
+  const uint32_t k  = uint32_t(k64);
+  const plan pl     = make_plan(res, params, ix, uint32_t(n_queries), k);
+  const uint32_t P  = pl.n_probes;
+  const uint32_t Qb = pl.batch;
+  hipStream_t s     = res.stream();
+
+  detail::scan_args sa{};
+  sa.n_probes     = P;
+  sa.k            = k;
+  sa.max_samples  = pl.max_samples;
+  sa.rot_dim      = ix.rot_dim;
+  sa.pq_dim       = ix.pq_dim;
+  sa.pq_len       = ix.pq_len;
+  sa.pq_bits      = ix.pq_bits;
+  sa.metric       = int(ix.metric);
+  sa.per_cluster  = ix.codebook_kind == codebook_gen::PER_CLUSTER;
+  sa.lut_dtype    = params.lut_dtype;
+  sa.out_half     = params.internal_distance_dtype == CUDA_R_16F;
+  sa.fused        = pl.fused;
+  sa.centers_rot  = ix.centers_rot.as<float>();
+  sa.pq_centers   = ix.pq_centers.as<float>();
+  sa.data_ptrs    = ix.data_ptrs.as<const uint8_t*>();
+  sa.inds_ptrs    = ix.inds_ptrs.as<const int64_t*>();
+  sa.list_sizes   = ix.list_sizes.as<uint32_t>();
+  sa.filter_bits  = filter_bits;
+  sa.filter_nbits = filter_nbits;
+  const size_t lds = detail::scan_lds_bytes(sa);
+  CUVS_EXPECTS(lds <= kMaxLds,
+               "the lookup table (pq_dim = %u, pq_bits = %u, lut_dtype = %d) needs %zu bytes of LDS, "
+               "more than the %zu available; use a smaller lut_dtype",
+               ix.pq_dim, ix.pq_bits, int(params.lut_dtype), lds, kMaxLds);
+
+  /* workspace carve-up for one batch */
+  res.reset_workspace();
+  res.reserve_workspace(pl.fixed_bytes + size_t(Qb) * (pl.per_query_bytes + 64) + 16 * 256);
+  auto* qf        = static_cast<float*>(res.workspace_alloc(size_t(Qb) * ix.dim * 4));
+  auto* scores    = static_cast<float*>(res.workspace_alloc(size_t(Qb) * ix.n_lists * 4));
+  auto* rot_q     = static_cast<float*>(res.workspace_alloc(size_t(Qb) * ix.rot_dim * 4));
+  auto* probes    = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * P * 4));
+  auto* chunk     = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * P * 4));
+  auto* order     = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * P * 4));
+  auto* n_samples = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * 4));
+  auto* kth       = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * 4));
+  auto* counters  = static_cast<uint32_t*>(res.workspace_alloc(size_t(ix.n_lists) * 8 + 16));
+  unsigned long long* keys = nullptr;
+  float* all_scores        = nullptr;
+  if (pl.fused) {
+    keys = static_cast<unsigned long long*>(res.workspace_alloc(size_t(Qb) * P * k * 8));
+  } else {
+    all_scores = static_cast<float*>(res.workspace_alloc(size_t(Qb) * pl.max_samples * 4));
+  }
+
+  /* profiling state */
+  const bool prof = res.profiling;
+  unsigned long long* d_stats = nullptr;
+  if (prof) {
+    if (res.prof == nullptr) {
+      res.prof = new cuvs::resources::profile_state();
+      for (auto& e : res.prof->ev) { CUVS_HIP_TRY(hipEventCreate(&e)); }
+      CUVS_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&res.prof->d_stats), 16));
+    }
+    d_stats = res.prof->d_stats;
+    detail::launch_fill_u32(reinterpret_cast<uint32_t*>(d_stats), 0, 4, s);
+    res.last_profile           = cuvs::search_profile{};
+    res.last_profile.n_queries = uint32_t(n_queries);
+    res.last_profile.n_probes  = P;
+    res.last_profile.k         = k;
+  }
+  auto mark = [&](int i) {
+    if (prof) { CUVS_HIP_TRY(hipEventRecord(res.prof->ev[i], s)); }
+  };
+
+  const bool cosine = ix.metric == detail::DistanceType::CosineExpanded;
+  for (int64_t q0 = 0; q0 < n_queries; q0 += Qb) {
+    const uint32_t nq = uint32_t(std::min<int64_t>(Qb, n_queries - q0));
+    const void* qptr  = static_cast<const char*>(queries) + size_t(q0) * ix.dim * elem_size(type);
+
+    mark(0);
+    run_coarse(res, params, ix, qptr, type, nq, P, coarse_buffers{qf, scores, probes});
+    mark(1);
+    detail::launch_rotate(qf, ix.rotation_t.as<float>(), nq, ix.dim, ix.rot_dim,
+                          ix.rotation_is_identity, cosine, rot_q, s);
+    detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
+                                 ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, s);
+    detail::launch_order_pairs(probes, nq * P, ix.n_lists, counters, order, s);
+    if (pl.fused) { detail::launch_fill_u32(kth, 0xFFFFFFFFu, nq, s); }
+    mark(2);
+
+    sa.n_queries     = nq;
+    sa.rot_q         = rot_q;
+    sa.probes        = probes;
+    sa.chunk_indices = chunk;
+    sa.pair_order    = order;
+    sa.query_kth     = kth;
+    sa.out_keys      = keys;
+    sa.out_scores    = all_scores;
+    detail::launch_scan(sa, s);
+    mark(3);
+
+    detail::merge_args ma{};
+    ma.n_queries     = nq;
+    ma.n_probes      = P;
+    ma.k             = k;
+    ma.max_samples   = pl.max_samples;
+    ma.fused         = pl.fused;
+    ma.metric        = int(ix.metric);
+    ma.scaling       = scaling_factor(type);
+    ma.in_keys       = keys;
+    ma.in_scores     = all_scores;
+    ma.n_samples     = n_samples;
+    ma.probes        = probes;
+    ma.chunk_indices = chunk;
+    ma.inds_ptrs     = ix.inds_ptrs.as<const int64_t*>();
+    ma.neighbors     = neighbors + q0 * k;
+    ma.distances     = distances + q0 * k;
+    detail::launch_merge(ma, s);
+    mark(4);
+
+    if (prof) {
+      CUVS_HIP_TRY(hipEventSynchronize(res.prof->ev[4]));
+      float ms[4] = {0, 0, 0, 0};
+      for (int i = 0; i < 4; i++) {
+        CUVS_HIP_TRY(hipEventElapsedTime(&ms[i], res.prof->ev[i], res.prof->ev[i + 1]));
+      }
+      auto& lp = res.last_profile;
+      lp.coarse_ms += ms[0];
+      lp.rotate_ms += ms[1];
+      lp.scan_ms += ms[2];
+      lp.merge_ms += ms[3];
+      lp.total_ms += ms[0] + ms[1] + ms[2] + ms[3];
+      lp.n_scan_launches += 1;
+    }
+  }
+  if (prof) {
+    unsigned long long h[2] = {0, 0};
+    CUVS_HIP_TRY(hipMemcpyAsync(h, d_stats, 16, hipMemcpyDeviceToHost, s));
+    CUVS_HIP_TRY(hipStreamSynchronize(s));
+    res.last_profile.scan_bytes = h[0];
+    res.last_profile.scan_rows  = h[1];
+  }
+  res.reset_workspace();
+}
+
+template <typename T>
+struct elem_of;
+template <>
+struct elem_of<float> {
+  static constexpr elem_type value = elem_type::f32;
+};
+template <>
+struct elem_of<_Float16> {
+  static constexpr elem_type value = elem_type::f16;
+};
+template <>
+struct elem_of<int8_t> {
+  static constexpr elem_type value = elem_type::i8;
+};
+template <>
+struct elem_of<uint8_t> {
+  static constexpr elem_type value = elem_type::u8;
+};
+
+template <typename T>
+void search(cuvs::resources const& res,
+            const search_params& params,
+            const index<int64_t>& idx,
+            device_matrix_view<const T> queries,
+            device_matrix_view<int64_t> neighbors,
+            device_matrix_view<float> distances,
+            const cuvs::neighbors::filtering::base_filter& sample_filter)
+{
+  // search_with_filtering (ivf_pq_search.cuh:1079-1108)
+  CUVS_EXPECTS(
+    queries.extent(0) == neighbors.extent(0) && queries.extent(0) == distances.extent(0),
+    "Number of rows in output neighbors and distances matrices must equal the number of queries.");
+  CUVS_EXPECTS(neighbors.extent(1) == distances.extent(1),
+               "Number of columns in output neighbors and distances matrices must equal k");
+  search(res, params, idx, queries.data_handle(), elem_of<T>::value, queries.extent(0),
+         queries.extent(1), neighbors.data_handle(), distances.data_handle(), neighbors.extent(1),
+         sample_filter);
+}
+
+#define INSTANTIATE_SEARCH(T)                                                              \
+  template void search<T>(cuvs::resources const&, const search_params&, const index<int64_t>&, \
+                          device_matrix_view<const T>, device_matrix_view<int64_t>,        \
+                          device_matrix_view<float>,                                       \
+                          const cuvs::neighbors::filtering::base_filter&);
+INSTANTIATE_SEARCH(float)
+INSTANTIATE_SEARCH(_Float16)
+INSTANTIATE_SEARCH(int8_t)
+INSTANTIATE_SEARCH(uint8_t)
+
+}  // namespace cuvs::neighbors::ivf_pq

@@ -1,0 +1,38 @@
+"""Mirror of cuvs.common.Resources (python/cuvs/cuvs/common/resources.pyx): owns a cuvsResources_t."""
+import ctypes as C
+
+from ._lib import check, lib
+
+
+class Resources:
+    def __init__(self, stream=None):
+        self._h = C.c_size_t(0)
+        check(lib().cuvsResourcesCreate(C.byref(self._h)))
+        if stream is not None:
+            self.set_stream(stream)
+
+    def set_stream(self, stream):
+        """`stream` is a raw hipStream_t value or an object with a `cuda_stream` attribute."""
+        raw = getattr(stream, "cuda_stream", stream)
+        check(lib().cuvsStreamSet(self._h, C.c_void_p(raw)))
+
+    def use_torch_current_stream(self):
+        import torch
+        self.set_stream(torch.cuda.current_stream().cuda_stream)
+
+    def sync(self):
+        check(lib().cuvsStreamSync(self._h))
+
+    def get_c_obj(self):
+        return self._h
+
+    def enable_profiling(self, on=True):
+        check(lib().cuvsAmdIvfPqProfilingEnable(self._h, bool(on)))
+
+    def __del__(self):
+        try:
+            if self._h.value:
+                lib().cuvsResourcesDestroy(self._h)
+                self._h = C.c_size_t(0)
+        except Exception:
+            pass

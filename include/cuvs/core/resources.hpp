@@ -1,0 +1,96 @@
+/*
+ * Minimal stand-ins for the RAFT types that appear in the signatures of the cuVS C++ search API
+ * (raft::resources, raft::device_matrix_view, raft::logic_error): a resources handle that owns a
+ * HIP stream choice and a reusable device workspace, and non-owning row-major views.
+ */
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace cuvs {
+
+/** Error type thrown by every C++ entry point (role of raft::logic_error / RAFT_EXPECTS). */
+struct logic_error : public std::runtime_error {
+  explicit logic_error(const std::string& msg) : std::runtime_error(msg) {}
+};
+
+/** Non-owning row-major 2-D view (role of raft::device_matrix_view<T, int64_t, row_major>). */
+template <typename T>
+struct device_matrix_view {
+  T* data      = nullptr;
+  int64_t rows = 0;
+  int64_t cols = 0;
+  T* data_handle() const { return data; }
+  int64_t extent(int i) const { return i == 0 ? rows : cols; }
+};
+
+template <typename T>
+device_matrix_view<T> make_device_matrix_view(T* data, int64_t rows, int64_t cols)
+{
+  return device_matrix_view<T>{data, rows, cols};
+}
+
+/** Per-stage timing of a search (filled when profiling is enabled on the resources). */
+struct search_profile {
+  uint32_t n_queries       = 0;
+  uint32_t n_probes        = 0;
+  uint32_t k               = 0;
+  uint32_t n_scan_launches = 0;
+  float coarse_ms          = 0;
+  float rotate_ms          = 0;
+  float scan_ms            = 0;
+  float merge_ms           = 0;
+  float total_ms           = 0;
+  uint64_t scan_bytes      = 0;
+  uint64_t scan_rows       = 0;
+};
+
+/**
+ * One stream plus a cached device workspace (role of raft::resources with a workspace memory
+ * resource).  Not thread-safe: use one handle per host thread; an index may be shared.
+ */
+class resources {
+ public:
+  resources();
+  ~resources();
+  resources(const resources&)            = delete;
+  resources& operator=(const resources&) = delete;
+
+  hipStream_t stream() const { return stream_; }
+  void set_stream(hipStream_t s) { stream_ = s; }
+  void sync() const;
+  int device_id() const { return device_; }
+
+  /** Upper bound for the cached workspace in bytes (0 = no explicit bound). */
+  void set_workspace_limit(size_t bytes) { workspace_limit_ = bytes; }
+  size_t workspace_limit() const { return workspace_limit_; }
+
+  /** Bump allocation out of the cached workspace; valid until the next reset_workspace(). */
+  void* workspace_alloc(size_t bytes);
+  /** Make sure the workspace can serve `bytes` in total before the first allocation of a call. */
+  void reserve_workspace(size_t bytes);
+  void reset_workspace() { workspace_used_ = 0; }
+  size_t workspace_capacity() const { return workspace_capacity_; }
+
+  bool profiling = false;
+  struct profile_state;
+  profile_state* prof = nullptr;  // lazily created event set
+  search_profile last_profile;
+
+ private:
+  int device_             = 0;
+  hipStream_t stream_     = nullptr;
+  void* workspace_        = nullptr;
+  size_t workspace_capacity_ = 0;
+  size_t workspace_used_  = 0;
+  size_t workspace_limit_ = 0;
+  std::vector<void*> retired_;  // outgrown workspaces, released at destruction / next sync point
+};
+
+}  // namespace cuvs

@@ -1,0 +1,216 @@
+/*
+ * C++ API of the IVF-PQ search path for AMD Instinct MI355X (gfx950).
+ *
+ * Same namespace, type names, field names, defaults and argument meaning as the cuVS header
+ * cpp/include/cuvs/neighbors/ivf_pq.hpp (index_params :47-151, search_params :160-213,
+ * index :475-675, search overloads :1821-1963, extend, build from a precomputed model), with
+ * cuvs::resources / cuvs::device_matrix_view standing in for the RAFT types.
+ */
+#pragma once
+
+#include <cuvs/core/data_type.h>
+#include <cuvs/core/resources.hpp>
+
+#include <cstdint>
+#include <memory>
+#include <string>
+
+namespace cuvs::distance {
+/** Numeric values of cuvs::distance::DistanceType (cpp/include/cuvs/distance/distance.hpp). */
+enum class DistanceType : int {
+  L2Expanded     = 0,
+  L2SqrtExpanded = 1,
+  CosineExpanded = 2,
+  InnerProduct   = 6,
+};
+}  // namespace cuvs::distance
+
+namespace cuvs::neighbors {
+
+/** cpp/include/cuvs/neighbors/common.hpp:125-132 */
+struct index_params {
+  cuvs::distance::DistanceType metric = cuvs::distance::DistanceType::L2Expanded;
+  float metric_arg                    = 2.0f;
+};
+struct search_params {};
+
+namespace filtering {
+/** cpp/include/cuvs/neighbors/common.hpp:1342-1480 -- only these two filters reach IVF-PQ search. */
+struct base_filter {
+  virtual ~base_filter() = default;
+};
+struct none_sample_filter : public base_filter {};
+/** Bit i set = source id i may be returned. `bits` is a device array of ceil(n_bits / 32) words. */
+struct bitset_filter : public base_filter {
+  const uint32_t* bits = nullptr;
+  int64_t n_bits       = 0;
+  bitset_filter(const uint32_t* b, int64_t n) : bits(b), n_bits(n) {}
+};
+}  // namespace filtering
+
+namespace ivf_pq {
+
+enum class codebook_gen { PER_SUBSPACE = 0, PER_CLUSTER = 1 };
+enum class list_layout { FLAT = 0, INTERLEAVED = 1 };
+
+constexpr uint32_t kIndexGroupSize   = 32;  // rows interleaved per group  (ivf_pq.hpp:222)
+constexpr uint32_t kIndexGroupVecLen = 16;  // bytes per interleaved chunk (ivf_pq.hpp:224)
+
+struct index_params : cuvs::neighbors::index_params {
+  uint32_t n_lists                      = 1024;
+  uint32_t kmeans_n_iters               = 20;
+  double kmeans_trainset_fraction       = 0.5;
+  uint32_t pq_bits                      = 8;
+  uint32_t pq_dim                       = 0;
+  codebook_gen codebook_kind            = codebook_gen::PER_SUBSPACE;
+  list_layout codes_layout              = list_layout::INTERLEAVED;
+  bool force_random_rotation            = false;
+  bool conservative_memory_allocation   = false;
+  bool add_data_on_build                = true;
+  uint32_t max_train_points_per_pq_code = 256;
+};
+
+struct search_params : cuvs::neighbors::search_params {
+  uint32_t n_probes                 = 20;
+  int lut_dtype                     = CUDA_R_32F;
+  int internal_distance_dtype       = CUDA_R_32F;
+  double preferred_shmem_carveout   = 1.0;
+  int coarse_search_dtype           = CUDA_R_32F;
+  uint32_t max_internal_batch_size  = 4096;
+};
+
+namespace detail {
+struct index_impl;
+}
+
+/** Element type of query / dataset rows. */
+enum class elem_type : int { f32 = 0, f16 = 1, i8 = 2, u8 = 3 };
+
+/**
+ * IVF-PQ index contents in device memory: coarse centres with fused norms, rotation matrix,
+ * PQ codebooks, and per-list interleaved codes + source ids.  Only IdxT = int64_t exists.
+ */
+template <typename IdxT>
+class index {
+  static_assert(sizeof(IdxT) == 8, "only int64_t ids are supported");
+
+ public:
+  index();
+  ~index();
+  index(index&&) noexcept;
+  index& operator=(index&&) noexcept;
+
+  int64_t size() const;
+  uint32_t dim() const;
+  uint32_t dim_ext() const;
+  uint32_t rot_dim() const;
+  uint32_t pq_bits() const;
+  uint32_t pq_dim() const;
+  uint32_t pq_len() const;
+  uint32_t pq_book_size() const;
+  uint32_t n_lists() const;
+  cuvs::distance::DistanceType metric() const;
+  codebook_gen codebook_kind() const;
+  list_layout codes_layout() const;
+  bool conservative_memory_allocation() const;
+
+  const float* centers() const;          // [n_lists, dim_ext]
+  const float* centers_rot() const;      // [n_lists, rot_dim]
+  const float* rotation_matrix() const;  // [rot_dim, dim]
+  const float* pq_centers() const;       // [pq_dim | n_lists, pq_len, pq_book_size]
+  const uint32_t* list_sizes() const;    // device [n_lists]
+  const uint8_t* const* data_ptrs() const;
+  const IdxT* const* inds_ptrs() const;
+  /** Host prefix sums of list sizes sorted in descending order, [n_lists + 1]. */
+  const int64_t* accum_sorted_sizes() const;
+
+  detail::index_impl* impl() const { return impl_.get(); }
+
+ private:
+  std::unique_ptr<detail::index_impl> impl_;
+};
+
+/** Index from a trained model (cuVS: build(res, params, dim, pq_centers, centers, centers_rot,
+ *  rotation_matrix), cpp/include/cuvs/neighbors/ivf_pq.hpp).  All inputs are device float32;
+ *  they are copied. */
+index<int64_t> build(cuvs::resources const& res,
+                     const index_params& params,
+                     uint32_t dim,
+                     const float* pq_centers,
+                     const float* centers,
+                     const float* centers_rot,
+                     const float* rotation_matrix);
+
+/** Encode and append rows.  `new_vectors` and `new_indices` are device pointers; a null
+ *  `new_indices` numbers the rows consecutively from the current size.  A non-null `labels`
+ *  (device uint32 [n]) overrides the nearest-centre assignment. */
+void extend(cuvs::resources const& res,
+            const void* new_vectors,
+            elem_type type,
+            int64_t n_rows,
+            const int64_t* new_indices,
+            index<int64_t>* idx,
+            const uint32_t* labels = nullptr);
+
+template <typename T>
+void extend(cuvs::resources const& res,
+            device_matrix_view<const T> new_vectors,
+            const int64_t* new_indices,
+            index<int64_t>* idx);
+
+/** Labels and bit-contiguous codes of rows, without modifying the index (cuVS: transform). */
+void transform(cuvs::resources const& res,
+               const index<int64_t>& idx,
+               const void* vectors,
+               elem_type type,
+               int64_t n_rows,
+               uint32_t* labels_out,
+               uint8_t* codes_out);
+
+/** cuVS: ivf_pq::search (cpp/include/cuvs/neighbors/ivf_pq.hpp:1821-1963), T in
+ *  {float, _Float16, int8_t, uint8_t}. */
+template <typename T>
+void search(cuvs::resources const& res,
+            const search_params& params,
+            const index<int64_t>& idx,
+            device_matrix_view<const T> queries,
+            device_matrix_view<int64_t> neighbors,
+            device_matrix_view<float> distances,
+            const cuvs::neighbors::filtering::base_filter& sample_filter =
+              cuvs::neighbors::filtering::none_sample_filter{});
+
+/** Type-erased form used by the C layer. */
+void search(cuvs::resources const& res,
+            const search_params& params,
+            const index<int64_t>& idx,
+            const void* queries,
+            elem_type type,
+            int64_t n_queries,
+            int64_t query_dim,
+            int64_t* neighbors,
+            float* distances,
+            int64_t k,
+            const cuvs::neighbors::filtering::base_filter& sample_filter);
+
+/** Coarse step only: clusters_to_probe is device uint32 [n_queries, min(n_probes, n_lists)]. */
+void select_clusters(cuvs::resources const& res,
+                     const search_params& params,
+                     const index<int64_t>& idx,
+                     const void* queries,
+                     elem_type type,
+                     int64_t n_queries,
+                     uint32_t* clusters_to_probe);
+
+/** cuVS helpers::codepacker::unpack_contiguous_list_data. */
+void unpack_contiguous_list_data(cuvs::resources const& res,
+                                 const index<int64_t>& idx,
+                                 uint8_t* out_codes,
+                                 uint32_t n_rows,
+                                 uint32_t label,
+                                 uint32_t offset);
+
+void serialize(cuvs::resources const& res, const std::string& filename, const index<int64_t>& idx);
+void deserialize(cuvs::resources const& res, const std::string& filename, index<int64_t>* idx);
+
+}  // namespace ivf_pq
+}  // namespace cuvs::neighbors

@@ -1,0 +1,263 @@
+"""GPU parity: the HIP path through the C ABI against the CPU oracle on the same index and queries.
+
+Bar: probe lists and stored codes bit-exact; neighbour ids equal except at distance ties; distances
+within 1e-5 relative for an fp32 lookup table and 2e-3 for fp16 / 8-bit tables.  Because the
+kernels use the same operation order as the oracle, most cases are in fact checked for exact
+equality (`exact=True`).
+"""
+import numpy as np
+import pytest
+import torch
+
+import gpu_helpers as G
+import helpers as H
+from cuvs_amd import ivf_pq
+from cuvs_amd._lib import CuvsError
+
+pytestmark = pytest.mark.gpu
+
+R_32F, R_16F, R_8U = np.float32, np.float16, np.uint8
+ORC_DT = {np.float32: 0, np.float16: 2, np.uint8: 8}
+
+
+def _case(orc, n, dim, n_lists, pq_dim, pq_bits, dtype=np.float32, metric="sqeuclidean",
+          kind="subspace", force_rot=False, seed=3, n_queries=64, batches=1):
+    print(f"case n={n} dim={dim} lists={n_lists} pq_dim={pq_dim} bits={pq_bits} "
+          f"dtype={np.dtype(dtype).name} metric={metric} kind={kind} rot={force_rot}", flush=True)
+    data = H.make_data(n, dim, dtype, seed)
+    model = H.train(data, n_lists, pq_dim, pq_bits, metric=metric, codebook_kind=kind,
+                    force_random_rotation=force_rot, iters=4)
+    queries = H.make_data(n_queries, dim, dtype, seed + 100)
+    index = G.build_gpu_index(model, data, pq_dim, pq_bits, metric, kind, batches=batches)
+    ix, gpu_codes = G.read_back(orc, index, model, dim, pq_dim, pq_bits, metric, kind)
+    return data, model, queries, index, ix, gpu_codes
+
+
+def _search_both(orc, index, ix, queries, k, n_probes, lut=R_32F, internal=R_32F, coarse=R_32F,
+                 **kw):
+    sp = ivf_pq.SearchParams(n_probes=n_probes, lut_dtype=lut, internal_distance_dtype=internal,
+                             coarse_search_dtype=coarse, **kw)
+    d, nb = ivf_pq.search(sp, index, G.to_dev(queries), k)
+    torch.cuda.synchronize()
+    want_nb, want_d = orc.search(ix, queries, k, n_probes, lut_dtype=ORC_DT[lut],
+                                 internal_distance_dtype=ORC_DT[internal],
+                                 coarse_search_dtype=ORC_DT[coarse])
+    return nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d
+
+
+def test_config1_tiny_l2_fp32(orc):
+    """BASELINE configs[0]: 10,000 x 128 fp32 from a 64-component mixture, 64 lists, pq_dim 32,
+    8-bit, 100 queries, k = 10, 8 probes, fp32 table and distances."""
+    from cuvs_amd import testing
+    x = testing.gaussian_mixture(10000, 128, 64, 0.3, seed=1234).numpy()
+    q = testing.gaussian_mixture(100, 128, 64, 0.3, seed=1234)  # same mixture
+    q = testing.gaussian_mixture(10100, 128, 64, 0.3, seed=1234).numpy()[10000:]
+    model = H.train(x, 64, 32, 8, iters=10)
+    index = G.build_gpu_index(model, x, 32, 8)
+    ix, gpu_codes = G.read_back(orc, index, model, 128, 32, 8)
+    # stored codes and list membership equal the oracle's encoding of the same rows
+    labels, codes = orc.encode(ix, x)
+    sizes = np.bincount(labels, minlength=64)
+    assert np.array_equal(sizes, ix.list_sizes)
+    for l in range(64):
+        order = np.argsort(ix.list_inds[l])
+        assert np.array_equal(ix.list_inds[l][order], np.nonzero(labels == l)[0])
+        assert np.array_equal(gpu_codes[l][order], codes[labels == l])
+    # probes bit-exact
+    sp = ivf_pq.SearchParams(n_probes=8)
+    probes = ivf_pq.select_clusters(sp, index, G.to_dev(q)).cpu().numpy().view(np.uint32)
+    want_probes, _ = orc.select_clusters(ix, q, 8)
+    assert np.array_equal(probes, want_probes)
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, q, 10, 8)
+    H.compare_results(nb, d, want_nb, want_d, 1e-5, exact=True)
+    truth = testing.exact_knn(torch.from_numpy(x), torch.from_numpy(q), 10).numpy()
+    assert abs(testing.recall(nb, truth) - testing.recall(want_nb, truth)) <= 0.005
+    assert testing.recall(nb, truth) > 0.7
+
+
+@pytest.mark.parametrize("pq_bits,pq_dim", [(4, 16), (5, 8), (6, 12), (7, 16), (8, 12), (8, 7)])
+@pytest.mark.parametrize("lut,internal,rtol", [(R_32F, R_32F, 1e-5), (R_16F, R_32F, 2e-3),
+                                               (R_8U, R_32F, 2e-3), (R_16F, R_16F, 2e-3),
+                                               (R_8U, R_16F, 2e-3)])
+def test_pq_bits_and_table_types(orc, pq_bits, pq_dim, lut, internal, rtol):
+    if (pq_bits * pq_dim) % 8 != 0:
+        pytest.skip("pq_bits * pq_dim must be a multiple of 8")
+    dim = pq_dim * 2
+    data, model, queries, index, ix, _ = _case(orc, 3000, dim, 10, pq_dim, pq_bits)
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, 10, 4, lut, internal)
+    H.compare_results(nb, d, want_nb, want_d, rtol, exact=True)
+
+
+@pytest.mark.parametrize("metric", ["sqeuclidean", "euclidean", "inner_product", "cosine"])
+@pytest.mark.parametrize("kind", ["subspace", "cluster"])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.int8, np.uint8])
+def test_metrics_codebooks_and_element_types(orc, metric, kind, dtype):
+    data, model, queries, index, ix, _ = _case(orc, 2500, 30, 8, 10, 8, dtype=dtype, metric=metric,
+                                               kind=kind, force_rot=(kind == "cluster"))
+    for lut, internal, rtol in [(R_32F, R_32F, 1e-5), (R_8U, R_16F, 2e-3)]:
+        nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, 7, 3, lut, internal)
+        H.compare_results(nb, d, want_nb, want_d, rtol, exact=(metric != "euclidean"))
+
+
+@pytest.mark.parametrize("k", [1, 2, 16, 17, 100, 128, 129, 256, 257, 700])
+def test_k_sweep_crosses_fused_boundary(orc, k):
+    data, model, queries, index, ix, _ = _case(orc, 6000, 16, 12, 8, 8, n_queries=20)
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, k, 5)
+    H.compare_results(nb, d, want_nb, want_d, 1e-5, exact=True)
+
+
+@pytest.mark.parametrize("n_probes", [1, 2, 5, 33, 64, 1000])
+def test_n_probes_sweep(orc, n_probes):
+    data, model, queries, index, ix, _ = _case(orc, 5000, 16, 64, 8, 8, n_queries=33)
+    sp = ivf_pq.SearchParams(n_probes=n_probes)
+    probes = ivf_pq.select_clusters(sp, index, G.to_dev(queries)).cpu().numpy().view(np.uint32)
+    want_probes, _ = orc.select_clusters(ix, queries, n_probes)
+    assert np.array_equal(probes, want_probes)
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, 10, n_probes)
+    H.compare_results(nb, d, want_nb, want_d, 1e-5, exact=True)
+
+
+@pytest.mark.parametrize("dim", [1, 2, 3, 5, 8, 13, 17])
+def test_small_dims(orc, dim):
+    pq_dim = dim
+    data, model, queries, index, ix, _ = _case(orc, 1200, dim, 6, pq_dim, 8, n_queries=16)
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, 5, 3)
+    H.compare_results(nb, d, want_nb, want_d, 1e-5, exact=True)
+
+
+def test_unfilled_slots_and_empty_lists(orc):
+    data, model, queries, index, ix, _ = _case(orc, 120, 8, 40, 4, 8, n_queries=10)
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, 30, 2)
+    assert (want_nb == np.iinfo(np.int64).max).any()
+    assert np.array_equal(nb, want_nb)
+    assert np.array_equal(d, want_d)
+
+
+def test_extend_in_batches_and_custom_ids(orc):
+    n, dim = 4000, 16
+    data = H.make_data(n, dim, np.float32, 8)
+    model = H.train(data, 10, 8, 8, iters=4)
+    ids = (np.arange(n, dtype=np.int64) * 3 + 17)
+    index = G.build_gpu_index(model, data, 8, 8, ids=ids, batches=3)
+    assert len(index) == n
+    ix, gpu_codes = G.read_back(orc, index, model, dim, 8, 8)
+    ref, labels, codes = H.oracle_index_with_data(orc, model, data, 8, 8, ids=ids)
+    assert np.array_equal(ix.list_sizes, ref.list_sizes)
+    for l in range(10):
+        order = np.argsort(ix.list_inds[l])
+        assert np.array_equal(ix.list_inds[l][order], ref.list_inds[l])
+        assert np.array_equal(gpu_codes[l][order], codes[labels == l])
+    queries = H.make_data(50, dim, np.float32, 99)
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, 10, 4)
+    H.compare_results(nb, d, want_nb, want_d, 1e-5, exact=True)
+    # default ids continue from the current size
+    more = H.make_data(100, dim, np.float32, 10)
+    ivf_pq.extend(index, G.to_dev(more), None)
+    assert len(index) == n + 100
+    all_ids = np.concatenate([index.list_indices(l).cpu().numpy() for l in range(10)])
+    assert set(all_ids.tolist()) == set(ids.tolist()) | set(range(n, n + 100))
+    # host input is accepted as well
+    ivf_pq.extend(index, more, np.arange(10 ** 6, 10 ** 6 + 100, dtype=np.int64))
+    assert len(index) == n + 200
+
+
+def test_transform_matches_stored_codes(orc):
+    """Codes returned by transform equal the codes extend stored (reference invariant:
+    python/cuvs/cuvs/tests/test_ivf_pq.py:339-378)."""
+    data, model, queries, index, ix, gpu_codes = _case(orc, 2000, 20, 7, 10, 6)
+    labels, flat = ivf_pq.transform(index, G.to_dev(data))
+    labels = labels.cpu().numpy().view(np.uint32)
+    codes = G.unpack_bits(flat.cpu().numpy(), 10, 6)
+    want_labels, want_codes = orc.encode(ix, data)
+    assert np.array_equal(labels, want_labels)
+    assert np.array_equal(codes, want_codes)
+    for l in range(7):
+        order = np.argsort(ix.list_inds[l])
+        assert np.array_equal(gpu_codes[l][order], codes[labels == l])
+
+
+def test_bitset_filter(orc):
+    data, model, queries, index, ix, _ = _case(orc, 3000, 16, 8, 8, 8)
+    n = data.shape[0]
+    keep = np.ones(n, dtype=bool)
+    keep[:300] = False
+    bits = np.packbits(keep, bitorder="little")
+    bits = np.concatenate([bits, np.zeros((-bits.size) % 4, dtype=np.uint8)]).view(np.uint32)
+    sp = ivf_pq.SearchParams(n_probes=8)
+    d, nb = ivf_pq.search(sp, index, G.to_dev(queries), 10,
+                          filter_bitset=G.to_dev(bits.view(np.int32)), filter_nbits=n)
+    want_nb, want_d = orc.search(ix, queries, 10, 8, filter_bitset=bits, filter_nbits=n)
+    H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 1e-5, exact=True)
+    assert nb.min().item() >= 300
+
+
+def test_batching_does_not_change_results(orc):
+    data, model, queries, index, ix, _ = _case(orc, 3000, 16, 8, 8, 8, n_queries=301)
+    a = _search_both(orc, index, ix, queries, 10, 4, max_internal_batch_size=4096)
+    b = _search_both(orc, index, ix, queries, 10, 4, max_internal_batch_size=37)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+    H.compare_results(a[0], a[1], a[2], a[3], 1e-5, exact=True)
+
+
+def test_half_precision_coarse_search(orc):
+    data, model, queries, index, ix, _ = _case(orc, 4000, 32, 50, 16, 8)
+    sp = ivf_pq.SearchParams(n_probes=6, coarse_search_dtype=np.float16)
+    probes = ivf_pq.select_clusters(sp, index, G.to_dev(queries)).cpu().numpy().view(np.uint32)
+    want_probes, _ = orc.select_clusters(ix, queries, 6, coarse_search_dtype=2)
+    assert np.array_equal(probes, want_probes)
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, 10, 6, coarse=np.float16)
+    H.compare_results(nb, d, want_nb, want_d, 1e-5, exact=True)
+
+
+def test_validation_errors(orc):
+    """Error behaviour of search (cuVS ivf_pq_search.cuh:901-923,1088-1096; c/src/neighbors/ivf_pq.cpp:315-325)."""
+    data, model, queries, index, ix, _ = _case(orc, 500, 8, 4, 4, 8, n_queries=4)
+    q = G.to_dev(queries)
+    ok = ivf_pq.SearchParams(n_probes=2)
+    with pytest.raises(CuvsError, match="must be positive"):
+        ivf_pq.search(ok, index, q, 0)
+    with pytest.raises(CuvsError, match="total size"):
+        ivf_pq.search(ok, index, q, 501)
+    with pytest.raises(CuvsError, match="n_probes"):
+        ivf_pq.search(ivf_pq.SearchParams(n_probes=0), index, q, 5)
+    with pytest.raises(CuvsError, match="combination"):
+        ivf_pq.search(ivf_pq.SearchParams(n_probes=2, internal_distance_dtype=np.float16), index, q, 5)
+    with pytest.raises(CuvsError, match="lut_dtype"):
+        ivf_pq.search(ivf_pq.SearchParams(n_probes=2, lut_dtype=np.int8), index, q, 5)
+    with pytest.raises(CuvsError, match="dimensions"):
+        ivf_pq.search(ok, index, G.to_dev(np.zeros((4, 9), dtype=np.float32)), 5)
+    with pytest.raises(CuvsError, match="int64"):
+        ivf_pq.search(ok, index, q, 5, neighbors=torch.empty((4, 5), dtype=torch.int32, device="cuda"))
+    with pytest.raises(CuvsError, match="float32"):
+        ivf_pq.search(ok, index, q, 5, distances=torch.empty((4, 5), dtype=torch.float16, device="cuda"))
+    with pytest.raises(CuvsError, match="device compatible"):
+        ivf_pq.search(ok, index, queries, 5)
+    with pytest.raises(CuvsError, match="number of queries"):
+        ivf_pq.search(ok, index, q, 5, neighbors=torch.empty((3, 5), dtype=torch.int64, device="cuda"))
+    with pytest.raises(CuvsError, match="row-major"):
+        from cuvs_amd import dlpack
+        from cuvs_amd._lib import check, lib
+        import ctypes as C
+        qv = dlpack.view(q)
+        qv.mt.dl_tensor.strides = (C.c_int64 * 2)(1, 4)
+        nb = torch.empty((4, 5), dtype=torch.int64, device="cuda")
+        dd = torch.empty((4, 5), dtype=torch.float32, device="cuda")
+        check(lib().cuvsIvfPqSearch(ivf_pq._default_resources().get_c_obj(), ok._p, index.index,
+                                    qv.ptr, dlpack.view(nb).ptr, dlpack.view(dd).ptr))
+    with pytest.raises(CuvsError, match="not part of this library"):
+        ivf_pq.build(ivf_pq.IndexParams(), q)
+    # a good call clears the error text and still works after the failures above
+    d, nb = ivf_pq.search(ok, index, q, 5)
+    want_nb, want_d = orc.search(ix, queries, 5, 2)
+    assert np.array_equal(nb.cpu().numpy(), want_nb)
+
+
+def test_getters_round_trip(orc):
+    data, model, queries, index, ix, _ = _case(orc, 800, 12, 5, 6, 8, kind="cluster")
+    assert (index.n_lists, index.dim, index.pq_dim, index.pq_bits, index.pq_len) == (5, 12, 6, 8, 2)
+    assert np.array_equal(index.centers_padded.cpu().numpy(), model["centers"])
+    assert np.array_equal(index.centers.cpu().numpy(), model["centers"][:, :12])
+    assert np.array_equal(index.centers_rot.cpu().numpy(), model["centers_rot"])
+    assert np.array_equal(index.rotation_matrix.cpu().numpy(), model["rotation_matrix"])
+    assert np.array_equal(index.pq_centers.cpu().numpy(), model["pq_centers"])
+    assert int(index.list_sizes.sum().item()) == 800
