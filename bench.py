@@ -1,0 +1,223 @@
+"""Benchmark of the IVF-PQ search path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one `cuvsIvfPqSearch` call over the whole query batch with the queries already in HBM.
+Workload (BASELINE.json configs[2], the configuration the metric is quoted on): 10M x 128 uint8
+SIFT-like rows, n_lists = 16384, pq_dim = 64, pq_bits = 8, 10,000 queries, k = 10, n_probes = 64,
+fp16 lookup table with fp32 internal distances.  Prints ONE JSON line with the QPS, recall@10, the
+roofline of the code-scan kernel and a CPU baseline (the oracle, multithreaded, on a bounded
+query sample).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+
+
+def log(msg):
+    print(f"[bench {time.strftime('%H:%M:%S')}] {msg}", file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--rows", type=int, default=10_000_000)
+    ap.add_argument("--lists", type=int, default=16384)
+    ap.add_argument("--queries", type=int, default=10_000)
+    ap.add_argument("--probes", type=int, default=64)
+    ap.add_argument("--k", type=int, default=10)
+    ap.add_argument("--lut", default="f16", choices=["f32", "f16", "fp8"])
+    ap.add_argument("--internal", default="f32", choices=["f32", "f16"])
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import numpy as np
+    import torch
+
+    from cuvs_amd import ivf_pq, testing
+    from cuvs_amd.resources import Resources
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = "cuda"
+    dim, pq_dim, pq_bits = 128, 64, 8
+    n, nq, n_lists, P, k = args.rows, args.queries, args.lists, args.probes, args.k
+    lut_np = {"f32": np.float32, "f16": np.float16, "fp8": np.uint8}[args.lut]
+    int_np = {"f32": np.float32, "f16": np.float16}[args.internal]
+
+    t0 = time.time()
+    allrows = testing.sift_like_u8(n + nq, dim, 4096, seed=1234, device=dev)
+    data, queries = allrows[:n], allrows[n:].contiguous()
+    log(f"data {tuple(data.shape)} uint8 generated in {time.time() - t0:.1f}s")
+
+    t0 = time.time()
+    g = torch.Generator(device="cpu")
+    g.manual_seed(137)
+    n_train = min(n, max(n_lists * 32, 200_000))
+    sel = torch.randperm(n, generator=g)[:n_train].to(dev)
+    model = testing.train_model(data[sel], n_lists, pq_dim, pq_bits, kmeans_iters=6, pq_iters=8,
+                                seed=137, half_assign=True)
+    torch.cuda.synchronize()
+    log(f"model trained on {n_train} rows in {time.time() - t0:.1f}s")
+
+    t0 = time.time()
+    labels = testing.assign_nearest(data, model["centers"][:, :dim], half=True).to(torch.int32)
+    torch.cuda.synchronize()
+    log(f"lists assigned in {time.time() - t0:.1f}s")
+
+    t0 = time.time()
+    res = Resources()
+    res.use_torch_current_stream()
+    params = ivf_pq.IndexParams(n_lists=n_lists, pq_bits=pq_bits, pq_dim=pq_dim)
+    index = ivf_pq.build_precomputed(params, dim, model["pq_centers"], model["centers"],
+                                     model["centers_rot"], model["rotation_matrix"], resources=res)
+    ivf_pq.extend(index, data, None, resources=res, labels=labels)
+    res.sync()
+    log(f"index populated ({len(index)} rows) in {time.time() - t0:.1f}s")
+
+    t0 = time.time()
+    truth = testing.exact_knn(data, queries, k, half=True).cpu().numpy()
+    log(f"exact ground truth in {time.time() - t0:.1f}s")
+
+    sp = ivf_pq.SearchParams(n_probes=P, lut_dtype=lut_np, internal_distance_dtype=int_np,
+                             max_internal_batch_size=max(nq, 1))
+    neighbors = torch.empty((nq, k), dtype=torch.int64, device=dev)
+    distances = torch.empty((nq, k), dtype=torch.float32, device=dev)
+
+    def step():
+        ivf_pq.search(sp, index, queries, k, neighbors=neighbors, distances=distances, resources=res)
+
+    for _ in range(args.warmup):
+        step()
+    res.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    res.sync()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    qps = nq * args.steps / elapsed
+    gpu_ids = neighbors.cpu().numpy()
+    gpu_recall = testing.recall(gpu_ids, truth)
+    log(f"{ms_per_step:.2f} ms per batch of {nq}: {qps:,.0f} QPS, recall@{k} {gpu_recall:.4f}")
+
+    # per-kernel time of the scan: HIP events on the library's stream, same steps again
+    res.enable_profiling(True)
+    scan_ms, stage = [], None
+    for _ in range(args.steps):
+        step()
+        stage = ivf_pq.get_search_profile(res)
+        scan_ms.append(stage["scan_ms"] / max(stage["n_scan_launches"], 1))
+    res.enable_profiling(False)
+    scan_avg_ms = float(np.mean(scan_ms))
+    bytes_per_launch = stage["scan_bytes"] / max(stage["n_scan_launches"], 1)
+    achieved = bytes_per_launch / (scan_avg_ms * 1e-3) / 1e9
+    log(f"scan kernel {scan_avg_ms:.3f} ms per launch, {bytes_per_launch / 1e9:.2f} GB algorithmic "
+        f"-> {achieved:.0f} GB/s ({achieved / HBM_PEAK_GBS:.1%} of HBM peak); stages: "
+        f"coarse {stage['coarse_ms']:.2f} rotate {stage['rotate_ms']:.2f} scan {stage['scan_ms']:.2f} "
+        f"merge {stage['merge_ms']:.2f} ms")
+
+    out = {
+        "metric": "QPS@recall@10 (10M x 128 IVF-PQ, batch 10k); code-scan HBM GB/s vs peak",
+        "value": qps, "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32" if args.internal == "f32" else "f16",
+        "data": "synthetic",
+        "config": {"workload": f"configs[2]: {n} x {dim} uint8 SIFT-like, n_lists={n_lists}, "
+                               f"pq_dim={pq_dim}, pq_bits={pq_bits}, {nq} queries, k={k}, "
+                               f"n_probes={P}, lut={args.lut}, internal={args.internal}, L2",
+                   "n_rows": n, "dim": dim, "n_lists": n_lists, "pq_dim": pq_dim,
+                   "pq_bits": pq_bits, "n_queries": nq, "k": k, "n_probes": P,
+                   "lut_dtype": args.lut, "internal_distance_dtype": args.internal,
+                   "recall_at_k": gpu_recall,
+                   "stage_ms": {s: stage[s] for s in ("coarse_ms", "rotate_ms", "scan_ms", "merge_ms")}},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "scan_kernel", "kernel_ms": scan_avg_ms,
+                     "algorithmic_bytes_per_launch": bytes_per_launch},
+    }
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(args, index, model, queries, truth, gpu_ids, dim, pq_dim,
+                                           pq_bits, P, k, log)
+        out["config"]["oracle_recall_on_sample"] = out["cpu_baseline"].pop("oracle_recall")
+        out["config"]["gpu_recall_on_sample"] = out["cpu_baseline"].pop("gpu_recall")
+    print(json.dumps(out), flush=True)
+
+
+def cpu_baseline(args, index, model, queries, truth, gpu_ids, dim, pq_dim, pq_bits, P, k, log):
+    """The CPU oracle (a scalar restatement of the reference algorithm, multithreaded over
+    queries) timed on a bounded sample of the same queries against the same index contents."""
+    import numpy as np
+
+    import gpu_helpers as G
+    from cuvs_amd import testing
+    from oracle import oracle
+
+    t0 = time.time()
+    host_model = {kk: v.cpu().numpy() for kk, v in model.items()}
+    ix = read_back_bulk(oracle, index, host_model, dim, pq_dim, pq_bits)
+    log(f"index copied to the host for the CPU baseline in {time.time() - t0:.1f}s")
+    lut = {"f32": 0, "f16": 2, "fp8": 8}[args.lut]
+    internal = {"f32": 0, "f16": 2}[args.internal]
+    threads = oracle.default_threads()
+    q_host = queries.cpu().numpy()
+    pilot = min(2 * threads, q_host.shape[0])
+    t0 = time.perf_counter()
+    oracle.search(ix, q_host[:pilot], k, P, lut_dtype=lut, internal_distance_dtype=internal,
+                  n_threads=threads)
+    per_query = (time.perf_counter() - t0) / pilot
+    n_sample = int(min(q_host.shape[0], max(pilot, args.cpu_seconds / max(per_query, 1e-9))))
+    t0 = time.perf_counter()
+    nb, _ = oracle.search(ix, q_host[:n_sample], k, P, lut_dtype=lut,
+                          internal_distance_dtype=internal, n_threads=threads)
+    dt = time.perf_counter() - t0
+    o_rec = testing.recall(nb, truth[:n_sample])
+    g_rec = testing.recall(gpu_ids[:n_sample], truth[:n_sample])
+    same = float((nb == gpu_ids[:n_sample]).mean())
+    log(f"CPU oracle: {n_sample} queries in {dt:.1f}s on {threads} threads = {n_sample / dt:,.0f} QPS; "
+        f"recall {o_rec:.4f} (GPU on the same queries {g_rec:.4f}); identical ids {same:.4%}")
+    return {"value": n_sample / dt, "unit": "queries/s", "cores": threads, "kind": "port",
+            "sample": f"first {n_sample} of the {q_host.shape[0]} queries, same index and parameters",
+            "oracle_recall": o_rec, "gpu_recall": g_rec, "ids_identical_frac": same}
+
+
+def read_back_bulk(oracle, index, host_model, dim, pq_dim, pq_bits):
+    """Host copy of the index for the oracle: codes via the unpack entry point, ids via the getter."""
+    import numpy as np
+
+    import gpu_helpers as G
+    import helpers as H
+
+    sizes = index.list_sizes.cpu().numpy().astype(np.uint32)
+    datas, inds = [], []
+    for l in range(len(sizes)):
+        if sizes[l] == 0:
+            datas.append(np.zeros(0, dtype=np.uint8))
+            inds.append(np.zeros(0, dtype=np.int64))
+            continue
+        flat = index.list_data(l, n_rows=int(sizes[l])).cpu().numpy()
+        codes = flat if pq_bits == 8 else G.unpack_bits(flat, pq_dim, pq_bits)
+        datas.append(oracle.pack_list(codes, pq_bits))
+        inds.append(index.list_indices(l).cpu().numpy())
+    ix = H.oracle_index(oracle, host_model, dim, pq_dim, pq_bits)
+    ix.set_lists(sizes, datas, inds)
+    return ix
+
+
+if __name__ == "__main__":
+    main()
