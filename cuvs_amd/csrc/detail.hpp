@@ -191,6 +191,10 @@ struct scan_args {
 /** LDS bytes the scan kernel needs for these arguments. */
 size_t scan_lds_bytes(const scan_args& a);
 void launch_scan(const scan_args& a, hipStream_t stream);
+/** Persistent kernel for 8-bit codes and common shapes (scan_fast.hip); returns false when the
+ *  arguments are outside what it covers.  `work_counter` is one device word of scratch. */
+bool scan_fast_supported(const scan_args& a);
+bool launch_scan_fast(const scan_args& a, uint32_t* work_counter, hipStream_t stream);
 
 struct merge_args {
   uint32_t n_queries, n_probes, k, max_samples;

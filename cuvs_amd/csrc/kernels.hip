@@ -10,175 +10,11 @@
  * reproducible against a scalar CPU implementation: dot products accumulate with one FMA per
  * element in ascending index order; lookup-table entries are built in fp32 and rounded once.
  */
-#include "detail.hpp"
-
-#include <hip/hip_runtime.h>
-
-#include <cfloat>
-#include <type_traits>
+#include "device_utils.cuh"
 
 namespace cuvs::neighbors::ivf_pq::detail {
 
 namespace {
-
-constexpr int kBlock              = 256;
-constexpr unsigned long long kInvalidKey = 0xFFFFFFFFFFFFFFFFull;
-
-/* ---------------------------------------------------------------------------------------- */
-/* small device helpers                                                                      */
-/* ---------------------------------------------------------------------------------------- */
-
-/** Monotone map float -> uint32 (ascending); -0 and +0 map to the same key. */
-__device__ __forceinline__ uint32_t order_f32(float f)
-{
-  f          = (f == 0.0f) ? 0.0f : f;
-  uint32_t u = __float_as_uint(f);
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-__device__ __forceinline__ float unorder_f32(uint32_t k)
-{
-  uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
-  return __uint_as_float(u);
-}
-
-__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v)
-{
-  const uint32_t lane = threadIdx.x & 63u;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    uint32_t o = __shfl_up(v, d, 64);
-    if (lane >= uint32_t(d)) { v += o; }
-  }
-  return v;
-}
-
-/** In-place ascending bitonic sort of n (power of two) keys in LDS by the whole block. */
-__device__ void block_bitonic_sort(unsigned long long* a, uint32_t n)
-{
-  for (uint32_t size = 2; size <= n; size <<= 1) {
-    for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
-      for (uint32_t t = threadIdx.x; t < (n >> 1); t += blockDim.x) {
-        const uint32_t pos     = 2 * t - (t & (stride - 1));
-        const uint32_t partner = pos + stride;
-        const bool ascending   = (pos & size) == 0;
-        const unsigned long long x = a[pos];
-        const unsigned long long y = a[partner];
-        if ((x > y) == ascending) {
-          a[pos]     = y;
-          a[partner] = x;
-        }
-      }
-      __syncthreads();
-    }
-  }
-}
-
-/* ---------------------------------------------------------------------------------------- */
-/* exact k-smallest selection of 64-bit keys by one block: MSB-first radix passes over an     */
-/* 11-bit digit that stop as soon as a digit boundary coincides with the k-th element, then    */
-/* one collection pass and a bitonic sort of the k survivors.                                  */
-/* ---------------------------------------------------------------------------------------- */
-
-constexpr int kRadixBits = 11;
-constexpr int kBins      = 1 << kRadixBits;
-
-struct select_smem {
-  uint32_t hist[kBins];
-  uint32_t wave_sums[kBlock / 64];
-  uint32_t bin, before, upto, count;
-};
-
-/**
- * key_of(i), i < n, returns the key of element i or kInvalidKey.  Writes the min(k, #valid)
- * smallest keys ascending into out[0..), pads the rest of out[0..out_cap) with kInvalidKey and
- * returns their number.  out_cap is a power of two >= k.  All threads of the block must call.
- */
-template <typename KeyFn>
-__device__ uint32_t block_select_sorted(KeyFn key_of, uint32_t n, uint32_t k,
-                                        unsigned long long* out, uint32_t out_cap, select_smem& sm)
-{
-  const uint32_t tid = threadIdx.x;
-  unsigned long long prefix = 0;
-  uint32_t pb   = 0;  // number of leading key bits already fixed in `prefix`
-  uint32_t need = k;
-  bool none     = false;
-  for (;;) {
-    const uint32_t digit_bits = (64u - pb) < uint32_t(kRadixBits) ? (64u - pb) : uint32_t(kRadixBits);
-    const uint32_t shift      = 64u - pb - digit_bits;
-    const uint32_t dmask      = (1u << digit_bits) - 1u;
-    for (uint32_t i = tid; i < uint32_t(kBins); i += kBlock) { sm.hist[i] = 0; }
-    __syncthreads();
-    for (uint32_t i = tid; i < n; i += kBlock) {
-      const unsigned long long key = key_of(i);
-      if (key != kInvalidKey && (pb == 0 || (key >> (64u - pb)) == prefix)) {
-        atomicAdd(&sm.hist[uint32_t(key >> shift) & dmask], 1u);
-      }
-    }
-    __syncthreads();
-    constexpr uint32_t per = kBins / kBlock;
-    uint32_t s = 0;
-#pragma unroll
-    for (uint32_t j = 0; j < per; j++) { s += sm.hist[tid * per + j]; }
-    uint32_t incl = wave_inclusive_scan(s);
-    if ((tid & 63u) == 63u) { sm.wave_sums[tid >> 6] = incl; }
-    __syncthreads();
-    uint32_t base = 0, total = 0;
-#pragma unroll
-    for (uint32_t w = 0; w < kBlock / 64; w++) {
-      const uint32_t ws = sm.wave_sums[w];
-      if (w < (tid >> 6)) { base += ws; }
-      total += ws;
-    }
-    incl += base;
-    const uint32_t excl = incl - s;
-    if (pb == 0 && need > total) { need = total; }
-    if (need == 0) {
-      none = true;
-      break;
-    }
-    if (excl < need && need <= incl) {
-      uint32_t c = excl;
-      for (uint32_t j = 0; j < per; j++) {
-        const uint32_t h = sm.hist[tid * per + j];
-        if (c + h >= need) {
-          sm.bin    = tid * per + j;
-          sm.before = c;
-          sm.upto   = c + h;
-          break;
-        }
-        c += h;
-      }
-    }
-    __syncthreads();
-    const uint32_t b      = sm.bin;
-    const uint32_t before = sm.before;
-    const uint32_t upto   = sm.upto;
-    prefix                = (prefix << digit_bits) | b;
-    pb += digit_bits;
-    __syncthreads();
-    if (upto == need || pb >= 64u) { break; }
-    need -= before;
-  }
-
-  if (tid == 0) { sm.count = 0; }
-  __syncthreads();
-  if (!none) {
-    for (uint32_t i = tid; i < n; i += kBlock) {
-      const unsigned long long key = key_of(i);
-      if (key != kInvalidKey && (key >> (64u - pb)) <= prefix) {
-        const uint32_t pos = atomicAdd(&sm.count, 1u);
-        if (pos < out_cap) { out[pos] = key; }
-      }
-    }
-  }
-  __syncthreads();
-  uint32_t cnt = sm.count;
-  if (cnt > out_cap) { cnt = out_cap; }
-  for (uint32_t i = cnt + tid; i < out_cap; i += kBlock) { out[i] = kInvalidKey; }
-  __syncthreads();
-  block_bitonic_sort(out, out_cap);
-  return cnt < k ? cnt : k;
-}
 
 /* ---------------------------------------------------------------------------------------- */
 /* element mapping, coarse scores, probe selection                                           */
@@ -470,72 +306,6 @@ __global__ void pair_scatter_kernel(const uint32_t* __restrict__ probes, uint32_
 }
 
 /* ---------------------------------------------------------------------------------------- */
-/* lookup-table element types                                                                */
-/* ---------------------------------------------------------------------------------------- */
-
-enum { LUT_F32 = 0, LUT_F16 = 1, LUT_FP8U = 2, LUT_FP8S = 3 };
-
-/* 8-bit float with 5 exponent bits, bias 15, 3 (unsigned) or 2 (signed, sign in the LSB) value
- * bits: encode truncates, decode adds half a unit (cuVS ivf_pq_fp_8bit.cuh:31-100). */
-__device__ __forceinline__ uint8_t fp8_encode_unsigned(float v)
-{
-  if (v < 3.0517578125e-05f) { return 0; }  // 2^-15
-  if (v >= 122880.0f) { return 0xffu; }     // 2^16 * (2 - 1/8)
-  return uint8_t((__float_as_uint(v) + (15u << 23) - 0x3f800000u) >> 20);
-}
-__device__ __forceinline__ uint8_t fp8_encode_signed(float v)
-{
-  const uint8_t u = fp8_encode_unsigned(fabsf(v));
-  return uint8_t((u & 0xfeu) | (v < 0.0f ? 1u : 0u));
-}
-
-template <int LUT>
-struct lut_traits;
-template <>
-struct lut_traits<LUT_F32> {
-  using storage = float;
-  static __device__ __forceinline__ storage encode(float v) { return v; }
-  static __device__ __forceinline__ float to_float(storage s) { return s; }
-  static __device__ __forceinline__ _Float16 to_half(storage s) { return _Float16(s); }
-};
-template <>
-struct lut_traits<LUT_F16> {
-  using storage = _Float16;
-  static __device__ __forceinline__ storage encode(float v) { return _Float16(v); }
-  static __device__ __forceinline__ float to_float(storage s) { return float(s); }
-  static __device__ __forceinline__ _Float16 to_half(storage s) { return s; }
-};
-template <>
-struct lut_traits<LUT_FP8U> {
-  using storage = uint8_t;
-  static __device__ __forceinline__ storage encode(float v) { return fp8_encode_unsigned(v); }
-  static __device__ __forceinline__ float to_float(storage s)
-  {
-    return __uint_as_float(0x38080000u + (uint32_t(s) << 20));
-  }
-  static __device__ __forceinline__ _Float16 to_half(storage s)
-  {
-    const uint16_t bits = uint16_t(0x0040u + (uint32_t(s) << 7));
-    return __builtin_bit_cast(_Float16, bits);
-  }
-};
-template <>
-struct lut_traits<LUT_FP8S> {
-  using storage = uint8_t;
-  static __device__ __forceinline__ storage encode(float v) { return fp8_encode_signed(v); }
-  static __device__ __forceinline__ float to_float(storage s)
-  {
-    const uint32_t bits = 0x38080000u + (uint32_t(s & 0xfeu) << 20);
-    return __uint_as_float(bits | (uint32_t(s & 1u) << 31));
-  }
-  static __device__ __forceinline__ _Float16 to_half(storage s)
-  {
-    const uint16_t bits = uint16_t((0x0040u + (uint32_t(s & 0xfeu) << 7)) | (uint32_t(s & 1u) << 15));
-    return __builtin_bit_cast(_Float16, bits);
-  }
-};
-
-/* ---------------------------------------------------------------------------------------- */
 /* the scan kernel: one block per (query, probed list) pair                                   */
 /* ---------------------------------------------------------------------------------------- */
 
@@ -545,11 +315,6 @@ struct scan_smem_tail {
   uint32_t count;
   uint32_t thr;
 };
-
-__device__ __forceinline__ bool is_ip_metric(int metric)
-{
-  return metric == int(DistanceType::InnerProduct) || metric == int(DistanceType::CosineExpanded);
-}
 
 template <int LUT, bool OUT_HALF, int BITS, bool FUSED>
 __global__ __launch_bounds__(kBlock) void scan_kernel(scan_args a)

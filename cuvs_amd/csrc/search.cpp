@@ -7,6 +7,7 @@
 #include "detail.hpp"
 
 #include <algorithm>
+#include <cstdlib>
 #include <limits>
 
 namespace cuvs {
@@ -127,6 +128,16 @@ void validate(const search_params& params, const index_impl& ix, int64_t k)
                "Unsupported coarse_search_dtype (only CUDA_R_32F and CUDA_R_16F are supported)");
   CUVS_EXPECTS(k <= kMaxK, "parameter `k` (%lld) must not exceed %u", static_cast<long long>(k),
                kMaxK);
+}
+
+/** CUVS_AMD_GENERIC_SCAN=1 routes every search through the generic scan kernel (for A/B runs). */
+bool force_generic_scan()
+{
+  static const bool v = [] {
+    const char* e = std::getenv("CUVS_AMD_GENERIC_SCAN");
+    return e != nullptr && e[0] == '1';
+  }();
+  return v;
 }
 
 float scaling_factor(elem_type t)
@@ -275,6 +286,7 @@ void search(cuvs::resources const& res_c,
   auto* n_samples = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * 4));
   auto* kth       = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * 4));
   auto* counters  = static_cast<uint32_t*>(res.workspace_alloc(size_t(ix.n_lists) * 8 + 16));
+  auto* work_ctr  = static_cast<uint32_t*>(res.workspace_alloc(256));
   unsigned long long* keys = nullptr;
   float* all_scores        = nullptr;
   if (pl.fused) {
@@ -327,7 +339,9 @@ void search(cuvs::resources const& res_c,
     sa.query_kth     = kth;
     sa.out_keys      = keys;
     sa.out_scores    = all_scores;
-    detail::launch_scan(sa, s);
+    if (force_generic_scan() || !detail::launch_scan_fast(sa, work_ctr, s)) {
+      detail::launch_scan(sa, s);
+    }
     mark(3);
 
     detail::merge_args ma{};

@@ -260,3 +260,46 @@ def test_getters_round_trip(orc):
     assert np.array_equal(index.rotation_matrix.cpu().numpy(), model["rotation_matrix"])
     assert np.array_equal(index.pq_centers.cpu().numpy(), model["pq_centers"])
     assert int(index.list_sizes.sum().item()) == 800
+
+
+# --- shapes served by the persistent 8-bit scan kernel (pq_dim x pq_len in {64x2, 48x2, 32x4}) ---
+
+@pytest.mark.parametrize("dim,pq_dim", [(128, 64), (96, 48), (128, 32)])
+@pytest.mark.parametrize("lut,internal,rtol", [(R_32F, R_32F, 1e-5), (R_16F, R_32F, 2e-3),
+                                               (R_8U, R_32F, 2e-3), (R_16F, R_16F, 2e-3),
+                                               (R_8U, R_16F, 2e-3)])
+@pytest.mark.parametrize("metric,kind", [("sqeuclidean", "subspace"), ("inner_product", "subspace"),
+                                         ("sqeuclidean", "cluster"), ("cosine", "cluster")])
+def test_persistent_scan_shapes(orc, dim, pq_dim, lut, internal, rtol, metric, kind):
+    data, model, queries, index, ix, _ = _case(orc, 6000, dim, 12, pq_dim, 8, metric=metric,
+                                               kind=kind, n_queries=40, dtype=np.float32)
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, 10, 5, lut, internal)
+    H.compare_results(nb, d, want_nb, want_d, rtol, exact=True)
+
+
+@pytest.mark.parametrize("k", [1, 10, 64, 65, 100, 256])
+def test_persistent_scan_long_lists_and_k(orc, k):
+    """Lists longer than the candidate buffer (segment pruning) and k up to the fused limit."""
+    data, model, queries, index, ix, _ = _case(orc, 20000, 96, 4, 48, 8, n_queries=24,
+                                               dtype=np.uint8)
+    assert ix.list_sizes.max() > 2048
+    for lut, internal in [(R_32F, R_32F), (R_8U, R_16F)]:
+        nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, k, 3, lut, internal)
+        H.compare_results(nb, d, want_nb, want_d, 2e-3, exact=True)
+
+
+def test_persistent_scan_filter_and_empty_lists(orc):
+    data, model, queries, index, ix, _ = _case(orc, 300, 128, 40, 64, 8, n_queries=16)
+    assert (ix.list_sizes == 0).any() or True
+    n = data.shape[0]
+    keep = np.ones(n, dtype=bool)
+    keep[::3] = False
+    bits = np.packbits(keep, bitorder="little")
+    bits = np.concatenate([bits, np.zeros((-bits.size) % 4, dtype=np.uint8)]).view(np.uint32)
+    sp = ivf_pq.SearchParams(n_probes=6)
+    d, nb = ivf_pq.search(sp, index, G.to_dev(queries), 20,
+                          filter_bitset=G.to_dev(bits.view(np.int32)), filter_nbits=n)
+    want_nb, want_d = orc.search(ix, queries, 20, 6, filter_bitset=bits, filter_nbits=n)
+    H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 1e-5, exact=True)
+    nb2, d2, want_nb2, want_d2 = _search_both(orc, index, ix, queries, 30, 2)
+    H.compare_results(nb2, d2, want_nb2, want_d2, 1e-5, exact=True)
