@@ -7,7 +7,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libcuvs_c.so")
+LIB_PATH = os.environ.get("CUVS_AMD_LIB", os.path.join(_HERE, "libcuvs_c.so"))
 
 CUVS_ERROR, CUVS_SUCCESS = 0, 1
 

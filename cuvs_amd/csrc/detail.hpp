@@ -160,10 +160,26 @@ void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, ui
                           uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
                           uint32_t* n_samples, unsigned long long* stats, hipStream_t stream);
 
-/** pair_order = ids of the (query, probe) pairs grouped by probed list. `counters` is scratch of
+/** Everything the scan needs to know about one (query, probe) pair, gathered once so that the
+ *  scan kernel reads one 32-byte record instead of chasing four dependent pointers. */
+struct pair_desc {
+  const uint8_t* data;  // interleaved codes of the probed list
+  uint32_t q;           // query index inside the batch
+  uint32_t slot;        // q * n_probes + p: position of the pair's output
+  uint32_t label;       // probed list
+  uint32_t sample_off;  // sample number of the list's first row for this query
+  uint32_t n_rows;      // list size
+  uint32_t pad;
+};
+static_assert(sizeof(pair_desc) == 32, "pair_desc must stay 32 bytes");
+
+/** pair_order = ids of the (query, probe) pairs grouped by probed list; when `desc` is non-null the
+ *  record of every pair is written at the same position.  `counters` is scratch of
  *  2 * n_lists + 2 words. */
-void launch_order_pairs(const uint32_t* probes, uint32_t n_pairs, uint32_t n_lists,
-                        uint32_t* counters, uint32_t* pair_order, hipStream_t stream);
+void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
+                        const uint8_t* const* data_ptrs, uint32_t n_pairs, uint32_t n_probes,
+                        uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
+                        pair_desc* desc, hipStream_t stream);
 
 struct scan_args {
   uint32_t n_queries, n_probes, k, max_samples;
@@ -182,19 +198,21 @@ struct scan_args {
   const uint32_t* probes;         // [n_queries, n_probes]
   const uint32_t* chunk_indices;  // [n_queries, n_probes]
   const uint32_t* pair_order;     // [n_queries * n_probes] or null
+  const pair_desc* desc;          // [n_queries * n_probes] records in pair_order order, or null
   const uint32_t* filter_bits;    // or null
   int64_t filter_nbits;
   uint32_t* query_kth;            // [n_queries] ordered-score upper bounds (fused)
   unsigned long long* out_keys;   // fused: [n_queries, n_probes, k]
   float* out_scores;              // non-fused: [n_queries, max_samples]
+  unsigned long long* timing;     // per-phase cycle sums (instrumented builds only), or null
 };
 /** LDS bytes the scan kernel needs for these arguments. */
 size_t scan_lds_bytes(const scan_args& a);
 void launch_scan(const scan_args& a, hipStream_t stream);
 /** Persistent kernel for 8-bit codes and common shapes (scan_fast.hip); returns false when the
- *  arguments are outside what it covers.  `work_counter` is one device word of scratch. */
+ *  arguments are outside what it covers.  Needs `a.desc`. */
 bool scan_fast_supported(const scan_args& a);
-bool launch_scan_fast(const scan_args& a, uint32_t* work_counter, hipStream_t stream);
+bool launch_scan_fast(const scan_args& a, hipStream_t stream);
 
 struct merge_args {
   uint32_t n_queries, n_probes, k, max_samples;

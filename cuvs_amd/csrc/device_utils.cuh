@@ -46,7 +46,8 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v)
 }
 
 /** In-place ascending bitonic sort of n (power of two) keys in LDS by the whole block. */
-__device__ void block_bitonic_sort(unsigned long long* a, uint32_t n)
+template <typename KeyPtr>
+__device__ void block_bitonic_sort(KeyPtr a, uint32_t n)
 {
   for (uint32_t size = 2; size <= n; size <<= 1) {
     for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
@@ -183,9 +184,13 @@ enum { LUT_F32 = 0, LUT_F16 = 1, LUT_FP8U = 2, LUT_FP8S = 3 };
  * bits: encode truncates, decode adds half a unit (cuVS ivf_pq_fp_8bit.cuh:31-100). */
 __device__ __forceinline__ uint8_t fp8_encode_unsigned(float v)
 {
-  if (v < 3.0517578125e-05f) { return 0; }  // 2^-15
-  if (v >= 122880.0f) { return 0xffu; }     // 2^16 * (2 - 1/8)
-  return uint8_t((__float_as_uint(v) + (15u << 23) - 0x3f800000u) >> 20);
+  // Reference form: v < 2^-15 -> 0; v >= 2^16 * (2 - 1/8) -> 0xff; else
+  // (bits(v) + (15 << 23) - 0x3f800000) >> 20.  With the bit pattern read as a signed integer
+  // (negative floats are negative integers, positive floats order like their patterns) this is
+  // clamp(bits(v) - bits(2^-15), 0, 0x0fffffff) >> 20, which needs no branches.
+  const int x = int(__float_as_uint(v)) - 0x38000000;
+  const int c = x < 0 ? 0 : (x > 0x0fffffff ? 0x0fffffff : x);
+  return uint8_t(uint32_t(c) >> 20);
 }
 __device__ __forceinline__ uint8_t fp8_encode_signed(float v)
 {

@@ -294,14 +294,31 @@ __global__ __launch_bounds__(kBlock) void exclusive_scan_kernel(const uint32_t* 
   }
 }
 
-__global__ void pair_scatter_kernel(const uint32_t* __restrict__ probes, uint32_t n_pairs,
-                                    uint32_t* __restrict__ cursors,
-                                    uint32_t* __restrict__ pair_order)
+__global__ void pair_scatter_kernel(const uint32_t* __restrict__ probes,
+                                    const uint32_t* __restrict__ chunk_indices,
+                                    const uint8_t* const* __restrict__ data_ptrs, uint32_t n_pairs,
+                                    uint32_t n_probes, uint32_t* __restrict__ cursors,
+                                    uint32_t* __restrict__ pair_order, pair_desc* __restrict__ desc)
 {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n_pairs) {
-    const uint32_t pos = atomicAdd(&cursors[probes[i]], 1u);
-    pair_order[pos]    = i;
+    const uint32_t label = probes[i];
+    const uint32_t pos   = atomicAdd(&cursors[label], 1u);
+    pair_order[pos]      = i;
+    if (desc != nullptr) {
+      const uint32_t q   = i / n_probes;
+      const uint32_t p   = i - q * n_probes;
+      const uint32_t off = p > 0 ? chunk_indices[i - 1] : 0u;
+      pair_desc d;
+      d.data       = data_ptrs[label];
+      d.q          = q;
+      d.slot       = i;
+      d.label      = label;
+      d.sample_off = off;
+      d.n_rows     = chunk_indices[i] - off;
+      d.pad        = 0;
+      desc[pos]    = d;
+    }
   }
 }
 
@@ -829,8 +846,10 @@ void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, ui
   CUVS_LAUNCH_CHECK();
 }
 
-void launch_order_pairs(const uint32_t* probes, uint32_t n_pairs, uint32_t n_lists,
-                        uint32_t* counters, uint32_t* pair_order, hipStream_t stream)
+void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
+                        const uint8_t* const* data_ptrs, uint32_t n_pairs, uint32_t n_probes,
+                        uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
+                        pair_desc* desc, hipStream_t stream)
 {
   if (n_pairs == 0) { return; }
   uint32_t* counts  = counters;
@@ -840,7 +859,8 @@ void launch_order_pairs(const uint32_t* probes, uint32_t n_pairs, uint32_t n_lis
   CUVS_LAUNCH_CHECK();
   exclusive_scan_kernel<<<1, kBlock, 0, stream>>>(counts, n_lists, cursors);
   CUVS_LAUNCH_CHECK();
-  pair_scatter_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(probes, n_pairs, cursors, pair_order);
+  pair_scatter_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(
+    probes, chunk_indices, data_ptrs, n_pairs, n_probes, cursors, pair_order, desc);
   CUVS_LAUNCH_CHECK();
 }
 

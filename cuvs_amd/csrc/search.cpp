@@ -89,7 +89,7 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
   p.fused = k <= kMaxFusedK;
   const size_t P = p.n_probes;
   p.per_query_bytes = size_t(ix.dim) * 4 + size_t(ix.n_lists) * 4 + size_t(ix.rot_dim) * 4 +
-                      P * 4 * 3 + 16 +
+                      P * 4 * 3 + P * sizeof(detail::pair_desc) + 16 +
                       (p.fused ? P * k * 8 : size_t(p.max_samples) * 4);
   p.fixed_bytes = a256(size_t(ix.n_lists) * 8 + 16) + 16 * 256;
   const size_t budget = workspace_budget(res);
@@ -138,6 +138,37 @@ bool force_generic_scan()
     return e != nullptr && e[0] == '1';
   }();
   return v;
+}
+
+/** Instrumented builds (-DCUVS_SCAN_TIMING) accumulate per-phase cycle counts of the scan kernel
+ *  here and print them when the library unloads. */
+unsigned long long* scan_timing_buffer()
+{
+#ifdef CUVS_SCAN_TIMING
+  struct holder {
+    unsigned long long* d = nullptr;
+    holder()
+    {
+      (void)hipMalloc(reinterpret_cast<void**>(&d), 64);
+      (void)hipMemset(d, 0, 64);
+    }
+    ~holder()
+    {
+      unsigned long long h[6] = {};
+      (void)hipMemcpy(h, d, 48, hipMemcpyDeviceToHost);
+      const char* names[6] = {"stage", "lut", "bar_lut", "scan", "bar_scan", "prune_out"};
+      unsigned long long total = 0;
+      for (auto v : h) { total += v; }
+      for (int i = 0; i < 6; i++) {
+        fprintf(stderr, "[scan timing] %-10s %6.2f%%\n", names[i], 100.0 * double(h[i]) / double(total ? total : 1));
+      }
+    }
+  };
+  static holder h;
+  return h.d;
+#else
+  return nullptr;
+#endif
 }
 
 float scaling_factor(elem_type t)
@@ -286,9 +317,14 @@ void search(cuvs::resources const& res_c,
   auto* n_samples = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * 4));
   auto* kth       = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * 4));
   auto* counters  = static_cast<uint32_t*>(res.workspace_alloc(size_t(ix.n_lists) * 8 + 16));
-  auto* work_ctr  = static_cast<uint32_t*>(res.workspace_alloc(256));
+  detail::pair_desc* desc = nullptr;
   unsigned long long* keys = nullptr;
   float* all_scores        = nullptr;
+  sa.fused                 = pl.fused;
+  const bool fast_scan     = !force_generic_scan() && detail::scan_fast_supported(sa);
+  if (fast_scan) {
+    desc = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));
+  }
   if (pl.fused) {
     keys = static_cast<unsigned long long*>(res.workspace_alloc(size_t(Qb) * P * k * 8));
   } else {
@@ -327,7 +363,8 @@ void search(cuvs::resources const& res_c,
                           ix.rotation_is_identity, cosine, rot_q, s);
     detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
                                  ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, s);
-    detail::launch_order_pairs(probes, nq * P, ix.n_lists, counters, order, s);
+    detail::launch_order_pairs(probes, chunk, ix.data_ptrs.as<const uint8_t*>(), nq * P, P,
+                               ix.n_lists, counters, order, desc, s);
     if (pl.fused) { detail::launch_fill_u32(kth, 0xFFFFFFFFu, nq, s); }
     mark(2);
 
@@ -339,9 +376,9 @@ void search(cuvs::resources const& res_c,
     sa.query_kth     = kth;
     sa.out_keys      = keys;
     sa.out_scores    = all_scores;
-    if (force_generic_scan() || !detail::launch_scan_fast(sa, work_ctr, s)) {
-      detail::launch_scan(sa, s);
-    }
+    sa.desc   = desc;
+    sa.timing = scan_timing_buffer();
+    if (!fast_scan || !detail::launch_scan_fast(sa, s)) { detail::launch_scan(sa, s); }
     mark(3);
 
     detail::merge_args ma{};
