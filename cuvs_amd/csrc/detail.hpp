@@ -213,9 +213,15 @@ void launch_scan(const scan_args& a, hipStream_t stream);
  *  arguments are outside what it covers.  Needs `a.desc`. */
 bool scan_fast_supported(const scan_args& a);
 bool launch_scan_fast(const scan_args& a, hipStream_t stream);
+/** CU-wide kernel for 8-bit codes, k <= 64 and fp16 / 8-bit tables (scan_quad.hip).  It writes
+ *  several candidate groups per pair: scan_quad_keys_per_pair() is the number of keys the output
+ *  buffer must hold per (query, probe) pair, 0 when the arguments are outside what it covers. */
+uint32_t scan_quad_keys_per_pair(const scan_args& a);
+bool launch_scan_quad(const scan_args& a, hipStream_t stream);
 
 struct merge_args {
   uint32_t n_queries, n_probes, k, max_samples;
+  uint32_t keys_per_pair;  // fused: candidate keys stored per (query, probe) pair
   int fused;
   int metric;
   float scaling;

@@ -549,7 +549,7 @@ __global__ __launch_bounds__(kBlock) void merge_kernel(merge_args a, uint32_t ou
   const uint32_t q        = blockIdx.x;
   uint32_t n;
   if (a.fused) {
-    n                              = a.n_probes * a.k;
+    n                              = a.n_probes * a.keys_per_pair;
     const unsigned long long* keys = a.in_keys + uint64_t(q) * n;
     block_select_sorted([keys](uint32_t i) { return keys[i]; }, n, a.k, out, out_cap, sm);
   } else {

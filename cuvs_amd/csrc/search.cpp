@@ -90,7 +90,7 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
   const size_t P = p.n_probes;
   p.per_query_bytes = size_t(ix.dim) * 4 + size_t(ix.n_lists) * 4 + size_t(ix.rot_dim) * 4 +
                       P * 4 * 3 + P * sizeof(detail::pair_desc) + 16 +
-                      (p.fused ? P * k * 8 : size_t(p.max_samples) * 4);
+                      (p.fused ? P * k * 8 * 4 : size_t(p.max_samples) * 4);
   p.fixed_bytes = a256(size_t(ix.n_lists) * 8 + 16) + 16 * 256;
   const size_t budget = workspace_budget(res);
   size_t b = budget > p.fixed_bytes ? (budget - p.fixed_bytes) / (p.per_query_bytes + 64) : 1;
@@ -321,12 +321,14 @@ void search(cuvs::resources const& res_c,
   unsigned long long* keys = nullptr;
   float* all_scores        = nullptr;
   sa.fused                 = pl.fused;
-  const bool fast_scan     = !force_generic_scan() && detail::scan_fast_supported(sa);
+  const uint32_t quad_kpp  = force_generic_scan() ? 0u : detail::scan_quad_keys_per_pair(sa);
+  const bool fast_scan     = !force_generic_scan() && (quad_kpp != 0 || detail::scan_fast_supported(sa));
+  const uint32_t kpp       = quad_kpp != 0 ? quad_kpp : k;  // candidate keys stored per pair
   if (fast_scan) {
     desc = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));
   }
   if (pl.fused) {
-    keys = static_cast<unsigned long long*>(res.workspace_alloc(size_t(Qb) * P * k * 8));
+    keys = static_cast<unsigned long long*>(res.workspace_alloc(size_t(Qb) * P * kpp * 8));
   } else {
     all_scores = static_cast<float*>(res.workspace_alloc(size_t(Qb) * pl.max_samples * 4));
   }
@@ -378,7 +380,9 @@ void search(cuvs::resources const& res_c,
     sa.out_scores    = all_scores;
     sa.desc   = desc;
     sa.timing = scan_timing_buffer();
-    if (!fast_scan || !detail::launch_scan_fast(sa, s)) { detail::launch_scan(sa, s); }
+    const bool launched = fast_scan && (quad_kpp != 0 ? detail::launch_scan_quad(sa, s)
+                                                      : detail::launch_scan_fast(sa, s));
+    if (!launched) { detail::launch_scan(sa, s); }
     mark(3);
 
     detail::merge_args ma{};
@@ -387,6 +391,7 @@ void search(cuvs::resources const& res_c,
     ma.k             = k;
     ma.max_samples   = pl.max_samples;
     ma.fused         = pl.fused;
+    ma.keys_per_pair = kpp;
     ma.metric        = int(ix.metric);
     ma.scaling       = scaling_factor(type);
     ma.in_keys       = keys;
