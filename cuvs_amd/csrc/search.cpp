@@ -156,7 +156,7 @@ unsigned long long* scan_timing_buffer()
     {
       unsigned long long h[6] = {};
       (void)hipMemcpy(h, d, 48, hipMemcpyDeviceToHost);
-      const char* names[6] = {"stage", "lut", "bar_lut", "scan", "bar_scan", "prune_out"};
+      const char* names[6] = {"phase0", "phase1", "phase2", "phase3", "phase4", "phase5"};
       unsigned long long total = 0;
       for (auto v : h) { total += v; }
       for (int i = 0; i < 6; i++) {
