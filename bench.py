@@ -21,6 +21,11 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 
+# HBM bytes per scan launch on the default workload, from hardware counters (FETCH_SIZE + WRITE_SIZE
+# per dispatch, each scaled by its reading for the 1 GiB calibration copy below); the counter runs
+# are summarised under profiles/.  Keyed by (lut, internal); None where not measured.
+MEASURED_SCAN_TRAFFIC = {("f16", "f32"): 6.50e9, ("fp8", "f32"): 6.35e9}
+
 
 def log(msg):
     print(f"[bench {time.strftime('%H:%M:%S')}] {msg}", file=sys.stderr, flush=True)
@@ -131,6 +136,18 @@ def main():
         f"coarse {stage['coarse_ms']:.2f} rotate {stage['rotate_ms']:.2f} scan {stage['scan_ms']:.2f} "
         f"merge {stage['merge_ms']:.2f} ms")
 
+    # A plain copy of known size (1 GiB read + 1 GiB written), outside every timed region: it gives
+    # hardware-counter runs of this same command the reading of FETCH_SIZE / WRITE_SIZE per byte.
+    calib = torch.zeros(2 ** 28, dtype=torch.int32, device=dev)
+    calib_out = torch.empty_like(calib)
+    torch.add(calib, 1, out=calib_out)
+    torch.cuda.synchronize()
+    del calib, calib_out
+
+    default_workload = (n, nq, n_lists, P, k) == (10_000_000, 10_000, 16384, 64, 10)
+    traffic = MEASURED_SCAN_TRAFFIC.get((args.lut, args.internal)) if default_workload else None
+    scan_name = "scan_quad_kernel" if (args.lut != "f32" and k <= 64) else "scan_fast_kernel"
+
     out = {
         "metric": "QPS@recall@10 (10M x 128 IVF-PQ, batch 10k); code-scan HBM GB/s vs peak",
         "value": qps, "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -146,8 +163,8 @@ def main():
                    "recall_at_k": gpu_recall,
                    "stage_ms": {s: stage[s] for s in ("coarse_ms", "rotate_ms", "scan_ms", "merge_ms")}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "scan_kernel", "kernel_ms": scan_avg_ms,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "kernel": scan_name, "kernel_ms": scan_avg_ms,
                      "algorithmic_bytes_per_launch": bytes_per_launch},
     }
 
