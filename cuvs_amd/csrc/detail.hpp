@@ -174,12 +174,15 @@ struct pair_desc {
 static_assert(sizeof(pair_desc) == 32, "pair_desc must stay 32 bytes");
 
 /** pair_order = ids of the (query, probe) pairs grouped by probed list; when `desc` is non-null the
- *  record of every pair is written at the same position.  `counters` is scratch of
- *  2 * n_lists + 2 words. */
+ *  record of every pair is written at the same position.  With `lead_probes` < n_probes the pairs
+ *  of each query's first `lead_probes` probes come first (n_queries * lead_probes records, grouped
+ *  by list) and the others after them (grouped by list again); `alive`, when non-null, gets one
+ *  byte per pair slot: 1 for the leading pairs, 0 for the others.  `counters` is scratch of
+ *  4 * n_lists + 4 words. */
 void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
                         const uint8_t* const* data_ptrs, uint32_t n_pairs, uint32_t n_probes,
                         uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
-                        pair_desc* desc, hipStream_t stream);
+                        pair_desc* desc, uint32_t lead_probes, uint8_t* alive, hipStream_t stream);
 
 struct scan_args {
   uint32_t n_queries, n_probes, k, max_samples;
@@ -198,7 +201,9 @@ struct scan_args {
   const uint32_t* probes;         // [n_queries, n_probes]
   const uint32_t* chunk_indices;  // [n_queries, n_probes]
   const uint32_t* pair_order;     // [n_queries * n_probes] or null
-  const pair_desc* desc;          // [n_queries * n_probes] records in pair_order order, or null
+  const pair_desc* desc;          // records of the pairs to scan, in launch order, or null
+  uint32_t n_pairs;               // number of records in `desc` (persistent kernels)
+  const uint32_t* n_pairs_dev;    // when non-null the number of records is read from here instead
   const uint32_t* filter_bits;    // or null
   int64_t filter_nbits;
   uint32_t* query_kth;            // [n_queries] ordered-score upper bounds (fused)
@@ -219,6 +224,24 @@ bool launch_scan_fast(const scan_args& a, hipStream_t stream);
 uint32_t scan_quad_keys_per_pair(const scan_args& a);
 bool launch_scan_quad(const scan_args& a, hipStream_t stream);
 
+/**
+ * Early termination for L2 metrics, as compute_score's early stop in the reference
+ * (cpp/src/neighbors/ivf_pq/detail/jit_lto_kernels/compute_score_impl.cuh:70-74): a row whose
+ * partial sum over the first subspaces already exceeds the query's current k-th best score cannot
+ * enter the result.  The screen kernel (scan_screen.hip) builds the lookup table of the first 16
+ * subspaces only, sums the first 16-byte chunk of every row of a pair and keeps the pair only if
+ * some row is still below the query's bound; surviving records are appended to `survivors`
+ * (`n_survivors` counts them) and their slot is marked in `alive`.
+ */
+bool scan_screen_supported(const scan_args& a);
+void launch_scan_screen(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
+                        pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
+                        hipStream_t stream);
+/** query_kth[q] = min(query_kth[q], score of the k-th smallest valid key among the first `n_keys`
+ *  keys of query q's candidate block (`keys_per_query` keys apart)). */
+void launch_kth_bound(const unsigned long long* keys, uint32_t n_queries, uint64_t keys_per_query,
+                      uint32_t n_keys, uint32_t k, uint32_t* query_kth, hipStream_t stream);
+
 struct merge_args {
   uint32_t n_queries, n_probes, k, max_samples;
   uint32_t keys_per_pair;  // fused: candidate keys stored per (query, probe) pair
@@ -226,6 +249,7 @@ struct merge_args {
   int metric;
   float scaling;
   const unsigned long long* in_keys;  // fused
+  const uint8_t* alive;               // fused: per pair slot, 0 = no keys were written (or null: all)
   const float* in_scores;             // non-fused
   const uint32_t* n_samples;
   const uint32_t* probes;

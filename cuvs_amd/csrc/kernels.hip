@@ -262,11 +262,19 @@ __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __res
   }
 }
 
+/** Sort key of pair i: its list, the pairs past each query's leading probes in a second range. */
+__device__ __forceinline__ uint32_t pair_bin(uint32_t label, uint32_t i, uint32_t n_probes,
+                                             uint32_t lead_probes, uint32_t n_lists)
+{
+  return (i % n_probes) < lead_probes ? label : label + n_lists;
+}
+
 __global__ void pair_histogram_kernel(const uint32_t* __restrict__ probes, uint32_t n_pairs,
+                                      uint32_t n_probes, uint32_t lead_probes, uint32_t n_lists,
                                       uint32_t* __restrict__ counts)
 {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n_pairs) { atomicAdd(&counts[probes[i]], 1u); }
+  if (i < n_pairs) { atomicAdd(&counts[pair_bin(probes[i], i, n_probes, lead_probes, n_lists)], 1u); }
 }
 
 /** Single block: cursors[l] = exclusive prefix sum of counts[l]. */
@@ -297,14 +305,17 @@ __global__ __launch_bounds__(kBlock) void exclusive_scan_kernel(const uint32_t* 
 __global__ void pair_scatter_kernel(const uint32_t* __restrict__ probes,
                                     const uint32_t* __restrict__ chunk_indices,
                                     const uint8_t* const* __restrict__ data_ptrs, uint32_t n_pairs,
-                                    uint32_t n_probes, uint32_t* __restrict__ cursors,
-                                    uint32_t* __restrict__ pair_order, pair_desc* __restrict__ desc)
+                                    uint32_t n_probes, uint32_t lead_probes, uint32_t n_lists,
+                                    uint32_t* __restrict__ cursors,
+                                    uint32_t* __restrict__ pair_order, pair_desc* __restrict__ desc,
+                                    uint8_t* __restrict__ alive)
 {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n_pairs) {
     const uint32_t label = probes[i];
-    const uint32_t pos   = atomicAdd(&cursors[label], 1u);
+    const uint32_t pos   = atomicAdd(&cursors[pair_bin(label, i, n_probes, lead_probes, n_lists)], 1u);
     pair_order[pos]      = i;
+    if (alive != nullptr) { alive[i] = (i % n_probes) < lead_probes ? 1 : 0; }
     if (desc != nullptr) {
       const uint32_t q   = i / n_probes;
       const uint32_t p   = i - q * n_probes;
@@ -541,6 +552,27 @@ __device__ __forceinline__ float postprocess_distance(float d, int metric, float
   }
 }
 
+/** One wave per query: the k-th smallest valid key among the first n_keys keys of the query's
+ *  candidate block bounds the query's final k-th score from above. */
+constexpr uint32_t kKthMaxKeys = 1024;
+__global__ __launch_bounds__(64) void kth_bound_kernel(const unsigned long long* __restrict__ keys,
+                                                       uint64_t keys_per_query, uint32_t n_keys,
+                                                       uint32_t k, uint32_t* __restrict__ query_kth)
+{
+  __shared__ unsigned long long s[kKthMaxKeys];
+  const uint32_t q               = blockIdx.x;
+  const unsigned long long* mine = keys + uint64_t(q) * keys_per_query;
+  for (uint32_t i = threadIdx.x; i < n_keys; i += 64u) { s[i] = mine[i]; }
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < n_keys; i += 64u) {
+    const unsigned long long key = s[i];
+    if (key == kInvalidKey) { continue; }
+    uint32_t rank = 0;  // keys are distinct: the sample number is part of the key
+    for (uint32_t j = 0; j < n_keys; j++) { rank += s[j] < key ? 1u : 0u; }
+    if (rank == k - 1u) { atomicMin(&query_kth[q], uint32_t(key >> 32)); }
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void merge_kernel(merge_args a, uint32_t out_cap)
 {
   extern __shared__ __align__(16) unsigned char dyn_smem[];
@@ -551,7 +583,16 @@ __global__ __launch_bounds__(kBlock) void merge_kernel(merge_args a, uint32_t ou
   if (a.fused) {
     n                              = a.n_probes * a.keys_per_pair;
     const unsigned long long* keys = a.in_keys + uint64_t(q) * n;
-    block_select_sorted([keys](uint32_t i) { return keys[i]; }, n, a.k, out, out_cap, sm);
+    if (a.alive == nullptr) {
+      block_select_sorted([keys](uint32_t i) { return keys[i]; }, n, a.k, out, out_cap, sm);
+    } else {
+      // pairs that the screen dropped wrote no keys
+      const uint8_t* alive = a.alive + uint64_t(q) * a.n_probes;
+      const uint32_t kpp   = a.keys_per_pair;
+      block_select_sorted(
+        [keys, alive, kpp](uint32_t i) { return alive[i / kpp] != 0 ? keys[i] : kInvalidKey; }, n,
+        a.k, out, out_cap, sm);
+    }
   } else {
     n                = a.n_samples[q];
     const float* row = a.in_scores + uint64_t(q) * a.max_samples;
@@ -849,18 +890,21 @@ void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, ui
 void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
                         const uint8_t* const* data_ptrs, uint32_t n_pairs, uint32_t n_probes,
                         uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
-                        pair_desc* desc, hipStream_t stream)
+                        pair_desc* desc, uint32_t lead_probes, uint8_t* alive, hipStream_t stream)
 {
   if (n_pairs == 0) { return; }
-  uint32_t* counts  = counters;
-  uint32_t* cursors = counters + n_lists;
-  launch_fill_u32(counts, 0, n_lists, stream);
-  pair_histogram_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(probes, n_pairs, counts);
+  const uint32_t n_bins = lead_probes < n_probes ? 2 * n_lists : n_lists;
+  uint32_t* counts      = counters;
+  uint32_t* cursors     = counters + n_bins;
+  launch_fill_u32(counts, 0, n_bins, stream);
+  pair_histogram_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(probes, n_pairs, n_probes,
+                                                                      lead_probes, n_lists, counts);
   CUVS_LAUNCH_CHECK();
-  exclusive_scan_kernel<<<1, kBlock, 0, stream>>>(counts, n_lists, cursors);
+  exclusive_scan_kernel<<<1, kBlock, 0, stream>>>(counts, n_bins, cursors);
   CUVS_LAUNCH_CHECK();
   pair_scatter_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(
-    probes, chunk_indices, data_ptrs, n_pairs, n_probes, cursors, pair_order, desc);
+    probes, chunk_indices, data_ptrs, n_pairs, n_probes, lead_probes, n_lists, cursors, pair_order,
+    desc, alive);
   CUVS_LAUNCH_CHECK();
 }
 
@@ -949,6 +993,14 @@ void launch_merge(const merge_args& a, hipStream_t stream)
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
   }
   merge_kernel<<<a.n_queries, kBlock, smem, stream>>>(a, out_cap);
+  CUVS_LAUNCH_CHECK();
+}
+
+void launch_kth_bound(const unsigned long long* keys, uint32_t n_queries, uint64_t keys_per_query,
+                      uint32_t n_keys, uint32_t k, uint32_t* query_kth, hipStream_t stream)
+{
+  if (n_queries == 0 || n_keys < k || n_keys > kKthMaxKeys) { return; }  // no bound: nothing is pruned
+  kth_bound_kernel<<<n_queries, 64, 0, stream>>>(keys, keys_per_query, n_keys, k, query_kth);
   CUVS_LAUNCH_CHECK();
 }
 

@@ -104,9 +104,10 @@ __global__ __launch_bounds__(kQuadThreads, 4) void scan_quad_kernel(scan_args a)
   const uint32_t wig     = wid - grp * WG;   // wave index inside its group
   const uint32_t code    = tid & 255u;       // codebook entry this thread builds
   const uint32_t quarter = wid >> 2;         // which quarter of the subspaces
-  const uint32_t n_pairs = a.n_queries * a.n_probes;
+  const uint32_t n_pairs = a.n_pairs_dev != nullptr ? *a.n_pairs_dev : a.n_pairs;
   const uint32_t n_quads = (n_pairs + G - 1u) / G;
   const uint32_t stride  = gridDim.x;
+  if (blockIdx.x >= n_quads) { return; }  // whole block, before any barrier
   auto* my_cand          = cand_all + wid * kWaveCap;
   auto* my_lut           = lut_all + grp * lut_entries;
 
@@ -245,19 +246,28 @@ __global__ __launch_bounds__(kQuadThreads, 4) void scan_quad_kernel(scan_args a)
           valid = id >= 0 && id < a.filter_nbits && ((a.filter_bits[id >> 5] >> (id & 31)) & 1u) != 0;
         }
         acc_t acc = acc_t(0);
+        // L2 sums only grow: once every row of the tile is past the bound the remaining chunks
+        // cannot bring any of them back (early stop of compute_score in the reference)
+        const uint32_t stop_bits = thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u;
+        bool live                = true;
 #pragma unroll
         for (int m = 0; m < NCH; m++) {
-          const uint32_t w[4] = {cur[m].x, cur[m].y, cur[m].z, cur[m].w};
+          if (live) {
+            const uint32_t w[4] = {cur[m].x, cur[m].y, cur[m].z, cur[m].w};
 #pragma unroll
-          for (int kk = 0; kk < 16; kk++) {
-            const uint32_t c = (w[kk >> 2] >> ((kk & 3) * 8)) & 0xffu;
-            const lut_t v    = my_lut[(m * 16 + kk) * 256 + c];
-            if (OUT_HALF) {
-              acc = acc_t(acc + traits::to_half(v));
-            } else if (LUT == LUT_F16) {
-              acc = acc_t(fmaf(traits::to_float(v), one, float(acc)));
-            } else {
-              acc = acc_t(acc + traits::to_float(v));
+            for (int kk = 0; kk < 16; kk++) {
+              const uint32_t c = (w[kk >> 2] >> ((kk & 3) * 8)) & 0xffu;
+              const lut_t v    = my_lut[(m * 16 + kk) * 256 + c];
+              if (OUT_HALF) {
+                acc = acc_t(acc + traits::to_half(v));
+              } else if (LUT == LUT_F16) {
+                acc = acc_t(fmaf(traits::to_float(v), one, float(acc)));
+              } else {
+                acc = acc_t(acc + traits::to_float(v));
+              }
+            }
+            if (!IP && m + 1 < NCH) {
+              live = __ballot(valid && !(__float_as_uint(float(acc)) > stop_bits)) != 0ull;
             }
           }
         }
@@ -331,10 +341,12 @@ void launch_quad_instance(const scan_args& a, hipStream_t stream)
     CUVS_HIP_TRY(hipGetDevice(&dev));
     CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
   }
-  const uint32_t n_pairs = a.n_queries * a.n_probes;
-  const uint32_t n_quads = (n_pairs + G - 1) / G;
-  uint32_t grid          = uint32_t(n_cu);
-  if (grid > n_quads) { grid = n_quads; }
+  uint32_t grid = uint32_t(n_cu);
+  if (a.n_pairs_dev == nullptr) {
+    const uint32_t n_quads = (a.n_pairs + G - 1) / G;
+    if (grid > n_quads) { grid = n_quads; }
+    if (grid == 0) { return; }
+  }
   kernel<<<grid, kQuadThreads, smem, stream>>>(a);
   CUVS_HIP_TRY(hipGetLastError());
 }

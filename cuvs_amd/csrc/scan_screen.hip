@@ -1,0 +1,279 @@
+/*
+ * Screening pass of the L2 early stop (8-bit codes).
+ *
+ * A row's score is a sum of non-negative table entries taken in subspace order, so the partial sum
+ * over the first 16 subspaces (the first 16-byte chunk of the row) is a lower bound of its final
+ * score, and it is exactly the intermediate value the full scan kernels reach after that chunk.  A
+ * pair none of whose rows is still at or below the query's current k-th best score after that chunk
+ * cannot contribute a result (compute_score's early stop in the reference,
+ * cpp/src/neighbors/ivf_pq/detail/jit_lto_kernels/compute_score_impl.cuh:70-74, applied to the whole
+ * list at once).  For clustered data this removes most (query, probe) pairs at a quarter of the
+ * table-building and gather work or less, and only the survivors go through the full scan.
+ *
+ * Organisation: persistent 256-thread blocks, several per CU so that the table-building phase of
+ * one block overlaps the gather phase of another.  A block takes G = 4 pairs per iteration; thread
+ * c keeps entry c of the first 16 subspaces' codebooks in registers and builds entry c of the four
+ * 16 x 256 tables; then wave g scans the first chunk of every row of pair g and stops at the first
+ * tile with a row still in play.
+ */
+#include "device_utils.cuh"
+
+namespace cuvs::neighbors::ivf_pq::detail {
+
+namespace {
+
+#define LDS_AS __attribute__((address_space(3)))
+#define GLOBAL_AS __attribute__((address_space(1)))
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t kScreenThreads = 256;
+constexpr uint32_t kScreenG       = 4;   // pairs per block iteration = waves per block
+constexpr uint32_t kScreenSub     = 16;  // subspaces in the first chunk of 8-bit codes
+constexpr uint32_t kScreenLdsBase = 16;  // no LDS object at address 0: a null constant pointer folds badly
+
+__device__ __forceinline__ void lds_barrier_s()
+{
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+__device__ __forceinline__ float opaque_one_s()
+{
+  float one = 1.0f;
+  asm volatile("" : "+v"(one));
+  return one;
+}
+
+template <int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER>
+__global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
+  scan_args a, const pair_desc* __restrict__ desc, uint32_t n_pairs, uint32_t group_bytes,
+  pair_desc* __restrict__ survivors, uint32_t* __restrict__ n_survivors, uint8_t* __restrict__ alive)
+{
+  using traits = lut_traits<LUT>;
+  using lut_t  = typename traits::storage;
+  using acc_t  = typename std::conditional<OUT_HALF, _Float16, float>::type;
+  constexpr uint32_t G           = kScreenG;
+  constexpr uint32_t SUB         = kScreenSub;
+  constexpr uint32_t NDIFF       = SUB * PQ_LEN;  // leading rotated dimensions the first chunk covers
+  constexpr uint32_t lut_entries = SUB * 256u;
+  constexpr uint32_t off_diff    = kScreenLdsBase + G * lut_entries * uint32_t(sizeof(lut_t));
+  static_assert(G * NDIFF <= kScreenThreads, "one thread stages one (pair, dimension)");
+  auto* lut_all  = reinterpret_cast<LDS_AS lut_t*>(uintptr_t(kScreenLdsBase));
+  auto* diff_all = reinterpret_cast<LDS_AS float*>(uintptr_t(off_diff));
+  const float one = opaque_one_s();
+
+  const uint32_t tid     = threadIdx.x;
+  const uint32_t lane    = tid & 63u;
+  const uint32_t wid     = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t n_iters = (n_pairs + G - 1u) / G;
+  const uint32_t stride  = gridDim.x;
+  if (blockIdx.x >= n_iters) { return; }
+  auto* my_lut = lut_all + wid * lut_entries;
+
+  float book[PER_CLUSTER ? 1 : SUB][PQ_LEN];
+  if (!PER_CLUSTER) {
+#pragma unroll
+    for (uint32_t j = 0; j < SUB; j++) {
+#pragma unroll
+      for (int t = 0; t < PQ_LEN; t++) { book[j][t] = a.pq_centers[(j * PQ_LEN + t) * 256 + tid]; }
+    }
+  }
+
+  auto record = [&](uint32_t it, uint32_t g) -> pair_desc {
+    const uint32_t slot = it * G + g;
+    pair_desc d         = desc[slot < n_pairs ? slot : n_pairs - 1u];
+    if (slot >= n_pairs) { d.n_rows = 0; d.slot = 0xFFFFFFFFu; }
+    return d;
+  };
+  auto chunk_ptr = [&](const uint8_t* list_data, uint32_t row) {
+    return reinterpret_cast<const GLOBAL_AS u32x4*>(reinterpret_cast<uintptr_t>(list_data) +
+                                                    uint64_t(row >> 5) * group_bytes +
+                                                    uint64_t(row & 31u) * 16u);
+  };
+  // staging element (pair tid / NDIFF, dimension tid % NDIFF) of iteration `it`
+  auto fetch_diff = [&](uint32_t it) -> float {
+    float v = 0.0f;
+    if (tid < G * NDIFF) {
+      const pair_desc d = record(it, tid / NDIFF);
+      if (d.n_rows != 0) {
+        v = a.rot_q[uint64_t(d.q) * a.rot_dim + tid % NDIFF] -
+            a.centers_rot[uint64_t(d.label) * a.rot_dim + tid % NDIFF];
+      }
+    }
+    return v;
+  };
+
+  uint32_t it   = blockIdx.x;
+  float staged  = fetch_diff(it);
+  pair_desc my_d = record(it, wid);
+  u32x4 cur      = {0u, 0u, 0u, 0u};
+  uint32_t thr   = 0xFFFFFFFFu;
+  if (my_d.n_rows != 0) {
+    cur = *chunk_ptr(my_d.data, lane < my_d.n_rows ? lane : 0u);
+    thr = a.query_kth[my_d.q];
+  }
+  if (tid < G * NDIFF) { diff_all[tid] = staged; }
+  lds_barrier_s();
+
+  for (;;) {
+    const bool has_next    = it + stride < n_iters;
+    const uint32_t nxt_it  = has_next ? it + stride : it;
+    if (has_next) { staged = fetch_diff(nxt_it); }
+    const pair_desc nxt_d = record(nxt_it, wid);
+
+    /* ---- the G tables of the first chunk, entry `tid` of each subspace ---- */
+#pragma unroll
+    for (uint32_t g = 0; g < G; g++) {
+      const pair_desc dg = record(it, g);
+      if (dg.n_rows == 0) { continue; }  // uniform
+      float cb[PQ_LEN];
+      if (PER_CLUSTER) {
+#pragma unroll
+        for (int t = 0; t < PQ_LEN; t++) { cb[t] = a.pq_centers[(uint64_t(dg.label) * PQ_LEN + t) * 256 + tid]; }
+      }
+      const auto* diff = diff_all + g * NDIFF;
+      auto* lut        = lut_all + g * lut_entries;
+#pragma unroll
+      for (uint32_t j = 0; j < SUB; j++) {
+        float score = 0.0f;
+#pragma unroll
+        for (int t = 0; t < PQ_LEN; t++) {
+          const float pqc = PER_CLUSTER ? cb[t] : book[PER_CLUSTER ? 0 : j][t];
+          float df        = diff[j * PQ_LEN + t];
+          df -= pqc;
+          score = fmaf(df, df, score);
+        }
+        lut[j * 256 + tid] = traits::encode(score);
+      }
+    }
+    lds_barrier_s();  // tables complete; the staged terms are free again
+    if (has_next && tid < G * NDIFF) { diff_all[tid] = staged; }
+
+    /* ---- wave `wid` sums the first chunk of every row of its pair ---- */
+    if (my_d.slot != 0xFFFFFFFFu) {
+      const uint32_t n_rows    = my_d.n_rows;
+      const uint32_t n_tiles   = (n_rows + 63u) >> 6;
+      const uint32_t stop_bits = thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u;
+      bool in_play             = false;
+      for (uint32_t tile = 0; tile < n_tiles && !in_play; tile++) {
+        const uint32_t i = tile * 64u + lane;
+        u32x4 ahead      = cur;
+        if (tile + 1u < n_tiles) {
+          const uint32_t in = i + 64u;
+          ahead             = *chunk_ptr(my_d.data, in < n_rows ? in : 0u);
+        }
+        const uint32_t w[4] = {cur.x, cur.y, cur.z, cur.w};
+        acc_t acc           = acc_t(0);
+#pragma unroll
+        for (int kk = 0; kk < 16; kk++) {
+          const uint32_t c = (w[kk >> 2] >> ((kk & 3) * 8)) & 0xffu;
+          const lut_t v    = my_lut[kk * 256 + c];
+          if (OUT_HALF) {
+            acc = acc_t(acc + traits::to_half(v));
+          } else if (LUT == LUT_F16) {
+            acc = acc_t(fmaf(traits::to_float(v), one, float(acc)));
+          } else {
+            acc = acc_t(acc + traits::to_float(v));
+          }
+        }
+        in_play = __ballot(i < n_rows && !(__float_as_uint(float(acc)) > stop_bits)) != 0ull;
+        cur     = ahead;
+      }
+      if (lane == 0) {
+        if (in_play) {
+          const uint32_t pos = atomicAdd(n_survivors, 1u);
+          survivors[pos]     = my_d;
+          alive[my_d.slot]   = 1;
+        }
+      }
+    }
+
+    if (!has_next) { break; }
+    my_d = nxt_d;
+    thr  = 0xFFFFFFFFu;
+    if (my_d.n_rows != 0) {
+      cur = *chunk_ptr(my_d.data, lane < my_d.n_rows ? lane : 0u);
+      thr = a.query_kth[my_d.q];
+    }
+    it = nxt_it;
+    lds_barrier_s();  // every wave is done with the tables; next staged terms are visible
+  }
+}
+
+template <int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER>
+void launch_screen_instance(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
+                            pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
+                            hipStream_t stream)
+{
+  using lut_t       = typename lut_traits<LUT>::storage;
+  auto kernel       = scan_screen_kernel<PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>;
+  const size_t smem = kScreenLdsBase + size_t(kScreenG) * kScreenSub * 256 * sizeof(lut_t) +
+                      size_t(kScreenG) * kScreenSub * PQ_LEN * 4;
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+    int dev = 0;
+    CUVS_HIP_TRY(hipGetDevice(&dev));
+    CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+  }
+  const uint32_t n_iters = (n_pairs + kScreenG - 1) / kScreenG;
+  uint32_t grid          = uint32_t(n_cu) * 4u;
+  if (grid > n_iters) { grid = n_iters; }
+  const uint32_t n_chunks    = (a.pq_dim + 15u) / 16u;
+  const uint32_t group_bytes = n_chunks * 512u;
+  kernel<<<grid, kScreenThreads, smem, stream>>>(a, desc, n_pairs, group_bytes, survivors, n_survivors,
+                                                 alive);
+  CUVS_HIP_TRY(hipGetLastError());
+}
+
+template <int PQ_LEN, bool PER_CLUSTER>
+void launch_screen_types(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
+                         pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive, hipStream_t s)
+{
+  if (!a.out_half) {
+    if (a.lut_dtype == CUDA_R_16F) {
+      launch_screen_instance<PQ_LEN, LUT_F16, false, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, s);
+    } else {
+      launch_screen_instance<PQ_LEN, LUT_FP8U, false, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, s);
+    }
+  } else {
+    if (a.lut_dtype == CUDA_R_16F) {
+      launch_screen_instance<PQ_LEN, LUT_F16, true, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, s);
+    } else {
+      launch_screen_instance<PQ_LEN, LUT_FP8U, true, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, s);
+    }
+  }
+}
+
+}  // namespace
+
+bool scan_screen_supported(const scan_args& a)
+{
+  const bool l2 = a.metric == int(DistanceType::L2Expanded) || a.metric == int(DistanceType::L2SqrtExpanded);
+  if (!l2 || !a.fused || a.pq_bits != 8 || a.pq_dim < 32) { return false; }
+  if (a.lut_dtype != CUDA_R_16F && a.lut_dtype != CUDA_R_8U) { return false; }
+  return a.pq_len == 2 || a.pq_len == 4;
+}
+
+void launch_scan_screen(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
+                        pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
+                        hipStream_t stream)
+{
+  CUVS_EXPECTS(scan_screen_supported(a), "the screening pass does not cover these search arguments");
+  if (n_pairs == 0) { return; }
+  if (a.pq_len == 2) {
+    if (a.per_cluster) {
+      launch_screen_types<2, true>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+    } else {
+      launch_screen_types<2, false>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+    }
+  } else {
+    if (a.per_cluster) {
+      launch_screen_types<4, true>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+    } else {
+      launch_screen_types<4, false>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+    }
+  }
+}
+
+}  // namespace cuvs::neighbors::ivf_pq::detail

@@ -89,9 +89,9 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
   p.fused = k <= kMaxFusedK;
   const size_t P = p.n_probes;
   p.per_query_bytes = size_t(ix.dim) * 4 + size_t(ix.n_lists) * 4 + size_t(ix.rot_dim) * 4 +
-                      P * 4 * 3 + P * sizeof(detail::pair_desc) + 16 +
+                      P * 4 * 3 + P * (2 * sizeof(detail::pair_desc) + 1) + 16 +
                       (p.fused ? P * k * 8 * 4 : size_t(p.max_samples) * 4);
-  p.fixed_bytes = a256(size_t(ix.n_lists) * 8 + 16) + 16 * 256;
+  p.fixed_bytes = a256(size_t(ix.n_lists) * 16 + 16) + 16 * 256;
   const size_t budget = workspace_budget(res);
   size_t b = budget > p.fixed_bytes ? (budget - p.fixed_bytes) / (p.per_query_bytes + 64) : 1;
   b        = std::max<size_t>(b, 1);
@@ -129,6 +129,17 @@ void validate(const search_params& params, const index_impl& ix, int64_t k)
   CUVS_EXPECTS(k <= kMaxK, "parameter `k` (%lld) must not exceed %u", static_cast<long long>(k),
                kMaxK);
 }
+
+/** CUVS_AMD_NO_EARLY_STOP=1 scans every probed list in full (for A/B runs; read at every search). */
+bool early_stop_disabled()
+{
+  const char* e = std::getenv("CUVS_AMD_NO_EARLY_STOP");
+  return e != nullptr && e[0] == '1';
+}
+
+/** Probes per query whose lists are scanned in full before the others are screened against the
+ *  bound they give. */
+constexpr uint32_t kLeadProbes = 1;
 
 /** CUVS_AMD_GENERIC_SCAN=1 routes every search through the generic scan kernel (for A/B runs). */
 bool force_generic_scan()
@@ -316,7 +327,7 @@ void search(cuvs::resources const& res_c,
   auto* order     = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * P * 4));
   auto* n_samples = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * 4));
   auto* kth       = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * 4));
-  auto* counters  = static_cast<uint32_t*>(res.workspace_alloc(size_t(ix.n_lists) * 8 + 16));
+  auto* counters  = static_cast<uint32_t*>(res.workspace_alloc(size_t(ix.n_lists) * 16 + 16));
   detail::pair_desc* desc = nullptr;
   unsigned long long* keys = nullptr;
   float* all_scores        = nullptr;
@@ -326,6 +337,18 @@ void search(cuvs::resources const& res_c,
   const uint32_t kpp       = quad_kpp != 0 ? quad_kpp : k;  // candidate keys stored per pair
   if (fast_scan) {
     desc = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));
+  }
+  // L2 early stop: lists of the leading probes in full, the others screened on their first chunk
+  const bool early_stop = quad_kpp != 0 && P > kLeadProbes && detail::scan_screen_supported(sa) &&
+                          !early_stop_disabled();
+  const uint32_t lead          = early_stop ? kLeadProbes : P;
+  detail::pair_desc* survivors = nullptr;
+  uint8_t* alive               = nullptr;
+  uint32_t* n_survivors        = nullptr;
+  if (early_stop) {
+    survivors   = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));
+    alive       = static_cast<uint8_t*>(res.workspace_alloc(size_t(Qb) * P));
+    n_survivors = static_cast<uint32_t*>(res.workspace_alloc(256));
   }
   if (pl.fused) {
     keys = static_cast<unsigned long long*>(res.workspace_alloc(size_t(Qb) * P * kpp * 8));
@@ -366,7 +389,7 @@ void search(cuvs::resources const& res_c,
     detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
                                  ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, s);
     detail::launch_order_pairs(probes, chunk, ix.data_ptrs.as<const uint8_t*>(), nq * P, P,
-                               ix.n_lists, counters, order, desc, s);
+                               ix.n_lists, counters, order, desc, lead, alive, s);
     if (pl.fused) { detail::launch_fill_u32(kth, 0xFFFFFFFFu, nq, s); }
     mark(2);
 
@@ -378,11 +401,29 @@ void search(cuvs::resources const& res_c,
     sa.query_kth     = kth;
     sa.out_keys      = keys;
     sa.out_scores    = all_scores;
-    sa.desc   = desc;
-    sa.timing = scan_timing_buffer();
-    const bool launched = fast_scan && (quad_kpp != 0 ? detail::launch_scan_quad(sa, s)
-                                                      : detail::launch_scan_fast(sa, s));
-    if (!launched) { detail::launch_scan(sa, s); }
+    sa.desc        = desc;
+    sa.n_pairs     = nq * P;
+    sa.n_pairs_dev = nullptr;
+    sa.timing      = scan_timing_buffer();
+    if (early_stop) {
+      // 1. the leading probes' lists in full: candidates and a first bound per query
+      sa.n_pairs = nq * lead;
+      CUVS_EXPECTS(detail::launch_scan_quad(sa, s), "scan kernel launch failed");
+      detail::launch_kth_bound(keys, nq, uint64_t(P) * kpp, lead * kpp, k, kth, s);
+      // 2. every other pair on its first chunk only
+      detail::launch_fill_u32(n_survivors, 0, 1, s);
+      detail::launch_scan_screen(sa, desc + size_t(nq) * lead, nq * (P - lead), survivors, n_survivors,
+                                 alive, s);
+      // 3. the pairs still in play, in full
+      sa.desc        = survivors;
+      sa.n_pairs     = 0;
+      sa.n_pairs_dev = n_survivors;
+      CUVS_EXPECTS(detail::launch_scan_quad(sa, s), "scan kernel launch failed");
+    } else {
+      const bool launched = fast_scan && (quad_kpp != 0 ? detail::launch_scan_quad(sa, s)
+                                                        : detail::launch_scan_fast(sa, s));
+      if (!launched) { detail::launch_scan(sa, s); }
+    }
     mark(3);
 
     detail::merge_args ma{};
@@ -395,6 +436,7 @@ void search(cuvs::resources const& res_c,
     ma.metric        = int(ix.metric);
     ma.scaling       = scaling_factor(type);
     ma.in_keys       = keys;
+    ma.alive         = alive;
     ma.in_scores     = all_scores;
     ma.n_samples     = n_samples;
     ma.probes        = probes;
