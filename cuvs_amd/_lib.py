@@ -65,7 +65,12 @@ class SearchProfileStruct(C.Structure):
     _fields_ = [("n_queries", C.c_uint32), ("n_probes", C.c_uint32), ("k", C.c_uint32),
                 ("n_scan_launches", C.c_uint32), ("coarse_ms", C.c_float),
                 ("rotate_ms", C.c_float), ("scan_ms", C.c_float), ("merge_ms", C.c_float),
-                ("total_ms", C.c_float), ("scan_bytes", C.c_uint64), ("scan_rows", C.c_uint64)]
+                ("total_ms", C.c_float), ("scan_bytes", C.c_uint64), ("scan_rows", C.c_uint64),
+                ("lead_scan_ms", C.c_float), ("screen_ms", C.c_float),
+                ("survivor_scan_ms", C.c_float), ("reserved_", C.c_float),
+                ("lead_bytes", C.c_uint64), ("screen_bytes", C.c_uint64),
+                ("survivor_bytes", C.c_uint64), ("n_screened_pairs", C.c_uint64),
+                ("n_surviving_pairs", C.c_uint64)]
 
 
 # every symbol include/cuvs/core/c_api.h and include/cuvs/neighbors/ivf_pq.h declare

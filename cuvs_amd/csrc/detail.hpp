@@ -158,7 +158,8 @@ void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries,
  *  When `stats` is non-null, adds the scanned bytes and rows to stats[0], stats[1]. */
 void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
                           uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
-                          uint32_t* n_samples, unsigned long long* stats, hipStream_t stream);
+                          uint32_t* n_samples, unsigned long long* stats, uint32_t lead_probes,
+                          hipStream_t stream);
 
 /** Everything the scan needs to know about one (query, probe) pair, gathered once so that the
  *  scan kernel reads one 32-byte record instead of chasing four dependent pointers. */

@@ -628,6 +628,15 @@ cuvsError_t cuvsAmdIvfPqGetSearchProfile(cuvsResources_t res, cuvsAmdIvfPqSearch
     profile->total_ms        = p.total_ms;
     profile->scan_bytes      = p.scan_bytes;
     profile->scan_rows       = p.scan_rows;
+    profile->lead_scan_ms      = p.lead_scan_ms;
+    profile->screen_ms         = p.screen_ms;
+    profile->survivor_scan_ms  = p.survivor_scan_ms;
+    profile->reserved_         = 0;
+    profile->lead_bytes        = p.lead_bytes;
+    profile->screen_bytes      = p.screen_bytes;
+    profile->survivor_bytes    = p.survivor_bytes;
+    profile->n_screened_pairs  = p.n_screened_pairs;
+    profile->n_surviving_pairs = p.n_surviving_pairs;
   });
 }
 

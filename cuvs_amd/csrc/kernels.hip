@@ -235,17 +235,19 @@ __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __res
                                                             uint32_t row_chunk_bytes,
                                                             uint32_t* __restrict__ chunk_indices,
                                                             uint32_t* __restrict__ n_samples,
-                                                            unsigned long long* stats)
+                                                            unsigned long long* stats,
+                                                            uint32_t lead_probes)
 {
   const uint32_t q    = blockIdx.x;
   const uint32_t lane = threadIdx.x;
   uint32_t carry      = 0;
-  unsigned long long padded_rows = 0;
+  unsigned long long padded_rows = 0, lead_rows = 0;
   for (uint32_t p0 = 0; p0 < n_probes; p0 += 64) {
     const uint32_t p = p0 + lane;
     uint32_t sz      = 0;
     if (p < n_probes) { sz = list_sizes[probes[uint64_t(q) * n_probes + p]]; }
     padded_rows += (sz + 31u) & ~31u;
+    if (p < lead_probes) { lead_rows += (sz + 31u) & ~31u; }
     const uint32_t incl = wave_inclusive_scan(sz) + carry;
     if (p < n_probes) { chunk_indices[uint64_t(q) * n_probes + p] = incl; }
     carry = __shfl(incl, 63, 64);
@@ -254,10 +256,14 @@ __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __res
   if (stats != nullptr) {
     // wave reduction of the padded row count
 #pragma unroll
-    for (int d = 32; d > 0; d >>= 1) { padded_rows += __shfl_down(padded_rows, d, 64); }
+    for (int d = 32; d > 0; d >>= 1) {
+      padded_rows += __shfl_down(padded_rows, d, 64);
+      lead_rows += __shfl_down(lead_rows, d, 64);
+    }
     if (lane == 0) {
       atomicAdd(&stats[0], padded_rows * row_chunk_bytes);
       atomicAdd(&stats[1], static_cast<unsigned long long>(carry));
+      atomicAdd(&stats[2], lead_rows * row_chunk_bytes);
     }
   }
 }
@@ -879,11 +885,12 @@ void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries,
 
 void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
                           uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
-                          uint32_t* n_samples, unsigned long long* stats, hipStream_t stream)
+                          uint32_t* n_samples, unsigned long long* stats, uint32_t lead_probes,
+                          hipStream_t stream)
 {
   if (n_queries == 0) { return; }
   chunk_indices_kernel<<<n_queries, 64, 0, stream>>>(list_sizes, probes, n_probes, row_chunk_bytes,
-                                                     chunk_indices, n_samples, stats);
+                                                     chunk_indices, n_samples, stats, lead_probes);
   CUVS_LAUNCH_CHECK();
 }
 

@@ -9,11 +9,12 @@
 #include <algorithm>
 #include <cstdlib>
 #include <limits>
+#include <vector>
 
 namespace cuvs {
 
 struct resources::profile_state {
-  hipEvent_t ev[5]            = {};
+  hipEvent_t ev[7]            = {};
   unsigned long long* d_stats = nullptr;
 };
 
@@ -363,10 +364,10 @@ void search(cuvs::resources const& res_c,
     if (res.prof == nullptr) {
       res.prof = new cuvs::resources::profile_state();
       for (auto& e : res.prof->ev) { CUVS_HIP_TRY(hipEventCreate(&e)); }
-      CUVS_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&res.prof->d_stats), 16));
+      CUVS_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&res.prof->d_stats), 32));
     }
     d_stats = res.prof->d_stats;
-    detail::launch_fill_u32(reinterpret_cast<uint32_t*>(d_stats), 0, 4, s);
+    detail::launch_fill_u32(reinterpret_cast<uint32_t*>(d_stats), 0, 8, s);
     res.last_profile           = cuvs::search_profile{};
     res.last_profile.n_queries = uint32_t(n_queries);
     res.last_profile.n_probes  = P;
@@ -387,7 +388,7 @@ void search(cuvs::resources const& res_c,
     detail::launch_rotate(qf, ix.rotation_t.as<float>(), nq, ix.dim, ix.rot_dim,
                           ix.rotation_is_identity, cosine, rot_q, s);
     detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
-                                 ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, s);
+                                 ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead, s);
     detail::launch_order_pairs(probes, chunk, ix.data_ptrs.as<const uint8_t*>(), nq * P, P,
                                ix.n_lists, counters, order, desc, lead, alive, s);
     if (pl.fused) { detail::launch_fill_u32(kth, 0xFFFFFFFFu, nq, s); }
@@ -410,10 +411,12 @@ void search(cuvs::resources const& res_c,
       sa.n_pairs = nq * lead;
       CUVS_EXPECTS(detail::launch_scan_quad(sa, s), "scan kernel launch failed");
       detail::launch_kth_bound(keys, nq, uint64_t(P) * kpp, lead * kpp, k, kth, s);
+      mark(5);
       // 2. every other pair on its first chunk only
       detail::launch_fill_u32(n_survivors, 0, 1, s);
       detail::launch_scan_screen(sa, desc + size_t(nq) * lead, nq * (P - lead), survivors, n_survivors,
                                  alive, s);
+      mark(6);
       // 3. the pairs still in play, in full
       sa.desc        = survivors;
       sa.n_pairs     = 0;
@@ -460,14 +463,39 @@ void search(cuvs::resources const& res_c,
       lp.merge_ms += ms[3];
       lp.total_ms += ms[0] + ms[1] + ms[2] + ms[3];
       lp.n_scan_launches += 1;
+      if (early_stop) {
+        float lead_ms = 0, screen_ms = 0, surv_ms = 0;
+        CUVS_HIP_TRY(hipEventElapsedTime(&lead_ms, res.prof->ev[2], res.prof->ev[5]));
+        CUVS_HIP_TRY(hipEventElapsedTime(&screen_ms, res.prof->ev[5], res.prof->ev[6]));
+        CUVS_HIP_TRY(hipEventElapsedTime(&surv_ms, res.prof->ev[6], res.prof->ev[3]));
+        lp.lead_scan_ms += lead_ms;
+        lp.screen_ms += screen_ms;
+        lp.survivor_scan_ms += surv_ms;
+        // which pairs survived: their records are still in the workspace
+        uint32_t n_surv = 0;
+        CUVS_HIP_TRY(hipMemcpy(&n_surv, n_survivors, 4, hipMemcpyDeviceToHost));
+        std::vector<detail::pair_desc> h_surv(n_surv);
+        if (n_surv != 0) {
+          CUVS_HIP_TRY(hipMemcpy(h_surv.data(), survivors, size_t(n_surv) * sizeof(detail::pair_desc),
+                                 hipMemcpyDeviceToHost));
+        }
+        const uint64_t row_bytes = uint64_t(ix.n_chunks) * kIndexGroupVecLen;
+        for (const auto& d : h_surv) { lp.survivor_bytes += uint64_t((d.n_rows + 31u) & ~31u) * row_bytes; }
+        lp.n_surviving_pairs += n_surv;
+        lp.n_screened_pairs += uint64_t(nq) * (P - lead);
+      }
     }
   }
   if (prof) {
-    unsigned long long h[2] = {0, 0};
-    CUVS_HIP_TRY(hipMemcpyAsync(h, d_stats, 16, hipMemcpyDeviceToHost, s));
+    unsigned long long h[4] = {0, 0, 0, 0};
+    CUVS_HIP_TRY(hipMemcpyAsync(h, d_stats, 32, hipMemcpyDeviceToHost, s));
     CUVS_HIP_TRY(hipStreamSynchronize(s));
     res.last_profile.scan_bytes = h[0];
     res.last_profile.scan_rows  = h[1];
+    if (early_stop) {
+      res.last_profile.lead_bytes   = h[2];
+      res.last_profile.screen_bytes = (h[0] - h[2]) / ix.n_chunks;  // one 16-byte chunk per row
+    }
   }
   res.reset_workspace();
 }

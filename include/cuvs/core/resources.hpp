@@ -49,6 +49,15 @@ struct search_profile {
   float total_ms           = 0;
   uint64_t scan_bytes      = 0;
   uint64_t scan_rows       = 0;
+  // L2 early stop: the scan stage split into its three launches (zero when not used)
+  float lead_scan_ms         = 0;
+  float screen_ms            = 0;
+  float survivor_scan_ms     = 0;
+  uint64_t lead_bytes        = 0;
+  uint64_t screen_bytes      = 0;
+  uint64_t survivor_bytes    = 0;
+  uint64_t n_screened_pairs  = 0;
+  uint64_t n_surviving_pairs = 0;
 };
 
 /**

@@ -234,6 +234,16 @@ typedef struct {
   float total_ms;
   uint64_t scan_bytes; /* sum over (query, probe) of round_up(list size, 32) * bytes per row */
   uint64_t scan_rows;  /* sum over (query, probe) of list size */
+  /* L2 early stop (all zero when the search did not use it): the scan stage is three launches */
+  float lead_scan_ms;      /* full scan of each query's leading probes + bound per query */
+  float screen_ms;         /* first-chunk screening of all other pairs */
+  float survivor_scan_ms;  /* full scan of the pairs the screen kept */
+  float reserved_;
+  uint64_t lead_bytes;     /* scan_bytes share of the leading pairs */
+  uint64_t screen_bytes;   /* sum over screened pairs of round_up(list size, 32) * 16 */
+  uint64_t survivor_bytes; /* scan_bytes share of the pairs the screen kept */
+  uint64_t n_screened_pairs;
+  uint64_t n_surviving_pairs;
 } cuvsAmdIvfPqSearchProfile;
 
 /** Turn event timing of the search stages on or off (off by default: timing adds event records and

@@ -303,3 +303,73 @@ def test_persistent_scan_filter_and_empty_lists(orc):
     H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 1e-5, exact=True)
     nb2, d2, want_nb2, want_d2 = _search_both(orc, index, ix, queries, 30, 2)
     H.compare_results(nb2, d2, want_nb2, want_d2, 1e-5, exact=True)
+
+
+# --- L2 early stop: leading probes in full, first-chunk screening of the rest, survivors in full ---
+
+_CLUSTERED = {}
+
+
+def _clustered_case(orc, dtype=np.float32, kind="subspace"):
+    key = (np.dtype(dtype).name, kind)
+    if key not in _CLUSTERED:
+        _CLUSTERED[key] = _make_clustered_case(orc, dtype, kind)
+    return _CLUSTERED[key]
+
+
+def _make_clustered_case(orc, dtype, kind):
+    from cuvs_amd import testing
+    print(f"clustered case dtype={np.dtype(dtype).name} kind={kind}", flush=True)
+    if dtype == np.uint8:
+        allrows = testing.sift_like_u8(30200, 128, 96, seed=77).numpy()
+    else:
+        allrows = testing.gaussian_mixture(30200, 128, 96, 0.15, seed=77).numpy().astype(dtype)
+    x, q = allrows[:30000], allrows[30000:]
+    model = H.train(x, 200, 64, 8, codebook_kind=kind, iters=6)
+    index = G.build_gpu_index(model, x, 64, 8, "sqeuclidean", kind)
+    ix, _ = G.read_back(orc, index, model, 128, 64, 8, "sqeuclidean", kind)
+    return x, q, index, ix
+
+
+@pytest.mark.parametrize("lut,internal", [(R_16F, R_32F), (R_8U, R_32F), (R_16F, R_16F), (R_8U, R_16F)])
+@pytest.mark.parametrize("dtype,kind", [(np.float32, "subspace"), (np.uint8, "subspace"),
+                                        (np.float32, "cluster")])
+def test_early_stop_matches_oracle_and_full_scan(orc, monkeypatch, lut, internal, dtype, kind):
+    from cuvs_amd.resources import Resources
+    x, q, index, ix = _clustered_case(orc, dtype, kind)
+    res = Resources()
+    res.enable_profiling(True)
+    sp = ivf_pq.SearchParams(n_probes=48, lut_dtype=lut, internal_distance_dtype=internal)
+    for k in (1, 10, 64):
+        d, nb = ivf_pq.search(sp, index, G.to_dev(q), k, resources=res)
+        res.sync()
+        prof = ivf_pq.get_search_profile(res)
+        assert prof["n_screened_pairs"] == q.shape[0] * 47
+        # on clustered data most screened pairs are dropped
+        assert 0 < prof["n_surviving_pairs"] < prof["n_screened_pairs"] // 2
+        want_nb, want_d = orc.search(ix, q, k, 48, lut_dtype=ORC_DT[lut],
+                                     internal_distance_dtype=ORC_DT[internal])
+        H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
+        monkeypatch.setenv("CUVS_AMD_NO_EARLY_STOP", "1")
+        d2, nb2 = ivf_pq.search(sp, index, G.to_dev(q), k, resources=res)
+        res.sync()
+        assert ivf_pq.get_search_profile(res)["n_screened_pairs"] == 0
+        monkeypatch.delenv("CUVS_AMD_NO_EARLY_STOP")
+        assert torch.equal(nb, nb2) and torch.equal(d, d2)
+
+
+def test_early_stop_with_filter_and_small_lists(orc):
+    """A filter can leave the leading list with fewer than k rows (no bound: nothing is dropped),
+    and the screen ignores the filter (it may keep a pair whose rows in play are all filtered)."""
+    x, q, index, ix = _clustered_case(orc)
+    n = x.shape[0]
+    rng = np.random.default_rng(5)
+    keep = rng.random(n) < 0.1
+    bits = np.packbits(keep, bitorder="little")
+    bits = np.concatenate([bits, np.zeros((-bits.size) % 4, dtype=np.uint8)]).view(np.uint32)
+    sp = ivf_pq.SearchParams(n_probes=40, lut_dtype=R_16F)
+    d, nb = ivf_pq.search(sp, index, G.to_dev(q), 20, filter_bitset=G.to_dev(bits.view(np.int32)),
+                          filter_nbits=n)
+    want_nb, want_d = orc.search(ix, q, 20, 40, lut_dtype=ORC_DT[R_16F], filter_bitset=bits,
+                                 filter_nbits=n)
+    H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
