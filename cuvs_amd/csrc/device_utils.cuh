@@ -34,6 +34,11 @@ __device__ __forceinline__ float unorder_f32(uint32_t k)
   return __uint_as_float(u);
 }
 
+__device__ __forceinline__ uint32_t next_pow2_dev(uint32_t v)
+{
+  return v <= 1u ? 1u : 1u << (32 - __builtin_clz(v - 1u));
+}
+
 __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v)
 {
   const uint32_t lane = threadIdx.x & 63u;

@@ -164,6 +164,120 @@ __global__ __launch_bounds__(kBlock) void select_probes_kernel(const float* __re
   }
 }
 
+/*
+ * Probe selection with the score row held in registers (n_probes <= 256).
+ *
+ * A block takes one query and walks its row in segments of 256 x 64 scores, thread t holding
+ * scores t, t + 256, ... of the segment as ordered 32-bit keys.  Bound: the smallest score of each
+ * thread gives 256 distinct elements, so the n_probes-th smallest of those minima has at least
+ * n_probes elements at or below it - and, for scores in no particular order, only a few more.
+ * Everything at or below the bound (and the best of the earlier segments) is collected into a small
+ * LDS list and sorted by (score, list id); one pass over HBM, no histogram atomics.  If the list
+ * overflows (adversarially ordered rows) the block falls back to the radix selection.
+ */
+constexpr uint32_t kSelPerThread = 64;
+constexpr uint32_t kSelCap       = 1024;
+
+__global__ __launch_bounds__(kBlock) void select_probes_fast_kernel(const float* __restrict__ scores,
+                                                                     uint32_t n_lists,
+                                                                     uint32_t n_probes,
+                                                                     uint32_t* __restrict__ probes)
+{
+  __shared__ unsigned long long cand[kSelCap];
+  __shared__ __align__(16) uint32_t mins[kBlock];
+  __shared__ select_smem sm;
+  __shared__ uint32_t s_bound, s_count;
+  const uint32_t tid  = threadIdx.x;
+  const uint32_t lane = tid & 63u;
+  const uint32_t q    = blockIdx.x;
+  const float* row    = scores + uint64_t(q) * n_lists;
+  uint32_t have       = 0;  // sorted best-so-far in cand[0..have)
+  bool overflow       = false;
+
+  for (uint32_t seg0 = 0; seg0 < n_lists && !overflow; seg0 += kBlock * kSelPerThread) {
+    uint32_t key[kSelPerThread];
+    float raw[kSelPerThread];
+    // all loads first (clamped addresses, no branches), so that they are in flight together
+#pragma unroll
+    for (uint32_t j = 0; j < kSelPerThread; j++) {
+      const uint32_t i = seg0 + j * kBlock + tid;
+      raw[j]           = row[i < n_lists ? i : n_lists - 1u];
+    }
+    uint32_t mine = 0xFFFFFFFFu;
+#pragma unroll
+    for (uint32_t j = 0; j < kSelPerThread; j++) {
+      const uint32_t i = seg0 + j * kBlock + tid;
+      const float v    = raw[j];
+      // past the end or NaN: never selected
+      const uint32_t kk = (i < n_lists && v == v) ? order_f32(v) : 0xFFFFFFFFu;
+      key[j]            = kk;
+      mine              = kk < mine ? kk : mine;
+    }
+    if (tid == 0) {
+      s_bound = 0xFFFFFFFEu;
+      s_count = have;
+    }
+    mins[tid] = mine;
+    __syncthreads();
+    // rank of this thread's minimum among the 256 minima (ties share a rank range)
+    uint32_t below = 0, upto = 0;
+#pragma unroll 4
+    for (uint32_t x = 0; x < kBlock; x += 4) {
+      const uint4 m = *reinterpret_cast<const uint4*>(&mins[x]);
+      below += (m.x < mine) + (m.y < mine) + (m.z < mine) + (m.w < mine);
+      upto += (m.x <= mine) + (m.y <= mine) + (m.z <= mine) + (m.w <= mine);
+    }
+    if (mine != 0xFFFFFFFFu && below < n_probes && n_probes <= upto) { s_bound = mine; }
+    __syncthreads();
+    uint32_t bound = s_bound;
+    if (have == n_probes) {
+      const uint32_t prev = uint32_t(cand[n_probes - 1] >> 32);
+      bound               = prev < bound ? prev : bound;
+    }
+    // collect
+#pragma unroll
+    for (uint32_t j = 0; j < kSelPerThread; j++) {
+      const bool pass               = key[j] <= bound && key[j] != 0xFFFFFFFFu;
+      const unsigned long long mask = __ballot(pass);
+      if (mask != 0ull) {
+        uint32_t base = 0;
+        if (lane == 0) { base = atomicAdd(&s_count, uint32_t(__popcll(mask))); }
+        base = __shfl(base, 0, 64);
+        const uint32_t pos =
+          base + __builtin_amdgcn_mbcnt_hi(uint32_t(mask >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(mask), 0u));
+        if (pass && pos < kSelCap) {
+          cand[pos] = (static_cast<unsigned long long>(key[j]) << 32) | (seg0 + j * kBlock + tid);
+        }
+      }
+    }
+    __syncthreads();
+    const uint32_t total = s_count;
+    if (total > kSelCap) {
+      overflow = true;  // uniform
+    } else {
+      const uint32_t n_sort = next_pow2_dev(total < 2u ? 2u : total);
+      for (uint32_t i = total + tid; i < n_sort; i += kBlock) { cand[i] = kInvalidKey; }
+      __syncthreads();
+      block_bitonic_sort(cand, n_sort);
+      have = total < n_probes ? total : n_probes;
+    }
+  }
+  if (overflow) {
+    __syncthreads();
+    auto key_of = [row](uint32_t i) -> unsigned long long {
+      const float v = row[i];
+      if (v != v) { return kInvalidKey; }
+      return (static_cast<unsigned long long>(order_f32(v)) << 32) | i;
+    };
+    block_select_sorted(key_of, n_lists, n_probes, cand, next_pow2_dev(n_probes), sm);
+    have = n_probes;  // unfilled slots hold kInvalidKey
+  }
+  for (uint32_t r = tid; r < n_probes; r += kBlock) {
+    const unsigned long long k2 = r < have ? cand[r] : kInvalidKey;
+    probes[uint64_t(q) * n_probes + r] = k2 == kInvalidKey ? (r % n_lists) : uint32_t(k2);
+  }
+}
+
 /* ---------------------------------------------------------------------------------------- */
 /* rotation, chunk indices, pair ordering                                                    */
 /* ---------------------------------------------------------------------------------------- */
@@ -856,6 +970,11 @@ void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_li
                           uint32_t n_probes, uint32_t* probes, hipStream_t stream)
 {
   if (n_queries == 0) { return; }
+  if (n_probes <= kBlock) {
+    select_probes_fast_kernel<<<n_queries, kBlock, 0, stream>>>(scores, n_lists, n_probes, probes);
+    CUVS_LAUNCH_CHECK();
+    return;
+  }
   const uint32_t out_cap = next_pow2(n_probes);
   const size_t smem      = size_t(out_cap) * 8;
   CUVS_EXPECTS(smem <= 96 * 1024, "n_probes (%u) is too large for the probe selection kernel", n_probes);
