@@ -112,6 +112,7 @@ struct index_impl {
   uint32_t n_chunks = 0;  // 16-byte chunks per encoded row
 
   device_buffer centers, centers_rot, rotation, rotation_t, pq_centers;
+  device_buffer centers_t;  // [dim_ext][coarse_pad(n_lists)]: centres k-major for the matrix-core kernel
   bool rotation_is_identity = false;
 
   device_buffer codes_arena, ids_arena;
@@ -146,6 +147,17 @@ void launch_coarse_scores(const float* qf, const float* centers, uint32_t n_quer
                           bool half_inputs, float* scores, hipStream_t stream);
 
 /** probes[q, 0..P) = lists with the P smallest (score, list id), ascending. */
+/** Matrix-core variant of launch_coarse_scores (coarse.hip); same values bit for bit.  Operands are
+ *  k-major with the leading dimensions padded to coarse_pad(): `qt` = [dim_ext][coarse_pad(n_queries)]
+ *  from launch_map_queries_t, `ct` = [dim_ext][coarse_pad(n_lists)] from launch_transpose_centers. */
+uint32_t coarse_pad(uint32_t n);
+void launch_transpose_centers(const float* centers, uint32_t n_lists, uint32_t dim_ext, float* ct,
+                              hipStream_t stream);
+void launch_map_queries_t(const void* queries, elem_type type, uint32_t n_queries, uint32_t dim,
+                          uint32_t dim_ext, bool ip_like, float* qt, hipStream_t stream);
+void launch_coarse_scores_mfma(const float* qt, const float* ct, uint32_t n_queries, uint32_t n_lists,
+                               uint32_t dim_ext, bool ip_like, bool half_inputs, float* scores,
+                               hipStream_t stream);
 void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_lists,
                           uint32_t n_probes, uint32_t* probes, hipStream_t stream);
 

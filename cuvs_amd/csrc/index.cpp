@@ -157,6 +157,9 @@ index<int64_t> build(cuvs::resources const& res,
   copy_in(ix.pq_centers, pq_centers, n_books * ix.pq_len * ix.book_size);
   copy_in(ix.centers, centers, size_t(ix.n_lists) * ix.dim_ext);
   copy_in(ix.centers_rot, centers_rot, size_t(ix.n_lists) * ix.rot_dim);
+  ix.centers_t.allocate(size_t(ix.dim_ext) * detail::coarse_pad(ix.n_lists) * sizeof(float));
+  detail::launch_transpose_centers(ix.centers.as<float>(), ix.n_lists, ix.dim_ext,
+                                   ix.centers_t.as<float>(), stream);
   copy_in(ix.rotation, rotation_matrix, size_t(ix.rot_dim) * ix.dim);
 
   // transposed copy [dim, rot_dim] for coalesced reads, and the identity check

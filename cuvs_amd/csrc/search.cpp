@@ -89,10 +89,11 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
   }
   p.fused = k <= kMaxFusedK;
   const size_t P = p.n_probes;
-  p.per_query_bytes = size_t(ix.dim) * 4 + size_t(ix.n_lists) * 4 + size_t(ix.rot_dim) * 4 +
+  p.per_query_bytes = size_t(ix.dim) * 4 + size_t(ix.dim_ext) * 4 + size_t(ix.n_lists) * 4 +
+                      size_t(ix.rot_dim) * 4 +
                       P * 4 * 3 + P * (2 * sizeof(detail::pair_desc) + 1) + 16 +
                       (p.fused ? P * k * 8 * 4 : size_t(p.max_samples) * 4);
-  p.fixed_bytes = a256(size_t(ix.n_lists) * 16 + 16) + 16 * 256;
+  p.fixed_bytes = a256(size_t(ix.n_lists) * 16 + 16) + a256(size_t(ix.dim_ext) * 128 * 4) + 16 * 256;
   const size_t budget = workspace_budget(res);
   size_t b = budget > p.fixed_bytes ? (budget - p.fixed_bytes) / (p.per_query_bytes + 64) : 1;
   b        = std::max<size_t>(b, 1);
@@ -192,6 +193,7 @@ float scaling_factor(elem_type t)
 size_t elem_size(elem_type t) { return t == elem_type::f32 ? 4 : (t == elem_type::f16 ? 2 : 1); }
 
 struct coarse_buffers {
+  float* qt;  // [dim_ext][coarse_pad(batch)]
   float* qf;
   float* scores;
   uint32_t* probes;
@@ -206,8 +208,9 @@ void run_coarse(const cuvs::resources& res, const search_params& params, const i
   const bool ip     = ix.metric == detail::DistanceType::InnerProduct ||
                   ix.metric == detail::DistanceType::CosineExpanded;
   detail::launch_map_queries(queries, type, uint64_t(nq) * ix.dim, b.qf, s);
-  detail::launch_coarse_scores(b.qf, ix.centers.as<float>(), nq, ix.n_lists, ix.dim, ix.dim_ext,
-                               ip, params.coarse_search_dtype == CUDA_R_16F, b.scores, s);
+  detail::launch_map_queries_t(queries, type, nq, ix.dim, ix.dim_ext, ip, b.qt, s);
+  detail::launch_coarse_scores_mfma(b.qt, ix.centers_t.as<float>(), nq, ix.n_lists, ix.dim_ext, ip,
+                                    params.coarse_search_dtype == CUDA_R_16F, b.scores, s);
   detail::launch_select_probes(b.scores, nq, ix.n_lists, n_probes, b.probes, s);
 }
 
@@ -230,13 +233,16 @@ void select_clusters(cuvs::resources const& res_c,
   CUVS_EXPECTS(device_accessible(queries) && device_accessible(clusters_to_probe),
                "all pointers must be accessible from the device.");
   const uint32_t P       = std::min<uint32_t>(params.n_probes, ix.n_lists);
-  const size_t per_query = size_t(ix.dim) * 4 + size_t(ix.n_lists) * 4 + 64;
+  const size_t per_query = size_t(ix.dim) * 4 + size_t(ix.dim_ext) * 4 + size_t(ix.n_lists) * 4 + 64;
   size_t batch           = std::max<size_t>(1, workspace_budget(res) / per_query);
   batch                  = std::min<size_t>(batch, size_t(n_queries));
   batch                  = std::min<size_t>(batch, 65535u * 64u);
   res.reset_workspace();
-  res.reserve_workspace(a256(batch * ix.dim * 4) + a256(batch * size_t(ix.n_lists) * 4) + 1024);
+  const size_t qt_bytes = size_t(ix.dim_ext) * detail::coarse_pad(uint32_t(batch)) * 4;
+  res.reserve_workspace(a256(batch * ix.dim * 4) + a256(qt_bytes) +
+                        a256(batch * size_t(ix.n_lists) * 4) + 1024);
   coarse_buffers b;
+  b.qt     = static_cast<float*>(res.workspace_alloc(qt_bytes));
   b.qf     = static_cast<float*>(res.workspace_alloc(batch * ix.dim * 4));
   b.scores = static_cast<float*>(res.workspace_alloc(batch * size_t(ix.n_lists) * 4));
   for (int64_t q0 = 0; q0 < n_queries; q0 += int64_t(batch)) {
@@ -320,6 +326,8 @@ void search(cuvs::resources const& res_c,
   /* workspace carve-up for one batch */
   res.reset_workspace();
   res.reserve_workspace(pl.fixed_bytes + size_t(Qb) * (pl.per_query_bytes + 64) + 16 * 256);
+  auto* qt        = static_cast<float*>(
+    res.workspace_alloc(size_t(ix.dim_ext) * detail::coarse_pad(Qb) * 4));
   auto* qf        = static_cast<float*>(res.workspace_alloc(size_t(Qb) * ix.dim * 4));
   auto* scores    = static_cast<float*>(res.workspace_alloc(size_t(Qb) * ix.n_lists * 4));
   auto* rot_q     = static_cast<float*>(res.workspace_alloc(size_t(Qb) * ix.rot_dim * 4));
@@ -383,7 +391,7 @@ void search(cuvs::resources const& res_c,
     const void* qptr  = static_cast<const char*>(queries) + size_t(q0) * ix.dim * elem_size(type);
 
     mark(0);
-    run_coarse(res, params, ix, qptr, type, nq, P, coarse_buffers{qf, scores, probes});
+    run_coarse(res, params, ix, qptr, type, nq, P, coarse_buffers{qt, qf, scores, probes});
     mark(1);
     detail::launch_rotate(qf, ix.rotation_t.as<float>(), nq, ix.dim, ix.rot_dim,
                           ix.rotation_is_identity, cosine, rot_q, s);
