@@ -2,21 +2,26 @@
  * Screening pass of the L2 early stop (8-bit codes).
  *
  * A row's score is a sum of non-negative table entries taken in subspace order, so the partial sum
- * over the first 16 subspaces (the first 16-byte chunk of the row) is a lower bound of its final
- * score, and it is exactly the intermediate value the full scan kernels reach after that chunk.  A
- * pair none of whose rows is still at or below the query's current k-th best score after that chunk
- * cannot contribute a result (compute_score's early stop in the reference,
+ * over the first S subspaces is a lower bound of its final score, and it is exactly the
+ * intermediate value the full scan kernels reach after S additions.  A pair none of whose rows is
+ * still at or below the query's current k-th best score after those S terms cannot contribute a
+ * result (compute_score's early stop in the reference,
  * cpp/src/neighbors/ivf_pq/detail/jit_lto_kernels/compute_score_impl.cuh:70-74, applied to the whole
- * list at once).  For clustered data this removes most (query, probe) pairs at a quarter of the
- * table-building and gather work or less, and only the survivors go through the full scan.
+ * list at once).  For clustered data this removes most (query, probe) pairs for an eighth of the
+ * table-building and gather work, and only the survivors go through the full scan.  S = 8 by
+ * default (the first half of each row's first 16-byte chunk): on the benchmark data as many pairs
+ * are dropped as with 16, and with 4 three times as many survive.
  *
  * Organisation: persistent 256-thread blocks, several per CU so that the table-building phase of
  * one block overlaps the gather phase of another.  A block takes G = 4 pairs per iteration; thread
- * c keeps entry c of the first 16 subspaces' codebooks in registers and builds entry c of the four
- * 16 x 256 tables; then wave g scans the first chunk of every row of pair g and stops at the first
+ * c keeps entry c of the first S subspaces' codebooks in registers and builds entry c of the four
+ * S x 256 tables; then wave g sums the first S codes of every row of pair g and stops at the first
  * tile with a row still in play.
  */
 #include "device_utils.cuh"
+
+#include <algorithm>
+#include <cstdlib>
 
 namespace cuvs::neighbors::ivf_pq::detail {
 
@@ -28,7 +33,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t kScreenThreads = 256;
 constexpr uint32_t kScreenG       = 4;   // pairs per block iteration = waves per block
-constexpr uint32_t kScreenSub     = 16;  // subspaces in the first chunk of 8-bit codes
 constexpr uint32_t kScreenLdsBase = 16;  // no LDS object at address 0: a null constant pointer folds badly
 
 __device__ __forceinline__ void lds_barrier_s()
@@ -43,7 +47,7 @@ __device__ __forceinline__ float opaque_one_s()
   return one;
 }
 
-template <int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER>
+template <int SUBS, int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER>
 __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   scan_args a, const pair_desc* __restrict__ desc, uint32_t n_pairs, uint32_t group_bytes,
   pair_desc* __restrict__ survivors, uint32_t* __restrict__ n_survivors, uint8_t* __restrict__ alive)
@@ -52,7 +56,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   using lut_t  = typename traits::storage;
   using acc_t  = typename std::conditional<OUT_HALF, _Float16, float>::type;
   constexpr uint32_t G           = kScreenG;
-  constexpr uint32_t SUB         = kScreenSub;
+  constexpr uint32_t SUB         = SUBS;
   constexpr uint32_t NDIFF       = SUB * PQ_LEN;  // leading rotated dimensions the first chunk covers
   constexpr uint32_t lut_entries = SUB * 256u;
   constexpr uint32_t off_diff    = kScreenLdsBase + G * lut_entries * uint32_t(sizeof(lut_t));
@@ -164,7 +168,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
         const uint32_t w[4] = {cur.x, cur.y, cur.z, cur.w};
         acc_t acc           = acc_t(0);
 #pragma unroll
-        for (int kk = 0; kk < 16; kk++) {
+        for (int kk = 0; kk < SUBS; kk++) {
           const uint32_t c = (w[kk >> 2] >> ((kk & 3) * 8)) & 0xffu;
           const lut_t v    = my_lut[kk * 256 + c];
           if (OUT_HALF) {
@@ -199,15 +203,15 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   }
 }
 
-template <int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER>
-void launch_screen_instance(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
+template <int SUBS, int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER>
+void launch_screen_sub(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
                             pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
                             hipStream_t stream)
 {
   using lut_t       = typename lut_traits<LUT>::storage;
-  auto kernel       = scan_screen_kernel<PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>;
-  const size_t smem = kScreenLdsBase + size_t(kScreenG) * kScreenSub * 256 * sizeof(lut_t) +
-                      size_t(kScreenG) * kScreenSub * PQ_LEN * 4;
+  auto kernel       = scan_screen_kernel<SUBS, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>;
+  const size_t smem = kScreenLdsBase + size_t(kScreenG) * SUBS * 256 * sizeof(lut_t) +
+                      size_t(kScreenG) * SUBS * PQ_LEN * 4;
   static int n_cu = 0;
   if (n_cu == 0) {
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -217,13 +221,34 @@ void launch_screen_instance(const scan_args& a, const pair_desc* desc, uint32_t 
     CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
   }
   const uint32_t n_iters = (n_pairs + kScreenG - 1) / kScreenG;
-  uint32_t grid          = uint32_t(n_cu) * 4u;
+  const uint32_t per_cu  = std::min<uint32_t>(8u, uint32_t((150u * 1024u) / smem));
+  uint32_t grid          = uint32_t(n_cu) * std::max(per_cu, 1u);
   if (grid > n_iters) { grid = n_iters; }
   const uint32_t n_chunks    = (a.pq_dim + 15u) / 16u;
   const uint32_t group_bytes = n_chunks * 512u;
   kernel<<<grid, kScreenThreads, smem, stream>>>(a, desc, n_pairs, group_bytes, survivors, n_survivors,
                                                  alive);
   CUVS_HIP_TRY(hipGetLastError());
+}
+
+template <int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER>
+void launch_screen_instance(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
+                            pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
+                            hipStream_t stream)
+{
+  // how many leading subspaces the screen sums (of the 16 in the first chunk)
+  static const int subs = [] {
+    const char* e = std::getenv("CUVS_AMD_SCREEN_SUBSPACES");
+    const int v   = e != nullptr ? std::atoi(e) : 8;
+    return (v == 4 || v == 8 || v == 16) ? v : 8;
+  }();
+  if (subs == 4) {
+    launch_screen_sub<4, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+  } else if (subs == 8) {
+    launch_screen_sub<8, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+  } else {
+    launch_screen_sub<16, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+  }
 }
 
 template <int PQ_LEN, bool PER_CLUSTER>
