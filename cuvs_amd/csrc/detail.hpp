@@ -158,6 +158,9 @@ void launch_map_queries_t(const void* queries, elem_type type, uint32_t n_querie
 void launch_coarse_scores_mfma(const float* qt, const float* ct, uint32_t n_queries, uint32_t n_lists,
                                uint32_t dim_ext, bool ip_like, bool half_inputs, float* scores,
                                hipStream_t stream);
+/** The probe selection reads whole segments of 256 x 64 scores: the score buffer must have this
+ *  many readable bytes after its last row. */
+constexpr size_t kSelectSlackBytes = 256 * 64 * 4;
 void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_lists,
                           uint32_t n_probes, uint32_t* probes, hipStream_t stream);
 

@@ -126,7 +126,7 @@ void extend(cuvs::resources const& res,
     CUVS_HIP_TRY(hipMemcpyAsync(labels.ptr, labels_in, n_rows * sizeof(uint32_t),
                                 hipMemcpyDefault, s));
   } else {
-    scores.allocate(chunk * ix.n_lists * sizeof(float));
+    scores.allocate(chunk * ix.n_lists * sizeof(float) + detail::kSelectSlackBytes);
     for (uint64_t r0 = 0; r0 < n_rows; r0 += chunk) {
       const uint64_t n = std::min(chunk, n_rows - r0);
       float* xf        = stager.load(r0, n, cosine, s);
@@ -259,7 +259,7 @@ void transform(cuvs::resources const& res,
   const uint64_t chunk     = chunk_rows_for(ix, n_rows);
   const uint32_t row_bytes = (ix.pq_dim * ix.pq_bits + 7) / 8;
   row_stager stager(vectors, type, ix.dim, chunk);
-  device_buffer scores(chunk * ix.n_lists * sizeof(float));
+  device_buffer scores(chunk * ix.n_lists * sizeof(float) + detail::kSelectSlackBytes);
   device_buffer scratch(chunk * ix.rot_dim * sizeof(float));
   for (uint64_t r0 = 0; r0 < n_rows; r0 += chunk) {
     const uint64_t n = std::min(chunk, n_rows - r0);

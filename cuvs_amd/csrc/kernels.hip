@@ -178,17 +178,37 @@ __global__ __launch_bounds__(kBlock) void select_probes_kernel(const float* __re
 constexpr uint32_t kSelPerThread = 64;
 constexpr uint32_t kSelCap       = 1024;
 
-__global__ __launch_bounds__(kBlock) void select_probes_fast_kernel(const float* __restrict__ scores,
+/** Ascending bitonic sort of one 32-bit key per lane across the wave. */
+__device__ __forceinline__ uint32_t wave_sort_u32(uint32_t v, uint32_t lane)
+{
+#pragma unroll
+  for (uint32_t size = 2; size <= 64; size <<= 1) {
+#pragma unroll
+    for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+      const uint32_t other = __shfl_xor(v, int(stride), 64);
+      const bool ascending = (lane & size) == 0 || size == 64;
+      const bool low_half  = (lane & stride) == 0;
+      const uint32_t lo    = v < other ? v : other;
+      const uint32_t hi    = v < other ? other : v;
+      v                    = (low_half == ascending) ? lo : hi;
+    }
+  }
+  return v;
+}
+
+__global__ __launch_bounds__(kBlock, 3) void select_probes_fast_kernel(const float* __restrict__ scores,
                                                                      uint32_t n_lists,
                                                                      uint32_t n_probes,
                                                                      uint32_t* __restrict__ probes)
 {
   __shared__ unsigned long long cand[kSelCap];
-  __shared__ __align__(16) uint32_t mins[kBlock];
+  __shared__ unsigned long long ranked[kBlock];
+  __shared__ uint32_t mins[kBlock];  // the four waves' minima, each wave's 64 sorted ascending
   __shared__ select_smem sm;
   __shared__ uint32_t s_bound, s_count;
   const uint32_t tid  = threadIdx.x;
   const uint32_t lane = tid & 63u;
+  const uint32_t wid  = tid >> 6;
   const uint32_t q    = blockIdx.x;
   const float* row    = scores + uint64_t(q) * n_lists;
   uint32_t have       = 0;  // sorted best-so-far in cand[0..have)
@@ -196,57 +216,63 @@ __global__ __launch_bounds__(kBlock) void select_probes_fast_kernel(const float*
 
   for (uint32_t seg0 = 0; seg0 < n_lists && !overflow; seg0 += kBlock * kSelPerThread) {
     uint32_t key[kSelPerThread];
-    float raw[kSelPerThread];
-    // all loads first (clamped addresses, no branches), so that they are in flight together
+    // all loads first, so that they are in flight together
+    // uniform base + one per-thread offset, no clamping: the score buffer carries
+    // kSelectSlackBytes of readable slack after its last row
+    const float* seg = row + seg0;
 #pragma unroll
-    for (uint32_t j = 0; j < kSelPerThread; j++) {
-      const uint32_t i = seg0 + j * kBlock + tid;
-      raw[j]           = row[i < n_lists ? i : n_lists - 1u];
-    }
+    for (uint32_t j = 0; j < kSelPerThread; j++) { key[j] = __float_as_uint(seg[j * kBlock + tid]); }
     uint32_t mine = 0xFFFFFFFFu;
 #pragma unroll
     for (uint32_t j = 0; j < kSelPerThread; j++) {
       const uint32_t i = seg0 + j * kBlock + tid;
-      const float v    = raw[j];
+      const float v    = __uint_as_float(key[j]);
       // past the end or NaN: never selected
       const uint32_t kk = (i < n_lists && v == v) ? order_f32(v) : 0xFFFFFFFFu;
       key[j]            = kk;
       mine              = kk < mine ? kk : mine;
     }
     if (tid == 0) {
-      s_bound = 0xFFFFFFFEu;
+      s_bound = 0xFFFFFFFFu;
       s_count = have;
     }
-    mins[tid] = mine;
+    // n_probes-th smallest of the 256 minima: sort per wave, then rank across the waves
+    const uint32_t sorted_min = wave_sort_u32(mine, lane);
+    mins[tid]                 = sorted_min;
     __syncthreads();
-    // rank of this thread's minimum among the 256 minima (ties share a rank range)
-    uint32_t below = 0, upto = 0;
-#pragma unroll 4
-    for (uint32_t x = 0; x < kBlock; x += 4) {
-      const uint4 m = *reinterpret_cast<const uint4*>(&mins[x]);
-      below += (m.x < mine) + (m.y < mine) + (m.z < mine) + (m.w < mine);
-      upto += (m.x <= mine) + (m.y <= mine) + (m.z <= mine) + (m.w <= mine);
+    uint32_t rank = lane;
+#pragma unroll
+    for (uint32_t w = 0; w < kBlock / 64; w++) {
+      if (w == wid) { continue; }
+      // elements of wave w's list ordered before (sorted_min, wid): `<=` for earlier waves
+      const uint32_t* list = mins + w * 64u;
+      uint32_t lo = 0, hi = 64;
+#pragma unroll
+      for (int step = 0; step < 6; step++) {
+        const uint32_t mid = (lo + hi) >> 1;
+        const uint32_t m   = list[mid];
+        const bool before  = w < wid ? m <= sorted_min : m < sorted_min;
+        lo                 = before ? mid + 1u : lo;
+        hi                 = before ? hi : mid;
+      }
+      rank += lo;
     }
-    if (mine != 0xFFFFFFFFu && below < n_probes && n_probes <= upto) { s_bound = mine; }
+    if (rank == n_probes - 1u) { s_bound = sorted_min; }
     __syncthreads();
     uint32_t bound = s_bound;
     if (have == n_probes) {
       const uint32_t prev = uint32_t(cand[n_probes - 1] >> 32);
       bound               = prev < bound ? prev : bound;
     }
-    // collect
+    // collect: only threads whose minimum is within the bound hold anything
+    if (mine <= bound && mine != 0xFFFFFFFFu) {
 #pragma unroll
-    for (uint32_t j = 0; j < kSelPerThread; j++) {
-      const bool pass               = key[j] <= bound && key[j] != 0xFFFFFFFFu;
-      const unsigned long long mask = __ballot(pass);
-      if (mask != 0ull) {
-        uint32_t base = 0;
-        if (lane == 0) { base = atomicAdd(&s_count, uint32_t(__popcll(mask))); }
-        base = __shfl(base, 0, 64);
-        const uint32_t pos =
-          base + __builtin_amdgcn_mbcnt_hi(uint32_t(mask >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(mask), 0u));
-        if (pass && pos < kSelCap) {
-          cand[pos] = (static_cast<unsigned long long>(key[j]) << 32) | (seg0 + j * kBlock + tid);
+      for (uint32_t j = 0; j < kSelPerThread; j++) {
+        if (key[j] <= bound && key[j] != 0xFFFFFFFFu) {
+          const uint32_t pos = atomicAdd(&s_count, 1u);
+          if (pos < kSelCap) {
+            cand[pos] = (static_cast<unsigned long long>(key[j]) << 32) | (seg0 + j * kBlock + tid);
+          }
         }
       }
     }
@@ -254,8 +280,22 @@ __global__ __launch_bounds__(kBlock) void select_probes_fast_kernel(const float*
     const uint32_t total = s_count;
     if (total > kSelCap) {
       overflow = true;  // uniform
+    } else if (total <= kBlock) {
+      // few candidates: place each by counting the smaller ones
+      unsigned long long mykey = kInvalidKey;
+      uint32_t pos             = 0;
+      if (tid < total) {
+        mykey = cand[tid];
+        for (uint32_t x = 0; x < total; x++) { pos += cand[x] < mykey ? 1u : 0u; }
+      }
+      __syncthreads();
+      if (tid < total) { ranked[pos] = mykey; }
+      __syncthreads();
+      have = total < n_probes ? total : n_probes;
+      if (tid < have) { cand[tid] = ranked[tid]; }
+      __syncthreads();
     } else {
-      const uint32_t n_sort = next_pow2_dev(total < 2u ? 2u : total);
+      const uint32_t n_sort = next_pow2_dev(total);
       for (uint32_t i = total + tid; i < n_sort; i += kBlock) { cand[i] = kInvalidKey; }
       __syncthreads();
       block_bitonic_sort(cand, n_sort);

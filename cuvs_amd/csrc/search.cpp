@@ -93,7 +93,7 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
                       size_t(ix.rot_dim) * 4 +
                       P * 4 * 3 + P * (2 * sizeof(detail::pair_desc) + 1) + 16 +
                       (p.fused ? P * k * 8 * 4 : size_t(p.max_samples) * 4);
-  p.fixed_bytes = a256(size_t(ix.n_lists) * 16 + 16) + a256(size_t(ix.dim_ext) * 128 * 4) + 16 * 256;
+  p.fixed_bytes = a256(size_t(ix.n_lists) * 16 + 16) + a256(size_t(ix.dim_ext) * 128 * 4) + a256(detail::kSelectSlackBytes) + 16 * 256;
   const size_t budget = workspace_budget(res);
   size_t b = budget > p.fixed_bytes ? (budget - p.fixed_bytes) / (p.per_query_bytes + 64) : 1;
   b        = std::max<size_t>(b, 1);
@@ -240,11 +240,12 @@ void select_clusters(cuvs::resources const& res_c,
   res.reset_workspace();
   const size_t qt_bytes = size_t(ix.dim_ext) * detail::coarse_pad(uint32_t(batch)) * 4;
   res.reserve_workspace(a256(batch * ix.dim * 4) + a256(qt_bytes) +
-                        a256(batch * size_t(ix.n_lists) * 4) + 1024);
+                        a256(batch * size_t(ix.n_lists) * 4 + detail::kSelectSlackBytes) + 1024);
   coarse_buffers b;
   b.qt     = static_cast<float*>(res.workspace_alloc(qt_bytes));
   b.qf     = static_cast<float*>(res.workspace_alloc(batch * ix.dim * 4));
-  b.scores = static_cast<float*>(res.workspace_alloc(batch * size_t(ix.n_lists) * 4));
+  b.scores = static_cast<float*>(
+    res.workspace_alloc(batch * size_t(ix.n_lists) * 4 + detail::kSelectSlackBytes));
   for (int64_t q0 = 0; q0 < n_queries; q0 += int64_t(batch)) {
     const uint32_t nq = uint32_t(std::min<int64_t>(int64_t(batch), n_queries - q0));
     b.probes          = clusters_to_probe + q0 * P;
@@ -329,7 +330,8 @@ void search(cuvs::resources const& res_c,
   auto* qt        = static_cast<float*>(
     res.workspace_alloc(size_t(ix.dim_ext) * detail::coarse_pad(Qb) * 4));
   auto* qf        = static_cast<float*>(res.workspace_alloc(size_t(Qb) * ix.dim * 4));
-  auto* scores    = static_cast<float*>(res.workspace_alloc(size_t(Qb) * ix.n_lists * 4));
+  auto* scores    = static_cast<float*>(
+    res.workspace_alloc(size_t(Qb) * ix.n_lists * 4 + detail::kSelectSlackBytes));
   auto* rot_q     = static_cast<float*>(res.workspace_alloc(size_t(Qb) * ix.rot_dim * 4));
   auto* probes    = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * P * 4));
   auto* chunk     = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * P * 4));
