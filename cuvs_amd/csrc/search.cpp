@@ -141,7 +141,12 @@ bool early_stop_disabled()
 
 /** Probes per query whose lists are scanned in full before the others are screened against the
  *  bound they give. */
-constexpr uint32_t kLeadProbes = 1;
+uint32_t lead_probes()
+{
+  const char* e = std::getenv("CUVS_AMD_LEAD_PROBES");  // for A/B runs
+  const int v   = e != nullptr ? std::atoi(e) : 1;
+  return v >= 1 && v <= 16 ? uint32_t(v) : 1u;
+}
 
 /** CUVS_AMD_GENERIC_SCAN=1 routes every search through the generic scan kernel (for A/B runs). */
 bool force_generic_scan()
@@ -350,6 +355,7 @@ void search(cuvs::resources const& res_c,
     desc = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));
   }
   // L2 early stop: lists of the leading probes in full, the others screened on their first chunk
+  const uint32_t kLeadProbes = lead_probes();
   const bool early_stop = quad_kpp != 0 && P > kLeadProbes && detail::scan_screen_supported(sa) &&
                           !early_stop_disabled();
   const uint32_t lead          = early_stop ? kLeadProbes : P;
