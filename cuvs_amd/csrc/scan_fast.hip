@@ -139,8 +139,9 @@ __global__ __launch_bounds__(kBlock, 2) void scan_fast_kernel(scan_args a)
   const float one = opaque_one();
 
   const uint32_t tid     = threadIdx.x;
-  const uint32_t n_pairs = a.n_queries * a.n_probes;
+  const uint32_t n_pairs = a.n_pairs_dev != nullptr ? *a.n_pairs_dev : a.n_pairs;
   const uint32_t stride  = gridDim.x;
+  if (blockIdx.x >= n_pairs) { return; }  // whole block, before any barrier
 
   // codebook entry `tid` of every subspace, resident for the whole kernel
   float book[PER_CLUSTER ? 1 : M][PQ_LEN];
@@ -275,9 +276,13 @@ __global__ __launch_bounds__(kBlock, 2) void scan_fast_kernel(scan_args a)
           valid = id >= 0 && id < a.filter_nbits && ((a.filter_bits[id >> 5] >> (id & 31)) & 1u) != 0;
         }
         acc_t acc = acc_t(0);
-        if (__ballot(valid) != 0ull) {  // whole waves past the end of the list skip the tile
+        // whole waves past the end of the list skip the tile; L2 sums only grow, so a wave whose
+        // rows are all above the bound after a chunk skips the rest (compute_score's early stop)
+        const uint32_t stop_bits = thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u;
+        bool live                = __ballot(valid) != 0ull;
 #pragma unroll
-          for (int m = 0; m < NCH; m++) {
+        for (int m = 0; m < NCH; m++) {
+          if (live) {
             const uint32_t w[4] = {cur[m].x, cur[m].y, cur[m].z, cur[m].w};
 #pragma unroll
             for (int kk = 0; kk < 16; kk++) {
@@ -290,6 +295,9 @@ __global__ __launch_bounds__(kBlock, 2) void scan_fast_kernel(scan_args a)
               } else {
                 acc = acc_t(acc + traits::to_float(v));
               }
+            }
+            if (!IP && m + 1 < NCH) {
+              live = __ballot(valid && !(__float_as_uint(float(acc)) > stop_bits)) != 0ull;
             }
           }
         }
@@ -368,9 +376,11 @@ void launch_instance(const scan_args& a, hipStream_t stream)
     CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
     blocks_per_cu = occ > 0 ? occ : 1;
   }
-  const uint32_t n_pairs = a.n_queries * a.n_probes;
-  uint32_t grid          = uint32_t(blocks_per_cu) * uint32_t(n_cu);
-  if (grid > n_pairs) { grid = n_pairs; }
+  uint32_t grid = uint32_t(blocks_per_cu) * uint32_t(n_cu);
+  if (a.n_pairs_dev == nullptr) {
+    if (grid > a.n_pairs) { grid = a.n_pairs; }
+    if (grid == 0) { return; }
+  }
   kernel<<<grid, kBlock, smem, stream>>>(a);
   CUVS_HIP_TRY(hipGetLastError());
 }

@@ -256,7 +256,9 @@ void launch_screen_types(const scan_args& a, const pair_desc* desc, uint32_t n_p
                          pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive, hipStream_t s)
 {
   if (!a.out_half) {
-    if (a.lut_dtype == CUDA_R_16F) {
+    if (a.lut_dtype == CUDA_R_32F) {
+      launch_screen_instance<PQ_LEN, LUT_F32, false, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, s);
+    } else if (a.lut_dtype == CUDA_R_16F) {
       launch_screen_instance<PQ_LEN, LUT_F16, false, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, s);
     } else {
       launch_screen_instance<PQ_LEN, LUT_FP8U, false, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, s);
@@ -276,7 +278,7 @@ bool scan_screen_supported(const scan_args& a)
 {
   const bool l2 = a.metric == int(DistanceType::L2Expanded) || a.metric == int(DistanceType::L2SqrtExpanded);
   if (!l2 || !a.fused || a.pq_bits != 8 || a.pq_dim < 32) { return false; }
-  if (a.lut_dtype != CUDA_R_16F && a.lut_dtype != CUDA_R_8U) { return false; }
+  if (a.lut_dtype == CUDA_R_32F && a.out_half) { return false; }
   return a.pq_len == 2 || a.pq_len == 4;
 }
 

@@ -356,7 +356,7 @@ void search(cuvs::resources const& res_c,
   }
   // L2 early stop: lists of the leading probes in full, the others screened on their first chunk
   const uint32_t kLeadProbes = lead_probes();
-  const bool early_stop = quad_kpp != 0 && P > kLeadProbes && detail::scan_screen_supported(sa) &&
+  const bool early_stop = fast_scan && P > kLeadProbes && detail::scan_screen_supported(sa) &&
                           !early_stop_disabled();
   const uint32_t lead          = early_stop ? kLeadProbes : P;
   detail::pair_desc* survivors = nullptr;
@@ -424,8 +424,11 @@ void search(cuvs::resources const& res_c,
     sa.timing      = scan_timing_buffer();
     if (early_stop) {
       // 1. the leading probes' lists in full: candidates and a first bound per query
+      auto full_scan = [&] {
+        return quad_kpp != 0 ? detail::launch_scan_quad(sa, s) : detail::launch_scan_fast(sa, s);
+      };
       sa.n_pairs = nq * lead;
-      CUVS_EXPECTS(detail::launch_scan_quad(sa, s), "scan kernel launch failed");
+      CUVS_EXPECTS(full_scan(), "scan kernel launch failed");
       detail::launch_kth_bound(keys, nq, uint64_t(P) * kpp, lead * kpp, k, kth, s);
       mark(5);
       // 2. every other pair on its first chunk only
@@ -437,7 +440,7 @@ void search(cuvs::resources const& res_c,
       sa.desc        = survivors;
       sa.n_pairs     = 0;
       sa.n_pairs_dev = n_survivors;
-      CUVS_EXPECTS(detail::launch_scan_quad(sa, s), "scan kernel launch failed");
+      CUVS_EXPECTS(full_scan(), "scan kernel launch failed");
     } else {
       const bool launched = fast_scan && (quad_kpp != 0 ? detail::launch_scan_quad(sa, s)
                                                         : detail::launch_scan_fast(sa, s));

@@ -331,7 +331,8 @@ def _make_clustered_case(orc, dtype, kind):
     return x, q, index, ix
 
 
-@pytest.mark.parametrize("lut,internal", [(R_16F, R_32F), (R_8U, R_32F), (R_16F, R_16F), (R_8U, R_16F)])
+@pytest.mark.parametrize("lut,internal", [(R_32F, R_32F), (R_16F, R_32F), (R_8U, R_32F), (R_16F, R_16F),
+                                          (R_8U, R_16F)])
 @pytest.mark.parametrize("dtype,kind", [(np.float32, "subspace"), (np.uint8, "subspace"),
                                         (np.float32, "cluster")])
 def test_early_stop_matches_oracle_and_full_scan(orc, monkeypatch, lut, internal, dtype, kind):
@@ -340,13 +341,13 @@ def test_early_stop_matches_oracle_and_full_scan(orc, monkeypatch, lut, internal
     res = Resources()
     res.enable_profiling(True)
     sp = ivf_pq.SearchParams(n_probes=48, lut_dtype=lut, internal_distance_dtype=internal)
-    for k in (1, 10, 64):
+    for k in (1, 10, 64, 100, 256):  # up to 64: CU-wide kernel; above: block-per-pair kernel
         d, nb = ivf_pq.search(sp, index, G.to_dev(q), k, resources=res)
         res.sync()
         prof = ivf_pq.get_search_profile(res)
         assert prof["n_screened_pairs"] == q.shape[0] * 47
-        # on clustered data most screened pairs are dropped
-        assert 0 < prof["n_surviving_pairs"] < prof["n_screened_pairs"] // 2
+        # on clustered data most screened pairs are dropped (fewer for a large k: a looser bound)
+        assert 0 < prof["n_surviving_pairs"] < prof["n_screened_pairs"] // (2 if k <= 100 else 1)
         want_nb, want_d = orc.search(ix, q, k, 48, lut_dtype=ORC_DT[lut],
                                      internal_distance_dtype=ORC_DT[internal])
         H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
