@@ -174,7 +174,7 @@ void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries,
 void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
                           uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
                           uint32_t* n_samples, unsigned long long* stats, uint32_t lead_probes,
-                          hipStream_t stream);
+                          uint32_t* pair_counts, uint32_t n_lists, hipStream_t stream);
 
 /** Everything the scan needs to know about one (query, probe) pair, gathered once so that the
  *  scan kernel reads one 32-byte record instead of chasing four dependent pointers. */
@@ -194,11 +194,13 @@ static_assert(sizeof(pair_desc) == 32, "pair_desc must stay 32 bytes");
  *  of each query's first `lead_probes` probes come first (n_queries * lead_probes records, grouped
  *  by list) and the others after them (grouped by list again); `alive`, when non-null, gets one
  *  byte per pair slot: 1 for the leading pairs, 0 for the others.  `counters` is scratch of
- *  4 * n_lists + 4 words. */
+ *  4 * n_lists + 4 words; with `counted` its first half already holds the histogram of the pairs
+ *  (launch_chunk_indices with `pair_counts` makes it on the way). */
 void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
                         const uint8_t* const* data_ptrs, uint32_t n_pairs, uint32_t n_probes,
                         uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
-                        pair_desc* desc, uint32_t lead_probes, uint8_t* alive, hipStream_t stream);
+                        pair_desc* desc, uint32_t lead_probes, uint8_t* alive, bool counted,
+                        hipStream_t stream);
 
 struct scan_args {
   uint32_t n_queries, n_probes, k, max_samples;

@@ -158,7 +158,8 @@ void extend(cuvs::resources const& res,
     new_offsets[l + 1] = new_offsets[l] + round_up_u64(ns, kIndexGroupSize);
   }
   const uint64_t total_rows = new_offsets[ix.n_lists];
-  device_buffer new_codes((total_rows / kIndexGroupSize) * ix.group_bytes());
+  // two groups of slack: the scan kernels read whole 64-row tiles past a list's last group
+  device_buffer new_codes((total_rows / kIndexGroupSize + 2) * ix.group_bytes());
   device_buffer new_ids(total_rows * sizeof(int64_t));
   if (new_codes.bytes > 0) { CUVS_HIP_TRY(hipMemsetAsync(new_codes.ptr, 0, new_codes.bytes, s)); }
   if (new_ids.bytes > 0) { CUVS_HIP_TRY(hipMemsetAsync(new_ids.ptr, 0xFF, new_ids.bytes, s)); }

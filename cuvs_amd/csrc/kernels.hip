@@ -382,6 +382,13 @@ __global__ __launch_bounds__(kBlock) void rotate_kernel(const float* __restrict_
   }
 }
 
+/** Sort key of pair i: its list, the pairs past each query's leading probes in a second range. */
+__device__ __forceinline__ uint32_t pair_bin(uint32_t label, uint32_t i, uint32_t n_probes,
+                                             uint32_t lead_probes, uint32_t n_lists)
+{
+  return (i % n_probes) < lead_probes ? label : label + n_lists;
+}
+
 /** One wave per query: inclusive prefix sums of the probed list sizes in probe order. */
 __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __restrict__ list_sizes,
                                                             const uint32_t* __restrict__ probes,
@@ -390,7 +397,9 @@ __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __res
                                                             uint32_t* __restrict__ chunk_indices,
                                                             uint32_t* __restrict__ n_samples,
                                                             unsigned long long* stats,
-                                                            uint32_t lead_probes)
+                                                            uint32_t lead_probes,
+                                                            uint32_t* __restrict__ pair_counts,
+                                                            uint32_t n_lists)
 {
   const uint32_t q    = blockIdx.x;
   const uint32_t lane = threadIdx.x;
@@ -399,7 +408,12 @@ __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __res
   for (uint32_t p0 = 0; p0 < n_probes; p0 += 64) {
     const uint32_t p = p0 + lane;
     uint32_t sz      = 0;
-    if (p < n_probes) { sz = list_sizes[probes[uint64_t(q) * n_probes + p]]; }
+    if (p < n_probes) {
+      const uint32_t label = probes[uint64_t(q) * n_probes + p];
+      sz                   = list_sizes[label];
+      // histogram of the pair ordering, while the probe is at hand
+      if (pair_counts != nullptr) { atomicAdd(&pair_counts[pair_bin(label, p, n_probes, lead_probes, n_lists)], 1u); }
+    }
     padded_rows += (sz + 31u) & ~31u;
     if (p < lead_probes) { lead_rows += (sz + 31u) & ~31u; }
     const uint32_t incl = wave_inclusive_scan(sz) + carry;
@@ -422,13 +436,6 @@ __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __res
   }
 }
 
-/** Sort key of pair i: its list, the pairs past each query's leading probes in a second range. */
-__device__ __forceinline__ uint32_t pair_bin(uint32_t label, uint32_t i, uint32_t n_probes,
-                                             uint32_t lead_probes, uint32_t n_lists)
-{
-  return (i % n_probes) < lead_probes ? label : label + n_lists;
-}
-
 __global__ void pair_histogram_kernel(const uint32_t* __restrict__ probes, uint32_t n_pairs,
                                       uint32_t n_probes, uint32_t lead_probes, uint32_t n_lists,
                                       uint32_t* __restrict__ counts)
@@ -437,28 +444,30 @@ __global__ void pair_histogram_kernel(const uint32_t* __restrict__ probes, uint3
   if (i < n_pairs) { atomicAdd(&counts[pair_bin(probes[i], i, n_probes, lead_probes, n_lists)], 1u); }
 }
 
-/** Single block: cursors[l] = exclusive prefix sum of counts[l]. */
-__global__ __launch_bounds__(kBlock) void exclusive_scan_kernel(const uint32_t* __restrict__ counts,
-                                                                 uint32_t n,
-                                                                 uint32_t* __restrict__ cursors)
+/** Single block of 1024 threads: cursors[l] = exclusive prefix sum of counts[l].  Thread t owns
+ *  the contiguous range [t * per, (t + 1) * per). */
+constexpr uint32_t kScanThreads = 1024;
+__global__ __launch_bounds__(kScanThreads) void exclusive_scan_kernel(const uint32_t* __restrict__ counts,
+                                                                      uint32_t n,
+                                                                      uint32_t* __restrict__ cursors)
 {
-  __shared__ uint32_t wave_sums[kBlock / 64];
-  __shared__ uint32_t s_carry;
-  if (threadIdx.x == 0) { s_carry = 0; }
+  __shared__ uint32_t wave_sums[kScanThreads / 64];
+  const uint32_t tid = threadIdx.x;
+  const uint32_t per = (n + kScanThreads - 1u) / kScanThreads;
+  const uint32_t lo  = tid * per;
+  const uint32_t hi  = lo + per < n ? lo + per : n;
+  uint32_t sum       = 0;
+  for (uint32_t i = lo; i < hi; i++) { sum += counts[i]; }
+  uint32_t incl = wave_inclusive_scan(sum);
+  if ((tid & 63u) == 63u) { wave_sums[tid >> 6] = incl; }
   __syncthreads();
-  for (uint32_t i0 = 0; i0 < n; i0 += kBlock) {
-    const uint32_t i = i0 + threadIdx.x;
-    const uint32_t v = i < n ? counts[i] : 0u;
-    uint32_t incl    = wave_inclusive_scan(v);
-    if ((threadIdx.x & 63u) == 63u) { wave_sums[threadIdx.x >> 6] = incl; }
-    __syncthreads();
-    uint32_t base = s_carry;
-    for (uint32_t w = 0; w < (threadIdx.x >> 6); w++) { base += wave_sums[w]; }
-    incl += base;
-    if (i < n) { cursors[i] = incl - v; }
-    __syncthreads();
-    if (threadIdx.x == kBlock - 1) { s_carry = incl; }
-    __syncthreads();
+  uint32_t base = 0;
+  for (uint32_t w = 0; w < (tid >> 6); w++) { base += wave_sums[w]; }
+  uint32_t run = base + incl - sum;
+  for (uint32_t i = lo; i < hi; i++) {
+    const uint32_t v = counts[i];
+    cursors[i]       = run;
+    run += v;
   }
 }
 
@@ -1045,28 +1054,35 @@ void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries,
 void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
                           uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
                           uint32_t* n_samples, unsigned long long* stats, uint32_t lead_probes,
-                          hipStream_t stream)
+                          uint32_t* pair_counts, uint32_t n_lists, hipStream_t stream)
 {
   if (n_queries == 0) { return; }
+  if (pair_counts != nullptr) {
+    launch_fill_u32(pair_counts, 0, lead_probes < n_probes ? 2 * n_lists : n_lists, stream);
+  }
   chunk_indices_kernel<<<n_queries, 64, 0, stream>>>(list_sizes, probes, n_probes, row_chunk_bytes,
-                                                     chunk_indices, n_samples, stats, lead_probes);
+                                                     chunk_indices, n_samples, stats, lead_probes,
+                                                     pair_counts, n_lists);
   CUVS_LAUNCH_CHECK();
 }
 
 void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
                         const uint8_t* const* data_ptrs, uint32_t n_pairs, uint32_t n_probes,
                         uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
-                        pair_desc* desc, uint32_t lead_probes, uint8_t* alive, hipStream_t stream)
+                        pair_desc* desc, uint32_t lead_probes, uint8_t* alive, bool counted,
+                        hipStream_t stream)
 {
   if (n_pairs == 0) { return; }
   const uint32_t n_bins = lead_probes < n_probes ? 2 * n_lists : n_lists;
   uint32_t* counts      = counters;
   uint32_t* cursors     = counters + n_bins;
-  launch_fill_u32(counts, 0, n_bins, stream);
-  pair_histogram_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(probes, n_pairs, n_probes,
-                                                                      lead_probes, n_lists, counts);
-  CUVS_LAUNCH_CHECK();
-  exclusive_scan_kernel<<<1, kBlock, 0, stream>>>(counts, n_bins, cursors);
+  if (!counted) {
+    launch_fill_u32(counts, 0, n_bins, stream);
+    pair_histogram_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(probes, n_pairs, n_probes,
+                                                                        lead_probes, n_lists, counts);
+    CUVS_LAUNCH_CHECK();
+  }
+  exclusive_scan_kernel<<<1, kScanThreads, 0, stream>>>(counts, n_bins, cursors);
   CUVS_LAUNCH_CHECK();
   pair_scatter_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(
     probes, chunk_indices, data_ptrs, n_pairs, n_probes, lead_probes, n_lists, cursors, pair_order,

@@ -88,10 +88,12 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
     if (slot >= n_pairs) { d.n_rows = 0; d.slot = 0xFFFFFFFFu; }
     return d;
   };
-  auto chunk_ptr = [&](const uint8_t* list_data, uint32_t row) {
+  // first chunk of row (64 * tile + lane) of a list; the code arena carries two groups of slack
+  // after the last list, so whole tiles can be read without clamping the row
+  const uint32_t lane_off = (lane >> 5) * group_bytes + (lane & 31u) * 16u;
+  auto chunk_ptr = [&](const uint8_t* list_data, uint32_t tile) {
     return reinterpret_cast<const GLOBAL_AS u32x4*>(reinterpret_cast<uintptr_t>(list_data) +
-                                                    uint64_t(row >> 5) * group_bytes +
-                                                    uint64_t(row & 31u) * 16u);
+                                                    uint64_t(tile) * (2u * group_bytes) + lane_off);
   };
   // staging element (pair tid / NDIFF, dimension tid % NDIFF) of iteration `it`
   auto fetch_diff = [&](uint32_t it) -> float {
@@ -112,7 +114,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   u32x4 cur      = {0u, 0u, 0u, 0u};
   uint32_t thr   = 0xFFFFFFFFu;
   if (my_d.n_rows != 0) {
-    cur = *chunk_ptr(my_d.data, lane < my_d.n_rows ? lane : 0u);
+    cur = *chunk_ptr(my_d.data, 0u);
     thr = a.query_kth[my_d.q];
   }
   if (tid < G * NDIFF) { diff_all[tid] = staged; }
@@ -161,10 +163,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
       for (uint32_t tile = 0; tile < n_tiles && !in_play; tile++) {
         const uint32_t i = tile * 64u + lane;
         u32x4 ahead      = cur;
-        if (tile + 1u < n_tiles) {
-          const uint32_t in = i + 64u;
-          ahead             = *chunk_ptr(my_d.data, in < n_rows ? in : 0u);
-        }
+        if (tile + 1u < n_tiles) { ahead = *chunk_ptr(my_d.data, tile + 1u); }
         const uint32_t w[4] = {cur.x, cur.y, cur.z, cur.w};
         acc_t acc           = acc_t(0);
 #pragma unroll
@@ -195,7 +194,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
     my_d = nxt_d;
     thr  = 0xFFFFFFFFu;
     if (my_d.n_rows != 0) {
-      cur = *chunk_ptr(my_d.data, lane < my_d.n_rows ? lane : 0u);
+      cur = *chunk_ptr(my_d.data, 0u);
       thr = a.query_kth[my_d.q];
     }
     it = nxt_it;
@@ -212,17 +211,19 @@ void launch_screen_sub(const scan_args& a, const pair_desc* desc, uint32_t n_pai
   auto kernel       = scan_screen_kernel<SUBS, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>;
   const size_t smem = kScreenLdsBase + size_t(kScreenG) * SUBS * 256 * sizeof(lut_t) +
                       size_t(kScreenG) * SUBS * PQ_LEN * 4;
-  static int n_cu = 0;
+  static int n_cu = 0, per_cu = 0;  // per instance
   if (n_cu == 0) {
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
     int dev = 0;
     CUVS_HIP_TRY(hipGetDevice(&dev));
     CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+    // persistent blocks: exactly as many as are resident at once
+    CUVS_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kScreenThreads, smem));
+    per_cu = std::max(per_cu, 1);
   }
   const uint32_t n_iters = (n_pairs + kScreenG - 1) / kScreenG;
-  const uint32_t per_cu  = std::min<uint32_t>(8u, uint32_t((150u * 1024u) / smem));
-  uint32_t grid          = uint32_t(n_cu) * std::max(per_cu, 1u);
+  uint32_t grid          = uint32_t(n_cu) * uint32_t(per_cu);
   if (grid > n_iters) { grid = n_iters; }
   const uint32_t n_chunks    = (a.pq_dim + 15u) / 16u;
   const uint32_t group_bytes = n_chunks * 512u;

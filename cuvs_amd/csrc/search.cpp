@@ -404,9 +404,10 @@ void search(cuvs::resources const& res_c,
     detail::launch_rotate(qf, ix.rotation_t.as<float>(), nq, ix.dim, ix.rot_dim,
                           ix.rotation_is_identity, cosine, rot_q, s);
     detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
-                                 ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead, s);
+                                 ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead,
+                                 counters, ix.n_lists, s);
     detail::launch_order_pairs(probes, chunk, ix.data_ptrs.as<const uint8_t*>(), nq * P, P,
-                               ix.n_lists, counters, order, desc, lead, alive, s);
+                               ix.n_lists, counters, order, desc, lead, alive, true, s);
     if (pl.fused) { detail::launch_fill_u32(kth, 0xFFFFFFFFu, nq, s); }
     mark(2);
 
