@@ -135,7 +135,8 @@ def main():
     early_stop = stage["n_screened_pairs"] > 0
     if early_stop:
         # the scan stage is three launches; the screening kernel is the dominant one.  Its
-        # algorithmic bytes are one 16-byte chunk per (padded) row of every screened pair.
+        # algorithmic bytes are the leading 8 bytes (8 one-byte codes) of every (padded) row of every
+        # screened pair.
         parts = {"lead_scan": (mean("lead_scan_ms"), stage["lead_bytes"] / launches),
                  "screen": (mean("screen_ms"), stage["screen_bytes"] / launches),
                  "survivor_scan": (mean("survivor_scan_ms"), stage["survivor_bytes"] / launches)}

@@ -252,6 +252,8 @@ bool launch_scan_quad(const scan_args& a, hipStream_t stream);
  * (`n_survivors` counts them) and their slot is marked in `alive`.
  */
 bool scan_screen_supported(const scan_args& a);
+/** Bytes of each row the screen reads (8 or 16). */
+uint32_t scan_screen_bytes_per_row();
 void launch_scan_screen(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
                         pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
                         hipStream_t stream);

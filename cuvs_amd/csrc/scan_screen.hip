@@ -30,6 +30,13 @@ namespace {
 #define LDS_AS __attribute__((address_space(3)))
 #define GLOBAL_AS __attribute__((address_space(1)))
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+/** Leading codes of a row: 8 bytes when the screen sums at most 8 subspaces, else the 16-byte chunk. */
+template <int SUBS>
+struct screen_codes {
+  using type = typename std::conditional<(SUBS <= 8), u32x2, u32x4>::type;
+};
 
 constexpr uint32_t kScreenThreads = 256;
 constexpr uint32_t kScreenG       = 4;   // pairs per block iteration = waves per block
@@ -47,6 +54,17 @@ __device__ __forceinline__ float opaque_one_s()
   return one;
 }
 
+/** How many leading subspaces the screen sums (of the 16 in the first chunk): 8, or 4 / 16 for A/B runs. */
+inline int screen_subspaces()
+{
+  static const int subs = [] {
+    const char* e = std::getenv("CUVS_AMD_SCREEN_SUBSPACES");
+    const int v   = e != nullptr ? std::atoi(e) : 8;
+    return (v == 4 || v == 8 || v == 16) ? v : 8;
+  }();
+  return subs;
+}
+
 template <int SUBS, int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER>
 __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   scan_args a, const pair_desc* __restrict__ desc, uint32_t n_pairs, uint32_t group_bytes,
@@ -55,6 +73,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   using traits = lut_traits<LUT>;
   using lut_t  = typename traits::storage;
   using acc_t  = typename std::conditional<OUT_HALF, _Float16, float>::type;
+  using codes_t = typename screen_codes<SUBS>::type;
   constexpr uint32_t G           = kScreenG;
   constexpr uint32_t SUB         = SUBS;
   constexpr uint32_t NDIFF       = SUB * PQ_LEN;  // leading rotated dimensions the first chunk covers
@@ -92,8 +111,8 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   // after the last list, so whole tiles can be read without clamping the row
   const uint32_t lane_off = (lane >> 5) * group_bytes + (lane & 31u) * 16u;
   auto chunk_ptr = [&](const uint8_t* list_data, uint32_t tile) {
-    return reinterpret_cast<const GLOBAL_AS u32x4*>(reinterpret_cast<uintptr_t>(list_data) +
-                                                    uint64_t(tile) * (2u * group_bytes) + lane_off);
+    return reinterpret_cast<const GLOBAL_AS codes_t*>(reinterpret_cast<uintptr_t>(list_data) +
+                                                      uint64_t(tile) * (2u * group_bytes) + lane_off);
   };
   // staging element (pair tid / NDIFF, dimension tid % NDIFF) of iteration `it`
   auto fetch_diff = [&](uint32_t it) -> float {
@@ -111,7 +130,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   uint32_t it   = blockIdx.x;
   float staged  = fetch_diff(it);
   pair_desc my_d = record(it, wid);
-  u32x4 cur      = {0u, 0u, 0u, 0u};
+  codes_t cur{};
   uint32_t thr   = 0xFFFFFFFFu;
   if (my_d.n_rows != 0) {
     cur = *chunk_ptr(my_d.data, 0u);
@@ -162,23 +181,35 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
       bool in_play             = false;
       for (uint32_t tile = 0; tile < n_tiles && !in_play; tile++) {
         const uint32_t i = tile * 64u + lane;
-        u32x4 ahead      = cur;
+        codes_t ahead    = cur;
         if (tile + 1u < n_tiles) { ahead = *chunk_ptr(my_d.data, tile + 1u); }
-        const uint32_t w[4] = {cur.x, cur.y, cur.z, cur.w};
-        acc_t acc           = acc_t(0);
-#pragma unroll
-        for (int kk = 0; kk < SUBS; kk++) {
-          const uint32_t c = (w[kk >> 2] >> ((kk & 3) * 8)) & 0xffu;
-          const lut_t v    = my_lut[kk * 256 + c];
-          if (OUT_HALF) {
-            acc = acc_t(acc + traits::to_half(v));
-          } else if (LUT == LUT_F16) {
-            acc = acc_t(fmaf(traits::to_float(v), one, float(acc)));
-          } else {
-            acc = acc_t(acc + traits::to_float(v));
-          }
+        uint32_t w[4] = {cur.x, cur.y, 0u, 0u};
+        if constexpr (SUBS > 8) {
+          w[2] = cur.z;
+          w[3] = cur.w;
         }
+        acc_t acc           = acc_t(0);
+        auto add_codes = [&](int first, int last) __attribute__((always_inline)) {
+#pragma unroll
+          for (int kk = first; kk < last; kk++) {
+            const uint32_t c = (w[kk >> 2] >> ((kk & 3) * 8)) & 0xffu;
+            const lut_t v    = my_lut[kk * 256 + c];
+            if (OUT_HALF) {
+              acc = acc_t(acc + traits::to_half(v));
+            } else if (LUT == LUT_F16) {
+              acc = acc_t(fmaf(traits::to_float(v), one, float(acc)));
+            } else {
+              acc = acc_t(acc + traits::to_float(v));
+            }
+          }
+        };
+        // most tiles are decided by half of the screening subspaces already
+        add_codes(0, SUBS / 2);
         in_play = __ballot(i < n_rows && !(__float_as_uint(float(acc)) > stop_bits)) != 0ull;
+        if (in_play) {
+          add_codes(SUBS / 2, SUBS);
+          in_play = __ballot(i < n_rows && !(__float_as_uint(float(acc)) > stop_bits)) != 0ull;
+        }
         cur     = ahead;
       }
       if (lane == 0) {
@@ -237,12 +268,7 @@ void launch_screen_instance(const scan_args& a, const pair_desc* desc, uint32_t 
                             pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
                             hipStream_t stream)
 {
-  // how many leading subspaces the screen sums (of the 16 in the first chunk)
-  static const int subs = [] {
-    const char* e = std::getenv("CUVS_AMD_SCREEN_SUBSPACES");
-    const int v   = e != nullptr ? std::atoi(e) : 8;
-    return (v == 4 || v == 8 || v == 16) ? v : 8;
-  }();
+  const int subs = screen_subspaces();
   if (subs == 4) {
     launch_screen_sub<4, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
   } else if (subs == 8) {
@@ -274,6 +300,8 @@ void launch_screen_types(const scan_args& a, const pair_desc* desc, uint32_t n_p
 }
 
 }  // namespace
+
+uint32_t scan_screen_bytes_per_row() { return screen_subspaces() <= 8 ? 8u : 16u; }
 
 bool scan_screen_supported(const scan_args& a)
 {

@@ -514,7 +514,9 @@ void search(cuvs::resources const& res_c,
     res.last_profile.scan_rows  = h[1];
     if (early_stop) {
       res.last_profile.lead_bytes   = h[2];
-      res.last_profile.screen_bytes = (h[0] - h[2]) / ix.n_chunks;  // one 16-byte chunk per row
+      // rows x leading bytes the screen reads
+      res.last_profile.screen_bytes =
+        (h[0] - h[2]) / (uint64_t(ix.n_chunks) * kIndexGroupVecLen) * detail::scan_screen_bytes_per_row();
     }
   }
   res.reset_workspace();

@@ -240,7 +240,7 @@ typedef struct {
   float survivor_scan_ms;  /* full scan of the pairs the screen kept */
   float reserved_;
   uint64_t lead_bytes;     /* scan_bytes share of the leading pairs */
-  uint64_t screen_bytes;   /* sum over screened pairs of round_up(list size, 32) * 16 */
+  uint64_t screen_bytes;   /* sum over screened pairs of round_up(list size, 32) * bytes read per row (8) */
   uint64_t survivor_bytes; /* scan_bytes share of the pairs the screen kept */
   uint64_t n_screened_pairs;
   uint64_t n_surviving_pairs;
