@@ -152,7 +152,7 @@ index<int64_t> build(cuvs::resources const& res,
     ix.codebook_kind == codebook_gen::PER_SUBSPACE ? ix.pq_dim : ix.n_lists;
   auto copy_in = [&](device_buffer& dst, const float* src, size_t n) {
     dst.allocate(n * sizeof(float));
-    CUVS_HIP_TRY(hipMemcpyAsync(dst.ptr, src, n * sizeof(float), hipMemcpyDeviceToDevice, stream));
+    CUVS_HIP_TRY(hipMemcpyAsync(dst.ptr, src, n * sizeof(float), hipMemcpyDefault, stream));
   };
   copy_in(ix.pq_centers, pq_centers, n_books * ix.pq_len * ix.book_size);
   copy_in(ix.centers, centers, size_t(ix.n_lists) * ix.dim_ext);
@@ -165,7 +165,7 @@ index<int64_t> build(cuvs::resources const& res,
   // transposed copy [dim, rot_dim] for coalesced reads, and the identity check
   std::vector<float> rot(size_t(ix.rot_dim) * ix.dim), rot_t(size_t(ix.rot_dim) * ix.dim);
   CUVS_HIP_TRY(hipMemcpyAsync(rot.data(), rotation_matrix, rot.size() * sizeof(float),
-                              hipMemcpyDeviceToHost, stream));
+                              hipMemcpyDefault, stream));
   CUVS_HIP_TRY(hipStreamSynchronize(stream));
   bool identity = ix.rot_dim == ix.dim;
   for (uint32_t r = 0; r < ix.rot_dim; r++) {

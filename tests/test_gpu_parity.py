@@ -374,3 +374,86 @@ def test_early_stop_with_filter_and_small_lists(orc):
     want_nb, want_d = orc.search(ix, q, 20, 40, lut_dtype=ORC_DT[R_16F], filter_bitset=bits,
                                  filter_nbits=n)
     H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
+
+
+# --- index files: cuVS format version 4, a sequence of NumPy records ---
+
+def _read_records(path):
+    """Every record of the file through NumPy's own .npy reader."""
+    out = []
+    with open(path, "rb") as f:
+        f.seek(0, 2)
+        end = f.tell()
+        f.seek(0)
+        while f.tell() < end:
+            out.append(np.lib.format.read_array(f, allow_pickle=False))
+    return out
+
+
+@pytest.mark.parametrize("pq_bits,pq_dim,kind", [(8, 16, "subspace"), (5, 8, "cluster")])
+def test_serialize_round_trip_and_numpy_readable(orc, tmp_path, pq_bits, pq_dim, kind):
+    data, model, queries, index, ix, gpu_codes = _case(orc, 900, 32, 7, pq_dim, pq_bits, kind=kind,
+                                                       metric="inner_product", n_queries=20)
+    path = str(tmp_path / "index.bin")
+    ivf_pq.save(path, index)
+    rec = _read_records(path)
+    # header scalars (ivf_pq_serialize.cuh:49-59)
+    assert [int(r) for r in rec[:5]] == [4, 900, 32, pq_bits, pq_dim]
+    assert rec[1].dtype == np.int64 and rec[2].dtype == np.uint32
+    assert int(rec[6]) == 6 and int(rec[7]) == (1 if kind == "cluster" else 0) and int(rec[8]) == 1
+    assert int(rec[9]) == 7
+    # model tensors and list sizes
+    pq_len = 32 // pq_dim
+    assert rec[10].shape == ((7 if kind == "cluster" else pq_dim), pq_len, 1 << pq_bits)
+    assert np.array_equal(rec[10], model["pq_centers"])
+    assert np.array_equal(rec[11], model["centers"]) and rec[11].shape == (7, 40)
+    assert np.array_equal(rec[12], model["centers_rot"])
+    assert np.array_equal(rec[13], model["rotation_matrix"])
+    assert np.array_equal(rec[14], ix.list_sizes) and rec[14].dtype == np.uint32
+    # per list: size, interleaved codes, ids
+    pos = 15
+    n_chunks = -(-pq_dim // (128 // pq_bits))
+    for l in range(7):
+        size = int(rec[pos])
+        pos += 1
+        assert size == ix.list_sizes[l]
+        if size == 0:
+            continue
+        codes, ids = rec[pos], rec[pos + 1]
+        pos += 2
+        assert codes.shape == (-(-size // 32), n_chunks, 32, 16) and codes.dtype == np.uint8
+        assert ids.shape == (size,) and ids.dtype == np.int64
+        assert np.array_equal(orc.unpack_list(codes.reshape(-1), size, pq_dim, pq_bits), gpu_codes[l])
+        assert np.array_equal(ids, index.list_indices(l).cpu().numpy())
+    assert pos == len(rec)
+
+    loaded = ivf_pq.load(path)
+    assert len(loaded) == 900 and loaded.pq_dim == pq_dim and loaded.pq_bits == pq_bits
+    assert torch.equal(loaded.list_sizes, index.list_sizes)
+    assert torch.equal(loaded.centers, index.centers)
+    sp = ivf_pq.SearchParams(n_probes=4, lut_dtype=R_16F)
+    d1, n1 = ivf_pq.search(sp, index, G.to_dev(queries), 10)
+    d2, n2 = ivf_pq.search(sp, loaded, G.to_dev(queries), 10)
+    assert torch.equal(n1, n2) and torch.equal(d1, d2)
+    # a loaded index can be extended
+    ivf_pq.extend(loaded, G.to_dev(data[:50]), G.to_dev(np.arange(5000, 5050, dtype=np.int64)))
+    assert len(loaded) == 950
+
+
+def test_deserialize_rejects_damaged_files(orc, tmp_path):
+    data, model, queries, index, ix, _ = _case(orc, 300, 16, 4, 8, 8, n_queries=4)
+    path = str(tmp_path / "index.bin")
+    ivf_pq.save(path, index)
+    raw = open(path, "rb").read()
+    cut = str(tmp_path / "cut.bin")
+    open(cut, "wb").write(raw[: len(raw) // 2])
+    with pytest.raises(CuvsError, match="truncated|NumPy"):
+        ivf_pq.load(cut)
+    bad = bytearray(raw)
+    bad[raw.index(b"\x93NUMPY", 1)] = 0x00  # magic of the second record
+    badp = str(tmp_path / "bad.bin")
+    open(badp, "wb").write(bytes(bad))
+    with pytest.raises(CuvsError, match="bad magic"):
+        ivf_pq.load(badp)
+    with pytest.raises(CuvsError, match="Cannot open"):
+        ivf_pq.load(str(tmp_path / "missing.bin"))
