@@ -457,3 +457,48 @@ def test_deserialize_rejects_damaged_files(orc, tmp_path):
         ivf_pq.load(badp)
     with pytest.raises(CuvsError, match="Cannot open"):
         ivf_pq.load(str(tmp_path / "missing.bin"))
+
+
+# --- the other benchmark configurations, at a size the oracle finishes in seconds ---
+
+def _config_case(orc, x, q, n_lists, pq_dim, pq_bits, metric, kind):
+    model = H.train(x, n_lists, pq_dim, pq_bits, metric=metric, codebook_kind=kind, iters=5)
+    index = G.build_gpu_index(model, x, pq_dim, pq_bits, metric, kind)
+    ix, _ = G.read_back(orc, index, model, x.shape[1], pq_dim, pq_bits, metric, kind)
+    return index, ix
+
+
+@pytest.mark.parametrize("n_probes", [16, 32, 64])
+def test_config2_shape_normalised_fp32_l2(orc, n_probes):
+    """96-d L2-normalised fp32 mixture, pq_dim 48, 8 bit, fp16 table with fp32 distances."""
+    from cuvs_amd import testing
+    allrows = testing.gaussian_mixture(20200, 96, 100, 0.2, seed=1234, normalize_centers=True,
+                                       normalize_rows=True).numpy()
+    x, q = allrows[:20000], allrows[20000:]
+    index, ix = _config_case(orc, x, q, 128, 48, 8, "sqeuclidean", "subspace")
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, q, 10, n_probes, R_16F, R_32F)
+    H.compare_results(nb, d, want_nb, want_d, 2e-3, exact=True)
+
+
+def test_config4_shape_inner_product_4bit_fp8_half(orc):
+    """768-d unit-norm anisotropic mixture, inner product, pq_dim 384, 4-bit codes (two per byte),
+    8-bit table (signed variant), fp16 distances."""
+    from cuvs_amd import testing
+    allrows = testing.gaussian_mixture(3064, 768, 40, 0.05, seed=1234, dim_decay=0.9,
+                                       normalize_rows=True).numpy()
+    x, q = allrows[:3000], allrows[3000:]
+    index, ix = _config_case(orc, x, q, 24, 384, 4, "inner_product", "subspace")
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, q, 10, 8, R_8U, R_16F)
+    H.compare_results(nb, d, want_nb, want_d, 2e-3, exact=True)
+
+
+@pytest.mark.parametrize("batch", [1, 100])
+def test_config5_shape_half_rows_per_cluster(orc, batch):
+    """96-d fp16 rows, per-cluster codebooks, pq_dim 48, 8 bit, fp16 table, many probes; batch sizes
+    1 and 100."""
+    from cuvs_amd import testing
+    allrows = testing.gaussian_mixture(12100, 96, 300, 0.25, seed=1234).numpy().astype(np.float16)
+    x, q = allrows[:12000], allrows[12000:12000 + batch]
+    index, ix = _config_case(orc, x, q, 150, 48, 8, "sqeuclidean", "cluster")
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, q, 10, 100, R_16F, R_32F)
+    H.compare_results(nb, d, want_nb, want_d, 2e-3, exact=True)
