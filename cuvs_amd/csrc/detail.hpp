@@ -228,9 +228,14 @@ struct scan_args {
   unsigned long long* out_keys;   // fused: [n_queries, n_probes, k]
   float* out_scores;              // non-fused: [n_queries, max_samples]
   unsigned long long* timing;     // per-phase cycle sums (instrumented builds only), or null
+  void* global_lut;               // generic kernel: table scratch when it does not fit LDS, or null
 };
-/** LDS bytes the scan kernel needs for these arguments. */
+/** LDS bytes the scan kernel needs for these arguments (without the table when `global_lut` is
+ *  set), the bytes of one lookup table, and the number of blocks (= table slices) the generic
+ *  kernel runs with a global table. */
 size_t scan_lds_bytes(const scan_args& a);
+size_t scan_lut_bytes(const scan_args& a);
+uint32_t scan_global_lut_blocks();
 void launch_scan(const scan_args& a, hipStream_t stream);
 /** Persistent kernel for 8-bit codes and common shapes (scan_fast.hip); returns false when the
  *  arguments are outside what it covers.  Needs `a.desc`. */

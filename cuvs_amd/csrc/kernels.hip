@@ -12,6 +12,8 @@
  */
 #include "device_utils.cuh"
 
+#include <algorithm>
+
 namespace cuvs::neighbors::ivf_pq::detail {
 
 namespace {
@@ -513,7 +515,7 @@ struct scan_smem_tail {
   uint32_t thr;
 };
 
-template <int LUT, bool OUT_HALF, int BITS, bool FUSED>
+template <int LUT, bool OUT_HALF, int BITS, bool FUSED, bool GLOBAL_LUT>
 __global__ __launch_bounds__(kBlock) void scan_kernel(scan_args a)
 {
   using traits  = lut_traits<LUT>;
@@ -524,17 +526,22 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(scan_args a)
 
   extern __shared__ __align__(16) unsigned char dyn_smem[];
   const uint32_t lut_entries = a.pq_dim << BITS;
-  lut_t* lut                 = reinterpret_cast<lut_t*>(dyn_smem);
-  const uint32_t lut_bytes   = (lut_entries * uint32_t(sizeof(lut_t)) + 15u) & ~15u;
-  float* base_diff           = reinterpret_cast<float*>(dyn_smem + lut_bytes);
+  // the table lives in LDS, or, when it does not fit, in this block's slice of a global scratch
+  // buffer (the reference's third kernel variant, ivf_pq_compute_similarity_impl.cuh:337-596)
+  lut_t* lut = GLOBAL_LUT ? static_cast<lut_t*>(a.global_lut) + uint64_t(blockIdx.x) * lut_entries
+                          : reinterpret_cast<lut_t*>(dyn_smem);
+  const uint32_t lut_bytes = GLOBAL_LUT ? 0u : (lut_entries * uint32_t(sizeof(lut_t)) + 15u) & ~15u;
+  float* base_diff         = reinterpret_cast<float*>(dyn_smem + lut_bytes);
   const bool ip              = is_ip_metric(a.metric);
   const uint32_t diff_floats = a.rot_dim * (ip ? 2u : 1u);
   unsigned long long* cand =
     reinterpret_cast<unsigned long long*>(dyn_smem + lut_bytes + ((diff_floats * 4u + 15u) & ~15u));
   scan_smem_tail* tail = reinterpret_cast<scan_smem_tail*>(cand + (FUSED ? kCandCap : 0));
 
-  const uint32_t tid  = threadIdx.x;
-  const uint32_t pair = a.pair_order != nullptr ? a.pair_order[blockIdx.x] : blockIdx.x;
+  const uint32_t tid = threadIdx.x;
+  // one pair per block; with a global table a bounded grid walks over the pairs
+  for (uint32_t pb = blockIdx.x; pb < a.n_queries * a.n_probes; pb += gridDim.x) {
+  const uint32_t pair = a.pair_order != nullptr ? a.pair_order[pb] : pb;
   const uint32_t q    = pair / a.n_probes;
   const uint32_t p    = pair - q * a.n_probes;
   const uint32_t label = a.probes[uint64_t(q) * a.n_probes + p];
@@ -702,6 +709,8 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(scan_args a)
     }
     unsigned long long* out = a.out_keys + (uint64_t(q) * a.n_probes + p) * a.k;
     for (uint32_t r = tid; r < a.k; r += kBlock) { out[r] = r < cnt ? cand[r] : kInvalidKey; }
+  }
+  __syncthreads();  // the next pair of this block reuses the table and the candidate buffer
   }
 }
 
@@ -1090,10 +1099,26 @@ void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
   CUVS_LAUNCH_CHECK();
 }
 
-size_t scan_lds_bytes(const scan_args& a)
+size_t scan_lut_bytes(const scan_args& a)
 {
   const size_t elem = a.lut_dtype == CUDA_R_32F ? 4 : (a.lut_dtype == CUDA_R_16F ? 2 : 1);
-  const size_t lut  = ((size_t(a.pq_dim) << a.pq_bits) * elem + 15) & ~size_t(15);
+  return ((size_t(a.pq_dim) << a.pq_bits) * elem + 15) & ~size_t(15);
+}
+
+uint32_t scan_global_lut_blocks()
+{
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0;
+    CUVS_HIP_TRY(hipGetDevice(&dev));
+    CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+  }
+  return uint32_t(n_cu) * 4u;
+}
+
+size_t scan_lds_bytes(const scan_args& a)
+{
+  const size_t lut  = a.global_lut != nullptr ? 0 : scan_lut_bytes(a);
   const bool ip     = a.metric == int(DistanceType::InnerProduct) || a.metric == int(DistanceType::CosineExpanded);
   const size_t diff = (size_t(a.rot_dim) * (ip ? 2 : 1) * 4 + 15) & ~size_t(15);
   return lut + diff + (a.fused ? size_t(kCandCap) * 8 : 0) + 16;
@@ -1105,7 +1130,23 @@ template <int LUT, bool OUT_HALF, int BITS, bool FUSED>
 void launch_scan_instance(const scan_args& a, hipStream_t stream)
 {
   const size_t smem = scan_lds_bytes(a);
-  auto kernel       = scan_kernel<LUT, OUT_HALF, BITS, FUSED>;
+  if (a.global_lut != nullptr) {
+    if constexpr (BITS == 8) {
+      auto kernel = scan_kernel<LUT, OUT_HALF, BITS, FUSED, true>;
+      if (smem > 32 * 1024) {
+        CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+      }
+      const uint32_t n_pairs = a.n_queries * a.n_probes;
+      const uint32_t grid    = std::min(n_pairs, scan_global_lut_blocks());
+      kernel<<<grid, kBlock, smem, stream>>>(a);
+      CUVS_LAUNCH_CHECK();
+      return;
+    } else {
+      fail("a lookup table in global memory is only implemented for pq_bits = 8");
+    }
+  }
+  auto kernel = scan_kernel<LUT, OUT_HALF, BITS, FUSED, false>;
   if (smem > 32 * 1024) {
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));

@@ -323,15 +323,21 @@ void search(cuvs::resources const& res_c,
   sa.list_sizes   = ix.list_sizes.as<uint32_t>();
   sa.filter_bits  = filter_bits;
   sa.filter_nbits = filter_nbits;
-  const size_t lds = detail::scan_lds_bytes(sa);
-  CUVS_EXPECTS(lds <= kMaxLds,
-               "the lookup table (pq_dim = %u, pq_bits = %u, lut_dtype = %d) needs %zu bytes of LDS, "
-               "more than the %zu available; use a smaller lut_dtype",
-               ix.pq_dim, ix.pq_bits, int(params.lut_dtype), lds, kMaxLds);
+  // a table too large for LDS goes to global memory (8-bit codes, generic kernel)
+  const bool global_lut = detail::scan_lds_bytes(sa) > kMaxLds;
+  if (global_lut) {
+    CUVS_EXPECTS(ix.pq_bits == 8,
+                 "the lookup table (pq_dim = %u, pq_bits = %u, lut_dtype = %d) needs %zu bytes of LDS, "
+                 "more than the %zu available; use a smaller lut_dtype",
+                 ix.pq_dim, ix.pq_bits, int(params.lut_dtype), detail::scan_lds_bytes(sa), kMaxLds);
+  }
+  const size_t global_lut_bytes =
+    global_lut ? a256(detail::scan_lut_bytes(sa)) * detail::scan_global_lut_blocks() : 0;
 
   /* workspace carve-up for one batch */
   res.reset_workspace();
-  res.reserve_workspace(pl.fixed_bytes + size_t(Qb) * (pl.per_query_bytes + 64) + 16 * 256);
+  res.reserve_workspace(pl.fixed_bytes + size_t(Qb) * (pl.per_query_bytes + 64) + 16 * 256 +
+                        global_lut_bytes);
   auto* qt        = static_cast<float*>(
     res.workspace_alloc(size_t(ix.dim_ext) * detail::coarse_pad(Qb) * 4));
   auto* qf        = static_cast<float*>(res.workspace_alloc(size_t(Qb) * ix.dim * 4));
@@ -348,8 +354,10 @@ void search(cuvs::resources const& res_c,
   unsigned long long* keys = nullptr;
   float* all_scores        = nullptr;
   sa.fused                 = pl.fused;
-  const uint32_t quad_kpp  = force_generic_scan() ? 0u : detail::scan_quad_keys_per_pair(sa);
-  const bool fast_scan     = !force_generic_scan() && (quad_kpp != 0 || detail::scan_fast_supported(sa));
+  if (global_lut) { sa.global_lut = res.workspace_alloc(global_lut_bytes); }
+  const bool generic_only  = force_generic_scan() || global_lut;
+  const uint32_t quad_kpp  = generic_only ? 0u : detail::scan_quad_keys_per_pair(sa);
+  const bool fast_scan     = !generic_only && (quad_kpp != 0 || detail::scan_fast_supported(sa));
   const uint32_t kpp       = quad_kpp != 0 ? quad_kpp : k;  // candidate keys stored per pair
   if (fast_scan) {
     desc = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));

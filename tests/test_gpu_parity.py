@@ -502,3 +502,15 @@ def test_config5_shape_half_rows_per_cluster(orc, batch):
     index, ix = _config_case(orc, x, q, 150, 48, 8, "sqeuclidean", "cluster")
     nb, d, want_nb, want_d = _search_both(orc, index, ix, q, 10, 100, R_16F, R_32F)
     H.compare_results(nb, d, want_nb, want_d, 2e-3, exact=True)
+
+
+@pytest.mark.parametrize("k", [10, 300])
+def test_lookup_table_larger_than_lds_goes_to_global_memory(orc, k):
+    """pq_dim 192 x 256 entries x 4 bytes = 192 KB: more than the 160 KB of LDS."""
+    data, model, queries, index, ix, _ = _case(orc, 3000, 192, 8, 192, 8, n_queries=24)
+    for metric_lut in [(R_32F, R_32F)]:
+        nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, k, 4, *metric_lut)
+        H.compare_results(nb, d, want_nb, want_d, 1e-5, exact=True)
+    # the fp16 table of the same index (96 KB) stays in LDS and agrees with its own oracle run
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, k, 4, R_16F, R_32F)
+    H.compare_results(nb, d, want_nb, want_d, 2e-3, exact=True)
