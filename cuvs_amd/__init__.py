@@ -4,6 +4,7 @@ The Python layer is a thin ctypes binding over ``libcuvs_c.so`` (HIP kernels for
 cuVS C ABI); it mirrors ``cuvs.neighbors.ivf_pq`` of the reference Python package.
 """
 from . import ivf_pq  # noqa: F401
+from .refine import refine  # noqa: F401
 from .resources import Resources  # noqa: F401
 
-__all__ = ["ivf_pq", "Resources"]
+__all__ = ["ivf_pq", "refine", "Resources"]

@@ -90,6 +90,7 @@ EXPORTED_SYMBOLS = [
     "cuvsIvfPqSearch", "cuvsIvfPqSerialize", "cuvsIvfPqDeserialize", "cuvsIvfPqExtend",
     "cuvsIvfPqTransform", "cuvsAmdIvfPqSelectClusters", "cuvsAmdIvfPqSearchWithBitset",
     "cuvsAmdIvfPqExtendLabeled", "cuvsAmdIvfPqProfilingEnable", "cuvsAmdIvfPqGetSearchProfile",
+    "cuvsRefine",
 ]
 
 _lib = None
@@ -148,6 +149,7 @@ def lib():
     proto("cuvsIvfPqBuildPrecomputed", res_t, P(IndexParamsStruct), C.c_uint32, T, T, T, T,
           P(IndexStruct))
     proto("cuvsIvfPqSearch", res_t, P(SearchParamsStruct), P(IndexStruct), T, T, T)
+    proto("cuvsRefine", res_t, T, T, T, C.c_int, T, T)
     proto("cuvsIvfPqSerialize", res_t, C.c_char_p, P(IndexStruct))
     proto("cuvsIvfPqDeserialize", res_t, C.c_char_p, P(IndexStruct))
     proto("cuvsIvfPqExtend", res_t, T, T, P(IndexStruct))

@@ -285,6 +285,13 @@ struct merge_args {
 };
 void launch_merge(const merge_args& a, hipStream_t stream);
 
+/** Exact re-ranking of candidates (refine.hip): ids and distances of the k best candidates of every
+ *  query, ascending distance (descending similarity with `ip`). */
+void launch_refine(const void* dataset, const void* queries, elem_type type,
+                   const int64_t* candidates, int64_t n_rows, uint32_t n_queries, uint32_t dim,
+                   uint32_t n_candidates, uint32_t k, bool ip, bool sqrt_out, int64_t* indices,
+                   float* distances, hipStream_t stream);
+
 /* list maintenance and encoding */
 void launch_normalize_rows(float* x, uint64_t n_rows, uint32_t dim, hipStream_t stream);
 void launch_histogram(const uint32_t* labels, uint64_t n, uint32_t* counts, hipStream_t stream);

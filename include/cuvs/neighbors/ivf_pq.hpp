@@ -21,6 +21,8 @@ enum class DistanceType : int {
   L2Expanded     = 0,
   L2SqrtExpanded = 1,
   CosineExpanded = 2,
+  L2Unexpanded     = 4,
+  L2SqrtUnexpanded = 5,
   InnerProduct   = 6,
 };
 }  // namespace cuvs::distance

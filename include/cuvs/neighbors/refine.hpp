@@ -1,0 +1,30 @@
+/*
+ * C++ API of the refinement step (cuVS cpp/include/cuvs/neighbors/refine.hpp:62-68 and the
+ * overloads for half, int8_t and uint8_t that follow it).
+ */
+#pragma once
+
+#include <cuvs/core/resources.hpp>
+#include <cuvs/distance/distance.h>
+#include <cuvs/neighbors/ivf_pq.hpp>
+
+namespace cuvs::neighbors {
+
+/** For each query the exact distance to each of its candidates, the k = indices.extent(1) nearest
+ *  kept, ascending (descending similarity for InnerProduct).  T: float, _Float16, int8_t, uint8_t. */
+template <typename T>
+void refine(cuvs::resources const& res,
+            device_matrix_view<const T> dataset,
+            device_matrix_view<const T> queries,
+            device_matrix_view<const int64_t> neighbor_candidates,
+            device_matrix_view<int64_t> indices,
+            device_matrix_view<float> distances,
+            cuvs::distance::DistanceType metric = cuvs::distance::DistanceType::L2Unexpanded);
+
+/** Type-erased entry point behind the C API. */
+void refine(cuvs::resources const& res, const void* dataset, const void* queries,
+            ivf_pq::elem_type type, int64_t n_rows, int64_t n_queries, int64_t dim,
+            const int64_t* candidates, int64_t n_candidates, int64_t* indices, float* distances,
+            int64_t k, cuvs::distance::DistanceType metric);
+
+}  // namespace cuvs::neighbors

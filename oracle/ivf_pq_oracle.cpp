@@ -25,6 +25,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <cfloat>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -501,6 +502,86 @@ bool validate(const orc_index& ix, const orc_search_params& sp, uint32_t k, bool
 }  // namespace
 
 extern "C" {
+
+/* ---------------- refinement (refine_device.cuh:35-135) ---------------- */
+
+int orc_refine(const void* dataset, const void* queries, int row_type, int64_t n_rows,
+               uint32_t n_queries, uint32_t dim, const int64_t* candidates, uint32_t n_candidates,
+               uint32_t k, int metric, int64_t* indices, float* distances)
+{
+  if (k == 0 || k > n_candidates) {
+    g_error = "refine: k must be within [1, n_candidates]";
+    return 1;
+  }
+  if (metric != ORC_L2Expanded && metric != ORC_L2SqrtExpanded && metric != ORC_InnerProduct) {
+    g_error = "refine: unsupported metric";
+    return 1;
+  }
+  const bool ip = metric == ORC_InnerProduct;
+  struct scored {
+    float ordered;  // smaller is better
+    uint32_t slot;
+  };
+  std::vector<scored> v;
+  for (uint32_t q = 0; q < n_queries; q++) {
+    v.clear();
+    for (uint32_t c = 0; c < n_candidates; c++) {
+      const int64_t id = candidates[uint64_t(q) * n_candidates + c];
+      if (id < 0 || id >= n_rows) { continue; }
+      float dist = 0.0f;
+      if (row_type == ORC_T_F32 || row_type == ORC_T_F16) {
+        float acc = 0.0f;
+        for (uint32_t d = 0; d < dim; d++) {
+          float a, b;
+          if (row_type == ORC_T_F32) {
+            a = static_cast<const float*>(queries)[uint64_t(q) * dim + d];
+            b = static_cast<const float*>(dataset)[uint64_t(id) * dim + d];
+          } else {
+            a = half_to_float(static_cast<const uint16_t*>(queries)[uint64_t(q) * dim + d]);
+            b = half_to_float(static_cast<const uint16_t*>(dataset)[uint64_t(id) * dim + d]);
+          }
+          if (ip) {
+            acc += a * b;
+          } else {
+            const float diff = a - b;
+            acc += diff * diff;
+          }
+        }
+        dist = acc;
+      } else {
+        int64_t acc = 0;  // exact; the reference's 32-bit accumulators hold these sums too
+        for (uint32_t d = 0; d < dim; d++) {
+          int32_t a, b;
+          if (row_type == ORC_T_I8) {
+            a = static_cast<const int8_t*>(queries)[uint64_t(q) * dim + d];
+            b = static_cast<const int8_t*>(dataset)[uint64_t(id) * dim + d];
+          } else {
+            a = static_cast<const uint8_t*>(queries)[uint64_t(q) * dim + d];
+            b = static_cast<const uint8_t*>(dataset)[uint64_t(id) * dim + d];
+          }
+          acc += ip ? int64_t(a) * b : int64_t(a - b) * (a - b);
+        }
+        dist = row_type == ORC_T_I8 ? float(int32_t(acc)) : float(uint32_t(acc));
+      }
+      v.push_back(scored{ip ? -dist : dist, c});
+    }
+    std::sort(v.begin(), v.end(), [](const scored& x, const scored& y) {
+      return x.ordered < y.ordered || (x.ordered == y.ordered && x.slot < y.slot);
+    });
+    for (uint32_t r = 0; r < k; r++) {
+      int64_t id = -1;
+      float d    = FLT_MAX;
+      if (r < v.size()) {
+        id = candidates[uint64_t(q) * n_candidates + v[r].slot];
+        d  = ip ? -v[r].ordered : v[r].ordered;
+        if (metric == ORC_L2SqrtExpanded) { d = std::sqrt(d); }
+      }
+      indices[uint64_t(q) * k + r]   = id;
+      distances[uint64_t(q) * k + r] = d;
+    }
+  }
+  return 0;
+}
 
 const char* orc_last_error(void) { return g_error.c_str(); }
 

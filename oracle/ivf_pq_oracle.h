@@ -98,6 +98,16 @@ int orc_search(const orc_index* index, const orc_search_params* params, const vo
 int orc_encode(const orc_index* index, const void* rows, int row_type, uint64_t n_rows,
                uint32_t* labels, uint8_t* codes, int n_threads);
 
+/* refinement (cpp/src/neighbors/refine/refine_device.cuh:35-135, refine_host.hpp): exact distance of
+ * every query to each of its candidate rows, the k best kept in ascending (distance, candidate
+ * slot) order.  metric: ORC_L2Expanded (squared), ORC_L2SqrtExpanded, ORC_InnerProduct (largest
+ * first).  fp32 / fp16 rows accumulate in fp32 ascending dimension; int8 / uint8 rows in exact
+ * 32-bit integers, as the reference's accumulator types for them.  Candidates outside [0, n_rows)
+ * are skipped; unfilled outputs hold id -1 and FLT_MAX. */
+int orc_refine(const void* dataset, const void* queries, int row_type, int64_t n_rows,
+               uint32_t n_queries, uint32_t dim, const int64_t* candidates, uint32_t n_candidates,
+               uint32_t k, int metric, int64_t* indices, float* distances);
+
 const char* orc_last_error(void);
 
 #ifdef __cplusplus

@@ -88,6 +88,9 @@ def lib():
         L.orc_encode.restype = C.c_int
         L.orc_encode.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_uint64, C.c_void_p,
                                  C.c_void_p, C.c_int]
+        L.orc_refine.restype = C.c_int
+        L.orc_refine.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_uint32, C.c_uint32,
+                                 C.c_void_p, C.c_uint32, C.c_uint32, C.c_int, C.c_void_p, C.c_void_p]
         _lib = L
     return _lib
 
@@ -272,3 +275,21 @@ def encode(index, rows, n_threads=None):
     _check(lib().orc_encode(index.c_ptr(), _ptr(x), t, x.shape[0], _ptr(labels), _ptr(codes),
                             n_threads or default_threads()))
     return labels, codes
+
+
+def refine(dataset, queries, candidates, k, metric=0):
+    """Exact re-ranking of candidates (orc_refine): returns (indices, distances)."""
+    dataset = np.ascontiguousarray(dataset)
+    queries = np.ascontiguousarray(queries, dtype=dataset.dtype)
+    candidates = np.ascontiguousarray(candidates, dtype=np.int64)
+    row_type = {np.dtype(np.float32): 0, np.dtype(np.float16): 1, np.dtype(np.int8): 2,
+                np.dtype(np.uint8): 3}[dataset.dtype]
+    nq, nc = candidates.shape
+    indices = np.empty((nq, k), dtype=np.int64)
+    distances = np.empty((nq, k), dtype=np.float32)
+    rc = lib().orc_refine(_ptr(dataset), _ptr(queries), row_type, dataset.shape[0], nq,
+                          dataset.shape[1], _ptr(candidates), nc, k, metric, _ptr(indices),
+                          _ptr(distances))
+    if rc != 0:
+        raise RuntimeError(lib().orc_last_error().decode())
+    return indices, distances

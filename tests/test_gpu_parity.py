@@ -514,3 +514,63 @@ def test_lookup_table_larger_than_lds_goes_to_global_memory(orc, k):
     # the fp16 table of the same index (96 KB) stays in LDS and agrees with its own oracle run
     nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, k, 4, R_16F, R_32F)
     H.compare_results(nb, d, want_nb, want_d, 2e-3, exact=True)
+
+
+# --- refinement: exact re-ranking of the candidates an approximate search returned ---
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.int8, np.uint8])
+@pytest.mark.parametrize("metric", ["sqeuclidean", "euclidean", "inner_product"])
+def test_refine_matches_oracle(orc, dtype, metric):
+    from cuvs_amd import refine
+    rng = np.random.default_rng(5)
+    n, dim, nq, nc, k = 3000, 100, 70, 64, 10
+    data = H.make_data(n, dim, dtype, 21)
+    q = H.make_data(nq, dim, dtype, 22)
+    cand = rng.integers(0, n, (nq, nc)).astype(np.int64)
+    cand[0, :6] = [-1, n, -5, n + 1, 2 ** 40, -2 ** 40]
+    cand[1, :] = n
+    d, ids = refine(G.to_dev(data), G.to_dev(q), G.to_dev(cand), k, metric=metric)
+    code = {"sqeuclidean": 0, "euclidean": 1, "inner_product": 6}[metric]
+    want_ids, want_d = orc.refine(data, q, cand, k, code)
+    ids, d = ids.cpu().numpy(), d.cpu().numpy()
+    if np.dtype(dtype).kind in "iu":
+        # integer rows: exact arithmetic on both sides (the reduction order cannot matter)
+        assert np.array_equal(d, want_d)
+        # equal distances may come out in another candidate order only if the ids tie exactly
+        assert np.all((ids == want_ids) | (d == np.roll(d, 1, axis=1)) | (d == np.roll(d, -1, axis=1)))
+    else:
+        np.testing.assert_allclose(d, want_d, rtol=1e-5, atol=1e-6)
+        assert np.all((ids == want_ids) | np.isclose(d, want_d, rtol=1e-5, atol=1e-6))
+    assert (ids[1] == -1).all()
+
+
+def test_refine_after_search_raises_recall(orc):
+    """The use the reference documents: search 4k candidates, refine to k."""
+    from cuvs_amd import refine, testing
+    x, q, index, ix = _clustered_case(orc)
+    sp = ivf_pq.SearchParams(n_probes=20, lut_dtype=R_16F)
+    k = 10
+    _, cand = ivf_pq.search(sp, index, G.to_dev(q), 4 * k)
+    _, plain = ivf_pq.search(sp, index, G.to_dev(q), k)
+    d, ids = refine(G.to_dev(x), G.to_dev(q), cand, k)
+    truth = testing.exact_knn(torch.from_numpy(x), torch.from_numpy(q), k).numpy()
+    r_plain = testing.recall(plain.cpu().numpy(), truth)
+    r_ref = testing.recall(ids.cpu().numpy(), truth)
+    assert r_ref > r_plain and r_ref > 0.9
+    want_ids, want_d = orc.refine(x, q, cand.cpu().numpy(), k, 0)
+    np.testing.assert_allclose(d.cpu().numpy(), want_d, rtol=1e-5, atol=1e-6)
+
+
+def test_refine_validation(orc):
+    from cuvs_amd import refine
+    data = G.to_dev(np.zeros((10, 4), dtype=np.float32))
+    q = G.to_dev(np.zeros((3, 4), dtype=np.float32))
+    cand = G.to_dev(np.zeros((3, 5), dtype=np.int64))
+    with pytest.raises(CuvsError, match="candidates must not be smaller than k"):
+        refine(data, q, cand, 6)
+    with pytest.raises(CuvsError, match="Number of columns must be equal"):
+        refine(data, G.to_dev(np.zeros((3, 5), dtype=np.float32)), cand, 2)
+    with pytest.raises(CuvsError, match="type mismatch"):
+        refine(data, G.to_dev(np.zeros((3, 4), dtype=np.float16)), cand, 2)
+    with pytest.raises(ValueError):
+        refine(data, q, cand, 2, metric="cosine")
