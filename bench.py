@@ -43,6 +43,8 @@ def main():
     ap.add_argument("--k", type=int, default=10)
     ap.add_argument("--lut", default="f16", choices=["f32", "f16", "fp8"])
     ap.add_argument("--internal", default="f32", choices=["f32", "f16"])
+    ap.add_argument("--refine-ratio", type=int, default=1,
+                    help="search refine_ratio * k candidates and re-rank them exactly (1 = off)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
@@ -52,7 +54,7 @@ def main():
     import numpy as np
     import torch
 
-    from cuvs_amd import ivf_pq, testing
+    from cuvs_amd import ivf_pq, refine, testing
     from cuvs_amd.resources import Resources
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
@@ -93,16 +95,23 @@ def main():
     log(f"index populated ({len(index)} rows) in {time.time() - t0:.1f}s")
 
     t0 = time.time()
-    truth = testing.exact_knn(data, queries, k, half=True).cpu().numpy()
+    truth = testing.exact_knn(data, queries, k).cpu().numpy()  # fp32: exact for 8-bit data
     log(f"exact ground truth in {time.time() - t0:.1f}s")
 
     sp = ivf_pq.SearchParams(n_probes=P, lut_dtype=lut_np, internal_distance_dtype=int_np,
                              max_internal_batch_size=max(nq, 1))
-    neighbors = torch.empty((nq, k), dtype=torch.int64, device=dev)
-    distances = torch.empty((nq, k), dtype=torch.float32, device=dev)
+    k_search = k * max(args.refine_ratio, 1)
+    neighbors = torch.empty((nq, k_search), dtype=torch.int64, device=dev)
+    distances = torch.empty((nq, k_search), dtype=torch.float32, device=dev)
+    refined_ids = torch.empty((nq, k), dtype=torch.int64, device=dev)
+    refined_d = torch.empty((nq, k), dtype=torch.float32, device=dev)
 
     def step():
-        ivf_pq.search(sp, index, queries, k, neighbors=neighbors, distances=distances, resources=res)
+        ivf_pq.search(sp, index, queries, k_search, neighbors=neighbors, distances=distances,
+                      resources=res)
+        if args.refine_ratio > 1:
+            refine(data, queries, neighbors, k, indices=refined_ids, distances=refined_d,
+                   resources=res)
 
     for _ in range(args.warmup):
         step()
@@ -116,7 +125,7 @@ def main():
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
     qps = nq * args.steps / elapsed
-    gpu_ids = neighbors.cpu().numpy()
+    gpu_ids = (refined_ids if args.refine_ratio > 1 else neighbors).cpu().numpy()
     gpu_recall = testing.recall(gpu_ids, truth)
     log(f"{ms_per_step:.2f} ms per batch of {nq}: {qps:,.0f} QPS, recall@{k} {gpu_recall:.4f}")
 
@@ -180,6 +189,7 @@ def main():
                    "n_rows": n, "dim": dim, "n_lists": n_lists, "pq_dim": pq_dim,
                    "pq_bits": pq_bits, "n_queries": nq, "k": k, "n_probes": P,
                    "lut_dtype": args.lut, "internal_distance_dtype": args.internal,
+                   "refine_ratio": args.refine_ratio,
                    "recall_at_k": gpu_recall,
                    "stage_ms": {s: stage[s] for s in ("coarse_ms", "rotate_ms", "scan_ms", "merge_ms")}},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -199,7 +209,7 @@ def main():
         "pairs_surviving": int(stage["n_surviving_pairs"]),
     }
 
-    if not args.no_cpu:
+    if not args.no_cpu and args.refine_ratio <= 1:
         out["cpu_baseline"] = cpu_baseline(args, index, model, queries, truth, gpu_ids, dim, pq_dim,
                                            pq_bits, P, k, log)
         out["config"]["oracle_recall_on_sample"] = out["cpu_baseline"].pop("oracle_recall")
