@@ -751,6 +751,7 @@ __global__ __launch_bounds__(64) void kth_bound_kernel(const unsigned long long*
   }
 }
 
+constexpr uint32_t kMergeMaxProbes = 8192;  // with the alive list: slots are kept as 16-bit numbers
 __global__ __launch_bounds__(kBlock) void merge_kernel(merge_args a, uint32_t out_cap)
 {
   extern __shared__ __align__(16) unsigned char dyn_smem[];
@@ -764,12 +765,21 @@ __global__ __launch_bounds__(kBlock) void merge_kernel(merge_args a, uint32_t ou
     if (a.alive == nullptr) {
       block_select_sorted([keys](uint32_t i) { return keys[i]; }, n, a.k, out, out_cap, sm);
     } else {
-      // pairs that the screen dropped wrote no keys
+      // pairs that the screen dropped wrote no keys: gather the slots that did, select among those
+      __shared__ uint16_t live_slots[kMergeMaxProbes];
+      __shared__ uint32_t n_live;
       const uint8_t* alive = a.alive + uint64_t(q) * a.n_probes;
       const uint32_t kpp   = a.keys_per_pair;
+      if (threadIdx.x == 0) { n_live = 0; }
+      __syncthreads();
+      for (uint32_t p = threadIdx.x; p < a.n_probes; p += kBlock) {
+        if (alive[p] != 0) { live_slots[atomicAdd(&n_live, 1u)] = uint16_t(p); }
+      }
+      __syncthreads();
+      const uint32_t n_keys = n_live * kpp;
       block_select_sorted(
-        [keys, alive, kpp](uint32_t i) { return alive[i / kpp] != 0 ? keys[i] : kInvalidKey; }, n,
-        a.k, out, out_cap, sm);
+        [keys, kpp](uint32_t i) { return keys[uint32_t(live_slots[i / kpp]) * kpp + i % kpp]; },
+        n_keys, a.k, out, out_cap, sm);
     }
   } else {
     n                = a.n_samples[q];

@@ -364,7 +364,7 @@ void search(cuvs::resources const& res_c,
   }
   // L2 early stop: lists of the leading probes in full, the others screened on their first chunk
   const uint32_t kLeadProbes = lead_probes();
-  const bool early_stop = fast_scan && P > kLeadProbes && detail::scan_screen_supported(sa) &&
+  const bool early_stop = fast_scan && P > kLeadProbes && P <= 8192 && detail::scan_screen_supported(sa) &&
                           !early_stop_disabled();
   const uint32_t lead          = early_stop ? kLeadProbes : P;
   detail::pair_desc* survivors = nullptr;
