@@ -40,6 +40,9 @@ def main():
     ap.add_argument("--lists", type=int, default=16384)
     ap.add_argument("--queries", type=int, default=10_000)
     ap.add_argument("--probes", type=int, default=64)
+    ap.add_argument("--dim", type=int, default=128)
+    ap.add_argument("--pq-dim", type=int, default=64)
+    ap.add_argument("--pq-bits", type=int, default=8)
     ap.add_argument("--k", type=int, default=10)
     ap.add_argument("--lut", default="f16", choices=["f32", "f16", "fp8"])
     ap.add_argument("--internal", default="f32", choices=["f32", "f16"])
@@ -59,7 +62,7 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda"
-    dim, pq_dim, pq_bits = 128, 64, 8
+    dim, pq_dim, pq_bits = args.dim, args.pq_dim, args.pq_bits
     n, nq, n_lists, P, k = args.rows, args.queries, args.lists, args.probes, args.k
     lut_np = {"f32": np.float32, "f16": np.float16, "fp8": np.uint8}[args.lut]
     int_np = {"f32": np.float32, "f16": np.float16}[args.internal]
@@ -153,7 +156,8 @@ def main():
         kernel_ms, kernel_bytes = parts["screen"]
     else:
         parts = {}
-        kernel_name = "scan_quad_kernel" if (args.lut != "f32" and k <= 64) else "scan_fast_kernel"
+        kernel_name = ("scan_kernel" if (pq_bits != 8 or (pq_dim, dim // pq_dim) not in ((64, 2), (48, 2), (32, 4)))
+                       else "scan_quad_kernel" if (args.lut != "f32" and k <= 64) else "scan_fast_kernel")
         kernel_ms, kernel_bytes = scan_stage_ms, bytes_all_lists
     achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9
     log(f"{kernel_name} {kernel_ms:.3f} ms per launch, {kernel_bytes / 1e9:.2f} GB algorithmic "
@@ -173,7 +177,8 @@ def main():
     torch.cuda.synchronize()
     del calib, calib_out
 
-    default_workload = (n, nq, n_lists, P, k) == (10_000_000, 10_000, 16384, 64, 10)
+    default_workload = (n, nq, n_lists, P, k, dim, pq_dim, pq_bits) == (10_000_000, 10_000, 16384, 64, 10,
+                                                                       128, 64, 8)
     traffic = (MEASURED_TRAFFIC.get((kernel_name, args.lut, args.internal))
                if default_workload else None)
 

@@ -611,32 +611,41 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(scan_args a)
       valid = id >= 0 && id < a.filter_nbits && ((a.filter_bits[id >> 5] >> (id & 31)) & 1u) != 0;
     }
     float score_f = 0.0f;
-    if (valid) {
+    // L2 sums only grow: when every row of the wave is above the bound after a chunk, the rest of
+    // the row cannot matter (compute_score's early stop); the wave then leaves the chunk loop
+    const uint32_t stop_bits = thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u;
+    bool stopped             = false;  // wave-uniform
+    {
       const uint8_t* ptr =
-        list_data + uint64_t(i >> 5) * n_chunks * 512u + uint64_t(i & 31u) * 16u;
+        list_data + uint64_t(valid ? (i >> 5) : 0u) * n_chunks * 512u + uint64_t(i & 31u) * 16u;
       acc_t acc        = acc_t(0);
       const lut_t* lh  = lut;
-      for (uint32_t m = 0; m < n_full; m++) {
-        const uint4 v       = *reinterpret_cast<const uint4*>(ptr + uint64_t(m) * 512u);
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      for (uint32_t m = 0; m < n_full && !stopped; m++) {
+        if (valid) {
+          const uint4 v       = *reinterpret_cast<const uint4*>(ptr + uint64_t(m) * 512u);
+          const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-        for (uint32_t kk = 0; kk < CPC; kk++) {
-          constexpr uint32_t mask = B - 1u;
-          const uint32_t bit      = kk * BITS;
-          const uint32_t word     = bit >> 5;
-          const uint32_t off      = bit & 31u;
-          uint32_t c              = w[word] >> off;
-          if (off + BITS > 32u) { c |= w[(word + 1u) & 3u] << (32u - off); }
-          c &= mask;
-          if (OUT_HALF) {
-            acc = acc_t(acc + traits::to_half(lh[(kk << BITS) + c]));
-          } else {
-            acc = acc_t(acc + traits::to_float(lh[(kk << BITS) + c]));
+          for (uint32_t kk = 0; kk < CPC; kk++) {
+            constexpr uint32_t mask = B - 1u;
+            const uint32_t bit      = kk * BITS;
+            const uint32_t word     = bit >> 5;
+            const uint32_t off      = bit & 31u;
+            uint32_t c              = w[word] >> off;
+            if (off + BITS > 32u) { c |= w[(word + 1u) & 3u] << (32u - off); }
+            c &= mask;
+            if (OUT_HALF) {
+              acc = acc_t(acc + traits::to_half(lh[(kk << BITS) + c]));
+            } else {
+              acc = acc_t(acc + traits::to_float(lh[(kk << BITS) + c]));
+            }
           }
         }
         lh += CPC << BITS;
+        if (FUSED && !ip && m + 1u < n_chunks) {
+          stopped = __ballot(valid && !(__float_as_uint(float(acc)) > stop_bits)) == 0ull;
+        }
       }
-      if (n_full < n_chunks) {
+      if (n_full < n_chunks && valid && !stopped) {
         const uint4 v       = *reinterpret_cast<const uint4*>(ptr + uint64_t(n_full) * 512u);
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
         const uint32_t rem  = a.pq_dim - n_full * CPC;
