@@ -107,6 +107,20 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
     if (slot >= n_pairs) { d.n_rows = 0; d.slot = 0xFFFFFFFFu; }
     return d;
   };
+  // the record a wave scans is the same in all its lanes: say so, and the tile loop's trip count,
+  // addresses and bound stay in scalar registers
+  auto uniform = [](pair_desc d) -> pair_desc {
+    const uint64_t p = reinterpret_cast<uint64_t>(d.data);
+    // the builtin returns a signed int: widen through uint32_t, or the low half sign-extends
+    const uint32_t hi = uint32_t(__builtin_amdgcn_readfirstlane(uint32_t(p >> 32)));
+    const uint32_t lo = uint32_t(__builtin_amdgcn_readfirstlane(uint32_t(p)));
+    const uint64_t u  = (uint64_t(hi) << 32) | uint64_t(lo);
+    d.data       = reinterpret_cast<const uint8_t*>(u);
+    d.q          = uint32_t(__builtin_amdgcn_readfirstlane(d.q));
+    d.slot       = uint32_t(__builtin_amdgcn_readfirstlane(d.slot));
+    d.n_rows     = uint32_t(__builtin_amdgcn_readfirstlane(d.n_rows));
+    return d;
+  };
   // first chunk of row (64 * tile + lane) of a list; the code arena carries two groups of slack
   // after the last list, so whole tiles can be read without clamping the row
   const uint32_t lane_off = (lane >> 5) * group_bytes + (lane & 31u) * 16u;
@@ -129,12 +143,12 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
 
   uint32_t it   = blockIdx.x;
   float staged  = fetch_diff(it);
-  pair_desc my_d = record(it, wid);
+  pair_desc my_d = uniform(record(it, wid));
   codes_t cur{};
   uint32_t thr   = 0xFFFFFFFFu;
   if (my_d.n_rows != 0) {
     cur = *chunk_ptr(my_d.data, 0u);
-    thr = a.query_kth[my_d.q];
+    thr = uint32_t(__builtin_amdgcn_readfirstlane(a.query_kth[my_d.q]));
   }
   if (tid < G * NDIFF) { diff_all[tid] = staged; }
   lds_barrier_s();
@@ -143,7 +157,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
     const bool has_next    = it + stride < n_iters;
     const uint32_t nxt_it  = has_next ? it + stride : it;
     if (has_next) { staged = fetch_diff(nxt_it); }
-    const pair_desc nxt_d = record(nxt_it, wid);
+    const pair_desc nxt_d = uniform(record(nxt_it, wid));
 
     /* ---- the G tables of the first chunk, entry `tid` of each subspace ---- */
 #pragma unroll
@@ -226,7 +240,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
     thr  = 0xFFFFFFFFu;
     if (my_d.n_rows != 0) {
       cur = *chunk_ptr(my_d.data, 0u);
-      thr = a.query_kth[my_d.q];
+      thr = uint32_t(__builtin_amdgcn_readfirstlane(a.query_kth[my_d.q]));
     }
     it = nxt_it;
     lds_barrier_s();  // every wave is done with the tables; next staged terms are visible
