@@ -39,6 +39,16 @@ uint64_t chunk_rows_for(const index_impl& ix, uint64_t n_rows)
   return std::min<uint64_t>(c, n_rows);
 }
 
+/** Rows encoded per pass: enough to fill the GPU, bounded by about 1 GiB for the float copy of the
+ *  rows plus the rotated residuals. */
+uint64_t encode_chunk_rows_for(const index_impl& ix, uint64_t n_rows)
+{
+  uint64_t c = (uint64_t(1) << 28) / std::max<uint32_t>(ix.dim + ix.rot_dim, 1);
+  c          = std::max<uint64_t>(c, 1024);
+  c          = std::min<uint64_t>(c, uint64_t(1) << 20);
+  return std::min<uint64_t>(c, n_rows);
+}
+
 /** Stages one chunk of rows on the device (when the input is host memory) and maps it to float. */
 struct row_stager {
   const void* src;
@@ -115,24 +125,25 @@ void extend(cuvs::resources const& res,
   CUVS_EXPECTS(uint64_t(ix.size) + n_rows < (uint64_t(1) << 40), "index too large");
   hipStream_t s        = res.stream();
   const bool cosine    = ix.metric == detail::DistanceType::CosineExpanded;
-  const uint64_t chunk = chunk_rows_for(ix, n_rows);
-
-  row_stager stager(new_vectors, type, ix.dim, chunk);
   device_buffer labels(n_rows * sizeof(uint32_t));
-  device_buffer scores;
 
   /* 1. list labels */
   if (labels_in != nullptr) {
     CUVS_HIP_TRY(hipMemcpyAsync(labels.ptr, labels_in, n_rows * sizeof(uint32_t),
                                 hipMemcpyDefault, s));
   } else {
-    scores.allocate(chunk * ix.n_lists * sizeof(float) + detail::kSelectSlackBytes);
-    for (uint64_t r0 = 0; r0 < n_rows; r0 += chunk) {
-      const uint64_t n = std::min(chunk, n_rows - r0);
-      float* xf        = stager.load(r0, n, cosine, s);
+    const uint64_t label_chunk = chunk_rows_for(ix, n_rows);
+    row_stager label_stager(new_vectors, type, ix.dim, label_chunk);
+    device_buffer scores(label_chunk * ix.n_lists * sizeof(float) + detail::kSelectSlackBytes);
+    for (uint64_t r0 = 0; r0 < n_rows; r0 += label_chunk) {
+      const uint64_t n = std::min(label_chunk, n_rows - r0);
+      float* xf        = label_stager.load(r0, n, cosine, s);
       predict_labels(res, ix, xf, n, scores.as<float>(), labels.as<uint32_t>() + r0);
     }
+    CUVS_HIP_TRY(hipStreamSynchronize(s));  // the stager and the scores go out of scope
   }
+  const uint64_t chunk = encode_chunk_rows_for(ix, n_rows);
+  row_stager stager(new_vectors, type, ix.dim, chunk);
 
   /* 2. new list sizes */
   device_buffer counts(sizeof(uint32_t) * ix.n_lists);

@@ -889,23 +889,31 @@ __global__ __launch_bounds__(kBlock) void encode_kernel(encode_args a)
 {
   constexpr uint32_t B   = 1u << BITS;
   constexpr uint32_t CPC = 128u / BITS;
-  const uint64_t r       = uint64_t(blockIdx.x) * kBlock + threadIdx.x;
-  if (r >= a.n_rows) { return; }
+  // per-subspace codebooks: the block stages one subspace's book in LDS at a time (two buffers)
+  // and every lane reads the same entry at the same time, a broadcast
+  constexpr uint32_t kBookMaxLen = 8;  // pq_len up to which the LDS path is used
+  __shared__ float sbook[2][PER_CLUSTER ? 1 : B * kBookMaxLen];
+  const bool lds_book = !PER_CLUSTER && a.pq_len <= kBookMaxLen;
+  const uint64_t r0   = uint64_t(blockIdx.x) * kBlock + threadIdx.x;
+  const bool active   = r0 < a.n_rows;
+  const uint64_t r    = active ? r0 : a.n_rows - 1u;  // idle lanes shadow the last row, write nothing
   const uint32_t label = a.labels[r];
   const float* x       = a.xf + r * a.dim;
   const float* c       = a.centers + uint64_t(label) * a.dim_ext;
   float* res           = a.scratch + r;  // element d at res[d * n_rows]
   const uint64_t rs    = a.n_rows;
   auto xval = [&](uint32_t d) -> float { return x[d]; };
-  if (a.identity_rotation) {
-    for (uint32_t d = 0; d < a.rot_dim; d++) { res[d * rs] = d < a.dim ? xval(d) - c[d] : 0.0f; }
-  } else {
-    for (uint32_t o = 0; o < a.rot_dim; o++) {
-      float acc = 0.0f;
-      for (uint32_t d = 0; d < a.dim; d++) {
-        acc = fmaf(a.rotation_t[uint64_t(d) * a.rot_dim + o], xval(d) - c[d], acc);
+  if (active) {
+    if (a.identity_rotation) {
+      for (uint32_t d = 0; d < a.rot_dim; d++) { res[d * rs] = d < a.dim ? xval(d) - c[d] : 0.0f; }
+    } else {
+      for (uint32_t o = 0; o < a.rot_dim; o++) {
+        float acc = 0.0f;
+        for (uint32_t d = 0; d < a.dim; d++) {
+          acc = fmaf(a.rotation_t[uint64_t(d) * a.rot_dim + o], xval(d) - c[d], acc);
+        }
+        res[o * rs] = acc;
       }
-      res[o * rs] = acc;
     }
   }
 
@@ -913,13 +921,29 @@ __global__ __launch_bounds__(kBlock) void encode_kernel(encode_args a)
   uint8_t* list_base   = nullptr;
   uint8_t* flat_row    = nullptr;
   const uint32_t row_bytes = (a.pq_dim * BITS + 7u) / 8u;
-  if (a.flat_codes != nullptr) {
-    flat_row = a.flat_codes + r * row_bytes;
-    for (uint32_t b = 0; b < row_bytes; b++) { flat_row[b] = 0; }
-  } else {
-    slot      = atomicAdd(&a.cursors[label], 1u);
-    list_base = a.data_ptrs[label] + uint64_t(slot >> 5) * a.n_chunks * 512u + uint64_t(slot & 31u) * 16u;
-    a.inds_ptrs[label][slot] = a.ids != nullptr ? a.ids[r] : a.first_id + int64_t(r);
+  if (active) {
+    if (a.flat_codes != nullptr) {
+      flat_row = a.flat_codes + r * row_bytes;
+      for (uint32_t b = 0; b < row_bytes; b++) { flat_row[b] = 0; }
+    } else {
+      slot      = atomicAdd(&a.cursors[label], 1u);
+      list_base = a.data_ptrs[label] + uint64_t(slot >> 5) * a.n_chunks * 512u + uint64_t(slot & 31u) * 16u;
+      a.inds_ptrs[label][slot] = a.ids != nullptr ? a.ids[r] : a.first_id + int64_t(r);
+    }
+  }
+  auto stage_book = [&](uint32_t j) {
+    // [t][code] in global memory -> [code][t] in LDS, so that one entry is one contiguous read
+    const float* book = a.pq_centers + uint64_t(j) * a.pq_len * B;
+    float* dst        = sbook[j & 1u];
+    for (uint32_t i = threadIdx.x; i < a.pq_len * B; i += kBlock) {
+      const uint32_t t = i / B;
+      const uint32_t l = i - t * B;
+      dst[l * a.pq_len + t] = book[i];
+    }
+  };
+  if (lds_book) {
+    stage_book(0);
+    __syncthreads();
   }
 
   uint32_t w[4] = {0, 0, 0, 0};
@@ -928,17 +952,43 @@ __global__ __launch_bounds__(kBlock) void encode_kernel(encode_args a)
       a.pq_centers + (PER_CLUSTER ? uint64_t(label) : uint64_t(j)) * a.pq_len * B;
     float best        = __uint_as_float(0x7f800000u);
     uint32_t code     = 0;
-    for (uint32_t l = 0; l < B; l++) {
-      float d = 0.0f;
-      for (uint32_t t = 0; t < a.pq_len; t++) {
-        const float v = res[uint64_t(j * a.pq_len + t) * rs] - book[uint64_t(t) * B + l];
-        d             = fmaf(v, v, d);
+    if (lds_book) {
+      if (j + 1u < a.pq_dim) { stage_book(j + 1u); }  // the other buffer: free since the last barrier
+      float rj[kBookMaxLen];
+#pragma unroll
+      for (uint32_t t = 0; t < kBookMaxLen; t++) {
+        rj[t] = t < a.pq_len ? res[uint64_t(j * a.pq_len + t) * rs] : 0.0f;
       }
-      if (d < best) {
-        best = d;
-        code = l;
+      const float* sb = sbook[j & 1u];
+      for (uint32_t l = 0; l < B; l++) {
+        float d = 0.0f;
+#pragma unroll
+        for (uint32_t t = 0; t < kBookMaxLen; t++) {
+          if (t < a.pq_len) {
+            const float v = rj[t] - sb[l * a.pq_len + t];
+            d             = fmaf(v, v, d);
+          }
+        }
+        if (d < best) {
+          best = d;
+          code = l;
+        }
+      }
+      __syncthreads();  // everyone is done with this subspace's book; the next one is staged
+    } else {
+      for (uint32_t l = 0; l < B; l++) {
+        float d = 0.0f;
+        for (uint32_t t = 0; t < a.pq_len; t++) {
+          const float v = res[uint64_t(j * a.pq_len + t) * rs] - book[uint64_t(t) * B + l];
+          d             = fmaf(v, v, d);
+        }
+        if (d < best) {
+          best = d;
+          code = l;
+        }
       }
     }
+    if (!active) { continue; }
     if (flat_row != nullptr) {
       const uint32_t bit = j * BITS;
       flat_row[bit >> 3] |= uint8_t(code << (bit & 7u));
