@@ -30,8 +30,10 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte chun
 constexpr uint32_t kQuadThreads = 1024;
 constexpr uint32_t kQuadWaves   = kQuadThreads / 64;
 constexpr uint32_t kQuadLdsBase = 16;   // see scan_fast.hip: no pointer constant may be null
-constexpr uint32_t kWaveCap     = 128;  // candidate keys per wave
-constexpr uint32_t kQuadMaxK    = 64;
+constexpr uint32_t kQuadMaxK    = 128;
+
+/** Candidate keys a wave buffers: room for k kept ones plus one tile of 64 new ones. */
+inline __host__ __device__ uint32_t quad_wave_cap(uint32_t k) { return k <= 64u ? 128u : 192u; }
 
 __device__ __forceinline__ void lds_barrier_q()
 {
@@ -45,22 +47,40 @@ __device__ __forceinline__ float opaque_one_q()
   return one;
 }
 
-/** Ascending bitonic sort of the 128 keys of one wave's buffer; lane l owns one compare-exchange
- *  per stage.  LDS operations of a wave execute in program order, so no barrier is needed. */
-__device__ __forceinline__ void wave_sort128(LDS_AS unsigned long long* buf, uint32_t lane)
+/** Ascending sort of the first `cap` keys (at most 256) of one wave's buffer: a bitonic network made of
+ *  ascending comparators only (each merge starts with a mirror step), run on the next power of two
+ *  with the missing top slots standing for keys larger than any other - a comparator that would
+ *  touch one of them never swaps, so it is skipped.  Every slot takes part in one comparator per
+ *  step, so the two comparators a lane owns in the 256-wide network do not interfere; LDS
+ *  operations of a wave execute in program order, so no barrier is needed. */
+__device__ __forceinline__ void wave_sort_cap(LDS_AS unsigned long long* buf, uint32_t lane, uint32_t cap)
 {
+  // comparators per step: half the next power of two
+  const uint32_t n_half = cap <= 2u ? 1u : (1u << (31 - __builtin_clz(cap - 1u)));
+  auto compare_exchange = [&](uint32_t i, uint32_t l) __attribute__((always_inline)) {
+    if (l < cap) {
+      const unsigned long long x = buf[i];
+      const unsigned long long y = buf[l];
+      if (x > y) {
+        buf[i] = y;
+        buf[l] = x;
+      }
+    }
+  };
 #pragma unroll 1
-  for (uint32_t size = 2; size <= kWaveCap; size <<= 1) {
+  for (uint32_t size = 2; size <= 2u * n_half; size <<= 1) {
+    const uint32_t half = size >> 1;
+    for (uint32_t c = lane; c < n_half; c += 64u) {
+      const uint32_t base = (c / half) * size;
+      const uint32_t off  = c & (half - 1u);
+      compare_exchange(base + off, base + size - 1u - off);
+    }
+    __builtin_amdgcn_wave_barrier();
 #pragma unroll 1
-    for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
-      const uint32_t pos         = 2 * lane - (lane & (stride - 1));
-      const uint32_t partner     = pos + stride;
-      const bool ascending       = (pos & size) == 0;
-      const unsigned long long x = buf[pos];
-      const unsigned long long y = buf[partner];
-      if ((x > y) == ascending) {
-        buf[pos]     = y;
-        buf[partner] = x;
+    for (uint32_t stride = size >> 2; stride > 0; stride >>= 1) {
+      for (uint32_t c = lane; c < n_half; c += 64u) {
+        const uint32_t i = (c / stride) * (2u * stride) + (c & (stride - 1u));
+        compare_exchange(i, i + stride);
       }
       __builtin_amdgcn_wave_barrier();
     }
@@ -108,7 +128,8 @@ __global__ __launch_bounds__(kQuadThreads, 4) void scan_quad_kernel(scan_args a)
   const uint32_t n_quads = (n_pairs + G - 1u) / G;
   const uint32_t stride  = gridDim.x;
   if (blockIdx.x >= n_quads) { return; }  // whole block, before any barrier
-  auto* my_cand          = cand_all + wid * kWaveCap;
+  const uint32_t wave_cap = quad_wave_cap(a.k);
+  auto* my_cand          = cand_all + wid * wave_cap;
   auto* my_lut           = lut_all + grp * lut_entries;
 
   float book[PER_CLUSTER ? 1 : QUARTER][PQ_LEN];
@@ -278,10 +299,9 @@ __global__ __launch_bounds__(kQuadThreads, 4) void scan_quad_kernel(scan_args a)
         const bool pass     = valid && okey <= thr;
         const unsigned long long mask = __ballot(pass);
         if (mask != 0ull) {
-          if (wcount + 64u > kWaveCap) {
+          if (wcount + 64u > wave_cap) {
             // make room: keep the k best of the buffer and tighten the wave's bound
-            for (uint32_t t = wcount + lane; t < kWaveCap; t += 64u) { my_cand[t] = kInvalidKey; }
-            wave_sort128(my_cand, lane);
+            wave_sort_cap(my_cand, lane, wcount);
             if (wcount >= a.k) {
               wcount            = a.k;
               const uint32_t t2 = uint32_t(my_cand[a.k - 1] >> 32);
@@ -303,12 +323,11 @@ __global__ __launch_bounds__(kQuadThreads, 4) void scan_quad_kernel(scan_args a)
       // this wave's best candidates of the pair
       unsigned long long* out = a.out_keys + (uint64_t(my_d.slot) * WG + wig) * a.k;
       if (wcount >= a.k) {
-        for (uint32_t t = wcount + lane; t < kWaveCap; t += 64u) { my_cand[t] = kInvalidKey; }
-        wave_sort128(my_cand, lane);
+        wave_sort_cap(my_cand, lane, wcount);  // only as wide as there are candidates
         wcount = a.k;
         if (lane == 0) { atomicMin(&a.query_kth[my_d.q], uint32_t(my_cand[a.k - 1] >> 32)); }
       }
-      if (lane < a.k) { out[lane] = lane < wcount ? my_cand[lane] : kInvalidKey; }
+      for (uint32_t t = lane; t < a.k; t += 64u) { out[t] = t < wcount ? my_cand[t] : kInvalidKey; }
     }
 
     if (!has_next) { break; }
@@ -332,11 +351,14 @@ void launch_quad_instance(const scan_args& a, hipStream_t stream)
   using lut_t     = typename lut_traits<LUT>::storage;
   auto kernel     = scan_quad_kernel<NCH, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER, IP, G>;
   const size_t smem = kQuadLdsBase + size_t(G) * NCH * 16 * 256 * sizeof(lut_t) +
-                      size_t(G) * NCH * 16 * PQ_LEN * (IP ? 2 : 1) * 4 + size_t(kQuadWaves) * kWaveCap * 8;
+                      size_t(G) * NCH * 16 * PQ_LEN * (IP ? 2 : 1) * 4 +
+                      size_t(kQuadWaves) * quad_wave_cap(a.k) * 8;
   static int n_cu = 0;
   if (n_cu == 0) {
+    // the largest request of any k this kernel serves
+    const size_t smem_max = smem + size_t(kQuadWaves) * (quad_wave_cap(kQuadMaxK) - quad_wave_cap(a.k)) * 8;
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(smem_max)));
     int dev = 0;
     CUVS_HIP_TRY(hipGetDevice(&dev));
     CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
@@ -392,7 +414,7 @@ uint32_t scan_quad_keys_per_pair(const scan_args& a)
   // four tables plus the staged terms must fit the 160 KB of LDS
   const size_t elem = a.lut_dtype == CUDA_R_16F ? 2 : 1;
   const size_t lds  = kQuadLdsBase + 4 * size_t(a.pq_dim) * 256 * elem + 4 * size_t(a.rot_dim) * (ip ? 2 : 1) * 4 +
-                     size_t(kQuadWaves) * kWaveCap * 8;
+                     size_t(kQuadWaves) * quad_wave_cap(a.k) * 8;
   if (lds > 160 * 1024) { return 0; }
   const bool shape = (a.pq_dim == 64 && a.pq_len == 2) || (a.pq_dim == 48 && a.pq_len == 2) ||
                      (a.pq_dim == 32 && a.pq_len == 4);
