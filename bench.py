@@ -147,12 +147,13 @@ def main():
     early_stop = stage["n_screened_pairs"] > 0
     if early_stop:
         # the scan stage is three launches; the screening kernel is the dominant one.  Its
-        # algorithmic bytes are the leading 8 bytes (8 one-byte codes) of every (padded) row of every
-        # screened pair.
+        # algorithmic bytes are the leading 4 bytes (4 one-byte codes, from the packed plane of
+        # leading codes) of every (padded) row of every screened pair; per-cluster codebooks use the
+        # table-building screen, which reads the leading 8 bytes from the interleaved lists.
         parts = {"lead_scan": (mean("lead_scan_ms"), stage["lead_bytes"] / launches),
                  "screen": (mean("screen_ms"), stage["screen_bytes"] / launches),
                  "survivor_scan": (mean("survivor_scan_ms"), stage["survivor_bytes"] / launches)}
-        kernel_name = "scan_screen_kernel"
+        kernel_name = "scan_screen_direct_kernel"
         kernel_ms, kernel_bytes = parts["screen"]
     else:
         parts = {}

@@ -116,6 +116,11 @@ struct index_impl {
   bool rotation_is_identity = false;
 
   device_buffer codes_arena, ids_arena;
+  /** 8-bit codes: the first eight code bytes of every row slot, packed (8 bytes per row next to the
+   *  arena's n_chunks * 16): the early-stop screen decides on these alone, and reading them here
+   *  touches half the cache lines the interleaved arena would, in whole lines.  Rebuilt whenever
+   *  the arena changes; empty for other code widths or 2^32 and more row slots. */
+  device_buffer lead_plane;
   std::vector<uint32_t> h_list_sizes;
   std::vector<uint64_t> h_row_offsets;  // [n_lists + 1], in rows, multiples of 32
   device_buffer list_sizes, data_ptrs, inds_ptrs;
@@ -126,6 +131,8 @@ struct index_impl {
   /** Recompute pointer tables, device sizes and the sorted prefix sums from the host vectors
    *  (role of ivf::detail::recompute_internal_state, cpp/src/neighbors/ivf_common.cuh:255-290). */
   void recompute_internal_state(hipStream_t stream);
+  /** Refill `lead_plane` from the codes arena (after the arena's contents changed). */
+  void rebuild_lead_plane(hipStream_t stream);
 };
 
 void init_index(index_impl& ix, const index_params& params, uint32_t dim);
@@ -185,7 +192,7 @@ struct pair_desc {
   uint32_t label;       // probed list
   uint32_t sample_off;  // sample number of the list's first row for this query
   uint32_t n_rows;      // list size
-  uint32_t pad;
+  uint32_t row_off;     // the list's first row slot in the arenas (low 32 bits)
 };
 static_assert(sizeof(pair_desc) == 32, "pair_desc must stay 32 bytes");
 
@@ -197,7 +204,8 @@ static_assert(sizeof(pair_desc) == 32, "pair_desc must stay 32 bytes");
  *  4 * n_lists + 4 words; with `counted` its first half already holds the histogram of the pairs
  *  (launch_chunk_indices with `pair_counts` makes it on the way). */
 void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
-                        const uint8_t* const* data_ptrs, uint32_t n_pairs, uint32_t n_probes,
+                        const uint8_t* const* data_ptrs, const int64_t* const* inds_ptrs,
+                        const int64_t* ids_base, uint32_t n_pairs, uint32_t n_probes,
                         uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
                         pair_desc* desc, uint32_t lead_probes, uint8_t* alive, bool counted,
                         hipStream_t stream);
@@ -229,6 +237,7 @@ struct scan_args {
   float* out_scores;              // non-fused: [n_queries, max_samples]
   unsigned long long* timing;     // per-phase cycle sums (instrumented builds only), or null
   void* global_lut;               // generic kernel: table scratch when it does not fit LDS, or null
+  const uint64_t* lead_plane;     // first eight code bytes of every row slot (8-bit codes), or null
 };
 /** LDS bytes the scan kernel needs for these arguments (without the table when `global_lut` is
  *  set), the bytes of one lookup table, and the number of blocks (= table slices) the generic
@@ -237,6 +246,10 @@ size_t scan_lds_bytes(const scan_args& a);
 size_t scan_lut_bytes(const scan_args& a);
 uint32_t scan_global_lut_blocks();
 void launch_scan(const scan_args& a, hipStream_t stream);
+/** plane[slot] = first eight bytes of row slot `slot` of an arena of 8-bit codes. */
+void launch_build_lead_plane(const uint8_t* arena, uint64_t* plane, uint64_t n_slots,
+                             uint32_t n_chunks, hipStream_t stream);
+constexpr uint64_t kLeadPlaneSlack = 512;  // slots past the last list that look-ahead loads of whole tiles may read
 /** Persistent kernel for 8-bit codes and common shapes (scan_fast.hip); returns false when the
  *  arguments are outside what it covers.  Needs `a.desc`. */
 bool scan_fast_supported(const scan_args& a);
@@ -258,7 +271,7 @@ bool launch_scan_quad(const scan_args& a, hipStream_t stream);
  */
 bool scan_screen_supported(const scan_args& a);
 /** Bytes of each row the screen reads (8 or 16). */
-uint32_t scan_screen_bytes_per_row();
+uint32_t scan_screen_bytes_per_row(bool per_cluster, bool lead_plane);
 void launch_scan_screen(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
                         pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
                         hipStream_t stream);

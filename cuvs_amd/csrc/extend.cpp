@@ -229,6 +229,7 @@ void extend(cuvs::resources const& res,
     a.scratch    = scratch.as<float>();
     detail::launch_encode(a, s);
   }
+  ix.rebuild_lead_plane(s);
   CUVS_HIP_TRY(hipStreamSynchronize(s));  // temporaries go out of scope
 }
 

@@ -87,6 +87,20 @@ void index_impl::recompute_internal_state(hipStream_t stream)
   size = accum_sorted_sizes[n_lists];
 }
 
+void index_impl::rebuild_lead_plane(hipStream_t stream)
+{
+  const uint64_t n_slots = h_row_offsets.empty() ? 0 : h_row_offsets[n_lists];
+  if (pq_bits != 8 || n_slots == 0 || n_slots + kLeadPlaneSlack > 0xFFFFFFFFull) {
+    lead_plane = device_buffer();
+    return;
+  }
+  device_buffer plane((n_slots + kLeadPlaneSlack) * sizeof(uint64_t));
+  CUVS_HIP_TRY(hipMemsetAsync(plane.ptr, 0, plane.bytes, stream));
+  launch_build_lead_plane(codes_arena.as<uint8_t>(), plane.as<uint64_t>(), n_slots, n_chunks, stream);
+  CUVS_HIP_TRY(hipStreamSynchronize(stream));  // the old plane is released on assignment
+  lead_plane = std::move(plane);
+}
+
 }  // namespace detail
 
 template <typename IdxT>

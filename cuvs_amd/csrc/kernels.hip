@@ -475,7 +475,9 @@ __global__ __launch_bounds__(kScanThreads) void exclusive_scan_kernel(const uint
 
 __global__ void pair_scatter_kernel(const uint32_t* __restrict__ probes,
                                     const uint32_t* __restrict__ chunk_indices,
-                                    const uint8_t* const* __restrict__ data_ptrs, uint32_t n_pairs,
+                                    const uint8_t* const* __restrict__ data_ptrs,
+                                    const int64_t* const* __restrict__ inds_ptrs,
+                                    const int64_t* ids_base, uint32_t n_pairs,
                                     uint32_t n_probes, uint32_t lead_probes, uint32_t n_lists,
                                     uint32_t* __restrict__ cursors,
                                     uint32_t* __restrict__ pair_order, pair_desc* __restrict__ desc,
@@ -498,7 +500,7 @@ __global__ void pair_scatter_kernel(const uint32_t* __restrict__ probes,
       d.label      = label;
       d.sample_off = off;
       d.n_rows     = chunk_indices[i] - off;
-      d.pad        = 0;
+      d.row_off    = uint32_t(inds_ptrs[label] - ids_base);
       desc[pos]    = d;
     }
   }
@@ -1145,7 +1147,8 @@ void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, ui
 }
 
 void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
-                        const uint8_t* const* data_ptrs, uint32_t n_pairs, uint32_t n_probes,
+                        const uint8_t* const* data_ptrs, const int64_t* const* inds_ptrs,
+                        const int64_t* ids_base, uint32_t n_pairs, uint32_t n_probes,
                         uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
                         pair_desc* desc, uint32_t lead_probes, uint8_t* alive, bool counted,
                         hipStream_t stream)
@@ -1163,8 +1166,33 @@ void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
   exclusive_scan_kernel<<<1, kScanThreads, 0, stream>>>(counts, n_bins, cursors);
   CUVS_LAUNCH_CHECK();
   pair_scatter_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(
-    probes, chunk_indices, data_ptrs, n_pairs, n_probes, lead_probes, n_lists, cursors, pair_order,
-    desc, alive);
+    probes, chunk_indices, data_ptrs, inds_ptrs, ids_base, n_pairs, n_probes, lead_probes, n_lists,
+    cursors, pair_order, desc, alive);
+  CUVS_LAUNCH_CHECK();
+}
+
+namespace {
+__global__ void build_lead_plane_kernel(const uint8_t* __restrict__ arena, uint2* __restrict__ plane,
+                                        uint64_t n_slots, uint64_t group_bytes)
+{
+  const uint64_t slot = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (slot < n_slots) {
+    // chunk 0 of a group of 32 rows comes first: row r of the group at byte 16 * r
+    const uint8_t* row = arena + (slot >> 5) * group_bytes + (slot & 31u) * kIndexGroupVecLen;
+    plane[slot]        = *reinterpret_cast<const uint2*>(row);
+  }
+}
+}  // namespace
+
+void launch_build_lead_plane(const uint8_t* arena, uint64_t* plane, uint64_t n_slots,
+                             uint32_t n_chunks, hipStream_t stream)
+{
+  if (n_slots == 0) { return; }
+  const uint64_t group_bytes = uint64_t(n_chunks) * kIndexGroupSize * kIndexGroupVecLen;
+  const uint64_t blocks      = (n_slots + 255) / 256;
+  CUVS_EXPECTS(blocks <= 0x7FFFFFFFull, "too many row slots for one launch");
+  build_lead_plane_kernel<<<uint32_t(blocks), 256, 0, stream>>>(arena, reinterpret_cast<uint2*>(plane),
+                                                                n_slots, group_bytes);
   CUVS_LAUNCH_CHECK();
 }
 

@@ -247,6 +247,282 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   }
 }
 
+/*
+ * Screening without tables, for per-subspace codebooks.
+ *
+ * A list of the benchmark index has a few hundred rows, and most tiles of 64 rows are decided by
+ * their first two to four codes: a 256-entry table per subspace would be built for about as many
+ * lookups as it has entries.  Here the block keeps the first 8 subspaces' codebooks in LDS once,
+ * and a lane computes the table entry its row's code selects on the spot: the same subtractions,
+ * FMAs and rounding to the table's type, so the partial sums are the ones the table kernels form.
+ * Nothing is shared between the waves of a block after the codebooks are loaded: each wave walks
+ * its own sequence of pairs, with the next pair's record, first codes, bound and query-minus-centre
+ * terms in flight while it scans the current one.
+ */
+constexpr uint32_t kDirectThreads = 512;
+constexpr uint32_t kDirectSubs    = 8;
+
+template <int PQ_LEN>
+struct book_vec;
+template <>
+struct book_vec<2> {
+  typedef float type __attribute__((ext_vector_type(2)));
+};
+template <>
+struct book_vec<4> {
+  typedef float type __attribute__((ext_vector_type(4)));
+};
+
+template <int PQ_LEN, int LUT, bool OUT_HALF, int FIRST>
+__global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
+  scan_args a, const pair_desc* __restrict__ desc, uint32_t n_pairs, uint32_t group_bytes,
+  pair_desc* __restrict__ survivors, uint32_t* __restrict__ n_survivors, uint8_t* __restrict__ alive)
+{
+  using traits = lut_traits<LUT>;
+  using lut_t  = typename traits::storage;
+  using acc_t  = typename std::conditional<OUT_HALF, _Float16, float>::type;
+  using vec_t  = typename book_vec<PQ_LEN>::type;
+  constexpr uint32_t SUB   = kDirectSubs;
+  constexpr uint32_t NDIFF = SUB * PQ_LEN;
+  static_assert(NDIFF <= 64, "one lane per leading rotated dimension");
+  auto* book      = reinterpret_cast<LDS_AS vec_t*>(uintptr_t(kScreenLdsBase));
+  const float one = opaque_one_s();
+
+  const uint32_t tid  = threadIdx.x;
+  const uint32_t lane = tid & 63u;
+  const uint32_t wid  = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr uint32_t WPB = kDirectThreads / 64u;
+  const uint32_t total   = gridDim.x * WPB;
+  if (blockIdx.x * WPB >= n_pairs) { return; }
+
+  for (uint32_t e = tid; e < SUB * 256u; e += kDirectThreads) {
+    vec_t v;
+#pragma unroll
+    for (int t = 0; t < PQ_LEN; t++) { v[t] = a.pq_centers[((e >> 8) * PQ_LEN + t) * 256u + (e & 255u)]; }
+    book[e] = v;
+  }
+  lds_barrier_s();
+
+  uint32_t p = blockIdx.x * WPB + wid;
+  if (p >= n_pairs) { return; }
+
+  // A record is fetched two pairs ahead with a vector load (index hidden from the uniformity
+  // analysis): a scalar load would be waited for by the tile loop's first LDS read, since both
+  // count on the same counter, while vector loads return in order behind loads issued earlier.
+  auto record = [&](uint32_t idx) -> pair_desc {
+    uint32_t at = idx < n_pairs ? idx : n_pairs - 1u;
+    asm volatile("" : "+v"(at));
+    return desc[at];
+  };
+  auto uniform = [](pair_desc d) -> pair_desc {
+    const uint64_t ptr = reinterpret_cast<uint64_t>(d.data);
+    // the builtin returns a signed int: widen through uint32_t, or the low half sign-extends
+    const uint32_t hi = uint32_t(__builtin_amdgcn_readfirstlane(uint32_t(ptr >> 32)));
+    const uint32_t lo = uint32_t(__builtin_amdgcn_readfirstlane(uint32_t(ptr)));
+    d.data       = reinterpret_cast<const uint8_t*>((uint64_t(hi) << 32) | uint64_t(lo));
+    d.q          = uint32_t(__builtin_amdgcn_readfirstlane(d.q));
+    d.slot       = uint32_t(__builtin_amdgcn_readfirstlane(d.slot));
+    d.label      = uint32_t(__builtin_amdgcn_readfirstlane(d.label));
+    d.sample_off = uint32_t(__builtin_amdgcn_readfirstlane(d.sample_off));
+    d.n_rows     = uint32_t(__builtin_amdgcn_readfirstlane(d.n_rows));
+    d.row_off    = uint32_t(__builtin_amdgcn_readfirstlane(d.row_off));
+    return d;
+  };
+  // Codes 0..7 of row (64 * tile + lane) of a list come from the packed plane of leading codes
+  // (kLeadPlaneSlack slots of slack follow the last list).
+  const auto* plane = reinterpret_cast<const GLOBAL_AS u32x2*>(reinterpret_cast<uintptr_t>(a.lead_plane));
+  auto lead_codes = [&](const pair_desc& d, uint32_t tile) {
+    return plane[uint64_t(d.row_off) + tile * 64u + lane];
+  };
+  // lane d < NDIFF: (rotated query - rotated centre)[d] of a pair
+  auto fetch_diff = [&](const pair_desc& d) -> float {
+    const uint32_t dim = lane < NDIFF ? lane : 0u;
+    return a.rot_q[uint64_t(d.q) * a.rot_dim + dim] - a.centers_rot[uint64_t(d.label) * a.rot_dim + dim];
+  };
+
+  pair_desc d0 = uniform(record(p));
+  pair_desc d1 = uniform(record(p + total));
+  // leading codes of a pair's tiles 0 and 1 (the plane's slack covers tiles past a list's end)
+  u32x2 lead0 = lead_codes(d0, 0u);
+  u32x2 next0 = lead_codes(d0, 1u);
+  uint32_t thr0  = a.query_kth[d0.q];
+  float dv0     = fetch_diff(d0);
+
+  for (;;) {
+    const bool has1    = p + total < n_pairs;
+    const pair_desc d2 = record(p + 2u * total);
+    u32x2 lead1        = lead0;
+    u32x2 next1        = next0;
+    uint32_t thr1      = 0u;
+    float dv1          = 0.0f;
+    if (has1) {
+      lead1 = lead_codes(d1, 0u);
+      next1 = lead_codes(d1, 1u);
+      thr1  = a.query_kth[d1.q];
+      dv1  = fetch_diff(d1);
+    }
+
+    {
+      // terms of the first four subspaces, broadcast to scalar registers once per pair; those of
+      // subspaces 4..7 are read where the few tiles that get that far need them
+      constexpr uint32_t NEAGER = 4 * PQ_LEN;
+      float diff[NEAGER];
+#pragma unroll
+      for (uint32_t t = 0; t < NEAGER; t++) {
+        diff[t] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(dv0), int(t)));
+      }
+      const uint32_t thr       = uint32_t(__builtin_amdgcn_readfirstlane(thr0));
+      const uint32_t n_rows    = d0.n_rows;
+      const uint32_t n_tiles   = (n_rows + 63u) >> 6;
+      const uint32_t stop_bits = thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u;
+      bool in_play             = false;
+      const uint32_t full_tiles         = n_rows >> 6;
+      const unsigned long long tail_rows = (1ull << (n_rows & 63u)) - 1ull;
+      // sums the leading codes `cur` of the rows of tile `tile`
+      auto sum_tile = [&](const u32x2& cur, uint32_t tile) __attribute__((always_inline)) {
+        // lanes past the list's end count only in its last, partial tile
+        const unsigned long long rows = tile < full_tiles ? ~0ull : tail_rows;
+        const uint32_t w[2]           = {cur.x, cur.y};
+        acc_t acc        = acc_t(0);
+        auto add_codes = [&](int first, int last) __attribute__((always_inline)) {
+#pragma unroll
+          for (int kk = first; kk < last; kk++) {
+            const uint32_t c = (w[kk >> 2] >> ((kk & 3) * 8)) & 0xffu;
+            const vec_t b    = book[kk * 256 + c];
+            float score      = 0.0f;
+#pragma unroll
+            for (int t = 0; t < PQ_LEN; t++) {
+              float df;
+              if (kk < 4) {
+                df = diff[(kk & 3) * PQ_LEN + t];
+              } else {
+                int held = __float_as_int(dv0);
+                asm volatile("" : "+v"(held));  // keeps the broadcast inside the rare branch
+                df = __int_as_float(__builtin_amdgcn_readlane(held, kk * PQ_LEN + t));
+              }
+              df -= b[t];
+              score = fmaf(df, df, score);
+            }
+            const lut_t v = traits::encode(score);
+            if (OUT_HALF) {
+              acc = acc_t(acc + traits::to_half(v));
+            } else if (LUT == LUT_F16) {
+              acc = acc_t(fmaf(traits::to_float(v), one, float(acc)));
+            } else {
+              acc = acc_t(acc + traits::to_float(v));
+            }
+          }
+        };
+        auto any_in_play = [&]() __attribute__((always_inline)) {
+          return (__builtin_amdgcn_ballot_w64(!(__float_as_uint(float(acc)) > stop_bits)) & rows) != 0ull;
+        };
+        add_codes(0, FIRST);
+        in_play = any_in_play();
+        if (FIRST < 4 && in_play) {
+          add_codes(FIRST, 4);
+          in_play = any_in_play();
+        }
+        if (in_play) {
+          add_codes(4, int(SUB));
+          in_play = any_in_play();
+        }
+      };
+      // Three registers take turns: while tile t is summed, the codes of tiles t + 1 and t + 2
+      // are in flight; a register is reloaded right after the step that consumed it, and the loop
+      // is unrolled by three so that none is copied while its load is outstanding.  Loads are
+      // unconditional (they may run up to three tiles past the list, into the plane's slack or the
+      // next lists), so the waits in the loop count outstanding loads instead of draining them.
+      u32x2 r0 = lead0, r1 = next0, r2;
+      for (uint32_t tile = 0; tile < n_tiles; tile += 3u) {
+        r2 = lead_codes(d0, tile + 2u);
+        sum_tile(r0, tile);
+        if (in_play || tile + 1u >= n_tiles) { break; }
+        r0 = lead_codes(d0, tile + 3u);
+        sum_tile(r1, tile + 1u);
+        if (in_play || tile + 2u >= n_tiles) { break; }
+        r1 = lead_codes(d0, tile + 4u);
+        sum_tile(r2, tile + 2u);
+        if (in_play) { break; }
+      }
+      if (in_play && lane == 0) {
+        const uint32_t pos = atomicAdd(n_survivors, 1u);
+        survivors[pos]     = d0;
+        alive[d0.slot]     = 1;
+      }
+    }
+
+    if (!has1) { break; }
+    p += total;
+    d0    = d1;
+    d1    = uniform(d2);
+    lead0 = lead1;
+    next0 = next1;
+    thr0  = thr1;
+    dv0   = dv1;
+  }
+}
+
+/** Which subspace count the first check of the table-free screen follows (1, 2 or 4). */
+inline int screen_first_check()
+{
+  static const int first = [] {
+    const char* e = std::getenv("CUVS_AMD_SCREEN_FIRST_CHECK");
+    const int v   = e != nullptr ? std::atoi(e) : 2;
+    return (v == 1 || v == 2 || v == 4) ? v : 2;
+  }();
+  return first;
+}
+
+inline bool screen_tables_forced()
+{
+  static const bool forced = [] {
+    const char* e = std::getenv("CUVS_AMD_SCREEN_TABLES");
+    return e != nullptr && e[0] == '1';
+  }();
+  return forced;
+}
+
+template <int PQ_LEN, int LUT, bool OUT_HALF, int FIRST>
+void launch_screen_direct_first(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
+                                pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
+                                hipStream_t stream)
+{
+  auto kernel       = scan_screen_direct_kernel<PQ_LEN, LUT, OUT_HALF, FIRST>;
+  const size_t smem = kScreenLdsBase + size_t(kDirectSubs) * 256 * PQ_LEN * 4;
+  static int n_cu = 0, per_cu = 0;  // per instance
+  if (n_cu == 0) {
+    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+    int dev = 0;
+    CUVS_HIP_TRY(hipGetDevice(&dev));
+    CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+    CUVS_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kDirectThreads, smem));
+    per_cu = std::max(per_cu, 1);
+  }
+  constexpr uint32_t wpb = kDirectThreads / 64u;
+  uint32_t grid          = uint32_t(n_cu) * uint32_t(per_cu);
+  const uint32_t needed  = (n_pairs + wpb - 1u) / wpb;
+  if (grid > needed) { grid = needed; }
+  const uint32_t n_chunks    = (a.pq_dim + 15u) / 16u;
+  const uint32_t group_bytes = n_chunks * 512u;
+  kernel<<<grid, kDirectThreads, smem, stream>>>(a, desc, n_pairs, group_bytes, survivors, n_survivors, alive);
+  CUVS_HIP_TRY(hipGetLastError());
+}
+
+template <int PQ_LEN, int LUT, bool OUT_HALF>
+void launch_screen_direct(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
+                          pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive, hipStream_t stream)
+{
+  const int first = screen_first_check();
+  if (first == 1) {
+    launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, 1>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+  } else if (first == 2) {
+    launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, 2>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+  } else {
+    launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, 4>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+  }
+}
+
 template <int SUBS, int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER>
 void launch_screen_sub(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
                             pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
@@ -282,6 +558,12 @@ void launch_screen_instance(const scan_args& a, const pair_desc* desc, uint32_t 
                             pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
                             hipStream_t stream)
 {
+  if constexpr (!PER_CLUSTER) {
+    if (!screen_tables_forced() && a.lead_plane != nullptr) {
+      launch_screen_direct<PQ_LEN, LUT, OUT_HALF>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+      return;
+    }
+  }
   const int subs = screen_subspaces();
   if (subs == 4) {
     launch_screen_sub<4, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
@@ -315,7 +597,11 @@ void launch_screen_types(const scan_args& a, const pair_desc* desc, uint32_t n_p
 
 }  // namespace
 
-uint32_t scan_screen_bytes_per_row() { return screen_subspaces() <= 8 ? 8u : 16u; }
+uint32_t scan_screen_bytes_per_row(bool per_cluster, bool lead_plane)
+{
+  if (!per_cluster && lead_plane && !screen_tables_forced()) { return 8u; }
+  return screen_subspaces() <= 8 ? 8u : 16u;
+}
 
 bool scan_screen_supported(const scan_args& a)
 {

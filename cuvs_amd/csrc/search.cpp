@@ -319,6 +319,7 @@ void search(cuvs::resources const& res_c,
   sa.centers_rot  = ix.centers_rot.as<float>();
   sa.pq_centers   = ix.pq_centers.as<float>();
   sa.data_ptrs    = ix.data_ptrs.as<const uint8_t*>();
+  sa.lead_plane   = ix.lead_plane.bytes != 0 ? ix.lead_plane.as<uint64_t>() : nullptr;
   sa.inds_ptrs    = ix.inds_ptrs.as<const int64_t*>();
   sa.list_sizes   = ix.list_sizes.as<uint32_t>();
   sa.filter_bits  = filter_bits;
@@ -414,7 +415,8 @@ void search(cuvs::resources const& res_c,
     detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
                                  ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead,
                                  counters, ix.n_lists, s);
-    detail::launch_order_pairs(probes, chunk, ix.data_ptrs.as<const uint8_t*>(), nq * P, P,
+    detail::launch_order_pairs(probes, chunk, ix.data_ptrs.as<const uint8_t*>(),
+                               ix.inds_ptrs.as<const int64_t*>(), ix.ids_arena.as<int64_t>(), nq * P, P,
                                ix.n_lists, counters, order, desc, lead, alive, true, s);
     if (pl.fused) { detail::launch_fill_u32(kth, 0xFFFFFFFFu, nq, s); }
     mark(2);
@@ -524,7 +526,7 @@ void search(cuvs::resources const& res_c,
       res.last_profile.lead_bytes   = h[2];
       // rows x leading bytes the screen reads
       res.last_profile.screen_bytes =
-        (h[0] - h[2]) / (uint64_t(ix.n_chunks) * kIndexGroupVecLen) * detail::scan_screen_bytes_per_row();
+        (h[0] - h[2]) / (uint64_t(ix.n_chunks) * kIndexGroupVecLen) * detail::scan_screen_bytes_per_row(ix.codebook_kind == codebook_gen::PER_CLUSTER, ix.lead_plane.bytes != 0);
     }
   }
   res.reset_workspace();

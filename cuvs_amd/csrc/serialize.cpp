@@ -319,6 +319,7 @@ void deserialize(cuvs::resources const& res, const std::string& filename, index<
   ix.h_list_sizes  = sizes;
   ix.h_row_offsets = offsets;
   ix.recompute_internal_state(s);
+  ix.rebuild_lead_plane(s);
   *idx = std::move(loaded);
 }
 
