@@ -24,7 +24,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes per launch of the named kernel on the default workload, from hardware counters (FETCH_SIZE + WRITE_SIZE
 # per dispatch, each scaled by its reading for the 1 GiB calibration copy below); the counter runs
 # are summarised under profiles/.  Keyed by (kernel, lut, internal); None where not measured.
-MEASURED_TRAFFIC = {("scan_screen_kernel", "f16", "f32"): 1.358e9}
+MEASURED_TRAFFIC = {("scan_screen_direct_kernel", "f16", "f32"): 1.439e9}
 
 
 def log(msg):
@@ -147,9 +147,9 @@ def main():
     early_stop = stage["n_screened_pairs"] > 0
     if early_stop:
         # the scan stage is three launches; the screening kernel is the dominant one.  Its
-        # algorithmic bytes are the leading 4 bytes (4 one-byte codes, from the packed plane of
+        # algorithmic bytes are the leading 8 bytes (8 one-byte codes, from the packed plane of
         # leading codes) of every (padded) row of every screened pair; per-cluster codebooks use the
-        # table-building screen, which reads the leading 8 bytes from the interleaved lists.
+        # table-building screen, which reads the same 8 bytes from the interleaved lists.
         parts = {"lead_scan": (mean("lead_scan_ms"), stage["lead_bytes"] / launches),
                  "screen": (mean("screen_ms"), stage["screen_bytes"] / launches),
                  "survivor_scan": (mean("survivor_scan_ms"), stage["survivor_bytes"] / launches)}
