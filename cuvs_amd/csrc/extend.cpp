@@ -80,8 +80,11 @@ struct row_stager {
 void predict_labels(const cuvs::resources& res, const index_impl& ix, const float* xf, uint64_t n,
                     float* scores, uint32_t* labels)
 {
-  const bool ip = ix.metric == detail::DistanceType::InnerProduct ||
-                  ix.metric == detail::DistanceType::CosineExpanded;
+  // Rows join the list the coarse clustering would give them: nearest centre by L2 also for an
+  // inner-product index, by inner product of the normalised row for cosine
+  // (coarse_clustering_metric, cpp/src/neighbors/ivf_pq/ivf_pq_build.cuh:70-76, used by extend
+  // :1141 and transform, ivf_pq_transform.cuh:58).
+  const bool ip = ix.metric == detail::DistanceType::CosineExpanded;
   detail::launch_coarse_scores(xf, ix.centers.as<float>(), uint32_t(n), ix.n_lists, ix.dim,
                                ix.dim_ext, ip, false, scores, res.stream());
   detail::launch_select_probes(scores, uint32_t(n), ix.n_lists, 1, labels, res.stream());

@@ -803,6 +803,8 @@ int orc_encode(const orc_index* index, const void* rows, int row_type, uint64_t 
   const uint32_t B      = 1u << ix.pq_bits;
   const uint32_t de     = dim_ext_of(ix.dim);
   orc_search_params sp{1, ORC_R_32F, ORC_R_32F, ORC_R_32F};
+  orc_index ix_labels = ix;
+  if (ix.metric == ORC_InnerProduct) { ix_labels.metric = ORC_L2Expanded; }
   struct scratch {
     std::vector<float> xf, diff, res, scores;
     std::vector<cand> tmp;
@@ -822,8 +824,10 @@ int orc_encode(const orc_index* index, const void* rows, int row_type, uint64_t 
         for (uint32_t d = 0; d < ix.dim; d++) { w.xf[d] = w.xf[d] / nrm; }
       }
     }
+    // the list is chosen with the coarse clustering's metric: L2 also for an inner-product index
+    // (coarse_clustering_metric, ivf_pq_build.cuh:70-76, :1141; ivf_pq_transform.cuh:58)
     uint32_t label;
-    select_clusters_one(ix, sp, w.xf.data(), 1, w.scores, w.tmp, &label, nullptr);
+    select_clusters_one(ix_labels, sp, w.xf.data(), 1, w.scores, w.tmp, &label, nullptr);
     labels[r] = label;
     // residual = rotation_matrix * (x - centre[label])   (ivf_pq_build.cuh:140-206)
     const float* c = ix.centers + uint64_t(label) * de;

@@ -359,6 +359,28 @@ def test_early_stop_matches_oracle_and_full_scan(orc, monkeypatch, lut, internal
         assert torch.equal(nb, nb2) and torch.equal(d, d2)
 
 
+def test_early_stop_pq_len_4(orc):
+    """Four dimensions per subspace: 16-byte codebook entries in the table-free screen."""
+    from cuvs_amd import testing
+    from cuvs_amd.resources import Resources
+    allrows = testing.gaussian_mixture(20100, 128, 64, 0.15, seed=78).numpy()
+    x, q = allrows[:20000], allrows[20000:]
+    model = H.train(x, 128, 32, 8, iters=6)
+    index = G.build_gpu_index(model, x, 32, 8, "sqeuclidean", "subspace")
+    ix, _ = G.read_back(orc, index, model, 128, 32, 8, "sqeuclidean", "subspace")
+    res = Resources()
+    res.enable_profiling(True)
+    for lut in (R_16F, R_8U):
+        sp = ivf_pq.SearchParams(n_probes=40, lut_dtype=lut)
+        d, nb = ivf_pq.search(sp, index, G.to_dev(q), 10, resources=res)
+        res.sync()
+        prof = ivf_pq.get_search_profile(res)
+        assert prof["n_screened_pairs"] == q.shape[0] * 39
+        assert 0 < prof["n_surviving_pairs"] < prof["n_screened_pairs"] // 2
+        want_nb, want_d = orc.search(ix, q, 10, 40, lut_dtype=ORC_DT[lut])
+        H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
+
+
 def test_early_stop_with_filter_and_small_lists(orc):
     """A filter can leave the leading list with fewer than k rows (no bound: nothing is dropped),
     and the screen ignores the filter (it may keep a pair whose rows in play are all filtered)."""

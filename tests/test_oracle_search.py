@@ -312,3 +312,29 @@ def test_committed_toy_index(orc):
     book = g["pq_centers"].astype(np.float64)                      # [pq_dim, pq_len, B]
     dist = ((res[:, :, :, None] - book[None]) ** 2).sum(2)          # [n, pq_dim, B]
     assert np.array_equal(codes, dist.argmin(2))
+
+
+@pytest.mark.parametrize("metric", ["sqeuclidean", "inner_product", "cosine"])
+def test_encode_labels_follow_the_coarse_clustering_metric(orc, metric):
+    """Rows join the nearest centre by L2 for L2 and inner-product indexes, and the centre of
+    largest inner product with the normalised row for cosine (coarse_clustering_metric,
+    cpp/src/neighbors/ivf_pq/ivf_pq_build.cuh:70-76, :1141)."""
+    rng = np.random.default_rng(11)
+    dim, n_lists = 16, 24
+    data = rng.standard_normal((600, dim)).astype(np.float32)
+    # centres of very different norms, so that L2 and inner product disagree on most rows
+    centers = (rng.standard_normal((n_lists, dim)) * rng.uniform(0.2, 3.0, (n_lists, 1))).astype(np.float32)
+    model = H.train(data, n_lists, 8, 8, metric=metric, iters=2)
+    ext = model["centers"].copy()
+    ext[:, :dim] = centers
+    ext[:, dim] = (centers.astype(np.float64) ** 2).sum(1).astype(np.float32)
+    model["centers"] = ext
+    model["centers_rot"] = (centers @ model["rotation_matrix"].T).astype(np.float32)
+    ix = H.oracle_index(orc, model, dim, 8, 8, metric=metric)
+    labels, _ = orc.encode(ix, data)
+    x, c = data.astype(np.float64), centers.astype(np.float64)
+    by_l2 = ((x[:, None] - c[None]) ** 2).sum(-1).argmin(1)
+    by_ip = ((x / np.linalg.norm(x, axis=1, keepdims=True)) @ c.T).argmax(1)
+    want = by_ip if metric == "cosine" else by_l2
+    assert (by_l2 != by_ip).mean() > 0.3
+    assert np.array_equal(labels, want)
