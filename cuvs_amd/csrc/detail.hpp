@@ -246,6 +246,30 @@ size_t scan_lds_bytes(const scan_args& a);
 size_t scan_lut_bytes(const scan_args& a);
 uint32_t scan_global_lut_blocks();
 void launch_scan(const scan_args& a, hipStream_t stream);
+/* training (train.hip) */
+/** dst row i = src row i * ratio + hash(i, seed) % ratio, rows of `row_bytes` bytes. */
+void launch_gather_rows(const void* src, uint64_t row_bytes, uint64_t n_out, uint64_t ratio,
+                        uint32_t seed, void* dst, hipStream_t stream);
+/** ext [n_lists, dim_ext] = (centre, squared norm, zeros) from flat [n_lists, dim]. */
+void launch_set_centers(const float* flat, uint32_t n_lists, uint32_t dim, uint32_t dim_ext, float* ext,
+                        hipStream_t stream);
+void launch_accumulate(const float* x, const uint32_t* labels, uint64_t n_rows, uint32_t dim,
+                       float* sums, uint32_t* counts, uint32_t* member, hipStream_t stream);
+void launch_finish_centers(const float* sums, const uint32_t* counts, uint32_t n_lists, uint32_t dim,
+                           bool normalize, float* flat, hipStream_t stream);
+void launch_adjust_centers(const uint32_t* receivers, const uint32_t* donors, uint32_t n_pairs,
+                           const float* x, const uint32_t* member, uint32_t dim, float offset,
+                           float* flat, hipStream_t stream);
+void launch_residuals(const float* x, const uint32_t* labels, const float* centers_ext, uint64_t n_rows,
+                      uint32_t dim, uint32_t dim_ext, float* diff, hipStream_t stream);
+uint32_t train_codebook_max_pq_len();
+/** One balanced k-means per group (subspace or list) of `book` entries; output layout
+ *  [group][pq_len][book]. */
+void launch_train_codebooks(const float* res, uint32_t rot_dim, uint32_t pq_dim, uint32_t pq_len,
+                            uint32_t book, bool per_cluster, uint32_t n_groups, uint32_t n_rows,
+                            const uint32_t* rows, const uint32_t* offsets, uint32_t max_samples,
+                            uint32_t n_iters, uint32_t seed, float* pq_centers, hipStream_t stream);
+
 /** plane[slot] = first eight bytes of row slot `slot` of an arena of 8-bit codes. */
 void launch_build_lead_plane(const uint8_t* arena, uint64_t* plane, uint64_t n_slots,
                              uint32_t n_chunks, hipStream_t stream);

@@ -379,12 +379,27 @@ cuvsError_t cuvsIvfPqIndexGetListIndices(cuvsIvfPqIndex_t index, uint32_t label,
   });
 }
 
-cuvsError_t cuvsIvfPqBuild(cuvsResources_t, cuvsIvfPqIndexParams_t, DLManagedTensor*, cuvsIvfPqIndex_t)
+cuvsError_t cuvsIvfPqBuild(cuvsResources_t res,
+                           cuvsIvfPqIndexParams_t params,
+                           DLManagedTensor* dataset_tensor,
+                           cuvsIvfPqIndex_t index)
 {
   return translate_exceptions([=] {
-    cuvs::fail(
-      "cuvsIvfPqBuild: training (k-means and codebook fitting) is not part of this library; "
-      "pass a trained model to cuvsIvfPqBuildPrecomputed and add data with cuvsIvfPqExtend");
+    CUVS_EXPECTS(params != nullptr && index != nullptr, "params and index must not be null");
+    CUVS_EXPECTS(dataset_tensor != nullptr, "dataset must not be null");
+    // c/src/neighbors/ivf_pq.cpp:377-403: device or host dataset of float32, float16, int8 or uint8
+    auto& ds = dataset_tensor->dl_tensor;
+    elem_type t;
+    CUVS_EXPECTS(elem_type_of(ds.dtype, &t), "Unsupported dataset DLtensor dtype: %d and bits: %d",
+                 int(ds.dtype.code), int(ds.dtype.bits));
+    expect_tensor(dataset_tensor, "dataset", 2, ds.dtype.code, ds.dtype.bits);
+    auto ip   = convert_index_params(*params);
+    auto* idx = new ivfpq::index<int64_t>(
+      ivfpq::build(*res_of(res), ip, tensor_data(dataset_tensor), t, ds.shape[0], uint32_t(ds.shape[1])));
+    if (index->addr != 0) { delete reinterpret_cast<ivfpq::index<int64_t>*>(index->addr); }
+    index->addr       = reinterpret_cast<uintptr_t>(idx);
+    index->dtype.code = ds.dtype.code;
+    index->dtype.bits = ds.dtype.bits;
   });
 }
 

@@ -286,11 +286,14 @@ def _prep(res):
 
 
 def build(index_params, dataset, resources=None):
-    """ivf_pq.pyx:477 -- training is outside this library; raises with the C layer's message."""
-    res, _ = _prep(resources)
+    """ivf_pq.pyx:477 -- train an index on `dataset` and (add_data_on_build) add the rows."""
+    res, own = _prep(resources)
     index = Index()
     check(lib().cuvsIvfPqBuild(res.get_c_obj(), index_params._p, dlpack.view(dataset).ptr,
                                index.index))
+    if own:
+        res.sync()
+    index.trained = True
     return index
 
 

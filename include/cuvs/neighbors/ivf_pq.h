@@ -142,8 +142,8 @@ CUVS_EXPORT cuvsError_t cuvsIvfPqBuildPrecomputed(cuvsResources_t res,
                                                   DLManagedTensor* rotation_matrix,
                                                   cuvsIvfPqIndex_t index);
 
-/** ivf_pq.h:426-429 -- training is not part of this library: always fails with a message that
- *  points to cuvsIvfPqBuildPrecomputed. */
+/** ivf_pq.h:426-429 -- trains an index on `dataset` ([n_rows, dim] of float32, float16, int8 or
+ *  uint8, in device or host memory) and, with params->add_data_on_build, adds the dataset to it. */
 CUVS_EXPORT cuvsError_t cuvsIvfPqBuild(cuvsResources_t res,
                                        cuvsIvfPqIndexParams_t params,
                                        DLManagedTensor* dataset,

@@ -143,6 +143,22 @@ index<int64_t> build(cuvs::resources const& res,
                      const float* centers_rot,
                      const float* rotation_matrix);
 
+/** Train an index on a dataset and (params.add_data_on_build) add the dataset to it
+ *  (cuVS: ivf_pq::build(res, params, dataset), cpp/include/cuvs/neighbors/ivf_pq.hpp;
+ *  cpp/src/neighbors/ivf_pq/ivf_pq_build.cuh:1240-1410).  `dataset` is [n_rows, dim] row-major in
+ *  device or host memory. */
+index<int64_t> build(cuvs::resources const& res,
+                     const index_params& params,
+                     const void* dataset,
+                     elem_type type,
+                     int64_t n_rows,
+                     uint32_t dim);
+
+template <typename T>
+index<int64_t> build(cuvs::resources const& res,
+                     const index_params& params,
+                     device_matrix_view<const T> dataset);
+
 /** Encode and append rows.  `new_vectors` and `new_indices` are device pointers; a null
  *  `new_indices` numbers the rows consecutively from the current size.  A non-null `labels`
  *  (device uint32 [n]) overrides the nearest-centre assignment. */
