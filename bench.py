@@ -46,6 +46,8 @@ def main():
     ap.add_argument("--k", type=int, default=10)
     ap.add_argument("--lut", default="f16", choices=["f32", "f16", "fp8"])
     ap.add_argument("--internal", default="f32", choices=["f32", "f16"])
+    ap.add_argument("--build", choices=("native", "torch"), default="native",
+                    help="train the index with the library (cuvsIvfPqBuild) or with the torch helper")
     ap.add_argument("--refine-ratio", type=int, default=1,
                     help="search refine_ratio * k candidates and re-rank them exactly (1 = off)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
@@ -72,30 +74,40 @@ def main():
     data, queries = allrows[:n], allrows[n:].contiguous()
     log(f"data {tuple(data.shape)} uint8 generated in {time.time() - t0:.1f}s")
 
-    t0 = time.time()
-    g = torch.Generator(device="cpu")
-    g.manual_seed(137)
-    n_train = min(n, max(n_lists * 32, 200_000))
-    sel = torch.randperm(n, generator=g)[:n_train].to(dev)
-    model = testing.train_model(data[sel], n_lists, pq_dim, pq_bits, kmeans_iters=6, pq_iters=8,
-                                seed=137, half_assign=True)
-    torch.cuda.synchronize()
-    log(f"model trained on {n_train} rows in {time.time() - t0:.1f}s")
-
-    t0 = time.time()
-    labels = testing.assign_nearest(data, model["centers"][:, :dim], half=True).to(torch.int32)
-    torch.cuda.synchronize()
-    log(f"lists assigned in {time.time() - t0:.1f}s")
-
-    t0 = time.time()
     res = Resources()
     res.use_torch_current_stream()
-    params = ivf_pq.IndexParams(n_lists=n_lists, pq_bits=pq_bits, pq_dim=pq_dim)
-    index = ivf_pq.build_precomputed(params, dim, model["pq_centers"], model["centers"],
-                                     model["centers_rot"], model["rotation_matrix"], resources=res)
-    ivf_pq.extend(index, data, None, resources=res, labels=labels)
-    res.sync()
-    log(f"index populated ({len(index)} rows) in {time.time() - t0:.1f}s")
+    n_train = min(n, max(n_lists * 32, 200_000))
+    if args.build == "native":
+        # the library's own training (cuvsIvfPqBuild) on a subsample of n_train rows, then every row
+        # encoded and added (add_data_on_build)
+        t0 = time.time()
+        params = ivf_pq.IndexParams(n_lists=n_lists, pq_bits=pq_bits, pq_dim=pq_dim,
+                                    kmeans_trainset_fraction=min(1.0, n_train / n))
+        index = ivf_pq.build(params, data, resources=res)
+        res.sync()
+        log(f"index trained on ~{n_train} rows and populated ({len(index)} rows) in {time.time() - t0:.1f}s")
+    else:
+        t0 = time.time()
+        g = torch.Generator(device="cpu")
+        g.manual_seed(137)
+        sel = torch.randperm(n, generator=g)[:n_train].to(dev)
+        model = testing.train_model(data[sel], n_lists, pq_dim, pq_bits, kmeans_iters=6, pq_iters=8,
+                                    seed=137, half_assign=True)
+        torch.cuda.synchronize()
+        log(f"model trained on {n_train} rows in {time.time() - t0:.1f}s")
+
+        t0 = time.time()
+        labels = testing.assign_nearest(data, model["centers"][:, :dim], half=True).to(torch.int32)
+        torch.cuda.synchronize()
+        log(f"lists assigned in {time.time() - t0:.1f}s")
+
+        t0 = time.time()
+        params = ivf_pq.IndexParams(n_lists=n_lists, pq_bits=pq_bits, pq_dim=pq_dim)
+        index = ivf_pq.build_precomputed(params, dim, model["pq_centers"], model["centers"],
+                                         model["centers_rot"], model["rotation_matrix"], resources=res)
+        ivf_pq.extend(index, data, None, resources=res, labels=labels)
+        res.sync()
+        log(f"index populated ({len(index)} rows) in {time.time() - t0:.1f}s")
 
     t0 = time.time()
     truth = testing.exact_knn(data, queries, k).cpu().numpy()  # fp32: exact for 8-bit data
