@@ -5,6 +5,7 @@ cuVS C ABI); it mirrors ``cuvs.neighbors.ivf_pq`` of the reference Python packag
 """
 from . import ivf_pq  # noqa: F401
 from .refine import refine  # noqa: F401
+from .knn_merge_parts import knn_merge_parts  # noqa: F401
 from .resources import Resources  # noqa: F401
 
-__all__ = ["ivf_pq", "refine", "Resources"]
+__all__ = ["ivf_pq", "refine", "knn_merge_parts", "Resources"]

@@ -91,6 +91,7 @@ EXPORTED_SYMBOLS = [
     "cuvsIvfPqTransform", "cuvsAmdIvfPqSelectClusters", "cuvsAmdIvfPqSearchWithBitset",
     "cuvsAmdIvfPqExtendLabeled", "cuvsAmdIvfPqProfilingEnable", "cuvsAmdIvfPqGetSearchProfile",
     "cuvsRefine",
+    "cuvsAmdKnnMergeParts",
 ]
 
 _lib = None
@@ -150,6 +151,7 @@ def lib():
           P(IndexStruct))
     proto("cuvsIvfPqSearch", res_t, P(SearchParamsStruct), P(IndexStruct), T, T, T)
     proto("cuvsRefine", res_t, T, T, T, C.c_int, T, T)
+    proto("cuvsAmdKnnMergeParts", res_t, T, T, T, T, T)
     proto("cuvsIvfPqSerialize", res_t, C.c_char_p, P(IndexStruct))
     proto("cuvsIvfPqDeserialize", res_t, C.c_char_p, P(IndexStruct))
     proto("cuvsIvfPqExtend", res_t, T, T, P(IndexStruct))

@@ -9,7 +9,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def declared_symbols():
     names = set()
     for rel in ("include/cuvs/core/c_api.h", "include/cuvs/neighbors/ivf_pq.h",
-                "include/cuvs/neighbors/refine.h"):
+                "include/cuvs/neighbors/refine.h",
+                "include/cuvs/neighbors/knn_merge_parts.h"):
         with open(os.path.join(ROOT, rel)) as f:
             text = f.read()
         names |= set(re.findall(r"CUVS_EXPORT\s+[\w\s\*]+?\b(cuvs\w+)\s*\(", text))
