@@ -1,0 +1,493 @@
+/*
+ * Probe selection in two precisions, with the results of the fp32 path.
+ *
+ * select_clusters (cpp/src/neighbors/ivf_pq/ivf_pq_search.cuh:60-168) scores every centre for every
+ * query in fp32 and keeps the n_probes best.  The fp32 contraction is most of that cost, and all of
+ * it is spent on centres that are nowhere near the best.  Here the contraction runs on the fp16
+ * matrix cores first (centres rounded to binary16, products exact, fp32 accumulation), with a
+ * rigorous bound E_q on how far such a score can be from the fp32 one; every centre whose fp16
+ * score is within 2 E_q of (an upper bound of) the n_probes-th smallest fp16 score is kept as a
+ * candidate, which provably includes the fp32 path's n_probes best; the candidates - a few more
+ * than n_probes - are then scored by the fp32 path's own arithmetic (one FMA chain over ascending
+ * dimensions) and ordered by (score, list).  The probes are bit for bit those of the fp32 path.
+ *
+ *   pass 1  fp16 scores; per query the minimum of every group of 16 lists      (no score matrix)
+ *   bound   T_q = n_probes-th smallest of those minima (at least n_probes scores are <= T_q),
+ *           thr_q = T_q + 2 E_q
+ *   pass 2  the same fp16 scores again; lists with score <= thr_q are appended to the query's
+ *           candidate list
+ *   rescore exact fp32 score of every candidate, rank, write the probes; a query with more
+ *           candidates than fit (or fewer than n_probes: non-finite input) is flagged and goes
+ *           through the plain fp32 path afterwards
+ *
+ * Why the candidates suffice: let s be fp32-path scores, s' the fp16 ones, |s - s'| <= E.  If t is
+ * the n_probes-th smallest s, at most n_probes - 1 lists have s' < t - E, so the n_probes-th
+ * smallest s' is >= t - E, and every list with s <= t has s' <= t + E <= (n_probes-th smallest s')
+ * + 2E <= T + 2E.
+ */
+#include "device_utils.cuh"
+
+#include <algorithm>
+
+namespace cuvs::neighbors::ivf_pq::detail {
+
+namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t kTile    = 128;  // lists x queries per block
+constexpr uint32_t kSlab    = 64;   // the padded dimension is a multiple of this
+constexpr uint32_t kCandCapF = 256;  // candidates per query
+
+template <typename T>
+__device__ __forceinline__ float map_elem(T v);
+template <>
+__device__ __forceinline__ float map_elem<_Float16>(_Float16 v) { return float(v); }
+template <>
+__device__ __forceinline__ float map_elem<int8_t>(int8_t v) { return float(v) * (1.0f / 128.0f); }
+template <>
+__device__ __forceinline__ float map_elem<uint8_t>(uint8_t v) { return float(v) * (1.0f / 256.0f); }
+
+/** qh[q][d] = mapped query as binary16 (exact for these element types), zero padded to k_pad
+ *  columns and q_pad rows; qnorm[q] = an upper bound of the query's Euclidean norm. */
+template <typename T>
+__global__ void pack_queries_kernel(const T* __restrict__ in, uint32_t n_queries, uint32_t dim,
+                                    uint32_t k_pad, _Float16* __restrict__ qh, float* __restrict__ qnorm)
+{
+  const uint32_t q    = blockIdx.x;
+  const uint32_t lane = threadIdx.x;
+  float ss            = 0.0f;
+  for (uint32_t d = lane; d < k_pad; d += 64) {
+    float v = 0.0f;
+    if (q < n_queries && d < dim) { v = map_elem<T>(in[uint64_t(q) * dim + d]); }
+    qh[uint64_t(q) * k_pad + d] = _Float16(v);
+    ss                          = fmaf(v, v, ss);
+  }
+  for (int o = 32; o > 0; o >>= 1) { ss += __shfl_xor(ss, o); }
+  if (lane == 0) { qnorm[q] = sqrtf(ss) * 1.0001f; }
+}
+
+/** ch[l][d] = centre as binary16, zero padded; cn[l] = the stored squared norm (column dim). */
+__global__ void pack_centers_kernel(const float* __restrict__ centers, uint32_t n_lists, uint32_t dim,
+                                    uint32_t dim_ext, uint32_t k_pad, _Float16* __restrict__ ch,
+                                    float* __restrict__ cn, uint32_t* __restrict__ stats)
+{
+  const uint32_t l    = blockIdx.x;
+  const uint32_t lane = threadIdx.x;
+  float amax          = 0.0f;
+  float ss            = 0.0f;
+  for (uint32_t d = lane; d < k_pad; d += 64) {
+    float v = 0.0f;
+    if (l < n_lists && d < dim) { v = centers[uint64_t(l) * dim_ext + d]; }
+    ch[uint64_t(l) * k_pad + d] = _Float16(v);
+    amax                        = fmaxf(amax, fabsf(v));
+    ss                          = fmaf(v, v, ss);
+    if (v != v) { amax = __uint_as_float(0x7f800000u); }
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    amax = fmaxf(amax, __shfl_xor(amax, o));
+    ss += __shfl_xor(ss, o);
+  }
+  if (lane == 0) {
+    const float nrm = l < n_lists ? centers[uint64_t(l) * dim_ext + dim] : 0.0f;
+    cn[l]           = nrm;
+    // non-negative floats order like their bit patterns: largest |element|, largest |stored norm|,
+    // largest Euclidean length of a centre (rounded up)
+    const float inf = __uint_as_float(0x7f800000u);
+    atomicMax(&stats[0], __float_as_uint(amax));
+    atomicMax(&stats[1], __float_as_uint(nrm == nrm ? fabsf(nrm) : inf));
+    atomicMax(&stats[2], __float_as_uint(ss == ss ? sqrtf(ss) * 1.0001f : inf));
+  }
+}
+
+/**
+ * fp16 scores s' = alpha * (dot16(c, q) + cn * qterm) of a block's 128 queries against a run of
+ * list tiles (128 lists each).  The queries stay in LDS for the whole block; list tiles stream
+ * through two LDS buffers, the next tile's global loads in flight while the current one is
+ * multiplied (one barrier per tile).  Four waves, each a 64 x 64 quadrant as 2 x 2 MFMA tiles of
+ * v_mfma_f32_32x32x16_f16.  PASS 1 writes, per query, the minimum over every group of 16 lists;
+ * PASS 2 appends the lists whose score is at or below the query's threshold to its candidate list
+ * (one atomic per lane and tile column).  Both passes execute the same instructions up to the
+ * epilogue, so a list's score is the same number in both.  K_PAD = padded dimension (64 or 128).
+ */
+template <int PASS, uint32_t K_PAD>
+__global__ __launch_bounds__(256, 1) void coarse_f16_kernel(
+  const _Float16* __restrict__ ch, const _Float16* __restrict__ qh, const float* __restrict__ cn,
+  uint32_t n_lists, uint32_t n_queries, uint32_t n_list_tiles, uint32_t tiles_per_block, float alpha,
+  float qterm, float* __restrict__ minima, uint32_t n_groups, const float* __restrict__ thr,
+  uint32_t* __restrict__ cand_count, uint32_t* __restrict__ cand)
+{
+  constexpr uint32_t ROWB   = K_PAD * 2u + 16u;  // 16-byte reads of 32 consecutive rows hit all banks
+  constexpr uint32_t CHUNKS = K_PAD / 8u;        // 16-byte chunks per row
+  constexpr uint32_t PER_T  = kTile * CHUNKS / 256u;  // chunks per thread and tile (4 or 8)
+  extern __shared__ __align__(16) unsigned char smem[];
+  unsigned char* sb  = smem;                         // queries [128][ROWB]
+  unsigned char* sa0 = smem + kTile * ROWB;          // lists, two buffers
+  float* scn         = reinterpret_cast<float*>(smem + 3u * kTile * ROWB);  // [2][128] stored norms
+  const uint32_t tid  = threadIdx.x;
+  const uint32_t lane = tid & 63u;
+  const uint32_t wid  = tid >> 6;
+  const uint32_t wl   = wid >> 1;  // wave's half of the lists
+  const uint32_t wq   = wid & 1u;  // wave's half of the queries
+  const uint32_t q0   = blockIdx.y * kTile;
+  const uint32_t t0   = blockIdx.x * tiles_per_block;
+  const uint32_t t1   = t0 + tiles_per_block < n_list_tiles ? t0 + tiles_per_block : n_list_tiles;
+
+  // this thread's chunks of a tile: row and 16-byte part
+  uint32_t crow[PER_T], cpart[PER_T];
+#pragma unroll
+  for (uint32_t c = 0; c < PER_T; c++) {
+    const uint32_t chunk = tid + c * 256u;
+    crow[c]              = chunk / CHUNKS;
+    cpart[c]             = chunk % CHUNKS;
+  }
+  const float neg_inf = -__uint_as_float(0x7f800000u);
+
+  // the block's queries, once, and the first list tile
+#pragma unroll
+  for (uint32_t c = 0; c < PER_T; c++) {
+    *reinterpret_cast<uint4*>(sb + crow[c] * ROWB + cpart[c] * 16u) =
+      *reinterpret_cast<const uint4*>(qh + uint64_t(q0 + crow[c]) * K_PAD + cpart[c] * 8u);
+    *reinterpret_cast<uint4*>(sa0 + crow[c] * ROWB + cpart[c] * 16u) =
+      *reinterpret_cast<const uint4*>(ch + uint64_t(t0 * kTile + crow[c]) * K_PAD + cpart[c] * 8u);
+  }
+  // per list: the norm term of the score, and for the padding lists a value no maximum picks
+  if (tid < kTile) {
+    const uint32_t l = t0 * kTile + tid;
+    scn[tid]         = l < n_lists ? cn[l] * qterm : neg_inf;
+  }
+  __syncthreads();
+
+  // The epilogue works on v = dot + norm term; the score is alpha * v with alpha = -1 or -2, so the
+  // smallest score of a group is alpha * (its largest v) and "score <= thr" is "v >= thr / alpha",
+  // both exactly.
+  float limit[2] = {0.0f, 0.0f};
+  if (PASS == 2) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const uint32_t q = q0 + wq * 64u + j * 32u + (lane & 31u);
+      limit[j]         = q < n_queries ? thr[q] / alpha : __uint_as_float(0x7f800000u);
+    }
+  }
+
+  for (uint32_t tile = t0; tile < t1; tile++) {
+    const uint32_t buf = (tile - t0) & 1u;
+    // the next tile's loads go out now and land in the other buffer after the products below;
+    // after the last tile they fetch it once more (no branch around loads or stores)
+    const uint32_t nxt = tile + 1u < t1 ? tile + 1u : tile;
+    // The loads are written as instructions: as ordinary loads of read-only data the compiler
+    // sinks them to their first use, behind the matrix products they are meant to overlap (and as
+    // volatile loads it waits for each).  It does not count them, so the wait below is explicit.
+    u32x4 stage[PER_T];
+#pragma unroll
+    for (uint32_t c = 0; c < PER_T; c++) {
+      const _Float16* src = ch + uint64_t(nxt * kTile + crow[c]) * K_PAD + cpart[c] * 8u;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(stage[c]) : "v"(src) : "memory");
+    }
+    // cn has coarse_pad(n_lists) entries: every thread loads one (the upper half of the block a
+    // repeat), nothing branches around the load
+    const uint32_t nl = nxt * kTile + (tid & (kTile - 1u));
+    float stage_cn;
+    {
+      const float* src = cn + nl;
+      asm volatile("global_load_dword %0, %1, off" : "=v"(stage_cn) : "v"(src) : "memory");
+    }
+    const unsigned char* sa = sa0 + buf * (kTile * ROWB);
+    v16f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) { acc[i][j][r] = 0.0f; }
+      }
+    }
+#pragma unroll
+    for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) {
+      const uint32_t kb = (ks * 16u + (lane >> 5) * 8u) * 2u;  // byte offset of this lane's 8 values
+      v8h a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        a[i] = *reinterpret_cast<const v8h*>(sa + (wl * 64u + i * 32u + (lane & 31u)) * ROWB + kb);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        b[j] = *reinterpret_cast<const v8h*>(sb + (wq * 64u + j * 32u + (lane & 31u)) * ROWB + kb);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+      }
+    }
+
+    // element r of a tile: row (list) (r / 4) * 8 + (lane / 32) * 4 + r % 4, column (query) lane % 32
+    const uint32_t l0 = tile * kTile;
+    const float inf   = __uint_as_float(0x7f800000u);
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const uint32_t q = q0 + wq * 64u + j * 32u + (lane & 31u);
+      uint32_t hits    = 0;  // PASS 2: bit (i * 16 + r) set when that list is a candidate
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        const uint32_t rbase = wl * 64u + i * 32u + (lane >> 5) * 4u;  // row inside the block tile
+        float best           = -inf;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const uint32_t row = rbase + (r >> 2) * 8u + (r & 3);
+          const float v      = acc[i][j][r] + scn[buf * kTile + row];
+          if (PASS == 1) {
+            best = fmaxf(best, v);  // NaN scores are ignored here and never pass the threshold
+          } else {
+            hits |= (v >= limit[j]) ? (1u << (i * 16 + r)) : 0u;
+          }
+        }
+        if (PASS == 1 && q < n_queries) {
+          minima[uint64_t(q) * n_groups + ((l0 + wl * 64u + i * 32u) >> 4) + (lane >> 5)] = alpha * best;
+        }
+      }
+      if (PASS == 2 && hits != 0) {
+        const uint32_t n    = __popc(hits);
+        uint32_t slot       = atomicAdd(&cand_count[q], n);
+        while (hits != 0) {
+          const uint32_t bit = __builtin_ctz(hits);
+          hits &= hits - 1u;
+          const uint32_t row = wl * 64u + (bit >> 4) * 32u + (lane >> 5) * 4u + ((bit & 15u) >> 2) * 8u + (bit & 3u);
+          if (slot < kCandCapF) { cand[uint64_t(q) * kCandCapF + slot] = l0 + row; }
+          slot++;
+        }
+      }
+    }
+
+    // the staged tile has arrived
+    if constexpr (PER_T == 8) {
+      asm volatile("s_waitcnt vmcnt(0)"
+                   : "+v"(stage[0]), "+v"(stage[1]), "+v"(stage[2]), "+v"(stage[3]), "+v"(stage[4]),
+                     "+v"(stage[5]), "+v"(stage[6]), "+v"(stage[7]), "+v"(stage_cn)
+                   :
+                   : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)"
+                   : "+v"(stage[0]), "+v"(stage[1]), "+v"(stage[2]), "+v"(stage[3]), "+v"(stage_cn)
+                   :
+                   : "memory");
+    }
+    unsigned char* san = sa0 + (buf ^ 1u) * (kTile * ROWB);
+#pragma unroll
+    for (uint32_t c = 0; c < PER_T; c++) {
+      *reinterpret_cast<u32x4*>(san + crow[c] * ROWB + cpart[c] * 16u) = stage[c];
+    }
+    if (tid < kTile) { scn[(buf ^ 1u) * kTile + tid] = nl < n_lists ? stage_cn * qterm : neg_inf; }
+    __syncthreads();
+  }
+}
+
+/** thr[q] = (n_probes-th smallest of the query's group minima) + 2 E_q, rounded up.  One wave per
+ *  query: the minima sit in registers as ordered keys (16 per lane; more are re-read every round)
+ *  and a round of the bitwise search counts with ballots, without LDS or barriers. */
+__global__ __launch_bounds__(256) void coarse_threshold_kernel(
+  const float* __restrict__ minima, uint32_t n_queries, uint32_t n_groups, uint32_t n_probes,
+  const float* __restrict__ qnorm, float e_rel, float e_abs, float* __restrict__ thr)
+{
+  const uint32_t q    = blockIdx.x * 4u + (threadIdx.x >> 6);
+  const uint32_t lane = threadIdx.x & 63u;
+  if (q >= n_queries) { return; }
+  const float* row = minima + uint64_t(q) * n_groups;
+  constexpr uint32_t HELD = 16;
+  uint32_t held[HELD];
+#pragma unroll
+  for (uint32_t h = 0; h < HELD; h++) {
+    const uint32_t g = lane + h * 64u;
+    const float v    = g < n_groups ? row[g] : __uint_as_float(0x7fc00000u);
+    held[h]          = (v == v) ? order_f32(v) : 0xFFFFFFFFu;  // NaN and padding: above every probe but the last
+  }
+  // smallest ordered key K with count(keys <= K) >= n_probes, one bit at a time
+  uint32_t prefix = 0;
+  for (int bit = 31; bit >= 0; bit--) {
+    const uint32_t probe = prefix | ((1u << bit) - 1u);
+    uint32_t n           = 0;
+#pragma unroll
+    for (uint32_t h = 0; h < HELD; h++) { n += uint32_t(__popcll(__builtin_amdgcn_ballot_w64(held[h] <= probe))); }
+    for (uint32_t g0 = HELD * 64u; g0 < n_groups; g0 += 64u) {
+      const uint32_t g = g0 + lane;
+      const float v    = g < n_groups ? row[g] : __uint_as_float(0x7fc00000u);
+      n += uint32_t(__popcll(__builtin_amdgcn_ballot_w64(v == v && order_f32(v) <= probe)));
+    }
+    if (n < n_probes) { prefix |= 1u << bit; }
+  }
+  if (lane == 0) {
+    const float t = unorder_f32(prefix);
+    const float e = fmaf(e_rel, qnorm[q], e_abs);
+    float bound   = t + 2.0f * e;
+    bound += fabsf(bound) * 1e-6f;  // the additions above round to nearest
+    thr[q] = bound;
+  }
+}
+
+/** Exact fp32 score of every candidate by the fp32 path's arithmetic, then the n_probes best in
+ *  ascending (score, list) order.  One block of 256 threads per query. */
+template <typename T>
+__global__ __launch_bounds__(256) void coarse_rescore_kernel(
+  const T* __restrict__ queries, const float* __restrict__ centers, uint32_t dim, uint32_t dim_ext,
+  float qterm, float alpha, const uint32_t* __restrict__ cand_count, const uint32_t* __restrict__ cand,
+  uint32_t n_probes, uint32_t* __restrict__ probes, uint8_t* __restrict__ fallback)
+{
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* qf                 = reinterpret_cast<float*>(smem);  // [dim]
+  unsigned long long* keys  = reinterpret_cast<unsigned long long*>(smem + ((dim * 4u + 15u) & ~15u));
+  const uint32_t q   = blockIdx.x;
+  const uint32_t tid = threadIdx.x;
+  const uint32_t n   = cand_count[q];
+  if (n > kCandCapF || n < n_probes) {
+    if (tid == 0) { fallback[q] = 1; }
+    return;
+  }
+  for (uint32_t d = tid; d < dim; d += 256) { qf[d] = map_elem<T>(queries[uint64_t(q) * dim + d]); }
+  __syncthreads();
+  unsigned long long key = kInvalidKey;
+  if (tid < n) {
+    const uint32_t l = cand[uint64_t(q) * kCandCapF + tid];
+    const float* c   = centers + uint64_t(l) * dim_ext;
+    float acc        = 0.0f;
+    for (uint32_t d = 0; d < dim; d++) { acc = fmaf(c[d], qf[d], acc); }
+    acc           = fmaf(c[dim], qterm, acc);
+    const float s = alpha * acc;
+    key = (s != s) ? kInvalidKey : ((static_cast<unsigned long long>(order_f32(s)) << 32) | l);
+  }
+  keys[tid] = key;
+  __syncthreads();
+  if (tid < n) {
+    uint32_t rank = 0;
+    for (uint32_t t = 0; t < n; t++) { rank += keys[t] < key ? 1u : 0u; }
+    if (key == kInvalidKey) {
+      fallback[q] = 1;  // a NaN score: let the plain path decide what it means
+    } else if (rank < n_probes) {
+      probes[uint64_t(q) * n_probes + rank] = uint32_t(key);
+    }
+  }
+}
+
+/** fp32 scores of every list for the flagged queries, into their rows of the score matrix. */
+template <typename T>
+__global__ __launch_bounds__(256) void coarse_exact_rows_kernel(
+  const T* __restrict__ queries, const float* __restrict__ centers, uint32_t n_lists, uint32_t dim,
+  uint32_t dim_ext, float qterm, float alpha, const uint8_t* __restrict__ flagged,
+  float* __restrict__ scores)
+{
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* qf        = reinterpret_cast<float*>(smem);
+  const uint32_t q = blockIdx.x;
+  if (!flagged[q]) { return; }
+  for (uint32_t d = threadIdx.x; d < dim; d += 256) { qf[d] = map_elem<T>(queries[uint64_t(q) * dim + d]); }
+  __syncthreads();
+  for (uint32_t l = threadIdx.x; l < n_lists; l += 256) {
+    const float* c = centers + uint64_t(l) * dim_ext;
+    float acc      = 0.0f;
+    for (uint32_t d = 0; d < dim; d++) { acc = fmaf(c[d], qf[d], acc); }
+    acc                               = fmaf(c[dim], qterm, acc);
+    scores[uint64_t(q) * n_lists + l] = alpha * acc;
+  }
+}
+
+}  // namespace
+
+uint32_t coarse_fast_k_pad(uint32_t dim) { return (dim + kSlab - 1) / kSlab * kSlab; }
+uint32_t coarse_fast_groups(uint32_t n_lists) { return coarse_pad(n_lists) / 16u; }
+uint32_t coarse_fast_cand_cap() { return kCandCapF; }
+
+void launch_pack_centers_f16(const float* centers, uint32_t n_lists, uint32_t dim, uint32_t dim_ext,
+                             _Float16* ch, float* cn, uint32_t* stats, hipStream_t stream)
+{
+  const uint32_t l_pad = coarse_pad(n_lists);
+  CUVS_HIP_TRY(hipMemsetAsync(stats, 0, 16, stream));
+  pack_centers_kernel<<<l_pad, 64, 0, stream>>>(centers, n_lists, dim, dim_ext, coarse_fast_k_pad(dim), ch, cn, stats);
+  CUVS_HIP_TRY(hipGetLastError());
+}
+
+void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
+{
+  const uint32_t q_pad = coarse_pad(a.n_queries);
+  const uint32_t l_pad = coarse_pad(a.n_lists);
+  const uint32_t k_pad = coarse_fast_k_pad(a.dim);
+  const uint32_t n_groups = l_pad / 16u;
+  const float qterm    = a.ip_like ? 0.0f : -0.5f;
+  const float alpha    = a.ip_like ? -1.0f : -2.0f;
+  // |s - s'| <= |alpha| * [ (2^-11 + 9 (dim + 4) 2^-24) |q| Cmax + sqrt(dim) 2^-25 |q| + (dim + 4) 2^-24 * Nmax / 2 ],
+  // inflated by 5 %: binary16 rounding of the centre elements (relative 2^-11, absolute 2^-25 below
+  // the normal range), accumulation of dim + 1 terms in both chains, the epilogue's two roundings
+  const float n_terms = float(a.dim + 4);
+  const float two11 = 1.0f / 2048.0f, two24 = 1.0f / 16777216.0f;
+  const float abs_alpha = a.ip_like ? 1.0f : 2.0f;
+  const float e_rel = 1.05f * abs_alpha * ((two11 + 9.0f * n_terms * two24) * a.c_max + sqrtf(float(a.dim)) * two24 * 0.5f);
+  const float e_abs = 1.05f * abs_alpha * n_terms * two24 * 0.5f * a.n_max;
+
+  switch (a.type) {
+    case elem_type::f16:
+      pack_queries_kernel<_Float16><<<q_pad, 64, 0, stream>>>(static_cast<const _Float16*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm);
+      break;
+    case elem_type::i8:
+      pack_queries_kernel<int8_t><<<q_pad, 64, 0, stream>>>(static_cast<const int8_t*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm);
+      break;
+    case elem_type::u8:
+      pack_queries_kernel<uint8_t><<<q_pad, 64, 0, stream>>>(static_cast<const uint8_t*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm);
+      break;
+    default: fail("the two-precision probe selection takes float16, int8 or uint8 queries");
+  }
+  CUVS_HIP_TRY(hipGetLastError());
+
+  // list tiles per block: the queries of a block are loaded once for all of them
+  const uint32_t n_list_tiles    = l_pad / kTile;
+  const uint32_t tiles_per_block = std::min<uint32_t>(8u, n_list_tiles);
+  dim3 grid((n_list_tiles + tiles_per_block - 1) / tiles_per_block, q_pad / kTile);
+  auto run_pass = [&](auto k1, auto k2) {
+    const size_t smem = size_t(3) * kTile * (k_pad * 2 + 16) + 2 * kTile * 4;
+    static bool attr_set = false;
+    if (!attr_set) {
+      CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k1), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+      CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k2), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+      attr_set = true;
+    }
+    k1<<<grid, 256, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, n_list_tiles, tiles_per_block, alpha,
+                                    qterm, a.minima, n_groups, nullptr, nullptr, nullptr);
+    CUVS_HIP_TRY(hipGetLastError());
+    coarse_threshold_kernel<<<(a.n_queries + 3) / 4, 256, 0, stream>>>(a.minima, a.n_queries, n_groups, a.n_probes, a.qnorm, e_rel, e_abs, a.thr);
+    CUVS_HIP_TRY(hipGetLastError());
+    launch_fill_u32(a.cand_count, 0, q_pad, stream);
+    launch_fill_u32(reinterpret_cast<uint32_t*>(a.fallback), 0, (a.n_queries + 3) / 4, stream);
+    k2<<<grid, 256, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, n_list_tiles, tiles_per_block, alpha,
+                                    qterm, nullptr, n_groups, a.thr, a.cand_count, a.cand);
+    CUVS_HIP_TRY(hipGetLastError());
+  };
+  if (k_pad == 64) {
+    run_pass(coarse_f16_kernel<1, 64>, coarse_f16_kernel<2, 64>);
+  } else {
+    CUVS_EXPECTS(k_pad == 128, "the two-precision probe selection takes dim <= 128");
+    run_pass(coarse_f16_kernel<1, 128>, coarse_f16_kernel<2, 128>);
+  }
+  const size_t rsmem = ((size_t(a.dim) * 4 + 15) & ~size_t(15)) + size_t(256) * 8;
+  const size_t xsmem = size_t(a.dim) * 4;
+  CUVS_EXPECTS(rsmem <= 48 * 1024, "dim (%u) is too large for the two-precision probe selection", a.dim);
+  switch (a.type) {
+    case elem_type::f16:
+      coarse_rescore_kernel<_Float16><<<a.n_queries, 256, rsmem, stream>>>(static_cast<const _Float16*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
+      coarse_exact_rows_kernel<_Float16><<<a.n_queries, 256, xsmem, stream>>>(static_cast<const _Float16*>(a.queries), a.centers, a.n_lists, a.dim, a.dim_ext, qterm, alpha, a.fallback, a.scores);
+      break;
+    case elem_type::i8:
+      coarse_rescore_kernel<int8_t><<<a.n_queries, 256, rsmem, stream>>>(static_cast<const int8_t*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
+      coarse_exact_rows_kernel<int8_t><<<a.n_queries, 256, xsmem, stream>>>(static_cast<const int8_t*>(a.queries), a.centers, a.n_lists, a.dim, a.dim_ext, qterm, alpha, a.fallback, a.scores);
+      break;
+    default:
+      coarse_rescore_kernel<uint8_t><<<a.n_queries, 256, rsmem, stream>>>(static_cast<const uint8_t*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
+      coarse_exact_rows_kernel<uint8_t><<<a.n_queries, 256, xsmem, stream>>>(static_cast<const uint8_t*>(a.queries), a.centers, a.n_lists, a.dim, a.dim_ext, qterm, alpha, a.fallback, a.scores);
+      break;
+  }
+  CUVS_HIP_TRY(hipGetLastError());
+  // the flagged queries (normally none) take the plain selection over their exact rows
+  launch_select_probes(a.scores, a.n_queries, a.n_lists, a.n_probes, a.probes, stream, a.fallback);
+}
+
+}  // namespace cuvs::neighbors::ivf_pq::detail

@@ -113,6 +113,14 @@ struct index_impl {
 
   device_buffer centers, centers_rot, rotation, rotation_t, pq_centers;
   device_buffer centers_t;  // [dim_ext][coarse_pad(n_lists)]: centres k-major for the matrix-core kernel
+  // two-precision probe selection: centres as binary16 [coarse_pad(n_lists)][k_pad], their stored
+  // norms, and the largest centre length / |stored norm| (coarse_fast_ok: all finite and within
+  // binary16's range)
+  device_buffer centers_h, center_norms;
+  float c_max = 0.0f, n_max = 0.0f;
+  bool coarse_fast_ok = false;
+  /** centers_t, centers_h, center_norms and the maxima from `centers` (synchronises). */
+  void refresh_coarse(hipStream_t stream);
   bool rotation_is_identity = false;
 
   device_buffer codes_arena, ids_arena;
@@ -168,8 +176,38 @@ void launch_coarse_scores_mfma(const float* qt, const float* ct, uint32_t n_quer
 /** The probe selection reads whole segments of 256 x 64 scores: the score buffer must have this
  *  many readable bytes after its last row. */
 constexpr size_t kSelectSlackBytes = 256 * 64 * 4;
+/** With `only` non-null, queries whose byte there is zero are left alone. */
 void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_lists,
-                          uint32_t n_probes, uint32_t* probes, hipStream_t stream);
+                          uint32_t n_probes, uint32_t* probes, hipStream_t stream,
+                          const uint8_t* only = nullptr);
+
+/* probe selection in two precisions (coarse_fast.hip) */
+struct coarse_fast_args {
+  const void* queries;     // [n_queries, dim] of `type` (f16, i8 or u8)
+  elem_type type;
+  uint32_t n_queries, n_lists, dim, dim_ext, n_probes;
+  bool ip_like;
+  const float* centers;    // [n_lists, dim_ext]
+  const _Float16* ch;      // [coarse_pad(n_lists), k_pad] centres as binary16
+  const float* cn;         // [coarse_pad(n_lists)] stored squared norms
+  float c_max, n_max;      // largest centre length, largest |stored norm|
+  _Float16* qh;            // [coarse_pad(n_queries), k_pad]
+  float* qnorm;            // [coarse_pad(n_queries)]
+  float* minima;           // [n_queries, coarse_fast_groups(n_lists)]
+  float* thr;              // [n_queries]
+  uint32_t* cand_count;    // [coarse_pad(n_queries)]
+  uint32_t* cand;          // [n_queries, coarse_fast_cand_cap()]
+  uint8_t* fallback;       // [round_up(n_queries, 4)]
+  float* scores;           // [n_queries, n_lists]: rows of flagged queries only
+  uint32_t* probes;        // [n_queries, n_probes]
+};
+uint32_t coarse_fast_k_pad(uint32_t dim);
+uint32_t coarse_fast_groups(uint32_t n_lists);
+uint32_t coarse_fast_cand_cap();
+/** stats (3 words, device): bit patterns of the largest |element|, |stored norm| and centre length. */
+void launch_pack_centers_f16(const float* centers, uint32_t n_lists, uint32_t dim, uint32_t dim_ext,
+                             _Float16* ch, float* cn, uint32_t* stats, hipStream_t stream);
+void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream);
 
 /** rot_q = rotation * qf (+ row normalisation for cosine); rotation_t is [dim, rot_dim]. */
 void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries, uint32_t dim,

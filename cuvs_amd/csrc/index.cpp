@@ -7,6 +7,7 @@
 #include "detail.hpp"
 
 #include <algorithm>
+#include <cmath>
 #include <functional>
 
 namespace cuvs::neighbors::ivf_pq {
@@ -85,6 +86,27 @@ void index_impl::recompute_internal_state(hipStream_t stream)
     accum_sorted_sizes[l + 1] = accum_sorted_sizes[l] + sorted[l];
   }
   size = accum_sorted_sizes[n_lists];
+}
+
+void index_impl::refresh_coarse(hipStream_t stream)
+{
+  const uint32_t l_pad = coarse_pad(n_lists);
+  if (centers_t.bytes == 0) { centers_t.allocate(size_t(dim_ext) * l_pad * sizeof(float)); }
+  launch_transpose_centers(centers.as<float>(), n_lists, dim_ext, centers_t.as<float>(), stream);
+  const uint32_t k_pad = coarse_fast_k_pad(dim);
+  if (centers_h.bytes == 0) {
+    centers_h.allocate(size_t(l_pad) * k_pad * sizeof(_Float16));
+    center_norms.allocate(size_t(l_pad) * sizeof(float));
+  }
+  device_buffer stats(16);
+  launch_pack_centers_f16(centers.as<float>(), n_lists, dim, dim_ext, centers_h.as<_Float16>(),
+                          center_norms.as<float>(), stats.as<uint32_t>(), stream);
+  float h[4] = {0, 0, 0, 0};
+  CUVS_HIP_TRY(hipMemcpyAsync(h, stats.ptr, 16, hipMemcpyDeviceToHost, stream));
+  CUVS_HIP_TRY(hipStreamSynchronize(stream));
+  n_max          = h[1];
+  c_max          = h[2];
+  coarse_fast_ok = std::isfinite(h[0]) && h[0] < 60000.0f && std::isfinite(h[1]) && std::isfinite(h[2]);
 }
 
 void index_impl::rebuild_lead_plane(hipStream_t stream)
@@ -171,9 +193,7 @@ index<int64_t> build(cuvs::resources const& res,
   copy_in(ix.pq_centers, pq_centers, n_books * ix.pq_len * ix.book_size);
   copy_in(ix.centers, centers, size_t(ix.n_lists) * ix.dim_ext);
   copy_in(ix.centers_rot, centers_rot, size_t(ix.n_lists) * ix.rot_dim);
-  ix.centers_t.allocate(size_t(ix.dim_ext) * detail::coarse_pad(ix.n_lists) * sizeof(float));
-  detail::launch_transpose_centers(ix.centers.as<float>(), ix.n_lists, ix.dim_ext,
-                                   ix.centers_t.as<float>(), stream);
+  ix.refresh_coarse(stream);
   copy_in(ix.rotation, rotation_matrix, size_t(ix.rot_dim) * ix.dim);
 
   // transposed copy [dim, rot_dim] for coalesced reads, and the identity check

@@ -146,12 +146,14 @@ __global__ __launch_bounds__(kBlock) void select_probes_kernel(const float* __re
                                                                 uint32_t n_lists,
                                                                 uint32_t n_probes,
                                                                 uint32_t out_cap,
-                                                                uint32_t* __restrict__ probes)
+                                                                uint32_t* __restrict__ probes,
+                                                                const uint8_t* __restrict__ only)
 {
   extern __shared__ __align__(16) unsigned char dyn_smem[];
   __shared__ select_smem sm;
   unsigned long long* out = reinterpret_cast<unsigned long long*>(dyn_smem);
   const uint32_t q        = blockIdx.x;
+  if (only != nullptr && !only[q]) { return; }
   const float* row        = scores + uint64_t(q) * n_lists;
   auto key_of             = [row](uint32_t i) -> unsigned long long {
     const float v = row[i];
@@ -201,7 +203,8 @@ __device__ __forceinline__ uint32_t wave_sort_u32(uint32_t v, uint32_t lane)
 __global__ __launch_bounds__(kBlock, 3) void select_probes_fast_kernel(const float* __restrict__ scores,
                                                                      uint32_t n_lists,
                                                                      uint32_t n_probes,
-                                                                     uint32_t* __restrict__ probes)
+                                                                     uint32_t* __restrict__ probes,
+                                                                     const uint8_t* __restrict__ only)
 {
   __shared__ unsigned long long cand[kSelCap];
   __shared__ unsigned long long ranked[kBlock];
@@ -212,6 +215,7 @@ __global__ __launch_bounds__(kBlock, 3) void select_probes_fast_kernel(const flo
   const uint32_t lane = tid & 63u;
   const uint32_t wid  = tid >> 6;
   const uint32_t q    = blockIdx.x;
+  if (only != nullptr && !only[q]) { return; }
   const float* row    = scores + uint64_t(q) * n_lists;
   uint32_t have       = 0;  // sorted best-so-far in cand[0..have)
   bool overflow       = false;
@@ -1096,11 +1100,11 @@ void launch_coarse_scores(const float* qf, const float* centers, uint32_t n_quer
 }
 
 void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_lists,
-                          uint32_t n_probes, uint32_t* probes, hipStream_t stream)
+                          uint32_t n_probes, uint32_t* probes, hipStream_t stream, const uint8_t* only)
 {
   if (n_queries == 0) { return; }
   if (n_probes <= kBlock) {
-    select_probes_fast_kernel<<<n_queries, kBlock, 0, stream>>>(scores, n_lists, n_probes, probes);
+    select_probes_fast_kernel<<<n_queries, kBlock, 0, stream>>>(scores, n_lists, n_probes, probes, only);
     CUVS_LAUNCH_CHECK();
     return;
   }
@@ -1111,7 +1115,7 @@ void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_li
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(select_probes_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
   }
-  select_probes_kernel<<<n_queries, kBlock, smem, stream>>>(scores, n_lists, n_probes, out_cap, probes);
+  select_probes_kernel<<<n_queries, kBlock, smem, stream>>>(scores, n_lists, n_probes, out_cap, probes, only);
   CUVS_LAUNCH_CHECK();
 }
 

@@ -94,6 +94,12 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
                       P * 4 * 3 + P * (2 * sizeof(detail::pair_desc) + 1) + 16 +
                       (p.fused ? P * k * 8 * 4 : size_t(p.max_samples) * 4);
   p.fixed_bytes = a256(size_t(ix.n_lists) * 16 + 16) + a256(size_t(ix.dim_ext) * 128 * 4) + a256(detail::kSelectSlackBytes) + 16 * 256;
+  if (ix.coarse_fast_ok) {
+    // buffers of the two-precision probe selection (the batch must fit with them)
+    p.per_query_bytes += size_t(detail::coarse_fast_k_pad(ix.dim)) * 2 + size_t(detail::coarse_fast_groups(ix.n_lists)) * 4 +
+                         size_t(detail::coarse_fast_cand_cap()) * 4 + 16;
+    p.fixed_bytes += a256(size_t(128) * (detail::coarse_fast_k_pad(ix.dim) * 2 + 8)) + 8 * 256;
+  }
   const size_t budget = workspace_budget(res);
   size_t b = budget > p.fixed_bytes ? (budget - p.fixed_bytes) / (p.per_query_bytes + 64) : 1;
   b        = std::max<size_t>(b, 1);
@@ -202,7 +208,55 @@ struct coarse_buffers {
   float* qf;
   float* scores;
   uint32_t* probes;
+  // two-precision selection (null when it does not apply)
+  _Float16* qh      = nullptr;
+  float* qnorm      = nullptr;
+  float* minima     = nullptr;
+  float* thr        = nullptr;
+  uint32_t* cand_count = nullptr;
+  uint32_t* cand    = nullptr;
+  uint8_t* fallback = nullptr;
 };
+
+bool coarse_plain_forced()
+{
+  static const bool forced = [] {
+    const char* e = std::getenv("CUVS_AMD_COARSE_PLAIN");
+    return e != nullptr && e[0] == '1';
+  }();
+  return forced;
+}
+
+/** The two-precision probe selection applies to element types that binary16 holds exactly, to
+ *  fp32 coarse search, and to shapes where its candidate lists stay short. */
+bool coarse_fast_applies(const search_params& params, const index_impl& ix, elem_type type,
+                         uint32_t n_probes)
+{
+  return !coarse_plain_forced() && ix.coarse_fast_ok && type != elem_type::f32 &&
+         params.coarse_search_dtype == CUDA_R_32F && n_probes <= detail::coarse_fast_cand_cap() / 2 &&
+         ix.n_lists >= 1024 && ix.n_lists >= 32u * n_probes && ix.dim <= 128;
+}
+
+/** Workspace bytes of the two-precision selection for a batch, and its allocation. */
+size_t coarse_fast_bytes(const index_impl& ix, size_t batch)
+{
+  const size_t q_pad = detail::coarse_pad(uint32_t(batch));
+  return a256(q_pad * detail::coarse_fast_k_pad(ix.dim) * 2) + a256(q_pad * 4) +
+         a256(batch * detail::coarse_fast_groups(ix.n_lists) * 4) + a256(batch * 4) + a256(q_pad * 4) +
+         a256(batch * detail::coarse_fast_cand_cap() * 4) + a256(batch + 4);
+}
+
+void alloc_coarse_fast(cuvs::resources& res, const index_impl& ix, size_t batch, coarse_buffers& b)
+{
+  const size_t q_pad = detail::coarse_pad(uint32_t(batch));
+  b.qh         = static_cast<_Float16*>(res.workspace_alloc(q_pad * detail::coarse_fast_k_pad(ix.dim) * 2));
+  b.qnorm      = static_cast<float*>(res.workspace_alloc(q_pad * 4));
+  b.minima     = static_cast<float*>(res.workspace_alloc(batch * detail::coarse_fast_groups(ix.n_lists) * 4));
+  b.thr        = static_cast<float*>(res.workspace_alloc(batch * 4));
+  b.cand_count = static_cast<uint32_t*>(res.workspace_alloc(q_pad * 4));
+  b.cand       = static_cast<uint32_t*>(res.workspace_alloc(batch * detail::coarse_fast_cand_cap() * 4));
+  b.fallback   = static_cast<uint8_t*>(res.workspace_alloc(batch + 4));
+}
 
 /** mapping + centre scores + probe selection for one batch */
 void run_coarse(const cuvs::resources& res, const search_params& params, const index_impl& ix,
@@ -213,6 +267,33 @@ void run_coarse(const cuvs::resources& res, const search_params& params, const i
   const bool ip     = ix.metric == detail::DistanceType::InnerProduct ||
                   ix.metric == detail::DistanceType::CosineExpanded;
   detail::launch_map_queries(queries, type, uint64_t(nq) * ix.dim, b.qf, s);
+  if (b.qh != nullptr) {
+    detail::coarse_fast_args a{};
+    a.queries    = queries;
+    a.type       = type;
+    a.n_queries  = nq;
+    a.n_lists    = ix.n_lists;
+    a.dim        = ix.dim;
+    a.dim_ext    = ix.dim_ext;
+    a.n_probes   = n_probes;
+    a.ip_like    = ip;
+    a.centers    = ix.centers.as<float>();
+    a.ch         = ix.centers_h.as<_Float16>();
+    a.cn         = ix.center_norms.as<float>();
+    a.c_max      = ix.c_max;
+    a.n_max      = ix.n_max;
+    a.qh         = b.qh;
+    a.qnorm      = b.qnorm;
+    a.minima     = b.minima;
+    a.thr        = b.thr;
+    a.cand_count = b.cand_count;
+    a.cand       = b.cand;
+    a.fallback   = b.fallback;
+    a.scores     = b.scores;
+    a.probes     = b.probes;
+    detail::launch_coarse_fast(a, s);
+    return;
+  }
   detail::launch_map_queries_t(queries, type, nq, ix.dim, ix.dim_ext, ip, b.qt, s);
   detail::launch_coarse_scores_mfma(b.qt, ix.centers_t.as<float>(), nq, ix.n_lists, ix.dim_ext, ip,
                                     params.coarse_search_dtype == CUDA_R_16F, b.scores, s);
@@ -244,13 +325,16 @@ void select_clusters(cuvs::resources const& res_c,
   batch                  = std::min<size_t>(batch, 65535u * 64u);
   res.reset_workspace();
   const size_t qt_bytes = size_t(ix.dim_ext) * detail::coarse_pad(uint32_t(batch)) * 4;
+  const bool fast       = coarse_fast_applies(params, ix, type, P);
   res.reserve_workspace(a256(batch * ix.dim * 4) + a256(qt_bytes) +
-                        a256(batch * size_t(ix.n_lists) * 4 + detail::kSelectSlackBytes) + 1024);
-  coarse_buffers b;
+                        a256(batch * size_t(ix.n_lists) * 4 + detail::kSelectSlackBytes) + 1024 +
+                        (fast ? coarse_fast_bytes(ix, batch) : 0));
+  coarse_buffers b{};
   b.qt     = static_cast<float*>(res.workspace_alloc(qt_bytes));
   b.qf     = static_cast<float*>(res.workspace_alloc(batch * ix.dim * 4));
   b.scores = static_cast<float*>(
     res.workspace_alloc(batch * size_t(ix.n_lists) * 4 + detail::kSelectSlackBytes));
+  if (fast) { alloc_coarse_fast(res, ix, batch, b); }
   for (int64_t q0 = 0; q0 < n_queries; q0 += int64_t(batch)) {
     const uint32_t nq = uint32_t(std::min<int64_t>(int64_t(batch), n_queries - q0));
     b.probes          = clusters_to_probe + q0 * P;
@@ -337,8 +421,9 @@ void search(cuvs::resources const& res_c,
 
   /* workspace carve-up for one batch */
   res.reset_workspace();
+  const bool fast_coarse = coarse_fast_applies(params, ix, type, P);
   res.reserve_workspace(pl.fixed_bytes + size_t(Qb) * (pl.per_query_bytes + 64) + 16 * 256 +
-                        global_lut_bytes);
+                        global_lut_bytes + (fast_coarse ? coarse_fast_bytes(ix, Qb) : 0));
   auto* qt        = static_cast<float*>(
     res.workspace_alloc(size_t(ix.dim_ext) * detail::coarse_pad(Qb) * 4));
   auto* qf        = static_cast<float*>(res.workspace_alloc(size_t(Qb) * ix.dim * 4));
@@ -351,6 +436,8 @@ void search(cuvs::resources const& res_c,
   auto* n_samples = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * 4));
   auto* kth       = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * 4));
   auto* counters  = static_cast<uint32_t*>(res.workspace_alloc(size_t(ix.n_lists) * 16 + 16));
+  coarse_buffers cb{qt, qf, scores, probes};
+  if (fast_coarse) { alloc_coarse_fast(res, ix, Qb, cb); }
   detail::pair_desc* desc = nullptr;
   unsigned long long* keys = nullptr;
   float* all_scores        = nullptr;
@@ -408,7 +495,7 @@ void search(cuvs::resources const& res_c,
     const void* qptr  = static_cast<const char*>(queries) + size_t(q0) * ix.dim * elem_size(type);
 
     mark(0);
-    run_coarse(res, params, ix, qptr, type, nq, P, coarse_buffers{qt, qf, scores, probes});
+    run_coarse(res, params, ix, qptr, type, nq, P, cb);
     mark(1);
     detail::launch_rotate(qf, ix.rotation_t.as<float>(), nq, ix.dim, ix.rot_dim,
                           ix.rotation_is_identity, cosine, rot_q, s);

@@ -183,7 +183,6 @@ index<int64_t> build(cuvs::resources const& res_c,
   device_buffer labels(n_train * sizeof(uint32_t));
   device_buffer d_recv(size_t(L) * sizeof(uint32_t)), d_donor(size_t(L) * sizeof(uint32_t));
   cx.centers.allocate(size_t(L) * cx.dim_ext * sizeof(float));
-  cx.centers_t.allocate(size_t(cx.dim_ext) * detail::coarse_pad(L) * sizeof(float));
   // initial centres: training rows spread evenly over the set
   detail::launch_gather_rows(trainset.ptr, uint64_t(dim) * 4, L, n_train / L, kTrainSeed + 1, flat.ptr, s);
 
@@ -191,7 +190,7 @@ index<int64_t> build(cuvs::resources const& res_c,
   sp.n_probes = 1;
   auto assign = [&]() {
     detail::launch_set_centers(flat.as<float>(), L, dim, cx.dim_ext, cx.centers.as<float>(), s);
-    detail::launch_transpose_centers(cx.centers.as<float>(), L, cx.dim_ext, cx.centers_t.as<float>(), s);
+    cx.refresh_coarse(s);
     select_clusters(res, sp, coarse, trainset.ptr, elem_type::f32, int64_t(n_train), labels.as<uint32_t>());
   };
   std::vector<uint32_t> h_counts(L), receivers, donors;

@@ -243,7 +243,7 @@ def test_validation_errors(orc):
         dd = torch.empty((4, 5), dtype=torch.float32, device="cuda")
         check(lib().cuvsIvfPqSearch(ivf_pq._default_resources().get_c_obj(), ok._p, index.index,
                                     qv.ptr, dlpack.view(nb).ptr, dlpack.view(dd).ptr))
-    with pytest.raises(CuvsError, match="not part of this library"):
+    with pytest.raises(CuvsError, match="less than n_lists"):
         ivf_pq.build(ivf_pq.IndexParams(), q)
     # a good call clears the error text and still works after the failures above
     d, nb = ivf_pq.search(ok, index, q, 5)
