@@ -44,6 +44,8 @@ constexpr uint32_t kCandCapF = 256;  // candidates per query
 template <typename T>
 __device__ __forceinline__ float map_elem(T v);
 template <>
+__device__ __forceinline__ float map_elem<float>(float v) { return v; }
+template <>
 __device__ __forceinline__ float map_elem<_Float16>(_Float16 v) { return float(v); }
 template <>
 __device__ __forceinline__ float map_elem<int8_t>(int8_t v) { return float(v) * (1.0f / 128.0f); }
@@ -51,7 +53,8 @@ template <>
 __device__ __forceinline__ float map_elem<uint8_t>(uint8_t v) { return float(v) * (1.0f / 256.0f); }
 
 /** qh[q][d] = mapped query as binary16 (exact for these element types), zero padded to k_pad
- *  columns and q_pad rows; qnorm[q] = an upper bound of the query's Euclidean norm. */
+ *  columns and q_pad rows; qnorm[q] = an upper bound of the query's Euclidean norm (of the
+ *  unrounded values: float32 queries are the one type that binary16 does not hold exactly). */
 template <typename T>
 __global__ void pack_queries_kernel(const T* __restrict__ in, uint32_t n_queries, uint32_t dim,
                                     uint32_t k_pad, _Float16* __restrict__ qh, float* __restrict__ qnorm)
@@ -102,18 +105,24 @@ __global__ void pack_centers_kernel(const float* __restrict__ centers, uint32_t 
   }
 }
 
+constexpr uint32_t kGemmThreads = 512;
+constexpr uint32_t kLocalCap    = 32;  // PASS 2: candidates a block may hold per query before it gives up
+constexpr uint32_t kTilesPerBlock = 8;  // list tiles a block walks at most
+
 /**
  * fp16 scores s' = alpha * (dot16(c, q) + cn * qterm) of a block's 128 queries against a run of
  * list tiles (128 lists each).  The queries stay in LDS for the whole block; list tiles stream
  * through two LDS buffers, the next tile's global loads in flight while the current one is
- * multiplied (one barrier per tile).  Four waves, each a 64 x 64 quadrant as 2 x 2 MFMA tiles of
+ * multiplied (one barrier per tile).  Eight waves, two per SIMD so that one's matrix products
+ * overlap the other's epilogue; a wave owns 64 lists x 32 queries, two MFMA tiles of
  * v_mfma_f32_32x32x16_f16.  PASS 1 writes, per query, the minimum over every group of 16 lists;
- * PASS 2 appends the lists whose score is at or below the query's threshold to its candidate list
- * (one atomic per lane and tile column).  Both passes execute the same instructions up to the
- * epilogue, so a list's score is the same number in both.  K_PAD = padded dimension (64 or 128).
+ * PASS 2 collects the lists whose score is at or below the query's threshold in LDS and appends
+ * them to the query's candidate list when the block ends (one global atomic per query and block).
+ * Both passes execute the same instructions up to the epilogue, so a list's score is the same
+ * number in both.  K_PAD = padded dimension (64 or 128).
  */
 template <int PASS, uint32_t K_PAD>
-__global__ __launch_bounds__(256, 1) void coarse_f16_kernel(
+__global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
   const _Float16* __restrict__ ch, const _Float16* __restrict__ qh, const float* __restrict__ cn,
   uint32_t n_lists, uint32_t n_queries, uint32_t n_list_tiles, uint32_t tiles_per_block, float alpha,
   float qterm, float* __restrict__ minima, uint32_t n_groups, const float* __restrict__ thr,
@@ -121,16 +130,18 @@ __global__ __launch_bounds__(256, 1) void coarse_f16_kernel(
 {
   constexpr uint32_t ROWB   = K_PAD * 2u + 16u;  // 16-byte reads of 32 consecutive rows hit all banks
   constexpr uint32_t CHUNKS = K_PAD / 8u;        // 16-byte chunks per row
-  constexpr uint32_t PER_T  = kTile * CHUNKS / 256u;  // chunks per thread and tile (4 or 8)
+  constexpr uint32_t PER_T  = kTile * CHUNKS / kGemmThreads;  // chunks per thread and tile (2 or 4)
   extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char* sb  = smem;                         // queries [128][ROWB]
-  unsigned char* sa0 = smem + kTile * ROWB;          // lists, two buffers
-  float* scn         = reinterpret_cast<float*>(smem + 3u * kTile * ROWB);  // [2][128] stored norms
+  unsigned char* sa0 = smem;  // lists [2][128][ROWB], two buffers
+  float* scn         = reinterpret_cast<float*>(smem + 2u * kTile * ROWB);  // [2][128] norm terms
+  uint32_t* lcount   = reinterpret_cast<uint32_t*>(scn + 2u * kTile);       // PASS 2: [128]
+  uint32_t* lcand    = lcount + kTile;                                      // PASS 2: [128][kLocalCap]
+  float* lmin        = reinterpret_cast<float*>(lcount);  // PASS 1: [128][kTilesPerBlock * 8] group minima
   const uint32_t tid  = threadIdx.x;
   const uint32_t lane = tid & 63u;
   const uint32_t wid  = tid >> 6;
-  const uint32_t wl   = wid >> 1;  // wave's half of the lists
-  const uint32_t wq   = wid & 1u;  // wave's half of the queries
+  const uint32_t wl   = wid >> 2;  // wave's half of the lists (64)
+  const uint32_t wq   = wid & 3u;  // wave's quarter of the queries (32)
   const uint32_t q0   = blockIdx.y * kTile;
   const uint32_t t0   = blockIdx.x * tiles_per_block;
   const uint32_t t1   = t0 + tiles_per_block < n_list_tiles ? t0 + tiles_per_block : n_list_tiles;
@@ -139,17 +150,15 @@ __global__ __launch_bounds__(256, 1) void coarse_f16_kernel(
   uint32_t crow[PER_T], cpart[PER_T];
 #pragma unroll
   for (uint32_t c = 0; c < PER_T; c++) {
-    const uint32_t chunk = tid + c * 256u;
+    const uint32_t chunk = tid + c * kGemmThreads;
     crow[c]              = chunk / CHUNKS;
     cpart[c]             = chunk % CHUNKS;
   }
   const float neg_inf = -__uint_as_float(0x7f800000u);
 
-  // the block's queries, once, and the first list tile
+  // the first list tile
 #pragma unroll
   for (uint32_t c = 0; c < PER_T; c++) {
-    *reinterpret_cast<uint4*>(sb + crow[c] * ROWB + cpart[c] * 16u) =
-      *reinterpret_cast<const uint4*>(qh + uint64_t(q0 + crow[c]) * K_PAD + cpart[c] * 8u);
     *reinterpret_cast<uint4*>(sa0 + crow[c] * ROWB + cpart[c] * 16u) =
       *reinterpret_cast<const uint4*>(ch + uint64_t(t0 * kTile + crow[c]) * K_PAD + cpart[c] * 8u);
   }
@@ -157,132 +166,150 @@ __global__ __launch_bounds__(256, 1) void coarse_f16_kernel(
   if (tid < kTile) {
     const uint32_t l = t0 * kTile + tid;
     scn[tid]         = l < n_lists ? cn[l] * qterm : neg_inf;
+    if (PASS == 2) { lcount[tid] = 0; }
   }
   __syncthreads();
 
   // The epilogue works on v = dot + norm term; the score is alpha * v with alpha = -1 or -2, so the
   // smallest score of a group is alpha * (its largest v) and "score <= thr" is "v >= thr / alpha",
   // both exactly.
-  float limit[2] = {0.0f, 0.0f};
-  if (PASS == 2) {
+  const uint32_t qloc = wq * 32u + (lane & 31u);  // this lane's query inside the block
+  const uint32_t q    = q0 + qloc;
+  // the wave's query operand never changes: it lives in registers (8 values per 16 dimensions)
+  v8h bq[K_PAD / 16u];
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      const uint32_t q = q0 + wq * 64u + j * 32u + (lane & 31u);
-      limit[j]         = q < n_queries ? thr[q] / alpha : __uint_as_float(0x7f800000u);
-    }
+  for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) {
+    bq[ks] = *reinterpret_cast<const v8h*>(qh + uint64_t(q) * K_PAD + ks * 16u + (lane >> 5) * 8u);
   }
+  // Use them once here, so that the compiler's wait for these loads sits here and not inside the
+  // loop: there it would also wait for the staged loads below, which it does not count.
+#pragma unroll
+  for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) { asm volatile("" : "+v"(bq[ks])); }
+  float limit         = 0.0f;
+  if (PASS == 2) { limit = q < n_queries ? thr[q] / alpha : __uint_as_float(0x7f800000u); }
 
-  for (uint32_t tile = t0; tile < t1; tile++) {
-    const uint32_t buf = (tile - t0) & 1u;
-    // the next tile's loads go out now and land in the other buffer after the products below;
-    // after the last tile they fetch it once more (no branch around loads or stores)
-    const uint32_t nxt = tile + 1u < t1 ? tile + 1u : tile;
-    // The loads are written as instructions: as ordinary loads of read-only data the compiler
-    // sinks them to their first use, behind the matrix products they are meant to overlap (and as
-    // volatile loads it waits for each).  It does not count them, so the wait below is explicit.
-    u32x4 stage[PER_T];
+  // The next tile's loads go out at the top of an iteration and are written to the other LDS
+  // buffer at its end.  They are written as instructions: as ordinary loads of read-only data the
+  // compiler sinks them to their first use, behind the matrix products they are meant to overlap
+  // (and as volatile loads it waits for each).  It does not count them, so the wait is explicit.
+  // Tile numbers past the block's last tile repeat it (no branch around loads or stores).  (Loads
+  // two tiles ahead measured slower: the loop is not waiting on them.)
+  u32x4 sx[PER_T];
+  float cx = 0.0f;
+  auto issue = [&](uint32_t tile, u32x4(&st)[PER_T], float& sc) __attribute__((always_inline)) {
+    const uint32_t at = tile < t1 ? tile : t1 - 1u;
 #pragma unroll
     for (uint32_t c = 0; c < PER_T; c++) {
-      const _Float16* src = ch + uint64_t(nxt * kTile + crow[c]) * K_PAD + cpart[c] * 8u;
-      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(stage[c]) : "v"(src) : "memory");
+      const _Float16* src = ch + uint64_t(at * kTile + crow[c]) * K_PAD + cpart[c] * 8u;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(st[c]) : "v"(src) : "memory");
     }
-    // cn has coarse_pad(n_lists) entries: every thread loads one (the upper half of the block a
-    // repeat), nothing branches around the load
-    const uint32_t nl = nxt * kTile + (tid & (kTile - 1u));
-    float stage_cn;
-    {
-      const float* src = cn + nl;
-      asm volatile("global_load_dword %0, %1, off" : "=v"(stage_cn) : "v"(src) : "memory");
+    // cn has coarse_pad(n_lists) entries: every thread loads one (most of the block a repeat)
+    const float* src = cn + at * kTile + (tid & (kTile - 1u));
+    asm volatile("global_load_dword %0, %1, off" : "=v"(sc) : "v"(src) : "memory");
+  };
+  auto arrived = [&](u32x4(&st)[PER_T], float& sc) __attribute__((always_inline)) {
+    if constexpr (PER_T == 4) {
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(st[0]), "+v"(st[1]), "+v"(st[2]), "+v"(st[3]), "+v"(sc) : : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(st[0]), "+v"(st[1]), "+v"(sc) : : "memory");
     }
+  };
+  auto commit = [&](uint32_t tile, uint32_t buf, const u32x4(&st)[PER_T], float sc) __attribute__((always_inline)) {
+    const uint32_t at  = tile < t1 ? tile : t1 - 1u;
+    unsigned char* san = sa0 + buf * (kTile * ROWB);
+#pragma unroll
+    for (uint32_t c = 0; c < PER_T; c++) {
+      *reinterpret_cast<u32x4*>(san + crow[c] * ROWB + cpart[c] * 16u) = st[c];
+    }
+    if (tid < kTile) { scn[buf * kTile + tid] = at * kTile + tid < n_lists ? sc * qterm : neg_inf; }
+  };
+  // products and epilogue of one tile out of LDS buffer `buf`
+  auto multiply = [&](uint32_t tile, uint32_t buf) __attribute__((always_inline)) {
     const unsigned char* sa = sa0 + buf * (kTile * ROWB);
-    v16f acc[2][2];
+    v16f acc[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
 #pragma unroll
-      for (int j = 0; j < 2; j++) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) { acc[i][j][r] = 0.0f; }
-      }
+      for (int r = 0; r < 16; r++) { acc[i][r] = 0.0f; }
     }
 #pragma unroll
     for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) {
       const uint32_t kb = (ks * 16u + (lane >> 5) * 8u) * 2u;  // byte offset of this lane's 8 values
-      v8h a[2], b[2];
+      v8h a[2];
 #pragma unroll
       for (int i = 0; i < 2; i++) {
         a[i] = *reinterpret_cast<const v8h*>(sa + (wl * 64u + i * 32u + (lane & 31u)) * ROWB + kb);
       }
 #pragma unroll
-      for (int j = 0; j < 2; j++) {
-        b[j] = *reinterpret_cast<const v8h*>(sb + (wq * 64u + j * 32u + (lane & 31u)) * ROWB + kb);
-      }
-#pragma unroll
       for (int i = 0; i < 2; i++) {
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], bq[ks], acc[i], 0, 0, 0);
       }
     }
-
     // element r of a tile: row (list) (r / 4) * 8 + (lane / 32) * 4 + r % 4, column (query) lane % 32
     const uint32_t l0 = tile * kTile;
-    const float inf   = __uint_as_float(0x7f800000u);
+    uint32_t hits     = 0;  // PASS 2: bit (i * 16 + r) set when that list is a candidate
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      const uint32_t q = q0 + wq * 64u + j * 32u + (lane & 31u);
-      uint32_t hits    = 0;  // PASS 2: bit (i * 16 + r) set when that list is a candidate
+    for (int i = 0; i < 2; i++) {
+      const uint32_t rbase = wl * 64u + i * 32u + (lane >> 5) * 4u;  // row inside the block tile
+      float best           = neg_inf;
 #pragma unroll
-      for (int i = 0; i < 2; i++) {
-        const uint32_t rbase = wl * 64u + i * 32u + (lane >> 5) * 4u;  // row inside the block tile
-        float best           = -inf;
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const uint32_t row = rbase + (r >> 2) * 8u + (r & 3);
-          const float v      = acc[i][j][r] + scn[buf * kTile + row];
-          if (PASS == 1) {
-            best = fmaxf(best, v);  // NaN scores are ignored here and never pass the threshold
-          } else {
-            hits |= (v >= limit[j]) ? (1u << (i * 16 + r)) : 0u;
-          }
-        }
-        if (PASS == 1 && q < n_queries) {
-          minima[uint64_t(q) * n_groups + ((l0 + wl * 64u + i * 32u) >> 4) + (lane >> 5)] = alpha * best;
+      for (int r = 0; r < 16; r++) {
+        const uint32_t row = rbase + (r >> 2) * 8u + (r & 3);
+        const float v      = acc[i][r] + scn[buf * kTile + row];
+        if (PASS == 1) {
+          best = fmaxf(best, v);  // NaN scores are ignored here and never pass the threshold
+        } else {
+          hits |= (v >= limit) ? (1u << (i * 16 + r)) : 0u;
         }
       }
-      if (PASS == 2 && hits != 0) {
-        const uint32_t n    = __popc(hits);
-        uint32_t slot       = atomicAdd(&cand_count[q], n);
-        while (hits != 0) {
-          const uint32_t bit = __builtin_ctz(hits);
-          hits &= hits - 1u;
-          const uint32_t row = wl * 64u + (bit >> 4) * 32u + (lane >> 5) * 4u + ((bit & 15u) >> 2) * 8u + (bit & 3u);
-          if (slot < kCandCapF) { cand[uint64_t(q) * kCandCapF + slot] = l0 + row; }
-          slot++;
-        }
+      if (PASS == 1) {
+        lmin[qloc * (kTilesPerBlock * 8u) + (tile - t0) * 8u + ((wl * 64u + i * 32u) >> 4) + (lane >> 5)] = alpha * best;
       }
     }
+    if (PASS == 2 && hits != 0) {
+      uint32_t slot = atomicAdd(&lcount[qloc], uint32_t(__popc(hits)));
+      while (hits != 0) {
+        const uint32_t bit = __builtin_ctz(hits);
+        hits &= hits - 1u;
+        const uint32_t row = wl * 64u + (bit >> 4) * 32u + (lane >> 5) * 4u + ((bit & 15u) >> 2) * 8u + (bit & 3u);
+        if (slot < kLocalCap) { lcand[qloc * kLocalCap + slot] = l0 + row; }
+        slot++;
+      }
+    }
+  };
 
-    // the staged tile has arrived
-    if constexpr (PER_T == 8) {
-      asm volatile("s_waitcnt vmcnt(0)"
-                   : "+v"(stage[0]), "+v"(stage[1]), "+v"(stage[2]), "+v"(stage[3]), "+v"(stage[4]),
-                     "+v"(stage[5]), "+v"(stage[6]), "+v"(stage[7]), "+v"(stage_cn)
-                   :
-                   : "memory");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0)"
-                   : "+v"(stage[0]), "+v"(stage[1]), "+v"(stage[2]), "+v"(stage[3]), "+v"(stage_cn)
-                   :
-                   : "memory");
-    }
-    unsigned char* san = sa0 + (buf ^ 1u) * (kTile * ROWB);
-#pragma unroll
-    for (uint32_t c = 0; c < PER_T; c++) {
-      *reinterpret_cast<u32x4*>(san + crow[c] * ROWB + cpart[c] * 16u) = stage[c];
-    }
-    if (tid < kTile) { scn[(buf ^ 1u) * kTile + tid] = nl < n_lists ? stage_cn * qterm : neg_inf; }
+  for (uint32_t tile = t0; tile < t1; tile++) {
+    const uint32_t buf = (tile - t0) & 1u;
+    issue(tile + 1u, sx, cx);
+    multiply(tile, buf);
+    arrived(sx, cx);
+    commit(tile + 1u, buf ^ 1u, sx, cx);
     __syncthreads();
+  }
+
+  if (PASS == 1) {
+    // the block's minima, 8 per tile and query, in runs of consecutive groups
+    const uint32_t n_local = (t1 - t0) * 8u;
+    for (uint32_t e = tid; e < kTile * n_local; e += kGemmThreads) {
+      const uint32_t ql = e / n_local, g = e - ql * n_local;
+      if (q0 + ql < n_queries) {
+        minima[uint64_t(q0 + ql) * n_groups + t0 * 8u + g] = lmin[ql * (kTilesPerBlock * 8u) + g];
+      }
+    }
+  }
+  if (PASS == 2 && tid < kTile && q0 + tid < n_queries) {
+    const uint32_t n = lcount[tid];
+    if (n != 0) {
+      // more than the block can hold: push the query's count past the limit, it will be redone by
+      // the plain path
+      const uint32_t claim = n <= kLocalCap ? n : kCandCapF + 1u;
+      const uint32_t base  = atomicAdd(&cand_count[q0 + tid], claim);
+      if (n <= kLocalCap) {
+        for (uint32_t e = 0; e < n; e++) {
+          if (base + e < kCandCapF) { cand[uint64_t(q0 + tid) * kCandCapF + base + e] = lcand[tid * kLocalCap + e]; }
+        }
+      }
+    }
   }
 }
 
@@ -422,10 +449,17 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
   const float n_terms = float(a.dim + 4);
   const float two11 = 1.0f / 2048.0f, two24 = 1.0f / 16777216.0f;
   const float abs_alpha = a.ip_like ? 1.0f : 2.0f;
-  const float e_rel = 1.05f * abs_alpha * ((two11 + 9.0f * n_terms * two24) * a.c_max + sqrtf(float(a.dim)) * two24 * 0.5f);
-  const float e_abs = 1.05f * abs_alpha * n_terms * two24 * 0.5f * a.n_max;
+  // float32 queries are rounded to binary16 too: a second relative 2^-11 (and the product of the
+  // two), and 2^-25 per element of a centre below binary16's normal range
+  const bool rounded_q = a.type == elem_type::f32;
+  const float q_round  = rounded_q ? two11 * 1.001f : 0.0f;
+  const float e_rel = 1.05f * abs_alpha * ((two11 + q_round + 9.0f * n_terms * two24) * a.c_max + sqrtf(float(a.dim)) * two24 * 0.5f);
+  const float e_abs = 1.05f * abs_alpha * (n_terms * two24 * 0.5f * a.n_max + (rounded_q ? sqrtf(float(a.dim)) * two24 * 0.5f * a.c_max : 0.0f));
 
   switch (a.type) {
+    case elem_type::f32:
+      pack_queries_kernel<float><<<q_pad, 64, 0, stream>>>(static_cast<const float*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm);
+      break;
     case elem_type::f16:
       pack_queries_kernel<_Float16><<<q_pad, 64, 0, stream>>>(static_cast<const _Float16*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm);
       break;
@@ -435,30 +469,29 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
     case elem_type::u8:
       pack_queries_kernel<uint8_t><<<q_pad, 64, 0, stream>>>(static_cast<const uint8_t*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm);
       break;
-    default: fail("the two-precision probe selection takes float16, int8 or uint8 queries");
   }
   CUVS_HIP_TRY(hipGetLastError());
 
   // list tiles per block: the queries of a block are loaded once for all of them
   const uint32_t n_list_tiles    = l_pad / kTile;
-  const uint32_t tiles_per_block = std::min<uint32_t>(8u, n_list_tiles);
+  const uint32_t tiles_per_block = std::min<uint32_t>(kTilesPerBlock, n_list_tiles);
   dim3 grid((n_list_tiles + tiles_per_block - 1) / tiles_per_block, q_pad / kTile);
   auto run_pass = [&](auto k1, auto k2) {
-    const size_t smem = size_t(3) * kTile * (k_pad * 2 + 16) + 2 * kTile * 4;
+    const size_t smem = size_t(2) * kTile * (k_pad * 2 + 16) + 2 * kTile * 4 + size_t(kTile) * kTilesPerBlock * 8 * 4;
     static bool attr_set = false;
     if (!attr_set) {
       CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k1), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
       CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k2), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
       attr_set = true;
     }
-    k1<<<grid, 256, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, n_list_tiles, tiles_per_block, alpha,
+    k1<<<grid, kGemmThreads, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, n_list_tiles, tiles_per_block, alpha,
                                     qterm, a.minima, n_groups, nullptr, nullptr, nullptr);
     CUVS_HIP_TRY(hipGetLastError());
     coarse_threshold_kernel<<<(a.n_queries + 3) / 4, 256, 0, stream>>>(a.minima, a.n_queries, n_groups, a.n_probes, a.qnorm, e_rel, e_abs, a.thr);
     CUVS_HIP_TRY(hipGetLastError());
     launch_fill_u32(a.cand_count, 0, q_pad, stream);
     launch_fill_u32(reinterpret_cast<uint32_t*>(a.fallback), 0, (a.n_queries + 3) / 4, stream);
-    k2<<<grid, 256, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, n_list_tiles, tiles_per_block, alpha,
+    k2<<<grid, kGemmThreads, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, n_list_tiles, tiles_per_block, alpha,
                                     qterm, nullptr, n_groups, a.thr, a.cand_count, a.cand);
     CUVS_HIP_TRY(hipGetLastError());
   };
@@ -472,6 +505,10 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
   const size_t xsmem = size_t(a.dim) * 4;
   CUVS_EXPECTS(rsmem <= 48 * 1024, "dim (%u) is too large for the two-precision probe selection", a.dim);
   switch (a.type) {
+    case elem_type::f32:
+      coarse_rescore_kernel<float><<<a.n_queries, 256, rsmem, stream>>>(static_cast<const float*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
+      coarse_exact_rows_kernel<float><<<a.n_queries, 256, xsmem, stream>>>(static_cast<const float*>(a.queries), a.centers, a.n_lists, a.dim, a.dim_ext, qterm, alpha, a.fallback, a.scores);
+      break;
     case elem_type::f16:
       coarse_rescore_kernel<_Float16><<<a.n_queries, 256, rsmem, stream>>>(static_cast<const _Float16*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
       coarse_exact_rows_kernel<_Float16><<<a.n_queries, 256, xsmem, stream>>>(static_cast<const _Float16*>(a.queries), a.centers, a.n_lists, a.dim, a.dim_ext, qterm, alpha, a.fallback, a.scores);

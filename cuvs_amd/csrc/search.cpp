@@ -232,7 +232,8 @@ bool coarse_plain_forced()
 bool coarse_fast_applies(const search_params& params, const index_impl& ix, elem_type type,
                          uint32_t n_probes)
 {
-  return !coarse_plain_forced() && ix.coarse_fast_ok && type != elem_type::f32 &&
+  (void)type;
+  return !coarse_plain_forced() && ix.coarse_fast_ok &&
          params.coarse_search_dtype == CUDA_R_32F && n_probes <= detail::coarse_fast_cand_cap() / 2 &&
          ix.n_lists >= 1024 && ix.n_lists >= 32u * n_probes && ix.dim <= 128;
 }

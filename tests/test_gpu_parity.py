@@ -596,3 +596,81 @@ def test_refine_validation(orc):
         refine(data, G.to_dev(np.zeros((3, 4), dtype=np.float16)), cand, 2)
     with pytest.raises(ValueError):
         refine(data, q, cand, 2, metric="cosine")
+
+
+# --- probe selection in two precisions (fp16 matrix cores + exact rescoring of the candidates) ---
+
+def _coarse_model(n_lists, dim, pq_dim, seed, scale=1.0, cluster=True):
+    """A model with many lists and no training: centres drawn around a few hundred hubs (so that
+    scores near the n_probes-th best are close together), identity rotation, random codebooks."""
+    rng = np.random.default_rng(seed)
+    if cluster:
+        hubs = rng.standard_normal((max(n_lists // 16, 1), dim)).astype(np.float32)
+        centers = hubs[rng.integers(0, hubs.shape[0], n_lists)] + 0.05 * rng.standard_normal((n_lists, dim)).astype(np.float32)
+    else:
+        centers = rng.standard_normal((n_lists, dim)).astype(np.float32)
+    centers = (centers * scale).astype(np.float32)
+    ext = np.zeros((n_lists, ((dim + 1 + 7) // 8) * 8), dtype=np.float32)
+    ext[:, :dim] = centers
+    ext[:, dim] = (centers.astype(np.float64) ** 2).sum(1).astype(np.float32)
+    return {"centers": ext, "centers_rot": centers.copy(),
+            "rotation_matrix": np.eye(dim, dtype=np.float32),
+            "pq_centers": rng.standard_normal((pq_dim, dim // pq_dim, 256)).astype(np.float32)}
+
+
+@pytest.mark.parametrize("metric", ["sqeuclidean", "inner_product", "cosine"])
+@pytest.mark.parametrize("dtype,dim", [(np.float32, 96), (np.float16, 128), (np.int8, 64), (np.uint8, 40)])
+def test_two_precision_probe_selection_equals_the_fp32_path(orc, metric, dtype, dim):
+    n_lists, pq_dim = 4096, dim // 4
+    model = _coarse_model(n_lists, dim, pq_dim, 3, scale=(0.5 if dtype in (np.int8, np.uint8) else 1.0))
+    params = ivf_pq.IndexParams(n_lists=n_lists, metric=metric, pq_dim=pq_dim, pq_bits=8)
+    dev = {k: G.to_dev(v) for k, v in model.items()}
+    index = ivf_pq.build_precomputed(params, dim, dev["pq_centers"], dev["centers"], dev["centers_rot"],
+                                     dev["rotation_matrix"])
+    ix = H.oracle_index(orc, model, dim, pq_dim, 8, metric=metric)
+    rng = np.random.default_rng(8)
+    if dtype == np.uint8:
+        q = rng.integers(0, 256, (300, dim)).astype(np.uint8)
+    elif dtype == np.int8:
+        q = rng.integers(-128, 128, (300, dim)).astype(np.int8)
+    else:
+        # some queries sit on a centre, some between two
+        c = model["centers"][:, :dim]
+        q = np.concatenate([c[:100], 0.5 * (c[100:200] + c[200:300]),
+                            rng.standard_normal((100, dim)).astype(np.float32)]).astype(dtype)
+    for n_probes in (1, 20, 64, 128):
+        sp = ivf_pq.SearchParams(n_probes=n_probes)
+        got = ivf_pq.select_clusters(sp, index, G.to_dev(q)).cpu().numpy().view(np.uint32)
+        want, _ = orc.select_clusters(ix, q, n_probes)
+        assert np.array_equal(got, want), (metric, dtype, n_probes)
+
+
+def test_two_precision_probe_selection_falls_back(orc):
+    """Identical centres put hundreds of lists inside the error margin (more candidates than the
+    fast path holds), and a query with a NaN has no usable bound: both take the plain fp32 path and
+    still equal the oracle.  Centres beyond binary16's range switch the fast path off."""
+    dim, n_lists = 32, 2048
+    model = _coarse_model(n_lists, dim, 8, 4)
+    model["centers"][:600] = model["centers"][0]           # 600 identical centres
+    model["centers_rot"][:600] = model["centers_rot"][0]
+    params = ivf_pq.IndexParams(n_lists=n_lists, pq_dim=8, pq_bits=8)
+    dev = {k: G.to_dev(v) for k, v in model.items()}
+    index = ivf_pq.build_precomputed(params, dim, dev["pq_centers"], dev["centers"], dev["centers_rot"],
+                                     dev["rotation_matrix"])
+    ix = H.oracle_index(orc, model, dim, 8, 8)
+    rng = np.random.default_rng(9)
+    q = rng.standard_normal((64, dim)).astype(np.float32)
+    q[:8] = model["centers"][0, :dim] + 0.001 * rng.standard_normal((8, dim)).astype(np.float32)
+    got = ivf_pq.select_clusters(ivf_pq.SearchParams(n_probes=32), index, G.to_dev(q)).cpu().numpy().view(np.uint32)
+    want, _ = orc.select_clusters(ix, q, 32)
+    assert np.array_equal(got, want)
+    # huge centres: the fp16 copy would overflow, the index says so and the plain path runs
+    big = _coarse_model(n_lists, dim, 8, 5, scale=1e5)
+    devb = {k: G.to_dev(v) for k, v in big.items()}
+    index_b = ivf_pq.build_precomputed(params, dim, devb["pq_centers"], devb["centers"], devb["centers_rot"],
+                                       devb["rotation_matrix"])
+    ixb = H.oracle_index(orc, big, dim, 8, 8)
+    qb = (1e5 * rng.standard_normal((32, dim))).astype(np.float32)
+    got = ivf_pq.select_clusters(ivf_pq.SearchParams(n_probes=16), index_b, G.to_dev(qb)).cpu().numpy().view(np.uint32)
+    want, _ = orc.select_clusters(ixb, qb, 16)
+    assert np.array_equal(got, want)
