@@ -85,6 +85,8 @@ def main():
                                     kmeans_trainset_fraction=min(1.0, n_train / n))
         index = ivf_pq.build(params, data, resources=res)
         res.sync()
+        model = {"centers": index.centers_padded, "centers_rot": index.centers_rot,
+                 "rotation_matrix": index.rotation_matrix, "pq_centers": index.pq_centers}
         log(f"index trained on ~{n_train} rows and populated ({len(index)} rows) in {time.time() - t0:.1f}s")
     else:
         t0 = time.time()
