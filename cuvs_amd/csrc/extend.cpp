@@ -134,6 +134,13 @@ void extend(cuvs::resources const& res,
   if (labels_in != nullptr) {
     CUVS_HIP_TRY(hipMemcpyAsync(labels.ptr, labels_in, n_rows * sizeof(uint32_t),
                                 hipMemcpyDefault, s));
+  } else if (ix.metric != detail::DistanceType::InnerProduct && is_device_pointer(new_vectors)) {
+    // the nearest list under the index's own metric is the search path's coarse stage with one
+    // probe (for cosine the row's length does not change which centre has the largest product)
+    search_params sp;
+    sp.n_probes = 1;
+    select_clusters(res, sp, *idx, new_vectors, type, n_rows_signed, labels.as<uint32_t>());
+    CUVS_HIP_TRY(hipStreamSynchronize(s));
   } else {
     const uint64_t label_chunk = chunk_rows_for(ix, n_rows);
     row_stager label_stager(new_vectors, type, ix.dim, label_chunk);
