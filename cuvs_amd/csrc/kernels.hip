@@ -450,30 +450,54 @@ __global__ void pair_histogram_kernel(const uint32_t* __restrict__ probes, uint3
   if (i < n_pairs) { atomicAdd(&counts[pair_bin(probes[i], i, n_probes, lead_probes, n_lists)], 1u); }
 }
 
-/** Single block of 1024 threads: cursors[l] = exclusive prefix sum of counts[l].  Thread t owns
- *  the contiguous range [t * per, (t + 1) * per). */
+/** Single block of 1024 threads: cursors[l] = exclusive prefix sum of counts[l].  The counts pass
+ *  through LDS in tiles of 32 per thread: loads and stores are coalesced, and a thread scans its 32
+ *  consecutive values out of LDS (one padding word per 32 keeps the threads on different banks). */
 constexpr uint32_t kScanThreads = 1024;
+constexpr uint32_t kScanPer     = 32;
+constexpr uint32_t kScanTile    = kScanThreads * kScanPer;
 __global__ __launch_bounds__(kScanThreads) void exclusive_scan_kernel(const uint32_t* __restrict__ counts,
                                                                       uint32_t n,
                                                                       uint32_t* __restrict__ cursors)
 {
+  extern __shared__ __align__(16) uint32_t tile[];  // kScanTile + kScanThreads words
   __shared__ uint32_t wave_sums[kScanThreads / 64];
   const uint32_t tid = threadIdx.x;
-  const uint32_t per = (n + kScanThreads - 1u) / kScanThreads;
-  const uint32_t lo  = tid * per;
-  const uint32_t hi  = lo + per < n ? lo + per : n;
-  uint32_t sum       = 0;
-  for (uint32_t i = lo; i < hi; i++) { sum += counts[i]; }
-  uint32_t incl = wave_inclusive_scan(sum);
-  if ((tid & 63u) == 63u) { wave_sums[tid >> 6] = incl; }
-  __syncthreads();
-  uint32_t base = 0;
-  for (uint32_t w = 0; w < (tid >> 6); w++) { base += wave_sums[w]; }
-  uint32_t run = base + incl - sum;
-  for (uint32_t i = lo; i < hi; i++) {
-    const uint32_t v = counts[i];
-    cursors[i]       = run;
-    run += v;
+  auto slot          = [](uint32_t i) { return i + (i >> 5); };
+  uint32_t carry     = 0;
+  for (uint32_t base = 0; base < n; base += kScanTile) {
+    for (uint32_t i = tid; i < kScanTile; i += kScanThreads) {
+      tile[slot(i)] = base + i < n ? counts[base + i] : 0u;
+    }
+    __syncthreads();
+    uint32_t v[kScanPer];
+    uint32_t sum = 0;
+#pragma unroll
+    for (uint32_t e = 0; e < kScanPer; e++) {
+      v[e] = tile[slot(tid * kScanPer + e)];
+      sum += v[e];
+    }
+    const uint32_t incl = wave_inclusive_scan(sum);
+    if ((tid & 63u) == 63u) { wave_sums[tid >> 6] = incl; }
+    __syncthreads();
+    uint32_t run = carry + incl - sum;
+    uint32_t all = 0;
+    for (uint32_t w = 0; w < kScanThreads / 64; w++) {
+      const uint32_t ws = wave_sums[w];
+      run += w < (tid >> 6) ? ws : 0u;
+      all += ws;
+    }
+#pragma unroll
+    for (uint32_t e = 0; e < kScanPer; e++) {
+      tile[slot(tid * kScanPer + e)] = run;
+      run += v[e];
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < kScanTile; i += kScanThreads) {
+      if (base + i < n) { cursors[base + i] = tile[slot(i)]; }
+    }
+    carry += all;
+    __syncthreads();  // the tile and the wave sums are reused
   }
 }
 
@@ -792,9 +816,29 @@ __global__ __launch_bounds__(kBlock) void merge_kernel(merge_args a, uint32_t ou
       }
       __syncthreads();
       const uint32_t n_keys = n_live * kpp;
-      block_select_sorted(
-        [keys, kpp](uint32_t i) { return keys[uint32_t(live_slots[i / kpp]) * kpp + i % kpp]; },
-        n_keys, a.k, out, out_cap, sm);
+      constexpr uint32_t kSmall = 512;
+      if (n_keys <= kSmall) {
+        // a handful of live pairs (the usual case after screening): rank every key against all
+        // others in LDS; keys are distinct (the sample number is part of the key)
+        __shared__ unsigned long long small_keys[kSmall];
+        for (uint32_t i = threadIdx.x; i < n_keys; i += kBlock) {
+          small_keys[i] = keys[uint32_t(live_slots[i / kpp]) * kpp + i % kpp];
+        }
+        for (uint32_t r = threadIdx.x; r < a.k; r += kBlock) { out[r] = kInvalidKey; }
+        __syncthreads();
+        for (uint32_t i = threadIdx.x; i < n_keys; i += kBlock) {
+          const unsigned long long key = small_keys[i];
+          if (key == kInvalidKey) { continue; }
+          uint32_t rank = 0;
+          for (uint32_t j = 0; j < n_keys; j++) { rank += small_keys[j] < key ? 1u : 0u; }
+          if (rank < a.k) { out[rank] = key; }
+        }
+        __syncthreads();
+      } else {
+        block_select_sorted(
+          [keys, kpp](uint32_t i) { return keys[uint32_t(live_slots[i / kpp]) * kpp + i % kpp]; },
+          n_keys, a.k, out, out_cap, sm);
+      }
     }
   } else {
     n                = a.n_samples[q];
@@ -1167,7 +1211,16 @@ void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
                                                                         lead_probes, n_lists, counts);
     CUVS_LAUNCH_CHECK();
   }
-  exclusive_scan_kernel<<<1, kScanThreads, 0, stream>>>(counts, n_bins, cursors);
+  {
+    const size_t smem = size_t(kScanTile + kScanThreads) * 4;
+    static bool attr_set = false;
+    if (!attr_set) {
+      CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(exclusive_scan_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+      attr_set = true;
+    }
+    exclusive_scan_kernel<<<1, kScanThreads, smem, stream>>>(counts, n_bins, cursors);
+  }
   CUVS_LAUNCH_CHECK();
   pair_scatter_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(
     probes, chunk_indices, data_ptrs, inds_ptrs, ids_base, n_pairs, n_probes, lead_probes, n_lists,
