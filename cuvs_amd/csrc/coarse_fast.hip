@@ -57,10 +57,16 @@ __device__ __forceinline__ float map_elem<uint8_t>(uint8_t v) { return float(v) 
  *  unrounded values: float32 queries are the one type that binary16 does not hold exactly). */
 template <typename T>
 __global__ void pack_queries_kernel(const T* __restrict__ in, uint32_t n_queries, uint32_t dim,
-                                    uint32_t k_pad, _Float16* __restrict__ qh, float* __restrict__ qnorm)
+                                    uint32_t k_pad, _Float16* __restrict__ qh, float* __restrict__ qnorm,
+                                    uint32_t* __restrict__ cand_count, uint8_t* __restrict__ fallback)
 {
   const uint32_t q    = blockIdx.x;
   const uint32_t lane = threadIdx.x;
+  if (lane == 0) {
+    // also start the query's candidate count and fall-back flag at zero
+    cand_count[q] = 0;
+    if (q < n_queries) { fallback[q] = 0; }
+  }
   float ss            = 0.0f;
   for (uint32_t d = lane; d < k_pad; d += 64) {
     float v = 0.0f;
@@ -378,9 +384,17 @@ __global__ __launch_bounds__(256) void coarse_rescore_kernel(
   unsigned long long key = kInvalidKey;
   if (tid < n) {
     const uint32_t l = cand[uint64_t(q) * kCandCapF + tid];
-    const float* c   = centers + uint64_t(l) * dim_ext;
+    const float* c   = centers + uint64_t(l) * dim_ext;  // rows are 32-byte aligned (dim_ext % 8 == 0)
     float acc        = 0.0f;
-    for (uint32_t d = 0; d < dim; d++) { acc = fmaf(c[d], qf[d], acc); }
+    const uint32_t dim4 = dim & ~3u;
+    for (uint32_t d = 0; d < dim4; d += 4) {
+      const float4 v = *reinterpret_cast<const float4*>(c + d);
+      acc            = fmaf(v.x, qf[d], acc);
+      acc            = fmaf(v.y, qf[d + 1], acc);
+      acc            = fmaf(v.z, qf[d + 2], acc);
+      acc            = fmaf(v.w, qf[d + 3], acc);
+    }
+    for (uint32_t d = dim4; d < dim; d++) { acc = fmaf(c[d], qf[d], acc); }
     acc           = fmaf(c[dim], qterm, acc);
     const float s = alpha * acc;
     key = (s != s) ? kInvalidKey : ((static_cast<unsigned long long>(order_f32(s)) << 32) | l);
@@ -458,16 +472,16 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
 
   switch (a.type) {
     case elem_type::f32:
-      pack_queries_kernel<float><<<q_pad, 64, 0, stream>>>(static_cast<const float*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm);
+      pack_queries_kernel<float><<<q_pad, 64, 0, stream>>>(static_cast<const float*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm, a.cand_count, a.fallback);
       break;
     case elem_type::f16:
-      pack_queries_kernel<_Float16><<<q_pad, 64, 0, stream>>>(static_cast<const _Float16*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm);
+      pack_queries_kernel<_Float16><<<q_pad, 64, 0, stream>>>(static_cast<const _Float16*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm, a.cand_count, a.fallback);
       break;
     case elem_type::i8:
-      pack_queries_kernel<int8_t><<<q_pad, 64, 0, stream>>>(static_cast<const int8_t*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm);
+      pack_queries_kernel<int8_t><<<q_pad, 64, 0, stream>>>(static_cast<const int8_t*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm, a.cand_count, a.fallback);
       break;
     case elem_type::u8:
-      pack_queries_kernel<uint8_t><<<q_pad, 64, 0, stream>>>(static_cast<const uint8_t*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm);
+      pack_queries_kernel<uint8_t><<<q_pad, 64, 0, stream>>>(static_cast<const uint8_t*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm, a.cand_count, a.fallback);
       break;
   }
   CUVS_HIP_TRY(hipGetLastError());
@@ -489,8 +503,6 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
     CUVS_HIP_TRY(hipGetLastError());
     coarse_threshold_kernel<<<(a.n_queries + 3) / 4, 256, 0, stream>>>(a.minima, a.n_queries, n_groups, a.n_probes, a.qnorm, e_rel, e_abs, a.thr);
     CUVS_HIP_TRY(hipGetLastError());
-    launch_fill_u32(a.cand_count, 0, q_pad, stream);
-    launch_fill_u32(reinterpret_cast<uint32_t*>(a.fallback), 0, (a.n_queries + 3) / 4, stream);
     k2<<<grid, kGemmThreads, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, n_list_tiles, tiles_per_block, alpha,
                                     qterm, nullptr, n_groups, a.thr, a.cand_count, a.cand);
     CUVS_HIP_TRY(hipGetLastError());
