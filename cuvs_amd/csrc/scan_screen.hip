@@ -21,6 +21,7 @@
 #include "device_utils.cuh"
 
 #include <algorithm>
+#include <cstddef>
 #include <cstdlib>
 
 namespace cuvs::neighbors::ivf_pq::detail {
@@ -54,6 +55,55 @@ __device__ __forceinline__ float opaque_one_s()
   return one;
 }
 
+/*
+ * Surviving pairs are appended to one list shared by the whole grid.  One atomic add per pair on
+ * its counter would serialise every wave of the grid on a single address (about 11 ns per add,
+ * which bounds the kernel as soon as most pairs survive), so a wave collects up to
+ * kSurvivorBatch records in an LDS area of its own and claims their slots with one add.
+ * A record is 8 dwords: a full batch is one dword per lane.
+ */
+constexpr uint32_t kSurvivorBatch      = 8;
+constexpr uint32_t kSurvivorBatchBytes = kSurvivorBatch * uint32_t(sizeof(pair_desc));
+static_assert(kSurvivorBatchBytes == 64 * 4, "a full batch is one dword per lane");
+static_assert(offsetof(pair_desc, q) == 8 && offsetof(pair_desc, row_off) == 28, "record layout");
+
+__device__ __forceinline__ void flush_survivors(LDS_AS uint32_t* pending, uint32_t n, uint32_t lane,
+                                                pair_desc* __restrict__ survivors,
+                                                uint32_t* __restrict__ n_survivors)
+{
+  uint32_t pos = 0;
+  if (lane == 0) { pos = atomicAdd(n_survivors, n); }
+  pos = uint32_t(__builtin_amdgcn_readfirstlane(pos));
+  if (lane < n * 8u) { reinterpret_cast<uint32_t*>(survivors + pos)[lane] = pending[lane]; }
+}
+
+/** Adds a record to the wave's batch (all lanes call it; `n` is the same in all of them). */
+__device__ __forceinline__ void push_survivor(LDS_AS uint32_t* pending, uint32_t& n, uint32_t lane,
+                                              const pair_desc& d, pair_desc* __restrict__ survivors,
+                                              uint32_t* __restrict__ n_survivors,
+                                              uint8_t* __restrict__ alive)
+{
+  if (lane == 0) {
+    // the record's eight dwords in memory order
+    const uint64_t ptr   = reinterpret_cast<uint64_t>(d.data);
+    LDS_AS uint32_t* dst = pending + n * 8u;
+    dst[0]               = uint32_t(ptr);
+    dst[1]               = uint32_t(ptr >> 32);
+    dst[2]               = d.q;
+    dst[3]               = d.slot;
+    dst[4]               = d.label;
+    dst[5]               = d.sample_off;
+    dst[6]               = d.n_rows;
+    dst[7]               = d.row_off;
+    alive[d.slot]        = 1;
+  }
+  n++;
+  if (n == kSurvivorBatch) {
+    flush_survivors(pending, n, lane, survivors, n_survivors);
+    n = 0;
+  }
+}
+
 /** How many leading subspaces the screen sums (of the 16 in the first chunk): 8, or 4 / 16 for A/B runs. */
 inline int screen_subspaces()
 {
@@ -80,6 +130,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   constexpr uint32_t lut_entries = SUB * 256u;
   constexpr uint32_t off_diff    = kScreenLdsBase + G * lut_entries * uint32_t(sizeof(lut_t));
   static_assert(G * NDIFF <= kScreenThreads, "one thread stages one (pair, dimension)");
+  constexpr uint32_t off_pending = off_diff + G * NDIFF * 4u;
   auto* lut_all  = reinterpret_cast<LDS_AS lut_t*>(uintptr_t(kScreenLdsBase));
   auto* diff_all = reinterpret_cast<LDS_AS float*>(uintptr_t(off_diff));
   const float one = opaque_one_s();
@@ -91,6 +142,8 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   const uint32_t stride  = gridDim.x;
   if (blockIdx.x >= n_iters) { return; }
   auto* my_lut = lut_all + wid * lut_entries;
+  auto* pending = reinterpret_cast<LDS_AS uint32_t*>(uintptr_t(off_pending + wid * kSurvivorBatchBytes));
+  uint32_t n_pending = 0;
 
   float book[PER_CLUSTER ? 1 : SUB][PQ_LEN];
   if (!PER_CLUSTER) {
@@ -226,13 +279,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
         }
         cur     = ahead;
       }
-      if (lane == 0) {
-        if (in_play) {
-          const uint32_t pos = atomicAdd(n_survivors, 1u);
-          survivors[pos]     = my_d;
-          alive[my_d.slot]   = 1;
-        }
-      }
+      if (in_play) { push_survivor(pending, n_pending, lane, my_d, survivors, n_survivors, alive); }
     }
 
     if (!has_next) { break; }
@@ -245,6 +292,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
     it = nxt_it;
     lds_barrier_s();  // every wave is done with the tables; next staged terms are visible
   }
+  if (n_pending != 0) { flush_survivors(pending, n_pending, lane, survivors, n_survivors); }
 }
 
 /*
@@ -287,6 +335,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   static_assert(NDIFF <= 64, "one lane per leading rotated dimension");
   auto* book      = reinterpret_cast<LDS_AS vec_t*>(uintptr_t(kScreenLdsBase));
   const float one = opaque_one_s();
+  constexpr uint32_t off_pending = kScreenLdsBase + SUB * 256u * PQ_LEN * 4u;
 
   const uint32_t tid  = threadIdx.x;
   const uint32_t lane = tid & 63u;
@@ -305,6 +354,8 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
 
   uint32_t p = blockIdx.x * WPB + wid;
   if (p >= n_pairs) { return; }
+  auto* pending = reinterpret_cast<LDS_AS uint32_t*>(uintptr_t(off_pending + wid * kSurvivorBatchBytes));
+  uint32_t n_pending = 0;
 
   // A record is fetched two pairs ahead with a vector load (index hidden from the uniformity
   // analysis): a scalar load would be waited for by the tile loop's first LDS read, since both
@@ -444,11 +495,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
         sum_tile(r2, tile + 2u);
         if (in_play) { break; }
       }
-      if (in_play && lane == 0) {
-        const uint32_t pos = atomicAdd(n_survivors, 1u);
-        survivors[pos]     = d0;
-        alive[d0.slot]     = 1;
-      }
+      if (in_play) { push_survivor(pending, n_pending, lane, d0, survivors, n_survivors, alive); }
     }
 
     if (!has1) { break; }
@@ -460,6 +507,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
     thr0  = thr1;
     dv0   = dv1;
   }
+  if (n_pending != 0) { flush_survivors(pending, n_pending, lane, survivors, n_survivors); }
 }
 
 /** Which subspace count the first check of the table-free screen follows (1, 2 or 4). */
@@ -488,7 +536,8 @@ void launch_screen_direct_first(const scan_args& a, const pair_desc* desc, uint3
                                 hipStream_t stream)
 {
   auto kernel       = scan_screen_direct_kernel<PQ_LEN, LUT, OUT_HALF, FIRST>;
-  const size_t smem = kScreenLdsBase + size_t(kDirectSubs) * 256 * PQ_LEN * 4;
+  const size_t smem = kScreenLdsBase + size_t(kDirectSubs) * 256 * PQ_LEN * 4 +
+                      size_t(kDirectThreads / 64u) * kSurvivorBatchBytes;
   static int n_cu = 0, per_cu = 0;  // per instance
   if (n_cu == 0) {
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -531,7 +580,7 @@ void launch_screen_sub(const scan_args& a, const pair_desc* desc, uint32_t n_pai
   using lut_t       = typename lut_traits<LUT>::storage;
   auto kernel       = scan_screen_kernel<SUBS, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>;
   const size_t smem = kScreenLdsBase + size_t(kScreenG) * SUBS * 256 * sizeof(lut_t) +
-                      size_t(kScreenG) * SUBS * PQ_LEN * 4;
+                      size_t(kScreenG) * SUBS * PQ_LEN * 4 + size_t(kScreenG) * kSurvivorBatchBytes;
   static int n_cu = 0, per_cu = 0;  // per instance
   if (n_cu == 0) {
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),

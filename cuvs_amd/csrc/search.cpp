@@ -227,15 +227,17 @@ bool coarse_plain_forced()
   return forced;
 }
 
-/** The two-precision probe selection applies to element types that binary16 holds exactly, to
- *  fp32 coarse search, and to shapes where its candidate lists stay short. */
+/** The two-precision probe selection applies to fp32 coarse search and to shapes where its
+ *  candidate lists stay short: about 1.4 n_probes lists per query pass the threshold, and a
+ *  workgroup of the candidate pass (512 lists) holds at most 32 of them per query before the query
+ *  falls back to the plain path, so n_lists >= 64 n_probes keeps the expected load near 11. */
 bool coarse_fast_applies(const search_params& params, const index_impl& ix, elem_type type,
                          uint32_t n_probes)
 {
   (void)type;
   return !coarse_plain_forced() && ix.coarse_fast_ok &&
          params.coarse_search_dtype == CUDA_R_32F && n_probes <= detail::coarse_fast_cand_cap() / 2 &&
-         ix.n_lists >= 1024 && ix.n_lists >= 32u * n_probes && ix.dim <= 128;
+         ix.n_lists >= 1024 && ix.n_lists >= 64u * n_probes && ix.dim <= 128;
 }
 
 /** Workspace bytes of the two-precision selection for a batch, and its allocation. */
