@@ -316,6 +316,11 @@ constexpr uint64_t kLeadPlaneSlack = 512;  // slots past the last list that look
  *  arguments are outside what it covers.  Needs `a.desc`. */
 bool scan_fast_supported(const scan_args& a);
 bool launch_scan_fast(const scan_args& a, hipStream_t stream);
+
+/** The 4-bit variant of the block kernel (pq_bits = 4, pq_dim a multiple of 32; scan_nibble.hip):
+ *  same records, candidate keys and bound updates. */
+bool scan_nibble_supported(const scan_args& a);
+bool launch_scan_nibble(const scan_args& a, hipStream_t stream);
 /** CU-wide kernel for 8-bit codes, k <= 64 and fp16 / 8-bit tables (scan_quad.hip).  It writes
  *  several candidate groups per pair: scan_quad_keys_per_pair() is the number of keys the output
  *  buffer must hold per (query, probe) pair, 0 when the arguments are outside what it covers. */

@@ -448,7 +448,8 @@ void search(cuvs::resources const& res_c,
   if (global_lut) { sa.global_lut = res.workspace_alloc(global_lut_bytes); }
   const bool generic_only  = force_generic_scan() || global_lut;
   const uint32_t quad_kpp  = generic_only ? 0u : detail::scan_quad_keys_per_pair(sa);
-  const bool fast_scan     = !generic_only && (quad_kpp != 0 || detail::scan_fast_supported(sa));
+  const bool nibble_scan   = !generic_only && detail::scan_nibble_supported(sa);
+  const bool fast_scan     = !generic_only && (quad_kpp != 0 || detail::scan_fast_supported(sa) || nibble_scan);
   const uint32_t kpp       = quad_kpp != 0 ? quad_kpp : k;  // candidate keys stored per pair
   if (fast_scan) {
     desc = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));
@@ -543,7 +544,8 @@ void search(cuvs::resources const& res_c,
       sa.n_pairs_dev = n_survivors;
       CUVS_EXPECTS(full_scan(), "scan kernel launch failed");
     } else {
-      const bool launched = fast_scan && (quad_kpp != 0 ? detail::launch_scan_quad(sa, s)
+      const bool launched = fast_scan && (quad_kpp != 0   ? detail::launch_scan_quad(sa, s)
+                                          : nibble_scan ? detail::launch_scan_nibble(sa, s)
                                                         : detail::launch_scan_fast(sa, s));
       if (!launched) { detail::launch_scan(sa, s); }
     }

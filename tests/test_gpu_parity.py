@@ -359,15 +359,17 @@ def test_early_stop_matches_oracle_and_full_scan(orc, monkeypatch, lut, internal
         assert torch.equal(nb, nb2) and torch.equal(d, d2)
 
 
-def test_early_stop_pq_len_4(orc):
-    """Four dimensions per subspace: 16-byte codebook entries in the table-free screen."""
+@pytest.mark.parametrize("kind", ["subspace", "cluster"])
+def test_early_stop_pq_len_4(orc, kind):
+    """Four dimensions per subspace: 16-byte codebook entries in the table-free screen (shared by
+    the block for per-subspace codebooks, one list's codebook per wave for per-cluster ones)."""
     from cuvs_amd import testing
     from cuvs_amd.resources import Resources
     allrows = testing.gaussian_mixture(20100, 128, 64, 0.15, seed=78).numpy()
     x, q = allrows[:20000], allrows[20000:]
-    model = H.train(x, 128, 32, 8, iters=6)
-    index = G.build_gpu_index(model, x, 32, 8, "sqeuclidean", "subspace")
-    ix, _ = G.read_back(orc, index, model, 128, 32, 8, "sqeuclidean", "subspace")
+    model = H.train(x, 128, 32, 8, codebook_kind=kind, iters=6)
+    index = G.build_gpu_index(model, x, 32, 8, "sqeuclidean", kind)
+    ix, _ = G.read_back(orc, index, model, 128, 32, 8, "sqeuclidean", kind)
     res = Resources()
     res.enable_profiling(True)
     for lut in (R_16F, R_8U):
@@ -674,3 +676,53 @@ def test_two_precision_probe_selection_falls_back(orc):
     got = ivf_pq.select_clusters(ivf_pq.SearchParams(n_probes=16), index_b, G.to_dev(qb)).cpu().numpy().view(np.uint32)
     want, _ = orc.select_clusters(ixb, qb, 16)
     assert np.array_equal(got, want)
+
+
+# --- 4-bit codes: the block kernel with tables held in the accumulator's type ---
+
+_NIBBLE = {}
+
+
+def _nibble_case(orc, dim, pq_dim, metric, kind):
+    key = (dim, pq_dim, metric, kind)
+    if key not in _NIBBLE:
+        _NIBBLE[key] = _case(orc, 6000, dim, 24, pq_dim, 4, metric=metric, kind=kind, n_queries=48)
+    return _NIBBLE[key]
+
+
+@pytest.mark.parametrize("lut,internal", [(R_32F, R_32F), (R_16F, R_32F), (R_8U, R_32F), (R_16F, R_16F),
+                                          (R_8U, R_16F)])
+@pytest.mark.parametrize("dim,pq_dim,metric,kind", [
+    (128, 64, "sqeuclidean", "subspace"),    # two chunks (half a step), pq_len 2
+    (96, 96, "inner_product", "subspace"),   # three chunks: a partial step, pq_len 1
+    (128, 32, "cosine", "cluster"),          # one chunk, pq_len 4, per-cluster codebooks
+    (320, 160, "euclidean", "subspace"),     # five chunks: a full step and a partial one
+])
+def test_four_bit_block_kernel_matches_oracle(orc, lut, internal, dim, pq_dim, metric, kind):
+    data, model, queries, index, ix, _ = _nibble_case(orc, dim, pq_dim, metric, kind)
+    for k, n_probes in ((1, 3), (10, 8), (100, 24), (200, 24)):
+        nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, k, n_probes, lut=lut,
+                                              internal=internal)
+        H.compare_results(nb, d, want_nb, want_d, 1e-5 if lut == R_32F else 2e-3,
+                          exact=(metric != "euclidean"))
+
+
+def test_four_bit_block_kernel_filter_and_long_lists(orc):
+    """Lists of several thousand rows (more than one pruning segment of the candidate buffer) and a
+    bitset filter."""
+    data, model, queries, index, ix, _ = _case(orc, 40000, 64, 6, 32, 4, n_queries=24)
+    n = data.shape[0]
+    keep = np.ones(n, dtype=bool)
+    keep[::4] = False
+    bits = np.packbits(keep, bitorder="little")
+    bits = np.concatenate([bits, np.zeros((-bits.size) % 4, dtype=np.uint8)]).view(np.uint32)
+    for lut in (R_32F, R_16F, R_8U):
+        sp = ivf_pq.SearchParams(n_probes=4, lut_dtype=lut)
+        d, nb = ivf_pq.search(sp, index, G.to_dev(queries), 50,
+                              filter_bitset=G.to_dev(bits.view(np.int32)), filter_nbits=n)
+        want_nb, want_d = orc.search(ix, queries, 50, 4, lut_dtype=ORC_DT[lut], filter_bitset=bits,
+                                     filter_nbits=n)
+        H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d,
+                          1e-5 if lut == R_32F else 2e-3, exact=True)
+        nb2, d2, want_nb2, want_d2 = _search_both(orc, index, ix, queries, 128, 6, lut=lut)
+        H.compare_results(nb2, d2, want_nb2, want_d2, 1e-5 if lut == R_32F else 2e-3, exact=True)
