@@ -1,6 +1,6 @@
 """Benchmark of the IVF-PQ search path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config N]
 
 One step = one `cuvsIvfPqSearch` call over the whole query batch with the queries already in HBM.
 Workload (BASELINE.json configs[2], the configuration the metric is quoted on): 10M x 128 uint8
@@ -8,6 +8,11 @@ SIFT-like rows, n_lists = 16384, pq_dim = 64, pq_bits = 8, 10,000 queries, k = 1
 fp16 lookup table with fp32 internal distances.  Prints ONE JSON line with the QPS, recall@10, the
 roofline of the code-scan kernel and a CPU baseline (the oracle, multithreaded, on a bounded
 query sample).
+
+`--config N` (0..4) runs another of BASELINE.json's configurations at its real shape instead (same
+JSON line; the CPU baseline only with `--with-cpu`, since copying a large index to the host takes
+longer than the benchmark).  Single flags (`--probes 128`, `--k 100`, `--lut fp8`, `--queries 100`
+...) override the configuration's values.
 """
 import argparse
 import json
@@ -25,6 +30,41 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # per dispatch, each scaled by its reading for the 1 GiB calibration copy below); the counter runs
 # are summarised under profiles/.  Keyed by (kernel, lut, internal); None where not measured.
 MEASURED_TRAFFIC = {("scan_screen_direct_kernel", "f16", "f32"): 1.138e9}
+
+
+# BASELINE.json's configurations; `dataset` names the generator below
+CONFIGS = {
+    0: dict(rows=10_000, lists=64, queries=100, probes=8, dim=128, pq_dim=32, pq_bits=8, k=10, lut="f32",
+            internal="f32", metric="sqeuclidean", kind="subspace", dataset="mixture64_f32"),
+    1: dict(rows=1_000_000, lists=1024, queries=10_000, probes=32, dim=96, pq_dim=48, pq_bits=8, k=10,
+            lut="f16", internal="f32", metric="sqeuclidean", kind="subspace", dataset="unit_mixture_f32"),
+    2: dict(rows=10_000_000, lists=16384, queries=10_000, probes=64, dim=128, pq_dim=64, pq_bits=8, k=10,
+            lut="f16", internal="f32", metric="sqeuclidean", kind="subspace", dataset="sift_u8"),
+    3: dict(rows=10_000_000, lists=16384, queries=10_000, probes=64, dim=768, pq_dim=384, pq_bits=4, k=10,
+            lut="fp8", internal="f16", metric="inner_product", kind="subspace", dataset="decay_mixture_f32"),
+    4: dict(rows=100_000_000, lists=50_000, queries=10_000, probes=200, dim=96, pq_dim=48, pq_bits=8, k=10,
+            lut="f16", internal="f32", metric="sqeuclidean", kind="cluster", dataset="mixture_f16"),
+}
+
+
+def make_rows(name, n, dim, device):
+    """Synthetic rows of BASELINE.json's configurations (seeded)."""
+    import torch
+
+    from cuvs_amd import testing
+    if name == "sift_u8":
+        return testing.sift_like_u8(n, dim, 4096, seed=1234, device=device)
+    if name == "mixture64_f32":
+        return testing.gaussian_mixture(n, dim, 64, 0.3, seed=1234, device=device)
+    if name == "unit_mixture_f32":
+        return testing.gaussian_mixture(n, dim, 1000, 0.2, seed=1234, device=device, normalize_centers=True,
+                                        normalize_rows=True)
+    if name == "decay_mixture_f32":
+        return testing.gaussian_mixture(n, dim, 8192, 0.3, seed=1234, device=device, dim_decay=0.9,
+                                        normalize_rows=True)
+    if name == "mixture_f16":
+        return testing.gaussian_mixture(n, dim, 50_000, 0.25, seed=1234, device=device, dtype=torch.float16)
+    raise ValueError(name)
 
 
 def log(msg):
@@ -52,7 +92,16 @@ def main():
                     help="search refine_ratio * k candidates and re-rank them exactly (1 = off)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--with-cpu", action="store_true", help="time the CPU oracle also with --config")
+    ap.add_argument("--config", type=int, default=2, choices=sorted(CONFIGS))
+    ap.add_argument("--metric", default="sqeuclidean", choices=["sqeuclidean", "euclidean", "inner_product", "cosine"])
+    ap.add_argument("--kind", default="subspace", choices=["subspace", "cluster"])
+    ap.add_argument("--dataset", default="sift_u8")
+    first, _ = ap.parse_known_args()
+    ap.set_defaults(**CONFIGS[first.config])
     args = ap.parse_args()
+    if args.config != 2 and not args.with_cpu:
+        args.no_cpu = True
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
 
@@ -70,9 +119,11 @@ def main():
     int_np = {"f32": np.float32, "f16": np.float16}[args.internal]
 
     t0 = time.time()
-    allrows = testing.sift_like_u8(n + nq, dim, 4096, seed=1234, device=dev)
+    allrows = make_rows(args.dataset, n + nq, dim, dev)
     data, queries = allrows[:n], allrows[n:].contiguous()
-    log(f"data {tuple(data.shape)} uint8 generated in {time.time() - t0:.1f}s")
+    torch.cuda.synchronize()
+    log(f"data {tuple(data.shape)} {str(data.dtype).replace('torch.', '')} ({args.dataset}) generated in "
+        f"{time.time() - t0:.1f}s")
 
     res = Resources()
     res.use_torch_current_stream()
@@ -81,7 +132,8 @@ def main():
         # the library's own training (cuvsIvfPqBuild) on a subsample of n_train rows, then every row
         # encoded and added (add_data_on_build)
         t0 = time.time()
-        params = ivf_pq.IndexParams(n_lists=n_lists, pq_bits=pq_bits, pq_dim=pq_dim,
+        params = ivf_pq.IndexParams(n_lists=n_lists, metric=args.metric, pq_bits=pq_bits, pq_dim=pq_dim,
+                                    codebook_kind=args.kind,
                                     kmeans_trainset_fraction=min(1.0, n_train / n))
         index = ivf_pq.build(params, data, resources=res)
         res.sync()
@@ -89,6 +141,8 @@ def main():
                  "rotation_matrix": index.rotation_matrix, "pq_centers": index.pq_centers}
         log(f"index trained on ~{n_train} rows and populated ({len(index)} rows) in {time.time() - t0:.1f}s")
     else:
+        assert (args.metric, args.kind, args.dataset) == ("sqeuclidean", "subspace", "sift_u8"), \
+            "--build torch covers the default workload only"
         t0 = time.time()
         g = torch.Generator(device="cpu")
         g.manual_seed(137)
@@ -112,7 +166,7 @@ def main():
         log(f"index populated ({len(index)} rows) in {time.time() - t0:.1f}s")
 
     t0 = time.time()
-    truth = testing.exact_knn(data, queries, k).cpu().numpy()  # fp32: exact for 8-bit data
+    truth = testing.exact_knn(data, queries, k, metric=args.metric).cpu().numpy()  # fp32: exact for 8-bit data
     log(f"exact ground truth in {time.time() - t0:.1f}s")
 
     sp = ivf_pq.SearchParams(n_probes=P, lut_dtype=lut_np, internal_distance_dtype=int_np,
@@ -127,8 +181,8 @@ def main():
         ivf_pq.search(sp, index, queries, k_search, neighbors=neighbors, distances=distances,
                       resources=res)
         if args.refine_ratio > 1:
-            refine(data, queries, neighbors, k, indices=refined_ids, distances=refined_d,
-                   resources=res)
+            refine(data, queries, neighbors, k, metric=args.metric, indices=refined_ids,
+                   distances=refined_d, resources=res)
 
     for _ in range(args.warmup):
         step()
@@ -159,20 +213,27 @@ def main():
     scan_stage_ms = mean("scan_ms")
     bytes_all_lists = stage["scan_bytes"] / launches
     early_stop = stage["n_screened_pairs"] > 0
+    pq_len = dim // pq_dim
+    nibble = pq_bits == 4 and pq_dim % 32 == 0 and pq_len in (1, 2, 4) and (pq_dim // 16) * pq_len <= 48
+    full_name = ("scan_nibble_kernel" if nibble
+                 else "scan_kernel" if (pq_bits != 8 or (pq_dim, pq_len) not in ((64, 2), (48, 2), (32, 4)))
+                 else "scan_quad_kernel" if (args.lut != "f32" and k <= 64) else "scan_fast_kernel")
     if early_stop:
-        # the scan stage is three launches; the screening kernel is the dominant one.  Its
-        # algorithmic bytes are the leading 8 bytes (8 one-byte codes, from the packed plane of
-        # leading codes) of every (padded) row of every screened pair; per-cluster codebooks use the
-        # table-building screen, which reads the same 8 bytes from the interleaved lists.
+        # The scan stage is three launches: the leading probes' lists in full, the screen of every
+        # other pair on its leading 8 codes (8 bytes a row: from the packed plane of leading codes
+        # in the table-free screen, from the interleaved lists in the table-building screen that
+        # per-cluster codebooks use), and the surviving pairs in full.  The roofline is quoted
+        # for the longest of the three (the screen on the default workload).
+        screen_name = "scan_screen_kernel" if args.kind == "cluster" else "scan_screen_direct_kernel"
         parts = {"lead_scan": (mean("lead_scan_ms"), stage["lead_bytes"] / launches),
                  "screen": (mean("screen_ms"), stage["screen_bytes"] / launches),
                  "survivor_scan": (mean("survivor_scan_ms"), stage["survivor_bytes"] / launches)}
-        kernel_name = "scan_screen_direct_kernel"
-        kernel_ms, kernel_bytes = parts["screen"]
+        longest = max(parts, key=lambda name: parts[name][0])
+        kernel_name = screen_name if longest == "screen" else full_name
+        kernel_ms, kernel_bytes = parts[longest]
     else:
         parts = {}
-        kernel_name = ("scan_kernel" if (pq_bits != 8 or (pq_dim, dim // pq_dim) not in ((64, 2), (48, 2), (32, 4)))
-                       else "scan_quad_kernel" if (args.lut != "f32" and k <= 64) else "scan_fast_kernel")
+        kernel_name = full_name
         kernel_ms, kernel_bytes = scan_stage_ms, bytes_all_lists
     achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9
     log(f"{kernel_name} {kernel_ms:.3f} ms per launch, {kernel_bytes / 1e9:.2f} GB algorithmic "
@@ -192,20 +253,22 @@ def main():
     torch.cuda.synchronize()
     del calib, calib_out
 
-    default_workload = (n, nq, n_lists, P, k, dim, pq_dim, pq_bits) == (10_000_000, 10_000, 16384, 64, 10,
-                                                                       128, 64, 8)
+    default_workload = (args.config == 2 and (n, nq, n_lists, P, k, dim, pq_dim, pq_bits) ==
+                        (10_000_000, 10_000, 16384, 64, 10, 128, 64, 8))
     traffic = (MEASURED_TRAFFIC.get((kernel_name, args.lut, args.internal))
                if default_workload else None)
 
     out = {
-        "metric": "QPS@recall@10 (10M x 128 IVF-PQ, batch 10k); code-scan HBM GB/s vs peak",
+        "metric": ("QPS@recall@10 (10M x 128 IVF-PQ, batch 10k); code-scan HBM GB/s vs peak" if args.config == 2
+                   else f"QPS@recall@{k} ({n} x {dim} IVF-PQ, batch {nq}); code-scan HBM GB/s vs peak"),
         "value": qps, "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32" if args.internal == "f32" else "f16",
         "data": "synthetic",
-        "config": {"workload": f"configs[2]: {n} x {dim} uint8 SIFT-like, n_lists={n_lists}, "
-                               f"pq_dim={pq_dim}, pq_bits={pq_bits}, {nq} queries, k={k}, "
-                               f"n_probes={P}, lut={args.lut}, internal={args.internal}, L2",
+        "config": {"workload": f"configs[{args.config}]: {n} x {dim} {str(data.dtype).replace('torch.', '')} "
+                               f"({args.dataset}), n_lists={n_lists}, pq_dim={pq_dim}, pq_bits={pq_bits}, "
+                               f"{args.kind} codebooks, {nq} queries, k={k}, n_probes={P}, lut={args.lut}, "
+                               f"internal={args.internal}, {args.metric}",
                    "n_rows": n, "dim": dim, "n_lists": n_lists, "pq_dim": pq_dim,
                    "pq_bits": pq_bits, "n_queries": nq, "k": k, "n_probes": P,
                    "lut_dtype": args.lut, "internal_distance_dtype": args.internal,
@@ -248,7 +311,7 @@ def cpu_baseline(args, index, model, queries, truth, gpu_ids, dim, pq_dim, pq_bi
 
     t0 = time.time()
     host_model = {kk: v.cpu().numpy() for kk, v in model.items()}
-    ix = read_back_bulk(oracle, index, host_model, dim, pq_dim, pq_bits)
+    ix = G.read_back_bulk(oracle, index, host_model, dim, pq_dim, pq_bits, args.metric, args.kind)
     log(f"index copied to the host for the CPU baseline in {time.time() - t0:.1f}s")
     lut = {"f32": 0, "f16": 2, "fp8": 8}[args.lut]
     internal = {"f32": 0, "f16": 2}[args.internal]
@@ -272,29 +335,6 @@ def cpu_baseline(args, index, model, queries, truth, gpu_ids, dim, pq_dim, pq_bi
     return {"value": n_sample / dt, "unit": "queries/s", "cores": threads, "kind": "port",
             "sample": f"first {n_sample} of the {q_host.shape[0]} queries, same index and parameters",
             "oracle_recall": o_rec, "gpu_recall": g_rec, "ids_identical_frac": same}
-
-
-def read_back_bulk(oracle, index, host_model, dim, pq_dim, pq_bits):
-    """Host copy of the index for the oracle: codes via the unpack entry point, ids via the getter."""
-    import numpy as np
-
-    import gpu_helpers as G
-    import helpers as H
-
-    sizes = index.list_sizes.cpu().numpy().astype(np.uint32)
-    datas, inds = [], []
-    for l in range(len(sizes)):
-        if sizes[l] == 0:
-            datas.append(np.zeros(0, dtype=np.uint8))
-            inds.append(np.zeros(0, dtype=np.int64))
-            continue
-        flat = index.list_data(l, n_rows=int(sizes[l])).cpu().numpy()
-        codes = flat if pq_bits == 8 else G.unpack_bits(flat, pq_dim, pq_bits)
-        datas.append(oracle.pack_list(codes, pq_bits))
-        inds.append(index.list_indices(l).cpu().numpy())
-    ix = H.oracle_index(oracle, host_model, dim, pq_dim, pq_bits)
-    ix.set_lists(sizes, datas, inds)
-    return ix
 
 
 if __name__ == "__main__":

@@ -62,3 +62,22 @@ def read_back(orc, index, model, dim, pq_dim, pq_bits, metric="sqeuclidean", cod
     ix = H.oracle_index(orc, model, dim, pq_dim, pq_bits, metric, codebook_kind)
     ix.set_lists(sizes, datas, inds)
     return ix, all_codes
+
+
+def read_back_bulk(orc, index, host_model, dim, pq_dim, pq_bits, metric="sqeuclidean", codebook_kind="subspace"):
+    """read_back for large indexes: no per-list cross-checks, 8-bit codes taken as they come out of
+    the unpack entry point (one byte per code already)."""
+    sizes = index.list_sizes.cpu().numpy().astype(np.uint32)
+    datas, inds = [], []
+    for l in range(len(sizes)):
+        if sizes[l] == 0:
+            datas.append(np.zeros(0, dtype=np.uint8))
+            inds.append(np.zeros(0, dtype=np.int64))
+            continue
+        flat = index.list_data(l, n_rows=int(sizes[l])).cpu().numpy()
+        codes = flat if pq_bits == 8 else unpack_bits(flat, pq_dim, pq_bits)
+        datas.append(orc.pack_list(codes, pq_bits))
+        inds.append(index.list_indices(l).cpu().numpy())
+    ix = H.oracle_index(orc, host_model, dim, pq_dim, pq_bits, metric, codebook_kind)
+    ix.set_lists(sizes, datas, inds)
+    return ix
