@@ -245,7 +245,7 @@ void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
                         const uint8_t* const* data_ptrs, const int64_t* const* inds_ptrs,
                         const int64_t* ids_base, uint32_t n_pairs, uint32_t n_probes,
                         uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
-                        pair_desc* desc, uint32_t lead_probes, uint8_t* alive, bool counted,
+                        pair_desc* desc, uint32_t lead_probes, uint8_t* alive, bool counted, bool natural_order,
                         hipStream_t stream);
 
 struct scan_args {

@@ -514,8 +514,11 @@ __global__ void pair_scatter_kernel(const uint32_t* __restrict__ probes,
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n_pairs) {
     const uint32_t label = probes[i];
-    const uint32_t pos   = atomicAdd(&cursors[pair_bin(label, i, n_probes, lead_probes, n_lists)], 1u);
-    pair_order[pos]      = i;
+    // no cursors: the pairs keep their natural (query-major) order
+    const uint32_t pos = cursors != nullptr
+                           ? atomicAdd(&cursors[pair_bin(label, i, n_probes, lead_probes, n_lists)], 1u)
+                           : i;
+    pair_order[pos]    = i;
     if (alive != nullptr) { alive[i] = (i % n_probes) < lead_probes ? 1 : 0; }
     if (desc != nullptr) {
       const uint32_t q   = i / n_probes;
@@ -1199,9 +1202,17 @@ void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
                         const int64_t* ids_base, uint32_t n_pairs, uint32_t n_probes,
                         uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
                         pair_desc* desc, uint32_t lead_probes, uint8_t* alive, bool counted,
-                        hipStream_t stream)
+                        bool natural_order, hipStream_t stream)
 {
   if (n_pairs == 0) { return; }
+  if (natural_order) {
+    CUVS_EXPECTS(lead_probes >= n_probes, "natural pair order has no leading / other split");
+    pair_scatter_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(
+      probes, chunk_indices, data_ptrs, inds_ptrs, ids_base, n_pairs, n_probes, lead_probes, n_lists,
+      nullptr, pair_order, desc, alive);
+    CUVS_LAUNCH_CHECK();
+    return;
+  }
   const uint32_t n_bins = lead_probes < n_probes ? 2 * n_lists : n_lists;
   uint32_t* counts      = counters;
   uint32_t* cursors     = counters + n_bins;

@@ -39,6 +39,7 @@ using detail::index_impl;
 constexpr uint32_t kMaxFusedK = 256;   // larger k dumps all scores and selects afterwards
 constexpr uint32_t kMaxK      = 8192;  // bound of the per-query selection buffer in LDS
 constexpr size_t kMaxLds      = 160 * 1024;
+constexpr uint32_t kFewPairs  = 1024;  // (query, probe) pairs of a batch below which they are scanned in one plain launch
 
 /** A pointer is usable by kernels when HIP knows it as device, managed or pinned host memory
  *  (role of utils::check_pointer_residency, detail/ann_utils.cuh). */
@@ -455,9 +456,14 @@ void search(cuvs::resources const& res_c,
     desc = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));
   }
   // L2 early stop: lists of the leading probes in full, the others screened on their first chunk
+  // A batch of a few thousand pairs is over in one or two rounds of the persistent scan grid:
+  // the early stop's extra launches and the grouping of the pairs by list would cost more than
+  // they save (the reference skips the grouping when lists are rarely shared,
+  // expected_probe_coresidency, ivf_pq_search.cuh:353-373).
+  const bool few_pairs       = uint64_t(Qb) * P <= kFewPairs;
   const uint32_t kLeadProbes = lead_probes();
-  const bool early_stop = fast_scan && P > kLeadProbes && P <= 8192 && detail::scan_screen_supported(sa) &&
-                          !early_stop_disabled();
+  const bool early_stop = fast_scan && !few_pairs && P > kLeadProbes && P <= 8192 &&
+                          detail::scan_screen_supported(sa) && !early_stop_disabled();
   const uint32_t lead          = early_stop ? kLeadProbes : P;
   detail::pair_desc* survivors = nullptr;
   uint8_t* alive               = nullptr;
@@ -505,10 +511,10 @@ void search(cuvs::resources const& res_c,
                           ix.rotation_is_identity, cosine, rot_q, s);
     detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
                                  ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead,
-                                 counters, ix.n_lists, s);
+                                 few_pairs ? nullptr : counters, ix.n_lists, s);
     detail::launch_order_pairs(probes, chunk, ix.data_ptrs.as<const uint8_t*>(),
                                ix.inds_ptrs.as<const int64_t*>(), ix.ids_arena.as<int64_t>(), nq * P, P,
-                               ix.n_lists, counters, order, desc, lead, alive, true, s);
+                               ix.n_lists, counters, order, desc, lead, alive, true, few_pairs, s);
     if (pl.fused) { detail::launch_fill_u32(kth, 0xFFFFFFFFu, nq, s); }
     mark(2);
 
