@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 # HBM bytes per launch of the named kernel on the default workload, from hardware counters (FETCH_SIZE + WRITE_SIZE
 # per dispatch, each scaled by its reading for the 1 GiB calibration copy below); the counter runs
 # are summarised under profiles/.  Keyed by (kernel, lut, internal); None where not measured.
-MEASURED_TRAFFIC = {("scan_screen_direct_kernel", "f16", "f32"): 1.138e9}
+MEASURED_TRAFFIC = {("scan_screen_direct_kernel", "f16", "f32"): 1.216e9}
 
 
 # BASELINE.json's configurations; `dataset` names the generator below
