@@ -320,8 +320,11 @@ __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
 }
 
 /** thr[q] = (n_probes-th smallest of the query's group minima) + 2 E_q, rounded up.  One wave per
- *  query: the minima sit in registers as ordered keys (16 per lane; more are re-read every round)
- *  and a round of the bitwise search counts with ballots, without LDS or barriers. */
+ *  query: the minima sit in registers as ordered keys (HELD per lane: 16 cover 16,384 lists, 64
+ *  cover 65,536; more are re-read every round) and a round of the bitwise search counts with
+ *  ballots, without LDS or barriers.  One probe (labelling rows during extend) needs no search:
+ *  the threshold is the smallest minimum. */
+template <uint32_t HELD>
 __global__ __launch_bounds__(256) void coarse_threshold_kernel(
   const float* __restrict__ minima, uint32_t n_queries, uint32_t n_groups, uint32_t n_probes,
   const float* __restrict__ qnorm, float e_rel, float e_abs, float* __restrict__ thr)
@@ -330,7 +333,6 @@ __global__ __launch_bounds__(256) void coarse_threshold_kernel(
   const uint32_t lane = threadIdx.x & 63u;
   if (q >= n_queries) { return; }
   const float* row = minima + uint64_t(q) * n_groups;
-  constexpr uint32_t HELD = 16;
   uint32_t held[HELD];
 #pragma unroll
   for (uint32_t h = 0; h < HELD; h++) {
@@ -340,17 +342,34 @@ __global__ __launch_bounds__(256) void coarse_threshold_kernel(
   }
   // smallest ordered key K with count(keys <= K) >= n_probes, one bit at a time
   uint32_t prefix = 0;
-  for (int bit = 31; bit >= 0; bit--) {
-    const uint32_t probe = prefix | ((1u << bit) - 1u);
-    uint32_t n           = 0;
+  if (n_probes == 1u) {
+    uint32_t lowest = 0xFFFFFFFFu;
 #pragma unroll
-    for (uint32_t h = 0; h < HELD; h++) { n += uint32_t(__popcll(__builtin_amdgcn_ballot_w64(held[h] <= probe))); }
-    for (uint32_t g0 = HELD * 64u; g0 < n_groups; g0 += 64u) {
-      const uint32_t g = g0 + lane;
-      const float v    = g < n_groups ? row[g] : __uint_as_float(0x7fc00000u);
-      n += uint32_t(__popcll(__builtin_amdgcn_ballot_w64(v == v && order_f32(v) <= probe)));
+    for (uint32_t h = 0; h < HELD; h++) { lowest = held[h] < lowest ? held[h] : lowest; }
+    for (uint32_t g = HELD * 64u + lane; g < n_groups; g += 64u) {
+      const float v    = row[g];
+      const uint32_t k = (v == v) ? order_f32(v) : 0xFFFFFFFFu;
+      lowest           = k < lowest ? k : lowest;
     }
-    if (n < n_probes) { prefix |= 1u << bit; }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const uint32_t other = uint32_t(__shfl_xor(int(lowest), off, 64));
+      lowest               = other < lowest ? other : lowest;
+    }
+    prefix = lowest;
+  } else {
+    for (int bit = 31; bit >= 0; bit--) {
+      const uint32_t probe = prefix | ((1u << bit) - 1u);
+      uint32_t n           = 0;
+#pragma unroll
+      for (uint32_t h = 0; h < HELD; h++) { n += uint32_t(__popcll(__builtin_amdgcn_ballot_w64(held[h] <= probe))); }
+      for (uint32_t g0 = HELD * 64u; g0 < n_groups; g0 += 64u) {
+        const uint32_t g = g0 + lane;
+        const float v    = g < n_groups ? row[g] : __uint_as_float(0x7fc00000u);
+        n += uint32_t(__popcll(__builtin_amdgcn_ballot_w64(v == v && order_f32(v) <= probe)));
+      }
+      if (n < n_probes) { prefix |= 1u << bit; }
+    }
   }
   if (lane == 0) {
     const float t = unorder_f32(prefix);
@@ -501,7 +520,11 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
     k1<<<grid, kGemmThreads, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, n_list_tiles, tiles_per_block, alpha,
                                     qterm, a.minima, n_groups, nullptr, nullptr, nullptr);
     CUVS_HIP_TRY(hipGetLastError());
-    coarse_threshold_kernel<<<(a.n_queries + 3) / 4, 256, 0, stream>>>(a.minima, a.n_queries, n_groups, a.n_probes, a.qnorm, e_rel, e_abs, a.thr);
+    if (n_groups <= 16u * 64u) {
+      coarse_threshold_kernel<16><<<(a.n_queries + 3) / 4, 256, 0, stream>>>(a.minima, a.n_queries, n_groups, a.n_probes, a.qnorm, e_rel, e_abs, a.thr);
+    } else {
+      coarse_threshold_kernel<64><<<(a.n_queries + 3) / 4, 256, 0, stream>>>(a.minima, a.n_queries, n_groups, a.n_probes, a.qnorm, e_rel, e_abs, a.thr);
+    }
     CUVS_HIP_TRY(hipGetLastError());
     k2<<<grid, kGemmThreads, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, n_list_tiles, tiles_per_block, alpha,
                                     qterm, nullptr, n_groups, a.thr, a.cand_count, a.cand);

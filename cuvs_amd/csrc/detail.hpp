@@ -385,6 +385,7 @@ struct encode_args {
   uint32_t dim, dim_ext, rot_dim, pq_dim, pq_len, pq_bits, n_chunks;
   int per_cluster;
   const uint32_t* labels;
+  const uint32_t* perm;  // thread i encodes row perm[i] (rows grouped by list), or null: row i
   const float* centers;
   const float* rotation_t;
   int identity_rotation;
@@ -400,6 +401,11 @@ struct encode_args {
   float* scratch;       // [rot_dim, n] rotated residuals
 };
 void launch_encode(const encode_args& a, hipStream_t stream);
+
+/** perm = the row numbers 0..n-1 grouped by label (order inside a group unspecified);
+ *  `counters` holds 2 * n_lists words of scratch. */
+void launch_rows_by_label(const uint32_t* labels, uint64_t n, uint32_t n_lists, uint32_t* counters,
+                          uint32_t* perm, hipStream_t stream);
 
 void launch_unpack_contiguous(const uint8_t* list_data, uint32_t n_rows, uint32_t offset,
                               uint32_t pq_dim, uint32_t pq_bits, uint8_t* out, hipStream_t stream);

@@ -43,9 +43,12 @@ uint64_t chunk_rows_for(const index_impl& ix, uint64_t n_rows)
  *  rows plus the rotated residuals. */
 uint64_t encode_chunk_rows_for(const index_impl& ix, uint64_t n_rows)
 {
-  uint64_t c = (uint64_t(1) << 28) / std::max<uint32_t>(ix.dim + ix.rot_dim, 1);
+  // per-cluster codebooks: larger passes, so that a pass holds many rows of each list (the rows of
+  // a pass are encoded grouped by list)
+  const bool per_cluster = ix.codebook_kind == codebook_gen::PER_CLUSTER;
+  uint64_t c = (uint64_t(1) << (per_cluster ? 30 : 28)) / std::max<uint32_t>(ix.dim + ix.rot_dim, 1);
   c          = std::max<uint64_t>(c, 1024);
-  c          = std::min<uint64_t>(c, uint64_t(1) << 20);
+  c          = std::min<uint64_t>(c, uint64_t(1) << (per_cluster ? 22 : 20));
   return std::min<uint64_t>(c, n_rows);
 }
 
@@ -212,6 +215,12 @@ void extend(cuvs::resources const& res,
   /* 4. encode and append */
   device_buffer scratch(chunk * ix.rot_dim * sizeof(float));
   device_buffer ids_stage;
+  const bool group_rows = ix.codebook_kind == codebook_gen::PER_CLUSTER;
+  device_buffer perm, perm_counters;
+  if (group_rows) {
+    perm.allocate(chunk * sizeof(uint32_t));
+    perm_counters.allocate(size_t(2) * ix.n_lists * sizeof(uint32_t));
+  }
   const bool ids_on_device = new_indices == nullptr || is_device_pointer(new_indices);
   if (!ids_on_device) { ids_stage.allocate(chunk * sizeof(int64_t)); }
   for (uint64_t r0 = 0; r0 < n_rows; r0 += chunk) {
@@ -237,6 +246,11 @@ void extend(cuvs::resources const& res,
     }
     a.flat_codes = nullptr;
     a.scratch    = scratch.as<float>();
+    if (group_rows) {
+      detail::launch_rows_by_label(a.labels, n, ix.n_lists, perm_counters.as<uint32_t>(),
+                                   perm.as<uint32_t>(), s);
+      a.perm = perm.as<uint32_t>();
+    }
     detail::launch_encode(a, s);
   }
   ix.rebuild_lead_plane(s);

@@ -949,11 +949,14 @@ __global__ __launch_bounds__(kBlock) void encode_kernel(encode_args a)
   const bool lds_book = !PER_CLUSTER && a.pq_len <= kBookMaxLen;
   const uint64_t r0   = uint64_t(blockIdx.x) * kBlock + threadIdx.x;
   const bool active   = r0 < a.n_rows;
-  const uint64_t r    = active ? r0 : a.n_rows - 1u;  // idle lanes shadow the last row, write nothing
+  const uint64_t t0   = active ? r0 : a.n_rows - 1u;  // idle lanes shadow the last row, write nothing
+  // With per-cluster codebooks the rows come grouped by list, so that the lanes of a wave read
+  // the same few codebooks at the same time instead of 64 different ones.
+  const uint64_t r     = a.perm != nullptr ? a.perm[t0] : t0;
   const uint32_t label = a.labels[r];
   const float* x       = a.xf + r * a.dim;
   const float* c       = a.centers + uint64_t(label) * a.dim_ext;
-  float* res           = a.scratch + r;  // element d at res[d * n_rows]
+  float* res           = a.scratch + t0;  // element d at res[d * n_rows]
   const uint64_t rs    = a.n_rows;
   auto xval = [&](uint32_t d) -> float { return x[d]; };
   if (active) {
@@ -1063,6 +1066,13 @@ __global__ __launch_bounds__(kBlock) void encode_kernel(encode_args a)
       }
     }
   }
+}
+
+__global__ void rows_by_label_kernel(const uint32_t* __restrict__ labels, uint64_t n,
+                                     uint32_t* __restrict__ cursors, uint32_t* __restrict__ perm)
+{
+  const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) { perm[atomicAdd(&cursors[labels[i]], 1u)] = uint32_t(i); }
 }
 
 __global__ void unpack_contiguous_kernel(const uint8_t* __restrict__ list_data, uint32_t n_rows,
@@ -1429,6 +1439,25 @@ void launch_encode_bits(const encode_args& a, uint32_t grid, hipStream_t stream)
   }
 }
 }  // namespace
+
+void launch_rows_by_label(const uint32_t* labels, uint64_t n, uint32_t n_lists, uint32_t* counters,
+                          uint32_t* perm, hipStream_t stream)
+{
+  if (n == 0) { return; }
+  CUVS_EXPECTS(n <= 0xFFFFFFFFull, "too many rows in one pass");
+  uint32_t* counts  = counters;
+  uint32_t* cursors = counters + n_lists;
+  launch_fill_u32(counts, 0, n_lists, stream);
+  histogram_kernel<<<blocks_for(n, 256), 256, 0, stream>>>(labels, n, counts);
+  CUVS_LAUNCH_CHECK();
+  const size_t smem = size_t(kScanTile + kScanThreads) * 4;
+  CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(exclusive_scan_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+  exclusive_scan_kernel<<<1, kScanThreads, smem, stream>>>(counts, n_lists, cursors);
+  CUVS_LAUNCH_CHECK();
+  rows_by_label_kernel<<<blocks_for(n, 256), 256, 0, stream>>>(labels, n, cursors, perm);
+  CUVS_LAUNCH_CHECK();
+}
 
 void launch_encode(const encode_args& a, hipStream_t stream)
 {
