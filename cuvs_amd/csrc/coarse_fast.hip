@@ -39,7 +39,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t kTile    = 128;  // lists x queries per block
 constexpr uint32_t kSlab    = 64;   // the padded dimension is a multiple of this
-constexpr uint32_t kCandCapF = 256;  // candidates per query
+constexpr uint32_t kCandCapF = 512;  // candidate slots per query (256 are used up to 128 probes)
 
 template <typename T>
 __device__ __forceinline__ float map_elem(T v);
@@ -383,7 +383,7 @@ __global__ __launch_bounds__(256) void coarse_threshold_kernel(
 /** Exact fp32 score of every candidate by the fp32 path's arithmetic, then the n_probes best in
  *  ascending (score, list) order.  One block of 256 threads per query. */
 template <typename T>
-__global__ __launch_bounds__(256) void coarse_rescore_kernel(
+__global__ __launch_bounds__(512) void coarse_rescore_kernel(
   const T* __restrict__ queries, const float* __restrict__ centers, uint32_t dim, uint32_t dim_ext,
   float qterm, float alpha, const uint32_t* __restrict__ cand_count, const uint32_t* __restrict__ cand,
   uint32_t n_probes, uint32_t* __restrict__ probes, uint8_t* __restrict__ fallback)
@@ -394,11 +394,12 @@ __global__ __launch_bounds__(256) void coarse_rescore_kernel(
   const uint32_t q   = blockIdx.x;
   const uint32_t tid = threadIdx.x;
   const uint32_t n   = cand_count[q];
-  if (n > kCandCapF || n < n_probes) {
+  // one candidate per thread: the block is as wide as the longest candidate list it accepts
+  if (n > blockDim.x || n < n_probes) {
     if (tid == 0) { fallback[q] = 1; }
     return;
   }
-  for (uint32_t d = tid; d < dim; d += 256) { qf[d] = map_elem<T>(queries[uint64_t(q) * dim + d]); }
+  for (uint32_t d = tid; d < dim; d += blockDim.x) { qf[d] = map_elem<T>(queries[uint64_t(q) * dim + d]); }
   __syncthreads();
   unsigned long long key = kInvalidKey;
   if (tid < n) {
@@ -536,24 +537,26 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
     CUVS_EXPECTS(k_pad == 128, "the two-precision probe selection takes dim <= 128");
     run_pass(coarse_f16_kernel<1, 128>, coarse_f16_kernel<2, 128>);
   }
-  const size_t rsmem = ((size_t(a.dim) * 4 + 15) & ~size_t(15)) + size_t(256) * 8;
+  // up to 128 probes about 1.4 x 128 candidates pass the threshold: 256 threads; 512 beyond
+  const uint32_t rthreads = a.n_probes <= 128 ? 256u : 512u;
+  const size_t rsmem      = ((size_t(a.dim) * 4 + 15) & ~size_t(15)) + size_t(rthreads) * 8;
   const size_t xsmem = size_t(a.dim) * 4;
   CUVS_EXPECTS(rsmem <= 48 * 1024, "dim (%u) is too large for the two-precision probe selection", a.dim);
   switch (a.type) {
     case elem_type::f32:
-      coarse_rescore_kernel<float><<<a.n_queries, 256, rsmem, stream>>>(static_cast<const float*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
+      coarse_rescore_kernel<float><<<a.n_queries, rthreads, rsmem, stream>>>(static_cast<const float*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
       coarse_exact_rows_kernel<float><<<a.n_queries, 256, xsmem, stream>>>(static_cast<const float*>(a.queries), a.centers, a.n_lists, a.dim, a.dim_ext, qterm, alpha, a.fallback, a.scores);
       break;
     case elem_type::f16:
-      coarse_rescore_kernel<_Float16><<<a.n_queries, 256, rsmem, stream>>>(static_cast<const _Float16*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
+      coarse_rescore_kernel<_Float16><<<a.n_queries, rthreads, rsmem, stream>>>(static_cast<const _Float16*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
       coarse_exact_rows_kernel<_Float16><<<a.n_queries, 256, xsmem, stream>>>(static_cast<const _Float16*>(a.queries), a.centers, a.n_lists, a.dim, a.dim_ext, qterm, alpha, a.fallback, a.scores);
       break;
     case elem_type::i8:
-      coarse_rescore_kernel<int8_t><<<a.n_queries, 256, rsmem, stream>>>(static_cast<const int8_t*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
+      coarse_rescore_kernel<int8_t><<<a.n_queries, rthreads, rsmem, stream>>>(static_cast<const int8_t*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
       coarse_exact_rows_kernel<int8_t><<<a.n_queries, 256, xsmem, stream>>>(static_cast<const int8_t*>(a.queries), a.centers, a.n_lists, a.dim, a.dim_ext, qterm, alpha, a.fallback, a.scores);
       break;
     default:
-      coarse_rescore_kernel<uint8_t><<<a.n_queries, 256, rsmem, stream>>>(static_cast<const uint8_t*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
+      coarse_rescore_kernel<uint8_t><<<a.n_queries, rthreads, rsmem, stream>>>(static_cast<const uint8_t*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
       coarse_exact_rows_kernel<uint8_t><<<a.n_queries, 256, xsmem, stream>>>(static_cast<const uint8_t*>(a.queries), a.centers, a.n_lists, a.dim, a.dim_ext, qterm, alpha, a.fallback, a.scores);
       break;
   }

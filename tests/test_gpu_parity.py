@@ -647,6 +647,28 @@ def test_two_precision_probe_selection_equals_the_fp32_path(orc, metric, dtype, 
         assert np.array_equal(got, want), (metric, dtype, n_probes)
 
 
+@pytest.mark.parametrize("metric,dtype", [("sqeuclidean", np.float16), ("inner_product", np.float32)])
+def test_two_precision_probe_selection_many_lists_and_probes(orc, metric, dtype):
+    """50,000 lists (more group minima than a wave holds in 16 registers a lane) and up to 256
+    probes (candidate lists of up to 512)."""
+    n_lists, dim, pq_dim = 50_000, 96, 48
+    model = _coarse_model(n_lists, dim, pq_dim, 11)
+    params = ivf_pq.IndexParams(n_lists=n_lists, metric=metric, pq_dim=pq_dim, pq_bits=8)
+    dev = {k: G.to_dev(v) for k, v in model.items()}
+    index = ivf_pq.build_precomputed(params, dim, dev["pq_centers"], dev["centers"], dev["centers_rot"],
+                                     dev["rotation_matrix"])
+    ix = H.oracle_index(orc, model, dim, pq_dim, 8, metric=metric)
+    rng = np.random.default_rng(12)
+    c = model["centers"][:, :dim]
+    q = np.concatenate([c[:40], 0.5 * (c[100:140] + c[200:240]),
+                        rng.standard_normal((40, dim)).astype(np.float32)]).astype(dtype)
+    for n_probes in (1, 100, 200, 256):
+        sp = ivf_pq.SearchParams(n_probes=n_probes)
+        got = ivf_pq.select_clusters(sp, index, G.to_dev(q)).cpu().numpy().view(np.uint32)
+        want, _ = orc.select_clusters(ix, q, n_probes)
+        assert np.array_equal(got, want), (metric, n_probes)
+
+
 def test_two_precision_probe_selection_falls_back(orc):
     """Identical centres put hundreds of lists inside the error margin (more candidates than the
     fast path holds), and a query with a NaN has no usable bound: both take the plain fp32 path and
