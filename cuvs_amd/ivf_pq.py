@@ -64,6 +64,17 @@ class IndexParams:
             raise ValueError("Incorrect codes layout %s" % codes_layout)
         self.metric = metric
 
+    n_lists = property(lambda self: self._p.contents.n_lists)
+    metric_arg = property(lambda self: self._p.contents.metric_arg)
+    kmeans_n_iters = property(lambda self: self._p.contents.kmeans_n_iters)
+    kmeans_trainset_fraction = property(lambda self: self._p.contents.kmeans_trainset_fraction)
+    pq_bits = property(lambda self: self._p.contents.pq_bits)
+    pq_dim = property(lambda self: self._p.contents.pq_dim)
+    force_random_rotation = property(lambda self: bool(self._p.contents.force_random_rotation))
+    add_data_on_build = property(lambda self: bool(self._p.contents.add_data_on_build))
+    conservative_memory_allocation = property(lambda self: bool(self._p.contents.conservative_memory_allocation))
+    max_train_points_per_pq_code = property(lambda self: self._p.contents.max_train_points_per_pq_code)
+
     @property
     def params(self):
         return self._p.contents
@@ -196,10 +207,22 @@ class Index:
     def list_sizes(self):
         return self._device_copy(lib().cuvsIvfPqIndexGetListSizes, _torch().int32)
 
-    def list_indices(self, label):
+    def __repr__(self):
+        attrs = ", ".join(f"{name}={getattr(self, name)}" for name in ("n_lists", "dim", "pq_dim", "pq_len", "pq_bits"))
+        return f"Index(type=IvfPq, {attrs})"
+
+    def lists(self, resources=None):
+        """Iterates over the lists: (source indices, bit-contiguous codes) of each (ivf_pq.pyx:392-408)."""
+        for label, size in enumerate(self.list_sizes.cpu().tolist()):
+            yield self.list_indices(label, n_rows=size), self.list_data(label, n_rows=size, resources=resources)
+
+    def list_indices(self, label, n_rows=0):
+        """Source indices of one list; the first `n_rows` of them when given (ivf_pq.pyx:451-474)."""
         v = _BorrowedView()
         check(lib().cuvsIvfPqIndexGetListIndices(self._i, int(label), C.byref(v.mt)))
         n = v.mt.dl_tensor.shape[0]
+        if n_rows:
+            n = min(n, int(n_rows))
         torch = _torch()
         out = torch.empty(n, dtype=torch.int64, device="cuda")
         if n > 0:

@@ -182,3 +182,61 @@ def test_build_validation():
         ivf_pq.build(ivf_pq.IndexParams(n_lists=200, pq_dim=8), x)
     with pytest.raises(Exception, match="kmeans_trainset_fraction"):
         ivf_pq.build(ivf_pq.IndexParams(n_lists=4, pq_dim=8, kmeans_trainset_fraction=0.0), x)
+
+
+@pytest.mark.parametrize("codebook_kind", ["subspace", "cluster"])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.int8, np.uint8])
+@pytest.mark.parametrize("n_rows,pq_bits", [(500, 6), (100000, 8)])
+def test_transform_matches_the_stored_lists(codebook_kind, dtype, n_rows, pq_bits):
+    """The reference's own transform test (python/cuvs/cuvs/tests/test_ivf_pq.py:337-378):
+    transforming the dataset an index was built from gives the labels and codes the index stores."""
+    n_cols, n_lists, pq_dim = 32, 50, 8
+    dataset = _data(dtype, n_rows, n_cols, 33)
+    params = ivf_pq.IndexParams(n_lists=n_lists, pq_bits=pq_bits, pq_dim=pq_dim, codebook_kind=codebook_kind)
+    index = ivf_pq.build(params, G.to_dev(dataset))
+    labels_exp = np.zeros(n_rows, dtype=np.uint32)
+    transformed_exp = np.zeros((n_rows, int(np.ceil(index.pq_dim * index.pq_bits / 8))), dtype=np.uint8)
+    total = 0
+    for cluster_id, (ids, codes) in enumerate(index.lists()):
+        ids = ids.cpu().numpy()
+        labels_exp[ids] = cluster_id
+        transformed_exp[ids] = codes.cpu().numpy()
+        total += ids.size
+    assert total == n_rows == len(index)
+    labels, transformed = ivf_pq.transform(index, G.to_dev(dataset))
+    np.testing.assert_array_equal(labels.cpu().numpy().view(np.uint32), labels_exp)
+    np.testing.assert_array_equal(transformed.cpu().numpy(), transformed_exp)
+
+
+def test_python_mirror_of_the_reference_workflow(tmp_path):
+    """build on a host array, extend in two halves with explicit indices (device, then host
+    arrays), save / load, search with preallocated outputs, model getters: the calls of the
+    reference's run_ivf_pq_build_search_test (python/cuvs/cuvs/tests/test_ivf_pq.py:21-125)."""
+    n_rows, n_cols, n_queries, k = 10000, 10, 100, 10
+    rng = np.random.default_rng(3)
+    dataset = rng.random((n_rows, n_cols), dtype=np.float32)
+    queries = rng.random((n_queries, n_cols), dtype=np.float32)
+    params = ivf_pq.IndexParams(n_lists=100, metric="sqeuclidean", kmeans_n_iters=20, pq_bits=8, pq_dim=0,
+                                add_data_on_build=False)
+    assert params.n_lists == 100 and params.pq_bits == 8 and params.add_data_on_build is False
+    index = ivf_pq.build(params, torch.from_numpy(dataset))
+    assert index.trained and len(index) == 0 and "IvfPq" in repr(index)
+    half = n_rows // 2
+    ids = np.arange(n_rows, dtype=np.int64)
+    index = ivf_pq.extend(index, G.to_dev(dataset[:half]), G.to_dev(ids[:half]))
+    index = ivf_pq.extend(index, torch.from_numpy(dataset[half:]), torch.from_numpy(ids[half:]))
+    assert len(index) == n_rows
+    path = tmp_path / "index.bin"
+    ivf_pq.save(str(path), index)
+    index = ivf_pq.load(str(path))
+    out_idx = torch.zeros((n_queries, k), dtype=torch.int64, device="cuda")
+    out_dist = torch.zeros((n_queries, k), dtype=torch.float32, device="cuda")
+    sp = ivf_pq.SearchParams(n_probes=100, lut_dtype=np.float32, internal_distance_dtype=np.float32)
+    ret = ivf_pq.search(sp, index, G.to_dev(queries), k, neighbors=out_idx, distances=out_dist)
+    torch.cuda.synchronize()
+    assert ret[0].data_ptr() == out_dist.data_ptr() and ret[1].data_ptr() == out_idx.data_ptr()
+    d = ((queries[:, None, :] - dataset[None]) ** 2).sum(-1)
+    truth = np.argsort(d, axis=1)[:, :k]
+    assert _recall(out_idx.cpu().numpy(), truth) > 0.7  # the reference's own bar for this test
+    assert index.centers.shape == (100, n_cols) and index.pq_centers.shape[2] == 256
+    assert sum(i.shape[0] for i, _ in index.lists()) == n_rows
