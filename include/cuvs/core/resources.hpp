@@ -13,6 +13,10 @@
 #include <string>
 #include <vector>
 
+// The library is built with hidden visibility; what this header declares is its C++ interface
+// (the reference marks the same namespaces CUVS_EXPORT).
+#pragma GCC visibility push(default)
+
 namespace cuvs {
 
 /** Error type thrown by every C++ entry point (role of raft::logic_error / RAFT_EXPECTS). */
@@ -103,3 +107,5 @@ class resources {
 };
 
 }  // namespace cuvs
+
+#pragma GCC visibility pop

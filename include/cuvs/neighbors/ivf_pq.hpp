@@ -15,6 +15,10 @@
 #include <memory>
 #include <string>
 
+// The library is built with hidden visibility; what this header declares is its C++ interface
+// (the reference marks the same namespaces CUVS_EXPORT).
+#pragma GCC visibility push(default)
+
 namespace cuvs::distance {
 /** Numeric values of cuvs::distance::DistanceType (cpp/include/cuvs/distance/distance.hpp). */
 enum class DistanceType : int {
@@ -81,9 +85,11 @@ struct search_params : cuvs::neighbors::search_params {
   uint32_t max_internal_batch_size  = 4096;
 };
 
+#pragma GCC visibility pop
 namespace detail {
-struct index_impl;
+struct index_impl;  // the index's contents: not part of the interface
 }
+#pragma GCC visibility push(default)
 
 /** Element type of query / dataset rows. */
 enum class elem_type : int { f32 = 0, f16 = 1, i8 = 2, u8 = 3 };
@@ -232,3 +238,5 @@ void deserialize(cuvs::resources const& res, const std::string& filename, index<
 
 }  // namespace ivf_pq
 }  // namespace cuvs::neighbors
+
+#pragma GCC visibility pop

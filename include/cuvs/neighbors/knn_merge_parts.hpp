@@ -8,6 +8,10 @@
 
 #include <cstdint>
 
+// The library is built with hidden visibility; what this header declares is its C++ interface
+// (the reference marks the same namespaces CUVS_EXPORT).
+#pragma GCC visibility push(default)
+
 namespace cuvs::neighbors {
 
 /** in_keys / in_ids: [n_parts * n_samples, k], part-major (all rows of part 0, then part 1, ...),
@@ -25,3 +29,5 @@ void knn_merge_parts(cuvs::resources const& res,
                      int64_t n_parts);
 
 }  // namespace cuvs::neighbors
+
+#pragma GCC visibility pop

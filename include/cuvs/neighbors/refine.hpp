@@ -8,6 +8,10 @@
 #include <cuvs/distance/distance.h>
 #include <cuvs/neighbors/ivf_pq.hpp>
 
+// The library is built with hidden visibility; what this header declares is its C++ interface
+// (the reference marks the same namespaces CUVS_EXPORT).
+#pragma GCC visibility push(default)
+
 namespace cuvs::neighbors {
 
 /** For each query the exact distance to each of its candidates, the k = indices.extent(1) nearest
@@ -28,3 +32,5 @@ void refine(cuvs::resources const& res, const void* dataset, const void* queries
             int64_t k, cuvs::distance::DistanceType metric);
 
 }  // namespace cuvs::neighbors
+
+#pragma GCC visibility pop
