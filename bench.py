@@ -215,7 +215,9 @@ def main():
     early_stop = stage["n_screened_pairs"] > 0
     pq_len = dim // pq_dim
     nibble = pq_bits == 4 and pq_dim % 32 == 0 and pq_len in (1, 2, 4) and (pq_dim // 16) * pq_len <= 48
-    full_name = ("scan_nibble_kernel" if nibble
+    fused = k <= 256  # beyond that every score is stored and selected afterwards (generic kernel)
+    full_name = ("scan_kernel" if not fused
+                 else "scan_nibble_kernel" if nibble
                  else "scan_kernel" if (pq_bits != 8 or (pq_dim, pq_len) not in ((64, 2), (48, 2), (32, 4)))
                  else "scan_quad_kernel" if (args.lut != "f32" and k <= 64) else "scan_fast_kernel")
     if early_stop:
