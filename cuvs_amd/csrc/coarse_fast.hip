@@ -37,7 +37,8 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr uint32_t kTile    = 128;  // lists x queries per block
+constexpr uint32_t kTile    = 128;  // lists per tile
+constexpr uint32_t kQTile   = 256;  // queries per block: 4 waves x 64
 constexpr uint32_t kSlab    = 64;   // the padded dimension is a multiple of this
 constexpr uint32_t kCandCapF = 512;  // candidate slots per query (256 are used up to 128 probes)
 
@@ -113,15 +114,16 @@ __global__ void pack_centers_kernel(const float* __restrict__ centers, uint32_t 
 
 constexpr uint32_t kGemmThreads = 512;
 constexpr uint32_t kLocalCap    = 32;  // PASS 2: candidates a block may hold per query before it gives up
-constexpr uint32_t kTilesPerBlock = 8;  // list tiles a block walks at most
+constexpr uint32_t kTilesPerBlock = 10;  // list tiles a block walks at most (its group minima fill the LDS)
 
 /**
- * fp16 scores s' = alpha * (dot16(c, q) + cn * qterm) of a block's 128 queries against a run of
+ * fp16 scores s' = alpha * (dot16(c, q) + cn * qterm) of a block's 256 queries against a run of
  * list tiles (128 lists each).  The queries stay in LDS for the whole block; list tiles stream
  * through two LDS buffers, the next tile's global loads in flight while the current one is
  * multiplied (one barrier per tile).  Eight waves, two per SIMD so that one's matrix products
- * overlap the other's epilogue; a wave owns 64 lists x 32 queries, two MFMA tiles of
- * v_mfma_f32_32x32x16_f16.  PASS 1 writes, per query, the minimum over every group of 16 lists;
+ * overlap the other's epilogue; a wave owns 64 lists x 64 queries, four MFMA tiles of
+ * v_mfma_f32_32x32x16_f16 (each 16-byte read of the list operand out of LDS feeds two products:
+ * with 32 queries a wave the LDS bandwidth, not the matrix cores, set the pace).  PASS 1 writes, per query, the minimum over every group of 16 lists;
  * PASS 2 collects the lists whose score is at or below the query's threshold in LDS and appends
  * them to the query's candidate list when the block ends (one global atomic per query and block).
  * Both passes execute the same instructions up to the epilogue, so a list's score is the same
@@ -130,7 +132,7 @@ constexpr uint32_t kTilesPerBlock = 8;  // list tiles a block walks at most
 template <int PASS, uint32_t K_PAD>
 __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
   const _Float16* __restrict__ ch, const _Float16* __restrict__ qh, const float* __restrict__ cn,
-  uint32_t n_lists, uint32_t n_queries, uint32_t n_list_tiles, uint32_t tiles_per_block, float alpha,
+  uint32_t n_lists, uint32_t n_queries, uint32_t q_rows, uint32_t n_list_tiles, uint32_t tiles_per_block, float alpha,
   float qterm, float* __restrict__ minima, uint32_t n_groups, const float* __restrict__ thr,
   uint32_t* __restrict__ cand_count, uint32_t* __restrict__ cand)
 {
@@ -140,15 +142,15 @@ __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned char* sa0 = smem;  // lists [2][128][ROWB], two buffers
   float* scn         = reinterpret_cast<float*>(smem + 2u * kTile * ROWB);  // [2][128] norm terms
-  uint32_t* lcount   = reinterpret_cast<uint32_t*>(scn + 2u * kTile);       // PASS 2: [128]
-  uint32_t* lcand    = lcount + kTile;                                      // PASS 2: [128][kLocalCap]
-  float* lmin        = reinterpret_cast<float*>(lcount);  // PASS 1: [128][kTilesPerBlock * 8] group minima
+  uint32_t* lcount   = reinterpret_cast<uint32_t*>(scn + 2u * kTile);       // PASS 2: [256]
+  uint32_t* lcand    = lcount + kQTile;                                     // PASS 2: [256][kLocalCap]
+  float* lmin        = reinterpret_cast<float*>(lcount);  // PASS 1: [256][kTilesPerBlock * 8] group minima
   const uint32_t tid  = threadIdx.x;
   const uint32_t lane = tid & 63u;
   const uint32_t wid  = tid >> 6;
   const uint32_t wl   = wid >> 2;  // wave's half of the lists (64)
-  const uint32_t wq   = wid & 3u;  // wave's quarter of the queries (32)
-  const uint32_t q0   = blockIdx.y * kTile;
+  const uint32_t wq   = wid & 3u;  // wave's quarter of the queries (64)
+  const uint32_t q0   = blockIdx.y * kQTile;
   const uint32_t t0   = blockIdx.x * tiles_per_block;
   const uint32_t t1   = t0 + tiles_per_block < n_list_tiles ? t0 + tiles_per_block : n_list_tiles;
 
@@ -172,27 +174,36 @@ __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
   if (tid < kTile) {
     const uint32_t l = t0 * kTile + tid;
     scn[tid]         = l < n_lists ? cn[l] * qterm : neg_inf;
-    if (PASS == 2) { lcount[tid] = 0; }
   }
+  if (PASS == 2 && tid < kQTile) { lcount[tid] = 0; }
   __syncthreads();
 
   // The epilogue works on v = dot + norm term; the score is alpha * v with alpha = -1 or -2, so the
   // smallest score of a group is alpha * (its largest v) and "score <= thr" is "v >= thr / alpha",
   // both exactly.
-  const uint32_t qloc = wq * 32u + (lane & 31u);  // this lane's query inside the block
-  const uint32_t q    = q0 + qloc;
-  // the wave's query operand never changes: it lives in registers (8 values per 16 dimensions)
-  v8h bq[K_PAD / 16u];
+  // this lane's two queries inside the block (columns of the wave's two query tiles); the packed
+  // queries are padded to a multiple of 128 rows, a block's second half may lie beyond them
+  uint32_t qloc[2], q[2];
+  v8h bq[2][K_PAD / 16u];  // the wave's query operand never changes: it lives in registers
+  float limit[2] = {0.0f, 0.0f};
 #pragma unroll
-  for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) {
-    bq[ks] = *reinterpret_cast<const v8h*>(qh + uint64_t(q) * K_PAD + ks * 16u + (lane >> 5) * 8u);
+  for (int j = 0; j < 2; j++) {
+    qloc[j]             = wq * 64u + uint32_t(j) * 32u + (lane & 31u);
+    q[j]                = q0 + qloc[j];
+    const uint32_t q_rd = q[j] < q_rows ? q[j] : q_rows - 1u;
+#pragma unroll
+    for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) {
+      bq[j][ks] = *reinterpret_cast<const v8h*>(qh + uint64_t(q_rd) * K_PAD + ks * 16u + (lane >> 5) * 8u);
+    }
+    if (PASS == 2) { limit[j] = q[j] < n_queries ? thr[q[j]] / alpha : __uint_as_float(0x7f800000u); }
   }
   // Use them once here, so that the compiler's wait for these loads sits here and not inside the
   // loop: there it would also wait for the staged loads below, which it does not count.
 #pragma unroll
-  for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) { asm volatile("" : "+v"(bq[ks])); }
-  float limit         = 0.0f;
-  if (PASS == 2) { limit = q < n_queries ? thr[q] / alpha : __uint_as_float(0x7f800000u); }
+  for (int j = 0; j < 2; j++) {
+#pragma unroll
+    for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) { asm volatile("" : "+v"(bq[j][ks])); }
+  }
 
   // The next tile's loads go out at the top of an iteration and are written to the other LDS
   // buffer at its end.  They are written as instructions: as ordinary loads of read-only data the
@@ -232,11 +243,14 @@ __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
   // products and epilogue of one tile out of LDS buffer `buf`
   auto multiply = [&](uint32_t tile, uint32_t buf) __attribute__((always_inline)) {
     const unsigned char* sa = sa0 + buf * (kTile * ROWB);
-    v16f acc[2];
+    v16f acc[2][2];  // [list tile][query tile]
 #pragma unroll
     for (int i = 0; i < 2; i++) {
 #pragma unroll
-      for (int r = 0; r < 16; r++) { acc[i][r] = 0.0f; }
+      for (int j = 0; j < 2; j++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) { acc[i][j][r] = 0.0f; }
+      }
     }
 #pragma unroll
     for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) {
@@ -248,38 +262,44 @@ __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
       }
 #pragma unroll
       for (int i = 0; i < 2; i++) {
-        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], bq[ks], acc[i], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], bq[j][ks], acc[i][j], 0, 0, 0);
+        }
       }
     }
     // element r of a tile: row (list) (r / 4) * 8 + (lane / 32) * 4 + r % 4, column (query) lane % 32
     const uint32_t l0 = tile * kTile;
-    uint32_t hits     = 0;  // PASS 2: bit (i * 16 + r) set when that list is a candidate
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-      const uint32_t rbase = wl * 64u + i * 32u + (lane >> 5) * 4u;  // row inside the block tile
-      float best           = neg_inf;
+    for (int j = 0; j < 2; j++) {
+      uint32_t hits = 0;  // PASS 2: bit (i * 16 + r) set when that list is a candidate of query j
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const uint32_t row = rbase + (r >> 2) * 8u + (r & 3);
-        const float v      = acc[i][r] + scn[buf * kTile + row];
+      for (int i = 0; i < 2; i++) {
+        const uint32_t rbase = wl * 64u + i * 32u + (lane >> 5) * 4u;  // row inside the block tile
+        float best           = neg_inf;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const uint32_t row = rbase + (r >> 2) * 8u + (r & 3);
+          const float v      = acc[i][j][r] + scn[buf * kTile + row];
+          if (PASS == 1) {
+            best = fmaxf(best, v);  // NaN scores are ignored here and never pass the threshold
+          } else {
+            hits |= (v >= limit[j]) ? (1u << (i * 16 + r)) : 0u;
+          }
+        }
         if (PASS == 1) {
-          best = fmaxf(best, v);  // NaN scores are ignored here and never pass the threshold
-        } else {
-          hits |= (v >= limit) ? (1u << (i * 16 + r)) : 0u;
+          lmin[qloc[j] * (kTilesPerBlock * 8u) + (tile - t0) * 8u + ((wl * 64u + i * 32u) >> 4) + (lane >> 5)] = alpha * best;
         }
       }
-      if (PASS == 1) {
-        lmin[qloc * (kTilesPerBlock * 8u) + (tile - t0) * 8u + ((wl * 64u + i * 32u) >> 4) + (lane >> 5)] = alpha * best;
-      }
-    }
-    if (PASS == 2 && hits != 0) {
-      uint32_t slot = atomicAdd(&lcount[qloc], uint32_t(__popc(hits)));
-      while (hits != 0) {
-        const uint32_t bit = __builtin_ctz(hits);
-        hits &= hits - 1u;
-        const uint32_t row = wl * 64u + (bit >> 4) * 32u + (lane >> 5) * 4u + ((bit & 15u) >> 2) * 8u + (bit & 3u);
-        if (slot < kLocalCap) { lcand[qloc * kLocalCap + slot] = l0 + row; }
-        slot++;
+      if (PASS == 2 && hits != 0) {
+        uint32_t slot = atomicAdd(&lcount[qloc[j]], uint32_t(__popc(hits)));
+        while (hits != 0) {
+          const uint32_t bit = __builtin_ctz(hits);
+          hits &= hits - 1u;
+          const uint32_t row = wl * 64u + (bit >> 4) * 32u + (lane >> 5) * 4u + ((bit & 15u) >> 2) * 8u + (bit & 3u);
+          if (slot < kLocalCap) { lcand[qloc[j] * kLocalCap + slot] = l0 + row; }
+          slot++;
+        }
       }
     }
   };
@@ -296,14 +316,14 @@ __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
   if (PASS == 1) {
     // the block's minima, 8 per tile and query, in runs of consecutive groups
     const uint32_t n_local = (t1 - t0) * 8u;
-    for (uint32_t e = tid; e < kTile * n_local; e += kGemmThreads) {
+    for (uint32_t e = tid; e < kQTile * n_local; e += kGemmThreads) {
       const uint32_t ql = e / n_local, g = e - ql * n_local;
       if (q0 + ql < n_queries) {
         minima[uint64_t(q0 + ql) * n_groups + t0 * 8u + g] = lmin[ql * (kTilesPerBlock * 8u) + g];
       }
     }
   }
-  if (PASS == 2 && tid < kTile && q0 + tid < n_queries) {
+  if (PASS == 2 && tid < kQTile && q0 + tid < n_queries) {
     const uint32_t n = lcount[tid];
     if (n != 0) {
       // more than the block can hold: push the query's count past the limit, it will be redone by
@@ -507,18 +527,39 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
   CUVS_HIP_TRY(hipGetLastError());
 
   // list tiles per block: the queries of a block are loaded once for all of them
-  const uint32_t n_list_tiles    = l_pad / kTile;
-  const uint32_t tiles_per_block = std::min<uint32_t>(kTilesPerBlock, n_list_tiles);
-  dim3 grid((n_list_tiles + tiles_per_block - 1) / tiles_per_block, q_pad / kTile);
+  const uint32_t n_list_tiles = l_pad / kTile;
+  // A block costs about two tile-times of set-up besides its tiles, and the grid runs in rounds of
+  // one block per CU: take the run length whose rounds x (tiles + 2) is smallest.
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0;
+    CUVS_HIP_TRY(hipGetDevice(&dev));
+    CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+  }
+  const uint32_t n_qblocks = (q_pad + kQTile - 1) / kQTile;
+  uint32_t tiles_per_block = 1;
+  uint64_t best_cost       = ~uint64_t(0);
+  for (uint32_t t = 1; t <= std::min<uint32_t>(kTilesPerBlock, n_list_tiles); t++) {
+    const uint64_t blocks = uint64_t((n_list_tiles + t - 1) / t) * n_qblocks;
+    const uint64_t rounds = (blocks + uint64_t(n_cu) - 1) / uint64_t(n_cu);
+    const uint64_t cost   = rounds * (t + 2);
+    if (cost <= best_cost) {
+      best_cost       = cost;
+      tiles_per_block = t;
+    }
+  }
+  dim3 grid((n_list_tiles + tiles_per_block - 1) / tiles_per_block, n_qblocks);
   auto run_pass = [&](auto k1, auto k2) {
-    const size_t smem = size_t(2) * kTile * (k_pad * 2 + 16) + 2 * kTile * 4 + size_t(kTile) * kTilesPerBlock * 8 * 4;
+    // list tiles (two buffers), their norm terms, and the larger of the two passes' per-query areas
+    const size_t smem = size_t(2) * kTile * (k_pad * 2 + 16) + 2 * kTile * 4 +
+                        std::max<size_t>(size_t(kQTile) * kTilesPerBlock * 8 * 4, size_t(kQTile) * (1 + kLocalCap) * 4);
     static bool attr_set = false;
     if (!attr_set) {
       CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k1), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
       CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k2), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
       attr_set = true;
     }
-    k1<<<grid, kGemmThreads, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, n_list_tiles, tiles_per_block, alpha,
+    k1<<<grid, kGemmThreads, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, q_pad, n_list_tiles, tiles_per_block, alpha,
                                     qterm, a.minima, n_groups, nullptr, nullptr, nullptr);
     CUVS_HIP_TRY(hipGetLastError());
     if (n_groups <= 16u * 64u) {
@@ -527,7 +568,7 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
       coarse_threshold_kernel<64><<<(a.n_queries + 3) / 4, 256, 0, stream>>>(a.minima, a.n_queries, n_groups, a.n_probes, a.qnorm, e_rel, e_abs, a.thr);
     }
     CUVS_HIP_TRY(hipGetLastError());
-    k2<<<grid, kGemmThreads, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, n_list_tiles, tiles_per_block, alpha,
+    k2<<<grid, kGemmThreads, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, q_pad, n_list_tiles, tiles_per_block, alpha,
                                     qterm, nullptr, n_groups, a.thr, a.cand_count, a.cand);
     CUVS_HIP_TRY(hipGetLastError());
   };
