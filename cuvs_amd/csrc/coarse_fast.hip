@@ -210,7 +210,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
   // compiler sinks them to their first use, behind the matrix products they are meant to overlap
   // (and as volatile loads it waits for each).  It does not count them, so the wait is explicit.
   // Tile numbers past the block's last tile repeat it (no branch around loads or stores).  (Loads
-  // two tiles ahead measured slower: the loop is not waiting on them.)
+  // two tiles ahead measured slower, before and after the waves went to 64 queries: the loop is
+  // not waiting on them but on its own phases.)
   u32x4 sx[PER_T];
   float cx = 0.0f;
   auto issue = [&](uint32_t tile, u32x4(&st)[PER_T], float& sc) __attribute__((always_inline)) {
