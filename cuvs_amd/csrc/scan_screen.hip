@@ -60,11 +60,11 @@ __device__ __forceinline__ float opaque_one_s()
  * its counter would serialise every wave of the grid on a single address (about 11 ns per add,
  * which bounds the kernel as soon as most pairs survive), so a wave collects up to
  * kSurvivorBatch records in an LDS area of its own and claims their slots with one add.
- * A record is 8 dwords: a full batch is one dword per lane.
+ * A record is 8 dwords: a full batch is four dwords per lane.
  */
-constexpr uint32_t kSurvivorBatch      = 8;
+constexpr uint32_t kSurvivorBatch      = 32;
 constexpr uint32_t kSurvivorBatchBytes = kSurvivorBatch * uint32_t(sizeof(pair_desc));
-static_assert(kSurvivorBatchBytes == 64 * 4, "a full batch is one dword per lane");
+static_assert(kSurvivorBatchBytes == 4 * 64 * 4, "a full batch is four dwords per lane");
 static_assert(offsetof(pair_desc, q) == 8 && offsetof(pair_desc, row_off) == 28, "record layout");
 
 __device__ __forceinline__ void flush_survivors(LDS_AS uint32_t* pending, uint32_t n, uint32_t lane,
@@ -74,7 +74,8 @@ __device__ __forceinline__ void flush_survivors(LDS_AS uint32_t* pending, uint32
   uint32_t pos = 0;
   if (lane == 0) { pos = atomicAdd(n_survivors, n); }
   pos = uint32_t(__builtin_amdgcn_readfirstlane(pos));
-  if (lane < n * 8u) { reinterpret_cast<uint32_t*>(survivors + pos)[lane] = pending[lane]; }
+  auto* dst = reinterpret_cast<uint32_t*>(survivors + pos);
+  for (uint32_t w = lane; w < n * 8u; w += 64u) { dst[w] = pending[w]; }
 }
 
 /** Adds a record to the wave's batch (all lanes call it; `n` is the same in all of them). */
