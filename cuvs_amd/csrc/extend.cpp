@@ -137,13 +137,27 @@ void extend(cuvs::resources const& res,
   if (labels_in != nullptr) {
     CUVS_HIP_TRY(hipMemcpyAsync(labels.ptr, labels_in, n_rows * sizeof(uint32_t),
                                 hipMemcpyDefault, s));
-  } else if (ix.metric != detail::DistanceType::InnerProduct && is_device_pointer(new_vectors)) {
-    // the nearest list under the index's own metric is the search path's coarse stage with one
-    // probe (for cosine the row's length does not change which centre has the largest product)
+  } else if ((ix.metric == detail::DistanceType::L2Expanded || ix.metric == detail::DistanceType::L2SqrtExpanded) &&
+             is_device_pointer(new_vectors)) {
+    // the nearest list under the index's own metric is the search path's coarse stage with one probe
     search_params sp;
     sp.n_probes = 1;
     select_clusters(res, sp, *idx, new_vectors, type, n_rows_signed, labels.as<uint32_t>());
     CUVS_HIP_TRY(hipStreamSynchronize(s));
+  } else if (cosine) {
+    // cosine: the same stage on the normalised rows.  (On the rows as they are the largest product
+    // is the same centre in exact arithmetic, but not always in fp32: the labels must be the ones
+    // the normalised rows get, as in the reference's predict step.)
+    const uint64_t label_chunk = chunk_rows_for(ix, n_rows);
+    row_stager label_stager(new_vectors, type, ix.dim, label_chunk);
+    search_params sp;
+    sp.n_probes = 1;
+    for (uint64_t r0 = 0; r0 < n_rows; r0 += label_chunk) {
+      const uint64_t n = std::min(label_chunk, n_rows - r0);
+      const float* xf  = label_stager.load(r0, n, true, s);
+      select_clusters(res, sp, *idx, xf, elem_type::f32, int64_t(n), labels.as<uint32_t>() + r0);
+    }
+    CUVS_HIP_TRY(hipStreamSynchronize(s));  // the stager goes out of scope
   } else {
     const uint64_t label_chunk = chunk_rows_for(ix, n_rows);
     row_stager label_stager(new_vectors, type, ix.dim, label_chunk);
