@@ -78,7 +78,9 @@ EXPORTED_SYMBOLS = [
     "cuvsGetLastErrorText", "cuvsSetLastErrorText", "cuvsGetLogLevel", "cuvsSetLogLevel",
     "cuvsResourcesCreate", "cuvsResourcesDestroy", "cuvsStreamSet", "cuvsStreamGet",
     "cuvsStreamSync", "cuvsDeviceIdGet", "cuvsResourcesSetWorkspacePool", "cuvsRMMAlloc",
-    "cuvsRMMFree", "cuvsVersionGet",
+    "cuvsRMMFree", "cuvsVersionGet", "cuvsRMMPoolMemoryResourceEnable",
+    "cuvsRMMAsyncMemoryResourceEnable", "cuvsRMMMemoryResourceReset", "cuvsRMMHostAlloc",
+    "cuvsRMMHostFree", "cuvsMatrixCopy", "cuvsMatrixSliceRows",
     "cuvsIvfPqIndexParamsCreate", "cuvsIvfPqIndexParamsDestroy", "cuvsIvfPqSearchParamsCreate",
     "cuvsIvfPqSearchParamsDestroy", "cuvsIvfPqIndexCreate", "cuvsIvfPqIndexDestroy",
     "cuvsIvfPqIndexGetNLists", "cuvsIvfPqIndexGetDim", "cuvsIvfPqIndexGetSize",
@@ -128,7 +130,14 @@ def lib():
     proto("cuvsStreamGet", res_t, P(C.c_void_p))
     proto("cuvsStreamSync", res_t)
     proto("cuvsDeviceIdGet", res_t, P(C.c_int))
-    proto("cuvsResourcesSetWorkspacePool", res_t, C.c_int)
+    proto("cuvsResourcesSetWorkspacePool", res_t, C.c_size_t)
+    proto("cuvsRMMPoolMemoryResourceEnable", C.c_int, C.c_int, C.c_bool)
+    proto("cuvsRMMAsyncMemoryResourceEnable")
+    proto("cuvsRMMMemoryResourceReset")
+    proto("cuvsRMMHostAlloc", P(C.c_void_p), C.c_size_t)
+    proto("cuvsRMMHostFree", C.c_void_p, C.c_size_t)
+    proto("cuvsMatrixCopy", res_t, T, T)
+    proto("cuvsMatrixSliceRows", res_t, T, C.c_int64, C.c_int64, T)
     proto("cuvsRMMAlloc", res_t, P(C.c_void_p), C.c_size_t)
     proto("cuvsRMMFree", res_t, C.c_void_p, C.c_size_t)
     proto("cuvsVersionGet", P(C.c_uint16), P(C.c_uint16), P(C.c_uint16))

@@ -66,31 +66,64 @@ cuvsError_t cuvsDeviceIdGet(cuvsResources_t res, int* device_id)
   });
 }
 
-cuvsError_t cuvsResourcesSetWorkspacePool(cuvsResources_t res, int percent_of_free_memory)
+cuvsError_t cuvsResourcesSetWorkspacePool(cuvsResources_t res, size_t initial_size_bytes)
 {
-  return cuvs::core::translate_exceptions([=] {
-    CUVS_EXPECTS(percent_of_free_memory > 0 && percent_of_free_memory <= 100,
-                 "percent_of_free_memory must be within (0, 100]");
-    size_t free_b = 0, total_b = 0;
-    CUVS_HIP_TRY(hipMemGetInfo(&free_b, &total_b));
-    cuvs::core::res_of(res)->set_workspace_limit(free_b / 100 * size_t(percent_of_free_memory));
-  });
+  return cuvs::core::translate_exceptions(
+    [=] { cuvs::core::res_of(res)->set_workspace_pool(initial_size_bytes); });
 }
 
 cuvsError_t cuvsRMMAlloc(cuvsResources_t res, void** ptr, size_t bytes)
 {
   return cuvs::core::translate_exceptions([=] {
-    (void)cuvs::core::res_of(res);
+    auto* r = cuvs::core::res_of(res);
     CUVS_EXPECTS(ptr != nullptr, "ptr must not be null");
-    CUVS_HIP_TRY(hipMalloc(ptr, bytes));
+    if (auto* own = r->workspace_pool()) {
+      *ptr = cuvs::memory::pool_allocate(*own, bytes, r->stream(), true);
+    } else {
+      *ptr = cuvs::memory::allocate_on_stream(bytes, r->stream());
+    }
   });
 }
 
 cuvsError_t cuvsRMMFree(cuvsResources_t res, void* ptr, size_t)
 {
   return cuvs::core::translate_exceptions([=] {
-    (void)cuvs::core::res_of(res);
-    CUVS_HIP_TRY(hipFree(ptr));
+    auto* r   = cuvs::core::res_of(res);
+    auto* own = r->workspace_pool();
+    if (ptr == nullptr || (own && cuvs::memory::pool_deallocate(*own, ptr, r->stream(), true))) { return; }
+    cuvs::memory::deallocate_on_stream(ptr, r->stream());
+  });
+}
+
+cuvsError_t cuvsRMMPoolMemoryResourceEnable(int initial_pool_size_percent, int max_pool_size_percent,
+                                            bool managed)
+{
+  return cuvs::core::translate_exceptions(
+    [=] { cuvs::memory::enable_pool(initial_pool_size_percent, max_pool_size_percent, managed); });
+}
+
+cuvsError_t cuvsRMMAsyncMemoryResourceEnable(void)
+{
+  return cuvs::core::translate_exceptions([] { cuvs::memory::enable_async(); });
+}
+
+cuvsError_t cuvsRMMMemoryResourceReset(void)
+{
+  return cuvs::core::translate_exceptions([] { cuvs::memory::reset(); });
+}
+
+cuvsError_t cuvsRMMHostAlloc(void** ptr, size_t bytes)
+{
+  return cuvs::core::translate_exceptions([=] {
+    CUVS_EXPECTS(ptr != nullptr, "ptr must not be null");
+    CUVS_HIP_TRY(hipHostMalloc(ptr, bytes == 0 ? 1 : bytes, hipHostMallocDefault));
+  });
+}
+
+cuvsError_t cuvsRMMHostFree(void* ptr, size_t)
+{
+  return cuvs::core::translate_exceptions([=] {
+    if (ptr != nullptr) { CUVS_HIP_TRY(hipHostFree(ptr)); }
   });
 }
 
@@ -101,6 +134,99 @@ cuvsError_t cuvsVersionGet(uint16_t* major, uint16_t* minor, uint16_t* patch)
     *major = 26;  // API level of the cuVS release whose search entry points are mirrored
     *minor = 10;
     *patch = 0;
+  });
+}
+
+cuvsError_t cuvsMatrixCopy(cuvsResources_t res, DLManagedTensor* src_managed,
+                           DLManagedTensor* dst_managed)
+{
+  return cuvs::core::translate_exceptions([=] {
+    auto* r = cuvs::core::res_of(res);
+    CUVS_EXPECTS(src_managed != nullptr && dst_managed != nullptr, "src and dst must not be null");
+    const DLTensor& src = src_managed->dl_tensor;
+    const DLTensor& dst = dst_managed->dl_tensor;
+    CUVS_EXPECTS(src.ndim == dst.ndim, "src and dst tensors should have the same dimensions");
+    for (int i = 0; i < src.ndim; ++i) {
+      CUVS_EXPECTS(src.shape[i] == dst.shape[i], "shape mismatch between src and dst tensors");
+    }
+    CUVS_EXPECTS(src.dtype.code == dst.dtype.code, "dtype mismatch between src and dst tensors");
+    CUVS_EXPECTS(src.dtype.bits == dst.dtype.bits,
+                 "dtype bits width mismatch between src and dst tensors");
+    const int bits       = src.dtype.bits;
+    const bool supported = (src.dtype.code == kDLFloat && (bits == 16 || bits == 32 || bits == 64)) ||
+                           ((src.dtype.code == kDLInt || src.dtype.code == kDLUInt) &&
+                            (bits == 8 || bits == 16 || bits == 32 || bits == 64));
+    CUVS_EXPECTS(supported && src.dtype.lanes == 1, "Unsupported dtype: %d and bits: %d",
+                 int(src.dtype.code), bits);
+    const size_t elt = size_t(bits) / 8;
+    if (src.ndim == 2) {
+      // rows may be further apart than their length on either side
+      CUVS_EXPECTS((src.strides == nullptr || src.strides[1] == 1 || src.shape[1] <= 1) &&
+                     (dst.strides == nullptr || dst.strides[1] == 1 || dst.shape[1] <= 1),
+                   "cuvsMatrixCopy needs unit stride along the rows");
+      const int64_t src_row = src.strides == nullptr ? src.shape[1] : src.strides[0];
+      const int64_t dst_row = dst.strides == nullptr ? dst.shape[1] : dst.strides[0];
+      CUVS_EXPECTS(src_row >= src.shape[1] && dst_row >= dst.shape[1], "row strides shorter than the rows");
+      if (src.shape[0] == 0 || src.shape[1] == 0) { return; }
+      CUVS_HIP_TRY(hipMemcpy2DAsync(cuvs::core::tensor_data(dst_managed), size_t(dst_row) * elt,
+                                    cuvs::core::tensor_data(src_managed), size_t(src_row) * elt,
+                                    size_t(src.shape[1]) * elt, size_t(src.shape[0]), hipMemcpyDefault,
+                                    r->stream()));
+    } else {
+      CUVS_EXPECTS(src.strides == nullptr && dst.strides == nullptr,
+                   "cuvsCopyMatrix only supports strides with 2D inputs");
+      size_t elements = 1;
+      for (int i = 0; i < src.ndim; ++i) { elements *= size_t(src.shape[i]); }
+      if (elements == 0) { return; }
+      CUVS_HIP_TRY(hipMemcpyAsync(cuvs::core::tensor_data(dst_managed), cuvs::core::tensor_data(src_managed),
+                                  elements * elt, hipMemcpyDefault, r->stream()));
+    }
+  });
+}
+
+/** Deleter of the views cuvsMatrixSliceRows makes: they own their shape and stride arrays only. */
+static void release_matrix_view(DLManagedTensor* tensor)
+{
+  delete[] tensor->dl_tensor.shape;
+  tensor->dl_tensor.shape = nullptr;
+  delete[] tensor->dl_tensor.strides;
+  tensor->dl_tensor.strides = nullptr;
+}
+
+cuvsError_t cuvsMatrixSliceRows(cuvsResources_t res, DLManagedTensor* src_managed, int64_t start,
+                                int64_t end, DLManagedTensor* dst_managed)
+{
+  return cuvs::core::translate_exceptions([=] {
+    (void)cuvs::core::res_of(res);
+    CUVS_EXPECTS(src_managed != nullptr && dst_managed != nullptr, "src and dst must not be null");
+    CUVS_EXPECTS(end >= start, "end index must be greater than start index");
+    const DLTensor& src = src_managed->dl_tensor;
+    DLTensor& dst       = dst_managed->dl_tensor;
+    CUVS_EXPECTS(src.ndim == 1 || src.ndim == 2, "src should be a 1 or 2 dimensional tensor");
+    CUVS_EXPECTS(src.shape != nullptr, "shape should be initialized in the src tensor");
+    CUVS_EXPECTS(start >= 0 && end <= src.shape[0], "rows [%lld, %lld) are outside the %lld rows of src",
+                 static_cast<long long>(start), static_cast<long long>(end),
+                 static_cast<long long>(src.shape[0]));
+    dst.dtype       = src.dtype;
+    dst.device      = src.device;
+    dst.ndim        = src.ndim;
+    dst.byte_offset = src.byte_offset;
+    dst.strides     = nullptr;
+    dst.shape       = new int64_t[dst.ndim];
+    dst.shape[0]    = end - start;
+    int64_t row_stride = 1;
+    if (dst.ndim == 2) {
+      dst.shape[1] = src.shape[1];
+      row_stride   = src.shape[1];
+      if (src.strides != nullptr) {
+        dst.strides    = new int64_t[2];
+        dst.strides[0] = src.strides[0];
+        dst.strides[1] = src.strides[1];
+        row_stride     = src.strides[0];
+      }
+    }
+    dst.data = static_cast<char*>(src.data) + start * row_stride * int64_t(dst.dtype.bits / 8);
+    dst_managed->deleter     = release_matrix_view;
   });
 }
 

@@ -8,6 +8,8 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include "memory.hpp"
+
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -40,7 +42,7 @@ namespace cuvs {
     }                                                                                       \
   } while (0)
 
-/** Owning device allocation. */
+/** Owning device allocation out of the process's current memory source. */
 struct device_buffer {
   void* ptr    = nullptr;
   size_t bytes = 0;
@@ -69,13 +71,13 @@ struct device_buffer {
   {
     release();
     if (n > 0) {
-      CUVS_HIP_TRY(hipMalloc(&ptr, n));
+      ptr   = memory::allocate(n);
       bytes = n;
     }
   }
   void release()
   {
-    if (ptr != nullptr) { (void)hipFree(ptr); }
+    memory::deallocate(ptr);
     ptr   = nullptr;
     bytes = 0;
   }

@@ -13,13 +13,39 @@ resources::resources()
 
 resources::~resources()
 {
-  if (workspace_ != nullptr) { (void)hipFree(workspace_); }
-  for (void* p : retired_) { (void)hipFree(p); }
+  // a pool of this handle's own returns everything it holds when it goes, right after this body
+  if (!(workspace_pooled_ && pool_)) { release_workspace(); }
+  for (void* p : retired_) { memory::deallocate(p); }
   extern void destroy_profile_state(resources::profile_state*);
   destroy_profile_state(prof);
 }
 
 void resources::sync() const { CUVS_HIP_TRY(hipStreamSynchronize(stream_)); }
+
+void resources::release_workspace()
+{
+  if (workspace_ == nullptr) { return; }
+  void* p             = workspace_;
+  workspace_          = nullptr;
+  workspace_capacity_ = 0;
+  if (workspace_pooled_ && pool_) {
+    (void)memory::pool_deallocate(*pool_, p, stream_, true);
+  } else {
+    memory::deallocate(p);
+  }
+}
+
+void resources::set_workspace_pool(size_t initial_bytes)
+{
+  CUVS_EXPECTS(workspace_used_ == 0, "the workspace pool cannot change while allocations are live");
+  const size_t own = (workspace_pooled_ && workspace_ != nullptr) ? 1 : 0;
+  CUVS_EXPECTS(!pool_ || memory::pool_live_allocations(*pool_) == own,
+               "the previous workspace pool still has live allocations");
+  auto next = memory::make_pool(initial_bytes, 0, false);
+  CUVS_HIP_TRY(hipStreamSynchronize(stream_));
+  release_workspace();
+  pool_ = std::move(next);
+}
 
 void resources::reserve_workspace(size_t bytes)
 {
@@ -27,11 +53,15 @@ void resources::reserve_workspace(size_t bytes)
   CUVS_EXPECTS(workspace_used_ == 0, "workspace cannot grow while allocations are live");
   // work queued earlier may still read the old block: wait, then release it
   CUVS_HIP_TRY(hipStreamSynchronize(stream_));
-  if (workspace_ != nullptr) { CUVS_HIP_TRY(hipFree(workspace_)); }
-  workspace_          = nullptr;
-  workspace_capacity_ = 0;
-  const size_t want   = round_up_u64(bytes + bytes / 8, size_t(1) << 20);
-  CUVS_HIP_TRY(hipMalloc(&workspace_, want));
+  release_workspace();
+  const size_t want = round_up_u64(bytes + bytes / 8, size_t(1) << 20);
+  if (pool_) {
+    workspace_        = memory::pool_allocate(*pool_, want, stream_, true);
+    workspace_pooled_ = true;
+  } else {
+    workspace_        = memory::allocate(want);
+    workspace_pooled_ = false;
+  }
   workspace_capacity_ = want;
 }
 

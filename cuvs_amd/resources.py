@@ -23,6 +23,11 @@ class Resources:
     def sync(self):
         check(lib().cuvsStreamSync(self._h))
 
+    def set_workspace_pool(self, initial_size_bytes):
+        """Give the handle a device memory pool of its own (cuvsResourcesSetWorkspacePool): the search
+        workspace then comes out of memory reserved here instead of a device allocation on first use."""
+        check(lib().cuvsResourcesSetWorkspacePool(self._h, C.c_size_t(int(initial_size_bytes))))
+
     def get_c_obj(self):
         return self._h
 
@@ -36,3 +41,18 @@ class Resources:
                 self._h = C.c_size_t(0)
         except Exception:
             pass
+
+
+def pool_memory_resource_enable(initial_pool_size_percent, max_pool_size_percent, managed=False):
+    """One device memory pool for the whole process (cuvsRMMPoolMemoryResourceEnable; the Go binding's
+    memory_resource.go:58 makes the same call)."""
+    check(lib().cuvsRMMPoolMemoryResourceEnable(int(initial_pool_size_percent), int(max_pool_size_percent),
+                                                bool(managed)))
+
+
+def async_memory_resource_enable():
+    check(lib().cuvsRMMAsyncMemoryResourceEnable())
+
+
+def memory_resource_reset():
+    check(lib().cuvsRMMMemoryResourceReset())

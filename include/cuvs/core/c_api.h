@@ -7,10 +7,13 @@
 #ifndef CUVS_AMD_C_API_H
 #define CUVS_AMD_C_API_H
 
+#include <stdbool.h>
 #include <stddef.h>
 #include <stdint.h>
 
 #include <hip/hip_runtime_api.h>
+
+#include <dlpack/dlpack.h>
 
 #include <cuvs/core/data_type.h>
 
@@ -59,14 +62,37 @@ CUVS_EXPORT cuvsError_t cuvsStreamGet(cuvsResources_t res, cudaStream_t* stream)
 CUVS_EXPORT cuvsError_t cuvsStreamSync(cuvsResources_t res);
 /** c_api.h:159 */
 CUVS_EXPORT cuvsError_t cuvsDeviceIdGet(cuvsResources_t res, int* device_id);
-/** c_api.h:175 -- caps the size of the cached workspace to the given percentage of device memory. */
-CUVS_EXPORT cuvsError_t cuvsResourcesSetWorkspacePool(cuvsResources_t res, int percent_of_free_memory);
-/** c_api.h:230 */
+/** c_api.h:175 -- gives the handle a device memory pool of its own: `initial_size_bytes` are
+ *  reserved now, the pool grows on demand and never shrinks before the handle is destroyed.  The
+ *  handle's search workspace and cuvsRMMAlloc / cuvsRMMFree on it are then served from the pool. */
+CUVS_EXPORT cuvsError_t cuvsResourcesSetWorkspacePool(cuvsResources_t res, size_t initial_size_bytes);
+/** c_api.h:230 -- device memory, ordered on the handle's stream. */
 CUVS_EXPORT cuvsError_t cuvsRMMAlloc(cuvsResources_t res, void** ptr, size_t bytes);
 /** c_api.h:240 */
 CUVS_EXPORT cuvsError_t cuvsRMMFree(cuvsResources_t res, void* ptr, size_t bytes);
+/** c_api.h:256 -- from now on the whole process (cuvsRMMAlloc and the library's own buffers)
+ *  draws device memory from one pool: `initial_pool_size_percent` of the free memory reserved at
+ *  once, growing up to `max_pool_size_percent`; `managed` takes the pool's blocks from
+ *  hipMallocManaged.  Memory handed out before stays valid and is released where it came from. */
+CUVS_EXPORT cuvsError_t cuvsRMMPoolMemoryResourceEnable(int initial_pool_size_percent,
+                                                        int max_pool_size_percent, bool managed);
+/** c_api.h:270 -- cuvsRMMAlloc / cuvsRMMFree become hipMallocAsync / hipFreeAsync on the handle's stream. */
+CUVS_EXPORT cuvsError_t cuvsRMMAsyncMemoryResourceEnable(void);
+/** c_api.h:276 -- back to plain hipMalloc / hipFree. */
+CUVS_EXPORT cuvsError_t cuvsRMMMemoryResourceReset(void);
+/** c_api.h:284 -- pinned host memory. */
+CUVS_EXPORT cuvsError_t cuvsRMMHostAlloc(void** ptr, size_t bytes);
+/** c_api.h:292 */
+CUVS_EXPORT cuvsError_t cuvsRMMHostFree(void* ptr, size_t bytes);
 /** c_api.h:301 */
 CUVS_EXPORT cuvsError_t cuvsVersionGet(uint16_t* major, uint16_t* minor, uint16_t* patch);
+/** c_api.h:318 -- copies `src` into the allocated `dst` of the same shape and dtype on the handle's
+ *  stream; either side may be host or device memory, and 2-D tensors may have padded rows. */
+CUVS_EXPORT cuvsError_t cuvsMatrixCopy(cuvsResources_t res, DLManagedTensor* src, DLManagedTensor* dst);
+/** c_api.h:329 -- makes `dst` a view of rows [start, end) of the 1-D or 2-D `src` (no copy); the
+ *  view's deleter frees the shape and stride arrays it owns. */
+CUVS_EXPORT cuvsError_t cuvsMatrixSliceRows(cuvsResources_t res, DLManagedTensor* src, int64_t start,
+                                            int64_t end, DLManagedTensor* dst);
 
 #ifdef __cplusplus
 }

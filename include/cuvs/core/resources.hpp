@@ -9,9 +9,14 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <memory>
 #include <stdexcept>
 #include <string>
 #include <vector>
+
+namespace cuvs::memory {
+class pool;  // sub-allocating device memory pool, internal to the library
+}
 
 // The library is built with hidden visibility; what this header declares is its C++ interface
 // (the reference marks the same namespaces CUVS_EXPORT).
@@ -84,6 +89,14 @@ class resources {
   void set_workspace_limit(size_t bytes) { workspace_limit_ = bytes; }
   size_t workspace_limit() const { return workspace_limit_; }
 
+  /**
+   * Give this handle a device memory pool of its own, reserved up front and growing on demand
+   * (role of raft::resource::set_workspace_resource with an rmm pool_memory_resource): the cached
+   * workspace and the C API's cuvsRMMAlloc / cuvsRMMFree on this handle then come out of it.
+   */
+  void set_workspace_pool(size_t initial_bytes);
+  memory::pool* workspace_pool() const { return pool_.get(); }
+
   /** Bump allocation out of the cached workspace; valid until the next reset_workspace(). */
   void* workspace_alloc(size_t bytes);
   /** Make sure the workspace can serve `bytes` in total before the first allocation of a call. */
@@ -104,6 +117,9 @@ class resources {
   size_t workspace_used_  = 0;
   size_t workspace_limit_ = 0;
   std::vector<void*> retired_;  // outgrown workspaces, released at destruction / next sync point
+  std::shared_ptr<memory::pool> pool_;  // set_workspace_pool
+  bool workspace_pooled_ = false;       // workspace_ came out of pool_
+  void release_workspace();
 };
 
 }  // namespace cuvs

@@ -1,6 +1,6 @@
-"""Callers written against the public headers alone, built by the host compilers: a C99 program on
-the C ABI (tests/c_abi/ivf_pq_roundtrip.c) and a C++17 program on the C++ interface
-(tests/c_abi/ivf_pq_cpp_caller.cpp).  Without a GPU: the headers compile (as pedantic C99 / C++17)
+"""Callers written against the public headers alone, built by the host compilers: C99 programs on
+the C ABI (tests/c_abi/ivf_pq_roundtrip.c, tests/c_abi/core_c_api.c) and a C++17 program on the C++
+interface (tests/c_abi/ivf_pq_cpp_caller.cpp).  Without a GPU: the headers compile (as pedantic C99 / C++17)
 and the programs link against the library; on the GPU they run."""
 import os
 import subprocess
@@ -10,6 +10,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 PROGRAMS = {"ivf_pq_roundtrip": ("gcc", "-std=c99", "ivf_pq_roundtrip.c"),
+            "core_c_api": ("gcc", "-std=c99", "core_c_api.c"),
             "ivf_pq_cpp_caller": ("g++", "-std=c++17", "ivf_pq_cpp_caller.cpp")}
 
 
