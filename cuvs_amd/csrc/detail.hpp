@@ -412,4 +412,29 @@ void launch_rows_by_label(const uint32_t* labels, uint64_t n, uint32_t n_lists, 
 void launch_unpack_contiguous(const uint8_t* list_data, uint32_t n_rows, uint32_t offset,
                               uint32_t pq_dim, uint32_t pq_bits, uint8_t* out, hipStream_t stream);
 
+/* Codes of one list outside the search (list_codes.hip).  `rows` selects rows of the list by
+ * position; null: rows offset .. offset + n_rows - 1. */
+/** out [n_rows, pq_dim]: one code per byte. */
+void launch_unpack_codes(const uint8_t* list_data, uint32_t n_rows, uint32_t offset,
+                         const uint32_t* rows, uint32_t pq_dim, uint32_t pq_bits, uint8_t* out,
+                         hipStream_t stream);
+/** Overwrites rows offset .. offset + n_rows - 1 of the list; `codes` holds one code per byte
+ *  ([n_rows, pq_dim]) or, `contiguous`, bit strings of ceil(pq_dim * pq_bits / 8) bytes per row. */
+void launch_pack_codes(uint8_t* list_data, const uint8_t* codes, bool contiguous, uint32_t n_rows,
+                       uint32_t offset, uint32_t pq_dim, uint32_t pq_bits, hipStream_t stream);
+/** out [n_rows, pq_dim * pq_len]: the rows decoded in the rotated space (centre + codebook entries);
+ *  `book_base` is the list's codebook (per-cluster) or the first subspace's (per-subspace). */
+void launch_reconstruct_rot(const uint8_t* list_data, uint32_t n_rows, uint32_t offset,
+                            const uint32_t* rows, uint32_t pq_dim, uint32_t pq_bits, uint32_t pq_len,
+                            const float* book_base, bool per_subspace, const float* center_rot,
+                            float* out, hipStream_t stream);
+/** float values back to the rows' element type (the inverse of the scaling applied on the way in). */
+void launch_unmap_rows(const float* in, uint64_t n_elems, elem_type type, void* out, hipStream_t stream);
+
+/** Gives every list room for `new_sizes[l]` rows (not less than it holds): lays the two arenas out
+ *  again, moves the stored rows, and updates the host and device tables.  The device list sizes
+ *  become `new_sizes` as well; rows past a list's old size are zero codes and id -1 until written.
+ *  Synchronises the stream. */
+void relayout_lists(const cuvs::resources& res, index_impl& ix, const std::vector<uint32_t>& new_sizes);
+
 }  // namespace cuvs::neighbors::ivf_pq::detail

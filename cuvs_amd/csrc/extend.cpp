@@ -113,6 +113,46 @@ detail::encode_args base_encode_args(const index_impl& ix)
 
 }  // namespace
 
+namespace detail {
+
+void relayout_lists(const cuvs::resources& res, index_impl& ix, const std::vector<uint32_t>& new_sizes)
+{
+  hipStream_t s = res.stream();
+  CUVS_EXPECTS(new_sizes.size() == ix.n_lists, "one size per list is needed");
+  std::vector<uint64_t> new_offsets(ix.n_lists + 1, 0);
+  for (uint32_t l = 0; l < ix.n_lists; l++) {
+    CUVS_EXPECTS(new_sizes[l] >= ix.h_list_sizes[l], "list %u cannot shrink while it is moved", l);
+    new_offsets[l + 1] = new_offsets[l] + round_up_u64(new_sizes[l], kIndexGroupSize);
+  }
+  const uint64_t total_rows = new_offsets[ix.n_lists];
+  // two groups of slack: the scan kernels read whole 64-row tiles past a list's last group
+  device_buffer new_codes((total_rows / kIndexGroupSize + 2) * ix.group_bytes());
+  device_buffer new_ids(total_rows * sizeof(int64_t));
+  if (new_codes.bytes > 0) { CUVS_HIP_TRY(hipMemsetAsync(new_codes.ptr, 0, new_codes.bytes, s)); }
+  if (new_ids.bytes > 0) { CUVS_HIP_TRY(hipMemsetAsync(new_ids.ptr, 0xFF, new_ids.bytes, s)); }
+
+  device_buffer d_old_off(sizeof(uint64_t) * (ix.n_lists + 1));
+  device_buffer d_new_off(sizeof(uint64_t) * (ix.n_lists + 1));
+  CUVS_HIP_TRY(hipMemcpyAsync(d_old_off.ptr, ix.h_row_offsets.data(), d_old_off.bytes,
+                              hipMemcpyHostToDevice, s));
+  CUVS_HIP_TRY(hipMemcpyAsync(d_new_off.ptr, new_offsets.data(), d_new_off.bytes,
+                              hipMemcpyHostToDevice, s));
+  if (ix.size > 0) {
+    launch_relocate_lists(ix.codes_arena.as<uint8_t>(), ix.ids_arena.as<int64_t>(),
+                          new_codes.as<uint8_t>(), new_ids.as<int64_t>(), d_old_off.as<uint64_t>(),
+                          d_new_off.as<uint64_t>(), ix.list_sizes.as<uint32_t>(), ix.n_lists,
+                          ix.n_chunks, s);
+  }
+  CUVS_HIP_TRY(hipStreamSynchronize(s));  // old arenas are released below
+  ix.codes_arena   = std::move(new_codes);
+  ix.ids_arena     = std::move(new_ids);
+  ix.h_list_sizes  = new_sizes;
+  ix.h_row_offsets = new_offsets;
+  ix.recompute_internal_state(s);
+}
+
+}  // namespace detail
+
 void extend(cuvs::resources const& res,
             const void* new_vectors,
             elem_type type,
@@ -188,43 +228,17 @@ void extend(cuvs::resources const& res,
 
   /* 3. new arena layout: every list owns round_up(size, 32) rows */
   std::vector<uint32_t> new_sizes(ix.n_lists);
-  std::vector<uint64_t> new_offsets(ix.n_lists + 1, 0);
   for (uint32_t l = 0; l < ix.n_lists; l++) {
     const uint64_t ns = uint64_t(ix.h_list_sizes[l]) + h_counts[l];
     CUVS_EXPECTS(ns <= 0xFFFFFFFFull, "list %u would exceed 2^32 rows", l);
-    new_sizes[l]       = uint32_t(ns);
-    new_offsets[l + 1] = new_offsets[l] + round_up_u64(ns, kIndexGroupSize);
+    new_sizes[l] = uint32_t(ns);
   }
-  const uint64_t total_rows = new_offsets[ix.n_lists];
-  // two groups of slack: the scan kernels read whole 64-row tiles past a list's last group
-  device_buffer new_codes((total_rows / kIndexGroupSize + 2) * ix.group_bytes());
-  device_buffer new_ids(total_rows * sizeof(int64_t));
-  if (new_codes.bytes > 0) { CUVS_HIP_TRY(hipMemsetAsync(new_codes.ptr, 0, new_codes.bytes, s)); }
-  if (new_ids.bytes > 0) { CUVS_HIP_TRY(hipMemsetAsync(new_ids.ptr, 0xFF, new_ids.bytes, s)); }
-
-  device_buffer d_old_off(sizeof(uint64_t) * (ix.n_lists + 1));
-  device_buffer d_new_off(sizeof(uint64_t) * (ix.n_lists + 1));
-  device_buffer cursors(sizeof(uint32_t) * ix.n_lists);
-  CUVS_HIP_TRY(hipMemcpyAsync(d_old_off.ptr, ix.h_row_offsets.data(), d_old_off.bytes,
-                              hipMemcpyHostToDevice, s));
-  CUVS_HIP_TRY(hipMemcpyAsync(d_new_off.ptr, new_offsets.data(), d_new_off.bytes,
-                              hipMemcpyHostToDevice, s));
   // cursors start at the old sizes (the device copy of list_sizes still holds them)
+  device_buffer cursors(sizeof(uint32_t) * ix.n_lists);
   CUVS_HIP_TRY(hipMemcpyAsync(cursors.ptr, ix.list_sizes.ptr, cursors.bytes,
                               hipMemcpyDeviceToDevice, s));
-  if (ix.size > 0) {
-    detail::launch_relocate_lists(ix.codes_arena.as<uint8_t>(), ix.ids_arena.as<int64_t>(),
-                                  new_codes.as<uint8_t>(), new_ids.as<int64_t>(),
-                                  d_old_off.as<uint64_t>(), d_new_off.as<uint64_t>(),
-                                  ix.list_sizes.as<uint32_t>(), ix.n_lists, ix.n_chunks, s);
-  }
-  CUVS_HIP_TRY(hipStreamSynchronize(s));  // old arenas are released below
   const int64_t first_id = ix.size;
-  ix.codes_arena         = std::move(new_codes);
-  ix.ids_arena           = std::move(new_ids);
-  ix.h_list_sizes        = new_sizes;
-  ix.h_row_offsets       = new_offsets;
-  ix.recompute_internal_state(s);
+  detail::relayout_lists(res, ix, new_sizes);
 
   /* 4. encode and append */
   device_buffer scratch(chunk * ix.rot_dim * sizeof(float));
@@ -325,6 +339,41 @@ void transform(cuvs::resources const& res,
     detail::launch_encode(a, s);
   }
   CUVS_HIP_TRY(hipStreamSynchronize(s));
+}
+
+/** Bit-contiguous codes of rows encoded against list `label` (no nearest-centre search): what
+ *  cuVS' encode_list_data computes for helpers::codepacker::extend_list (ivf_pq_build.cuh:931-944). */
+void encode_for_list(cuvs::resources const& res,
+                     const index<int64_t>& idx,
+                     const void* vectors,
+                     elem_type type,
+                     int64_t n_rows_signed,
+                     uint32_t label,
+                     uint8_t* codes_out)
+{
+  const auto& ix = *idx.impl();
+  CUVS_EXPECTS(ix.centers.ptr != nullptr, "the index has no trained model");
+  if (n_rows_signed <= 0) { return; }
+  const uint64_t n_rows    = uint64_t(n_rows_signed);
+  hipStream_t s            = res.stream();
+  const bool cosine        = ix.metric == detail::DistanceType::CosineExpanded;
+  const uint64_t chunk     = encode_chunk_rows_for(ix, n_rows);
+  const uint32_t row_bytes = (ix.pq_dim * ix.pq_bits + 7) / 8;
+  row_stager stager(vectors, type, ix.dim, chunk);
+  device_buffer labels(chunk * sizeof(uint32_t));
+  device_buffer scratch(chunk * ix.rot_dim * sizeof(float));
+  detail::launch_fill_u32(labels.as<uint32_t>(), label, chunk, s);
+  for (uint64_t r0 = 0; r0 < n_rows; r0 += chunk) {
+    const uint64_t n = std::min(chunk, n_rows - r0);
+    auto a           = base_encode_args(ix);
+    a.xf             = stager.load(r0, n, cosine, s);
+    a.n_rows         = n;
+    a.labels         = labels.as<uint32_t>();
+    a.flat_codes     = codes_out + r0 * row_bytes;
+    a.scratch        = scratch.as<float>();
+    detail::launch_encode(a, s);
+  }
+  CUVS_HIP_TRY(hipStreamSynchronize(s));  // the temporaries go out of scope
 }
 
 }  // namespace cuvs::neighbors::ivf_pq

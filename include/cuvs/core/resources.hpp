@@ -45,6 +45,21 @@ device_matrix_view<T> make_device_matrix_view(T* data, int64_t rows, int64_t col
   return device_matrix_view<T>{data, rows, cols};
 }
 
+/** Non-owning 1-D view (role of raft::device_vector_view<T, uint32_t>). */
+template <typename T>
+struct device_vector_view {
+  T* data      = nullptr;
+  int64_t size = 0;
+  T* data_handle() const { return data; }
+  int64_t extent(int) const { return size; }
+};
+
+template <typename T>
+device_vector_view<T> make_device_vector_view(T* data, int64_t size)
+{
+  return device_vector_view<T>{data, size};
+}
+
 /** Per-stage timing of a search (filled when profiling is enabled on the resources). */
 struct search_profile {
   uint32_t n_queries       = 0;

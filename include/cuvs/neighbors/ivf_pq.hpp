@@ -236,6 +236,113 @@ void unpack_contiguous_list_data(cuvs::resources const& res,
 void serialize(cuvs::resources const& res, const std::string& filename, const index<int64_t>& idx);
 void deserialize(cuvs::resources const& res, const std::string& filename, index<int64_t>* idx);
 
+/**
+ * Reading and editing single lists of an index (cuVS: namespace ivf_pq::helpers,
+ * cpp/include/cuvs/neighbors/ivf_pq.hpp:2559-3376).  All tensors are device memory; rows of a list
+ * are addressed by their position in the list.  The functions taking `index*` change it and, like
+ * `extend`, must not run concurrently with searches on it.
+ */
+namespace helpers {
+namespace codepacker {
+
+/** ivf_pq.hpp:2818 -- codes of rows offset .. offset + out_codes.extent(0) - 1 of list `label`, one
+ *  code per byte: out_codes is [n_take, pq_dim]. */
+void unpack_list_data(cuvs::resources const& res,
+                      const index<int64_t>& idx,
+                      device_matrix_view<uint8_t> out_codes,
+                      uint32_t label,
+                      uint32_t offset);
+
+/** ivf_pq.hpp:2854 -- the same for the rows at positions `in_cluster_indices`. */
+void unpack_list_data(cuvs::resources const& res,
+                      const index<int64_t>& idx,
+                      device_vector_view<const uint32_t> in_cluster_indices,
+                      device_matrix_view<uint8_t> out_codes,
+                      uint32_t label);
+
+/** ivf_pq.hpp:2895 -- rows as bit strings of ceil(pq_dim * pq_bits / 8) bytes. */
+void unpack_contiguous_list_data(cuvs::resources const& res,
+                                 const index<int64_t>& idx,
+                                 uint8_t* out_codes,
+                                 uint32_t n_rows,
+                                 uint32_t label,
+                                 uint32_t offset);
+
+/** ivf_pq.hpp:2739 -- overwrites the codes of rows offset .. offset + new_codes.extent(0) - 1 of
+ *  list `label` (which must exist already) with `new_codes` [n_rows, pq_dim], one code per byte. */
+void pack_list_data(cuvs::resources const& res,
+                    index<int64_t>* idx,
+                    device_matrix_view<const uint8_t> new_codes,
+                    uint32_t label,
+                    uint32_t offset);
+
+/** ivf_pq.hpp:2782 -- the same from bit-contiguous rows. */
+void pack_contiguous_list_data(cuvs::resources const& res,
+                               index<int64_t>* idx,
+                               const uint8_t* new_codes,
+                               uint32_t n_rows,
+                               uint32_t label,
+                               uint32_t offset);
+
+/** ivf_pq.hpp:2932-2950 -- decodes rows offset .. of list `label` to vectors of the original space:
+ *  out_vectors [n_take, dim] = rotation^T (rotated centre + codebook entries), mapped to T
+ *  (float, _Float16, int8_t, uint8_t). */
+template <typename T>
+void reconstruct_list_data(cuvs::resources const& res,
+                           const index<int64_t>& idx,
+                           device_matrix_view<T> out_vectors,
+                           uint32_t label,
+                           uint32_t offset);
+
+/** ivf_pq.hpp:2987-3002 -- the same for the rows at positions `in_cluster_indices`. */
+template <typename T>
+void reconstruct_list_data(cuvs::resources const& res,
+                           const index<int64_t>& idx,
+                           device_vector_view<const uint32_t> in_cluster_indices,
+                           device_matrix_view<T> out_vectors,
+                           uint32_t label);
+
+/** ivf_pq.hpp:3035 -- appends rows given by their codes ([n_rows, pq_dim], one per byte) and source
+ *  indices to list `label`, in the order given. */
+void extend_list_with_codes(cuvs::resources const& res,
+                            index<int64_t>* idx,
+                            device_matrix_view<const uint8_t> new_codes,
+                            device_vector_view<const int64_t> new_indices,
+                            uint32_t label);
+
+/** ivf_pq.hpp:3074 -- the same from bit-contiguous rows [n_rows, ceil(pq_dim * pq_bits / 8)]. */
+void extend_list_with_contiguous_codes(cuvs::resources const& res,
+                                       index<int64_t>* idx,
+                                       device_matrix_view<const uint8_t> new_codes,
+                                       device_vector_view<const int64_t> new_indices,
+                                       uint32_t label);
+
+/** ivf_pq.hpp:3109-3119 -- encodes `new_vectors` against list `label` (no nearest-centre search) and
+ *  appends them in the order given. */
+template <typename T>
+void extend_list(cuvs::resources const& res,
+                 index<int64_t>* idx,
+                 device_matrix_view<const T> new_vectors,
+                 device_vector_view<const int64_t> new_indices,
+                 uint32_t label);
+
+}  // namespace codepacker
+
+/** ivf_pq.hpp:3144 -- list `label` becomes empty. */
+void erase_list(cuvs::resources const& res, index<int64_t>* idx, uint32_t label);
+
+/** ivf_pq.hpp:3166 -- every list becomes empty; the trained model stays. */
+void reset_index(cuvs::resources const& res, index<int64_t>* idx);
+
+/** ivf_pq.hpp:3231-3236 -- the cluster centres without the norm column: `cluster_centers` is
+ *  [n_lists, dim] float in device or host memory. */
+void extract_centers(cuvs::resources const& res, const index<int64_t>& idx, float* cluster_centers);
+
+/** ivf_pq.hpp:3265 -- rebuilds the tables derived from the list sizes and addresses. */
+void recompute_internal_state(cuvs::resources const& res, index<int64_t>* idx);
+
+}  // namespace helpers
+
 }  // namespace ivf_pq
 }  // namespace cuvs::neighbors
 
