@@ -305,6 +305,21 @@ template void extend<_Float16>(cuvs::resources const&, device_matrix_view<const 
 template void extend<int8_t>(cuvs::resources const&, device_matrix_view<const int8_t>, const int64_t*, index<int64_t>*);
 template void extend<uint8_t>(cuvs::resources const&, device_matrix_view<const uint8_t>, const int64_t*, index<int64_t>*);
 
+template <typename T>
+index<int64_t> extend(cuvs::resources const& res,
+                      device_matrix_view<const T> new_vectors,
+                      const int64_t* new_indices,
+                      const index<int64_t>& orig)
+{
+  index<int64_t> out = clone(res, orig);
+  extend<T>(res, new_vectors, new_indices, &out);
+  return out;
+}
+template index<int64_t> extend<float>(cuvs::resources const&, device_matrix_view<const float>, const int64_t*, const index<int64_t>&);
+template index<int64_t> extend<_Float16>(cuvs::resources const&, device_matrix_view<const _Float16>, const int64_t*, const index<int64_t>&);
+template index<int64_t> extend<int8_t>(cuvs::resources const&, device_matrix_view<const int8_t>, const int64_t*, const index<int64_t>&);
+template index<int64_t> extend<uint8_t>(cuvs::resources const&, device_matrix_view<const uint8_t>, const int64_t*, const index<int64_t>&);
+
 void transform(cuvs::resources const& res,
                const index<int64_t>& idx,
                const void* vectors,

@@ -217,6 +217,55 @@ index<int64_t> build(cuvs::resources const& res,
   return idx;
 }
 
+index<int64_t> clone(cuvs::resources const& res, const index<int64_t>& source)
+{
+  CUVS_EXPECTS(source.impl() != nullptr, "index must not be null");
+  const auto& src = *source.impl();
+  index<int64_t> out;
+  auto& dst          = *out.impl();
+  hipStream_t stream = res.stream();
+  auto copy          = [&](device_buffer& to, const device_buffer& from) {
+    to.allocate(from.bytes);
+    if (from.bytes > 0) {
+      CUVS_HIP_TRY(hipMemcpyAsync(to.ptr, from.ptr, from.bytes, hipMemcpyDeviceToDevice, stream));
+    }
+  };
+  dst.metric                         = src.metric;
+  dst.codebook_kind                  = src.codebook_kind;
+  dst.conservative_memory_allocation = src.conservative_memory_allocation;
+  dst.n_lists                        = src.n_lists;
+  dst.dim                            = src.dim;
+  dst.pq_bits                        = src.pq_bits;
+  dst.pq_dim                         = src.pq_dim;
+  dst.dim_ext                        = src.dim_ext;
+  dst.pq_len                         = src.pq_len;
+  dst.rot_dim                        = src.rot_dim;
+  dst.book_size                      = src.book_size;
+  dst.n_chunks                       = src.n_chunks;
+  dst.c_max                          = src.c_max;
+  dst.n_max                          = src.n_max;
+  dst.coarse_fast_ok                 = src.coarse_fast_ok;
+  dst.rotation_is_identity           = src.rotation_is_identity;
+  copy(dst.centers, src.centers);
+  copy(dst.centers_rot, src.centers_rot);
+  copy(dst.rotation, src.rotation);
+  copy(dst.rotation_t, src.rotation_t);
+  copy(dst.pq_centers, src.pq_centers);
+  copy(dst.centers_t, src.centers_t);
+  copy(dst.centers_h, src.centers_h);
+  copy(dst.center_norms, src.center_norms);
+  copy(dst.codes_arena, src.codes_arena);
+  copy(dst.ids_arena, src.ids_arena);
+  copy(dst.lead_plane, src.lead_plane);
+  dst.h_list_sizes  = src.h_list_sizes;
+  dst.h_row_offsets = src.h_row_offsets;
+  dst.list_sizes.allocate(sizeof(uint32_t) * dst.n_lists);
+  dst.data_ptrs.allocate(sizeof(void*) * dst.n_lists);
+  dst.inds_ptrs.allocate(sizeof(void*) * dst.n_lists);
+  dst.recompute_internal_state(stream);  // the tables point into the copy's own arenas; synchronises
+  return out;
+}
+
 void unpack_contiguous_list_data(cuvs::resources const& res,
                                  const index<int64_t>& idx,
                                  uint8_t* out_codes,

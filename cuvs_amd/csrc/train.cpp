@@ -312,4 +312,16 @@ template index<int64_t> build<_Float16>(cuvs::resources const&, const index_para
 template index<int64_t> build<int8_t>(cuvs::resources const&, const index_params&, device_matrix_view<const int8_t>);
 template index<int64_t> build<uint8_t>(cuvs::resources const&, const index_params&, device_matrix_view<const uint8_t>);
 
+template <typename T>
+void build(cuvs::resources const& res, const index_params& params, device_matrix_view<const T> dataset,
+           index<int64_t>* idx)
+{
+  CUVS_EXPECTS(idx != nullptr, "index must not be null");
+  *idx = build<T>(res, params, dataset);
+}
+template void build<float>(cuvs::resources const&, const index_params&, device_matrix_view<const float>, index<int64_t>*);
+template void build<_Float16>(cuvs::resources const&, const index_params&, device_matrix_view<const _Float16>, index<int64_t>*);
+template void build<int8_t>(cuvs::resources const&, const index_params&, device_matrix_view<const int8_t>, index<int64_t>*);
+template void build<uint8_t>(cuvs::resources const&, const index_params&, device_matrix_view<const uint8_t>, index<int64_t>*);
+
 }  // namespace cuvs::neighbors::ivf_pq

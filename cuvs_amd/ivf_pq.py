@@ -74,10 +74,16 @@ class IndexParams:
     add_data_on_build = property(lambda self: bool(self._p.contents.add_data_on_build))
     conservative_memory_allocation = property(lambda self: bool(self._p.contents.conservative_memory_allocation))
     max_train_points_per_pq_code = property(lambda self: self._p.contents.max_train_points_per_pq_code)
+    codebook_kind = property(lambda self: self._p.contents.codebook_kind)
+    codes_layout = property(lambda self: "flat" if self._p.contents.codes_layout == 0 else "interleaved")
 
     @property
     def params(self):
         return self._p.contents
+
+    def get_handle(self):
+        """Address of the C parameter struct (ivf_pq.pyx:236)."""
+        return C.cast(self._p, C.c_void_p).value
 
     def __del__(self):
         try:
@@ -109,6 +115,10 @@ class SearchParams:
     internal_distance_dtype = property(lambda self: self.params.internal_distance_dtype)
     coarse_search_dtype = property(lambda self: self.params.coarse_search_dtype)
     max_internal_batch_size = property(lambda self: self.params.max_internal_batch_size)
+
+    def get_handle(self):
+        """Address of the C parameter struct (ivf_pq.pyx:739)."""
+        return C.cast(self._p, C.c_void_p).value
 
     def __del__(self):
         try:

@@ -165,6 +165,17 @@ index<int64_t> build(cuvs::resources const& res,
                      const index_params& params,
                      device_matrix_view<const T> dataset);
 
+/** ivf_pq.hpp:732-890 -- the same, into an index object the caller holds. */
+template <typename T>
+void build(cuvs::resources const& res,
+           const index_params& params,
+           device_matrix_view<const T> dataset,
+           index<int64_t>* idx);
+
+/** A deep copy of an index: model, lists and tables in memory of its own (cuVS detail::clone,
+ *  ivf_pq_build.cuh:962-996, shares the list data between the two until one of them is extended). */
+index<int64_t> clone(cuvs::resources const& res, const index<int64_t>& source);
+
 /** Encode and append rows.  `new_vectors` and `new_indices` are device pointers; a null
  *  `new_indices` numbers the rows consecutively from the current size.  A non-null `labels`
  *  (device uint32 [n]) overrides the nearest-centre assignment. */
@@ -181,6 +192,14 @@ void extend(cuvs::resources const& res,
             device_matrix_view<const T> new_vectors,
             const int64_t* new_indices,
             index<int64_t>* idx);
+
+/** ivf_pq.hpp:1296-1737 (the forms that return an index) -- `orig` stays as it is; the result holds
+ *  its rows and the new ones. */
+template <typename T>
+index<int64_t> extend(cuvs::resources const& res,
+                      device_matrix_view<const T> new_vectors,
+                      const int64_t* new_indices,
+                      const index<int64_t>& orig);
 
 /** Labels and bit-contiguous codes of rows, without modifying the index (cuVS: transform). */
 void transform(cuvs::resources const& res,

@@ -326,6 +326,36 @@ void run(uint32_t pq_bits, ivf_pq::codebook_gen kind, const std::vector<float>& 
   again = search_all(res, index, d_data, n_queries, k);
   REQUIRE(again.dist == before_search.dist);  // the same rows under the same model
 
+  /* copies: a clone is independent of its source; extend that returns an index leaves `orig` alone */
+  {
+    const auto base = search_all(res, index, d_data, n_queries, k);
+    auto copy       = ivf_pq::clone(res, index);
+    const auto same = search_all(res, copy, d_data, n_queries, k);
+    REQUIRE(same.ids == base.ids && same.dist == base.dist);
+    ivf_pq::helpers::erase_list(res, &copy, label);
+    REQUIRE(copy.size() == n_rows - int64_t(to_host(index.list_sizes(), n_lists)[label]) && index.size() == n_rows);
+    auto grown = ivf_pq::extend<float>(res, make_device_matrix_view<const float>(d_data, 500, dim), nullptr, index);
+    REQUIRE(index.size() == n_rows && grown.size() == n_rows + 500);
+    const auto still = search_all(res, index, d_data, n_queries, k);
+    REQUIRE(still.ids == base.ids && still.dist == base.dist);
+    // rows 0 .. 499 are in `grown` twice, as ids i and n_rows + i, with the same code in the same list
+    const auto twice = search_all(res, grown, d_data, n_queries, k);
+    for (int64_t q = 0; q < n_queries; q++) {
+      for (int64_t r = 0; r + 1 < k; r++) {
+        const int64_t id = twice.ids[q * k + r];
+        if (id >= 500 && id < n_rows) { continue; }
+        const int64_t twin = id < 500 ? id + n_rows : id - n_rows;
+        REQUIRE(std::count(twice.ids.begin() + q * k, twice.ids.begin() + (q + 1) * k, twin) == 1 ||
+                twice.dist[q * k + r] == twice.dist[q * k + k - 1]);
+      }
+    }
+    ivf_pq::index<int64_t> held;
+    ivf_pq::index_params untrained = ip;
+    untrained.add_data_on_build    = false;
+    ivf_pq::build<float>(res, untrained, make_device_matrix_view<const float>(d_data, n_rows, dim), &held);
+    REQUIRE(held.n_lists() == n_lists && held.size() == 0 && held.pq_bits() == pq_bits);
+  }
+
   for (void* p : {static_cast<void*>(d_data), static_cast<void*>(d_codes), static_cast<void*>(d_part), static_cast<void*>(d_picks),
                   static_cast<void*>(d_flat), static_cast<void*>(d_ids), static_cast<void*>(d_rec),
                   static_cast<void*>(d_i8), static_cast<void*>(d_u8), static_cast<void*>(d_codes_2), static_cast<void*>(d_rec_2)}) {
