@@ -431,6 +431,10 @@ void launch_reconstruct_rot(const uint8_t* list_data, uint32_t n_rows, uint32_t 
 /** float values back to the rows' element type (the inverse of the scaling applied on the way in). */
 void launch_unmap_rows(const float* in, uint64_t n_elems, elem_type type, void* out, hipStream_t stream);
 
+/** rotation [rot_dim, dim] on the host: the identity unless a random one is asked for or needed
+ *  (rot_dim != dim): then `dim` orthonormal columns (train.cpp). */
+std::vector<float> make_rotation(uint32_t rot_dim, uint32_t dim, bool force_random);
+
 /** Gives every list room for `new_sizes[l]` rows (not less than it holds): lays the two arenas out
  *  again, moves the stored rows, and updates the host and device tables.  The device list sizes
  *  become `new_sizes` as well; rows past a list's old size are zero codes and id -1 until written.

@@ -303,6 +303,67 @@ void extract_centers(cuvs::resources const& res, const index<int64_t>& idx, floa
                                 ix.n_lists, hipMemcpyDefault, res.stream()));
 }
 
+void pad_centers_with_norms(cuvs::resources const& res, device_matrix_view<const float> centers,
+                            device_matrix_view<float> padded_centers)
+{
+  const int64_t n = centers.extent(0), dim = centers.extent(1), dim_ext = padded_centers.extent(1);
+  CUVS_EXPECTS(padded_centers.extent(0) == n, "centers and padded_centers must have the same number of rows");
+  CUVS_EXPECTS(dim > 0 && dim_ext > dim, "padded_centers needs at least one column more than centers");
+  if (n == 0) { return; }
+  hipStream_t s    = res.stream();
+  const float* src = centers.data_handle();
+  device_buffer stage;
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, src) != hipSuccess || attr.type == hipMemoryTypeUnregistered) {
+    (void)hipGetLastError();
+    stage.allocate(size_t(n) * dim * sizeof(float));
+    CUVS_HIP_TRY(hipMemcpyAsync(stage.ptr, src, stage.bytes, hipMemcpyHostToDevice, s));
+    src = stage.as<float>();
+  }
+  detail::launch_set_centers(src, uint32_t(n), uint32_t(dim), uint32_t(dim_ext), padded_centers.data_handle(), s);
+  CUVS_HIP_TRY(hipStreamSynchronize(s));  // the staging copy goes out of scope
+}
+
+void rotate_padded_centers(cuvs::resources const& res, device_matrix_view<const float> padded_centers,
+                           device_matrix_view<const float> rotation_matrix,
+                           device_matrix_view<float> rotated_centers)
+{
+  const int64_t n = padded_centers.extent(0), dim_ext = padded_centers.extent(1);
+  const int64_t rot_dim = rotation_matrix.extent(0), dim = rotation_matrix.extent(1);
+  CUVS_EXPECTS(rotated_centers.extent(0) == n && rotated_centers.extent(1) == rot_dim,
+               "rotated_centers must be [n_centers, rot_dim]");
+  CUVS_EXPECTS(dim_ext > dim, "padded_centers must be wider than the rotation matrix's dim");
+  if (n == 0) { return; }
+  hipStream_t s = res.stream();
+  // the rows without their padding, then the rotation applied to each: y = R x
+  device_buffer flat(size_t(n) * dim * sizeof(float)), rot_t(size_t(rot_dim) * dim * sizeof(float));
+  CUVS_HIP_TRY(hipMemcpy2DAsync(flat.ptr, size_t(dim) * sizeof(float), padded_centers.data_handle(),
+                                size_t(dim_ext) * sizeof(float), size_t(dim) * sizeof(float), size_t(n),
+                                hipMemcpyDeviceToDevice, s));
+  std::vector<float> r(size_t(rot_dim) * dim), rt(size_t(rot_dim) * dim);
+  CUVS_HIP_TRY(hipMemcpyAsync(r.data(), rotation_matrix.data_handle(), r.size() * sizeof(float),
+                              hipMemcpyDefault, s));
+  CUVS_HIP_TRY(hipStreamSynchronize(s));
+  for (int64_t o = 0; o < rot_dim; o++) {
+    for (int64_t d = 0; d < dim; d++) { rt[size_t(d) * rot_dim + o] = r[size_t(o) * dim + d]; }
+  }
+  CUVS_HIP_TRY(hipMemcpyAsync(rot_t.ptr, rt.data(), rt.size() * sizeof(float), hipMemcpyHostToDevice, s));
+  detail::launch_rotate(flat.as<float>(), rot_t.as<float>(), uint32_t(n), uint32_t(dim), uint32_t(rot_dim),
+                        false, false, rotated_centers.data_handle(), s);
+  CUVS_HIP_TRY(hipStreamSynchronize(s));  // the temporaries go out of scope
+}
+
+void make_rotation_matrix(cuvs::resources const& res, device_matrix_view<float> rotation_matrix,
+                          bool force_random_rotation)
+{
+  const int64_t rot_dim = rotation_matrix.extent(0), dim = rotation_matrix.extent(1);
+  CUVS_EXPECTS(rot_dim >= dim && dim > 0, "the rotation matrix is [rot_dim, dim] with rot_dim >= dim");
+  const std::vector<float> r = detail::make_rotation(uint32_t(rot_dim), uint32_t(dim), force_random_rotation);
+  CUVS_HIP_TRY(hipMemcpyAsync(rotation_matrix.data_handle(), r.data(), r.size() * sizeof(float),
+                              hipMemcpyHostToDevice, res.stream()));
+  CUVS_HIP_TRY(hipStreamSynchronize(res.stream()));  // `r` goes out of scope
+}
+
 void recompute_internal_state(cuvs::resources const& res, index<int64_t>* idx)
 {
   CUVS_EXPECTS(idx != nullptr && idx->impl() != nullptr, "index must not be null");

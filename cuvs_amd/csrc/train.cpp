@@ -100,6 +100,10 @@ uint32_t balance_pairs(const std::vector<uint32_t>& sizes, uint64_t n_rows, std:
   return uint32_t(receivers.size());
 }
 
+}  // namespace
+
+namespace detail {
+
 /** rotation [rot_dim, dim]: the identity (zero-padded) unless a random one is asked for or needed
  *  (make_rotation_matrix, ivf_pq_build_common.cu:235-261): then `dim` orthonormal columns. */
 std::vector<float> make_rotation(uint32_t rot_dim, uint32_t dim, bool force_random)
@@ -134,7 +138,8 @@ std::vector<float> make_rotation(uint32_t rot_dim, uint32_t dim, bool force_rand
   return r;
 }
 
-}  // namespace
+
+}  // namespace detail
 
 index<int64_t> build(cuvs::resources const& res_c,
                      const index_params& params,
@@ -226,7 +231,7 @@ index<int64_t> build(cuvs::resources const& res_c,
   assign();  // labels of the training rows under the final centres (ivf_pq_build.cuh:1361-1369)
 
   /* 3. rotation and rotated centres */
-  const std::vector<float> rot = make_rotation(cx.rot_dim, dim, params.force_random_rotation);
+  const std::vector<float> rot = detail::make_rotation(cx.rot_dim, dim, params.force_random_rotation);
   std::vector<float> rot_t(rot.size());
   bool identity = cx.rot_dim == dim;
   for (uint32_t o = 0; o < cx.rot_dim; o++) {

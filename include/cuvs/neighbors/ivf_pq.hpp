@@ -357,6 +357,26 @@ void reset_index(cuvs::resources const& res, index<int64_t>* idx);
  *  [n_lists, dim] float in device or host memory. */
 void extract_centers(cuvs::resources const& res, const index<int64_t>& idx, float* cluster_centers);
 
+/** ivf_pq.hpp:3179-3195 -- `padded_centers` [n_centers, dim_ext] (device) = the rows of `centers`
+ *  [n_centers, dim] (device or host), their squared L2 norm in column dim, zeros behind it: the form
+ *  `build` from a precomputed model takes. */
+void pad_centers_with_norms(cuvs::resources const& res,
+                            device_matrix_view<const float> centers,
+                            device_matrix_view<float> padded_centers);
+
+/** ivf_pq.hpp:3208 -- `rotated_centers` [n_centers, rot_dim] = rotation_matrix [rot_dim, dim] applied
+ *  to the first dim columns of `padded_centers`. */
+void rotate_padded_centers(cuvs::resources const& res,
+                           device_matrix_view<const float> padded_centers,
+                           device_matrix_view<const float> rotation_matrix,
+                           device_matrix_view<float> rotated_centers);
+
+/** ivf_pq.hpp:3292 -- fills `rotation_matrix` [rot_dim, dim] (device): the identity when rot_dim == dim
+ *  and no random rotation is asked for, else a matrix with orthonormal columns. */
+void make_rotation_matrix(cuvs::resources const& res,
+                          device_matrix_view<float> rotation_matrix,
+                          bool force_random_rotation);
+
 /** ivf_pq.hpp:3265 -- rebuilds the tables derived from the list sizes and addresses. */
 void recompute_internal_state(cuvs::resources const& res, index<int64_t>* idx);
 

@@ -356,6 +356,72 @@ void run(uint32_t pq_bits, ivf_pq::codebook_gen kind, const std::vector<float>& 
     REQUIRE(held.n_lists() == n_lists && held.size() == 0 && held.pq_bits() == pq_bits);
   }
 
+  /* a model put together from its parts with the centre / rotation helpers is the trained model */
+  {
+    const uint32_t dim_ext = index.dim_ext();
+    auto* d_flat_centres   = device_array<float>(size_t(n_lists) * dim);
+    ivf_pq::helpers::extract_centers(res, index, d_flat_centres);
+    auto* d_padded  = device_array<float>(size_t(n_lists) * dim_ext);
+    auto* d_padded2 = device_array<float>(size_t(n_lists) * dim_ext);
+    ivf_pq::helpers::pad_centers_with_norms(res, make_device_matrix_view<const float>(d_flat_centres, n_lists, dim),
+                                            make_device_matrix_view(d_padded, n_lists, dim_ext));
+    ivf_pq::helpers::pad_centers_with_norms(res, make_device_matrix_view<const float>(centres.data(), n_lists, dim),
+                                            make_device_matrix_view(d_padded2, n_lists, dim_ext));  // from the host
+    const auto padded = to_host(d_padded, size_t(n_lists) * dim_ext);
+    REQUIRE(padded == to_host(d_padded2, size_t(n_lists) * dim_ext));
+    for (uint32_t l = 0; l < n_lists; l++) {
+      double ss = 0.0;
+      for (uint32_t d = 0; d < dim; d++) {
+        REQUIRE(padded[size_t(l) * dim_ext + d] == centres[size_t(l) * dim + d]);
+        ss += double(centres[size_t(l) * dim + d]) * double(centres[size_t(l) * dim + d]);
+      }
+      REQUIRE(std::fabs(double(padded[size_t(l) * dim_ext + dim]) - ss) <= 1e-5 * ss);
+      for (uint32_t d = dim + 1; d < dim_ext; d++) { REQUIRE(padded[size_t(l) * dim_ext + d] == 0.0f); }
+    }
+    auto* d_rotation = device_array<float>(size_t(rot_dim) * dim);
+    ivf_pq::helpers::make_rotation_matrix(res, make_device_matrix_view(d_rotation, rot_dim, dim), false);
+    REQUIRE(to_host(d_rotation, size_t(rot_dim) * dim) == rotation);  // rot_dim == dim here: the identity
+    auto* d_rotated = device_array<float>(size_t(n_lists) * rot_dim);
+    ivf_pq::helpers::rotate_padded_centers(res, make_device_matrix_view<const float>(d_padded, n_lists, dim_ext),
+                                           make_device_matrix_view<const float>(d_rotation, rot_dim, dim),
+                                           make_device_matrix_view(d_rotated, n_lists, rot_dim));
+    REQUIRE(to_host(d_rotated, size_t(n_lists) * rot_dim) == centers_rot);
+    auto rebuilt = ivf_pq::build(res, ip, dim, index.pq_centers(), d_padded, d_rotated, d_rotation);
+    ivf_pq::extend<float>(res, make_device_matrix_view<const float>(d_data, n_rows, dim), nullptr, &rebuilt);
+    const auto base = search_all(res, index, d_data, n_queries, k);
+    const auto same = search_all(res, rebuilt, d_data, n_queries, k);
+    REQUIRE(same.dist == base.dist);
+    // a random rotation to a wider space: orthonormal columns, and rotated centres = R c
+    const uint32_t wide = dim + 8;
+    auto* d_wide = device_array<float>(size_t(wide) * dim);
+    ivf_pq::helpers::make_rotation_matrix(res, make_device_matrix_view(d_wide, wide, dim), true);
+    const auto r = to_host(d_wide, size_t(wide) * dim);
+    for (uint32_t a = 0; a < dim; a++) {
+      for (uint32_t b = 0; b <= a; b++) {
+        double dot = 0.0;
+        for (uint32_t o = 0; o < wide; o++) { dot += double(r[size_t(o) * dim + a]) * double(r[size_t(o) * dim + b]); }
+        REQUIRE(std::fabs(dot - (a == b ? 1.0 : 0.0)) < 1e-5);
+      }
+    }
+    auto* d_rotated_wide = device_array<float>(size_t(n_lists) * wide);
+    ivf_pq::helpers::rotate_padded_centers(res, make_device_matrix_view<const float>(d_padded, n_lists, dim_ext),
+                                           make_device_matrix_view<const float>(d_wide, wide, dim),
+                                           make_device_matrix_view(d_rotated_wide, n_lists, wide));
+    const auto rotated_wide = to_host(d_rotated_wide, size_t(n_lists) * wide);
+    for (uint32_t l = 0; l < n_lists; l += 7) {
+      for (uint32_t o = 0; o < wide; o++) {
+        double y = 0.0;
+        for (uint32_t d = 0; d < dim; d++) { y += double(r[size_t(o) * dim + d]) * double(centres[size_t(l) * dim + d]); }
+        REQUIRE(std::fabs(double(rotated_wide[size_t(l) * wide + o]) - y) < 1e-5);
+      }
+    }
+    for (void* p : {static_cast<void*>(d_flat_centres), static_cast<void*>(d_padded), static_cast<void*>(d_padded2),
+                    static_cast<void*>(d_rotation), static_cast<void*>(d_rotated), static_cast<void*>(d_wide),
+                    static_cast<void*>(d_rotated_wide)}) {
+      REQUIRE(hipFree(p) == hipSuccess);
+    }
+  }
+
   for (void* p : {static_cast<void*>(d_data), static_cast<void*>(d_codes), static_cast<void*>(d_part), static_cast<void*>(d_picks),
                   static_cast<void*>(d_flat), static_cast<void*>(d_ids), static_cast<void*>(d_rec),
                   static_cast<void*>(d_i8), static_cast<void*>(d_u8), static_cast<void*>(d_codes_2), static_cast<void*>(d_rec_2)}) {
