@@ -217,7 +217,9 @@ void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries,
                    hipStream_t stream);
 
 /** chunk_indices[q, p] = inclusive prefix sum of list_sizes[probes[q, p]]; n_samples[q] = total.
- *  When `stats` is non-null, adds the scanned bytes and rows to stats[0], stats[1]. */
+ *  When `stats` is non-null (kStatSlots x 4 words), query q adds the scanned bytes, the rows and
+ *  the bytes of its leading probes to words 0, 1, 2 of slot q % kStatSlots. */
+constexpr uint32_t kStatSlots = 256;
 void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
                           uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
                           uint32_t* n_samples, unsigned long long* stats, uint32_t lead_probes,

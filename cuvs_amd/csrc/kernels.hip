@@ -435,9 +435,12 @@ __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __res
       lead_rows += __shfl_down(lead_rows, d, 64);
     }
     if (lane == 0) {
-      atomicAdd(&stats[0], padded_rows * row_chunk_bytes);
-      atomicAdd(&stats[1], static_cast<unsigned long long>(carry));
-      atomicAdd(&stats[2], lead_rows * row_chunk_bytes);
+      // kStatSlots partial sums (the host adds them up): thousands of waves adding to one
+      // address would serialise and show up in the stage times being measured
+      unsigned long long* slot = stats + uint64_t(q % kStatSlots) * 4;
+      atomicAdd(&slot[0], padded_rows * row_chunk_bytes);
+      atomicAdd(&slot[1], static_cast<unsigned long long>(carry));
+      atomicAdd(&slot[2], lead_rows * row_chunk_bytes);
     }
   }
 }

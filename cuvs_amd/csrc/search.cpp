@@ -486,10 +486,10 @@ void search(cuvs::resources const& res_c,
     if (res.prof == nullptr) {
       res.prof = new cuvs::resources::profile_state();
       for (auto& e : res.prof->ev) { CUVS_HIP_TRY(hipEventCreate(&e)); }
-      CUVS_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&res.prof->d_stats), 32));
+      CUVS_HIP_TRY(hipMalloc(reinterpret_cast<void**>(&res.prof->d_stats), size_t(detail::kStatSlots) * 32));
     }
     d_stats = res.prof->d_stats;
-    detail::launch_fill_u32(reinterpret_cast<uint32_t*>(d_stats), 0, 8, s);
+    detail::launch_fill_u32(reinterpret_cast<uint32_t*>(d_stats), 0, detail::kStatSlots * 8, s);
     res.last_profile           = cuvs::search_profile{};
     res.last_profile.n_queries = uint32_t(n_queries);
     res.last_profile.n_probes  = P;
@@ -615,9 +615,11 @@ void search(cuvs::resources const& res_c,
     }
   }
   if (prof) {
-    unsigned long long h[4] = {0, 0, 0, 0};
-    CUVS_HIP_TRY(hipMemcpyAsync(h, d_stats, 32, hipMemcpyDeviceToHost, s));
+    std::vector<unsigned long long> slots(size_t(detail::kStatSlots) * 4);
+    CUVS_HIP_TRY(hipMemcpyAsync(slots.data(), d_stats, slots.size() * 8, hipMemcpyDeviceToHost, s));
     CUVS_HIP_TRY(hipStreamSynchronize(s));
+    unsigned long long h[4] = {0, 0, 0, 0};
+    for (size_t i = 0; i < slots.size(); i++) { h[i % 4] += slots[i]; }
     res.last_profile.scan_bytes = h[0];
     res.last_profile.scan_rows  = h[1];
     if (early_stop) {
