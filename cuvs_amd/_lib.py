@@ -80,7 +80,7 @@ EXPORTED_SYMBOLS = [
     "cuvsStreamSync", "cuvsDeviceIdGet", "cuvsResourcesSetWorkspacePool", "cuvsRMMAlloc",
     "cuvsRMMFree", "cuvsVersionGet", "cuvsRMMPoolMemoryResourceEnable",
     "cuvsRMMAsyncMemoryResourceEnable", "cuvsRMMMemoryResourceReset", "cuvsRMMHostAlloc",
-    "cuvsRMMHostFree", "cuvsMatrixCopy", "cuvsMatrixSliceRows",
+    "cuvsRMMHostFree", "cuvsMatrixCopy", "cuvsMatrixSliceRows", "cuvsResourcesCreateWithMemoryTracking",
     "cuvsIvfPqIndexParamsCreate", "cuvsIvfPqIndexParamsDestroy", "cuvsIvfPqSearchParamsCreate",
     "cuvsIvfPqSearchParamsDestroy", "cuvsIvfPqIndexCreate", "cuvsIvfPqIndexDestroy",
     "cuvsIvfPqIndexGetNLists", "cuvsIvfPqIndexGetDim", "cuvsIvfPqIndexGetSize",
@@ -125,6 +125,7 @@ def lib():
         f.argtypes = list(args)
 
     proto("cuvsResourcesCreate", P(res_t))
+    proto("cuvsResourcesCreateWithMemoryTracking", P(res_t), C.c_char_p, C.c_int64)
     proto("cuvsResourcesDestroy", res_t)
     proto("cuvsStreamSet", res_t, C.c_void_p)
     proto("cuvsStreamGet", res_t, P(C.c_void_p))

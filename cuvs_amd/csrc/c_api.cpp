@@ -5,6 +5,8 @@
  */
 #include "c_common.hpp"
 
+#include <memory>
+
 namespace {
 thread_local std::string last_error_text;
 cuvsLogLevel_t g_log_level = CUVS_LOG_LEVEL_INFO;
@@ -32,6 +34,17 @@ cuvsError_t cuvsResourcesCreate(cuvsResources_t* res)
     CUVS_EXPECTS(res != nullptr, "res must not be null");
     auto* r = new cuvs::resources();
     *res    = reinterpret_cast<uintptr_t>(r);
+  });
+}
+
+cuvsError_t cuvsResourcesCreateWithMemoryTracking(cuvsResources_t* res, const char* csv_path,
+                                                  int64_t sample_interval_ms)
+{
+  return cuvs::core::translate_exceptions([=] {
+    CUVS_EXPECTS(res != nullptr, "res must not be null");
+    auto r = std::make_unique<cuvs::resources>();
+    r->track_memory(csv_path, sample_interval_ms);
+    *res = reinterpret_cast<uintptr_t>(r.release());
   });
 }
 
@@ -116,14 +129,14 @@ cuvsError_t cuvsRMMHostAlloc(void** ptr, size_t bytes)
 {
   return cuvs::core::translate_exceptions([=] {
     CUVS_EXPECTS(ptr != nullptr, "ptr must not be null");
-    CUVS_HIP_TRY(hipHostMalloc(ptr, bytes == 0 ? 1 : bytes, hipHostMallocDefault));
+    *ptr = cuvs::memory::host_allocate(bytes);
   });
 }
 
 cuvsError_t cuvsRMMHostFree(void* ptr, size_t)
 {
   return cuvs::core::translate_exceptions([=] {
-    if (ptr != nullptr) { CUVS_HIP_TRY(hipHostFree(ptr)); }
+    cuvs::memory::host_deallocate(ptr);
   });
 }
 

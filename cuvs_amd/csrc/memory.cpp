@@ -6,9 +6,16 @@
 #include "detail.hpp"
 
 #include <algorithm>
+#include <atomic>
+#include <chrono>
+#include <condition_variable>
+#include <cstdio>
 #include <map>
 #include <mutex>
 #include <set>
+#include <string>
+#include <thread>
+#include <unordered_map>
 #include <unordered_set>
 #include <utility>
 #include <vector>
@@ -54,6 +61,148 @@ void merge_fences(fence_list& into, const fence_list& from)
   }
 }
 }  // namespace
+
+/* ---------------------------------------------------------------------------------------- */
+/* allocation tracking                                                                       */
+/* ---------------------------------------------------------------------------------------- */
+
+enum class space { device = 0, pinned = 1 };
+
+class tracker {
+ public:
+  tracker(const char* csv_path, int64_t interval_ms)
+    : interval_(interval_ms), start_(std::chrono::steady_clock::now())
+  {
+    file_ = std::fopen(csv_path, "w");
+    CUVS_EXPECTS(file_ != nullptr, "cannot open %s for writing", csv_path);
+    std::fputs("elapsed_ms,device_current_bytes,device_peak_bytes,pinned_current_bytes,pinned_peak_bytes,"
+               "allocations,deallocations\n",
+               file_);
+    std::fflush(file_);
+    sampler_ = std::thread([this] { run(); });
+  }
+
+  ~tracker()
+  {
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      stop_ = true;
+    }
+    wake_.notify_all();
+    if (sampler_.joinable()) { sampler_.join(); }
+    write_row();  // the state at the end, whatever the sampler saw last
+    std::fclose(file_);
+  }
+
+  void allocated(void* ptr, size_t bytes, space where)
+  {
+    std::lock_guard<std::mutex> lock(mutex_);
+    live_[ptr] = {bytes, where};
+    auto& u    = usage_[int(where)];
+    u.current += bytes;
+    u.peak = std::max(u.peak, u.current);
+    n_alloc_ += 1;
+    dirty_ = true;
+    wake_.notify_all();
+  }
+
+  /** Ranges handed out before tracking began are not known here and pass unnoticed. */
+  void released(void* ptr)
+  {
+    std::lock_guard<std::mutex> lock(mutex_);
+    auto it = live_.find(ptr);
+    if (it == live_.end()) { return; }
+    usage_[int(it->second.second)].current -= it->second.first;
+    live_.erase(it);
+    n_free_ += 1;
+    dirty_ = true;
+    wake_.notify_all();
+  }
+
+ private:
+  struct usage {
+    size_t current = 0, peak = 0;
+  };
+
+  void run()
+  {
+    std::unique_lock<std::mutex> lock(mutex_);
+    while (!stop_) {
+      wake_.wait(lock, [this] { return dirty_ || stop_; });
+      if (stop_) { break; }
+      dirty_ = false;
+      lock.unlock();
+      write_row();
+      lock.lock();
+      // the interval is the least time between two rows; a stop request ends the wait
+      wake_.wait_for(lock, std::chrono::milliseconds(interval_), [this] { return stop_; });
+    }
+  }
+
+  void write_row()
+  {
+    usage dev, pin;
+    uint64_t n_alloc, n_free;
+    {
+      std::lock_guard<std::mutex> lock(mutex_);
+      dev     = usage_[0];
+      pin     = usage_[1];
+      n_alloc = n_alloc_;
+      n_free  = n_free_;
+    }
+    const double ms =
+      std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - start_).count();
+    std::lock_guard<std::mutex> lock(file_mutex_);
+    std::fprintf(file_, "%.3f,%zu,%zu,%zu,%zu,%llu,%llu\n", ms, dev.current, dev.peak, pin.current, pin.peak,
+                 static_cast<unsigned long long>(n_alloc), static_cast<unsigned long long>(n_free));
+    std::fflush(file_);
+  }
+
+  int64_t interval_;
+  std::chrono::steady_clock::time_point start_;
+  std::FILE* file_ = nullptr;
+  std::mutex mutex_, file_mutex_;
+  std::condition_variable wake_;
+  std::thread sampler_;
+  bool stop_ = false, dirty_ = false;
+  usage usage_[2];
+  uint64_t n_alloc_ = 0, n_free_ = 0;
+  std::unordered_map<void*, std::pair<size_t, space>> live_;
+};
+
+namespace {
+std::atomic<tracker*> g_tracker{nullptr};
+
+inline void note_allocated(void* ptr, size_t bytes, space where = space::device)
+{
+  if (tracker* t = g_tracker.load(std::memory_order_acquire)) { t->allocated(ptr, bytes, where); }
+}
+inline void note_released(void* ptr)
+{
+  if (tracker* t = g_tracker.load(std::memory_order_acquire)) { t->released(ptr); }
+}
+}  // namespace
+
+tracker* start_tracking(const char* csv_path, int64_t interval_ms)
+{
+  CUVS_EXPECTS(csv_path != nullptr && csv_path[0] != '\0', "csv_path must be a non-empty string");
+  CUVS_EXPECTS(interval_ms >= 0, "sample_interval_ms must be >= 0");
+  auto* t            = new tracker(csv_path, interval_ms);
+  tracker* expected  = nullptr;
+  if (!g_tracker.compare_exchange_strong(expected, t)) {
+    delete t;
+    fail("memory tracking is already active in this process: one tracking handle at a time");
+  }
+  return t;
+}
+
+void stop_tracking(tracker* t) noexcept
+{
+  if (t == nullptr) { return; }
+  tracker* expected = t;
+  g_tracker.compare_exchange_strong(expected, nullptr);
+  delete t;
+}
 
 class pool {
  public:
@@ -114,6 +263,7 @@ class pool {
         fail("waiting for the previous owner of pooled memory failed: %s", hipGetErrorString(st));
       }
     }
+    note_allocated(addr, size);
     return addr;
   }
 
@@ -127,6 +277,7 @@ class pool {
       // the caller does not say which stream used the range last: wait for all of them
       CUVS_HIP_TRY(hipDeviceSynchronize());
     }
+    note_released(ptr);
     std::lock_guard<std::mutex> lock(mutex_);
     return release_locked(static_cast<char*>(ptr), marks);
   }
@@ -329,6 +480,7 @@ void* allocate(size_t bytes)
   if (p) { return p->allocate(bytes, nullptr, false); }
   void* ptr = nullptr;
   CUVS_HIP_TRY(hipMalloc(&ptr, bytes));
+  note_allocated(ptr, bytes);
   return ptr;
 }
 
@@ -351,6 +503,7 @@ void deallocate(void* ptr) noexcept
     drop_empty_retired(s);
     return;
   }
+  note_released(ptr);
   (void)hipFree(ptr);  // also releases what hipMallocAsync handed out, after waiting for the device
 }
 
@@ -368,11 +521,13 @@ void* allocate_on_stream(size_t bytes, hipStream_t stream)
   void* ptr = nullptr;
   if (how == source::async) {
     CUVS_HIP_TRY(hipMallocAsync(&ptr, bytes == 0 ? 1 : bytes, stream));
+    note_allocated(ptr, bytes);
     std::lock_guard<std::mutex> lock(s.mutex);
     s.async_live.insert(ptr);
     return ptr;
   }
   CUVS_HIP_TRY(hipMalloc(&ptr, bytes));
+  note_allocated(ptr, bytes);
   return ptr;
 }
 
@@ -393,11 +548,27 @@ void deallocate_on_stream(void* ptr, hipStream_t stream)
     drop_empty_retired(s);
     return;
   }
+  note_released(ptr);
   if (from_async) {
     CUVS_HIP_TRY(hipFreeAsync(ptr, stream));
     return;
   }
   CUVS_HIP_TRY(hipFree(ptr));
+}
+
+void* host_allocate(size_t bytes)
+{
+  void* ptr = nullptr;
+  CUVS_HIP_TRY(hipHostMalloc(&ptr, bytes == 0 ? 1 : bytes, hipHostMallocDefault));
+  note_allocated(ptr, bytes, space::pinned);
+  return ptr;
+}
+
+void host_deallocate(void* ptr)
+{
+  if (ptr == nullptr) { return; }
+  note_released(ptr);
+  CUVS_HIP_TRY(hipHostFree(ptr));
 }
 
 void enable_pool(int initial_percent, int maximum_percent, bool managed)

@@ -45,6 +45,23 @@ void enable_pool(int initial_percent, int maximum_percent, bool managed);
 void enable_async();
 void reset();
 
+/** Pinned host memory (cuvsRMMHostAlloc / cuvsRMMHostFree). */
+void* host_allocate(size_t bytes);
+void host_deallocate(void* ptr);
+
+/**
+ * Allocation tracking (role of raft::memory_tracking_resources behind
+ * cuvsResourcesCreateWithMemoryTracking, c/src/core/c_api.cpp:57-72): while a tracker is alive every
+ * allocation and release made through this file is counted, and a background thread writes samples
+ * to a CSV file: the header at once, then one row after each burst of activity, not more often
+ * than every `interval_ms`, each flushed as written, and a last row when tracking stops.
+ * Columns: elapsed_ms, device_current_bytes, device_peak_bytes, pinned_current_bytes,
+ * pinned_peak_bytes, allocations, deallocations.  One tracker per process at a time.
+ */
+class tracker;
+tracker* start_tracking(const char* csv_path, int64_t interval_ms);
+void stop_tracking(tracker* t) noexcept;
+
 /** rmm::percent_of_free_device_memory: that share of the free memory, a multiple of 256 bytes. */
 size_t percent_of_free_device_memory(int percent);
 

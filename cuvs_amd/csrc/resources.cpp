@@ -18,6 +18,16 @@ resources::~resources()
   for (void* p : retired_) { memory::deallocate(p); }
   extern void destroy_profile_state(resources::profile_state*);
   destroy_profile_state(prof);
+  if (tracker_ != nullptr) {
+    // the handle's own pool goes after this body: what it still holds counts as live in the last row
+    memory::stop_tracking(tracker_);
+  }
+}
+
+void resources::track_memory(const char* csv_path, int64_t sample_interval_ms)
+{
+  CUVS_EXPECTS(tracker_ == nullptr, "this handle tracks memory already");
+  tracker_ = memory::start_tracking(csv_path, sample_interval_ms);
 }
 
 void resources::sync() const { CUVS_HIP_TRY(hipStreamSynchronize(stream_)); }

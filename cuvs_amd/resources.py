@@ -5,9 +5,16 @@ from ._lib import check, lib
 
 
 class Resources:
-    def __init__(self, stream=None):
+    def __init__(self, stream=None, memory_tracking_csv_path=None, memory_tracking_sample_interval_ms=10):
+        """`memory_tracking_csv_path`: the handle also counts the library's allocations and writes samples
+        to that CSV file until it is destroyed (resources.pyx:75-84)."""
         self._h = C.c_size_t(0)
-        check(lib().cuvsResourcesCreate(C.byref(self._h)))
+        if memory_tracking_csv_path:
+            check(lib().cuvsResourcesCreateWithMemoryTracking(
+                C.byref(self._h), str(memory_tracking_csv_path).encode("utf-8"),
+                int(memory_tracking_sample_interval_ms)))
+        else:
+            check(lib().cuvsResourcesCreate(C.byref(self._h)))
         if stream is not None:
             self.set_stream(stream)
 

@@ -52,6 +52,14 @@ typedef uintptr_t cuvsResources_t;
 
 /** c_api.h:88 */
 CUVS_EXPORT cuvsError_t cuvsResourcesCreate(cuvsResources_t* res);
+/** c_api.h:113 -- a handle like cuvsResourcesCreate's that also counts every allocation and release
+ *  the library makes (device memory from any of the three sources, pinned host memory) until it is
+ *  destroyed, and writes samples to `csv_path` from a background thread: the header at once, then a
+ *  row after each burst of activity, at least `sample_interval_ms` apart, flushed as written, and a
+ *  last row on destruction.  Columns: elapsed_ms, device_current_bytes, device_peak_bytes,
+ *  pinned_current_bytes, pinned_peak_bytes, allocations, deallocations.  One at a time per process. */
+CUVS_EXPORT cuvsError_t cuvsResourcesCreateWithMemoryTracking(cuvsResources_t* res, const char* csv_path,
+                                                              int64_t sample_interval_ms);
 /** c_api.h:123 */
 CUVS_EXPORT cuvsError_t cuvsResourcesDestroy(cuvsResources_t res);
 /** c_api.h:133 */

@@ -15,7 +15,8 @@
 #include <vector>
 
 namespace cuvs::memory {
-class pool;  // sub-allocating device memory pool, internal to the library
+class pool;     // sub-allocating device memory pool, internal to the library
+class tracker;  // allocation tracking with a CSV reporter, internal to the library
 }
 
 // The library is built with hidden visibility; what this header declares is its C++ interface
@@ -112,6 +113,13 @@ class resources {
   void set_workspace_pool(size_t initial_bytes);
   memory::pool* workspace_pool() const { return pool_.get(); }
 
+  /**
+   * From now until this handle is destroyed, every allocation and release the library makes is
+   * counted and sampled into a CSV file by a background thread (role of
+   * raft::memory_tracking_resources).  One tracking handle per process at a time.
+   */
+  void track_memory(const char* csv_path, int64_t sample_interval_ms);
+
   /** Bump allocation out of the cached workspace; valid until the next reset_workspace(). */
   void* workspace_alloc(size_t bytes);
   /** Make sure the workspace can serve `bytes` in total before the first allocation of a call. */
@@ -135,6 +143,7 @@ class resources {
   std::shared_ptr<memory::pool> pool_;  // set_workspace_pool
   bool workspace_pooled_ = false;       // workspace_ came out of pool_
   void release_workspace();
+  memory::tracker* tracker_ = nullptr;  // track_memory
 };
 
 }  // namespace cuvs

@@ -116,3 +116,37 @@ def test_search_workspace_out_of_the_handles_own_pool(workload):
     got = ivf_pq.search(ivf_pq.SearchParams(n_probes=16), index, queries, 10, resources=res)
     res.sync()
     assert torch.equal(got[0], want_d) and torch.equal(got[1], want_nb)
+
+
+def test_memory_tracking_writes_csv(tmp_path, workload):
+    """The reference's own test of the tracking handle (python/cuvs/cuvs/tests/test_memory_tracking.py:
+    the file exists, is not empty and starts with a header), plus what the rows must say."""
+    import time
+    data, queries, model = workload
+    csv = tmp_path / "alloc.csv"
+    res = Resources(memory_tracking_csv_path=str(csv), memory_tracking_sample_interval_ms=2)
+    assert csv.read_text().startswith("elapsed_ms,device_current_bytes,device_peak_bytes")  # flushed at once
+    from cuvs_amd._lib import CuvsError
+    with pytest.raises(CuvsError, match="already active"):
+        Resources(memory_tracking_csv_path=str(tmp_path / "second.csv"))
+    try:
+        index, d, nb = _fill_and_search(data, queries, model)
+        time.sleep(0.05)
+        arena_bytes = sum(((s + 31) // 32) * 32 for s in index.list_sizes.cpu().tolist()) * (PQ_DIM + 8)
+        del index
+        time.sleep(0.05)
+    finally:
+        del res
+    rows = [line.split(",") for line in csv.read_text().splitlines()]
+    assert rows[0][0] == "elapsed_ms" and len(rows) >= 3
+    body = [[float(v) for v in r] for r in rows[1:]]
+    assert all(len(r) == 7 for r in body)
+    times = [r[0] for r in body]
+    assert times == sorted(times)
+    assert all(b - a >= 1.9 for a, b in zip(times[:-2], times[1:-1]))  # at least the interval apart
+    peak = max(r[2] for r in body)
+    assert peak >= arena_bytes  # the codes and ids of the lists were live at some point
+    last = body[-1]
+    assert last[5] >= last[6] > 0 and last[2] == peak
+    # what the index held is gone; the default handle's workspace may still be there
+    assert last[1] < peak
