@@ -219,7 +219,7 @@ def main():
     full_name = ("scan_kernel" if not fused
                  else "scan_nibble_kernel" if nibble
                  else "scan_kernel" if (pq_bits != 8 or (pq_dim, pq_len) not in ((64, 2), (48, 2), (32, 4)))
-                 else "scan_quad_kernel" if (args.lut != "f32" and k <= 64) else "scan_fast_kernel")
+                 else "scan_quad_kernel" if (args.lut != "f32" and k <= 128) else "scan_fast_kernel")
     if early_stop:
         # The scan stage is three launches: the leading probes' lists in full, the screen of every
         # other pair on its leading 8 codes (8 bytes a row: from the packed plane of leading codes
