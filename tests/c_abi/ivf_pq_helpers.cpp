@@ -5,7 +5,8 @@
  * check_packing) plus closed forms computed here on the host: the bit-contiguous form of a row
  * (code j at bit j * pq_bits, least significant first) and the decoded vector
  * rotation^T (rotated centre + codebook entries) in double precision from the model tensors.
- * Runs 8-, 5- and 4-bit codes with per-subspace and per-cluster codebooks.  Prints "ok".
+ * Runs 4- to 8-bit codes, rows of one and of two chunks, per-subspace and per-cluster codebooks.
+ * Prints "ok".
  */
 #include <cuvs/neighbors/ivf_pq.hpp>
 
@@ -125,15 +126,17 @@ bool throws(Fn fn)
   return false;
 }
 
-void run(uint32_t pq_bits, ivf_pq::codebook_gen kind, const std::vector<float>& data, int64_t n_rows, uint32_t dim)
+void run(uint32_t pq_bits, ivf_pq::codebook_gen kind, uint32_t pq_dim_asked, const std::vector<float>& data,
+         int64_t n_rows, uint32_t dim)
 {
-  std::printf("pq_bits %u, %s codebooks\n", pq_bits, kind == ivf_pq::codebook_gen::PER_SUBSPACE ? "per-subspace" : "per-cluster");
+  std::printf("pq_bits %u, pq_dim %u, %s codebooks\n", pq_bits, pq_dim_asked,
+              kind == ivf_pq::codebook_gen::PER_SUBSPACE ? "per-subspace" : "per-cluster");
   std::fflush(stdout);
   cuvs::resources res;
   float* d_data = to_device(data);
   ivf_pq::index_params ip;
   ip.n_lists       = 40;
-  ip.pq_dim        = 16;
+  ip.pq_dim        = pq_dim_asked;
   ip.pq_bits       = pq_bits;
   ip.codebook_kind = kind;
   auto index       = ivf_pq::build<float>(res, ip, make_device_matrix_view<const float>(d_data, n_rows, dim));
@@ -445,9 +448,14 @@ int main()
     for (uint32_t d = 0; d < dim; d++) { data[i * dim + d] = centres[c * dim + d] + noise(gen); }
   }
   for (uint32_t bits : {8u, 5u, 4u}) {
-    run(bits, ivf_pq::codebook_gen::PER_SUBSPACE, data, n_rows, dim);
-    run(bits, ivf_pq::codebook_gen::PER_CLUSTER, data, n_rows, dim);
+    run(bits, ivf_pq::codebook_gen::PER_SUBSPACE, 16, data, n_rows, dim);
+    run(bits, ivf_pq::codebook_gen::PER_CLUSTER, 16, data, n_rows, dim);
   }
+  // rows of more than one 16-byte chunk, the last one partly filled (16, 25, 21 and 18 codes per chunk)
+  run(8, ivf_pq::codebook_gen::PER_SUBSPACE, 32, data, n_rows, dim);
+  run(5, ivf_pq::codebook_gen::PER_CLUSTER, 32, data, n_rows, dim);
+  run(6, ivf_pq::codebook_gen::PER_SUBSPACE, 32, data, n_rows, dim);
+  run(7, ivf_pq::codebook_gen::PER_CLUSTER, 32, data, n_rows, dim);
   std::printf("ok\n");
   return 0;
 }
