@@ -5,6 +5,8 @@
  */
 #include "c_common.hpp"
 
+#include <cuvs/version_config.h>
+
 #include <memory>
 
 namespace {
@@ -144,9 +146,9 @@ cuvsError_t cuvsVersionGet(uint16_t* major, uint16_t* minor, uint16_t* patch)
 {
   return cuvs::core::translate_exceptions([=] {
     CUVS_EXPECTS(major && minor && patch, "output pointers must not be null");
-    *major = 26;  // API level of the cuVS release whose search entry points are mirrored
-    *minor = 10;
-    *patch = 0;
+    *major = CUVS_VERSION_MAJOR;  // API level of the cuVS release whose entry points are mirrored
+    *minor = CUVS_VERSION_MINOR;
+    *patch = CUVS_VERSION_PATCH;
   });
 }
 

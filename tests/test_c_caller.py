@@ -26,7 +26,7 @@ def _compile(name, out):
 
 
 def test_headers_compile_as_c_and_the_programs_link(tmp_path):
-    headers = ["cuvs/core/c_api.h", "cuvs/neighbors/ivf_pq.h", "cuvs/neighbors/refine.h",
+    headers = ["cuvs/core/c_api.h", "cuvs/version_config.h", "cuvs/neighbors/ivf_pq.h", "cuvs/neighbors/refine.h",
                "cuvs/neighbors/knn_merge_parts.h"]
     probe = tmp_path / "probe.c"
     probe.write_text("".join(f"#include <{h}>\n" for h in headers) + "int main(void) { return 0; }\n")
