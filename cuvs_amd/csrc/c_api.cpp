@@ -44,6 +44,8 @@ cuvsError_t cuvsResourcesCreateWithMemoryTracking(cuvsResources_t* res, const ch
 {
   return cuvs::core::translate_exceptions([=] {
     CUVS_EXPECTS(res != nullptr, "res must not be null");
+    CUVS_EXPECTS(csv_path != nullptr && csv_path[0] != '\0', "csv_path must be a non-empty string");
+    CUVS_EXPECTS(sample_interval_ms >= 0, "sample_interval_ms must be >= 0");
     auto r = std::make_unique<cuvs::resources>();
     r->track_memory(csv_path, sample_interval_ms);
     *res = reinterpret_cast<uintptr_t>(r.release());

@@ -82,3 +82,22 @@ def test_python_mirror_keeps_reference_defaults():
     import pytest
     with pytest.raises(ValueError):
         ivf_pq.IndexParams(codebook_kind="nope")
+    # the read-only views of the reference's parameter objects (ivf_pq.pyx:174-236, 716-739)
+    assert (ip.n_lists, ip.pq_bits, ip.codebook_kind, ip.codes_layout, ip.add_data_on_build) == (
+        10, 5, 1, "interleaved", True)
+    assert ivf_pq.IndexParams(codes_layout="flat").codes_layout == "flat"
+    import ctypes
+    from cuvs_amd._lib import IndexParamsStruct, SearchParamsStruct
+    assert ctypes.cast(ip.get_handle(), ctypes.POINTER(IndexParamsStruct)).contents.n_lists == 10
+    assert ctypes.cast(sp.get_handle(), ctypes.POINTER(SearchParamsStruct)).contents.n_probes == 7
+
+
+def test_memory_entry_points_reject_bad_arguments_without_a_gpu():
+    """Argument checks that come before any device call."""
+    from cuvs_amd import _lib
+    L = _lib.lib()
+    res = C.c_size_t(0)
+    assert L.cuvsResourcesCreateWithMemoryTracking(C.byref(res), b"", 10) == _lib.CUVS_ERROR
+    assert b"csv_path" in L.cuvsGetLastErrorText()
+    assert L.cuvsResourcesCreateWithMemoryTracking(C.byref(res), None, 10) == _lib.CUVS_ERROR
+    assert L.cuvsRMMHostFree(None, 0) == _lib.CUVS_SUCCESS
