@@ -221,6 +221,39 @@ void run(uint32_t pq_bits, ivf_pq::codebook_gen kind, uint32_t pq_dim_asked, con
   again = search_all(res, index, d_data, n_queries, k);
   REQUIRE(again.ids == before_search.ids && again.dist == before_search.dist);
 
+  /* growing a list in place (the padding of its last group) and by moving the arenas */
+  {
+    auto grow_by = [&](uint32_t extra) {
+      const uint32_t size0 = to_host(index.list_sizes(), n_lists)[label];
+      packer::extend_list_with_codes(res, &index, make_device_matrix_view<const uint8_t>(d_codes, extra, pq_dim),
+                                     make_device_vector_view<const int64_t>(d_ids, extra), label);
+      const auto now = snapshot(index, label);
+      REQUIRE(now.size == size0 + extra && index.size() == n_rows + int64_t(size0 + extra - n));
+      REQUIRE(std::equal(now.ids.begin(), now.ids.begin() + n, before.ids.begin()));
+      REQUIRE(std::equal(now.ids.begin() + size0, now.ids.end(), before.ids.begin()));
+      auto* d_tail = device_array<uint8_t>(size_t(extra) * pq_dim);
+      packer::unpack_list_data(res, index, make_device_matrix_view(d_tail, extra, pq_dim), label, size0);
+      res.sync();
+      REQUIRE(to_host(d_tail, size_t(extra) * pq_dim) == std::vector<uint8_t>(codes.begin(), codes.begin() + size_t(extra) * pq_dim));
+      packer::unpack_list_data(res, index, make_device_matrix_view(d_part, 20, pq_dim), label, 37);
+      res.sync();
+      REQUIRE(to_host(d_part, size_t(20) * pq_dim) == std::vector<uint8_t>(codes.begin() + 37 * pq_dim, codes.begin() + 57 * pq_dim));
+      REQUIRE(hipFree(d_tail) == hipSuccess);
+    };
+    grow_by(1);
+    grow_by(40);
+    grow_by(31);
+    grow_by(32 - (n + 72) % 32);  // up to a group boundary exactly
+    grow_by(1);
+    ivf_pq::helpers::erase_list(res, &index, label);
+    packer::extend_list_with_codes(res, &index, make_device_matrix_view<const uint8_t>(d_codes, n, pq_dim),
+                                   make_device_vector_view<const int64_t>(d_ids, n), label);
+    after = snapshot(index, label);
+    REQUIRE(after.size == n && after.ids == before.ids && after.bytes == before.bytes);
+    again = search_all(res, index, d_data, n_queries, k);
+    REQUIRE(again.ids == before_search.ids && again.dist == before_search.dist);
+  }
+
   /* check_reconstruction: decoded rows against the closed form, and near the rows they encode */
   const auto rotation    = to_host(index.rotation_matrix(), size_t(rot_dim) * dim);
   const auto centers_rot = to_host(index.centers_rot(), size_t(n_lists) * rot_dim);
