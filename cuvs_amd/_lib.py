@@ -81,6 +81,8 @@ EXPORTED_SYMBOLS = [
     "cuvsRMMFree", "cuvsVersionGet", "cuvsRMMPoolMemoryResourceEnable",
     "cuvsRMMAsyncMemoryResourceEnable", "cuvsRMMMemoryResourceReset", "cuvsRMMHostAlloc",
     "cuvsRMMHostFree", "cuvsMatrixCopy", "cuvsMatrixSliceRows", "cuvsResourcesCreateWithMemoryTracking",
+    "cuvsMultiGpuResourcesCreate", "cuvsMultiGpuResourcesCreateWithDeviceIds",
+    "cuvsMultiGpuResourcesDestroy", "cuvsMultiGpuResourcesSetMemoryPool",
     "cuvsIvfPqIndexParamsCreate", "cuvsIvfPqIndexParamsDestroy", "cuvsIvfPqSearchParamsCreate",
     "cuvsIvfPqSearchParamsDestroy", "cuvsIvfPqIndexCreate", "cuvsIvfPqIndexDestroy",
     "cuvsIvfPqIndexGetNLists", "cuvsIvfPqIndexGetDim", "cuvsIvfPqIndexGetSize",
@@ -126,6 +128,10 @@ def lib():
 
     proto("cuvsResourcesCreate", P(res_t))
     proto("cuvsResourcesCreateWithMemoryTracking", P(res_t), C.c_char_p, C.c_int64)
+    proto("cuvsMultiGpuResourcesCreate", P(res_t))
+    proto("cuvsMultiGpuResourcesCreateWithDeviceIds", P(res_t), T)
+    proto("cuvsMultiGpuResourcesDestroy", res_t)
+    proto("cuvsMultiGpuResourcesSetMemoryPool", res_t, C.c_int)
     proto("cuvsResourcesDestroy", res_t)
     proto("cuvsStreamSet", res_t, C.c_void_p)
     proto("cuvsStreamGet", res_t, P(C.c_void_p))

@@ -52,6 +52,33 @@ cuvsError_t cuvsResourcesCreateWithMemoryTracking(cuvsResources_t* res, const ch
   });
 }
 
+namespace {
+[[noreturn]] void no_multi_gpu()
+{
+  cuvs::fail("multi-GPU resources are not part of this library: it drives one GPU per process");
+}
+}  // namespace
+
+cuvsError_t cuvsMultiGpuResourcesCreate(cuvsResources_t*)
+{
+  return cuvs::core::translate_exceptions([] { no_multi_gpu(); });
+}
+
+cuvsError_t cuvsMultiGpuResourcesCreateWithDeviceIds(cuvsResources_t*, DLManagedTensor*)
+{
+  return cuvs::core::translate_exceptions([] { no_multi_gpu(); });
+}
+
+cuvsError_t cuvsMultiGpuResourcesDestroy(cuvsResources_t)
+{
+  return cuvs::core::translate_exceptions([] { no_multi_gpu(); });
+}
+
+cuvsError_t cuvsMultiGpuResourcesSetMemoryPool(cuvsResources_t, int)
+{
+  return cuvs::core::translate_exceptions([] { no_multi_gpu(); });
+}
+
 cuvsError_t cuvsResourcesDestroy(cuvsResources_t res)
 {
   return cuvs::core::translate_exceptions([=] { delete reinterpret_cast<cuvs::resources*>(res); });

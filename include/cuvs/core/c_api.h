@@ -74,6 +74,14 @@ CUVS_EXPORT cuvsError_t cuvsDeviceIdGet(cuvsResources_t res, int* device_id);
  *  reserved now, the pool grows on demand and never shrinks before the handle is destroyed.  The
  *  handle's search workspace and cuvsRMMAlloc / cuvsRMMFree on it are then served from the pool. */
 CUVS_EXPORT cuvsError_t cuvsResourcesSetWorkspacePool(cuvsResources_t res, size_t initial_size_bytes);
+/** c_api.h:184-214 -- handles over several GPUs of one process.  This library drives one GPU: the
+ *  four calls exist so that callers of the whole C API link, and every one of them fails with
+ *  CUVS_ERROR and a message that says so (row-sharded search across GPUs is a merge of per-GPU
+ *  answers, cuvsAmdKnnMergeParts; the exchange itself is the caller's). */
+CUVS_EXPORT cuvsError_t cuvsMultiGpuResourcesCreate(cuvsResources_t* res);
+CUVS_EXPORT cuvsError_t cuvsMultiGpuResourcesCreateWithDeviceIds(cuvsResources_t* res, DLManagedTensor* device_ids);
+CUVS_EXPORT cuvsError_t cuvsMultiGpuResourcesDestroy(cuvsResources_t res);
+CUVS_EXPORT cuvsError_t cuvsMultiGpuResourcesSetMemoryPool(cuvsResources_t res, int percent_of_free_memory);
 /** c_api.h:230 -- device memory, ordered on the handle's stream. */
 CUVS_EXPORT cuvsError_t cuvsRMMAlloc(cuvsResources_t res, void** ptr, size_t bytes);
 /** c_api.h:240 */

@@ -101,3 +101,7 @@ def test_memory_entry_points_reject_bad_arguments_without_a_gpu():
     assert b"csv_path" in L.cuvsGetLastErrorText()
     assert L.cuvsResourcesCreateWithMemoryTracking(C.byref(res), None, 10) == _lib.CUVS_ERROR
     assert L.cuvsRMMHostFree(None, 0) == _lib.CUVS_SUCCESS
+    # one GPU per process: the multi-GPU handles exist to link against and say so when called
+    assert L.cuvsMultiGpuResourcesCreate(C.byref(res)) == _lib.CUVS_ERROR
+    assert b"one GPU" in L.cuvsGetLastErrorText()
+    assert L.cuvsMultiGpuResourcesSetMemoryPool(res, 50) == _lib.CUVS_ERROR
