@@ -134,6 +134,9 @@ struct index_impl {
   std::vector<uint32_t> h_list_sizes;
   std::vector<uint64_t> h_row_offsets;  // [n_lists + 1], in rows, multiples of 32
   device_buffer list_sizes, data_ptrs, inds_ptrs;
+  /** Position of every list among all lists by size, largest first (ties by list number): the
+   *  order in which the search takes the pairs of each query's leading probe, long lists first. */
+  device_buffer list_rank;
   std::vector<int64_t> accum_sorted_sizes;  // [n_lists + 1]
   int64_t size = 0;
 
@@ -223,7 +226,8 @@ constexpr uint32_t kStatSlots = 256;
 void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
                           uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
                           uint32_t* n_samples, unsigned long long* stats, uint32_t lead_probes,
-                          uint32_t* pair_counts, uint32_t n_lists, hipStream_t stream);
+                          uint32_t* pair_counts, uint32_t n_lists, const uint32_t* list_rank,
+                          hipStream_t stream);
 
 /** Everything the scan needs to know about one (query, probe) pair, gathered once so that the
  *  scan kernel reads one 32-byte record instead of chasing four dependent pointers. */
@@ -244,13 +248,15 @@ static_assert(sizeof(pair_desc) == 32, "pair_desc must stay 32 bytes");
  *  by list) and the others after them (grouped by list again); `alive`, when non-null, gets one
  *  byte per pair slot: 1 for the leading pairs, 0 for the others.  `counters` is scratch of
  *  4 * n_lists + 4 words; with `counted` its first half already holds the histogram of the pairs
- *  (launch_chunk_indices with `pair_counts` makes it on the way). */
+ *  (launch_chunk_indices with `pair_counts` makes it on the way).  `list_rank` (n_lists words, a
+ *  permutation; null: the identity) gives the order of the groups of leading pairs: group of list
+ *  l at position list_rank[l]; both launchers must be given the same table. */
 void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
                         const uint8_t* const* data_ptrs, const int64_t* const* inds_ptrs,
                         const int64_t* ids_base, uint32_t n_pairs, uint32_t n_probes,
                         uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
                         pair_desc* desc, uint32_t lead_probes, uint8_t* alive, bool counted, bool natural_order,
-                        hipStream_t stream);
+                        const uint32_t* list_rank, hipStream_t stream);
 
 struct scan_args {
   uint32_t n_queries, n_probes, k, max_samples;

@@ -78,6 +78,14 @@ void index_impl::recompute_internal_state(hipStream_t stream)
                               hipMemcpyHostToDevice, stream));
   CUVS_HIP_TRY(hipMemcpyAsync(list_sizes.ptr, h_list_sizes.data(), sizeof(uint32_t) * n_lists,
                               hipMemcpyHostToDevice, stream));
+  std::vector<uint32_t> by_size(n_lists), rank(n_lists);
+  for (uint32_t l = 0; l < n_lists; l++) { by_size[l] = l; }
+  std::stable_sort(by_size.begin(), by_size.end(),
+                   [&](uint32_t a, uint32_t b) { return h_list_sizes[a] > h_list_sizes[b]; });
+  for (uint32_t i = 0; i < n_lists; i++) { rank[by_size[i]] = i; }
+  if (list_rank.bytes != sizeof(uint32_t) * n_lists) { list_rank.allocate(sizeof(uint32_t) * n_lists); }
+  CUVS_HIP_TRY(hipMemcpyAsync(list_rank.ptr, rank.data(), sizeof(uint32_t) * n_lists,
+                              hipMemcpyHostToDevice, stream));
   CUVS_HIP_TRY(hipStreamSynchronize(stream));  // the host vectors above go out of scope
   std::vector<uint32_t> sorted(h_list_sizes);
   std::sort(sorted.begin(), sorted.end(), std::greater<uint32_t>());

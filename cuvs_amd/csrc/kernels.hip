@@ -388,11 +388,17 @@ __global__ __launch_bounds__(kBlock) void rotate_kernel(const float* __restrict_
   }
 }
 
-/** Sort key of pair i: its list, the pairs past each query's leading probes in a second range. */
+/** Sort key of pair i: its list, the pairs past each query's leading probes in a second range.
+ *  The leading pairs go through `rank`, when given: the list's position among all lists by size,
+ *  largest first, so that they run from long lists to short ones and the pairs that share a block
+ *  are of similar length (every one of them is scanned in full, a few per compute unit in all; the
+ *  other pairs keep the order of the list numbers, which is the order of the lists in memory). */
 __device__ __forceinline__ uint32_t pair_bin(uint32_t label, uint32_t i, uint32_t n_probes,
-                                             uint32_t lead_probes, uint32_t n_lists)
+                                             uint32_t lead_probes, uint32_t n_lists,
+                                             const uint32_t* __restrict__ rank)
 {
-  return (i % n_probes) < lead_probes ? label : label + n_lists;
+  if ((i % n_probes) >= lead_probes) { return label + n_lists; }
+  return rank != nullptr ? rank[label] : label;
 }
 
 /** One wave per query: inclusive prefix sums of the probed list sizes in probe order. */
@@ -405,7 +411,8 @@ __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __res
                                                             unsigned long long* stats,
                                                             uint32_t lead_probes,
                                                             uint32_t* __restrict__ pair_counts,
-                                                            uint32_t n_lists)
+                                                            uint32_t n_lists,
+                                                            const uint32_t* __restrict__ rank)
 {
   const uint32_t q    = blockIdx.x;
   const uint32_t lane = threadIdx.x;
@@ -418,7 +425,7 @@ __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __res
       const uint32_t label = probes[uint64_t(q) * n_probes + p];
       sz                   = list_sizes[label];
       // histogram of the pair ordering, while the probe is at hand
-      if (pair_counts != nullptr) { atomicAdd(&pair_counts[pair_bin(label, p, n_probes, lead_probes, n_lists)], 1u); }
+      if (pair_counts != nullptr) { atomicAdd(&pair_counts[pair_bin(label, p, n_probes, lead_probes, n_lists, rank)], 1u); }
     }
     padded_rows += (sz + 31u) & ~31u;
     if (p < lead_probes) { lead_rows += (sz + 31u) & ~31u; }
@@ -447,10 +454,10 @@ __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __res
 
 __global__ void pair_histogram_kernel(const uint32_t* __restrict__ probes, uint32_t n_pairs,
                                       uint32_t n_probes, uint32_t lead_probes, uint32_t n_lists,
-                                      uint32_t* __restrict__ counts)
+                                      const uint32_t* __restrict__ rank, uint32_t* __restrict__ counts)
 {
   const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n_pairs) { atomicAdd(&counts[pair_bin(probes[i], i, n_probes, lead_probes, n_lists)], 1u); }
+  if (i < n_pairs) { atomicAdd(&counts[pair_bin(probes[i], i, n_probes, lead_probes, n_lists, rank)], 1u); }
 }
 
 /** Single block of 1024 threads: cursors[l] = exclusive prefix sum of counts[l].  The counts pass
@@ -510,7 +517,7 @@ __global__ void pair_scatter_kernel(const uint32_t* __restrict__ probes,
                                     const int64_t* const* __restrict__ inds_ptrs,
                                     const int64_t* ids_base, uint32_t n_pairs,
                                     uint32_t n_probes, uint32_t lead_probes, uint32_t n_lists,
-                                    uint32_t* __restrict__ cursors,
+                                    const uint32_t* __restrict__ rank, uint32_t* __restrict__ cursors,
                                     uint32_t* __restrict__ pair_order, pair_desc* __restrict__ desc,
                                     uint8_t* __restrict__ alive)
 {
@@ -519,7 +526,7 @@ __global__ void pair_scatter_kernel(const uint32_t* __restrict__ probes,
     const uint32_t label = probes[i];
     // no cursors: the pairs keep their natural (query-major) order
     const uint32_t pos = cursors != nullptr
-                           ? atomicAdd(&cursors[pair_bin(label, i, n_probes, lead_probes, n_lists)], 1u)
+                           ? atomicAdd(&cursors[pair_bin(label, i, n_probes, lead_probes, n_lists, rank)], 1u)
                            : i;
     pair_order[pos]    = i;
     if (alive != nullptr) { alive[i] = (i % n_probes) < lead_probes ? 1 : 0; }
@@ -1198,7 +1205,8 @@ void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries,
 void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
                           uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
                           uint32_t* n_samples, unsigned long long* stats, uint32_t lead_probes,
-                          uint32_t* pair_counts, uint32_t n_lists, hipStream_t stream)
+                          uint32_t* pair_counts, uint32_t n_lists, const uint32_t* list_rank,
+                          hipStream_t stream)
 {
   if (n_queries == 0) { return; }
   if (pair_counts != nullptr) {
@@ -1206,7 +1214,7 @@ void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, ui
   }
   chunk_indices_kernel<<<n_queries, 64, 0, stream>>>(list_sizes, probes, n_probes, row_chunk_bytes,
                                                      chunk_indices, n_samples, stats, lead_probes,
-                                                     pair_counts, n_lists);
+                                                     pair_counts, n_lists, list_rank);
   CUVS_LAUNCH_CHECK();
 }
 
@@ -1215,14 +1223,14 @@ void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
                         const int64_t* ids_base, uint32_t n_pairs, uint32_t n_probes,
                         uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
                         pair_desc* desc, uint32_t lead_probes, uint8_t* alive, bool counted,
-                        bool natural_order, hipStream_t stream)
+                        bool natural_order, const uint32_t* list_rank, hipStream_t stream)
 {
   if (n_pairs == 0) { return; }
   if (natural_order) {
     CUVS_EXPECTS(lead_probes >= n_probes, "natural pair order has no leading / other split");
     pair_scatter_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(
       probes, chunk_indices, data_ptrs, inds_ptrs, ids_base, n_pairs, n_probes, lead_probes, n_lists,
-      nullptr, pair_order, desc, alive);
+      nullptr, nullptr, pair_order, desc, alive);
     CUVS_LAUNCH_CHECK();
     return;
   }
@@ -1232,7 +1240,7 @@ void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
   if (!counted) {
     launch_fill_u32(counts, 0, n_bins, stream);
     pair_histogram_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(probes, n_pairs, n_probes,
-                                                                        lead_probes, n_lists, counts);
+                                                                        lead_probes, n_lists, list_rank, counts);
     CUVS_LAUNCH_CHECK();
   }
   {
@@ -1248,7 +1256,7 @@ void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
   CUVS_LAUNCH_CHECK();
   pair_scatter_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(
     probes, chunk_indices, data_ptrs, inds_ptrs, ids_base, n_pairs, n_probes, lead_probes, n_lists,
-    cursors, pair_order, desc, alive);
+    list_rank, cursors, pair_order, desc, alive);
   CUVS_LAUNCH_CHECK();
 }
 

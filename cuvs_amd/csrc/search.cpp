@@ -146,6 +146,14 @@ bool early_stop_disabled()
   return e != nullptr && e[0] == '1';
 }
 
+/** CUVS_AMD_PAIR_ORDER=label: the leading (query, list) pairs are grouped in the order of the list
+ *  numbers instead of from long lists to short ones (for measurements; the results are the same). */
+bool pair_order_by_label()
+{
+  const char* e = std::getenv("CUVS_AMD_PAIR_ORDER");
+  return e != nullptr && std::string(e) == "label";
+}
+
 /** Probes per query whose lists are scanned in full before the others are screened against the
  *  bound they give. */
 uint32_t lead_probes()
@@ -500,6 +508,8 @@ void search(cuvs::resources const& res_c,
   };
 
   const bool cosine = ix.metric == detail::DistanceType::CosineExpanded;
+  // the leading pairs run from long lists to short ones (CUVS_AMD_PAIR_ORDER=label: by list number)
+  const uint32_t* list_rank = pair_order_by_label() ? nullptr : ix.list_rank.as<uint32_t>();
   for (int64_t q0 = 0; q0 < n_queries; q0 += Qb) {
     const uint32_t nq = uint32_t(std::min<int64_t>(Qb, n_queries - q0));
     const void* qptr  = static_cast<const char*>(queries) + size_t(q0) * ix.dim * elem_size(type);
@@ -511,10 +521,10 @@ void search(cuvs::resources const& res_c,
                           ix.rotation_is_identity, cosine, rot_q, s);
     detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
                                  ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead,
-                                 few_pairs ? nullptr : counters, ix.n_lists, s);
+                                 few_pairs ? nullptr : counters, ix.n_lists, list_rank, s);
     detail::launch_order_pairs(probes, chunk, ix.data_ptrs.as<const uint8_t*>(),
                                ix.inds_ptrs.as<const int64_t*>(), ix.ids_arena.as<int64_t>(), nq * P, P,
-                               ix.n_lists, counters, order, desc, lead, alive, true, few_pairs, s);
+                               ix.n_lists, counters, order, desc, lead, alive, true, few_pairs, list_rank, s);
     if (pl.fused) { detail::launch_fill_u32(kth, 0xFFFFFFFFu, nq, s); }
     mark(2);
 
