@@ -93,6 +93,7 @@ EXPORTED_SYMBOLS = [
     "cuvsIvfPqIndexGetListIndices", "cuvsIvfPqBuild", "cuvsIvfPqBuildPrecomputed",
     "cuvsIvfPqSearch", "cuvsIvfPqSerialize", "cuvsIvfPqDeserialize", "cuvsIvfPqExtend",
     "cuvsIvfPqTransform", "cuvsAmdIvfPqSelectClusters", "cuvsAmdIvfPqSearchWithBitset",
+    "cuvsAmdIvfPqSearchNoAlloc",
     "cuvsAmdIvfPqExtendLabeled", "cuvsAmdIvfPqProfilingEnable", "cuvsAmdIvfPqGetSearchProfile",
     "cuvsRefine",
     "cuvsAmdKnnMergeParts",
@@ -175,6 +176,7 @@ def lib():
     proto("cuvsAmdIvfPqSelectClusters", res_t, P(SearchParamsStruct), P(IndexStruct), T, T)
     proto("cuvsAmdIvfPqSearchWithBitset", res_t, P(SearchParamsStruct), P(IndexStruct), T, T, T,
           T, C.c_int64)
+    proto("cuvsAmdIvfPqSearchNoAlloc", res_t, P(SearchParamsStruct), P(IndexStruct), T, T, T)
     proto("cuvsAmdIvfPqExtendLabeled", res_t, T, T, T, P(IndexStruct))
     proto("cuvsAmdIvfPqProfilingEnable", res_t, C.c_bool)
     proto("cuvsAmdIvfPqGetSearchProfile", res_t, P(SearchProfileStruct))

@@ -8,6 +8,7 @@
 #include "detail.hpp"
 
 #include <cuvs/core/c_api.h>
+#include <cuvs/neighbors/ivf_pq.h>
 #include <dlpack/dlpack.h>
 
 #include <exception>
@@ -84,6 +85,13 @@ inline void expect_tensor(const DLManagedTensor* mt, const char* name, int ndim,
     CUVS_EXPECTS(t.shape[i] >= 0, "%s has a negative extent", name);
   }
 }
+
+/** Body of cuvsIvfPqSearch / cuvsAmdIvfPqSearchWithBitset on a given handle: tensor checks, then
+ *  the C++ search (ivf_pq_c.cpp). */
+void ivf_pq_search_tensors(cuvs::resources& res, cuvsIvfPqSearchParams_t params,
+                           cuvsIvfPqIndex_t index, DLManagedTensor* queries,
+                           DLManagedTensor* neighbors, DLManagedTensor* distances,
+                           DLManagedTensor* bitset, int64_t n_bits);
 
 inline void* tensor_data(const DLManagedTensor* mt)
 {

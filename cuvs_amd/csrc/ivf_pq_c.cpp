@@ -112,9 +112,14 @@ void make_view(DLManagedTensor* out, const void* data, int ndim, const int64_t* 
   out->deleter                    = view_deleter;
 }
 
-void do_search(cuvsResources_t res, cuvsIvfPqSearchParams_t params, cuvsIvfPqIndex_t index_c,
-               DLManagedTensor* queries_t, DLManagedTensor* neighbors_t,
-               DLManagedTensor* distances_t, DLManagedTensor* bitset_t, int64_t n_bits)
+}  // namespace
+
+namespace cuvs::core {
+
+void ivf_pq_search_tensors(cuvs::resources& res, cuvsIvfPqSearchParams_t params,
+                           cuvsIvfPqIndex_t index_c, DLManagedTensor* queries_t,
+                           DLManagedTensor* neighbors_t, DLManagedTensor* distances_t,
+                           DLManagedTensor* bitset_t, int64_t n_bits)
 {
   CUVS_EXPECTS(params != nullptr, "search_params must not be null");
   CUVS_EXPECTS(queries_t && neighbors_t && distances_t, "tensors must not be null");
@@ -153,15 +158,27 @@ void do_search(cuvsResources_t res, cuvsIvfPqSearchParams_t params, cuvsIvfPqInd
                  "bitset is shorter than n_bits");
     cuvs::neighbors::filtering::bitset_filter f(static_cast<const uint32_t*>(tensor_data(bitset_t)),
                                                 n_bits);
-    ivfpq::search(*res_of(res), sp, *idx, tensor_data(queries_t), t, queries.shape[0], queries.shape[1],
+    ivfpq::search(res, sp, *idx, tensor_data(queries_t), t, queries.shape[0], queries.shape[1],
            static_cast<int64_t*>(tensor_data(neighbors_t)),
            static_cast<float*>(tensor_data(distances_t)), neighbors.shape[1], f);
   } else {
     cuvs::neighbors::filtering::none_sample_filter f;
-    ivfpq::search(*res_of(res), sp, *idx, tensor_data(queries_t), t, queries.shape[0], queries.shape[1],
+    ivfpq::search(res, sp, *idx, tensor_data(queries_t), t, queries.shape[0], queries.shape[1],
            static_cast<int64_t*>(tensor_data(neighbors_t)),
            static_cast<float*>(tensor_data(distances_t)), neighbors.shape[1], f);
   }
+}
+
+}  // namespace cuvs::core
+
+namespace {
+
+void do_search(cuvsResources_t res, cuvsIvfPqSearchParams_t params, cuvsIvfPqIndex_t index_c,
+               DLManagedTensor* queries_t, DLManagedTensor* neighbors_t,
+               DLManagedTensor* distances_t, DLManagedTensor* bitset_t, int64_t n_bits)
+{
+  cuvs::core::ivf_pq_search_tensors(*res_of(res), params, index_c, queries_t, neighbors_t,
+                                    distances_t, bitset_t, n_bits);
 }
 
 void do_extend(cuvsResources_t res, DLManagedTensor* new_vectors, DLManagedTensor* new_indices,

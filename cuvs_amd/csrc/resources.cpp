@@ -32,12 +32,27 @@ void resources::track_memory(const char* csv_path, int64_t sample_interval_ms)
 
 void resources::sync() const { CUVS_HIP_TRY(hipStreamSynchronize(stream_)); }
 
+void resources::borrow_workspace(void* ptr, size_t bytes)
+{
+  CUVS_EXPECTS(workspace_ == nullptr && workspace_used_ == 0,
+               "a handle that already caches a workspace cannot borrow one");
+  CUVS_EXPECTS(ptr != nullptr && reinterpret_cast<uintptr_t>(ptr) % 256 == 0,
+               "a borrowed workspace must be 256-byte aligned device memory");
+  workspace_          = ptr;
+  workspace_capacity_ = bytes;
+  workspace_borrowed_ = true;
+}
+
 void resources::release_workspace()
 {
   if (workspace_ == nullptr) { return; }
   void* p             = workspace_;
   workspace_          = nullptr;
   workspace_capacity_ = 0;
+  if (workspace_borrowed_) {
+    workspace_borrowed_ = false;
+    return;
+  }
   if (workspace_pooled_ && pool_) {
     (void)memory::pool_deallocate(*pool_, p, stream_, true);
   } else {
@@ -60,6 +75,9 @@ void resources::set_workspace_pool(size_t initial_bytes)
 void resources::reserve_workspace(size_t bytes)
 {
   if (bytes <= workspace_capacity_) { return; }
+  CUVS_EXPECTS(!workspace_borrowed_,
+               "this call needs %zu bytes of workspace, more than the %zu bytes the handle borrowed",
+               bytes, workspace_capacity_);
   CUVS_EXPECTS(workspace_used_ == 0, "workspace cannot grow while allocations are live");
   // work queued earlier may still read the old block: wait, then release it
   CUVS_HIP_TRY(hipStreamSynchronize(stream_));

@@ -57,6 +57,7 @@ bool device_accessible(const void* p)
 
 size_t workspace_budget(const cuvs::resources& res)
 {
+  if (res.workspace_borrowed()) { return res.workspace_capacity(); }
   size_t free_b = 0, total_b = 0;
   CUVS_HIP_TRY(hipMemGetInfo(&free_b, &total_b));
   // what is already cached in the workspace counts as available
@@ -106,6 +107,12 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
   b        = std::max<size_t>(b, 1);
   b        = std::min<size_t>(b, std::max<uint32_t>(params.max_internal_batch_size, 1u));
   b        = std::min<size_t>(b, n_queries);
+  if (res.workspace_borrowed()) {
+    // a fixed workspace does not shrink the batch behind the caller's back: one internal batch
+    // (n_queries, or max_internal_batch_size of them) has to fit, or the call is refused
+    const size_t want = std::min<size_t>(n_queries, std::max<uint32_t>(params.max_internal_batch_size, 1u));
+    b                 = want;
+  }
   // keep the pair count of a batch within uint32 indexing
   while (b > 1 && b * P >= (size_t(1) << 31)) { b /= 2; }
   p.batch = uint32_t(b);
@@ -434,8 +441,14 @@ void search(cuvs::resources const& res_c,
   /* workspace carve-up for one batch */
   res.reset_workspace();
   const bool fast_coarse = coarse_fast_applies(params, ix, type, P);
-  res.reserve_workspace(pl.fixed_bytes + size_t(Qb) * (pl.per_query_bytes + 64) + 16 * 256 +
-                        global_lut_bytes + (fast_coarse ? coarse_fast_bytes(ix, Qb) : 0));
+  const size_t workspace_bytes = pl.fixed_bytes + size_t(Qb) * (pl.per_query_bytes + 64) + 16 * 256 +
+                                 global_lut_bytes + (fast_coarse ? coarse_fast_bytes(ix, Qb) : 0);
+  CUVS_EXPECTS(!res.workspace_borrowed() || workspace_bytes <= res.workspace_capacity(),
+               "a batch of %u queries (n_probes = %u, k = %u, n_lists = %u) needs %zu bytes of workspace; "
+               "the fixed workspace of this call holds %zu: pass fewer queries per call or lower "
+               "max_internal_batch_size",
+               Qb, P, k, ix.n_lists, workspace_bytes, res.workspace_capacity());
+  res.reserve_workspace(workspace_bytes);
   auto* qt        = static_cast<float*>(
     res.workspace_alloc(size_t(ix.dim_ext) * detail::coarse_pad(Qb) * 4));
   auto* qf        = static_cast<float*>(res.workspace_alloc(size_t(Qb) * ix.dim * 4));
@@ -488,7 +501,7 @@ void search(cuvs::resources const& res_c,
   }
 
   /* profiling state */
-  const bool prof = res.profiling;
+  const bool prof = res.profiling && !res.workspace_borrowed();  // the profile allocates
   unsigned long long* d_stats = nullptr;
   if (prof) {
     if (res.prof == nullptr) {

@@ -385,6 +385,22 @@ def search(search_params, index, queries, k, neighbors=None, distances=None, res
     return distances, neighbors
 
 
+NO_ALLOC_WORKSPACE_BYTES = 32 << 20
+
+
+def search_no_alloc(search_params, index, queries, neighbors, distances, resources=None):
+    """cuvsAmdIvfPqSearchNoAlloc: `search` into outputs the caller made, on a fixed workspace that
+    is part of the library (at most NO_ALLOC_WORKSPACE_BYTES per internal batch; larger searches
+    raise CuvsError), without allocating device memory.  Returns (distances, neighbors)."""
+    res, own = _prep(resources)
+    qv, nv, dv = dlpack.view(queries), dlpack.view(neighbors), dlpack.view(distances)
+    check(lib().cuvsAmdIvfPqSearchNoAlloc(res.get_c_obj(), search_params._p, index.index, qv.ptr,
+                                          nv.ptr, dv.ptr))
+    if own:
+        res.sync()
+    return distances, neighbors
+
+
 def select_clusters(search_params, index, queries, resources=None):
     """Probe lists [n_queries, min(n_probes, n_lists)] as an int32 tensor holding uint32 values."""
     torch = _torch()

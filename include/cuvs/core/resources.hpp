@@ -126,6 +126,13 @@ class resources {
   void reserve_workspace(size_t bytes);
   void reset_workspace() { workspace_used_ = 0; }
   size_t workspace_capacity() const { return workspace_capacity_; }
+  /**
+   * Serve the workspace from `bytes` of device memory that somebody else owns (256-byte aligned)
+   * from now on: the handle then never allocates or frees device memory for it, and a call that
+   * needs more fails instead of growing it.  For handles that have no workspace yet.
+   */
+  void borrow_workspace(void* ptr, size_t bytes);
+  bool workspace_borrowed() const { return workspace_borrowed_; }
 
   bool profiling = false;
   struct profile_state;
@@ -142,6 +149,7 @@ class resources {
   std::vector<void*> retired_;  // outgrown workspaces, released at destruction / next sync point
   std::shared_ptr<memory::pool> pool_;  // set_workspace_pool
   bool workspace_pooled_ = false;       // workspace_ came out of pool_
+  bool workspace_borrowed_ = false;     // workspace_ belongs to the caller of borrow_workspace
   void release_workspace();
   memory::tracker* tracker_ = nullptr;  // track_memory
 };

@@ -209,6 +209,25 @@ CUVS_EXPORT cuvsError_t cuvsAmdIvfPqSearchWithBitset(cuvsResources_t res,
                                                      DLManagedTensor* bitset,
                                                      int64_t n_bits);
 
+/** cuvsIvfPqSearch for callers that cannot allocate device memory: code under HIP graph capture,
+ *  tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the cuVS C API.  Same
+ *  arguments, checks and results as cuvsIvfPqSearch (it runs the same kernels on the stream of
+ *  `res`), but the workspace between the stages of the search is a fixed array of
+ *  CUVS_AMD_NO_ALLOC_WORKSPACE_BYTES in the library's device image instead of the handle's cached
+ *  allocation, and the call makes no hipMalloc / hipFree.  One internal batch
+ *  (min(n_queries, max_internal_batch_size) queries) must fit that array, or the call fails with a
+ *  message that states the bytes needed: roughly 4 * n_lists + 32 * n_probes * k + 100 * n_probes
+ *  + 12 * dim bytes per query (a few hundred queries at 16384 lists, 64 probes, k = 10).  Every
+ *  GPU holds one such array: calls that overlap on one GPU race on it.  Profiling
+ *  (cuvsAmdIvfPqProfilingEnable) does not apply to this call. */
+#define CUVS_AMD_NO_ALLOC_WORKSPACE_BYTES ((size_t)32 << 20)
+CUVS_EXPORT cuvsError_t cuvsAmdIvfPqSearchNoAlloc(cuvsResources_t res,
+                                                  cuvsIvfPqSearchParams_t search_params,
+                                                  cuvsIvfPqIndex_t index,
+                                                  DLManagedTensor* queries,
+                                                  DLManagedTensor* neighbors,
+                                                  DLManagedTensor* distances);
+
 /** cuvsIvfPqExtend with list labels chosen by the caller (device uint32 [n]) instead of the
  *  library's own nearest-centre assignment; the C form of extending lists the way the C++ helper
  *  cuvs::neighbors::ivf_pq::helpers::extend_list does for pre-assigned rows.  For callers that
