@@ -5,9 +5,17 @@
 One step = one `cuvsIvfPqSearch` call over the whole query batch with the queries already in HBM.
 Workload (BASELINE.json configs[2], the configuration the metric is quoted on): 10M x 128 uint8
 SIFT-like rows, n_lists = 16384, pq_dim = 64, pq_bits = 8, 10,000 queries, k = 10, n_probes = 64,
-fp16 lookup table with fp32 internal distances.  Prints ONE JSON line with the QPS, recall@10, the
-roofline of the code-scan kernel and a CPU baseline (the oracle, multithreaded, on a bounded
-query sample).
+fp16 lookup table with fp32 internal distances.  Prints ONE JSON line with the QPS and recall@10 of the
+library's default path, the roofline of the code-scan kernel and a CPU baseline (the oracle,
+multithreaded, on a bounded query sample).
+
+The roofline is the one the metric defines: algorithmic bytes of the code stream = sum over all
+(query, probed list) pairs of round_up(list size, 32) * bytes per encoded row, over the duration of
+the kernel that streams them.  The default path does not stream those bytes for L2 metrics (it
+drops most pairs after their leading codes), so the same batch is also run with the early stop
+switched off on the handle (cuvsAmdIvfPqSetSearchTuning): one launch of the scan kernel over every
+probed list in full, timed with HIP events on the library's stream.  `roofline` is that launch;
+`default_path` holds the launches of the path that `value` was measured on.
 
 `--config N` (0..4) runs another of BASELINE.json's configurations at its real shape instead (same
 JSON line; the CPU baseline only with `--with-cpu`, since copying a large index to the host takes
@@ -25,12 +33,6 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
-
-# HBM bytes per launch of the named kernel on the default workload, from hardware counters (FETCH_SIZE + WRITE_SIZE
-# per dispatch, each scaled by its reading for the 1 GiB calibration copy below); the counter runs
-# are summarised under profiles/.  Keyed by (kernel, lut, internal); None where not measured.
-MEASURED_TRAFFIC = {("scan_screen_direct_kernel", "f16", "f32"): 1.216e9}
-
 
 # BASELINE.json's configurations; `dataset` names the generator below
 CONFIGS = {
@@ -51,7 +53,7 @@ def make_rows(name, n, dim, device):
     """Synthetic rows of BASELINE.json's configurations (seeded)."""
     import torch
 
-    from cuvs_amd import testing
+    import datasets as testing
     if name == "sift_u8":
         return testing.sift_like_u8(n, dim, 4096, seed=1234, device=device)
     if name == "mixture64_f32":
@@ -108,7 +110,9 @@ def main():
     import numpy as np
     import torch
 
-    from cuvs_amd import ivf_pq, refine, testing
+    import datasets as testing
+
+    from cuvs_amd import ivf_pq, refine
     from cuvs_amd.resources import Resources
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
@@ -201,17 +205,32 @@ def main():
     log(f"{ms_per_step:.2f} ms per batch of {nq}: {qps:,.0f} QPS, recall@{k} {gpu_recall:.4f}")
 
     # per-kernel times of the scan stage: HIP events on the library's stream, same steps again
-    res.enable_profiling(True)
-    prof = []
-    for _ in range(args.steps):
-        step()
-        prof.append(ivf_pq.get_search_profile(res))
-    res.enable_profiling(False)
+    def profiled(steps):
+        res.enable_profiling(True)
+        prof = []
+        for _ in range(steps):
+            step()
+            prof.append(ivf_pq.get_search_profile(res))
+        res.enable_profiling(False)
+        return prof
+
+    def timed(steps, warmup):
+        for _ in range(warmup):
+            step()
+        res.sync()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        res.sync()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
+    prof = profiled(args.steps)
     stage = prof[-1]
     launches = max(stage["n_scan_launches"], 1)
-    mean = lambda f: float(np.mean([p[f] for p in prof])) / launches
-    scan_stage_ms = mean("scan_ms")
-    bytes_all_lists = stage["scan_bytes"] / launches
+    mean = lambda pr, f: float(np.mean([p[f] for p in pr]))
+    scan_bytes = float(stage["scan_bytes"])  # all probed lists in full, summed on the device from the probe lists
     early_stop = stage["n_screened_pairs"] > 0
     pq_len = dim // pq_dim
     nibble = pq_bits == 4 and pq_dim % 32 == 0 and pq_len in (1, 2, 4) and (pq_dim // 16) * pq_len <= 48
@@ -220,32 +239,60 @@ def main():
                  else "scan_nibble_kernel" if nibble
                  else "scan_kernel" if (pq_bits != 8 or (pq_dim, pq_len) not in ((64, 2), (48, 2), (32, 4)))
                  else "scan_quad_kernel" if (args.lut != "f32" and k <= 128) else "scan_fast_kernel")
+    default_path = {"early_stop": bool(early_stop), "ms_per_step": ms_per_step, "qps": qps,
+                    "scan_stage_ms": mean(prof, "scan_ms"),
+                    "stage_ms": {s_: mean(prof, s_) for s_ in ("coarse_ms", "rotate_ms", "scan_ms", "merge_ms")}}
     if early_stop:
-        # The scan stage is three launches: the leading probes' lists in full, the screen of every
-        # other pair on its leading 8 codes (8 bytes a row: from the packed plane of leading codes
-        # in the table-free screen, from the interleaved lists in the table-building screen that
-        # per-cluster codebooks use), and the surviving pairs in full.  The roofline is quoted
-        # for the longest of the three (the screen on the default workload).
+        # three launches: the leading probes' lists in full, the screen of every other pair on its
+        # 8 leading codes (8 bytes a row), the surviving pairs in full
         screen_name = "scan_screen_kernel" if args.kind == "cluster" else "scan_screen_direct_kernel"
-        parts = {"lead_scan": (mean("lead_scan_ms"), stage["lead_bytes"] / launches),
-                 "screen": (mean("screen_ms"), stage["screen_bytes"] / launches),
-                 "survivor_scan": (mean("survivor_scan_ms"), stage["survivor_bytes"] / launches)}
-        longest = max(parts, key=lambda name: parts[name][0])
-        kernel_name = screen_name if longest == "screen" else full_name
-        kernel_ms, kernel_bytes = parts[longest]
-    else:
-        parts = {}
-        kernel_name = full_name
-        kernel_ms, kernel_bytes = scan_stage_ms, bytes_all_lists
-    achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9
-    log(f"{kernel_name} {kernel_ms:.3f} ms per launch, {kernel_bytes / 1e9:.2f} GB algorithmic "
-        f"-> {achieved:.0f} GB/s ({achieved / HBM_PEAK_GBS:.1%} of HBM peak); stages: "
-        f"coarse {stage['coarse_ms']:.2f} rotate {stage['rotate_ms']:.2f} scan {stage['scan_ms']:.2f} "
-        f"merge {stage['merge_ms']:.2f} ms")
-    if early_stop:
-        log("scan stage: " + ", ".join(f"{n} {ms:.3f} ms / {b / 1e9:.2f} GB" for n, (ms, b) in parts.items())
+        parts = {"lead_scan": (full_name, mean(prof, "lead_scan_ms"), float(stage["lead_bytes"])),
+                 "screen": (screen_name, mean(prof, "screen_ms"), float(stage["screen_bytes"])),
+                 "survivor_scan": (full_name, mean(prof, "survivor_scan_ms"), float(stage["survivor_bytes"]))}
+        default_path["launches"] = {
+            name: {"kernel": kn, "ms": ms, "bytes_read_by_the_algorithm": b,
+                   "rate_on_those_bytes_GBs": b / (ms * 1e-3) / 1e9 if ms > 0 else None}
+            for name, (kn, ms, b) in parts.items()}
+        default_path["launches"]["screen"]["note"] = (
+            "8 bytes per padded row of every screened pair: a unit of this library's own, served "
+            "largely from L2 (pairs run in list order), not the metric's code stream")
+        default_path["pairs_screened"] = int(stage["n_screened_pairs"])
+        default_path["pairs_surviving"] = int(stage["n_surviving_pairs"])
+        log("default path, scan stage: " + ", ".join(f"{n_} {ms:.3f} ms / {b / 1e9:.2f} GB"
+                                                     for n_, (_, ms, b) in parts.items())
             + f"; {stage['n_surviving_pairs']} of {stage['n_screened_pairs']} screened pairs kept; "
-            f"all probed lists in full would be {bytes_all_lists / 1e9:.2f} GB")
+            f"all probed lists in full are {scan_bytes / 1e9:.2f} GB")
+
+    # The code stream in full: the same batch with the early stop switched off on the handle.  One
+    # launch of the scan kernel per internal batch reads every probed list.
+    if early_stop:
+        res.set_search_tuning(early_stop="off")
+        full_ms_per_step = timed(args.steps, args.warmup)
+        full_prof = profiled(args.steps)
+        full_ids = neighbors.cpu().numpy().copy()
+        res.set_search_tuning(early_stop="auto")
+        assert full_prof[-1]["n_screened_pairs"] == 0
+        same_ids = bool((full_ids == gpu_ids).all()) if args.refine_ratio <= 1 else None
+    else:
+        full_ms_per_step, full_prof, same_ids = ms_per_step, prof, None
+    full_launches = max(full_prof[-1]["n_scan_launches"], 1)
+    kernel_ms = mean(full_prof, "scan_ms") / full_launches
+    kernel_bytes = float(full_prof[-1]["scan_bytes"]) / full_launches
+    achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9
+    log(f"code stream in full: {full_name} {kernel_ms:.3f} ms per launch, {kernel_bytes / 1e9:.2f} GB algorithmic "
+        f"-> {achieved:.0f} GB/s ({achieved / HBM_PEAK_GBS:.1%} of HBM peak); {full_ms_per_step:.2f} ms per batch = "
+        f"{nq / full_ms_per_step * 1e3:,.0f} QPS" + (f"; ids identical to the default path: {same_ids}" if same_ids is not None else ""))
+
+    # the reference's default max_internal_batch_size (4096): what a drop-in caller gets
+    sp_saved = sp
+    default_batching = None
+    if nq > 4096:
+        sp = ivf_pq.SearchParams(n_probes=P, lut_dtype=lut_np, internal_distance_dtype=int_np)
+        ms_4096 = timed(args.steps, args.warmup)
+        default_batching = {"max_internal_batch_size": 4096, "ms_per_step": ms_4096, "qps": nq / ms_4096 * 1e3}
+        log(f"max_internal_batch_size = 4096 (the reference's default): {ms_4096:.2f} ms per batch = "
+            f"{nq / ms_4096 * 1e3:,.0f} QPS")
+        sp = sp_saved
 
     # A plain copy of known size (1 GiB read + 1 GiB written), outside every timed region: it gives
     # hardware-counter runs of this same command the reading of FETCH_SIZE / WRITE_SIZE per byte.
@@ -254,11 +301,6 @@ def main():
     torch.add(calib, 1, out=calib_out)
     torch.cuda.synchronize()
     del calib, calib_out
-
-    default_workload = (args.config == 2 and (n, nq, n_lists, P, k, dim, pq_dim, pq_bits) ==
-                        (10_000_000, 10_000, 16384, 64, 10, 128, 64, 8))
-    traffic = (MEASURED_TRAFFIC.get((kernel_name, args.lut, args.internal))
-               if default_workload else None)
 
     out = {
         "metric": ("QPS@recall@10 (10M x 128 IVF-PQ, batch 10k); code-scan HBM GB/s vs peak" if args.config == 2
@@ -275,24 +317,23 @@ def main():
                    "pq_bits": pq_bits, "n_queries": nq, "k": k, "n_probes": P,
                    "lut_dtype": args.lut, "internal_distance_dtype": args.internal,
                    "refine_ratio": args.refine_ratio,
-                   "recall_at_k": gpu_recall,
-                   "stage_ms": {s: stage[s] for s in ("coarse_ms", "rotate_ms", "scan_ms", "merge_ms")}},
+                   "recall_at_k": gpu_recall},
+        # the code-scan kernel streaming every probed list in full: algorithmic bytes as the metric
+        # defines them over the HIP-event time of that one launch; HBM traffic from hardware
+        # counters is not measured by this script (profiles/ holds the counter runs)
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": kernel_name, "kernel_ms": kernel_ms,
-                     "algorithmic_bytes_per_launch": kernel_bytes},
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": full_name, "kernel_ms": kernel_ms,
+                     "algorithmic_bytes_per_launch": kernel_bytes,
+                     "path": ("early stop switched off on the handle: every probed list streamed in full"
+                              if early_stop else "the default path streams every probed list in full"),
+                     "ms_per_step_on_this_path": full_ms_per_step,
+                     "qps_on_this_path": nq / full_ms_per_step * 1e3,
+                     "ids_identical_to_default_path": same_ids},
+        "default_path": default_path,
     }
-    # the whole scan stage: with the L2 early stop most probed lists are dropped after their first
-    # chunk, so the bytes of all probed lists in full are NOT what is streamed; both are stated
-    out["scan_stage"] = {
-        "ms": scan_stage_ms, "early_stop": bool(early_stop),
-        "bytes_all_probed_lists_in_full": bytes_all_lists,
-        "equivalent_GBs_if_all_lists_were_streamed": bytes_all_lists / (scan_stage_ms * 1e-3) / 1e9,
-        "launches": {n: {"ms": ms, "algorithmic_bytes": b, "GBs": b / (ms * 1e-3) / 1e9 if ms > 0 else None}
-                     for n, (ms, b) in parts.items()},
-        "pairs_screened": int(stage["n_screened_pairs"]),
-        "pairs_surviving": int(stage["n_surviving_pairs"]),
-    }
+    if default_batching is not None:
+        out["default_batching"] = default_batching
 
     if not args.no_cpu and args.refine_ratio <= 1:
         out["cpu_baseline"] = cpu_baseline(args, index, model, queries, truth, gpu_ids, dim, pq_dim,
@@ -308,7 +349,7 @@ def cpu_baseline(args, index, model, queries, truth, gpu_ids, dim, pq_dim, pq_bi
     import numpy as np
 
     import gpu_helpers as G
-    from cuvs_amd import testing
+    import datasets as testing
     from oracle import oracle
 
     t0 = time.time()

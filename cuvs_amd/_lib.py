@@ -61,6 +61,11 @@ class IndexStruct(C.Structure):
     _fields_ = [("addr", C.c_void_p), ("dtype", DLDataType)]
 
 
+class SearchTuningStruct(C.Structure):
+    _fields_ = [("early_stop", C.c_int32), ("generic_scan", C.c_int32), ("plain_coarse", C.c_int32),
+                ("reserved_", C.c_int32 * 5)]
+
+
 class SearchProfileStruct(C.Structure):
     _fields_ = [("n_queries", C.c_uint32), ("n_probes", C.c_uint32), ("k", C.c_uint32),
                 ("n_scan_launches", C.c_uint32), ("coarse_ms", C.c_float),
@@ -93,7 +98,7 @@ EXPORTED_SYMBOLS = [
     "cuvsIvfPqIndexGetListIndices", "cuvsIvfPqBuild", "cuvsIvfPqBuildPrecomputed",
     "cuvsIvfPqSearch", "cuvsIvfPqSerialize", "cuvsIvfPqDeserialize", "cuvsIvfPqExtend",
     "cuvsIvfPqTransform", "cuvsAmdIvfPqSelectClusters", "cuvsAmdIvfPqSearchWithBitset",
-    "cuvsAmdIvfPqSearchNoAlloc",
+    "cuvsAmdIvfPqSearchNoAlloc", "cuvsAmdIvfPqSetSearchTuning",
     "cuvsAmdIvfPqExtendLabeled", "cuvsAmdIvfPqProfilingEnable", "cuvsAmdIvfPqGetSearchProfile",
     "cuvsRefine",
     "cuvsAmdKnnMergeParts",
@@ -178,6 +183,7 @@ def lib():
           T, C.c_int64)
     proto("cuvsAmdIvfPqSearchNoAlloc", res_t, P(SearchParamsStruct), P(IndexStruct), T, T, T)
     proto("cuvsAmdIvfPqExtendLabeled", res_t, T, T, T, P(IndexStruct))
+    proto("cuvsAmdIvfPqSetSearchTuning", res_t, P(SearchTuningStruct))
     proto("cuvsAmdIvfPqProfilingEnable", res_t, C.c_bool)
     proto("cuvsAmdIvfPqGetSearchProfile", res_t, P(SearchProfileStruct))
     _lib = L

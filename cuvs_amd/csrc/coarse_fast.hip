@@ -27,6 +27,8 @@
  */
 #include "device_utils.cuh"
 
+#include <mutex>
+
 #include <algorithm>
 
 namespace cuvs::neighbors::ivf_pq::detail {
@@ -490,6 +492,18 @@ void launch_pack_centers_f16(const float* centers, uint32_t n_lists, uint32_t di
   CUVS_HIP_TRY(hipGetLastError());
 }
 
+namespace {
+template <typename K1, typename K2>
+void lds_limit_once(int which, K1 k1, K2 k2, size_t smem)
+{
+  static std::once_flag flags[2];
+  std::call_once(flags[which], [&] {
+    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k1), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k2), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+  });
+}
+}  // namespace
+
 void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
 {
   const uint32_t q_pad = coarse_pad(a.n_queries);
@@ -531,12 +545,7 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
   const uint32_t n_list_tiles = l_pad / kTile;
   // A block costs about two tile-times of set-up besides its tiles, and the grid runs in rounds of
   // one block per CU: take the run length whose rounds x (tiles + 2) is smallest.
-  static int n_cu = 0;
-  if (n_cu == 0) {
-    int dev = 0;
-    CUVS_HIP_TRY(hipGetDevice(&dev));
-    CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-  }
+  const int n_cu = device_cu_count();
   const uint32_t n_qblocks = (q_pad + kQTile - 1) / kQTile;
   uint32_t tiles_per_block = 1;
   uint64_t best_cost       = ~uint64_t(0);
@@ -554,12 +563,9 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
     // list tiles (two buffers), their norm terms, and the larger of the two passes' per-query areas
     const size_t smem = size_t(2) * kTile * (k_pad * 2 + 16) + 2 * kTile * 4 +
                         std::max<size_t>(size_t(kQTile) * kTilesPerBlock * 8 * 4, size_t(kQTile) * (1 + kLocalCap) * 4);
-    static bool attr_set = false;
-    if (!attr_set) {
-      CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k1), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
-      CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k2), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
-      attr_set = true;
-    }
+    // a generic lambda has one body per pair of argument types, and the kernels of both K_PAD
+    // values have the same type: the flag is keyed by K_PAD explicitly
+    lds_limit_once(k_pad == 64 ? 0 : 1, k1, k2, smem);
     k1<<<grid, kGemmThreads, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, q_pad, n_list_tiles, tiles_per_block, alpha,
                                     qterm, a.minima, n_groups, nullptr, nullptr, nullptr);
     CUVS_HIP_TRY(hipGetLastError());

@@ -119,6 +119,7 @@ struct index_impl {
   // norms, and the largest centre length / |stored norm| (coarse_fast_ok: all finite and within
   // binary16's range)
   device_buffer centers_h, center_norms;
+  device_buffer centers_i8;  // [coarse_i8_words(dim)][coarse_pad(n_lists)] words: centres for the 8-bit coarse search
   float c_max = 0.0f, n_max = 0.0f;
   bool coarse_fast_ok = false;
   /** centers_t, centers_h, center_norms and the maxima from `centers` (synchronises). */
@@ -186,6 +187,14 @@ void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_li
                           uint32_t n_probes, uint32_t* probes, hipStream_t stream,
                           const uint8_t* only = nullptr);
 
+/* coarse search in 8-bit integers (coarse_i8.hip): 32-bit words of the quantised centre rows,
+ * word-major, and scores written as floats that order like the integer scores */
+uint32_t coarse_i8_words(uint32_t dim);
+void launch_pack_centers_i8(const float* centers, uint32_t n_lists, uint32_t dim, uint32_t dim_ext,
+                            uint32_t* ct8, hipStream_t stream);
+void launch_coarse_scores_i8(const float* qf, const uint32_t* ct8, uint32_t n_queries, uint32_t n_lists,
+                             uint32_t dim, bool ip_like, float* scores, hipStream_t stream);
+
 /* probe selection in two precisions (coarse_fast.hip) */
 struct coarse_fast_args {
   const void* queries;     // [n_queries, dim] of `type` (f16, i8 or u8)
@@ -214,9 +223,13 @@ void launch_pack_centers_f16(const float* centers, uint32_t n_lists, uint32_t di
                              _Float16* ch, float* cn, uint32_t* stats, hipStream_t stream);
 void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream);
 
-/** rot_q = rotation * qf (+ row normalisation for cosine); rotation_t is [dim, rot_dim]. */
+/** rot_q = rotation * qf (+ row normalisation for cosine); rotation_t is [dim, rot_dim].
+ *  `operand_dtype` is the coarse search's type, whose query rows and copy of the rotation matrix
+ *  the reference's rotation GEMM takes (ivf_pq_search.cuh:996-1019): CUDA_R_32F as they are,
+ *  CUDA_R_16F both rounded to binary16, CUDA_R_8I both as trunc(clamp(128 x)) with the integer
+ *  dot product scaled by 1 / 128^2. */
 void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries, uint32_t dim,
-                   uint32_t rot_dim, bool identity, bool normalize, float* rot_q,
+                   uint32_t rot_dim, bool identity, bool normalize, int operand_dtype, float* rot_q,
                    hipStream_t stream);
 
 /** chunk_indices[q, p] = inclusive prefix sum of list_sizes[probes[q, p]]; n_samples[q] = total.
@@ -283,7 +296,6 @@ struct scan_args {
   uint32_t* query_kth;            // [n_queries] ordered-score upper bounds (fused)
   unsigned long long* out_keys;   // fused: [n_queries, n_probes, k]
   float* out_scores;              // non-fused: [n_queries, max_samples]
-  unsigned long long* timing;     // per-phase cycle sums (instrumented builds only), or null
   void* global_lut;               // generic kernel: table scratch when it does not fit LDS, or null
   const uint64_t* lead_plane;     // first eight code bytes of every row slot (8-bit codes), or null
 };
@@ -384,7 +396,9 @@ void launch_refine(const void* dataset, const void* queries, elem_type type,
 
 /* list maintenance and encoding */
 void launch_normalize_rows(float* x, uint64_t n_rows, uint32_t dim, hipStream_t stream);
-void launch_histogram(const uint32_t* labels, uint64_t n, uint32_t* counts, hipStream_t stream);
+/** counts[l] += number of labels equal to l, for l < n_bins; larger labels are skipped. */
+void launch_histogram(const uint32_t* labels, uint64_t n, uint32_t n_bins, uint32_t* counts,
+                      hipStream_t stream);
 void launch_relocate_lists(const uint8_t* old_codes, const int64_t* old_ids, uint8_t* new_codes,
                            int64_t* new_ids, const uint64_t* old_row_offsets,
                            const uint64_t* new_row_offsets, const uint32_t* old_sizes,

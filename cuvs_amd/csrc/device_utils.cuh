@@ -21,6 +21,32 @@ constexpr unsigned long long kInvalidKey = 0xFFFFFFFFFFFFFFFFull;
 /* small device helpers                                                                      */
 /* ---------------------------------------------------------------------------------------- */
 
+/** Compute units of the current device, asked once per process (function-local statics are
+ *  initialised exactly once also when several host threads make their first call together). */
+inline int device_cu_count()
+{
+  static const int n = [] {
+    int dev = 0, count = 0;
+    CUVS_HIP_TRY(hipGetDevice(&dev));
+    CUVS_HIP_TRY(hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, dev));
+    return count;
+  }();
+  return n;
+}
+
+/** Raises the kernel's dynamic LDS limit to `smem_limit` and returns how many blocks of `block`
+ *  threads with `smem` bytes of dynamic LDS fit one compute unit (at least 1).  Meant to initialise
+ *  a `static const int` of the launcher of one kernel instance. */
+template <typename Kernel>
+inline int prepare_persistent_kernel(Kernel kernel, int block, size_t smem, size_t smem_limit)
+{
+  CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, int(smem_limit)));
+  int occ = 0;
+  CUVS_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kernel, block, smem));
+  return occ > 0 ? occ : 1;
+}
+
 /** Monotone map float -> uint32 (ascending); -0 and +0 map to the same key. */
 __device__ __forceinline__ uint32_t order_f32(float f)
 {

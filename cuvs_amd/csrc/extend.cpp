@@ -215,7 +215,7 @@ void extend(cuvs::resources const& res,
   /* 2. new list sizes */
   device_buffer counts(sizeof(uint32_t) * ix.n_lists);
   detail::launch_fill_u32(counts.as<uint32_t>(), 0, ix.n_lists, s);
-  detail::launch_histogram(labels.as<uint32_t>(), n_rows, counts.as<uint32_t>(), s);
+  detail::launch_histogram(labels.as<uint32_t>(), n_rows, ix.n_lists, counts.as<uint32_t>(), s);
   std::vector<uint32_t> h_counts(ix.n_lists);
   CUVS_HIP_TRY(hipMemcpyAsync(h_counts.data(), counts.ptr, sizeof(uint32_t) * ix.n_lists,
                               hipMemcpyDeviceToHost, s));
@@ -223,7 +223,10 @@ void extend(cuvs::resources const& res,
   if (labels_in != nullptr) {
     uint64_t total = 0;
     for (uint32_t c : h_counts) { total += c; }
-    CUVS_EXPECTS(total == n_rows, "labels must be smaller than n_lists");
+    // labels >= n_lists were left out of the histogram (nothing has been written to the index yet)
+    CUVS_EXPECTS(total == n_rows, "labels must be smaller than n_lists (%u): %llu of %llu are not",
+                 ix.n_lists, static_cast<unsigned long long>(n_rows - total),
+                 static_cast<unsigned long long>(n_rows));
   }
 
   /* 3. new arena layout: every list owns round_up(size, 32) rows */

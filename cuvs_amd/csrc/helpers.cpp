@@ -82,7 +82,7 @@ void reconstruct(cuvs::resources const& res, const index_impl& ix, void* out, el
     xf = flat.as<float>();
   }
   detail::launch_rotate(rot.as<float>(), ix.rotation.as<float>(), uint32_t(n_rows), ix.rot_dim, ix.dim,
-                        false, false, xf, s);
+                        false, false, CUDA_R_32F, xf, s);
   if (type != elem_type::f32) { detail::launch_unmap_rows(xf, uint64_t(n_rows) * ix.dim, type, out, s); }
   CUVS_HIP_TRY(hipStreamSynchronize(s));  // the temporaries go out of scope
 }
@@ -349,7 +349,7 @@ void rotate_padded_centers(cuvs::resources const& res, device_matrix_view<const 
   }
   CUVS_HIP_TRY(hipMemcpyAsync(rot_t.ptr, rt.data(), rt.size() * sizeof(float), hipMemcpyHostToDevice, s));
   detail::launch_rotate(flat.as<float>(), rot_t.as<float>(), uint32_t(n), uint32_t(dim), uint32_t(rot_dim),
-                        false, false, rotated_centers.data_handle(), s);
+                        false, false, CUDA_R_32F, rotated_centers.data_handle(), s);
   CUVS_HIP_TRY(hipStreamSynchronize(s));  // the temporaries go out of scope
 }
 

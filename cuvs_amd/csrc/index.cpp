@@ -106,6 +106,8 @@ void index_impl::refresh_coarse(hipStream_t stream)
     centers_h.allocate(size_t(l_pad) * k_pad * sizeof(_Float16));
     center_norms.allocate(size_t(l_pad) * sizeof(float));
   }
+  if (centers_i8.bytes == 0) { centers_i8.allocate(size_t(coarse_i8_words(dim)) * l_pad * sizeof(uint32_t)); }
+  launch_pack_centers_i8(centers.as<float>(), n_lists, dim, dim_ext, centers_i8.as<uint32_t>(), stream);
   device_buffer stats(16);
   launch_pack_centers_f16(centers.as<float>(), n_lists, dim, dim_ext, centers_h.as<_Float16>(),
                           center_norms.as<float>(), stats.as<uint32_t>(), stream);
@@ -262,6 +264,7 @@ index<int64_t> clone(cuvs::resources const& res, const index<int64_t>& source)
   copy(dst.centers_t, src.centers_t);
   copy(dst.centers_h, src.centers_h);
   copy(dst.center_norms, src.center_norms);
+  copy(dst.centers_i8, src.centers_i8);
   copy(dst.codes_arena, src.codes_arena);
   copy(dst.ids_arena, src.ids_arena);
   copy(dst.lead_plane, src.lead_plane);

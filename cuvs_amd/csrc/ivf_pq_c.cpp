@@ -637,6 +637,18 @@ cuvsError_t cuvsIvfPqDeserialize(cuvsResources_t res, const char* filename, cuvs
   });
 }
 
+cuvsError_t cuvsAmdIvfPqSetSearchTuning(cuvsResources_t res, const cuvsAmdIvfPqSearchTuning* tuning)
+{
+  return translate_exceptions([=] {
+    CUVS_EXPECTS(tuning != nullptr, "tuning must not be null");
+    CUVS_EXPECTS(tuning->early_stop >= 0 && tuning->early_stop <= 2, "early_stop must be 0, 1 or 2");
+    auto& t        = res_of(res)->tuning;
+    t.early_stop   = tuning->early_stop;
+    t.generic_scan = tuning->generic_scan != 0;
+    t.plain_coarse = tuning->plain_coarse != 0;
+  });
+}
+
 cuvsError_t cuvsAmdIvfPqProfilingEnable(cuvsResources_t res, bool enable)
 {
   return translate_exceptions([=] { res_of(res)->profiling = enable; });

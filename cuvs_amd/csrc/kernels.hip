@@ -334,26 +334,36 @@ __global__ __launch_bounds__(kBlock) void rotate_kernel(const float* __restrict_
                                                          const float* __restrict__ rotation_t,
                                                          uint32_t n_queries, uint32_t dim,
                                                          uint32_t rot_dim, int identity,
-                                                         int normalize, float* __restrict__ rot_q)
+                                                         int normalize, int mode,
+                                                         float* __restrict__ rot_q)
 {
+  // mode 0: fp32 operands; 1: both rounded to binary16; 2: both as trunc(clamp(128 x)), an integer
+  // dot product (exact in fp32 for dim <= 1024) times 1 / 128^2
+  auto operand = [mode](float v) -> float {
+    if (mode == 1) { return float(_Float16(v)); }
+    if (mode == 2) { return float(int(fmaxf(-128.0f, fminf(127.0f, v * 128.0f)))); }
+    return v;
+  };
   extern __shared__ __align__(16) unsigned char dyn_smem[];
   float* sq           = reinterpret_cast<float*>(dyn_smem);  // [kRotQueries][dim]
   float* sr           = sq + kRotQueries * dim;              // [kRotQueries][rot_dim]
   __shared__ float s_norm[kRotQueries];
   const uint32_t q0   = blockIdx.x * kRotQueries;
   const uint32_t nq   = (n_queries - q0) < uint32_t(kRotQueries) ? (n_queries - q0) : kRotQueries;
-  for (uint32_t i = threadIdx.x; i < nq * dim; i += kBlock) { sq[i] = qf[uint64_t(q0) * dim + i]; }
+  for (uint32_t i = threadIdx.x; i < nq * dim; i += kBlock) { sq[i] = operand(qf[uint64_t(q0) * dim + i]); }
   __syncthreads();
   for (uint32_t r = threadIdx.x; r < rot_dim; r += kBlock) {
     float acc[kRotQueries];
 #pragma unroll
     for (int i = 0; i < kRotQueries; i++) { acc[i] = 0.0f; }
     if (identity) {
+      // a diagonal of ones: exact in binary16; 127 as an 8-bit integer
+      const float one = operand(1.0f);
 #pragma unroll
-      for (int i = 0; i < kRotQueries; i++) { acc[i] = (uint32_t(i) < nq) ? sq[i * dim + r] : 0.0f; }
+      for (int i = 0; i < kRotQueries; i++) { acc[i] = (uint32_t(i) < nq) ? one * sq[i * dim + r] : 0.0f; }
     } else {
       for (uint32_t d = 0; d < dim; d++) {
-        const float w = rotation_t[uint64_t(d) * rot_dim + r];
+        const float w = operand(rotation_t[uint64_t(d) * rot_dim + r]);
 #pragma unroll
         for (int i = 0; i < kRotQueries; i++) {
           if (uint32_t(i) < nq) { acc[i] = fmaf(w, sq[i * dim + d], acc[i]); }
@@ -362,7 +372,7 @@ __global__ __launch_bounds__(kBlock) void rotate_kernel(const float* __restrict_
     }
 #pragma unroll
     for (int i = 0; i < kRotQueries; i++) {
-      if (uint32_t(i) < nq) { sr[i * rot_dim + r] = acc[i]; }
+      if (uint32_t(i) < nq) { sr[i * rot_dim + r] = mode == 2 ? acc[i] * (1.0f / 128.0f / 128.0f) : acc[i]; }
     }
   }
   __syncthreads();
@@ -911,11 +921,15 @@ __global__ void normalize_rows_kernel(float* __restrict__ x, uint64_t n_rows, ui
   }
 }
 
-__global__ void histogram_kernel(const uint32_t* __restrict__ labels, uint64_t n,
+__global__ void histogram_kernel(const uint32_t* __restrict__ labels, uint64_t n, uint32_t n_bins,
                                  uint32_t* __restrict__ counts)
 {
+  // labels outside the bins are not counted: the caller sees them as a short total
   const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i < n) { atomicAdd(&counts[labels[i]], 1u); }
+  if (i < n) {
+    const uint32_t l = labels[i];
+    if (l < n_bins) { atomicAdd(&counts[l], 1u); }
+  }
 }
 
 /** One block per list: move the occupied 32-row groups and ids to their new arena position. */
@@ -1187,10 +1201,11 @@ void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_li
 }
 
 void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries, uint32_t dim,
-                   uint32_t rot_dim, bool identity, bool normalize, float* rot_q,
+                   uint32_t rot_dim, bool identity, bool normalize, int operand_dtype, float* rot_q,
                    hipStream_t stream)
 {
   if (n_queries == 0) { return; }
+  const int mode = operand_dtype == CUDA_R_16F ? 1 : (operand_dtype == CUDA_R_8I ? 2 : 0);
   const size_t smem = size_t(kRotQueries) * (dim + rot_dim) * sizeof(float);
   CUVS_EXPECTS(smem <= 150 * 1024, "dim (%u) is too large for the rotation kernel", dim);
   if (smem > 32 * 1024) {
@@ -1198,7 +1213,7 @@ void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries,
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
   }
   rotate_kernel<<<blocks_for(n_queries, kRotQueries), kBlock, smem, stream>>>(
-    qf, rotation_t, n_queries, dim, rot_dim, identity ? 1 : 0, normalize ? 1 : 0, rot_q);
+    qf, rotation_t, n_queries, dim, rot_dim, identity ? 1 : 0, normalize ? 1 : 0, mode, rot_q);
   CUVS_LAUNCH_CHECK();
 }
 
@@ -1245,12 +1260,12 @@ void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
   }
   {
     const size_t smem = size_t(kScanTile + kScanThreads) * 4;
-    static bool attr_set = false;
-    if (!attr_set) {
+    static const int attr_set = [&] {
       CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(exclusive_scan_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
-      attr_set = true;
-    }
+      return 1;
+    }();
+    (void)attr_set;
     exclusive_scan_kernel<<<1, kScanThreads, smem, stream>>>(counts, n_bins, cursors);
   }
   CUVS_LAUNCH_CHECK();
@@ -1293,13 +1308,7 @@ size_t scan_lut_bytes(const scan_args& a)
 
 uint32_t scan_global_lut_blocks()
 {
-  static int n_cu = 0;
-  if (n_cu == 0) {
-    int dev = 0;
-    CUVS_HIP_TRY(hipGetDevice(&dev));
-    CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-  }
-  return uint32_t(n_cu) * 4u;
+  return uint32_t(device_cu_count()) * 4u;
 }
 
 size_t scan_lds_bytes(const scan_args& a)
@@ -1420,10 +1429,11 @@ void launch_normalize_rows(float* x, uint64_t n_rows, uint32_t dim, hipStream_t 
   CUVS_LAUNCH_CHECK();
 }
 
-void launch_histogram(const uint32_t* labels, uint64_t n, uint32_t* counts, hipStream_t stream)
+void launch_histogram(const uint32_t* labels, uint64_t n, uint32_t n_bins, uint32_t* counts,
+                      hipStream_t stream)
 {
   if (n == 0) { return; }
-  histogram_kernel<<<blocks_for(n, 256), 256, 0, stream>>>(labels, n, counts);
+  histogram_kernel<<<blocks_for(n, 256), 256, 0, stream>>>(labels, n, n_bins, counts);
   CUVS_LAUNCH_CHECK();
 }
 
@@ -1459,7 +1469,7 @@ void launch_rows_by_label(const uint32_t* labels, uint64_t n, uint32_t n_lists, 
   uint32_t* counts  = counters;
   uint32_t* cursors = counters + n_lists;
   launch_fill_u32(counts, 0, n_lists, stream);
-  histogram_kernel<<<blocks_for(n, 256), 256, 0, stream>>>(labels, n, counts);
+  histogram_kernel<<<blocks_for(n, 256), 256, 0, stream>>>(labels, n, n_lists, counts);
   CUVS_LAUNCH_CHECK();
   const size_t smem = size_t(kScanTile + kScanThreads) * 4;
   CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(exclusive_scan_kernel),

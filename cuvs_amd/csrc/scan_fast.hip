@@ -90,19 +90,6 @@ __global__ __launch_bounds__(kBlock, 2) void scan_fast_kernel(scan_args a)
     }
   };
 
-#ifdef CUVS_SCAN_TIMING
-  unsigned long long tm[6] = {0, 0, 0, 0, 0, 0};
-  unsigned long long t_prev = __builtin_readcyclecounter();
-#define TICK(i)                                                    \
-  do {                                                             \
-    const unsigned long long t_now = __builtin_readcyclecounter(); \
-    tm[i] += t_now - t_prev;                                       \
-    t_prev = t_now;                                                \
-  } while (0)
-#else
-#define TICK(i)
-#endif
-
   // software pipeline over the block's pairs: records two pairs ahead, operands one pair ahead
   uint32_t it     = blockIdx.x;
   pair_desc cur_d = a.desc[it];
@@ -142,7 +129,6 @@ __global__ __launch_bounds__(kBlock, 2) void scan_fast_kernel(scan_args a)
         tail->thr   = 0xFFFFFFFFu;
       }
       lds_barrier();
-      TICK(0);  // waiting for the prefetched query / centre, staging
 
       /* ---- lookup table ---- */
 #pragma unroll
@@ -164,9 +150,7 @@ __global__ __launch_bounds__(kBlock, 2) void scan_fast_kernel(scan_args a)
         }
         lut[j * 256 + tid] = traits::encode(score);
       }
-      TICK(1);  // table construction
       lds_barrier();
-      TICK(2);  // barrier after the table
 
       /* ---- scan ---- */
       uint32_t thr           = cur_f.thr;
@@ -241,16 +225,13 @@ __global__ __launch_bounds__(kBlock, 2) void scan_fast_kernel(scan_args a)
           }
         }
       }
-      TICK(3);  // scan
       lds_barrier();
-      TICK(4);  // barrier after the scan
       const uint32_t before = tail->count;
       lds_barrier();
       block_prune(cand, tail, a.k, before);
       const uint32_t cnt = before < a.k ? before : a.k;
       for (uint32_t r = tid; r < a.k; r += kBlock) { out[r] = r < cnt ? cand[r] : kInvalidKey; }
       if (tid == 0 && before >= a.k) { atomicMin(&a.query_kth[q], tail->thr); }
-      TICK(5);  // prune + output
     }
     if (!has_next) { break; }
     it += stride;
@@ -260,11 +241,6 @@ __global__ __launch_bounds__(kBlock, 2) void scan_fast_kernel(scan_args a)
 #pragma unroll
     for (int m = 0; m < NCH; m++) { cur[m] = ahead[m]; }
   }
-#ifdef CUVS_SCAN_TIMING
-  if (a.timing != nullptr && (tid & 63u) == 0) {
-    for (int i = 0; i < 6; i++) { atomicAdd(&a.timing[i], tm[i]); }
-  }
-#endif
 }
 
 template <int NCH, int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER, bool IP>
@@ -274,18 +250,8 @@ void launch_instance(const scan_args& a, hipStream_t stream)
   auto kernel = scan_fast_kernel<NCH, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER, IP>;
   const size_t smem = kLdsBase + size_t(NCH) * 16 * 256 * sizeof(lut_t) +
                       size_t(NCH) * 16 * PQ_LEN * (IP ? 2 : 1) * 4 + size_t(kFastCap) * 8 + sizeof(fast_tail);
-  static int blocks_per_cu = 0;  // per instance
-  static int n_cu          = 0;
-  if (blocks_per_cu == 0) {
-    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
-    int occ = 0;
-    CUVS_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kernel, kBlock, smem));
-    int dev = 0;
-    CUVS_HIP_TRY(hipGetDevice(&dev));
-    CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-    blocks_per_cu = occ > 0 ? occ : 1;
-  }
+  static const int blocks_per_cu = prepare_persistent_kernel(kernel, kBlock, smem, smem);  // per instance
+  const int n_cu                 = device_cu_count();
   uint32_t grid = uint32_t(blocks_per_cu) * uint32_t(n_cu);
   if (a.n_pairs_dev == nullptr) {
     if (grid > a.n_pairs) { grid = a.n_pairs; }

@@ -271,19 +271,6 @@ __global__ __launch_bounds__(kBlock, 2) void scan_nibble_kernel(scan_args a)
     }
   }
 
-#ifdef CUVS_SCAN_TIMING
-  unsigned long long tm[6] = {0, 0, 0, 0, 0, 0};
-  unsigned long long t_prev = __builtin_readcyclecounter();
-#define TICK(i)                                                    \
-  do {                                                             \
-    const unsigned long long t_now = __builtin_readcyclecounter(); \
-    tm[i] += t_now - t_prev;                                       \
-    t_prev = t_now;                                                \
-  } while (0)
-#else
-#define TICK(i)
-#endif
-
   uint32_t it     = blockIdx.x;
   pair_desc cur_d = a.desc[it];
   pair_desc nxt_d = a.desc[it + stride < n_pairs ? it + stride : it];
@@ -335,7 +322,6 @@ __global__ __launch_bounds__(kBlock, 2) void scan_nibble_kernel(scan_args a)
         }
       }
       lds_barrier();
-      TICK(0);  // waiting for the prefetched query / centre, staging
 
       /* ---- lookup table, entries already in the accumulator's type ---- */
       {
@@ -384,9 +370,7 @@ __global__ __launch_bounds__(kBlock, 2) void scan_nibble_kernel(scan_args a)
           }
         }
       }
-      TICK(1);  // table construction
       lds_barrier();
-      TICK(2);  // barrier after the table
 
       /* ---- scan ---- */
       uint32_t thr           = cur_f.thr;
@@ -462,16 +446,13 @@ __global__ __launch_bounds__(kBlock, 2) void scan_nibble_kernel(scan_args a)
           thr               = t2 < thr ? t2 : thr;
         }
       }
-      TICK(3);  // scan
       lds_barrier();
-      TICK(4);  // barrier after the scan
       const uint32_t before = tail->count;
       lds_barrier();
       block_prune(cand, tail, a.k, before);
       const uint32_t cnt = before < a.k ? before : a.k;
       for (uint32_t r = tid; r < a.k; r += kBlock) { out[r] = r < cnt ? cand[r] : kInvalidKey; }
       if (tid == 0 && before >= a.k) { atomicMin(&a.query_kth[q], tail->thr); }
-      TICK(5);  // prune + output
     }
     if (!has_next) { break; }
     if (n_rows == 0) {
@@ -483,12 +464,6 @@ __global__ __launch_bounds__(kBlock, 2) void scan_nibble_kernel(scan_args a)
     nxt_d = after_d;
     cur_f = nxt_f;
   }
-#ifdef CUVS_SCAN_TIMING
-  if (a.timing != nullptr && (tid & 63u) == 0) {
-    for (int i = 0; i < 6; i++) { atomicAdd(&a.timing[i], tm[i]); }
-  }
-#endif
-#undef TICK
 }
 
 size_t nibble_smem(const scan_args& a, bool out_half)
@@ -504,19 +479,17 @@ void launch_nibble_instance(const scan_args& a, hipStream_t stream)
 {
   auto kernel       = scan_nibble_kernel<OUT_HALF, IP, PQ_LEN>;
   const size_t smem = nibble_smem(a, OUT_HALF);
-  // per instance: the grid for the last table size seen (it changes with pq_dim only)
-  static size_t known_smem = 0;
-  static uint32_t known_grid = 0;
-  if (known_smem != smem) {
+  // per instance: the LDS limit once; the occupancy depends on the table size (pq_dim) and is asked
+  // at every launch (a host-side computation)
+  static const int attr_set = [&] {
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
-    int occ = 0, dev = 0, n_cu = 0;
-    CUVS_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kernel, kBlock, smem));
-    CUVS_HIP_TRY(hipGetDevice(&dev));
-    CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-    known_grid = uint32_t(occ > 0 ? occ : 1) * uint32_t(n_cu);
-    known_smem = smem;
-  }
+    return 1;
+  }();
+  (void)attr_set;
+  int occ = 0;
+  CUVS_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kernel, kBlock, smem));
+  const uint32_t known_grid = uint32_t(occ > 0 ? occ : 1) * uint32_t(device_cu_count());
   uint32_t grid = known_grid;
   if (a.n_pairs_dev == nullptr) {
     if (grid > a.n_pairs) { grid = a.n_pairs; }

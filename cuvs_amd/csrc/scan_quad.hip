@@ -353,16 +353,15 @@ void launch_quad_instance(const scan_args& a, hipStream_t stream)
   const size_t smem = kQuadLdsBase + size_t(G) * NCH * 16 * 256 * sizeof(lut_t) +
                       size_t(G) * NCH * 16 * PQ_LEN * (IP ? 2 : 1) * 4 +
                       size_t(kQuadWaves) * quad_wave_cap(a.k) * 8;
-  static int n_cu = 0;
-  if (n_cu == 0) {
-    // the largest request of any k this kernel serves
+  // per instance: the LDS limit is raised once, to the largest request of any k this kernel serves
+  static const int attr_set = [&] {
     const size_t smem_max = smem + size_t(kQuadWaves) * (quad_wave_cap(kQuadMaxK) - quad_wave_cap(a.k)) * 8;
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(smem_max)));
-    int dev = 0;
-    CUVS_HIP_TRY(hipGetDevice(&dev));
-    CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-  }
+    return 1;
+  }();
+  (void)attr_set;
+  const int n_cu = device_cu_count();
   uint32_t grid = uint32_t(n_cu);
   if (a.n_pairs_dev == nullptr) {
     const uint32_t n_quads = (a.n_pairs + G - 1) / G;

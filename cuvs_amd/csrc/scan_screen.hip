@@ -105,16 +105,11 @@ __device__ __forceinline__ void push_survivor(LDS_AS uint32_t* pending, uint32_t
   }
 }
 
-/** How many leading subspaces the screen sums (of the 16 in the first chunk): 8, or 4 / 16 for A/B runs. */
-inline int screen_subspaces()
-{
-  static const int subs = [] {
-    const char* e = std::getenv("CUVS_AMD_SCREEN_SUBSPACES");
-    const int v   = e != nullptr ? std::atoi(e) : 8;
-    return (v == 4 || v == 8 || v == 16) ? v : 8;
-  }();
-  return subs;
-}
+/** Leading subspaces the table-building screen sums (of the 16 in the first chunk): with 16 the
+ *  same pairs survive on clustered data, with 4 three times as many. */
+constexpr int kScreenSubs = 8;
+/** The table-free screen checks for the first time after this many subspaces, then after 4 and 8. */
+constexpr int kScreenFirstCheck = 2;
 
 template <int SUBS, int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER>
 __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
@@ -511,26 +506,6 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   if (n_pending != 0) { flush_survivors(pending, n_pending, lane, survivors, n_survivors); }
 }
 
-/** Which subspace count the first check of the table-free screen follows (1, 2 or 4). */
-inline int screen_first_check()
-{
-  static const int first = [] {
-    const char* e = std::getenv("CUVS_AMD_SCREEN_FIRST_CHECK");
-    const int v   = e != nullptr ? std::atoi(e) : 2;
-    return (v == 1 || v == 2 || v == 4) ? v : 2;
-  }();
-  return first;
-}
-
-inline bool screen_tables_forced()
-{
-  static const bool forced = [] {
-    const char* e = std::getenv("CUVS_AMD_SCREEN_TABLES");
-    return e != nullptr && e[0] == '1';
-  }();
-  return forced;
-}
-
 template <int PQ_LEN, int LUT, bool OUT_HALF, int FIRST>
 void launch_screen_direct_first(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
                                 pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
@@ -539,16 +514,9 @@ void launch_screen_direct_first(const scan_args& a, const pair_desc* desc, uint3
   auto kernel       = scan_screen_direct_kernel<PQ_LEN, LUT, OUT_HALF, FIRST>;
   const size_t smem = kScreenLdsBase + size_t(kDirectSubs) * 256 * PQ_LEN * 4 +
                       size_t(kDirectThreads / 64u) * kSurvivorBatchBytes;
-  static int n_cu = 0, per_cu = 0;  // per instance
-  if (n_cu == 0) {
-    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
-    int dev = 0;
-    CUVS_HIP_TRY(hipGetDevice(&dev));
-    CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-    CUVS_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kDirectThreads, smem));
-    per_cu = std::max(per_cu, 1);
-  }
+  // persistent blocks: exactly as many as are resident at once (per instance)
+  static const int per_cu = prepare_persistent_kernel(kernel, kDirectThreads, smem, smem);
+  const int n_cu          = device_cu_count();
   constexpr uint32_t wpb = kDirectThreads / 64u;
   uint32_t grid          = uint32_t(n_cu) * uint32_t(per_cu);
   const uint32_t needed  = (n_pairs + wpb - 1u) / wpb;
@@ -563,14 +531,7 @@ template <int PQ_LEN, int LUT, bool OUT_HALF>
 void launch_screen_direct(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
                           pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive, hipStream_t stream)
 {
-  const int first = screen_first_check();
-  if (first == 1) {
-    launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, 1>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
-  } else if (first == 2) {
-    launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, 2>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
-  } else {
-    launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, 4>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
-  }
+  launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, kScreenFirstCheck>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
 }
 
 template <int SUBS, int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER>
@@ -582,17 +543,9 @@ void launch_screen_sub(const scan_args& a, const pair_desc* desc, uint32_t n_pai
   auto kernel       = scan_screen_kernel<SUBS, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>;
   const size_t smem = kScreenLdsBase + size_t(kScreenG) * SUBS * 256 * sizeof(lut_t) +
                       size_t(kScreenG) * SUBS * PQ_LEN * 4 + size_t(kScreenG) * kSurvivorBatchBytes;
-  static int n_cu = 0, per_cu = 0;  // per instance
-  if (n_cu == 0) {
-    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
-    int dev = 0;
-    CUVS_HIP_TRY(hipGetDevice(&dev));
-    CUVS_HIP_TRY(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-    // persistent blocks: exactly as many as are resident at once
-    CUVS_HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, kScreenThreads, smem));
-    per_cu = std::max(per_cu, 1);
-  }
+  // persistent blocks: exactly as many as are resident at once (per instance)
+  static const int per_cu = prepare_persistent_kernel(kernel, kScreenThreads, smem, smem);
+  const int n_cu          = device_cu_count();
   const uint32_t n_iters = (n_pairs + kScreenG - 1) / kScreenG;
   uint32_t grid          = uint32_t(n_cu) * uint32_t(per_cu);
   if (grid > n_iters) { grid = n_iters; }
@@ -609,19 +562,12 @@ void launch_screen_instance(const scan_args& a, const pair_desc* desc, uint32_t 
                             hipStream_t stream)
 {
   if constexpr (!PER_CLUSTER) {
-    if (!screen_tables_forced() && a.lead_plane != nullptr) {
+    if (a.lead_plane != nullptr) {
       launch_screen_direct<PQ_LEN, LUT, OUT_HALF>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
       return;
     }
   }
-  const int subs = screen_subspaces();
-  if (subs == 4) {
-    launch_screen_sub<4, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
-  } else if (subs == 8) {
-    launch_screen_sub<8, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
-  } else {
-    launch_screen_sub<16, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
-  }
+  launch_screen_sub<kScreenSubs, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
 }
 
 template <int PQ_LEN, bool PER_CLUSTER>
@@ -649,8 +595,9 @@ void launch_screen_types(const scan_args& a, const pair_desc* desc, uint32_t n_p
 
 uint32_t scan_screen_bytes_per_row(bool per_cluster, bool lead_plane)
 {
-  if (!per_cluster && lead_plane && !screen_tables_forced()) { return 8u; }
-  return screen_subspaces() <= 8 ? 8u : 16u;
+  (void)per_cluster;
+  (void)lead_plane;
+  return kScreenSubs <= 8 ? 8u : 16u;
 }
 
 bool scan_screen_supported(const scan_args& a)

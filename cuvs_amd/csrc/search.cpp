@@ -5,6 +5,7 @@
  * plan are this library's own (results do not depend on how queries are batched).
  */
 #include "detail.hpp"
+#include "tracing.hpp"
 
 #include <algorithm>
 #include <cstdlib>
@@ -140,76 +141,16 @@ void validate(const search_params& params, const index_impl& ix, int64_t k)
                "Unexpected lut_dtype / internal_distance_dtype combination (%d, %d). Size of the "
                "internal_distance_dtype should be not smaller than the size of the lut_dtype.",
                int(params.lut_dtype), int(params.internal_distance_dtype));
-  CUVS_EXPECTS(params.coarse_search_dtype == CUDA_R_32F || params.coarse_search_dtype == CUDA_R_16F,
-               "Unsupported coarse_search_dtype (only CUDA_R_32F and CUDA_R_16F are supported)");
+  CUVS_EXPECTS(params.coarse_search_dtype == CUDA_R_32F || params.coarse_search_dtype == CUDA_R_16F ||
+                 params.coarse_search_dtype == CUDA_R_8I,
+               "Unsupported coarse_search_dtype (only CUDA_R_32F, CUDA_R_16F, and CUDA_R_8I are supported)");
   CUVS_EXPECTS(k <= kMaxK, "parameter `k` (%lld) must not exceed %u", static_cast<long long>(k),
                kMaxK);
 }
 
-/** CUVS_AMD_NO_EARLY_STOP=1 scans every probed list in full (for A/B runs; read at every search). */
-bool early_stop_disabled()
-{
-  const char* e = std::getenv("CUVS_AMD_NO_EARLY_STOP");
-  return e != nullptr && e[0] == '1';
-}
-
-/** CUVS_AMD_PAIR_ORDER=label: the leading (query, list) pairs are grouped in the order of the list
- *  numbers instead of from long lists to short ones (for measurements; the results are the same). */
-bool pair_order_by_label()
-{
-  const char* e = std::getenv("CUVS_AMD_PAIR_ORDER");
-  return e != nullptr && std::string(e) == "label";
-}
-
 /** Probes per query whose lists are scanned in full before the others are screened against the
- *  bound they give. */
-uint32_t lead_probes()
-{
-  const char* e = std::getenv("CUVS_AMD_LEAD_PROBES");  // for A/B runs
-  const int v   = e != nullptr ? std::atoi(e) : 1;
-  return v >= 1 && v <= 16 ? uint32_t(v) : 1u;
-}
-
-/** CUVS_AMD_GENERIC_SCAN=1 routes every search through the generic scan kernel (for A/B runs). */
-bool force_generic_scan()
-{
-  static const bool v = [] {
-    const char* e = std::getenv("CUVS_AMD_GENERIC_SCAN");
-    return e != nullptr && e[0] == '1';
-  }();
-  return v;
-}
-
-/** Instrumented builds (-DCUVS_SCAN_TIMING) accumulate per-phase cycle counts of the scan kernel
- *  here and print them when the library unloads. */
-unsigned long long* scan_timing_buffer()
-{
-#ifdef CUVS_SCAN_TIMING
-  struct holder {
-    unsigned long long* d = nullptr;
-    holder()
-    {
-      (void)hipMalloc(reinterpret_cast<void**>(&d), 64);
-      (void)hipMemset(d, 0, 64);
-    }
-    ~holder()
-    {
-      unsigned long long h[6] = {};
-      (void)hipMemcpy(h, d, 48, hipMemcpyDeviceToHost);
-      const char* names[6] = {"phase0", "phase1", "phase2", "phase3", "phase4", "phase5"};
-      unsigned long long total = 0;
-      for (auto v : h) { total += v; }
-      for (int i = 0; i < 6; i++) {
-        fprintf(stderr, "[scan timing] %-10s %6.2f%%\n", names[i], 100.0 * double(h[i]) / double(total ? total : 1));
-      }
-    }
-  };
-  static holder h;
-  return h.d;
-#else
-  return nullptr;
-#endif
-}
+ *  bound they give (2 to 16 measured no better on clustered data). */
+constexpr uint32_t kLeadProbes = 1;
 
 float scaling_factor(elem_type t)
 {
@@ -234,24 +175,14 @@ struct coarse_buffers {
   uint8_t* fallback = nullptr;
 };
 
-bool coarse_plain_forced()
-{
-  static const bool forced = [] {
-    const char* e = std::getenv("CUVS_AMD_COARSE_PLAIN");
-    return e != nullptr && e[0] == '1';
-  }();
-  return forced;
-}
-
 /** The two-precision probe selection applies to fp32 coarse search and to shapes where its
  *  candidate lists stay short: about 1.4 n_probes lists per query pass the threshold, and a
  *  workgroup of the candidate pass (512 lists) holds at most 32 of them per query before the query
  *  falls back to the plain path, so n_lists >= 64 n_probes keeps the expected load near 11. */
-bool coarse_fast_applies(const search_params& params, const index_impl& ix, elem_type type,
-                         uint32_t n_probes)
+bool coarse_fast_applies(const cuvs::resources& res, const search_params& params,
+                         const index_impl& ix, uint32_t n_probes)
 {
-  (void)type;
-  return !coarse_plain_forced() && ix.coarse_fast_ok &&
+  return !res.tuning.plain_coarse && ix.coarse_fast_ok &&
          params.coarse_search_dtype == CUDA_R_32F && n_probes <= detail::coarse_fast_cand_cap() / 2 &&
          ix.n_lists >= 1024 && ix.n_lists >= 64u * n_probes && ix.dim <= 128;
 }
@@ -282,6 +213,8 @@ void run_coarse(const cuvs::resources& res, const search_params& params, const i
                 const void* queries, elem_type type, uint32_t nq, uint32_t n_probes,
                 const coarse_buffers& b)
 {
+  cuvs::tracing::range scope("ivf_pq::search::select_clusters(n_probes = %u, n_queries = %u, n_lists = %u, dim = %u)",
+                             n_probes, nq, ix.n_lists, ix.dim);
   hipStream_t s     = res.stream();
   const bool ip     = ix.metric == detail::DistanceType::InnerProduct ||
                   ix.metric == detail::DistanceType::CosineExpanded;
@@ -313,6 +246,13 @@ void run_coarse(const cuvs::resources& res, const search_params& params, const i
     detail::launch_coarse_fast(a, s);
     return;
   }
+  if (params.coarse_search_dtype == CUDA_R_8I) {
+    // ivf_pq_search.cuh:170-256
+    detail::launch_coarse_scores_i8(b.qf, ix.centers_i8.as<uint32_t>(), nq, ix.n_lists, ix.dim, ip,
+                                    b.scores, s);
+    detail::launch_select_probes(b.scores, nq, ix.n_lists, n_probes, b.probes, s);
+    return;
+  }
   detail::launch_map_queries_t(queries, type, nq, ix.dim, ix.dim_ext, ip, b.qt, s);
   detail::launch_coarse_scores_mfma(b.qt, ix.centers_t.as<float>(), nq, ix.n_lists, ix.dim_ext, ip,
                                     params.coarse_search_dtype == CUDA_R_16F, b.scores, s);
@@ -333,8 +273,9 @@ void select_clusters(cuvs::resources const& res_c,
   const auto& ix = *idx.impl();
   CUVS_EXPECTS(params.n_probes > 0,
                "n_probes (number of clusters to probe in the search) must be positive.");
-  CUVS_EXPECTS(params.coarse_search_dtype == CUDA_R_32F || params.coarse_search_dtype == CUDA_R_16F,
-               "Unsupported coarse_search_dtype (only CUDA_R_32F and CUDA_R_16F are supported)");
+  CUVS_EXPECTS(params.coarse_search_dtype == CUDA_R_32F || params.coarse_search_dtype == CUDA_R_16F ||
+                 params.coarse_search_dtype == CUDA_R_8I,
+               "Unsupported coarse_search_dtype (only CUDA_R_32F, CUDA_R_16F, and CUDA_R_8I are supported)");
   CUVS_EXPECTS(device_accessible(queries) && device_accessible(clusters_to_probe),
                "all pointers must be accessible from the device.");
   const uint32_t P       = std::min<uint32_t>(params.n_probes, ix.n_lists);
@@ -344,7 +285,7 @@ void select_clusters(cuvs::resources const& res_c,
   batch                  = std::min<size_t>(batch, 65535u * 64u);
   res.reset_workspace();
   const size_t qt_bytes = size_t(ix.dim_ext) * detail::coarse_pad(uint32_t(batch)) * 4;
-  const bool fast       = coarse_fast_applies(params, ix, type, P);
+  const bool fast       = coarse_fast_applies(res, params, ix, P);
   res.reserve_workspace(a256(batch * ix.dim * 4) + a256(qt_bytes) +
                         a256(batch * size_t(ix.n_lists) * 4 + detail::kSelectSlackBytes) + 1024 +
                         (fast ? coarse_fast_bytes(ix, batch) : 0));
@@ -401,6 +342,8 @@ void search(cuvs::resources const& res_c,
                "all pointers must be accessible from the device.");
 
   const uint32_t k  = uint32_t(k64);
+  cuvs::tracing::range search_scope("ivf_pq::search(n_queries = %u, n_probes = %u, k = %u, dim = %u)",
+                                    uint32_t(n_queries), params.n_probes, k, ix.dim);
   const plan pl     = make_plan(res, params, ix, uint32_t(n_queries), k);
   const uint32_t P  = pl.n_probes;
   const uint32_t Qb = pl.batch;
@@ -440,7 +383,7 @@ void search(cuvs::resources const& res_c,
 
   /* workspace carve-up for one batch */
   res.reset_workspace();
-  const bool fast_coarse = coarse_fast_applies(params, ix, type, P);
+  const bool fast_coarse = coarse_fast_applies(res, params, ix, P);
   const size_t workspace_bytes = pl.fixed_bytes + size_t(Qb) * (pl.per_query_bytes + 64) + 16 * 256 +
                                  global_lut_bytes + (fast_coarse ? coarse_fast_bytes(ix, Qb) : 0);
   CUVS_EXPECTS(!res.workspace_borrowed() || workspace_bytes <= res.workspace_capacity(),
@@ -468,7 +411,7 @@ void search(cuvs::resources const& res_c,
   float* all_scores        = nullptr;
   sa.fused                 = pl.fused;
   if (global_lut) { sa.global_lut = res.workspace_alloc(global_lut_bytes); }
-  const bool generic_only  = force_generic_scan() || global_lut;
+  const bool generic_only  = res.tuning.generic_scan || global_lut;
   const uint32_t quad_kpp  = generic_only ? 0u : detail::scan_quad_keys_per_pair(sa);
   const bool nibble_scan   = !generic_only && detail::scan_nibble_supported(sa);
   const bool fast_scan     = !generic_only && (quad_kpp != 0 || detail::scan_fast_supported(sa) || nibble_scan);
@@ -482,9 +425,8 @@ void search(cuvs::resources const& res_c,
   // they save (the reference skips the grouping when lists are rarely shared,
   // expected_probe_coresidency, ivf_pq_search.cuh:353-373).
   const bool few_pairs       = uint64_t(Qb) * P <= kFewPairs;
-  const uint32_t kLeadProbes = lead_probes();
   const bool early_stop = fast_scan && !few_pairs && P > kLeadProbes && P <= 8192 &&
-                          detail::scan_screen_supported(sa) && !early_stop_disabled();
+                          detail::scan_screen_supported(sa) && res.tuning.early_stop != 1;
   const uint32_t lead          = early_stop ? kLeadProbes : P;
   detail::pair_desc* survivors = nullptr;
   uint8_t* alive               = nullptr;
@@ -521,17 +463,20 @@ void search(cuvs::resources const& res_c,
   };
 
   const bool cosine = ix.metric == detail::DistanceType::CosineExpanded;
-  // the leading pairs run from long lists to short ones (CUVS_AMD_PAIR_ORDER=label: by list number)
-  const uint32_t* list_rank = pair_order_by_label() ? nullptr : ix.list_rank.as<uint32_t>();
+  // the leading pairs run from long lists to short ones
+  const uint32_t* list_rank = ix.list_rank.as<uint32_t>();
   for (int64_t q0 = 0; q0 < n_queries; q0 += Qb) {
     const uint32_t nq = uint32_t(std::min<int64_t>(Qb, n_queries - q0));
     const void* qptr  = static_cast<const char*>(queries) + size_t(q0) * ix.dim * elem_size(type);
 
+    cuvs::tracing::range batch_scope("ivf_pq::search-batch(queries: %u - %u)", uint32_t(q0), uint32_t(q0) + nq);
     mark(0);
     run_coarse(res, params, ix, qptr, type, nq, P, cb);
     mark(1);
+    cuvs::tracing::range worker_scope("ivf_pq::search-worker(n_queries = %u, n_probes = %u, k = %u, dim = %u)", nq, P,
+                                      k, ix.dim);
     detail::launch_rotate(qf, ix.rotation_t.as<float>(), nq, ix.dim, ix.rot_dim,
-                          ix.rotation_is_identity, cosine, rot_q, s);
+                          ix.rotation_is_identity, cosine, params.coarse_search_dtype, rot_q, s);
     detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
                                  ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead,
                                  few_pairs ? nullptr : counters, ix.n_lists, list_rank, s);
@@ -541,6 +486,8 @@ void search(cuvs::resources const& res_c,
     if (pl.fused) { detail::launch_fill_u32(kth, 0xFFFFFFFFu, nq, s); }
     mark(2);
 
+    {
+    cuvs::tracing::range scan_scope("ivf_pq::search-worker::scan");
     sa.n_queries     = nq;
     sa.rot_q         = rot_q;
     sa.probes        = probes;
@@ -552,7 +499,6 @@ void search(cuvs::resources const& res_c,
     sa.desc        = desc;
     sa.n_pairs     = nq * P;
     sa.n_pairs_dev = nullptr;
-    sa.timing      = scan_timing_buffer();
     if (early_stop) {
       // 1. the leading probes' lists in full: candidates and a first bound per query
       auto full_scan = [&] {
@@ -578,8 +524,10 @@ void search(cuvs::resources const& res_c,
                                                         : detail::launch_scan_fast(sa, s));
       if (!launched) { detail::launch_scan(sa, s); }
     }
+    }
     mark(3);
 
+    cuvs::tracing::range merge_scope("ivf_pq::search-worker::merge");
     detail::merge_args ma{};
     ma.n_queries     = nq;
     ma.n_probes      = P;

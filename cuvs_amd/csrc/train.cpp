@@ -246,7 +246,7 @@ index<int64_t> build(cuvs::resources const& res_c,
   CUVS_HIP_TRY(hipMemcpyAsync(d_rot_t.ptr, rot_t.data(), d_rot_t.bytes, hipMemcpyHostToDevice, s));
   device_buffer centers_rot(size_t(L) * cx.rot_dim * sizeof(float));
   detail::launch_rotate(flat.as<float>(), d_rot_t.as<float>(), L, dim, cx.rot_dim, identity, false,
-                        centers_rot.as<float>(), s);
+                        CUDA_R_32F, centers_rot.as<float>(), s);
 
   /* 4. codebooks on the rotated residuals of the training rows */
   const bool per_cluster = cx.codebook_kind == codebook_gen::PER_CLUSTER;
@@ -261,7 +261,7 @@ index<int64_t> build(cuvs::resources const& res_c,
   for (uint64_t r0 = 0; r0 < n_pq; r0 += (1u << 20)) {
     const uint32_t n = uint32_t(std::min<uint64_t>(1u << 20, n_pq - r0));
     detail::launch_rotate(diff.as<float>() + r0 * dim, d_rot_t.as<float>(), n, dim, cx.rot_dim, identity,
-                          false, resid.as<float>() + r0 * cx.rot_dim, s);
+                          false, CUDA_R_32F, resid.as<float>() + r0 * cx.rot_dim, s);
   }
   const uint32_t n_groups = per_cluster ? L : cx.pq_dim;
   device_buffer pq_centers(size_t(n_groups) * cx.pq_len * book * sizeof(float));

@@ -1,7 +1,7 @@
 """Mirror of cuvs.common.Resources (python/cuvs/cuvs/common/resources.pyx): owns a cuvsResources_t."""
 import ctypes as C
 
-from ._lib import check, lib
+from ._lib import SearchTuningStruct, check, lib
 
 
 class Resources:
@@ -37,6 +37,15 @@ class Resources:
 
     def get_c_obj(self):
         return self._h
+
+    def set_search_tuning(self, early_stop="auto", generic_scan=False, plain_coarse=False):
+        """cuvsAmdIvfPqSetSearchTuning: fix choices the search otherwise makes by itself (results do
+        not depend on them).  early_stop: "auto", "off" (every probed list streamed in full) or "on"."""
+        t = SearchTuningStruct()
+        t.early_stop = {"auto": 0, "off": 1, "on": 2}[early_stop]
+        t.generic_scan = int(bool(generic_scan))
+        t.plain_coarse = int(bool(plain_coarse))
+        check(lib().cuvsAmdIvfPqSetSearchTuning(self._h, C.byref(t)))
 
     def enable_profiling(self, on=True):
         check(lib().cuvsAmdIvfPqProfilingEnable(self._h, bool(on)))

@@ -85,6 +85,19 @@ struct search_profile {
   uint64_t n_surviving_pairs = 0;
 };
 
+/** Choices the search otherwise makes by itself, for measurements and tests that compare the
+ *  library's code paths with each other.  None of them changes a result. */
+struct search_tuning {
+  /** L2 early stop (leading lists in full, the others screened, survivors in full):
+   *  0 = the library decides per batch, 1 = never: every probed list is scanned in full,
+   *  2 = whenever the kernels support the search's parameters. */
+  int early_stop = 0;
+  /** Every search goes through the generic scan kernel. */
+  bool generic_scan = false;
+  /** Coarse search by the fp32 contraction and selection instead of the two-precision selection. */
+  bool plain_coarse = false;
+};
+
 /**
  * One stream plus a cached device workspace (role of raft::resources with a workspace memory
  * resource).  Not thread-safe: use one handle per host thread; an index may be shared.
@@ -97,7 +110,13 @@ class resources {
   resources& operator=(const resources&) = delete;
 
   hipStream_t stream() const { return stream_; }
-  void set_stream(hipStream_t s) { stream_ = s; }
+  /**
+   * Work the library queues from now on goes to `s`.  The cached workspace is shared by
+   * consecutive calls: when the stream changes while work queued on the previous one may still use
+   * it, the new stream is made to wait for that work first (an event recorded on the previous
+   * stream), so calls on the same handle stay ordered across the switch.
+   */
+  void set_stream(hipStream_t s);
   void sync() const;
   int device_id() const { return device_; }
 
@@ -134,6 +153,7 @@ class resources {
   void borrow_workspace(void* ptr, size_t bytes);
   bool workspace_borrowed() const { return workspace_borrowed_; }
 
+  search_tuning tuning;
   bool profiling = false;
   struct profile_state;
   profile_state* prof = nullptr;  // lazily created event set
@@ -146,7 +166,12 @@ class resources {
   size_t workspace_capacity_ = 0;
   size_t workspace_used_  = 0;
   size_t workspace_limit_ = 0;
-  std::vector<void*> retired_;  // outgrown workspaces, released at destruction / next sync point
+  // workspaces outgrown after a call was captured into a HIP graph while they were current: the
+  // graph keeps their addresses, so they stay allocated until the handle goes
+  std::vector<void*> retired_;
+  std::vector<bool> retired_pooled_;
+  bool workspace_captured_ = false;  // a call ran under stream capture on the current workspace
+  hipEvent_t order_event_  = nullptr;  // set_stream: orders the new stream after the previous one
   std::shared_ptr<memory::pool> pool_;  // set_workspace_pool
   bool workspace_pooled_ = false;       // workspace_ came out of pool_
   bool workspace_borrowed_ = false;     // workspace_ belongs to the caller of borrow_workspace

@@ -265,6 +265,22 @@ typedef struct {
   uint64_t n_surviving_pairs;
 } cuvsAmdIvfPqSearchProfile;
 
+/** Choices the search otherwise makes by itself, fixed on one resources handle: for measurements
+ *  and tests that compare the library's code paths (no result depends on them).
+ *  early_stop: 0 = the library decides per batch whether the L2 early stop (leading lists in full,
+ *  the others screened on their leading codes, survivors in full) pays; 1 = never, every probed
+ *  list is streamed in full by the scan kernel; 2 = whenever the search's parameters allow it.
+ *  generic_scan != 0: every search goes through the generic scan kernel.  plain_coarse != 0: coarse
+ *  search by the fp32 contraction and selection instead of the two-precision selection. */
+typedef struct {
+  int32_t early_stop;
+  int32_t generic_scan;
+  int32_t plain_coarse;
+  int32_t reserved_[5]; /* zero */
+} cuvsAmdIvfPqSearchTuning;
+CUVS_EXPORT cuvsError_t cuvsAmdIvfPqSetSearchTuning(cuvsResources_t res,
+                                                    const cuvsAmdIvfPqSearchTuning* tuning);
+
 /** Turn event timing of the search stages on or off (off by default: timing adds event records and
  *  one device reduction per search). */
 CUVS_EXPORT cuvsError_t cuvsAmdIvfPqProfilingEnable(cuvsResources_t res, bool enable);

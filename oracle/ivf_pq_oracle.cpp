@@ -262,6 +262,70 @@ void coarse_scores_f16(const orc_index& ix, const float* qf, float* scores)
   }
 }
 
+/* 8-bit integer variant (ivf_pq_search.cuh:170-256; centres quantised as in
+ * cpp/src/neighbors/ivf_pq_index.cu:661-738).  Rows have dim_ext_int8 = round_up(dim + 2, 16)
+ * columns.  Centre side: column c < dim is trunc(clamp(128 c)); the squared norm x is split as
+ * y = clamp(x * 64 / (m - 1)), m = dim_ext_int8 - dim: every column past `dim` holds round(y) and
+ * column `dim` holds trunc(clamp(128 (y - round(y)))).  Query side: mapping<int8_t> of the element
+ * (trunc(clamp(128 q)) for float types, x >> 1 for uint8, x for int8), column `dim` holds 1 - m,
+ * the columns past it -128 (L2) or 0 (inner product, cosine).  Scores are int32: alpha times the
+ * dot product, alpha = -2 (L2) or -1.
+ *
+ * The reference lays the query rows out with dim_ext = round_up(dim + 1, 8) columns and hands the
+ * centre matrix (dim_ext_int8 columns a row) to the GEMM with that same leading dimension, so
+ * whenever the two paddings differ its GEMM reads the centre rows at the wrong stride; its own
+ * test asks a recall of 0.1 of this variant (cpp/tests/neighbors/ann_ivf_pq.cuh:1040-1046).  This
+ * restatement uses the centre matrix's padding on both sides, which is what the comment in
+ * ivf_pq_index.cu describes and equals the reference's arithmetic where the paddings agree
+ * (dim % 16 in 7..14).  Parity unpinned for the other dims. */
+inline uint32_t dim_ext_int8_of(uint32_t dim) { return round_up(dim + 2, 16); }
+
+inline int8_t clamp_to_int8(float v)
+{
+  // static_cast<int8_t>(fmaxf(-128, fminf(127, v))): truncation toward zero
+  return int8_t(std::fmax(-128.0f, std::fmin(127.0f, v)));
+}
+
+void center_row_int8(const orc_index& ix, uint32_t l, int8_t* out)
+{
+  const uint32_t de  = dim_ext_of(ix.dim);
+  const uint32_t de8 = dim_ext_int8_of(ix.dim);
+  const float* c     = ix.centers + uint64_t(l) * de;
+  for (uint32_t d = 0; d < ix.dim; d++) { out[d] = clamp_to_int8(c[d] * 128.0f); }
+  const float x = c[ix.dim];
+  const float f = 64.0f / float(de8 - ix.dim - 1);
+  const float y = std::fmax(-128.0f, std::fmin(127.0f, x * f));
+  const float z = std::fmax(-128.0f, std::fmin(127.0f, (y - std::round(y)) * 128.0f));
+  out[ix.dim]   = int8_t(z);
+  for (uint32_t d = ix.dim + 1; d < de8; d++) { out[d] = int8_t(std::round(y)); }
+}
+
+void query_row_int8(const orc_index& ix, const float* qf, int8_t* out)
+{
+  const uint32_t de8 = dim_ext_int8_of(ix.dim);
+  const int m        = int(de8 - ix.dim);
+  const int8_t nf    = is_ip_like(ix.metric) ? int8_t(0) : int8_t(-128);
+  // qf = mapping<float>(element): x / 256 (uint8), x / 128 (int8): 128 qf gives x / 2 and x, and
+  // truncation gives mapping<int8_t>'s x >> 1 and x
+  for (uint32_t d = 0; d < ix.dim; d++) { out[d] = clamp_to_int8(qf[d] * 128.0f); }
+  out[ix.dim] = int8_t(1 - m);
+  for (uint32_t d = ix.dim + 1; d < de8; d++) { out[d] = nf; }
+}
+
+void coarse_scores_i8(const orc_index& ix, const float* qf, int32_t* scores)
+{
+  const uint32_t de8  = dim_ext_int8_of(ix.dim);
+  const int32_t alpha = is_ip_like(ix.metric) ? -1 : -2;
+  std::vector<int8_t> q8(de8), c8(de8);
+  query_row_int8(ix, qf, q8.data());
+  for (uint32_t l = 0; l < ix.n_lists; l++) {
+    center_row_int8(ix, l, c8.data());
+    int32_t acc = 0;
+    for (uint32_t d = 0; d < de8; d++) { acc += int32_t(c8[d]) * int32_t(q8[d]); }
+    scores[l] = alpha * acc;
+  }
+}
+
 /* total order used by every selection in this file: smaller score first, then smaller index.
  * -0.0 and +0.0 compare equal, as they do on the device. */
 struct cand {
@@ -291,6 +355,18 @@ void select_clusters_one(const orc_index& ix, const orc_search_params& sp, const
                          uint32_t n_probes, std::vector<float>& scores, std::vector<cand>& tmp,
                          uint32_t* probes, float* probe_scores)
 {
+  if (sp.coarse_search_dtype == ORC_R_8I) {
+    std::vector<int32_t> si(ix.n_lists);
+    coarse_scores_i8(ix, qf, si.data());
+    std::vector<std::pair<int32_t, uint32_t>> order(ix.n_lists);
+    for (uint32_t l = 0; l < ix.n_lists; l++) { order[l] = {si[l], l}; }
+    std::partial_sort(order.begin(), order.begin() + n_probes, order.end());
+    for (uint32_t p = 0; p < n_probes; p++) {
+      probes[p] = order[p].second;
+      if (probe_scores) { probe_scores[p] = float(order[p].first); }
+    }
+    return;
+  }
   scores.resize(ix.n_lists);
   if (sp.coarse_search_dtype == ORC_R_16F) {
     coarse_scores_f16(ix, qf, scores.data());
@@ -308,13 +384,31 @@ void select_clusters_one(const orc_index& ix, const orc_search_params& sp, const
 
 /* ---------------- query rotation (ivf_pq_search.cuh:996-1025) ---------------- */
 
-void rotate_query(const orc_index& ix, const float* qf, float* rq)
+/* The rotation GEMM takes the query rows the coarse search made and the rotation matrix in the
+ * same type (get_rotation_matrix<value_type>, ivf_pq_search.cuh:996-1019): fp32; binary16 copies of
+ * both (products accumulated in fp32 here, result fp32); or int8 copies (mapping<int8_t>: 128 x
+ * clamped and truncated) with the integer dot product scaled by 1 / 128^2. */
+void rotate_query(const orc_index& ix, int coarse_dtype, const float* qf, float* rq)
 {
   const uint32_t rot_dim = pq_len_of(ix.dim, ix.pq_dim) * ix.pq_dim;
   for (uint32_t r = 0; r < rot_dim; r++) {
     const float* row = ix.rotation_matrix + uint64_t(r) * ix.dim;
-    float acc        = 0.0f;
-    for (uint32_t d = 0; d < ix.dim; d++) { acc = std::fmaf(row[d], qf[d], acc); }
+    if (coarse_dtype == ORC_R_8I) {
+      int32_t acc = 0;
+      for (uint32_t d = 0; d < ix.dim; d++) {
+        acc += int32_t(clamp_to_int8(row[d] * 128.0f)) * int32_t(clamp_to_int8(qf[d] * 128.0f));
+      }
+      rq[r] = float(acc) * (1.0f / 128.0f / 128.0f);
+      continue;
+    }
+    float acc = 0.0f;
+    if (coarse_dtype == ORC_R_16F) {
+      for (uint32_t d = 0; d < ix.dim; d++) {
+        acc = std::fmaf(half_to_float(float_to_half(row[d])), half_to_float(float_to_half(qf[d])), acc);
+      }
+    } else {
+      for (uint32_t d = 0; d < ix.dim; d++) { acc = std::fmaf(row[d], qf[d], acc); }
+    }
     rq[r] = acc;
   }
   if (ix.metric == ORC_CosineExpanded) {
@@ -476,7 +570,8 @@ bool validate(const orc_index& ix, const orc_search_params& sp, uint32_t k, bool
     g_error = "Unexpected lut_dtype / internal_distance_dtype combination";
     return false;
   }
-  if (sp.coarse_search_dtype != ORC_R_32F && sp.coarse_search_dtype != ORC_R_16F) {
+  if (sp.coarse_search_dtype != ORC_R_32F && sp.coarse_search_dtype != ORC_R_16F &&
+      sp.coarse_search_dtype != ORC_R_8I) {
     g_error = "Unsupported coarse_search_dtype in the oracle";
     return false;
   }
@@ -674,7 +769,7 @@ int orc_make_lut(const orc_index* index, const orc_search_params* params, const 
   const uint32_t rot  = orc_rot_dim(ix.dim, ix.pq_dim);
   std::vector<float> qf(ix.dim), rq(rot), raw(uint64_t(ix.pq_dim) << ix.pq_bits);
   map_query(ix, query, query_type, 0, qf.data());
-  rotate_query(ix, qf.data(), rq.data());
+  rotate_query(ix, params->coarse_search_dtype, qf.data(), rq.data());
   make_lut_f32(ix, rq.data(), label, raw.data());
   const lut_kind kind = lut_kind_of(ix, *params);
   for (size_t i = 0; i < raw.size(); i++) {
@@ -724,7 +819,7 @@ int orc_search(const orc_index* index, const orc_search_params* params, const vo
     map_query(ix, queries, query_type, q, w.qf.data());
     select_clusters_one(ix, *params, w.qf.data(), P, w.scores, w.tmp, w.probes.data(), nullptr);
     if (probes_out) { std::memcpy(probes_out + q * P, w.probes.data(), P * sizeof(uint32_t)); }
-    rotate_query(ix, w.qf.data(), w.rq.data());
+    rotate_query(ix, params->coarse_search_dtype, w.qf.data(), w.rq.data());
 
     // calc_chunk_indices (ivf_common.cu:21-50): inclusive prefix sums of probed list sizes
     uint32_t total = 0;

@@ -49,7 +49,7 @@ typedef struct {
   uint32_t n_probes;
   int32_t lut_dtype;               /* ORC_R_32F | ORC_R_16F | ORC_R_8U */
   int32_t internal_distance_dtype; /* ORC_R_32F | ORC_R_16F */
-  int32_t coarse_search_dtype;     /* ORC_R_32F | ORC_R_16F */
+  int32_t coarse_search_dtype;     /* ORC_R_32F | ORC_R_16F | ORC_R_8I */
 } orc_search_params;
 
 /* derived dimensions (cpp/src/neighbors/ivf_pq_index.cu:78-111) */

@@ -236,11 +236,11 @@ def select_clusters(index, queries, n_probes, coarse_search_dtype=R_32F, n_threa
     return probes, scores
 
 
-def make_lut(index, query, label, lut_dtype=R_32F):
+def make_lut(index, query, label, lut_dtype=R_32F, coarse_search_dtype=R_32F):
     q, t = _rows(np.asarray(query).reshape(1, -1))
     n = index.pq_dim << index.pq_bits
     out = np.empty(n, dtype={R_32F: np.float32, R_16F: np.uint16, R_8U: np.uint8}[lut_dtype])
-    p = _params(1, lut_dtype, R_32F, R_32F)
+    p = _params(1, lut_dtype, R_32F, coarse_search_dtype)
     _check(lib().orc_make_lut(index.c_ptr(), C.addressof(p), _ptr(q), t, int(label), _ptr(out)))
     return out.reshape(index.pq_dim, 1 << index.pq_bits)
 

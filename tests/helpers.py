@@ -2,7 +2,7 @@
 import numpy as np
 import torch
 
-from cuvs_amd import testing
+import datasets as testing
 
 METRIC_CODES = {"sqeuclidean": 0, "euclidean": 1, "cosine": 2, "inner_product": 6}
 KIND_CODES = {"subspace": 0, "cluster": 1}

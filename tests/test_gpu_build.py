@@ -14,7 +14,8 @@ import torch
 
 import gpu_helpers as G
 import helpers as H
-from cuvs_amd import ivf_pq, testing
+import datasets as testing
+from cuvs_amd import ivf_pq
 
 pytestmark = pytest.mark.gpu
 

@@ -6,7 +6,9 @@ import numpy as np
 import pytest
 import torch
 
-from cuvs_amd import ivf_pq, testing
+import datasets as testing
+
+from cuvs_amd import ivf_pq
 from cuvs_amd.resources import Resources
 
 pytestmark = pytest.mark.gpu

@@ -8,7 +8,8 @@ import torch
 
 import gpu_helpers as G
 import helpers as H
-from cuvs_amd import ivf_pq, resources, testing
+import datasets as testing
+from cuvs_amd import ivf_pq, resources
 from cuvs_amd.resources import Resources
 
 pytestmark = pytest.mark.gpu

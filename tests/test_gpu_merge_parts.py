@@ -7,7 +7,8 @@ import pytest
 import torch
 
 import gpu_helpers as G
-from cuvs_amd import ivf_pq, knn_merge_parts, testing
+import datasets as testing
+from cuvs_amd import ivf_pq, knn_merge_parts
 
 pytestmark = pytest.mark.gpu
 

@@ -17,7 +17,7 @@ from cuvs_amd._lib import CuvsError
 pytestmark = pytest.mark.gpu
 
 R_32F, R_16F, R_8U = np.float32, np.float16, np.uint8
-ORC_DT = {np.float32: 0, np.float16: 2, np.uint8: 8}
+ORC_DT = {np.float32: 0, np.float16: 2, np.int8: 3, np.uint8: 8}
 
 
 def _case(orc, n, dim, n_lists, pq_dim, pq_bits, dtype=np.float32, metric="sqeuclidean",
@@ -48,7 +48,7 @@ def _search_both(orc, index, ix, queries, k, n_probes, lut=R_32F, internal=R_32F
 def test_config1_tiny_l2_fp32(orc):
     """BASELINE configs[0]: 10,000 x 128 fp32 from a 64-component mixture, 64 lists, pq_dim 32,
     8-bit, 100 queries, k = 10, 8 probes, fp32 table and distances."""
-    from cuvs_amd import testing
+    import datasets as testing
     x = testing.gaussian_mixture(10000, 128, 64, 0.3, seed=1234).numpy()
     q = testing.gaussian_mixture(10100, 128, 64, 0.3, seed=1234).numpy()[10000:]
     model = H.train(x, 64, 32, 8, iters=10)
@@ -208,6 +208,55 @@ def test_half_precision_coarse_search(orc):
     H.compare_results(nb, d, want_nb, want_d, 1e-5, exact=True)
 
 
+@pytest.mark.parametrize("coarse", [np.float16, np.int8])
+@pytest.mark.parametrize("dtype,metric,force_rot,dim", [
+    (np.float32, "sqeuclidean", True, 30), (np.float32, "inner_product", False, 32),
+    (np.uint8, "sqeuclidean", False, 32), (np.int8, "euclidean", True, 32),
+    (np.float16, "cosine", True, 24)])
+def test_reduced_precision_coarse_search(orc, coarse, dtype, metric, force_rot, dim):
+    """coarse_search_dtype 16F / 8I (ivf_pq_search.cuh:170-340): probes from the rounded operands,
+    and the rotation applied to the same rounded query rows with the rotation matrix in that type
+    (:996-1019); everything bit-equal to the oracle."""
+    data, model, queries, index, ix, _ = _case(orc, 4000, dim, 50, 16 if dim != 30 else 15, 8, dtype=dtype,
+                                               metric=metric, force_rot=force_rot)
+    if dtype in (np.float32, np.float16):
+        queries = (queries * 0.4).astype(dtype)   # most elements within the 8-bit range after x 128
+    sp = ivf_pq.SearchParams(n_probes=6, coarse_search_dtype=coarse)
+    probes = ivf_pq.select_clusters(sp, index, G.to_dev(queries)).cpu().numpy().view(np.uint32)
+    want_probes, _ = orc.select_clusters(ix, queries, 6, coarse_search_dtype=ORC_DT[coarse])
+    assert np.array_equal(probes, want_probes)
+    want32, _ = orc.select_clusters(ix, queries, 6)
+    print("rows whose probes differ from the fp32 search:", int((want32 != want_probes).any(1).sum()), flush=True)
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, 10, 6, coarse=coarse)
+    H.compare_results(nb, d, want_nb, want_d, 1e-5, exact=True)
+    # the operands' precision is visible in the results (the rotation is not the fp32 one)
+    nb32, d32, _, _ = _search_both(orc, index, ix, queries, 10, 6)
+    if dtype == np.float32:
+        assert not np.array_equal(d, d32)
+
+
+def test_extend_rejects_labels_outside_the_lists(orc):
+    """A caller-supplied label >= n_lists is refused before anything is written: the lists and the
+    size stay as they were, and the index still searches like the oracle."""
+    data, model, queries, index, ix, _ = _case(orc, 2000, 16, 10, 8, 8)
+    sizes = index.list_sizes.cpu().tolist()
+    before = [index.list_indices(l).cpu().numpy()[:sizes[l]].copy() for l in range(10)]
+    extra = H.make_data(64, 16, np.float32, 77)
+    for bad in (10, 11, 2 ** 31, 2 ** 32 - 1):
+        labels = np.full(64, 3, dtype=np.uint32)
+        labels[17] = bad
+        with pytest.raises(CuvsError, match="smaller than n_lists"):
+            ivf_pq.extend(index, G.to_dev(extra), None, labels=G.to_dev(labels.view(np.int32)))
+    assert len(index) == 2000 and index.list_sizes.cpu().tolist() == sizes
+    for l in range(10):
+        assert np.array_equal(index.list_indices(l).cpu().numpy()[:sizes[l]], before[l])
+    nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, 10, 4)
+    H.compare_results(nb, d, want_nb, want_d, 1e-5, exact=True)
+    # valid labels still go through
+    ivf_pq.extend(index, G.to_dev(extra), None, labels=G.to_dev(np.full(64, 9, dtype=np.int32)))
+    assert len(index) == 2064
+
+
 def test_validation_errors(orc):
     """Error behaviour of search (cuVS ivf_pq_search.cuh:901-923,1088-1096; c/src/neighbors/ivf_pq.cpp:315-325)."""
     data, model, queries, index, ix, _ = _case(orc, 500, 8, 4, 4, 8, n_queries=4)
@@ -318,7 +367,7 @@ def _clustered_case(orc, dtype=np.float32, kind="subspace"):
 
 
 def _make_clustered_case(orc, dtype, kind):
-    from cuvs_amd import testing
+    import datasets as testing
     print(f"clustered case dtype={np.dtype(dtype).name} kind={kind}", flush=True)
     if dtype == np.uint8:
         allrows = testing.sift_like_u8(30200, 128, 96, seed=77).numpy()
@@ -335,7 +384,7 @@ def _make_clustered_case(orc, dtype, kind):
                                           (R_8U, R_16F)])
 @pytest.mark.parametrize("dtype,kind", [(np.float32, "subspace"), (np.uint8, "subspace"),
                                         (np.float32, "cluster")])
-def test_early_stop_matches_oracle_and_full_scan(orc, monkeypatch, lut, internal, dtype, kind):
+def test_early_stop_matches_oracle_and_full_scan(orc, lut, internal, dtype, kind):
     from cuvs_amd.resources import Resources
     x, q, index, ix = _clustered_case(orc, dtype, kind)
     res = Resources()
@@ -351,11 +400,11 @@ def test_early_stop_matches_oracle_and_full_scan(orc, monkeypatch, lut, internal
         want_nb, want_d = orc.search(ix, q, k, 48, lut_dtype=ORC_DT[lut],
                                      internal_distance_dtype=ORC_DT[internal])
         H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
-        monkeypatch.setenv("CUVS_AMD_NO_EARLY_STOP", "1")
+        res.set_search_tuning(early_stop="off")
         d2, nb2 = ivf_pq.search(sp, index, G.to_dev(q), k, resources=res)
         res.sync()
         assert ivf_pq.get_search_profile(res)["n_screened_pairs"] == 0
-        monkeypatch.delenv("CUVS_AMD_NO_EARLY_STOP")
+        res.set_search_tuning(early_stop="auto")
         assert torch.equal(nb, nb2) and torch.equal(d, d2)
 
 
@@ -363,7 +412,7 @@ def test_early_stop_matches_oracle_and_full_scan(orc, monkeypatch, lut, internal
 def test_early_stop_pq_len_4(orc, kind):
     """Four dimensions per subspace: 16-byte codebook entries in the table-free screen (shared by
     the block for per-subspace codebooks, one list's codebook per wave for per-cluster ones)."""
-    from cuvs_amd import testing
+    import datasets as testing
     from cuvs_amd.resources import Resources
     allrows = testing.gaussian_mixture(20100, 128, 64, 0.15, seed=78).numpy()
     x, q = allrows[:20000], allrows[20000:]
@@ -495,7 +544,7 @@ def _config_case(orc, x, q, n_lists, pq_dim, pq_bits, metric, kind):
 @pytest.mark.parametrize("n_probes", [16, 32, 64])
 def test_config2_shape_normalised_fp32_l2(orc, n_probes):
     """96-d L2-normalised fp32 mixture, pq_dim 48, 8 bit, fp16 table with fp32 distances."""
-    from cuvs_amd import testing
+    import datasets as testing
     allrows = testing.gaussian_mixture(20200, 96, 100, 0.2, seed=1234, normalize_centers=True,
                                        normalize_rows=True).numpy()
     x, q = allrows[:20000], allrows[20000:]
@@ -507,7 +556,7 @@ def test_config2_shape_normalised_fp32_l2(orc, n_probes):
 def test_config4_shape_inner_product_4bit_fp8_half(orc):
     """768-d unit-norm anisotropic mixture, inner product, pq_dim 384, 4-bit codes (two per byte),
     8-bit table (signed variant), fp16 distances."""
-    from cuvs_amd import testing
+    import datasets as testing
     allrows = testing.gaussian_mixture(3064, 768, 40, 0.05, seed=1234, dim_decay=0.9,
                                        normalize_rows=True).numpy()
     x, q = allrows[:3000], allrows[3000:]
@@ -520,7 +569,7 @@ def test_config4_shape_inner_product_4bit_fp8_half(orc):
 def test_config5_shape_half_rows_per_cluster(orc, batch):
     """96-d fp16 rows, per-cluster codebooks, pq_dim 48, 8 bit, fp16 table, many probes; batch sizes
     1 and 100."""
-    from cuvs_amd import testing
+    import datasets as testing
     allrows = testing.gaussian_mixture(12100, 96, 300, 0.25, seed=1234).numpy().astype(np.float16)
     x, q = allrows[:12000], allrows[12000:12000 + batch]
     index, ix = _config_case(orc, x, q, 150, 48, 8, "sqeuclidean", "cluster")
@@ -570,7 +619,8 @@ def test_refine_matches_oracle(orc, dtype, metric):
 
 def test_refine_after_search_raises_recall(orc):
     """The use the reference documents: search 4k candidates, refine to k."""
-    from cuvs_amd import refine, testing
+    import datasets as testing
+    from cuvs_amd import refine
     x, q, index, ix = _clustered_case(orc)
     sp = ivf_pq.SearchParams(n_probes=20, lut_dtype=R_16F)
     k = 10

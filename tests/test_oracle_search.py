@@ -338,3 +338,175 @@ def test_encode_labels_follow_the_coarse_clustering_metric(orc, metric):
     want = by_ip if metric == "cosine" else by_l2
     assert (by_l2 != by_ip).mean() > 0.3
     assert np.array_equal(labels, want)
+
+
+# --- coarse search in reduced precision (ivf_pq_search.cuh:170-340) ---
+
+R_8I = 3
+
+
+def _f32_fma_chain(a, b):
+    """sum_d a[..., d] * b[..., d] as one fp32 fused-multiply-add chain over ascending d, with numpy
+    scalars only.  The operands used below (binary16 values) have 11-bit significands, so a product
+    is exact in float64 and `product + acc` in float64 is the exact sum unless the exponents are
+    more than 29 binades apart, where the smaller term is far below half an fp32 ulp anyway: one
+    rounding to float32 per step is the fused multiply-add."""
+    acc = np.zeros(np.broadcast_shapes(a.shape, b.shape)[:-1], dtype=np.float32)
+    for d in range(a.shape[-1]):
+        acc = (a[..., d].astype(np.float64) * b[..., d].astype(np.float64)
+               + acc.astype(np.float64)).astype(np.float32)
+    return acc
+
+
+def _half_scores_numpy(model, dim, qf, ip):
+    """The binary16 coarse score of every (query, list) from numpy's own float16: centres (norm
+    column included) and queries rounded to binary16, products accumulated in fp32 over ascending
+    columns, the norm column times -0.5 (L2) last, times alpha, rounded to binary16."""
+    ch = model["centers"].astype(np.float16).astype(np.float32)
+    qh = qf.astype(np.float16).astype(np.float32)
+    acc = _f32_fma_chain(ch[None, :, :dim], qh[:, None, :])
+    if not ip:
+        acc = (ch[None, :, dim].astype(np.float64) * -0.5 + acc.astype(np.float64)).astype(np.float32)
+    alpha = np.float32(-1.0 if ip else -2.0)
+    return (alpha * acc).astype(np.float16).astype(np.float32)
+
+
+@pytest.mark.parametrize("metric,dtype", [("sqeuclidean", np.float32), ("inner_product", np.float32),
+                                          ("sqeuclidean", np.uint8), ("cosine", np.float16)])
+def test_half_coarse_scores_equal_numpy_float16(orc, metric, dtype):
+    dim = 24
+    data, model, ix, labels, codes, queries = _setup(orc, n_lists=40, metric=metric, n=800, dtype=dtype)
+    ip = metric != "sqeuclidean"
+    # centres whose norms (8 .. 40 here after scaling) and elements need rounding to binary16
+    assert np.any(model["centers"].astype(np.float16).astype(np.float32) != model["centers"])
+    want = _half_scores_numpy(model, dim, H.to_float(queries), ip)
+    P = ix.n_lists  # all lists: every score is compared
+    probes, scores = orc.select_clusters(ix, queries, P, coarse_search_dtype=R_16F)
+    for q in range(queries.shape[0]):
+        assert sorted(probes[q].tolist()) == list(range(P))
+        np.testing.assert_array_equal(scores[q], want[q, probes[q]])
+        # ascending (score, list)
+        key = list(zip(scores[q].tolist(), probes[q].tolist()))
+        assert key == sorted(key)
+    # the half scores differ from the fp32 ones (the test would not notice a path that ignores the dtype)
+    _, s32 = orc.select_clusters(ix, queries, P, coarse_search_dtype=R_32F)
+    assert np.any(np.sort(s32, axis=1) != np.sort(scores, axis=1))
+
+
+def test_half_coarse_scores_on_exact_integers(orc):
+    """Integer-valued centres and queries: every product and partial sum is exact, so the score has
+    a closed form, and the norm column (2049 -> 2048 in binary16) shows whether it was rounded."""
+    dim, pq_dim = 8, 4
+    rng = np.random.default_rng(3)
+    c = rng.integers(-20, 21, (6, dim)).astype(np.float32)
+    c[0] = [32, 32, 1, 0, 0, 0, 0, 0]          # squared norm 2049: not a binary16 number
+    de = orc.dim_ext(dim)
+    centers = np.zeros((6, de), dtype=np.float32)
+    centers[:, :dim] = c
+    centers[:, dim] = (c.astype(np.float64) ** 2).sum(1)
+    assert centers[0, dim] == 2049
+    model = {"centers": centers, "centers_rot": c.copy(), "rotation_matrix": np.eye(dim, dtype=np.float32),
+             "pq_centers": np.zeros((pq_dim, 2, 256), dtype=np.float32)}
+    ix = H.oracle_index(orc, model, dim, pq_dim, 8)
+    q = rng.integers(-9, 10, (5, dim)).astype(np.float32)
+    probes, scores = orc.select_clusters(ix, q, 6, coarse_search_dtype=R_16F)
+    n16 = centers[:, dim].astype(np.float16).astype(np.float64)
+    assert n16[0] == 2048
+    want = (n16[None, :] - 2.0 * (q.astype(np.float64) @ c.astype(np.float64).T))
+    want = want.astype(np.float16).astype(np.float32)
+    for i in range(5):
+        np.testing.assert_array_equal(scores[i], want[i, probes[i]])
+
+
+def _int8_rows_numpy(model, dim, qf, ip):
+    """Quantised centre and query rows of the 8-bit coarse search from the formulas in
+    ivf_pq_index.cu:661-738 and ivf_pq_search.cuh:199-210, in numpy."""
+    de8 = (dim + 2 + 15) // 16 * 16
+    m = de8 - dim
+    c = model["centers"]
+    n = c.shape[0]
+    c8 = np.zeros((n, de8), dtype=np.int64)
+    c8[:, :dim] = np.trunc(np.clip(c[:, :dim] * np.float32(128), -128, 127))
+    x = c[:, dim]
+    y = np.clip(x * (np.float32(64) / np.float32(m - 1)), -128, 127).astype(np.float32)
+    ry = np.where(y >= 0, np.floor(y + np.float32(0.5)), np.ceil(y - np.float32(0.5)))  # roundf: half away from zero
+    z = np.clip((y - ry.astype(np.float32)) * np.float32(128), -128, 127)
+    c8[:, dim] = np.trunc(z)
+    c8[:, dim + 1:] = ry[:, None]
+    q8 = np.zeros((qf.shape[0], de8), dtype=np.int64)
+    q8[:, :dim] = np.trunc(np.clip(qf * np.float32(128), -128, 127))
+    q8[:, dim] = 1 - m
+    q8[:, dim + 1:] = 0 if ip else -128
+    return c8, q8
+
+
+@pytest.mark.parametrize("metric,dtype,dim", [("sqeuclidean", np.float32, 24), ("inner_product", np.float32, 24),
+                                              ("sqeuclidean", np.uint8, 24), ("sqeuclidean", np.int8, 12)])
+def test_int8_coarse_scores_equal_the_formulas(orc, metric, dtype, dim):
+    pq_dim = dim // 2
+    data = H.make_data(800, dim, dtype, 5)
+    if dtype == np.float32:
+        data = (data * 0.25).astype(np.float32)  # keep 128 x within int8 for most elements
+    model = H.train(data, 40, pq_dim, 8, metric=metric, iters=4)
+    ix, labels, codes = H.oracle_index_with_data(orc, model, data, pq_dim, 8, metric)
+    queries = H.make_data(40, dim, dtype, 105)
+    if dtype == np.float32:
+        queries = (queries * 0.25).astype(np.float32)
+    ip = metric != "sqeuclidean"
+    qf = H.to_float(queries)
+    c8, q8 = _int8_rows_numpy(model, dim, qf, ip)
+    if dtype == np.uint8:   # mapping<int8_t>(uint8_t x) = x >> 1
+        np.testing.assert_array_equal(q8[:, :dim], queries.astype(np.int64) >> 1)
+    if dtype == np.int8:
+        np.testing.assert_array_equal(q8[:, :dim], queries.astype(np.int64))
+    want = (-1 if ip else -2) * (q8 @ c8.T)
+    P = ix.n_lists
+    probes, scores = orc.select_clusters(ix, queries, P, coarse_search_dtype=R_8I)
+    for q in range(queries.shape[0]):
+        np.testing.assert_array_equal(scores[q].astype(np.int64), want[q, probes[q]])
+        key = list(zip(scores[q].tolist(), probes[q].tolist()))
+        assert key == sorted(key)
+    if not ip:
+        # what the split norm is for: the integer score tracks 128^2 (||c||^2 - 2 q.c) to within the
+        # quantisation of the elements, so the nearest list by the fp32 score is among the first few
+        p32, _ = orc.select_clusters(ix, queries, 1, coarse_search_dtype=R_32F)
+        hits = sum(int(p32[q, 0]) in probes[q, :4].tolist() for q in range(queries.shape[0]))
+        assert hits >= 0.9 * queries.shape[0]
+
+
+def test_int8_split_norm_identity():
+    """dot of the padding columns = -(m - 1) (128 round(y) + z) ~ -128^2 * ||c||^2 / 2."""
+    dim = 24
+    model = {"centers": np.zeros((3, 32), dtype=np.float32)}
+    model["centers"][:, dim] = [0.3, 1.0, 2.5]
+    c8, q8 = _int8_rows_numpy(model, dim, np.zeros((1, dim), dtype=np.float32), False)
+    pad = (q8[:, dim:] @ c8[:, dim:].T)[0]
+    np.testing.assert_allclose(pad, -8192.0 * model["centers"][:, dim], atol=8)  # z is truncated: up to m - 1 = 7 off
+
+
+@pytest.mark.parametrize("coarse", [R_16F, R_8I])
+@pytest.mark.parametrize("force_rot", [False, True])
+def test_rotation_takes_the_coarse_search_operands(orc, coarse, force_rot):
+    """With a 16-bit or 8-bit coarse search the rotation GEMM multiplies the rounded query rows by
+    the rotation matrix in the same type (ivf_pq_search.cuh:996-1019): seen through the fp32 lookup
+    table, whose entries are (rot_q - centre - codebook entry)^2."""
+    dim = 22 if force_rot else 24
+    data, model, ix, labels, codes, queries = _setup(orc, dim=dim, force_rot=force_rot, n=600)
+    queries = (queries * 0.3).astype(np.float32)
+    qf = H.to_float(queries)
+    R = model["rotation_matrix"]
+    if coarse == R_16F:
+        rq = qf.astype(np.float16).astype(np.float64) @ R.astype(np.float16).astype(np.float64).T
+    else:
+        q8 = np.trunc(np.clip(qf * np.float32(128), -128, 127)).astype(np.float64)
+        r8 = np.trunc(np.clip(R * np.float32(128), -128, 127)).astype(np.float64)
+        rq = (q8 @ r8.T) / 16384.0
+    rq32 = qf.astype(np.float64) @ R.astype(np.float64).T
+    assert np.abs(rq - rq32).max() > 1e-4   # the rounded operands are visible
+    for qi in (0, 7):
+        for l in (1, 5):
+            got = orc.make_lut(ix, queries[qi], l, R_32F, coarse_search_dtype=coarse)
+            diff = rq[qi] - model["centers_rot"][l].astype(np.float64)
+            book = model["pq_centers"].astype(np.float64)      # [pq_dim, pq_len, B]
+            want = ((diff.reshape(ix.pq_dim, ix.pq_len, 1) - book) ** 2).sum(1)
+            np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-7)
