@@ -92,6 +92,8 @@ def main():
                     help="train the index with the library (cuvsIvfPqBuild) or with the torch helper")
     ap.add_argument("--refine-ratio", type=int, default=1,
                     help="search refine_ratio * k candidates and re-rank them exactly (1 = off)")
+    ap.add_argument("--early-stop", choices=("auto", "off", "on"), default="auto",
+                    help="fix the library's choice of the L2 early stop for the whole run (profiling runs)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--with-cpu", action="store_true", help="time the CPU oracle also with --config")
@@ -131,6 +133,7 @@ def main():
 
     res = Resources()
     res.use_torch_current_stream()
+    res.set_search_tuning(early_stop=args.early_stop)
     n_train = min(n, max(n_lists * 32, 200_000))
     if args.build == "native":
         # the library's own training (cuvsIvfPqBuild) on a subsample of n_train rows, then every row
@@ -238,7 +241,7 @@ def main():
     full_name = ("scan_kernel" if not fused
                  else "scan_nibble_kernel" if nibble
                  else "scan_kernel" if (pq_bits != 8 or (pq_dim, pq_len) not in ((64, 2), (48, 2), (32, 4)))
-                 else "scan_quad_kernel" if (args.lut != "f32" and k <= 128) else "scan_fast_kernel")
+                 else "scan_stream_kernel" if (args.lut != "f32" and k <= 128) else "scan_fast_kernel")
     default_path = {"early_stop": bool(early_stop), "ms_per_step": ms_per_step, "qps": qps,
                     "scan_stage_ms": mean(prof, "scan_ms"),
                     "stage_ms": {s_: mean(prof, s_) for s_ in ("coarse_ms", "rotate_ms", "scan_ms", "merge_ms")}}
@@ -270,7 +273,7 @@ def main():
         full_ms_per_step = timed(args.steps, args.warmup)
         full_prof = profiled(args.steps)
         full_ids = neighbors.cpu().numpy().copy()
-        res.set_search_tuning(early_stop="auto")
+        res.set_search_tuning(early_stop=args.early_stop)
         assert full_prof[-1]["n_screened_pairs"] == 0
         same_ids = bool((full_ids == gpu_ids).all()) if args.refine_ratio <= 1 else None
     else:

@@ -343,11 +343,11 @@ bool launch_scan_fast(const scan_args& a, hipStream_t stream);
  *  same records, candidate keys and bound updates. */
 bool scan_nibble_supported(const scan_args& a);
 bool launch_scan_nibble(const scan_args& a, hipStream_t stream);
-/** CU-wide kernel for 8-bit codes, k <= 64 and fp16 / 8-bit tables (scan_quad.hip).  It writes
- *  several candidate groups per pair: scan_quad_keys_per_pair() is the number of keys the output
+/** CU-wide kernel for 8-bit codes, k <= 128 and fp16 / 8-bit tables (scan_stream.hip).  It writes
+ *  several candidate groups per pair: scan_stream_keys_per_pair() is the number of keys the output
  *  buffer must hold per (query, probe) pair, 0 when the arguments are outside what it covers. */
-uint32_t scan_quad_keys_per_pair(const scan_args& a);
-bool launch_scan_quad(const scan_args& a, hipStream_t stream);
+uint32_t scan_stream_keys_per_pair(const scan_args& a);
+bool launch_scan_stream(const scan_args& a, hipStream_t stream);
 
 /**
  * Early termination for L2 metrics, as compute_score's early stop in the reference

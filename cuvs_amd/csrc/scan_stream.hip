@@ -1,0 +1,708 @@
+/*
+ * CU-wide LUT + code-scan kernel for 8-bit codes, k <= 128 and fp16 / 8-bit tables: the kernel
+ * that streams the probed lists in the benchmark configurations.  Same arithmetic as the other
+ * scan kernels (compute_similarity of the reference: create_lut_impl.cuh:16-79,
+ * compute_distances_impl.cuh:40-105, compute_score_impl.cuh:55-79); the organisation is a
+ * producer / consumer split inside one persistent 1024-thread block per CU:
+ *
+ *   - 8 of the 16 waves build lookup tables, the other 8 scan codes with them, at the same time:
+ *     while the scanners work through the two (query, probe) pairs of iteration i, the builders
+ *     make the two tables of iteration i + 1 in the other half of a double buffer.  One block
+ *     barrier per iteration is the only synchronisation.  On every SIMD two waves of each kind
+ *     share the issue slots, so the vector work of the table build fills the cycles in which the
+ *     scanners wait for their LDS gathers and code loads;
+ *   - a builder thread owns one codebook entry of half the subspaces and keeps those codebook
+ *     components in registers for the whole kernel (the scanners spend their registers on code
+ *     tiles instead: the two roles are separate loops, so neither pays for the other's state);
+ *   - every table entry is stored as a binary16 number in the form the scan adds: the entry itself
+ *     for fp16 tables; for 8-bit tables the decoded value decode(encode(score)), which the reference
+ *     computes again at every lookup - as it is when the sums are binary16, and halved when they are
+ *     fp32 (half of every decoded 8-bit value is a binary16 number, the largest ones themselves are
+ *     not), the scan then adding twice the entry, which is exact;
+ *   - a lookup is two vector instructions: the code byte is shifted into the low half of an address
+ *     register by one sub-dword instruction (the high half holds the table's 64 KB window, the
+ *     subspace's offset sits in the read's immediate field), and the entry is added;
+ *   - four scanner waves share a pair; each keeps its own candidate buffer and bound, and writes
+ *     its <= k best candidates of the pair (the per-query merge sees 4 k keys per pair);
+ *   - blocks that run on one XCD take neighbouring pairs, which probe the same lists: a list's
+ *     codes come from HBM once and are then served by that XCD's L2.
+ */
+#include "device_utils.cuh"
+
+namespace cuvs::neighbors::ivf_pq::detail {
+
+namespace {
+
+#define LDS_AS __attribute__((address_space(3)))
+#define GLOBAL_AS __attribute__((address_space(1)))
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte chunk of codes
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t kStreamThreads  = 1024;
+constexpr uint32_t kStreamPairs    = 2;  // pairs per iteration
+constexpr uint32_t kStreamScanners = 8;  // scanner waves (and as many builder waves)
+constexpr uint32_t kStreamWG       = kStreamScanners / kStreamPairs;  // scanner waves per pair
+constexpr uint32_t kStreamMaxK     = 128;
+
+/* LDS map (bytes).  The four tables sit at multiples of 32 KB so that a table's address splits
+ * into a 64 KB window (high half of the address register) and an immediate offset below 64 K:
+ *   table of (buffer b, pair 0) at 0x08000 + b * 0x10000, of (b, pair 1) at 0x10000 + b * 0x10000. */
+constexpr uint32_t kStreamLdsBytes  = 160 * 1024;
+constexpr uint32_t kStreamStageBase = 16;               // 2 buffers x 2 pairs x 256 floats
+constexpr uint32_t kStreamStageSlot = 256 * 4;          // bytes per (buffer, pair)
+constexpr uint32_t kStreamCandBase  = 16 + 4 * kStreamStageSlot;
+__host__ __device__ constexpr uint32_t stream_table_base(uint32_t buffer, uint32_t g)
+{
+  return (g == 0 ? 0x08000u : 0x10000u) + buffer * 0x10000u;
+}
+
+/** Candidate keys a wave buffers: room for k kept ones plus one tile of 64 new ones. */
+inline __host__ __device__ uint32_t stream_wave_cap(uint32_t k) { return k <= 64u ? 128u : 192u; }
+static_assert(kStreamCandBase + kStreamScanners * 192u * 8u <= 0x08000u, "small buffers must end below the tables");
+
+__device__ __forceinline__ void block_barrier()
+{
+  // LDS traffic of this wave is complete; global loads stay in flight across the barrier
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+/** `v` in a register the compiler knows nothing about (it would otherwise fold a multiplication by
+ *  one away and lose the single-instruction widening multiply-add). */
+__device__ __forceinline__ float opaque_float(float v)
+{
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
+/** Ascending sort of the first `cap` keys (at most 256) of one wave's buffer: a bitonic network made of
+ *  ascending comparators only (each merge starts with a mirror step), run on the next power of two
+ *  with the missing top slots standing for keys larger than any other - a comparator that would
+ *  touch one of them never swaps, so it is skipped.  LDS operations of a wave execute in program
+ *  order, so no barrier is needed. */
+__device__ __forceinline__ void wave_sort_keys(LDS_AS unsigned long long* buf, uint32_t lane, uint32_t cap)
+{
+  const uint32_t n_half = cap <= 2u ? 1u : (1u << (31 - __builtin_clz(cap - 1u)));
+  auto compare_exchange = [&](uint32_t i, uint32_t l) __attribute__((always_inline)) {
+    if (l < cap) {
+      const unsigned long long x = buf[i];
+      const unsigned long long y = buf[l];
+      if (x > y) {
+        buf[i] = y;
+        buf[l] = x;
+      }
+    }
+  };
+#pragma unroll 1
+  for (uint32_t size = 2; size <= 2u * n_half; size <<= 1) {
+    const uint32_t half = size >> 1;
+    for (uint32_t c = lane; c < n_half; c += 64u) {
+      const uint32_t base = (c / half) * size;
+      const uint32_t off  = c & (half - 1u);
+      compare_exchange(base + off, base + size - 1u - off);
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll 1
+    for (uint32_t stride = size >> 2; stride > 0; stride >>= 1) {
+      for (uint32_t c = lane; c < n_half; c += 64u) {
+        const uint32_t i = (c / stride) * (2u * stride) + (c & (stride - 1u));
+        compare_exchange(i, i + stride);
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+}
+
+/** The 16 bits stored for a table entry (see the file comment). */
+template <int LUT, bool OUT_HALF>
+__device__ __forceinline__ uint16_t table_entry(float score)
+{
+  using traits = lut_traits<LUT>;
+  const auto e = traits::encode(score);
+  if constexpr (LUT == LUT_F16) {
+    return __builtin_bit_cast(uint16_t, e);
+  } else if constexpr (OUT_HALF) {
+    return __builtin_bit_cast(uint16_t, traits::to_half(e));
+  } else {
+    // 2^-16 * 1.0625 .. 63488, four significant bits: exact in binary16 (subnormal at the low end)
+    return __builtin_bit_cast(uint16_t, _Float16(traits::to_float(e) * 0.5f));
+  }
+}
+
+/* ---- the lookups, as inline assembly: the compiler would otherwise extract each byte, form a
+ * full address and wait for every read ---- */
+
+/** low half of `addr` = 2 * byte SEL of `w`; the high half is kept. */
+template <int SEL>
+__device__ __forceinline__ void code_offset(uint32_t& addr, uint32_t one, uint32_t w)
+{
+  static_assert(SEL >= 0 && SEL < 4, "byte of a dword");
+  if constexpr (SEL == 0) {
+    asm volatile("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:BYTE_0"
+                 : "+v"(addr) : "v"(one), "v"(w));
+  } else if constexpr (SEL == 1) {
+    asm volatile("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:BYTE_1"
+                 : "+v"(addr) : "v"(one), "v"(w));
+  } else if constexpr (SEL == 2) {
+    asm volatile("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:BYTE_2"
+                 : "+v"(addr) : "v"(one), "v"(w));
+  } else {
+    asm volatile("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:BYTE_3"
+                 : "+v"(addr) : "v"(one), "v"(w));
+  }
+}
+
+/** Entry read: 16 bits, zero-extended. */
+template <int IMM>
+__device__ __forceinline__ void entry_read(uint32_t& val, uint32_t addr)
+{
+  static_assert(IMM >= 0 && IMM < 65536, "the read's offset field has 16 bits");
+  // an output only: a register that the compiler believed to hold a value before the read could be
+  // copied by it right after the read was issued, before the data is there
+  asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(val) : "v"(addr), "n"(IMM));
+}
+
+/** Issues the eight lookups of code words w0, w1 (subspaces J0 .. J0 + 7 of the tile's rows). */
+template <int IMM0>
+__device__ __forceinline__ void issue8(uint32_t w0, uint32_t w1, uint32_t one, uint32_t (&addr)[8], uint32_t (&val)[8])
+{
+  code_offset<0>(addr[0], one, w0);
+  code_offset<1>(addr[1], one, w0);
+  code_offset<2>(addr[2], one, w0);
+  code_offset<3>(addr[3], one, w0);
+  code_offset<0>(addr[4], one, w1);
+  code_offset<1>(addr[5], one, w1);
+  code_offset<2>(addr[6], one, w1);
+  code_offset<3>(addr[7], one, w1);
+  entry_read<IMM0 + 0 * 512>(val[0], addr[0]);
+  entry_read<IMM0 + 1 * 512>(val[1], addr[1]);
+  entry_read<IMM0 + 2 * 512>(val[2], addr[2]);
+  entry_read<IMM0 + 3 * 512>(val[3], addr[3]);
+  entry_read<IMM0 + 4 * 512>(val[4], addr[4]);
+  entry_read<IMM0 + 5 * 512>(val[5], addr[5]);
+  entry_read<IMM0 + 6 * 512>(val[6], addr[6]);
+  entry_read<IMM0 + 7 * 512>(val[7], addr[7]);
+}
+
+/** The eight reads issued into `val` have landed; MORE: eight younger ones may still be in flight
+ *  (LDS reads return in order; other outstanding operations only make the wait longer). */
+template <bool MORE>
+__device__ __forceinline__ void landed8(uint32_t (&val)[8])
+{
+  if constexpr (MORE) {
+    asm volatile("s_waitcnt lgkmcnt(8)"
+                 : "+v"(val[0]), "+v"(val[1]), "+v"(val[2]), "+v"(val[3]), "+v"(val[4]), "+v"(val[5]), "+v"(val[6]), "+v"(val[7]));
+  } else {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(val[0]), "+v"(val[1]), "+v"(val[2]), "+v"(val[3]), "+v"(val[4]), "+v"(val[5]), "+v"(val[6]), "+v"(val[7]));
+  }
+}
+
+template <int NCH, int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER, bool IP>
+struct stream_kernel {
+  using traits = lut_traits<LUT>;
+  using acc_t  = typename std::conditional<OUT_HALF, _Float16, float>::type;
+  static constexpr int M              = NCH * 16;  // pq_dim
+  static constexpr int HALFM          = M / 2;     // subspaces whose codebook a builder thread holds
+  static constexpr uint32_t ROT       = uint32_t(M) * PQ_LEN;
+  static constexpr uint32_t n_diff    = ROT * (IP ? 2u : 1u);
+  static constexpr uint32_t G         = kStreamPairs;
+  static constexpr uint32_t WG        = kStreamWG;
+  // fp32 sums: entry * kEntryScale is added (one instruction: the binary16 entry is widened inside a
+  // multiply-add); 8-bit tables hold half the decoded value
+  static constexpr float kEntryScale = LUT == LUT_F16 ? 1.0f : 2.0f;
+  static_assert(n_diff * 4u <= kStreamStageSlot, "staged terms of a pair must fit their slot");
+  static_assert(ROT * G <= 512u, "one builder thread stages one (pair, dimension)");
+  static_assert(uint32_t(M) * 512u <= 0x8000u, "a table must fit its 32 KB slot");
+
+  const scan_args& a;
+  uint32_t n_pairs, n_quads, grid, lb, n_it;
+  uint32_t lane, rw;  // lane; index of the wave among the waves of its role (0..7)
+
+  __device__ __forceinline__ pair_desc record(uint32_t quad, uint32_t g) const
+  {
+    // slots past the end read as an empty pair
+    const uint32_t slot = quad * G + g;
+    pair_desc d         = a.desc[slot < n_pairs ? slot : n_pairs - 1u];
+    if (slot >= n_pairs) {
+      d.n_rows = 0;
+      d.slot   = 0xFFFFFFFFu;
+    }
+    return d;
+  }
+  __device__ __forceinline__ uint32_t quad_of(uint32_t it) const { return lb + it * grid; }
+
+  /* ------------------------------------ builders ------------------------------------ */
+
+  /** What the builders need to know about the two pairs of an iteration: which query and list
+   *  (for the operands they fetch) and the row count (nothing is built for an empty pair).  Raw
+   *  fields of the records: they are requested an iteration before anything looks at them. */
+  struct quad_info {
+    uint32_t q[G], label[G], n_rows[G];
+  };
+  __device__ __forceinline__ quad_info load_info(uint32_t it) const
+  {
+    quad_info r;
+#pragma unroll
+    for (uint32_t g = 0; g < G; g++) {
+      r.q[g]      = 0;
+      r.label[g]  = 0;
+      r.n_rows[g] = 0;
+    }
+    if (it < n_it) {  // uniform
+#pragma unroll
+      for (uint32_t g = 0; g < G; g++) {
+        const uint32_t slot = quad_of(it) * G + g;
+        if (slot < n_pairs) {
+          const pair_desc* d = a.desc + slot;
+          r.q[g]             = d->q;
+          r.label[g]         = d->label;
+          r.n_rows[g]        = d->n_rows;
+        }
+      }
+    }
+    return r;
+  }
+
+  struct staged {
+    float q, c;
+    float cb[PER_CLUSTER ? G : 1][PQ_LEN];  // per-cluster codebook components of the builder's entry
+    bool live[G];
+  };
+
+  /** ds_write_b16 at addr + IMM. */
+  template <int IMM>
+  __device__ __forceinline__ static void entry_write(uint32_t addr, uint32_t bits16)
+  {
+    static_assert(IMM >= 0 && IMM < 65536, "the write's offset field has 16 bits");
+    asm volatile("ds_write_b16 %0, %1 offset:%2" : : "v"(addr), "v"(bits16), "n"(IMM) : "memory");
+  }
+
+  static constexpr int TERMS   = IP ? 2 : 1;
+  static constexpr int FPS     = PQ_LEN * TERMS;  // staged floats per subspace
+  static constexpr int GROUP   = 16 / FPS;        // subspaces whose terms make four 16-byte reads
+  static constexpr int NGROUPS = HALFM / GROUP;
+  static_assert(GROUP >= 1 && HALFM % GROUP == 0, "the subspaces of a builder thread split into whole groups");
+
+  /** Entries of subspaces first .. first + GROUP - 1 of the thread's half from their 16 staged floats. */
+  template <int gi, int u = 0>
+  __device__ __forceinline__ static void build_group(const float (&term)[16], const float (&book)[PER_CLUSTER ? 1 : HALFM][PQ_LEN],
+                                                     const float (&cb)[PQ_LEN], uint32_t waddr)
+  {
+    if constexpr (u < GROUP) {
+      constexpr int jj = gi * GROUP + u;
+      float score      = 0.0f;
+#pragma unroll
+      for (int t = 0; t < PQ_LEN; t++) {
+        const float pqc = PER_CLUSTER ? cb[t] : book[PER_CLUSTER ? 0 : jj][t];
+        if constexpr (!IP) {
+          float df = term[u * FPS + t];
+          df -= pqc;
+          score = fmaf(df, df, score);
+        } else {
+          const float qv = term[u * FPS + 2 * t];
+          score -= term[u * FPS + 2 * t + 1];
+          score = fmaf(-qv, pqc, score);
+        }
+      }
+      entry_write<jj * 512>(waddr, table_entry<LUT, OUT_HALF>(score));
+      build_group<gi, u + 1>(term, book, cb, waddr);
+    }
+  }
+
+  template <int gi>
+  __device__ __forceinline__ static void build_groups(const LDS_AS f32x4* terms, f32x4 (&cur4)[4],
+                                                      const float (&book)[PER_CLUSTER ? 1 : HALFM][PQ_LEN],
+                                                      const float (&cb)[PQ_LEN], uint32_t waddr)
+  {
+    // the next group's terms are requested before this group is computed
+    f32x4 nxt4[4];
+    if constexpr (gi + 1 < NGROUPS) {
+#pragma unroll
+      for (int x = 0; x < 4; x++) { nxt4[x] = terms[(gi + 1) * 4 + x]; }
+    }
+    float term[16];
+#pragma unroll
+    for (int x = 0; x < 4; x++) {
+      term[4 * x + 0] = cur4[x].x;
+      term[4 * x + 1] = cur4[x].y;
+      term[4 * x + 2] = cur4[x].z;
+      term[4 * x + 3] = cur4[x].w;
+    }
+    build_group<gi>(term, book, cb, waddr);
+    if constexpr (gi + 1 < NGROUPS) {
+#pragma unroll
+      for (int x = 0; x < 4; x++) { cur4[x] = nxt4[x]; }
+      build_groups<gi + 1>(terms, cur4, book, cb, waddr);
+    }
+  }
+
+  __device__ __forceinline__ void run_builder() const
+  {
+    const uint32_t bt   = rw * 64u + lane;  // 0..511
+    const uint32_t code = bt & 255u;
+    const uint32_t half = rw >> 2;          // wave-uniform
+    float book[PER_CLUSTER ? 1 : HALFM][PQ_LEN];
+    if constexpr (!PER_CLUSTER) {
+#pragma unroll
+      for (int jj = 0; jj < HALFM; jj++) {
+#pragma unroll
+        for (int t = 0; t < PQ_LEN; t++) {
+          book[jj][t] = a.pq_centers[((half * HALFM + jj) * PQ_LEN + t) * 256 + code];
+        }
+      }
+    } else {
+      book[0][0] = 0.0f;
+    }
+    // operands of the pairs in `info`: the staging element (pair bt / ROT, dimension bt % ROT) and,
+    // for per-cluster codebooks, this thread's components of both pairs' codebooks
+    auto fetch = [&](const quad_info& info, staged& f) {
+      f.q = 0.0f;
+      f.c = 0.0f;
+#pragma unroll
+      for (uint32_t g = 0; g < G; g++) { f.live[g] = info.n_rows[g] != 0; }
+      if (bt < ROT * G) {
+        const uint32_t g   = bt / ROT;
+        const uint32_t dim = bt - g * ROT;
+        const bool live    = (g == 0 ? info.n_rows[0] : info.n_rows[G - 1]) != 0;
+        if (live) {
+          f.q = a.rot_q[uint64_t(g == 0 ? info.q[0] : info.q[G - 1]) * ROT + dim];
+          f.c = a.centers_rot[uint64_t(g == 0 ? info.label[0] : info.label[G - 1]) * ROT + dim];
+        }
+      }
+      if constexpr (PER_CLUSTER) {
+#pragma unroll
+        for (uint32_t g = 0; g < G; g++) {
+#pragma unroll
+          for (int t = 0; t < PQ_LEN; t++) {
+            f.cb[g][t] = info.n_rows[g] != 0 ? a.pq_centers[(uint64_t(info.label[g]) * PQ_LEN + t) * 256 + code] : 0.0f;
+          }
+        }
+      }
+    };
+    auto stage = [&](uint32_t buffer, const staged& f) {
+      if (bt < ROT * G) {
+        auto* dst = reinterpret_cast<LDS_AS float*>(
+          uintptr_t(kStreamStageBase + (buffer * G + bt / ROT) * kStreamStageSlot));
+        if constexpr (!IP) {
+          dst[bt % ROT] = f.q - f.c;
+        } else {
+          dst[2 * (bt % ROT)]     = f.q;
+          dst[2 * (bt % ROT) + 1] = f.c * f.q;
+        }
+      }
+    };
+    // tables of iteration `it` from the terms staged in buffer it & 1
+    auto build = [&](uint32_t it, const staged& f) {
+      const uint32_t buffer = it & 1u;
+#pragma unroll
+      for (uint32_t g = 0; g < G; g++) {
+        if (!f.live[g]) { continue; }  // uniform
+        const auto* terms = reinterpret_cast<const LDS_AS f32x4*>(
+          uintptr_t(kStreamStageBase + (buffer * G + g) * kStreamStageSlot + half * uint32_t(HALFM * FPS) * 4u));
+        // entry (j, code) of the table at base + j * 512 + code * 2; j = half * HALFM + jj
+        const uint32_t waddr = stream_table_base(buffer, g) + half * uint32_t(HALFM) * 512u + code * 2u;
+        f32x4 cur4[4];
+#pragma unroll
+        for (int x = 0; x < 4; x++) { cur4[x] = terms[x]; }
+        build_groups<0>(terms, cur4, book, f.cb[PER_CLUSTER ? g : 0], waddr);
+      }
+    };
+
+    staged cur_f{}, nxt_f{};
+    quad_info info_a = load_info(0);
+    quad_info info_b = load_info(1);
+    fetch(info_a, cur_f);
+    stage(0, cur_f);
+    if (n_it > 1) { fetch(info_b, nxt_f); }
+    info_a = load_info(2);  // always the records two iterations past the tables being built
+    block_barrier();        // terms of iteration 0 visible
+    build(0, cur_f);
+    if (n_it > 1) { stage(1, nxt_f); }
+    block_barrier();  // tables of iteration 0 and terms of iteration 1 visible
+    for (uint32_t it = 0; it < n_it; it++) {
+      // the scanners are working on iteration `it`; nxt_f holds the operands of it + 1 (their terms
+      // are staged), info_a the records of it + 2
+      staged after_f{};
+      const bool two_ahead = it + 2 < n_it;
+      if (two_ahead) { fetch(info_a, after_f); }
+      info_b = load_info(it + 3);
+      if (it + 1 < n_it) { build(it + 1, nxt_f); }
+      // buffer it & 1 was read by the build of iteration `it`, which is over
+      if (two_ahead) { stage(it & 1u, after_f); }
+      nxt_f  = after_f;
+      info_a = info_b;
+      block_barrier();
+    }
+  }
+
+  /* ------------------------------------ scanners ------------------------------------ */
+
+  /** Address of chunk 0 of `row`; chunk m is 32 vectors further on. */
+  __device__ __forceinline__ static const GLOBAL_AS u32x4* row_ptr(const uint8_t* list_data, uint32_t row)
+  {
+    return reinterpret_cast<const GLOBAL_AS u32x4*>(
+      reinterpret_cast<uintptr_t>(list_data) + uint64_t(row >> 5) * (NCH * 512u) + uint64_t(row & 31u) * 16u);
+  }
+  __device__ __forceinline__ static void load_tile(const GLOBAL_AS u32x4* ptr, u32x4 (&dst)[NCH])
+  {
+#pragma unroll
+    for (int m = 0; m < NCH; m++) { dst[m] = ptr[m * 32]; }
+  }
+
+  __device__ __forceinline__ static acc_t add8(acc_t acc, const uint32_t (&val)[8], float one)
+  {
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      if constexpr (OUT_HALF) {
+        acc = acc_t(acc + __builtin_bit_cast(_Float16, uint16_t(val[i])));
+      } else {
+        // `one` holds kEntryScale; the product is exact, so this is acc + value with one rounding
+        acc = fmaf(float(__builtin_bit_cast(_Float16, uint16_t(val[i]))), one, acc);
+      }
+    }
+    return acc;
+  }
+
+  /** Chunk m of a tile and, by recursion, the chunks after it.  The sixteen lookups of a chunk are
+   *  issued together and the first eight are added while the other eight arrive.  Between the issue
+   *  of a lookup and the wait for it there is straight-line code only: the registers the reads
+   *  write are values to the compiler from the moment of issue, and at a branch it may copy them.
+   *  For L2 metrics the wave stops after a chunk once every row is past `stop_bits` (sums only
+   *  grow; early stop of compute_score in the reference).  IMMG = offset of the wave's table inside
+   *  its 64 KB window. */
+  template <int IMMG, int m>
+  __device__ __forceinline__ static acc_t chunk_sum(acc_t acc, const u32x4 (&cur)[NCH], uint32_t one_u, float one,
+                                                    bool valid, uint32_t stop_bits, uint32_t (&addr)[8])
+  {
+    uint32_t va[8], vb[8];
+    issue8<IMMG + (m * 16) * 512>(cur[m].x, cur[m].y, one_u, addr, va);
+    issue8<IMMG + (m * 16 + 8) * 512>(cur[m].z, cur[m].w, one_u, addr, vb);
+    landed8<true>(va);
+    acc = add8(acc, va, one);
+    landed8<false>(vb);
+    acc = add8(acc, vb, one);
+    if constexpr (m + 1 < NCH) {
+      if constexpr (!IP) {
+        const bool live = __builtin_amdgcn_ballot_w64(valid && !(__float_as_uint(float(acc)) > stop_bits)) != 0ull;
+        if (!live) { return acc; }
+      }
+      return chunk_sum<IMMG, m + 1>(acc, cur, one_u, one, valid, stop_bits, addr);
+    } else {
+      return acc;
+    }
+  }
+
+  /** Sum of the tile's table entries in subspace order. */
+  template <int IMMG>
+  __device__ __forceinline__ static acc_t tile_sum(const u32x4 (&cur)[NCH], uint32_t one_u, float one, bool valid,
+                                                   uint32_t stop_bits, uint32_t window)
+  {
+    // address registers: the table's 64 KB window in the high halves, code offsets go to the low ones
+    uint32_t addr[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      addr[i] = window;
+      asm volatile("" : "+v"(addr[i]));
+    }
+    return chunk_sum<IMMG, 0>(acc_t(0), cur, one_u, one, valid, stop_bits, addr);
+  }
+
+  template <int GI>
+  __device__ __forceinline__ void run_scanner() const
+  {
+    constexpr int IMMG     = GI == 0 ? 0x8000 : 0;
+    const uint32_t wig     = rw & 3u;
+    const uint32_t sw      = rw;  // scanner wave 0..7
+    const uint32_t cap     = stream_wave_cap(a.k);
+    auto* my_cand          = reinterpret_cast<LDS_AS unsigned long long*>(uintptr_t(kStreamCandBase)) + sw * cap;
+    const float one        = opaque_float(kEntryScale);
+    uint32_t one_u         = 1u;
+    asm volatile("" : "+v"(one_u));
+
+    pair_desc my_d = record(quad_of(0), GI);
+    u32x4 cur[NCH], ahead[NCH];
+    if (wig * 64u < my_d.n_rows) {
+      const uint32_t r0 = wig * 64u + lane;
+      load_tile(row_ptr(my_d.data, r0 < my_d.n_rows ? r0 : 0u), cur);
+    }
+    uint32_t pre_thr = my_d.n_rows != 0 ? a.query_kth[my_d.q] : 0xFFFFFFFFu;
+    block_barrier();
+    block_barrier();  // tables of iteration 0 are complete
+
+    for (uint32_t it = 0; it < n_it; it++) {
+      const bool has_next   = it + 1 < n_it;
+      const pair_desc nxt_d = record(quad_of(has_next ? it + 1 : it), GI);
+      // window of this iteration's table in the high halves of the address registers
+      const uint32_t window = (((it & 1u) + (GI == 0 ? 0u : 1u)) << 16);
+
+      if (my_d.slot != 0xFFFFFFFFu) {
+        const uint32_t n_rows     = my_d.n_rows;
+        const uint32_t sample_off = my_d.sample_off;
+        const uint8_t* list_data  = my_d.data;
+        const int64_t* list_ids   = a.filter_bits != nullptr && n_rows != 0 ? a.inds_ptrs[my_d.label] : nullptr;
+        const uint32_t n_tiles    = (n_rows + 63u) >> 6;
+        uint32_t thr              = pre_thr;
+        uint32_t wcount           = 0;
+        for (uint32_t tile = wig; tile < n_tiles; tile += WG) {
+          const uint32_t i = tile * 64u + lane;
+          if (tile + WG < n_tiles) {
+            const uint32_t in = i + WG * 64u;
+            load_tile(row_ptr(list_data, in < n_rows ? in : 0u), ahead);
+          }
+          bool valid = i < n_rows;
+          if (valid && list_ids != nullptr) {
+            const int64_t id = reinterpret_cast<const GLOBAL_AS int64_t*>(reinterpret_cast<uintptr_t>(list_ids))[i];
+            valid = id >= 0 && id < a.filter_nbits && ((a.filter_bits[id >> 5] >> (id & 31)) & 1u) != 0;
+          }
+          const uint32_t stop_bits = thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u;
+          acc_t acc = tile_sum<IMMG>(cur, one_u, one, valid, stop_bits, window);
+          if (a.metric == int(DistanceType::CosineExpanded)) { acc = acc_t(acc + acc_t(1)); }
+          const float score_f = float(acc);
+          if (score_f != score_f) { valid = false; }
+          const uint32_t okey = order_f32(score_f);
+          const bool pass     = valid && okey <= thr;
+          const unsigned long long mask = __ballot(pass);
+          if (mask != 0ull) {
+            if (wcount + 64u > cap) {
+              // make room: keep the k best of the buffer and tighten the wave's bound
+              wave_sort_keys(my_cand, lane, wcount);
+              if (wcount >= a.k) {
+                wcount            = a.k;
+                const uint32_t t2 = uint32_t(my_cand[a.k - 1] >> 32);
+                thr               = t2 < thr ? t2 : thr;
+              }
+            }
+            const bool pass2 = pass && okey <= thr;
+            const unsigned long long mask2 = __ballot(pass2);
+            const uint32_t below =
+              __builtin_amdgcn_mbcnt_hi(uint32_t(mask2 >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(mask2), 0u));
+            if (pass2) { my_cand[wcount + below] = (static_cast<unsigned long long>(okey) << 32) | (sample_off + i); }
+            wcount += uint32_t(__popcll(mask2));
+          }
+          if (tile + WG < n_tiles) {
+#pragma unroll
+            for (int m = 0; m < NCH; m++) { cur[m] = ahead[m]; }
+          }
+        }
+        // this wave's best candidates of the pair
+        unsigned long long* out = a.out_keys + (uint64_t(my_d.slot) * WG + wig) * a.k;
+        if (wcount >= a.k) {
+          wave_sort_keys(my_cand, lane, wcount);  // only as wide as there are candidates
+          wcount = a.k;
+          if (lane == 0) { atomicMin(&a.query_kth[my_d.q], uint32_t(my_cand[a.k - 1] >> 32)); }
+        }
+        for (uint32_t t = lane; t < a.k; t += 64u) { out[t] = t < wcount ? my_cand[t] : kInvalidKey; }
+      }
+
+      // first tile and bound of the next pair: they arrive while the other waves finish
+      if (has_next) {
+        my_d = nxt_d;
+        if (wig * 64u < my_d.n_rows) {
+          const uint32_t r0 = wig * 64u + lane;
+          load_tile(row_ptr(my_d.data, r0 < my_d.n_rows ? r0 : 0u), cur);
+        }
+        if (my_d.n_rows != 0) { pre_thr = a.query_kth[my_d.q]; }
+      }
+      block_barrier();
+    }
+  }
+};
+
+template <int NCH, int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER, bool IP>
+__global__ __launch_bounds__(kStreamThreads) void scan_stream_kernel(scan_args a)
+{
+  using body = stream_kernel<NCH, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER, IP>;
+  const uint32_t tid = threadIdx.x;
+  const uint32_t wid = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it scalar
+  // the same in every lane: keep it (and everything derived from it) in scalar registers
+  const uint32_t n_pairs = __builtin_amdgcn_readfirstlane(a.n_pairs_dev != nullptr ? *a.n_pairs_dev : a.n_pairs);
+  const uint32_t n_quads = (n_pairs + kStreamPairs - 1u) / kStreamPairs;
+  const uint32_t grid    = gridDim.x;
+  // Workgroups go to the XCDs in turn; the blocks of one XCD take a contiguous run of pairs.
+  const uint32_t lb = (grid & 7u) == 0u ? (blockIdx.x & 7u) * (grid >> 3) + (blockIdx.x >> 3) : blockIdx.x;
+  if (lb >= n_quads) { return; }  // whole block, before any barrier
+  body k{a, n_pairs, n_quads, grid, lb, (n_quads - lb + grid - 1u) / grid, tid & 63u,
+         (wid & 3u) | ((wid >> 3) << 2)};
+  // waves 0-3 and 8-11 build, 4-7 and 12-15 scan: two of each kind on every SIMD
+  if (((wid >> 2) & 1u) == 0u) {
+    k.run_builder();
+  } else if ((k.rw >> 2) == 0u) {
+    k.template run_scanner<0>();
+  } else {
+    k.template run_scanner<1>();
+  }
+}
+
+template <int NCH, int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER, bool IP>
+void launch_stream_instance(const scan_args& a, hipStream_t stream)
+{
+  auto kernel = scan_stream_kernel<NCH, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER, IP>;
+  // per instance: the whole LDS of a CU belongs to the one resident block
+  static const int attr_set = [&] {
+    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(kStreamLdsBytes)));
+    return 1;
+  }();
+  (void)attr_set;
+  uint32_t grid = uint32_t(device_cu_count());
+  if (a.n_pairs_dev == nullptr) {
+    const uint32_t n_quads = (a.n_pairs + kStreamPairs - 1) / kStreamPairs;
+    if (grid > n_quads) { grid = n_quads; }
+    if (grid == 0) { return; }
+  }
+  kernel<<<grid, kStreamThreads, kStreamLdsBytes, stream>>>(a);
+  CUVS_HIP_TRY(hipGetLastError());
+}
+
+template <int NCH, int PQ_LEN, bool PER_CLUSTER>
+bool launch_stream_types(const scan_args& a, hipStream_t s)
+{
+  const bool ip = a.metric == int(DistanceType::InnerProduct) || a.metric == int(DistanceType::CosineExpanded);
+  if (!ip) {
+    if (!a.out_half) {
+      if (a.lut_dtype == CUDA_R_16F) { launch_stream_instance<NCH, PQ_LEN, LUT_F16, false, PER_CLUSTER, false>(a, s); return true; }
+      if (a.lut_dtype == CUDA_R_8U) { launch_stream_instance<NCH, PQ_LEN, LUT_FP8U, false, PER_CLUSTER, false>(a, s); return true; }
+    } else {
+      if (a.lut_dtype == CUDA_R_16F) { launch_stream_instance<NCH, PQ_LEN, LUT_F16, true, PER_CLUSTER, false>(a, s); return true; }
+      if (a.lut_dtype == CUDA_R_8U) { launch_stream_instance<NCH, PQ_LEN, LUT_FP8U, true, PER_CLUSTER, false>(a, s); return true; }
+    }
+  } else {
+    if (!a.out_half) {
+      if (a.lut_dtype == CUDA_R_16F) { launch_stream_instance<NCH, PQ_LEN, LUT_F16, false, PER_CLUSTER, true>(a, s); return true; }
+      if (a.lut_dtype == CUDA_R_8U) { launch_stream_instance<NCH, PQ_LEN, LUT_FP8S, false, PER_CLUSTER, true>(a, s); return true; }
+    } else {
+      if (a.lut_dtype == CUDA_R_16F) { launch_stream_instance<NCH, PQ_LEN, LUT_F16, true, PER_CLUSTER, true>(a, s); return true; }
+      if (a.lut_dtype == CUDA_R_8U) { launch_stream_instance<NCH, PQ_LEN, LUT_FP8S, true, PER_CLUSTER, true>(a, s); return true; }
+    }
+  }
+  return false;
+}
+
+template <int NCH, int PQ_LEN>
+bool launch_stream_kind(const scan_args& a, hipStream_t s)
+{
+  return a.per_cluster ? launch_stream_types<NCH, PQ_LEN, true>(a, s) : launch_stream_types<NCH, PQ_LEN, false>(a, s);
+}
+
+}  // namespace
+
+uint32_t scan_stream_keys_per_pair(const scan_args& a)
+{
+  if (!a.fused || a.pq_bits != 8 || a.k > kStreamMaxK) { return 0; }
+  if (a.rot_dim != a.pq_dim * a.pq_len) { return 0; }
+  if (a.lut_dtype != CUDA_R_16F && a.lut_dtype != CUDA_R_8U) { return 0; }
+  const bool shape = (a.pq_dim == 64 && a.pq_len == 2) || (a.pq_dim == 48 && a.pq_len == 2) ||
+                     (a.pq_dim == 32 && a.pq_len == 4);
+  return shape ? kStreamWG * a.k : 0;
+}
+
+bool launch_scan_stream(const scan_args& a, hipStream_t stream)
+{
+  if (scan_stream_keys_per_pair(a) == 0 || a.n_queries == 0 || a.desc == nullptr) { return false; }
+  if (a.pq_dim == 64 && a.pq_len == 2) { return launch_stream_kind<4, 2>(a, stream); }
+  if (a.pq_dim == 48 && a.pq_len == 2) { return launch_stream_kind<3, 2>(a, stream); }
+  if (a.pq_dim == 32 && a.pq_len == 4) { return launch_stream_kind<2, 4>(a, stream); }
+  return false;
+}
+
+}  // namespace cuvs::neighbors::ivf_pq::detail

@@ -412,7 +412,7 @@ void search(cuvs::resources const& res_c,
   sa.fused                 = pl.fused;
   if (global_lut) { sa.global_lut = res.workspace_alloc(global_lut_bytes); }
   const bool generic_only  = res.tuning.generic_scan || global_lut;
-  const uint32_t quad_kpp  = generic_only ? 0u : detail::scan_quad_keys_per_pair(sa);
+  const uint32_t quad_kpp  = generic_only ? 0u : detail::scan_stream_keys_per_pair(sa);
   const bool nibble_scan   = !generic_only && detail::scan_nibble_supported(sa);
   const bool fast_scan     = !generic_only && (quad_kpp != 0 || detail::scan_fast_supported(sa) || nibble_scan);
   const uint32_t kpp       = quad_kpp != 0 ? quad_kpp : k;  // candidate keys stored per pair
@@ -502,7 +502,7 @@ void search(cuvs::resources const& res_c,
     if (early_stop) {
       // 1. the leading probes' lists in full: candidates and a first bound per query
       auto full_scan = [&] {
-        return quad_kpp != 0 ? detail::launch_scan_quad(sa, s) : detail::launch_scan_fast(sa, s);
+        return quad_kpp != 0 ? detail::launch_scan_stream(sa, s) : detail::launch_scan_fast(sa, s);
       };
       sa.n_pairs = nq * lead;
       CUVS_EXPECTS(full_scan(), "scan kernel launch failed");
@@ -519,7 +519,7 @@ void search(cuvs::resources const& res_c,
       sa.n_pairs_dev = n_survivors;
       CUVS_EXPECTS(full_scan(), "scan kernel launch failed");
     } else {
-      const bool launched = fast_scan && (quad_kpp != 0   ? detail::launch_scan_quad(sa, s)
+      const bool launched = fast_scan && (quad_kpp != 0   ? detail::launch_scan_stream(sa, s)
                                           : nibble_scan ? detail::launch_scan_nibble(sa, s)
                                                         : detail::launch_scan_fast(sa, s));
       if (!launched) { detail::launch_scan(sa, s); }
