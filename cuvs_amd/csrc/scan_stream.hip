@@ -11,8 +11,9 @@
  *     barrier per iteration is the only synchronisation.  On every SIMD two waves of each kind
  *     share the issue slots, so the vector work of the table build fills the cycles in which the
  *     scanners wait for their LDS gathers and code loads;
- *   - a builder thread owns one codebook entry of half the subspaces and keeps those codebook
- *     components in registers for the whole kernel (the scanners spend their registers on code
+ *   - a builder thread owns two neighbouring codebook entries of a quarter of the subspaces and keeps
+ *     those codebook components in registers for the whole kernel; the two table entries of a
+ *     subspace go out as one 32-bit write (the scanners spend their registers on code
  *     tiles instead: the two roles are separate loops, so neither pays for the other's state);
  *   - every table entry is stored as a binary16 number in the form the scan adds: the entry itself
  *     for fp16 tables; for 8-bit tables the decoded value decode(encode(score)), which the reference
@@ -202,7 +203,6 @@ struct stream_kernel {
   using traits = lut_traits<LUT>;
   using acc_t  = typename std::conditional<OUT_HALF, _Float16, float>::type;
   static constexpr int M              = NCH * 16;  // pq_dim
-  static constexpr int HALFM          = M / 2;     // subspaces whose codebook a builder thread holds
   static constexpr uint32_t ROT       = uint32_t(M) * PQ_LEN;
   static constexpr uint32_t n_diff    = ROT * (IP ? 2u : 1u);
   static constexpr uint32_t G         = kStreamPairs;
@@ -265,64 +265,87 @@ struct stream_kernel {
 
   struct staged {
     float q, c;
-    float cb[PER_CLUSTER ? G : 1][PQ_LEN];  // per-cluster codebook components of the builder's entry
+    float cb[PER_CLUSTER ? G : 1][PQ_LEN][2];  // per-cluster codebook components of the builder's two entries
     bool live[G];
   };
 
-  /** ds_write_b16 at addr + IMM. */
+  /** ds_write_b32 at addr + IMM: the entries of two neighbouring codes of one subspace. */
   template <int IMM>
-  __device__ __forceinline__ static void entry_write(uint32_t addr, uint32_t bits16)
+  __device__ __forceinline__ static void entries_write(uint32_t addr, uint32_t two_entries)
   {
     static_assert(IMM >= 0 && IMM < 65536, "the write's offset field has 16 bits");
-    asm volatile("ds_write_b16 %0, %1 offset:%2" : : "v"(addr), "v"(bits16), "n"(IMM) : "memory");
+    asm volatile("ds_write_b32 %0, %1 offset:%2" : : "v"(addr), "v"(two_entries), "n"(IMM) : "memory");
+  }
+
+  /** The entries of two scores side by side, the first in the low half. */
+  __device__ __forceinline__ static uint32_t pack_entries(float s0, float s1)
+  {
+    if constexpr (LUT == LUT_F16) {
+      // One rounding of each fp32 score to binary16.  The registers are made opaque first: the
+      // compiler would otherwise fold the last multiply-add of a score into the conversion, which
+      // rounds the exact product sum once instead of twice and changes values.
+      asm volatile("" : "+v"(s0), "+v"(s1));
+      typedef float f32x2 __attribute__((ext_vector_type(2)));
+      typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+      const f16x2 h = __builtin_convertvector(f32x2{s0, s1}, f16x2);
+      return __builtin_bit_cast(uint32_t, h);
+    } else {
+      return uint32_t(table_entry<LUT, OUT_HALF>(s0)) | (uint32_t(table_entry<LUT, OUT_HALF>(s1)) << 16);
+    }
   }
 
   static constexpr int TERMS   = IP ? 2 : 1;
   static constexpr int FPS     = PQ_LEN * TERMS;  // staged floats per subspace
-  static constexpr int GROUP   = 16 / FPS;        // subspaces whose terms make four 16-byte reads
-  static constexpr int NGROUPS = HALFM / GROUP;
-  static_assert(GROUP >= 1 && HALFM % GROUP == 0, "the subspaces of a builder thread split into whole groups");
+  static constexpr int QM      = M / 4;           // subspaces of a builder thread
+  static constexpr int GROUP   = 8 / FPS;         // subspaces whose terms make two 16-byte reads
+  static constexpr int NGROUPS = QM / GROUP;
+  static_assert(GROUP >= 1 && QM % GROUP == 0, "the subspaces of a builder thread split into whole groups");
 
-  /** Entries of subspaces first .. first + GROUP - 1 of the thread's half from their 16 staged floats. */
+  /** Entries of subspaces gi * GROUP .. + GROUP - 1 of the thread's quarter, for its two codes, from
+   *  the subspaces' 8 staged floats. */
   template <int gi, int u = 0>
-  __device__ __forceinline__ static void build_group(const float (&term)[16], const float (&book)[PER_CLUSTER ? 1 : HALFM][PQ_LEN],
-                                                     const float (&cb)[PQ_LEN], uint32_t waddr)
+  __device__ __forceinline__ static void build_group(const float (&term)[8],
+                                                     const float (&book)[PER_CLUSTER ? 1 : QM][PQ_LEN][2],
+                                                     const float (&cb)[PQ_LEN][2], uint32_t waddr)
   {
     if constexpr (u < GROUP) {
       constexpr int jj = gi * GROUP + u;
-      float score      = 0.0f;
+      float score[2]   = {0.0f, 0.0f};
 #pragma unroll
-      for (int t = 0; t < PQ_LEN; t++) {
-        const float pqc = PER_CLUSTER ? cb[t] : book[PER_CLUSTER ? 0 : jj][t];
-        if constexpr (!IP) {
-          float df = term[u * FPS + t];
-          df -= pqc;
-          score = fmaf(df, df, score);
-        } else {
-          const float qv = term[u * FPS + 2 * t];
-          score -= term[u * FPS + 2 * t + 1];
-          score = fmaf(-qv, pqc, score);
+      for (int e = 0; e < 2; e++) {
+#pragma unroll
+        for (int t = 0; t < PQ_LEN; t++) {
+          const float pqc = PER_CLUSTER ? cb[t][e] : book[PER_CLUSTER ? 0 : jj][t][e];
+          if constexpr (!IP) {
+            float df = term[u * FPS + t];
+            df -= pqc;
+            score[e] = fmaf(df, df, score[e]);
+          } else {
+            const float qv = term[u * FPS + 2 * t];
+            score[e] -= term[u * FPS + 2 * t + 1];
+            score[e] = fmaf(-qv, pqc, score[e]);
+          }
         }
       }
-      entry_write<jj * 512>(waddr, table_entry<LUT, OUT_HALF>(score));
+      entries_write<jj * 512>(waddr, pack_entries(score[0], score[1]));
       build_group<gi, u + 1>(term, book, cb, waddr);
     }
   }
 
   template <int gi>
-  __device__ __forceinline__ static void build_groups(const LDS_AS f32x4* terms, f32x4 (&cur4)[4],
-                                                      const float (&book)[PER_CLUSTER ? 1 : HALFM][PQ_LEN],
-                                                      const float (&cb)[PQ_LEN], uint32_t waddr)
+  __device__ __forceinline__ static void build_groups(const LDS_AS f32x4* terms, f32x4 (&cur4)[2],
+                                                      const float (&book)[PER_CLUSTER ? 1 : QM][PQ_LEN][2],
+                                                      const float (&cb)[PQ_LEN][2], uint32_t waddr)
   {
     // the next group's terms are requested before this group is computed
-    f32x4 nxt4[4];
+    f32x4 nxt4[2];
     if constexpr (gi + 1 < NGROUPS) {
 #pragma unroll
-      for (int x = 0; x < 4; x++) { nxt4[x] = terms[(gi + 1) * 4 + x]; }
+      for (int x = 0; x < 2; x++) { nxt4[x] = terms[(gi + 1) * 2 + x]; }
     }
-    float term[16];
+    float term[8];
 #pragma unroll
-    for (int x = 0; x < 4; x++) {
+    for (int x = 0; x < 2; x++) {
       term[4 * x + 0] = cur4[x].x;
       term[4 * x + 1] = cur4[x].y;
       term[4 * x + 2] = cur4[x].z;
@@ -331,27 +354,32 @@ struct stream_kernel {
     build_group<gi>(term, book, cb, waddr);
     if constexpr (gi + 1 < NGROUPS) {
 #pragma unroll
-      for (int x = 0; x < 4; x++) { cur4[x] = nxt4[x]; }
+      for (int x = 0; x < 2; x++) { cur4[x] = nxt4[x]; }
       build_groups<gi + 1>(terms, cur4, book, cb, waddr);
     }
   }
 
   __device__ __forceinline__ void run_builder() const
   {
-    const uint32_t bt   = rw * 64u + lane;  // 0..511
-    const uint32_t code = bt & 255u;
-    const uint32_t half = rw >> 2;          // wave-uniform
-    float book[PER_CLUSTER ? 1 : HALFM][PQ_LEN];
+    // a builder thread owns two neighbouring codebook entries (their table entries share a dword)
+    // of a quarter of the subspaces: the staged terms of a subspace serve both
+    const uint32_t bt      = rw * 64u + lane;  // 0..511
+    const uint32_t code    = (bt & 127u) * 2u;
+    const uint32_t quarter = rw >> 1;          // wave-uniform
+    float book[PER_CLUSTER ? 1 : QM][PQ_LEN][2];
     if constexpr (!PER_CLUSTER) {
 #pragma unroll
-      for (int jj = 0; jj < HALFM; jj++) {
+      for (int jj = 0; jj < QM; jj++) {
 #pragma unroll
         for (int t = 0; t < PQ_LEN; t++) {
-          book[jj][t] = a.pq_centers[((half * HALFM + jj) * PQ_LEN + t) * 256 + code];
+          const float2 two = *reinterpret_cast<const float2*>(
+            a.pq_centers + ((quarter * QM + jj) * PQ_LEN + t) * 256 + code);
+          book[jj][t][0] = two.x;
+          book[jj][t][1] = two.y;
         }
       }
     } else {
-      book[0][0] = 0.0f;
+      book[0][0][0] = 0.0f;
     }
     // operands of the pairs in `info`: the staging element (pair bt / ROT, dimension bt % ROT) and,
     // for per-cluster codebooks, this thread's components of both pairs' codebooks
@@ -374,7 +402,12 @@ struct stream_kernel {
         for (uint32_t g = 0; g < G; g++) {
 #pragma unroll
           for (int t = 0; t < PQ_LEN; t++) {
-            f.cb[g][t] = info.n_rows[g] != 0 ? a.pq_centers[(uint64_t(info.label[g]) * PQ_LEN + t) * 256 + code] : 0.0f;
+            float2 two = make_float2(0.0f, 0.0f);
+            if (info.n_rows[g] != 0) {
+              two = *reinterpret_cast<const float2*>(a.pq_centers + (uint64_t(info.label[g]) * PQ_LEN + t) * 256 + code);
+            }
+            f.cb[g][t][0] = two.x;
+            f.cb[g][t][1] = two.y;
           }
         }
       }
@@ -398,12 +431,12 @@ struct stream_kernel {
       for (uint32_t g = 0; g < G; g++) {
         if (!f.live[g]) { continue; }  // uniform
         const auto* terms = reinterpret_cast<const LDS_AS f32x4*>(
-          uintptr_t(kStreamStageBase + (buffer * G + g) * kStreamStageSlot + half * uint32_t(HALFM * FPS) * 4u));
-        // entry (j, code) of the table at base + j * 512 + code * 2; j = half * HALFM + jj
-        const uint32_t waddr = stream_table_base(buffer, g) + half * uint32_t(HALFM) * 512u + code * 2u;
-        f32x4 cur4[4];
+          uintptr_t(kStreamStageBase + (buffer * G + g) * kStreamStageSlot + quarter * uint32_t(QM * FPS) * 4u));
+        // entry (j, code) of the table at base + j * 512 + code * 2; j = quarter * QM + jj
+        const uint32_t waddr = stream_table_base(buffer, g) + quarter * uint32_t(QM) * 512u + code * 2u;
+        f32x4 cur4[2];
 #pragma unroll
-        for (int x = 0; x < 4; x++) { cur4[x] = terms[x]; }
+        for (int x = 0; x < 2; x++) { cur4[x] = terms[x]; }
         build_groups<0>(terms, cur4, book, f.cb[PER_CLUSTER ? g : 0], waddr);
       }
     };
