@@ -45,21 +45,19 @@ constexpr uint32_t kStreamScanners = 8;  // scanner waves (and as many builder w
 constexpr uint32_t kStreamWG       = kStreamScanners / kStreamPairs;  // scanner waves per pair
 constexpr uint32_t kStreamMaxK     = 128;
 
-/* LDS map (bytes).  The four tables sit at multiples of 32 KB so that a table's address splits
+/* LDS map (bytes).  The two tables sit at multiples of 32 KB so that a table's address splits
  * into a 64 KB window (high half of the address register) and an immediate offset below 64 K:
- *   table of (buffer b, pair 0) at 0x08000 + b * 0x10000, of (b, pair 1) at 0x10000 + b * 0x10000. */
-constexpr uint32_t kStreamLdsBytes  = 160 * 1024;
+ *   table of pair 0 at 0x08000, of pair 1 at 0x10000. */
+constexpr uint32_t kStreamLdsBytes  = 0x18000;
 constexpr uint32_t kStreamStageBase = 16;               // 2 buffers x 2 pairs x 256 floats
 constexpr uint32_t kStreamStageSlot = 256 * 4;          // bytes per (buffer, pair)
 constexpr uint32_t kStreamCandBase  = 16 + 4 * kStreamStageSlot;
-__host__ __device__ constexpr uint32_t stream_table_base(uint32_t buffer, uint32_t g)
-{
-  return (g == 0 ? 0x08000u : 0x10000u) + buffer * 0x10000u;
-}
+__host__ __device__ constexpr uint32_t stream_table_base(uint32_t g) { return g == 0 ? 0x08000u : 0x10000u; }
 
 /** Candidate keys a wave buffers: room for k kept ones plus one tile of 64 new ones. */
 inline __host__ __device__ uint32_t stream_wave_cap(uint32_t k) { return k <= 64u ? 128u : 192u; }
-static_assert(kStreamCandBase + kStreamScanners * 192u * 8u <= 0x08000u, "small buffers must end below the tables");
+static_assert(kStreamCandBase % 8u == 0u && kStreamCandBase + kStreamScanners * 192u * 8u <= 0x08000u,
+              "small buffers must end below the tables");
 
 __device__ __forceinline__ void block_barrier()
 {
@@ -75,42 +73,123 @@ __device__ __forceinline__ float opaque_float(float v)
   return v;
 }
 
-/** Ascending sort of the first `cap` keys (at most 256) of one wave's buffer: a bitonic network made of
- *  ascending comparators only (each merge starts with a mirror step), run on the next power of two
- *  with the missing top slots standing for keys larger than any other - a comparator that would
- *  touch one of them never swaps, so it is skipped.  LDS operations of a wave execute in program
- *  order, so no barrier is needed. */
-__device__ __forceinline__ void wave_sort_keys(LDS_AS unsigned long long* buf, uint32_t lane, uint32_t cap)
+/** Largest value of the wave (unsigned; lanes that take no part pass 0): prefix maxima inside the
+ *  rows of 16 lanes, then across the rows; lane 63 ends up with the result. */
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v)
 {
-  const uint32_t n_half = cap <= 2u ? 1u : (1u << (31 - __builtin_clz(cap - 1u)));
-  auto compare_exchange = [&](uint32_t i, uint32_t l) __attribute__((always_inline)) {
-    if (l < cap) {
-      const unsigned long long x = buf[i];
-      const unsigned long long y = buf[l];
-      if (x > y) {
-        buf[i] = y;
-        buf[l] = x;
-      }
-    }
+  auto step = [&](auto ctrl, auto rows) {
+    const uint32_t other = uint32_t(__builtin_amdgcn_update_dpp(0, int(v), decltype(ctrl)::value, decltype(rows)::value, 0xf, false));
+    v                    = other > v ? other : v;
   };
+  step(std::integral_constant<int, 0x111>{}, std::integral_constant<int, 0xf>{});  // row_shr:1
+  step(std::integral_constant<int, 0x112>{}, std::integral_constant<int, 0xf>{});  // row_shr:2
+  step(std::integral_constant<int, 0x114>{}, std::integral_constant<int, 0xf>{});  // row_shr:4
+  step(std::integral_constant<int, 0x118>{}, std::integral_constant<int, 0xf>{});  // row_shr:8
+  step(std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xa>{});  // row_bcast:15 into rows 1, 3
+  step(std::integral_constant<int, 0x143>{}, std::integral_constant<int, 0xc>{});  // row_bcast:31 into rows 2, 3
+  return uint32_t(__builtin_amdgcn_readlane(int(v), 63));
+}
+
+/** Binary radix selection of the r smallest (r >= 1) of the wave's values value[j] of the lanes in
+ *  live[j], which are at least r, from bit `top` down (all the values agree above it and `prefix`
+ *  holds those bits).  Ballots and counts only: the state is scalar and nothing goes through LDS.
+ *  Ends as soon as a group of exactly the right size is split off: then the r smallest are the
+ *  values v with (v >> bit) <= (prefix >> bit) for the returned bit.  Otherwise returns -1 and
+ *  prefix is the r-th smallest value itself (which may occur several times). */
+template <int NK>
+__device__ __forceinline__ int wave_radix_select(const uint32_t (&value)[NK], const unsigned long long (&live)[NK],
+                                                 uint32_t r, int top, uint32_t& prefix)
+{
 #pragma unroll 1
-  for (uint32_t size = 2; size <= 2u * n_half; size <<= 1) {
-    const uint32_t half = size >> 1;
-    for (uint32_t c = lane; c < n_half; c += 64u) {
-      const uint32_t base = (c / half) * size;
-      const uint32_t off  = c & (half - 1u);
-      compare_exchange(base + off, base + size - 1u - off);
+  for (int bit = top; bit >= 0; bit--) {
+    // values that share the decided bits and have a zero at `bit`
+    uint32_t zeros = 0;
+#pragma unroll
+    for (int j = 0; j < NK; j++) {
+      zeros += uint32_t(__popcll(__builtin_amdgcn_ballot_w64((value[j] >> bit) == (prefix >> bit)) & live[j]));
     }
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll 1
-    for (uint32_t stride = size >> 2; stride > 0; stride >>= 1) {
-      for (uint32_t c = lane; c < n_half; c += 64u) {
-        const uint32_t i = (c / stride) * (2u * stride) + (c & (stride - 1u));
-        compare_exchange(i, i + stride);
-      }
-      __builtin_amdgcn_wave_barrier();
+    if (zeros == r) { return bit; }
+    if (zeros < r) {
+      r -= zeros;
+      prefix |= 1u << bit;
     }
   }
+  return -1;
+}
+
+/** Keeps the k smallest of the first n >= k keys (n <= 64 * NK) of one wave's buffer, in buf[0 .. k)
+ *  in no particular order, and returns the high word of the k-th smallest.  Keys are distinct (the
+ *  low word numbers the sample); among equal high words the smaller low words win, as in a sort of
+ *  the whole keys.  The keys sit in registers while the selection runs; LDS operations of a wave
+ *  execute in program order, so the compacting writes come after every read. */
+template <int NK>
+__device__ __forceinline__ uint32_t wave_select_keys(LDS_AS unsigned long long* buf, uint32_t lane, uint32_t n, uint32_t k)
+{
+  unsigned long long key[NK], live[NK];
+  uint32_t hi[NK], lo[NK];
+#pragma unroll
+  for (int j = 0; j < NK; j++) {
+    const bool in = uint32_t(j) * 64u + lane < n;
+    live[j]       = __builtin_amdgcn_ballot_w64(in);
+    key[j]        = in ? buf[uint32_t(j) * 64u + lane] : 0ull;
+    hi[j]         = uint32_t(key[j] >> 32);
+    lo[j]         = uint32_t(key[j]);
+  }
+  // the bits in which the high words differ at all: scores of one pair share their leading bits
+  const uint32_t first = uint32_t(__builtin_amdgcn_readfirstlane(int(hi[0])));  // lane 0 holds a key: n >= 1
+  uint32_t differ      = 0;
+#pragma unroll
+  for (int j = 0; j < NK; j++) { differ |= uint32_t(j) * 64u + lane < n ? hi[j] ^ first : 0u; }
+  int top = -1;  // highest bit set in any lane's `differ`
+  if (__builtin_amdgcn_ballot_w64(differ != 0u) != 0ull) {
+    top = 0;
+#pragma unroll
+    for (int s = 16; s >= 1; s >>= 1) {
+      if (__builtin_amdgcn_ballot_w64((differ >> (top + s)) != 0u) != 0ull) { top += s; }
+    }
+  }
+  uint32_t kth  = top >= 0 ? (first >> top >> 1 << top << 1) : first;  // the common bits
+  const int cut = wave_radix_select<NK>(hi, live, k, top, kth);
+  bool keep[NK];
+  if (cut >= 0) {
+    // exactly k keys lie at or below the group that was split off; its largest is the k-th
+    uint32_t largest = 0;
+#pragma unroll
+    for (int j = 0; j < NK; j++) {
+      keep[j] = uint32_t(j) * 64u + lane < n && (hi[j] >> cut) <= (kth >> cut);
+      largest = keep[j] && hi[j] > largest ? hi[j] : largest;
+    }
+    kth = wave_max_u32(largest);
+  } else {
+    uint32_t less = 0, ties = 0;
+    unsigned long long tied[NK];
+#pragma unroll
+    for (int j = 0; j < NK; j++) {
+      tied[j] = __builtin_amdgcn_ballot_w64(hi[j] == kth) & live[j];
+      less += uint32_t(__popcll(__builtin_amdgcn_ballot_w64(hi[j] < kth) & live[j]));
+      ties += uint32_t(__popcll(tied[j]));
+    }
+    // of the keys whose high word is kth, those with low words up to here are kept
+    uint32_t last_low = 0xFFFFFFFFu;
+    if (less + ties > k) {
+      last_low      = 0;
+      const int at  = wave_radix_select<NK>(lo, tied, k - less, 31, last_low);
+      if (at >= 0) { last_low |= (1u << at) - 1u; }  // every low word of the group that was split off
+    }
+#pragma unroll
+    for (int j = 0; j < NK; j++) {
+      keep[j] = uint32_t(j) * 64u + lane < n && (hi[j] < kth || (hi[j] == kth && lo[j] <= last_low));
+    }
+  }
+  uint32_t base = 0;
+#pragma unroll
+  for (int j = 0; j < NK; j++) {
+    const unsigned long long mask = __builtin_amdgcn_ballot_w64(keep[j]);
+    const uint32_t below = __builtin_amdgcn_mbcnt_hi(uint32_t(mask >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(mask), 0u));
+    if (keep[j]) { buf[base + below] = key[j]; }
+    base += uint32_t(__popcll(mask));
+  }
+  return kth;
 }
 
 /** The 16 bits stored for a table entry (see the file comment). */
@@ -231,6 +310,14 @@ struct stream_kernel {
   }
   __device__ __forceinline__ uint32_t quad_of(uint32_t it) const { return lb + it * grid; }
 
+  /** The k best of the n >= k keys in a wave's buffer; as narrow as the keys allow. */
+  __device__ __forceinline__ uint32_t select_keys(LDS_AS unsigned long long* buf, uint32_t n) const
+  {
+    if (n <= 64u) { return wave_select_keys<1>(buf, lane, n, a.k); }
+    if (n <= 128u) { return wave_select_keys<2>(buf, lane, n, a.k); }
+    return wave_select_keys<3>(buf, lane, n, a.k);
+  }
+
   /* ------------------------------------ builders ------------------------------------ */
 
   /** What the builders need to know about the two pairs of an iteration: which query and list
@@ -306,7 +393,7 @@ struct stream_kernel {
   template <int gi, int u = 0>
   __device__ __forceinline__ static void build_group(const float (&term)[8],
                                                      const float (&book)[PER_CLUSTER ? 1 : QM][PQ_LEN][2],
-                                                     const float (&cb)[PQ_LEN][2], uint32_t waddr)
+                                                     const float (&cb)[PQ_LEN][2], uint32_t (&entries)[QM])
   {
     if constexpr (u < GROUP) {
       constexpr int jj = gi * GROUP + u;
@@ -327,15 +414,15 @@ struct stream_kernel {
           }
         }
       }
-      entries_write<jj * 512>(waddr, pack_entries(score[0], score[1]));
-      build_group<gi, u + 1>(term, book, cb, waddr);
+      entries[jj] = pack_entries(score[0], score[1]);
+      build_group<gi, u + 1>(term, book, cb, entries);
     }
   }
 
   template <int gi>
   __device__ __forceinline__ static void build_groups(const LDS_AS f32x4* terms, f32x4 (&cur4)[2],
                                                       const float (&book)[PER_CLUSTER ? 1 : QM][PQ_LEN][2],
-                                                      const float (&cb)[PQ_LEN][2], uint32_t waddr)
+                                                      const float (&cb)[PQ_LEN][2], uint32_t (&entries)[QM])
   {
     // the next group's terms are requested before this group is computed
     f32x4 nxt4[2];
@@ -351,11 +438,21 @@ struct stream_kernel {
       term[4 * x + 2] = cur4[x].z;
       term[4 * x + 3] = cur4[x].w;
     }
-    build_group<gi>(term, book, cb, waddr);
+    build_group<gi>(term, book, cb, entries);
     if constexpr (gi + 1 < NGROUPS) {
 #pragma unroll
       for (int x = 0; x < 2; x++) { cur4[x] = nxt4[x]; }
-      build_groups<gi + 1>(terms, cur4, book, cb, waddr);
+      build_groups<gi + 1>(terms, cur4, book, cb, entries);
+    }
+  }
+
+  /** The thread's entries of one table go to LDS: entry (j, code) at base + j * 512 + code * 2. */
+  template <int jj = 0>
+  __device__ __forceinline__ static void write_entries(uint32_t waddr, const uint32_t (&entries)[QM])
+  {
+    if constexpr (jj < QM) {
+      entries_write<jj * 512>(waddr, entries[jj]);
+      write_entries<jj + 1>(waddr, entries);
     }
   }
 
@@ -424,20 +521,29 @@ struct stream_kernel {
         }
       }
     };
-    // tables of iteration `it` from the terms staged in buffer it & 1
-    auto build = [&](uint32_t it, const staged& f) {
+    // the thread's table entries of iteration `it`, from the terms staged in buffer it & 1, into
+    // registers: nothing is written while the scanners gather
+    uint32_t entries[G][QM];
+    auto compute = [&](uint32_t it, const staged& f) {
       const uint32_t buffer = it & 1u;
 #pragma unroll
       for (uint32_t g = 0; g < G; g++) {
         if (!f.live[g]) { continue; }  // uniform
         const auto* terms = reinterpret_cast<const LDS_AS f32x4*>(
           uintptr_t(kStreamStageBase + (buffer * G + g) * kStreamStageSlot + quarter * uint32_t(QM * FPS) * 4u));
-        // entry (j, code) of the table at base + j * 512 + code * 2; j = quarter * QM + jj
-        const uint32_t waddr = stream_table_base(buffer, g) + quarter * uint32_t(QM) * 512u + code * 2u;
         f32x4 cur4[2];
 #pragma unroll
         for (int x = 0; x < 2; x++) { cur4[x] = terms[x]; }
-        build_groups<0>(terms, cur4, book, f.cb[PER_CLUSTER ? g : 0], waddr);
+        build_groups<0>(terms, cur4, book, f.cb[PER_CLUSTER ? g : 0], entries[g]);
+      }
+    };
+    // ... and from the registers into the tables, while no scanner reads
+    auto write_tables = [&](const staged& f) {
+#pragma unroll
+      for (uint32_t g = 0; g < G; g++) {
+        if (!f.live[g]) { continue; }  // uniform
+        // entry (j, code) of the table at base + j * 512 + code * 2; j = quarter * QM + jj
+        write_entries<0>(stream_table_base(g) + quarter * uint32_t(QM) * 512u + code * 2u, entries[g]);
       }
     };
 
@@ -449,8 +555,9 @@ struct stream_kernel {
     if (n_it > 1) { fetch(info_b, nxt_f); }
     info_a = load_info(2);  // always the records two iterations past the tables being built
     block_barrier();        // terms of iteration 0 visible
-    build(0, cur_f);
+    compute(0, cur_f);
     if (n_it > 1) { stage(1, nxt_f); }
+    write_tables(cur_f);
     block_barrier();  // tables of iteration 0 and terms of iteration 1 visible
     for (uint32_t it = 0; it < n_it; it++) {
       // the scanners are working on iteration `it`; nxt_f holds the operands of it + 1 (their terms
@@ -459,12 +566,14 @@ struct stream_kernel {
       const bool two_ahead = it + 2 < n_it;
       if (two_ahead) { fetch(info_a, after_f); }
       info_b = load_info(it + 3);
-      if (it + 1 < n_it) { build(it + 1, nxt_f); }
-      // buffer it & 1 was read by the build of iteration `it`, which is over
+      if (it + 1 < n_it) { compute(it + 1, nxt_f); }
+      block_barrier();  // the scanners are through with the tables of iteration `it`
+      if (it + 1 < n_it) { write_tables(nxt_f); }
+      // buffer it & 1 was read when the entries of iteration `it` were computed, which is over
       if (two_ahead) { stage(it & 1u, after_f); }
       nxt_f  = after_f;
       info_a = info_b;
-      block_barrier();
+      block_barrier();  // tables of iteration it + 1 and terms of iteration it + 2 visible
     }
   }
 
@@ -544,6 +653,9 @@ struct stream_kernel {
   __device__ __forceinline__ void run_scanner() const
   {
     constexpr int IMMG     = GI == 0 ? 0x8000 : 0;
+    // The scanners' instructions go first: their adds release the next lookups, and the LDS pipeline
+    // they feed is the scarcest resource; the builders' arithmetic fills the slots they leave.
+    __builtin_amdgcn_s_setprio(3);
     const uint32_t wig     = rw & 3u;
     const uint32_t sw      = rw;  // scanner wave 0..7
     const uint32_t cap     = stream_wave_cap(a.k);
@@ -565,9 +677,11 @@ struct stream_kernel {
     for (uint32_t it = 0; it < n_it; it++) {
       const bool has_next   = it + 1 < n_it;
       const pair_desc nxt_d = record(quad_of(has_next ? it + 1 : it), GI);
-      // window of this iteration's table in the high halves of the address registers
-      const uint32_t window = (((it & 1u) + (GI == 0 ? 0u : 1u)) << 16);
+      // window of the group's table in the high halves of the address registers
+      const uint32_t window = (GI == 0 ? 0u : 1u) << 16;
 
+      const pair_desc done_d = my_d;
+      uint32_t n_keys        = 0;
       if (my_d.slot != 0xFFFFFFFFu) {
         const uint32_t n_rows     = my_d.n_rows;
         const uint32_t sample_off = my_d.sample_off;
@@ -597,13 +711,10 @@ struct stream_kernel {
           const unsigned long long mask = __ballot(pass);
           if (mask != 0ull) {
             if (wcount + 64u > cap) {
-              // make room: keep the k best of the buffer and tighten the wave's bound
-              wave_sort_keys(my_cand, lane, wcount);
-              if (wcount >= a.k) {
-                wcount            = a.k;
-                const uint32_t t2 = uint32_t(my_cand[a.k - 1] >> 32);
-                thr               = t2 < thr ? t2 : thr;
-              }
+              // make room (the buffer holds more than k keys): keep the k best and tighten the wave's bound
+              const uint32_t t2 = select_keys(my_cand, wcount);
+              wcount            = a.k;
+              thr               = t2 < thr ? t2 : thr;
             }
             const bool pass2 = pass && okey <= thr;
             const unsigned long long mask2 = __ballot(pass2);
@@ -617,14 +728,7 @@ struct stream_kernel {
             for (int m = 0; m < NCH; m++) { cur[m] = ahead[m]; }
           }
         }
-        // this wave's best candidates of the pair
-        unsigned long long* out = a.out_keys + (uint64_t(my_d.slot) * WG + wig) * a.k;
-        if (wcount >= a.k) {
-          wave_sort_keys(my_cand, lane, wcount);  // only as wide as there are candidates
-          wcount = a.k;
-          if (lane == 0) { atomicMin(&a.query_kth[my_d.q], uint32_t(my_cand[a.k - 1] >> 32)); }
-        }
-        for (uint32_t t = lane; t < a.k; t += 64u) { out[t] = t < wcount ? my_cand[t] : kInvalidKey; }
+        n_keys = wcount;
       }
 
       // first tile and bound of the next pair: they arrive while the other waves finish
@@ -636,7 +740,19 @@ struct stream_kernel {
         }
         if (my_d.n_rows != 0) { pre_thr = a.query_kth[my_d.q]; }
       }
-      block_barrier();
+      block_barrier();  // every scanner is through with this iteration's tables
+      // While the builders write the next tables: this wave's best candidates of the pair go out,
+      // and their k-th bounds the query from now on.
+      if (done_d.slot != 0xFFFFFFFFu) {
+        unsigned long long* out = a.out_keys + (uint64_t(done_d.slot) * WG + wig) * a.k;
+        if (n_keys >= a.k) {
+          const uint32_t kth = select_keys(my_cand, n_keys);
+          n_keys             = a.k;
+          if (lane == 0) { atomicMin(&a.query_kth[done_d.q], kth); }
+        }
+        for (uint32_t t = lane; t < a.k; t += 64u) { out[t] = t < n_keys ? my_cand[t] : kInvalidKey; }
+      }
+      block_barrier();  // the builders have written the next ones
     }
   }
 };
