@@ -208,73 +208,115 @@ __device__ __forceinline__ uint16_t table_entry(float score)
   }
 }
 
-/* ---- the lookups, as inline assembly: the compiler would otherwise extract each byte, form a
- * full address and wait for every read ---- */
+/* ---- One tile of 64 rows, as a single block of assembly.  The compiler would extract each code
+ * byte, form a full address and wait for every read; and a lookup whose register is written some
+ * hundred cycles after the read was issued cannot be left to it piecewise (it treats the register as
+ * holding its value from the instruction that issued the read on, and may copy it at a branch).
+ *
+ * A lookup is two vector instructions: one sub-dword shift puts 2 * code into the low half of an
+ * address register whose high half holds the table's 64 KB window (the subspace's offset sits in
+ * the read's immediate field), and the entry that ds_read_u16 returns is added.  The lookups go in
+ * groups of eight (two code dwords); two groups are in flight while a third is added, so a wave
+ * always has reads queued.  After each chunk of sixteen subspaces but the last, an L2 scan ends the
+ * tile if no row in play can still beat the bound (sums only grow; early stop of compute_score in
+ * the reference): the group that is in flight then is awaited and dropped. ---- */
+#define ST_SDWA(a, c, sel)                                                                                   \
+  "v_lshlrev_b32_sdwa %[" #a "], %[one_u], %[" #c "] dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD " \
+  "src1_sel:BYTE_" #sel "\n\t"
+#define ST_READ(v, a, o, i) "ds_read_u16 %[" #v "], %[" #a "] offset:%[immg]+" #o "*4096+" #i "*512\n\t"
+/* group o: subspaces 8 o .. 8 o + 7, code dwords ca, cb, entries into V0 .. V7 */
+#define ST_ISSUE(o, ca, cb, V)                                                                     \
+  ST_SDWA(a0, ca, 0) ST_SDWA(a1, ca, 1) ST_SDWA(a2, ca, 2) ST_SDWA(a3, ca, 3)                      \
+  ST_SDWA(a4, cb, 0) ST_SDWA(a5, cb, 1) ST_SDWA(a6, cb, 2) ST_SDWA(a7, cb, 3)                      \
+  ST_READ(V##0, a0, o, 0) ST_READ(V##1, a1, o, 1) ST_READ(V##2, a2, o, 2) ST_READ(V##3, a3, o, 3)  \
+  ST_READ(V##4, a4, o, 4) ST_READ(V##5, a5, o, 5) ST_READ(V##6, a6, o, 6) ST_READ(V##7, a7, o, 7)
+#define ST_WAIT8 "s_waitcnt lgkmcnt(8)\n\t"
+#define ST_WAIT0 "s_waitcnt lgkmcnt(0)\n\t"
+/* fp32 sums: entry * scale + sum in one instruction that widens the binary16 entry (exact product) */
+#define ST_ADD_F32_1(v) "v_fma_mix_f32 %[acc], %[" #v "], %[one], %[acc] op_sel_hi:[1,0,0]\n\t"
+#define ST_ADD_F16_1(v) "v_add_f16_e32 %[acc], %[acc], %[" #v "]\n\t"
+#define ST_ADD8(ADD1, V) ADD1(V##0) ADD1(V##1) ADD1(V##2) ADD1(V##3) ADD1(V##4) ADD1(V##5) ADD1(V##6) ADD1(V##7)
+#define ST_ADD_F32(V) ST_ADD8(ST_ADD_F32_1, V)
+#define ST_ADD_F16(V) ST_ADD8(ST_ADD_F16_1, V)
+/* rows in play whose sum is not past the bound; none: leave */
+#define ST_CHECK_F32                                 \
+  "v_cmp_ge_u32_e32 vcc, %[stop], %[acc]\n\t"        \
+  "s_and_b64 %[tmp], vcc, %[valid]\n\t"              \
+  "s_cbranch_scc0 .Ltile_done%=\n\t"
+#define ST_CHECK_F16                                 \
+  "v_cvt_f32_f16_e32 %[chk], %[acc]\n\t"             \
+  "v_cmp_ge_u32_e32 vcc, %[stop], %[chk]\n\t"        \
+  "s_and_b64 %[tmp], vcc, %[valid]\n\t"              \
+  "s_cbranch_scc0 .Ltile_done%=\n\t"
+#define ST_NO_CHECK ""
+#define ST_HEAD                                                                                              \
+  "v_mov_b32 %[a0], %[window]\n\tv_mov_b32 %[a1], %[window]\n\tv_mov_b32 %[a2], %[window]\n\t"               \
+  "v_mov_b32 %[a3], %[window]\n\tv_mov_b32 %[a4], %[window]\n\tv_mov_b32 %[a5], %[window]\n\t"               \
+  "v_mov_b32 %[a6], %[window]\n\tv_mov_b32 %[a7], %[window]\n\tv_mov_b32 %[acc], 0\n\t"                      \
+  ST_ISSUE(0, c0, c1, va) ST_ISSUE(1, c2, c3, vb)
+/* a chunk that is not the last: its two groups are added, groups o + 2 and o + 3 issued */
+#define ST_CHUNK(o0, o1, o2, o3, c4, c5, c6, c7, ADD, CHECK)  \
+  ST_WAIT8 ADD(va) ST_ISSUE(o2, c4, c5, va)                   \
+  ST_WAIT8 ADD(vb) CHECK ST_ISSUE(o3, c6, c7, vb)
+#define ST_TAIL(ADD) ST_WAIT8 ADD(va) ST_WAIT0 ADD(vb) ".Ltile_done%=:\n\t" ST_WAIT0
+#define ST_BODY_2(ADD, CHECK) ST_HEAD ST_CHUNK(0, 1, 2, 3, c4, c5, c6, c7, ADD, CHECK) ST_TAIL(ADD)
+#define ST_BODY_3(ADD, CHECK) \
+  ST_HEAD ST_CHUNK(0, 1, 2, 3, c4, c5, c6, c7, ADD, CHECK) ST_CHUNK(2, 3, 4, 5, c8, c9, c10, c11, ADD, CHECK) ST_TAIL(ADD)
+#define ST_BODY_4(ADD, CHECK)                                                                                     \
+  ST_HEAD ST_CHUNK(0, 1, 2, 3, c4, c5, c6, c7, ADD, CHECK) ST_CHUNK(2, 3, 4, 5, c8, c9, c10, c11, ADD, CHECK)     \
+  ST_CHUNK(4, 5, 6, 7, c12, c13, c14, c15, ADD, CHECK) ST_TAIL(ADD)
 
-/** low half of `addr` = 2 * byte SEL of `w`; the high half is kept. */
-template <int SEL>
-__device__ __forceinline__ void code_offset(uint32_t& addr, uint32_t one, uint32_t w)
+#define ST_OUTPUTS                                                                                              \
+  [acc] "=&v"(acc), [chk] "=&v"(chk), [tmp] "=&s"(tmp), [a0] "=&v"(ad[0]), [a1] "=&v"(ad[1]), [a2] "=&v"(ad[2]), \
+    [a3] "=&v"(ad[3]), [a4] "=&v"(ad[4]), [a5] "=&v"(ad[5]), [a6] "=&v"(ad[6]), [a7] "=&v"(ad[7]),              \
+    [va0] "=&v"(va[0]), [va1] "=&v"(va[1]), [va2] "=&v"(va[2]), [va3] "=&v"(va[3]), [va4] "=&v"(va[4]),         \
+    [va5] "=&v"(va[5]), [va6] "=&v"(va[6]), [va7] "=&v"(va[7]), [vb0] "=&v"(vb[0]), [vb1] "=&v"(vb[1]),         \
+    [vb2] "=&v"(vb[2]), [vb3] "=&v"(vb[3]), [vb4] "=&v"(vb[4]), [vb5] "=&v"(vb[5]), [vb6] "=&v"(vb[6]),         \
+    [vb7] "=&v"(vb[7])
+#define ST_COMMON_INPUTS \
+  [one_u] "v"(one_u), [one] "v"(one), [stop] "s"(stop), [valid] "s"(valid), [immg] "n"(IMMG), [window] "n"(WINDOW)
+#define ST_CODES_2                                                                                              \
+  [c0] "v"(cur[0].x), [c1] "v"(cur[0].y), [c2] "v"(cur[0].z), [c3] "v"(cur[0].w), [c4] "v"(cur[1].x),           \
+    [c5] "v"(cur[1].y), [c6] "v"(cur[1].z), [c7] "v"(cur[1].w)
+#define ST_CODES_3 \
+  ST_CODES_2, [c8] "v"(cur[2].x), [c9] "v"(cur[2].y), [c10] "v"(cur[2].z), [c11] "v"(cur[2].w)
+#define ST_CODES_4 \
+  ST_CODES_3, [c12] "v"(cur[3].x), [c13] "v"(cur[3].y), [c14] "v"(cur[3].z), [c15] "v"(cur[3].w)
+
+/** Sum of the table entries of a tile's rows in subspace order, as the bits of a float (HALF: of a
+ *  binary16 number in the low half).  CHECK: end the tile when no row of `valid` has a sum whose
+ *  bits are at most `stop`.  IMMG: offset of the table inside its 64 KB window WINDOW (a multiple of
+ *  64 K); `one` is the factor of the entries (fp32 sums), one_u the integer 1. */
+template <int NCH, bool HALF, bool CHECK, int IMMG, int WINDOW>
+__device__ __forceinline__ uint32_t stream_tile_sum(const u32x4 (&cur)[NCH], uint32_t one_u, float one, uint32_t stop,
+                                                    unsigned long long valid)
 {
-  static_assert(SEL >= 0 && SEL < 4, "byte of a dword");
-  if constexpr (SEL == 0) {
-    asm volatile("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:BYTE_0"
-                 : "+v"(addr) : "v"(one), "v"(w));
-  } else if constexpr (SEL == 1) {
-    asm volatile("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:BYTE_1"
-                 : "+v"(addr) : "v"(one), "v"(w));
-  } else if constexpr (SEL == 2) {
-    asm volatile("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:BYTE_2"
-                 : "+v"(addr) : "v"(one), "v"(w));
-  } else {
-    asm volatile("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:BYTE_3"
-                 : "+v"(addr) : "v"(one), "v"(w));
+  static_assert(NCH >= 2 && NCH <= 4, "two to four chunks of sixteen subspaces");
+  static_assert(IMMG >= 0 && IMMG + (NCH * 16 - 1) * 512 < 65536, "the read's offset field has 16 bits");
+  uint32_t acc, chk, ad[8], va[8], vb[8];
+  unsigned long long tmp;
+#define ST_EMIT(BODY, ADD, CHK, ...) \
+  asm volatile(BODY(ADD, CHK) : ST_OUTPUTS : ST_COMMON_INPUTS, __VA_ARGS__ : "vcc", "scc", "memory")
+#define ST_EMIT_KIND(BODY, ...)                                              \
+  if constexpr (!HALF && CHECK) {                                            \
+    ST_EMIT(BODY, ST_ADD_F32, ST_CHECK_F32, __VA_ARGS__);                    \
+  } else if constexpr (!HALF && !CHECK) {                                    \
+    ST_EMIT(BODY, ST_ADD_F32, ST_NO_CHECK, __VA_ARGS__);                     \
+  } else if constexpr (HALF && CHECK) {                                      \
+    ST_EMIT(BODY, ST_ADD_F16, ST_CHECK_F16, __VA_ARGS__);                    \
+  } else {                                                                   \
+    ST_EMIT(BODY, ST_ADD_F16, ST_NO_CHECK, __VA_ARGS__);                     \
   }
-}
-
-/** Entry read: 16 bits, zero-extended. */
-template <int IMM>
-__device__ __forceinline__ void entry_read(uint32_t& val, uint32_t addr)
-{
-  static_assert(IMM >= 0 && IMM < 65536, "the read's offset field has 16 bits");
-  // an output only: a register that the compiler believed to hold a value before the read could be
-  // copied by it right after the read was issued, before the data is there
-  asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(val) : "v"(addr), "n"(IMM));
-}
-
-/** Issues the eight lookups of code words w0, w1 (subspaces J0 .. J0 + 7 of the tile's rows). */
-template <int IMM0>
-__device__ __forceinline__ void issue8(uint32_t w0, uint32_t w1, uint32_t one, uint32_t (&addr)[8], uint32_t (&val)[8])
-{
-  code_offset<0>(addr[0], one, w0);
-  code_offset<1>(addr[1], one, w0);
-  code_offset<2>(addr[2], one, w0);
-  code_offset<3>(addr[3], one, w0);
-  code_offset<0>(addr[4], one, w1);
-  code_offset<1>(addr[5], one, w1);
-  code_offset<2>(addr[6], one, w1);
-  code_offset<3>(addr[7], one, w1);
-  entry_read<IMM0 + 0 * 512>(val[0], addr[0]);
-  entry_read<IMM0 + 1 * 512>(val[1], addr[1]);
-  entry_read<IMM0 + 2 * 512>(val[2], addr[2]);
-  entry_read<IMM0 + 3 * 512>(val[3], addr[3]);
-  entry_read<IMM0 + 4 * 512>(val[4], addr[4]);
-  entry_read<IMM0 + 5 * 512>(val[5], addr[5]);
-  entry_read<IMM0 + 6 * 512>(val[6], addr[6]);
-  entry_read<IMM0 + 7 * 512>(val[7], addr[7]);
-}
-
-/** The eight reads issued into `val` have landed; MORE: eight younger ones may still be in flight
- *  (LDS reads return in order; other outstanding operations only make the wait longer). */
-template <bool MORE>
-__device__ __forceinline__ void landed8(uint32_t (&val)[8])
-{
-  if constexpr (MORE) {
-    asm volatile("s_waitcnt lgkmcnt(8)"
-                 : "+v"(val[0]), "+v"(val[1]), "+v"(val[2]), "+v"(val[3]), "+v"(val[4]), "+v"(val[5]), "+v"(val[6]), "+v"(val[7]));
+  if constexpr (NCH == 2) {
+    ST_EMIT_KIND(ST_BODY_2, ST_CODES_2)
+  } else if constexpr (NCH == 3) {
+    ST_EMIT_KIND(ST_BODY_3, ST_CODES_3)
   } else {
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(val[0]), "+v"(val[1]), "+v"(val[2]), "+v"(val[3]), "+v"(val[4]), "+v"(val[5]), "+v"(val[6]), "+v"(val[7]));
+    ST_EMIT_KIND(ST_BODY_4, ST_CODES_4)
   }
+#undef ST_EMIT_KIND
+#undef ST_EMIT
+  return acc;
 }
 
 template <int NCH, int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER, bool IP>
@@ -591,64 +633,6 @@ struct stream_kernel {
     for (int m = 0; m < NCH; m++) { dst[m] = ptr[m * 32]; }
   }
 
-  __device__ __forceinline__ static acc_t add8(acc_t acc, const uint32_t (&val)[8], float one)
-  {
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      if constexpr (OUT_HALF) {
-        acc = acc_t(acc + __builtin_bit_cast(_Float16, uint16_t(val[i])));
-      } else {
-        // `one` holds kEntryScale; the product is exact, so this is acc + value with one rounding
-        acc = fmaf(float(__builtin_bit_cast(_Float16, uint16_t(val[i]))), one, acc);
-      }
-    }
-    return acc;
-  }
-
-  /** Chunk m of a tile and, by recursion, the chunks after it.  The sixteen lookups of a chunk are
-   *  issued together and the first eight are added while the other eight arrive.  Between the issue
-   *  of a lookup and the wait for it there is straight-line code only: the registers the reads
-   *  write are values to the compiler from the moment of issue, and at a branch it may copy them.
-   *  For L2 metrics the wave stops after a chunk once every row is past `stop_bits` (sums only
-   *  grow; early stop of compute_score in the reference).  IMMG = offset of the wave's table inside
-   *  its 64 KB window. */
-  template <int IMMG, int m>
-  __device__ __forceinline__ static acc_t chunk_sum(acc_t acc, const u32x4 (&cur)[NCH], uint32_t one_u, float one,
-                                                    bool valid, uint32_t stop_bits, uint32_t (&addr)[8])
-  {
-    uint32_t va[8], vb[8];
-    issue8<IMMG + (m * 16) * 512>(cur[m].x, cur[m].y, one_u, addr, va);
-    issue8<IMMG + (m * 16 + 8) * 512>(cur[m].z, cur[m].w, one_u, addr, vb);
-    landed8<true>(va);
-    acc = add8(acc, va, one);
-    landed8<false>(vb);
-    acc = add8(acc, vb, one);
-    if constexpr (m + 1 < NCH) {
-      if constexpr (!IP) {
-        const bool live = __builtin_amdgcn_ballot_w64(valid && !(__float_as_uint(float(acc)) > stop_bits)) != 0ull;
-        if (!live) { return acc; }
-      }
-      return chunk_sum<IMMG, m + 1>(acc, cur, one_u, one, valid, stop_bits, addr);
-    } else {
-      return acc;
-    }
-  }
-
-  /** Sum of the tile's table entries in subspace order. */
-  template <int IMMG>
-  __device__ __forceinline__ static acc_t tile_sum(const u32x4 (&cur)[NCH], uint32_t one_u, float one, bool valid,
-                                                   uint32_t stop_bits, uint32_t window)
-  {
-    // address registers: the table's 64 KB window in the high halves, code offsets go to the low ones
-    uint32_t addr[8];
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      addr[i] = window;
-      asm volatile("" : "+v"(addr[i]));
-    }
-    return chunk_sum<IMMG, 0>(acc_t(0), cur, one_u, one, valid, stop_bits, addr);
-  }
-
   template <int GI>
   __device__ __forceinline__ void run_scanner() const
   {
@@ -677,9 +661,6 @@ struct stream_kernel {
     for (uint32_t it = 0; it < n_it; it++) {
       const bool has_next   = it + 1 < n_it;
       const pair_desc nxt_d = record(quad_of(has_next ? it + 1 : it), GI);
-      // window of the group's table in the high halves of the address registers
-      const uint32_t window = (GI == 0 ? 0u : 1u) << 16;
-
       const pair_desc done_d = my_d;
       uint32_t n_keys        = 0;
       if (my_d.slot != 0xFFFFFFFFu) {
@@ -701,8 +682,17 @@ struct stream_kernel {
             const int64_t id = reinterpret_cast<const GLOBAL_AS int64_t*>(reinterpret_cast<uintptr_t>(list_ids))[i];
             valid = id >= 0 && id < a.filter_nbits && ((a.filter_bits[id >> 5] >> (id & 31)) & 1u) != 0;
           }
-          const uint32_t stop_bits = thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u;
-          acc_t acc = tile_sum<IMMG>(cur, one_u, one, valid, stop_bits, window);
+          // sums are not negative: past the bound means past its bits
+          const uint32_t stop_bits =
+            uint32_t(__builtin_amdgcn_readfirstlane(int(thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u)));
+          const uint32_t sum_bits = stream_tile_sum<NCH, OUT_HALF, !IP, IMMG, (GI == 0 ? 0 : 1) << 16>(
+            cur, one_u, one, stop_bits, __builtin_amdgcn_ballot_w64(valid));
+          acc_t acc;
+          if constexpr (OUT_HALF) {
+            acc = __builtin_bit_cast(_Float16, uint16_t(sum_bits));
+          } else {
+            acc = __uint_as_float(sum_bits);
+          }
           if (a.metric == int(DistanceType::CosineExpanded)) { acc = acc_t(acc + acc_t(1)); }
           const float score_f = float(acc);
           if (score_f != score_f) { valid = false; }
