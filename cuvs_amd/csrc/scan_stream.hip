@@ -249,11 +249,7 @@ __device__ __forceinline__ uint16_t table_entry(float score)
   "s_and_b64 %[tmp], vcc, %[valid]\n\t"              \
   "s_cbranch_scc0 .Ltile_done%=\n\t"
 #define ST_NO_CHECK ""
-#define ST_HEAD                                                                                              \
-  "v_mov_b32 %[a0], %[window]\n\tv_mov_b32 %[a1], %[window]\n\tv_mov_b32 %[a2], %[window]\n\t"               \
-  "v_mov_b32 %[a3], %[window]\n\tv_mov_b32 %[a4], %[window]\n\tv_mov_b32 %[a5], %[window]\n\t"               \
-  "v_mov_b32 %[a6], %[window]\n\tv_mov_b32 %[a7], %[window]\n\tv_mov_b32 %[acc], 0\n\t"                      \
-  ST_ISSUE(0, c0, c1, va) ST_ISSUE(1, c2, c3, vb)
+#define ST_HEAD "v_mov_b32 %[acc], 0\n\t" ST_ISSUE(0, c0, c1, va) ST_ISSUE(1, c2, c3, vb)
 /* a chunk that is not the last: its two groups are added, groups o + 2 and o + 3 issued */
 #define ST_CHUNK(o0, o1, o2, o3, c4, c5, c6, c7, ADD, CHECK)  \
   ST_WAIT8 ADD(va) ST_ISSUE(o2, c4, c5, va)                   \
@@ -267,14 +263,14 @@ __device__ __forceinline__ uint16_t table_entry(float score)
   ST_CHUNK(4, 5, 6, 7, c12, c13, c14, c15, ADD, CHECK) ST_TAIL(ADD)
 
 #define ST_OUTPUTS                                                                                              \
-  [acc] "=&v"(acc), [chk] "=&v"(chk), [tmp] "=&s"(tmp), [a0] "=&v"(ad[0]), [a1] "=&v"(ad[1]), [a2] "=&v"(ad[2]), \
-    [a3] "=&v"(ad[3]), [a4] "=&v"(ad[4]), [a5] "=&v"(ad[5]), [a6] "=&v"(ad[6]), [a7] "=&v"(ad[7]),              \
+  [acc] "=&v"(acc), [chk] "=&v"(chk), [tmp] "=&s"(tmp), [a0] "+v"(ad[0]), [a1] "+v"(ad[1]), [a2] "+v"(ad[2]),    \
+    [a3] "+v"(ad[3]), [a4] "+v"(ad[4]), [a5] "+v"(ad[5]), [a6] "+v"(ad[6]), [a7] "+v"(ad[7]),                   \
     [va0] "=&v"(va[0]), [va1] "=&v"(va[1]), [va2] "=&v"(va[2]), [va3] "=&v"(va[3]), [va4] "=&v"(va[4]),         \
     [va5] "=&v"(va[5]), [va6] "=&v"(va[6]), [va7] "=&v"(va[7]), [vb0] "=&v"(vb[0]), [vb1] "=&v"(vb[1]),         \
     [vb2] "=&v"(vb[2]), [vb3] "=&v"(vb[3]), [vb4] "=&v"(vb[4]), [vb5] "=&v"(vb[5]), [vb6] "=&v"(vb[6]),         \
     [vb7] "=&v"(vb[7])
 #define ST_COMMON_INPUTS \
-  [one_u] "v"(one_u), [one] "v"(one), [stop] "s"(stop), [valid] "s"(valid), [immg] "n"(IMMG), [window] "n"(WINDOW)
+  [one_u] "v"(one_u), [one] "v"(one), [stop] "s"(stop), [valid] "s"(valid), [immg] "n"(IMMG)
 #define ST_CODES_2                                                                                              \
   [c0] "v"(cur[0].x), [c1] "v"(cur[0].y), [c2] "v"(cur[0].z), [c3] "v"(cur[0].w), [c4] "v"(cur[1].x),           \
     [c5] "v"(cur[1].y), [c6] "v"(cur[1].z), [c7] "v"(cur[1].w)
@@ -285,15 +281,16 @@ __device__ __forceinline__ uint16_t table_entry(float score)
 
 /** Sum of the table entries of a tile's rows in subspace order, as the bits of a float (HALF: of a
  *  binary16 number in the low half).  CHECK: end the tile when no row of `valid` has a sum whose
- *  bits are at most `stop`.  IMMG: offset of the table inside its 64 KB window WINDOW (a multiple of
- *  64 K); `one` is the factor of the entries (fp32 sums), one_u the integer 1. */
-template <int NCH, bool HALF, bool CHECK, int IMMG, int WINDOW>
-__device__ __forceinline__ uint32_t stream_tile_sum(const u32x4 (&cur)[NCH], uint32_t one_u, float one, uint32_t stop,
-                                                    unsigned long long valid)
+ *  bits are at most `stop`.  IMMG: offset of the table inside its 64 KB window, which the high
+ *  halves of the address registers `ad` name (the routine changes their low halves only); `one` is
+ *  the factor of the entries (fp32 sums), one_u the integer 1. */
+template <int NCH, bool HALF, bool CHECK, int IMMG>
+__device__ __forceinline__ uint32_t stream_tile_sum(const u32x4 (&cur)[NCH], uint32_t (&ad)[8], uint32_t one_u, float one,
+                                                    uint32_t stop, unsigned long long valid)
 {
   static_assert(NCH >= 2 && NCH <= 4, "two to four chunks of sixteen subspaces");
   static_assert(IMMG >= 0 && IMMG + (NCH * 16 - 1) * 512 < 65536, "the read's offset field has 16 bits");
-  uint32_t acc, chk, ad[8], va[8], vb[8];
+  uint32_t acc, chk, va[8], vb[8];
   unsigned long long tmp;
 #define ST_EMIT(BODY, ADD, CHK, ...) \
   asm volatile(BODY(ADD, CHK) : ST_OUTPUTS : ST_COMMON_INPUTS, __VA_ARGS__ : "vcc", "scc", "memory")
@@ -648,6 +645,14 @@ struct stream_kernel {
     uint32_t one_u         = 1u;
     asm volatile("" : "+v"(one_u));
 
+    // address registers of the lookups: the window of the group's table in the high halves
+    uint32_t addr[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      addr[i] = (GI == 0 ? 0u : 1u) << 16;
+      asm volatile("" : "+v"(addr[i]));
+    }
+
     pair_desc my_d = record(quad_of(0), GI);
     u32x4 cur[NCH], ahead[NCH];
     if (wig * 64u < my_d.n_rows) {
@@ -669,54 +674,62 @@ struct stream_kernel {
         const uint8_t* list_data  = my_d.data;
         const int64_t* list_ids   = a.filter_bits != nullptr && n_rows != 0 ? a.inds_ptrs[my_d.label] : nullptr;
         const uint32_t n_tiles    = (n_rows + 63u) >> 6;
-        uint32_t thr              = pre_thr;
-        uint32_t wcount           = 0;
-        for (uint32_t tile = wig; tile < n_tiles; tile += WG) {
+        // the wave's bound: a key, and the same as a score (no bound: +inf; NaN scores never pass)
+        uint32_t thr = uint32_t(__builtin_amdgcn_readfirstlane(int(pre_thr)));
+        float thr_f  = thr >= 0xFF800000u ? __uint_as_float(0x7F800000u) : unorder_f32(thr);
+        // sums of an L2 scan are not negative: past the bound means past its bits
+        uint32_t stop_bits = thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u;
+        uint32_t wcount    = 0;
+        const bool cosine  = a.metric == int(DistanceType::CosineExpanded);
+        // One tile: the codes in `now` are scanned while those of the wave's next tile arrive in `next`.
+        auto scan_tile = [&](uint32_t tile, const u32x4 (&now)[NCH], u32x4 (&next)[NCH]) {
           const uint32_t i = tile * 64u + lane;
-          if (tile + WG < n_tiles) {
-            const uint32_t in = i + WG * 64u;
-            load_tile(row_ptr(list_data, in < n_rows ? in : 0u), ahead);
-          }
+          // requested without a condition (past the end: row 0 again), so that the wait for `now`
+          // is known to leave exactly these loads in flight
+          const uint32_t in = i + WG * 64u;
+          load_tile(row_ptr(list_data, in < n_rows ? in : 0u), next);
           bool valid = i < n_rows;
-          if (valid && list_ids != nullptr) {
-            const int64_t id = reinterpret_cast<const GLOBAL_AS int64_t*>(reinterpret_cast<uintptr_t>(list_ids))[i];
-            valid = id >= 0 && id < a.filter_nbits && ((a.filter_bits[id >> 5] >> (id & 31)) & 1u) != 0;
+          if (list_ids != nullptr) {
+            if (valid) {
+              const int64_t id = reinterpret_cast<const GLOBAL_AS int64_t*>(reinterpret_cast<uintptr_t>(list_ids))[i];
+              valid = id >= 0 && id < a.filter_nbits && ((a.filter_bits[id >> 5] >> (id & 31)) & 1u) != 0;
+            }
           }
-          // sums are not negative: past the bound means past its bits
-          const uint32_t stop_bits =
-            uint32_t(__builtin_amdgcn_readfirstlane(int(thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u)));
-          const uint32_t sum_bits = stream_tile_sum<NCH, OUT_HALF, !IP, IMMG, (GI == 0 ? 0 : 1) << 16>(
-            cur, one_u, one, stop_bits, __builtin_amdgcn_ballot_w64(valid));
-          acc_t acc;
+          const unsigned long long in_play = __builtin_amdgcn_ballot_w64(valid);
+          const uint32_t sum_bits = stream_tile_sum<NCH, OUT_HALF, !IP, IMMG>(now, addr, one_u, one, stop_bits, in_play);
+          float score;
           if constexpr (OUT_HALF) {
-            acc = __builtin_bit_cast(_Float16, uint16_t(sum_bits));
+            score = float(__builtin_bit_cast(_Float16, uint16_t(sum_bits)));
+            if (cosine) { score = float(_Float16(__builtin_bit_cast(_Float16, uint16_t(sum_bits)) + _Float16(1))); }
           } else {
-            acc = __uint_as_float(sum_bits);
+            score = __uint_as_float(sum_bits);
+            if (cosine) { score += 1.0f; }
           }
-          if (a.metric == int(DistanceType::CosineExpanded)) { acc = acc_t(acc + acc_t(1)); }
-          const float score_f = float(acc);
-          if (score_f != score_f) { valid = false; }
-          const uint32_t okey = order_f32(score_f);
-          const bool pass     = valid && okey <= thr;
-          const unsigned long long mask = __ballot(pass);
+          const unsigned long long mask = __builtin_amdgcn_ballot_w64(score <= thr_f) & in_play;
           if (mask != 0ull) {
             if (wcount + 64u > cap) {
               // make room (the buffer holds more than k keys): keep the k best and tighten the wave's bound
               const uint32_t t2 = select_keys(my_cand, wcount);
               wcount            = a.k;
-              thr               = t2 < thr ? t2 : thr;
+              if (t2 < thr) {
+                thr       = t2;
+                thr_f     = unorder_f32(thr);
+                stop_bits = thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u;
+              }
             }
-            const bool pass2 = pass && okey <= thr;
-            const unsigned long long mask2 = __ballot(pass2);
+            const uint32_t okey            = order_f32(score);
+            const bool pass                = ((mask >> lane) & 1ull) != 0ull && okey <= thr;
+            const unsigned long long mask2 = __builtin_amdgcn_ballot_w64(pass);
             const uint32_t below =
               __builtin_amdgcn_mbcnt_hi(uint32_t(mask2 >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(mask2), 0u));
-            if (pass2) { my_cand[wcount + below] = (static_cast<unsigned long long>(okey) << 32) | (sample_off + i); }
+            if (pass) { my_cand[wcount + below] = (static_cast<unsigned long long>(okey) << 32) | (sample_off + i); }
             wcount += uint32_t(__popcll(mask2));
           }
-          if (tile + WG < n_tiles) {
-#pragma unroll
-            for (int m = 0; m < NCH; m++) { cur[m] = ahead[m]; }
-          }
+        };
+        // the two code buffers swap roles from tile to tile
+        for (uint32_t tile = wig; tile < n_tiles; tile += 2u * WG) {
+          scan_tile(tile, cur, ahead);
+          if (tile + WG < n_tiles) { scan_tile(tile + WG, ahead, cur); }
         }
         n_keys = wcount;
       }
