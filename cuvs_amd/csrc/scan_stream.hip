@@ -653,7 +653,11 @@ struct stream_kernel {
       asm volatile("" : "+v"(addr[i]));
     }
 
-    pair_desc my_d = record(quad_of(0), GI);
+    // The record of the next iteration's pair is requested an iteration before it is looked at: the
+    // first wait for codes after a request also waits for the request, and nothing should wait for
+    // a record.
+    pair_desc my_d  = record(quad_of(0), GI);
+    pair_desc nxt_d = record(quad_of(n_it > 1 ? 1 : 0), GI);
     u32x4 cur[NCH], ahead[NCH];
     if (wig * 64u < my_d.n_rows) {
       const uint32_t r0 = wig * 64u + lane;
@@ -664,8 +668,7 @@ struct stream_kernel {
     block_barrier();  // tables of iteration 0 are complete
 
     for (uint32_t it = 0; it < n_it; it++) {
-      const bool has_next   = it + 1 < n_it;
-      const pair_desc nxt_d = record(quad_of(has_next ? it + 1 : it), GI);
+      const bool has_next    = it + 1 < n_it;
       const pair_desc done_d = my_d;
       uint32_t n_keys        = 0;
       if (my_d.slot != 0xFFFFFFFFu) {
@@ -743,6 +746,7 @@ struct stream_kernel {
         }
         if (my_d.n_rows != 0) { pre_thr = a.query_kth[my_d.q]; }
       }
+      nxt_d = record(quad_of(it + 2 < n_it ? it + 2 : it), GI);
       block_barrier();  // every scanner is through with this iteration's tables
       // While the builders write the next tables: this wave's best candidates of the pair go out,
       // and their k-th bounds the query from now on.
