@@ -14,6 +14,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <string>
+#include <mutex>
 #include <vector>
 
 namespace cuvs {
@@ -105,6 +106,35 @@ using cuvs::distance::DistanceType;
 
 /** Index contents.  Lists live in two arenas (codes, ids); list `l` starts at row `row_offset[l]`
  *  (a multiple of 32) and owns round_up(size, 32) rows. */
+/** What the early-stop screen achieved on an index lately, fed back to the searches that decide
+ *  whether to use it: on data whose lists all lie about as far from a query as its nearest one, the
+ *  screen keeps nearly every pair and its launches only add to the scan.  One screened search at a
+ *  time is observed (its survivor count is copied to pinned memory behind the search; a later
+ *  search folds it in once it has landed - nothing waits), and while the verdict for the same
+ *  (n_probes, k) is "does not pay", searches in the automatic mode scan plainly, except every
+ *  kScreenRecheck-th one, which is screened and observed again. */
+struct screen_feedback {
+  static constexpr uint32_t kScreenRecheck = 64;
+  static constexpr double kKeepLimit       = 0.7;  // survivors / screened pairs above which the screen is off
+  std::mutex mu;
+  uint32_t* host    = nullptr;  // pinned: survivors of the search under observation
+  hipEvent_t landed = nullptr;  // recorded behind the copy into `host`
+  bool pending      = false;
+  uint64_t pending_pairs  = 0;  // pairs that search screened
+  uint32_t pending_probes = 0, pending_k = 0;
+  bool off          = false;    // verdict, for searches with these parameters:
+  uint32_t probes = 0, k = 0;
+  uint32_t plain_searches = 0;  // since the verdict
+  /** The pinned word and the event (allocates; called when an index is made, never by a search). */
+  void create();
+  /** Folds in an observation that has landed.  Call with `mu` held. */
+  void collect();
+  screen_feedback() = default;
+  screen_feedback(const screen_feedback&)            = delete;
+  screen_feedback& operator=(const screen_feedback&) = delete;
+  ~screen_feedback();
+};
+
 struct index_impl {
   DistanceType metric        = DistanceType::L2Expanded;
   codebook_gen codebook_kind = codebook_gen::PER_SUBSPACE;
@@ -140,6 +170,7 @@ struct index_impl {
   device_buffer list_rank;
   std::vector<int64_t> accum_sorted_sizes;  // [n_lists + 1]
   int64_t size = 0;
+  mutable screen_feedback feedback;
 
   uint64_t group_bytes() const { return uint64_t(n_chunks) * kIndexGroupSize * kIndexGroupVecLen; }
   /** Recompute pointer tables, device sizes and the sorted prefix sums from the host vectors

@@ -14,6 +14,34 @@ namespace cuvs::neighbors::ivf_pq {
 
 namespace detail {
 
+void screen_feedback::create()
+{
+  if (host != nullptr) { return; }
+  CUVS_HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&host), 64, hipHostMallocDefault));
+  host[0] = 0;
+  CUVS_HIP_TRY(hipEventCreateWithFlags(&landed, hipEventDisableTiming));
+}
+
+void screen_feedback::collect()
+{
+  if (!pending || hipEventQuery(landed) != hipSuccess) { return; }
+  pending = false;
+  if (pending_pairs == 0) { return; }
+  off            = double(host[0]) > kKeepLimit * double(pending_pairs);
+  probes         = pending_probes;
+  k              = pending_k;
+  plain_searches = 0;
+}
+
+screen_feedback::~screen_feedback()
+{
+  if (landed != nullptr) {
+    (void)hipEventSynchronize(landed);  // a copy into `host` may still be on its way
+    (void)hipEventDestroy(landed);
+  }
+  if (host != nullptr) { (void)hipHostFree(host); }
+}
+
 void init_index(index_impl& ix, const index_params& params, uint32_t dim)
 {
   CUVS_EXPECTS(params.pq_bits >= 4 && params.pq_bits <= 8,
@@ -61,6 +89,7 @@ void init_index(index_impl& ix, const index_params& params, uint32_t dim)
   ix.data_ptrs.allocate(sizeof(void*) * ix.n_lists);
   ix.inds_ptrs.allocate(sizeof(void*) * ix.n_lists);
   ix.size = 0;
+  ix.feedback.create();
 }
 
 void index_impl::recompute_internal_state(hipStream_t stream)
@@ -256,6 +285,7 @@ index<int64_t> clone(cuvs::resources const& res, const index<int64_t>& source)
   dst.n_max                          = src.n_max;
   dst.coarse_fast_ok                 = src.coarse_fast_ok;
   dst.rotation_is_identity           = src.rotation_is_identity;
+  dst.feedback.create();
   copy(dst.centers, src.centers);
   copy(dst.centers_rot, src.centers_rot);
   copy(dst.rotation, src.rotation);

@@ -425,8 +425,23 @@ void search(cuvs::resources const& res_c,
   // they save (the reference skips the grouping when lists are rarely shared,
   // expected_probe_coresidency, ivf_pq_search.cuh:353-373).
   const bool few_pairs       = uint64_t(Qb) * P <= kFewPairs;
-  const bool early_stop = fast_scan && !few_pairs && P > kLeadProbes && P <= 8192 &&
-                          detail::scan_screen_supported(sa) && res.tuning.early_stop != 1;
+  bool early_stop = fast_scan && !few_pairs && P > kLeadProbes && P <= 8192 &&
+                    detail::scan_screen_supported(sa) && res.tuning.early_stop != 1;
+  // In the automatic mode the index remembers whether the screen pays on its data: where it kept
+  // most pairs the last time it ran with these parameters, this search scans plainly.
+  bool observe_screen = false;
+  if (early_stop && res.tuning.early_stop == 0 && ix.feedback.host != nullptr) {
+    auto& fb = ix.feedback;
+    std::lock_guard<std::mutex> guard(fb.mu);
+    fb.collect();
+    if (fb.off && fb.probes == P && fb.k == k) {
+      fb.plain_searches += 1;
+      if (fb.plain_searches % detail::screen_feedback::kScreenRecheck != 0) { early_stop = false; }
+    }
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    CUVS_HIP_TRY(hipStreamIsCapturing(s, &capture));
+    observe_screen = early_stop && capture == hipStreamCaptureStatusNone;
+  }
   const uint32_t lead          = early_stop ? kLeadProbes : P;
   detail::pair_desc* survivors = nullptr;
   uint8_t* alive               = nullptr;
@@ -512,6 +527,21 @@ void search(cuvs::resources const& res_c,
       detail::launch_fill_u32(n_survivors, 0, 1, s);
       detail::launch_scan_screen(sa, desc + size_t(nq) * lead, nq * (P - lead), survivors, n_survivors,
                                  alive, s);
+      if (observe_screen) {
+        // the survivor count follows the search to the host, for the searches after this one
+        observe_screen = false;
+        auto& fb       = ix.feedback;
+        std::lock_guard<std::mutex> guard(fb.mu);
+        fb.collect();
+        if (!fb.pending) {
+          CUVS_HIP_TRY(hipMemcpyAsync(fb.host, n_survivors, 4, hipMemcpyDeviceToHost, s));
+          CUVS_HIP_TRY(hipEventRecord(fb.landed, s));
+          fb.pending        = true;
+          fb.pending_pairs  = uint64_t(nq) * (P - lead);
+          fb.pending_probes = P;
+          fb.pending_k      = uint32_t(k);
+        }
+      }
       mark(6);
       // 3. the pairs still in play, in full
       sa.desc        = survivors;

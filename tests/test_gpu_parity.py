@@ -408,6 +408,47 @@ def test_early_stop_matches_oracle_and_full_scan(orc, lut, internal, dtype, kind
         assert torch.equal(nb, nb2) and torch.equal(d, d2)
 
 
+def test_screen_turns_itself_off_where_it_does_not_pay(orc):
+    """Rows without cluster structure: every probed list is about as far from a query as its nearest
+    one, the screen keeps nearly every pair, and the index remembers: searches after the one that was
+    observed scan plainly (every 64th is screened again), with the same results either way - the
+    oracle's."""
+    from cuvs_amd.resources import Resources
+    rng = np.random.default_rng(11)
+    allrows = rng.standard_normal((30300, 128)).astype(np.float32)
+    x, q = allrows[:30000], allrows[30000:]
+    model = H.train(x, 100, 64, 8, iters=4)
+    index = G.build_gpu_index(model, x, 64, 8, "sqeuclidean", "subspace")
+    ix, _ = G.read_back(orc, index, model, 128, 64, 8, "sqeuclidean", "subspace")
+    res = Resources()
+    res.enable_profiling(True)
+    sp = ivf_pq.SearchParams(n_probes=24, lut_dtype=R_16F)
+    want_nb, want_d = orc.search(ix, q, 10, 24, lut_dtype=ORC_DT[R_16F])
+    screened = []
+    for call in range(70):
+        d, nb = ivf_pq.search(sp, index, G.to_dev(q), 10, resources=res)
+        res.sync()
+        prof = ivf_pq.get_search_profile(res)
+        screened.append(prof["n_screened_pairs"])
+        if call in (0, 1, 2, 64, 65):
+            if prof["n_screened_pairs"]:
+                assert prof["n_surviving_pairs"] > 0.7 * prof["n_screened_pairs"]
+            H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
+    assert screened[0] == q.shape[0] * 23           # observed
+    assert screened[1] == 0 and screened[2] == 0    # verdict in: plain scans
+    assert sum(1 for n in screened if n) == 2       # and one more look, 64 plain searches later
+    # other parameters: no verdict yet, the screen runs (and is observed in its turn)
+    d, nb = ivf_pq.search(ivf_pq.SearchParams(n_probes=16, lut_dtype=R_16F), index, G.to_dev(q), 10, resources=res)
+    res.sync()
+    assert ivf_pq.get_search_profile(res)["n_screened_pairs"] == q.shape[0] * 15
+    # forced on, it runs whatever the verdict
+    res.set_search_tuning(early_stop="on")
+    d2, nb2 = ivf_pq.search(sp, index, G.to_dev(q), 10, resources=res)
+    res.sync()
+    assert ivf_pq.get_search_profile(res)["n_screened_pairs"] == q.shape[0] * 23
+    H.compare_results(nb2.cpu().numpy(), d2.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
+
+
 @pytest.mark.parametrize("kind", ["subspace", "cluster"])
 def test_early_stop_pq_len_4(orc, kind):
     """Four dimensions per subspace: 16-byte codebook entries in the table-free screen (shared by
