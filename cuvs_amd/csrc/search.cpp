@@ -550,7 +550,8 @@ void search(cuvs::resources const& res_c,
       CUVS_EXPECTS(full_scan(), "scan kernel launch failed");
     } else {
       const bool launched = fast_scan && (quad_kpp != 0   ? detail::launch_scan_stream(sa, s)
-                                          : nibble_scan ? detail::launch_scan_nibble(sa, s)
+                                          : nibble_scan ? (detail::launch_scan_nibble_pack(sa, s) ||
+                                                           detail::launch_scan_nibble(sa, s))
                                                         : detail::launch_scan_fast(sa, s));
       if (!launched) { detail::launch_scan(sa, s); }
     }

@@ -820,6 +820,42 @@ def test_four_bit_block_kernel_matches_oracle(orc, lut, internal, dim, pq_dim, m
                           exact=(metric != "euclidean"))
 
 
+@pytest.mark.parametrize("lut", [R_16F, R_8U])
+@pytest.mark.parametrize("dim,pq_dim,metric,kind", [
+    (256, 128, "sqeuclidean", "subspace"),   # two steps, pq_len 2, early stop inside a tile
+    (128, 128, "inner_product", "subspace"), # pq_len 1
+    (512, 128, "cosine", "cluster"),         # pq_len 4, per-cluster codebooks
+    (512, 256, "euclidean", "subspace"),     # four steps
+])
+def test_four_bit_two_rows_per_lane_kernel_matches_oracle(orc, lut, dim, pq_dim, metric, kind):
+    """binary16 sums, pq_dim a multiple of 128, k <= 64: the kernel that scores two rows per lane
+    with packed adds, one wave per pair."""
+    data, model, queries, index, ix, _ = _nibble_case(orc, dim, pq_dim, metric, kind)
+    for k, n_probes in ((1, 3), (10, 8), (64, 24)):
+        nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, k, n_probes, lut=lut, internal=R_16F)
+        H.compare_results(nb, d, want_nb, want_d, 2e-3, exact=(metric != "euclidean"))
+
+
+def test_four_bit_two_rows_per_lane_kernel_filter_and_long_lists(orc):
+    """Lists of several thousand rows (many tiles of 128 rows per wave, the candidate buffer is
+    reduced several times) and a bitset filter."""
+    data, model, queries, index, ix, _ = _case(orc, 40000, 128, 6, 128, 4, n_queries=24)
+    n = data.shape[0]
+    keep = np.ones(n, dtype=bool)
+    keep[::4] = False
+    bits = np.packbits(keep, bitorder="little")
+    bits = np.concatenate([bits, np.zeros((-bits.size) % 4, dtype=np.uint8)]).view(np.uint32)
+    for lut in (R_16F, R_8U):
+        sp = ivf_pq.SearchParams(n_probes=4, lut_dtype=lut, internal_distance_dtype=R_16F)
+        d, nb = ivf_pq.search(sp, index, G.to_dev(queries), 50,
+                              filter_bitset=G.to_dev(bits.view(np.int32)), filter_nbits=n)
+        want_nb, want_d = orc.search(ix, queries, 50, 4, lut_dtype=ORC_DT[lut], internal_distance_dtype=ORC_DT[R_16F],
+                                     filter_bitset=bits, filter_nbits=n)
+        H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
+        nb2, d2, want_nb2, want_d2 = _search_both(orc, index, ix, queries, 64, 6, lut=lut, internal=R_16F)
+        H.compare_results(nb2, d2, want_nb2, want_d2, 2e-3, exact=True)
+
+
 def test_four_bit_block_kernel_filter_and_long_lists(orc):
     """Lists of several thousand rows (more than one pruning segment of the candidate buffer) and a
     bitset filter."""
