@@ -228,7 +228,11 @@ __global__ __launch_bounds__(kPackThreads) void scan_nibble_pack_kernel(scan_arg
               diff -= pqc;
               score = fmaf(diff, diff, score);
             } else {
-              score -= cd * qd;
+              // the rounded product, as the reference subtracts it: kept out of the compiler's sight, which
+              // would fuse the multiplication into the subtraction (one rounding instead of two)
+              float cq = cd * qd;
+              asm volatile("" : "+v"(cq));
+              score -= cq;
               score = fmaf(-qd, pqc, score);
             }
           }

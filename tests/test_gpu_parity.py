@@ -856,6 +856,51 @@ def test_four_bit_two_rows_per_lane_kernel_filter_and_long_lists(orc):
         H.compare_results(nb2, d2, want_nb2, want_d2, 2e-3, exact=True)
 
 
+_BITS = {}
+
+
+def _bits_case(orc, dim, pq_dim, pq_bits, metric, kind):
+    key = (dim, pq_dim, pq_bits, metric, kind)
+    if key not in _BITS:
+        _BITS[key] = _case(orc, 6000, dim, 24, pq_dim, pq_bits, metric=metric, kind=kind, n_queries=48)
+    return _BITS[key]
+
+
+@pytest.mark.parametrize("lut,internal", [(R_16F, R_32F), (R_8U, R_32F), (R_16F, R_16F), (R_8U, R_16F)])
+@pytest.mark.parametrize("dim,pq_dim,pq_bits,metric,kind", [
+    (128, 64, 5, "sqeuclidean", "subspace"),    # 25 codes a chunk: three chunks, the last one 14 codes
+    (128, 64, 6, "inner_product", "subspace"),  # 21 codes a chunk: four chunks, the last one a single code
+    (128, 64, 7, "sqeuclidean", "cluster"),     # 18 codes a chunk, per-cluster codebooks
+    (96, 96, 6, "cosine", "subspace"),          # pq_len 1, five chunks
+    (128, 32, 7, "euclidean", "subspace"),      # pq_len 4, two chunks
+])
+def test_five_to_seven_bit_codes_match_oracle(orc, lut, internal, dim, pq_dim, pq_bits, metric, kind):
+    """Codes of 5, 6 and 7 bits (bit-packed, some straddling two words of a chunk, the last chunk
+    partly filled) at the benchmark's subspace counts."""
+    data, model, queries, index, ix, _ = _bits_case(orc, dim, pq_dim, pq_bits, metric, kind)
+    for k, n_probes in ((1, 3), (10, 8), (64, 24)):
+        nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, k, n_probes, lut=lut, internal=internal)
+        H.compare_results(nb, d, want_nb, want_d, 2e-3, exact=(metric != "euclidean"))
+
+
+def test_five_to_seven_bit_codes_filter_and_long_lists(orc):
+    """Lists of several thousand rows and a bitset filter, 6-bit codes."""
+    data, model, queries, index, ix, _ = _case(orc, 40000, 64, 6, 32, 6, n_queries=24)
+    n = data.shape[0]
+    keep = np.ones(n, dtype=bool)
+    keep[::4] = False
+    bits = np.packbits(keep, bitorder="little")
+    bits = np.concatenate([bits, np.zeros((-bits.size) % 4, dtype=np.uint8)]).view(np.uint32)
+    for lut in (R_16F, R_8U):
+        sp = ivf_pq.SearchParams(n_probes=4, lut_dtype=lut)
+        d, nb = ivf_pq.search(sp, index, G.to_dev(queries), 50,
+                              filter_bitset=G.to_dev(bits.view(np.int32)), filter_nbits=n)
+        want_nb, want_d = orc.search(ix, queries, 50, 4, lut_dtype=ORC_DT[lut], filter_bitset=bits, filter_nbits=n)
+        H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
+        nb2, d2, want_nb2, want_d2 = _search_both(orc, index, ix, queries, 64, 6, lut=lut)
+        H.compare_results(nb2, d2, want_nb2, want_d2, 2e-3, exact=True)
+
+
 def test_four_bit_block_kernel_filter_and_long_lists(orc):
     """Lists of several thousand rows (more than one pruning segment of the candidate buffer) and a
     bitset filter."""
