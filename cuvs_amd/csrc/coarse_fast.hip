@@ -25,7 +25,7 @@
  * smallest s' is >= t - E, and every list with s <= t has s' <= t + E <= (n_probes-th smallest s')
  * + 2E <= T + 2E.
  */
-#include "device_utils.cuh"
+#include "scan_wave_select.cuh"
 
 #include <mutex>
 
@@ -380,6 +380,12 @@ __global__ __launch_bounds__(256) void coarse_threshold_kernel(
       lowest               = other < lowest ? other : lowest;
     }
     prefix = lowest;
+  } else if (n_groups <= HELD * 64u) {
+    // every minimum is in a register: radix selection over the bits in which they differ at all
+    unsigned long long live[HELD];
+#pragma unroll
+    for (uint32_t h = 0; h < HELD; h++) { live[h] = __builtin_amdgcn_ballot_w64(lane + h * 64u < n_groups); }
+    prefix = wave_kth_smallest<int(HELD)>(held, live, n_probes, lane);
   } else {
     for (int bit = 31; bit >= 0; bit--) {
       const uint32_t probe = prefix | ((1u << bit) - 1u);
@@ -422,15 +428,36 @@ __global__ __launch_bounds__(512) void coarse_rescore_kernel(
     if (tid == 0) { fallback[q] = 1; }
     return;
   }
-  for (uint32_t d = tid; d < dim; d += blockDim.x) { qf[d] = map_elem<T>(queries[uint64_t(q) * dim + d]); }
+  // The waves without a candidate leave at once (the barrier below counts the waves that are still
+  // there): a typical query has ~70 candidates, and the slots of the idle waves let the next
+  // queries' blocks start.
+  const uint32_t n_active = (n + 63u) & ~63u;
+  if (tid >= n_active) { return; }
+  for (uint32_t d = tid; d < dim; d += n_active) { qf[d] = map_elem<T>(queries[uint64_t(q) * dim + d]); }
   __syncthreads();
   unsigned long long key = kInvalidKey;
   if (tid < n) {
     const uint32_t l = cand[uint64_t(q) * kCandCapF + tid];
     const float* c   = centers + uint64_t(l) * dim_ext;  // rows are 32-byte aligned (dim_ext % 8 == 0)
     float acc        = 0.0f;
-    const uint32_t dim4 = dim & ~3u;
-    for (uint32_t d = 0; d < dim4; d += 4) {
+    // The FMA chain is sequential; the loads are not: 32 dimensions of the centre row are requested
+    // together (one latency for eight 16-byte loads), then multiplied in.
+    const uint32_t dim32 = dim & ~31u;
+    const uint32_t dim4  = dim & ~3u;
+    for (uint32_t d0 = 0; d0 < dim32; d0 += 32) {
+      float4 v[8];
+#pragma unroll
+      for (uint32_t x = 0; x < 8; x++) { v[x] = *reinterpret_cast<const float4*>(c + d0 + 4 * x); }
+#pragma unroll
+      for (uint32_t x = 0; x < 8; x++) {
+        const uint32_t d = d0 + 4 * x;
+        acc              = fmaf(v[x].x, qf[d], acc);
+        acc              = fmaf(v[x].y, qf[d + 1], acc);
+        acc              = fmaf(v[x].z, qf[d + 2], acc);
+        acc              = fmaf(v[x].w, qf[d + 3], acc);
+      }
+    }
+    for (uint32_t d = dim32; d < dim4; d += 4) {
       const float4 v = *reinterpret_cast<const float4*>(c + d);
       acc            = fmaf(v.x, qf[d], acc);
       acc            = fmaf(v.y, qf[d + 1], acc);

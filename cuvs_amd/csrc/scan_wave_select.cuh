@@ -61,6 +61,38 @@ __device__ __forceinline__ int wave_radix_select(const uint32_t (&value)[NK], co
   return -1;
 }
 
+/** The r-th smallest (r >= 1) of the wave's values value[j] of the lanes in live[j] (at least r of
+ *  them; lane 0 of value[0] must be one).  The bits that all values share are skipped, and the
+ *  selection ends as soon as a group of exactly the right size is split off, whose largest member
+ *  is the answer. */
+template <int NK>
+__device__ __forceinline__ uint32_t wave_kth_smallest(const uint32_t (&value)[NK], const unsigned long long (&live)[NK],
+                                                      uint32_t r, uint32_t lane)
+{
+  const uint32_t first = uint32_t(__builtin_amdgcn_readfirstlane(int(value[0])));
+  uint32_t differ      = 0;
+#pragma unroll
+  for (int j = 0; j < NK; j++) { differ |= ((live[j] >> lane) & 1ull) != 0ull ? value[j] ^ first : 0u; }
+  int top = -1;  // highest bit set in any lane's `differ`
+  if (__builtin_amdgcn_ballot_w64(differ != 0u) != 0ull) {
+    top = 0;
+#pragma unroll
+    for (int s = 16; s >= 1; s >>= 1) {
+      if (__builtin_amdgcn_ballot_w64((differ >> (top + s)) != 0u) != 0ull) { top += s; }
+    }
+  }
+  uint32_t kth  = top >= 0 ? (first >> top >> 1 << top << 1) : first;  // the common bits
+  const int cut = wave_radix_select<NK>(value, live, r, top, kth);
+  if (cut < 0) { return kth; }
+  uint32_t largest = 0;
+#pragma unroll
+  for (int j = 0; j < NK; j++) {
+    const bool in = ((live[j] >> lane) & 1ull) != 0ull && (value[j] >> cut) <= (kth >> cut);
+    largest       = in && value[j] > largest ? value[j] : largest;
+  }
+  return wave_max_u32(largest);
+}
+
 /** Keeps the k smallest of the first n >= k keys (n <= 64 * NK) of one wave's buffer, in buf[0 .. k)
  *  in no particular order, and returns the high word of the k-th smallest.  Keys are distinct (the
  *  low word numbers the sample); among equal high words the smaller low words win, as in a sort of
