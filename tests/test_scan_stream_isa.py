@@ -1,10 +1,11 @@
-"""The lookups of scan_stream.hip are issued and waited for by separate inline-assembly statements,
-so that the adds of one batch overlap the reads of the next.  From the compiler's point of view a
-read's destination register holds its value as soon as the read is issued; nothing stops it from
-copying or reusing that register before the data has arrived, except that it has no reason to in
-straight-line code with registers to spare.  This test compiles the file for gfx950 and checks the
-generated code for exactly that: between an inline `ds_read_u16` and the inline `s_waitcnt` that
-covers it, no compiler-generated instruction, label or branch touches the destination register.
+"""The table lookups of scan_stream.hip and scan_nibble_pack.hip are issued and waited for in
+inline assembly, so that the adds of one group overlap the reads of the next.  From the compiler's
+point of view a read's destination register holds its value as soon as the read is issued; nothing
+stops it from copying or reusing that register before the data has arrived.  Both files therefore
+keep a whole tile (or step) of lookups in one assembly block.  This test compiles them for gfx950
+and checks the generated code for what that is meant to guarantee: between an inline `ds_read_u16`
+and the inline `s_waitcnt` that covers it, no compiler-generated instruction, label or branch
+touches the destination register, and no other inline instruction reads it.
 """
 import os
 import re
@@ -14,7 +15,7 @@ import subprocess
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-SRC = os.path.join(ROOT, "cuvs_amd", "csrc", "scan_stream.hip")
+SOURCES = {"scan_stream.hip": 48 * 32, "scan_nibble_pack.hip": 128 * 24}  # file: inline reads at least expected
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 
@@ -70,14 +71,15 @@ def check_lookup_windows(asm_text):
 
 
 @pytest.mark.skipif(shutil.which(HIPCC) is None and not os.path.exists(HIPCC), reason="needs hipcc")
-def test_no_instruction_touches_a_lookup_in_flight(tmp_path):
-    out = tmp_path / "scan_stream.s"
+@pytest.mark.parametrize("name", sorted(SOURCES))
+def test_no_instruction_touches_a_lookup_in_flight(tmp_path, name):
+    out = tmp_path / (name + ".s")
     subprocess.check_call([HIPCC, "-O3", "-std=c++17", "--offload-arch=gfx950", "--cuda-device-only", "-S",
                            "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(ROOT, "cuvs_amd", "csrc"),
                            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-fvisibility=hidden",
-                           SRC, "-o", str(out)], stderr=subprocess.DEVNULL)
+                           os.path.join(ROOT, "cuvs_amd", "csrc", name), "-o", str(out)], stderr=subprocess.DEVNULL)
     n_reads, problems = check_lookup_windows(out.read_text())
-    assert n_reads >= 48 * 32, "the kernels' inline lookups were not found in the generated code"
+    assert n_reads >= SOURCES[name], "the kernels' inline lookups were not found in the generated code"
     assert not problems, "instructions inside a lookup window:\n" + "\n".join(f"{n}: {t}" for n, t in problems[:20])
 
 
