@@ -19,7 +19,9 @@
  * the fp_8bit codec, IEEE half conversion/addition, the interleaved list layout,
  * the lookup-table + scan identity  sum_j LUT[j][code_j] == ||(q - c) - decode(codes)||^2,
  * coarse selection vs. textbook L2, chunk indices vs. cumsum, id translation vs. searchsorted,
- * distance post-processing.
+ * distance post-processing; the reduced-precision coarse scores: coarse_scores_f16 against numpy's
+ * float16 roundings around an fp32 FMA chain (and an exact-integer case), coarse_scores_i8 against
+ * the published formulas restated in numpy (tests/test_oracle_search.py).
  */
 #include "ivf_pq_oracle.h"
 
@@ -242,7 +244,9 @@ void coarse_scores_f32(const orc_index& ix, const float* qf, float* scores)
 
 /* half-precision variant (ivf_pq_search.cuh:258-340): centres and queries rounded to binary16,
  * products accumulated in fp32 (FMA, ascending), result rounded to binary16 after scaling.
- * parity unpinned: the reference's half GEMM accumulation type is a cuBLAS detail. */
+ * The arithmetic stated here is pinned by tests/test_oracle_search.py (numpy float16); that the
+ * reference's half GEMM accumulates this way is a cuBLAS detail: parity unpinned for the
+ * accumulation type. */
 void coarse_scores_f16(const orc_index& ix, const float* qf, float* scores)
 {
   const uint32_t de = dim_ext_of(ix.dim);
