@@ -39,7 +39,7 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr uint32_t kTile    = 128;  // lists per tile
+constexpr uint32_t kTile    = 64;   // lists per tile
 constexpr uint32_t kQTile   = 256;  // queries per block: 4 waves x 64
 constexpr uint32_t kSlab    = 64;   // the padded dimension is a multiple of this
 constexpr uint32_t kCandCapF = 512;  // candidate slots per query (256 are used up to 128 probes)
@@ -114,25 +114,28 @@ __global__ void pack_centers_kernel(const float* __restrict__ centers, uint32_t 
   }
 }
 
-constexpr uint32_t kGemmThreads = 512;
-constexpr uint32_t kLocalCap    = 32;  // PASS 2: candidates a block may hold per query before it gives up
-constexpr uint32_t kTilesPerBlock = 10;  // list tiles a block walks at most (its group minima fill the LDS)
+constexpr uint32_t kGemmThreads = 256;
+constexpr uint32_t kLocalCap    = 32;  // PASS 2: candidates a query may collect between two flushes before its block gives up
+constexpr uint32_t kFlushTiles  = 8;   // list tiles between two flushes: 32 group minima, one 128-byte line of a query's row
+constexpr uint32_t kMinRow      = kFlushTiles * 4u + 4u;  // floats per query in the staged minima (rows 144 bytes apart)
 
 /**
- * fp16 scores s' = alpha * (dot16(c, q) + cn * qterm) of a block's 256 queries against a run of
- * list tiles (128 lists each).  The queries stay in LDS for the whole block; list tiles stream
- * through two LDS buffers, the next tile's global loads in flight while the current one is
- * multiplied (one barrier per tile).  Eight waves, two per SIMD so that one's matrix products
- * overlap the other's epilogue; a wave owns 64 lists x 64 queries, four MFMA tiles of
- * v_mfma_f32_32x32x16_f16 (each 16-byte read of the list operand out of LDS feeds two products:
- * with 32 queries a wave the LDS bandwidth, not the matrix cores, set the pace).  PASS 1 writes, per query, the minimum over every group of 16 lists;
- * PASS 2 collects the lists whose score is at or below the query's threshold in LDS and appends
- * them to the query's candidate list when the block ends (one global atomic per query and block).
+ * fp16 scores s' = alpha * (cn * qterm + dot16(c, q)) of a block's 256 queries against a run of
+ * list tiles (64 lists each).  Four waves, one per SIMD, each with 64 of the queries and all 64
+ * lists of a tile: four MFMA tiles of v_mfma_f32_32x32x16_f16 (each 16-byte read of the list
+ * operand out of LDS feeds two products), the query operand in registers for the whole block.  Two
+ * blocks fit a CU, so that one block's matrix products run under the other's epilogue, staging
+ * and barrier.  List tiles stream through two LDS buffers, the next tile's global loads in flight
+ * while the current one is multiplied (one barrier per tile).  The norm term is the accumulators'
+ * starting value.  PASS 1 keeps, per query, the minimum of every group of 16 lists; PASS 2 collects
+ * the lists whose score is at or below the query's threshold.  Both results are staged in LDS by
+ * the wave that owns the query and written out by that wave every kFlushTiles tiles (the minima
+ * as whole 128-byte lines; the candidates with one global atomic per query), without a barrier.
  * Both passes execute the same instructions up to the epilogue, so a list's score is the same
  * number in both.  K_PAD = padded dimension (64 or 128).
  */
 template <int PASS, uint32_t K_PAD>
-__global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
+__global__ __launch_bounds__(kGemmThreads, 2) void coarse_f16_kernel(
   const _Float16* __restrict__ ch, const _Float16* __restrict__ qh, const float* __restrict__ cn,
   uint32_t n_lists, uint32_t n_queries, uint32_t q_rows, uint32_t n_list_tiles, uint32_t tiles_per_block, float alpha,
   float qterm, float* __restrict__ minima, uint32_t n_groups, const float* __restrict__ thr,
@@ -142,19 +145,42 @@ __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
   constexpr uint32_t CHUNKS = K_PAD / 8u;        // 16-byte chunks per row
   constexpr uint32_t PER_T  = kTile * CHUNKS / kGemmThreads;  // chunks per thread and tile (2 or 4)
   extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char* sa0 = smem;  // lists [2][128][ROWB], two buffers
-  float* scn         = reinterpret_cast<float*>(smem + 2u * kTile * ROWB);  // [2][128] norm terms
+  unsigned char* sa0 = smem;  // lists [2][64][ROWB], two buffers
+  float* scn         = reinterpret_cast<float*>(smem + 2u * kTile * ROWB);  // [2][64] norm terms
   uint32_t* lcount   = reinterpret_cast<uint32_t*>(scn + 2u * kTile);       // PASS 2: [256]
   uint32_t* lcand    = lcount + kQTile;                                     // PASS 2: [256][kLocalCap]
-  float* lmin        = reinterpret_cast<float*>(lcount);  // PASS 1: [256][kTilesPerBlock * 8] group minima
+  float* lmin        = reinterpret_cast<float*>(lcount);  // PASS 1: [256][kMinRow] group minima
   const uint32_t tid  = threadIdx.x;
   const uint32_t lane = tid & 63u;
-  const uint32_t wid  = tid >> 6;
-  const uint32_t wl   = wid >> 2;  // wave's half of the lists (64)
-  const uint32_t wq   = wid & 3u;  // wave's quarter of the queries (64)
+  const uint32_t wid  = tid >> 6;  // the wave's quarter of the queries (64)
+  const uint32_t half = lane >> 5;
   const uint32_t q0   = blockIdx.y * kQTile;
   const uint32_t t0   = blockIdx.x * tiles_per_block;
   const uint32_t t1   = t0 + tiles_per_block < n_list_tiles ? t0 + tiles_per_block : n_list_tiles;
+  const float neg_inf   = -__uint_as_float(0x7f800000u);
+  const float inv_alpha = 1.0f / alpha;
+
+  // this lane's two queries inside the block (columns of the wave's two query tiles); the packed
+  // queries are padded to a multiple of 128 rows, a block's second half may lie beyond them.  The
+  // wave's query operand never changes: it lives in registers.
+  uint32_t qloc[2], q[2];
+  v8h bq[2][K_PAD / 16u];
+  float limit[2] = {0.0f, 0.0f};
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    qloc[j]             = wid * 64u + uint32_t(j) * 32u + (lane & 31u);
+    q[j]                = q0 + qloc[j];
+    const uint32_t q_rd = q[j] < q_rows ? q[j] : q_rows - 1u;
+#pragma unroll
+    for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) {
+      bq[j][ks] = *reinterpret_cast<const v8h*>(qh + uint64_t(q_rd) * K_PAD + ks * 16u + half * 8u);
+    }
+    // The epilogue works on v = norm term + dot; the score is alpha * v with alpha = -1 or -2, so
+    // the smallest score of a group is alpha * (its largest v) and "score <= thr" is
+    // "v >= thr / alpha", both exactly.  The threshold is only requested here: the first epilogue
+    // is its first use, a tile of products later.
+    if (PASS == 2) { limit[j] = q[j] < n_queries ? thr[q[j]] : neg_inf; }
+  }
 
   // this thread's chunks of a tile: row and 16-byte part
   uint32_t crow[PER_T], cpart[PER_T];
@@ -164,8 +190,6 @@ __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
     crow[c]              = chunk / CHUNKS;
     cpart[c]             = chunk % CHUNKS;
   }
-  const float neg_inf = -__uint_as_float(0x7f800000u);
-
   // the first list tile
 #pragma unroll
   for (uint32_t c = 0; c < PER_T; c++) {
@@ -177,30 +201,10 @@ __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
     const uint32_t l = t0 * kTile + tid;
     scn[tid]         = l < n_lists ? cn[l] * qterm : neg_inf;
   }
-  if (PASS == 2 && tid < kQTile) { lcount[tid] = 0; }
+  if (PASS == 2) { lcount[tid] = 0; }
   __syncthreads();
-
-  // The epilogue works on v = dot + norm term; the score is alpha * v with alpha = -1 or -2, so the
-  // smallest score of a group is alpha * (its largest v) and "score <= thr" is "v >= thr / alpha",
-  // both exactly.
-  // this lane's two queries inside the block (columns of the wave's two query tiles); the packed
-  // queries are padded to a multiple of 128 rows, a block's second half may lie beyond them
-  uint32_t qloc[2], q[2];
-  v8h bq[2][K_PAD / 16u];  // the wave's query operand never changes: it lives in registers
-  float limit[2] = {0.0f, 0.0f};
-#pragma unroll
-  for (int j = 0; j < 2; j++) {
-    qloc[j]             = wq * 64u + uint32_t(j) * 32u + (lane & 31u);
-    q[j]                = q0 + qloc[j];
-    const uint32_t q_rd = q[j] < q_rows ? q[j] : q_rows - 1u;
-#pragma unroll
-    for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) {
-      bq[j][ks] = *reinterpret_cast<const v8h*>(qh + uint64_t(q_rd) * K_PAD + ks * 16u + (lane >> 5) * 8u);
-    }
-    if (PASS == 2) { limit[j] = q[j] < n_queries ? thr[q[j]] / alpha : __uint_as_float(0x7f800000u); }
-  }
-  // Use them once here, so that the compiler's wait for these loads sits here and not inside the
-  // loop: there it would also wait for the staged loads below, which it does not count.
+  // Use the query operand once here, so that the compiler's wait for these loads sits here and not
+  // inside the loop: there it would also wait for the staged loads below, which it does not count.
 #pragma unroll
   for (int j = 0; j < 2; j++) {
 #pragma unroll
@@ -212,8 +216,8 @@ __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
   // compiler sinks them to their first use, behind the matrix products they are meant to overlap
   // (and as volatile loads it waits for each).  It does not count them, so the wait is explicit.
   // Tile numbers past the block's last tile repeat it (no branch around loads or stores).  (Loads
-  // two tiles ahead measured slower, before and after the waves went to 64 queries: the loop is
-  // not waiting on them but on its own phases.)
+  // two tiles ahead, written to LDS half way through the next tile's products, measured the same:
+  // the loop does not wait for them.)
   u32x4 sx[PER_T];
   float cx = 0.0f;
   auto issue = [&](uint32_t tile, u32x4(&st)[PER_T], float& sc) __attribute__((always_inline)) {
@@ -246,62 +250,114 @@ __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
   // products and epilogue of one tile out of LDS buffer `buf`
   auto multiply = [&](uint32_t tile, uint32_t buf) __attribute__((always_inline)) {
     const unsigned char* sa = sa0 + buf * (kTile * ROWB);
-    v16f acc[2][2];  // [list tile][query tile]
+    // element r of an MFMA tile: row (list) (r / 4) * 8 + (lane / 32) * 4 + r % 4, column (query) lane % 32
+    v16f nv[2];  // the norm terms of this lane's rows: where the sums start
 #pragma unroll
     for (int i = 0; i < 2; i++) {
 #pragma unroll
-      for (int j = 0; j < 2; j++) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) { acc[i][j][r] = 0.0f; }
+      for (int g = 0; g < 4; g++) {
+        const float4 t = *reinterpret_cast<const float4*>(scn + buf * kTile + uint32_t(i) * 32u + half * 4u + uint32_t(g) * 8u);
+        nv[i][g * 4 + 0] = t.x;
+        nv[i][g * 4 + 1] = t.y;
+        nv[i][g * 4 + 2] = t.z;
+        nv[i][g * 4 + 3] = t.w;
       }
     }
+    v16f acc[2][2];  // [list tile][query tile]
 #pragma unroll
     for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) {
-      const uint32_t kb = (ks * 16u + (lane >> 5) * 8u) * 2u;  // byte offset of this lane's 8 values
+      const uint32_t kb = (ks * 16u + half * 8u) * 2u;  // byte offset of this lane's 8 values
       v8h a[2];
 #pragma unroll
       for (int i = 0; i < 2; i++) {
-        a[i] = *reinterpret_cast<const v8h*>(sa + (wl * 64u + i * 32u + (lane & 31u)) * ROWB + kb);
+        a[i] = *reinterpret_cast<const v8h*>(sa + (uint32_t(i) * 32u + (lane & 31u)) * ROWB + kb);
       }
 #pragma unroll
       for (int i = 0; i < 2; i++) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], bq[j][ks], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], bq[j][ks], ks == 0 ? nv[i] : acc[i][j], 0, 0, 0);
         }
       }
     }
-    // element r of a tile: row (list) (r / 4) * 8 + (lane / 32) * 4 + r % 4, column (query) lane % 32
-    const uint32_t l0 = tile * kTile;
+    if (PASS == 1) {
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      uint32_t hits = 0;  // PASS 2: bit (i * 16 + r) set when that list is a candidate of query j
+      for (int j = 0; j < 2; j++) {
 #pragma unroll
-      for (int i = 0; i < 2; i++) {
-        const uint32_t rbase = wl * 64u + i * 32u + (lane >> 5) * 4u;  // row inside the block tile
-        float best           = neg_inf;
+        for (int i = 0; i < 2; i++) {
+          float best = neg_inf;
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const uint32_t row = rbase + (r >> 2) * 8u + (r & 3);
-          const float v      = acc[i][j][r] + scn[buf * kTile + row];
-          if (PASS == 1) {
-            best = fmaxf(best, v);  // NaN scores are ignored here and never pass the threshold
-          } else {
-            hits |= (v >= limit[j]) ? (1u << (i * 16 + r)) : 0u;
-          }
-        }
-        if (PASS == 1) {
-          lmin[qloc[j] * (kTilesPerBlock * 8u) + (tile - t0) * 8u + ((wl * 64u + i * 32u) >> 4) + (lane >> 5)] = alpha * best;
+          for (int r = 0; r < 16; r++) { best = fmaxf(best, acc[i][j][r]); }  // NaN scores are ignored here and never pass the threshold
+          lmin[qloc[j] * kMinRow + (tile % kFlushTiles) * 4u + uint32_t(i) * 2u + half] = alpha * best;
         }
       }
-      if (PASS == 2 && hits != 0) {
-        uint32_t slot = atomicAdd(&lcount[qloc[j]], uint32_t(__popc(hits)));
+    } else {
+      // bit (j * 32 + i * 16 + r) of `hits`: that list is a candidate of query j.  The sign of
+      // v - limit is shifted in element by element (two instructions an element), last element
+      // lowest: set bits are misses.  A NaN may land on either side: a NaN candidate sends the
+      // query to the plain path when it is rescored.
+      uint32_t miss[2];
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        uint32_t m      = 0;
+        const float lim = limit[j] * inv_alpha;  // alpha is -1 or -2: exact
+#pragma unroll
+        for (int i = 1; i >= 0; i--) {
+#pragma unroll
+          for (int r = 15; r >= 0; r--) { m = __builtin_amdgcn_alignbit(m, __float_as_uint(acc[i][j][r] - lim), 31); }
+        }
+        miss[j] = m;
+      }
+      unsigned long long hits = ~((static_cast<unsigned long long>(miss[1]) << 32) | miss[0]);
+      if (hits != 0) {
+        uint32_t slot[2];
+        slot[0] = atomicAdd(&lcount[qloc[0]], uint32_t(__popc(~miss[0])));
+        slot[1] = atomicAdd(&lcount[qloc[1]], uint32_t(__popc(~miss[1])));
         while (hits != 0) {
-          const uint32_t bit = __builtin_ctz(hits);
+          const uint32_t bit = uint32_t(__builtin_ctzll(hits));
           hits &= hits - 1u;
-          const uint32_t row = wl * 64u + (bit >> 4) * 32u + (lane >> 5) * 4u + ((bit & 15u) >> 2) * 8u + (bit & 3u);
-          if (slot < kLocalCap) { lcand[qloc[j] * kLocalCap + slot] = l0 + row; }
-          slot++;
+          const uint32_t j   = bit >> 5;
+          const uint32_t row = ((bit >> 4) & 1u) * 32u + half * 4u + ((bit & 15u) >> 2) * 8u + (bit & 3u);
+          const uint32_t s   = j ? slot[1]++ : slot[0]++;
+          if (s < kLocalCap) { lcand[(j ? qloc[1] : qloc[0]) * kLocalCap + s] = tile * kTile + row; }
+        }
+      }
+    }
+  };
+  // The wave writes out what it has staged for its 64 queries since the last flush (its own LDS
+  // writes, in order: no barrier).  PASS 1: the minima of tiles [first, tile], parts of one
+  // 128-byte line per query, 8 queries an instruction.  PASS 2: a lane per query.
+  auto flush = [&](uint32_t tile) __attribute__((always_inline)) {
+    if (PASS == 1) {
+      const uint32_t slot  = tile % kFlushTiles;
+      const uint32_t line  = tile - slot;                        // first tile of the line
+      const uint32_t lo    = line < t0 ? t0 - line : 0u;         // the block's first part of it
+      const uint32_t part  = lane & 7u;
+      // (all eight reads first and the stores after them measured 20 % slower for the whole kernel)
+#pragma unroll
+      for (uint32_t it = 0; it < 8; it++) {
+        const uint32_t ql = wid * 64u + it * 8u + (lane >> 3);
+        if (part >= lo && part <= slot && q0 + ql < n_queries) {
+          *reinterpret_cast<float4*>(minima + uint64_t(q0 + ql) * n_groups + (line + part) * 4u) =
+            *reinterpret_cast<const float4*>(lmin + ql * kMinRow + part * 4u);
+        }
+      }
+    } else {
+      const uint32_t ql = wid * 64u + lane;
+      const uint32_t n  = lcount[ql];
+      if (n != 0) {
+        lcount[ql] = 0;
+        if (q0 + ql < n_queries) {
+          // more than the block can hold: push the query's count past the limit, it will be redone
+          // by the plain path
+          const uint32_t claim = n <= kLocalCap ? n : kCandCapF + 1u;
+          const uint32_t base  = atomicAdd(&cand_count[q0 + ql], claim);
+          if (n <= kLocalCap) {
+            for (uint32_t e = 0; e < n; e++) {
+              const uint32_t l = lcand[ql * kLocalCap + e];
+              if (base + e < kCandCapF && l < n_lists) { cand[uint64_t(q0 + ql) * kCandCapF + base + e] = l; }
+            }
+          }
         }
       }
     }
@@ -311,34 +367,12 @@ __global__ __launch_bounds__(kGemmThreads, 1) void coarse_f16_kernel(
     const uint32_t buf = (tile - t0) & 1u;
     issue(tile + 1u, sx, cx);
     multiply(tile, buf);
+    if ((tile + 1u) % kFlushTiles == 0 || tile + 1u == t1) { flush(tile); }
     arrived(sx, cx);
     commit(tile + 1u, buf ^ 1u, sx, cx);
-    __syncthreads();
-  }
-
-  if (PASS == 1) {
-    // the block's minima, 8 per tile and query, in runs of consecutive groups
-    const uint32_t n_local = (t1 - t0) * 8u;
-    for (uint32_t e = tid; e < kQTile * n_local; e += kGemmThreads) {
-      const uint32_t ql = e / n_local, g = e - ql * n_local;
-      if (q0 + ql < n_queries) {
-        minima[uint64_t(q0 + ql) * n_groups + t0 * 8u + g] = lmin[ql * (kTilesPerBlock * 8u) + g];
-      }
-    }
-  }
-  if (PASS == 2 && tid < kQTile && q0 + tid < n_queries) {
-    const uint32_t n = lcount[tid];
-    if (n != 0) {
-      // more than the block can hold: push the query's count past the limit, it will be redone by
-      // the plain path
-      const uint32_t claim = n <= kLocalCap ? n : kCandCapF + 1u;
-      const uint32_t base  = atomicAdd(&cand_count[q0 + tid], claim);
-      if (n <= kLocalCap) {
-        for (uint32_t e = 0; e < n; e++) {
-          if (base + e < kCandCapF) { cand[uint64_t(q0 + tid) * kCandCapF + base + e] = lcand[tid * kLocalCap + e]; }
-        }
-      }
-    }
+    // the barrier orders LDS traffic only (the staged tile); the flushes' global stores stay in
+    // flight across it
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   }
 }
 
@@ -571,14 +605,15 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
   // list tiles per block: the queries of a block are loaded once for all of them
   const uint32_t n_list_tiles = l_pad / kTile;
   // A block costs about two tile-times of set-up besides its tiles, and the grid runs in rounds of
-  // one block per CU: take the run length whose rounds x (tiles + 2) is smallest.
-  const int n_cu = device_cu_count();
+  // two blocks per CU: take the run length whose rounds x (tiles + 2) is smallest (the longest of
+  // those: fewer blocks load the queries).
+  const uint64_t n_slots   = uint64_t(device_cu_count()) * 2u;
   const uint32_t n_qblocks = (q_pad + kQTile - 1) / kQTile;
   uint32_t tiles_per_block = 1;
   uint64_t best_cost       = ~uint64_t(0);
-  for (uint32_t t = 1; t <= std::min<uint32_t>(kTilesPerBlock, n_list_tiles); t++) {
+  for (uint32_t t = 1; t <= n_list_tiles; t++) {
     const uint64_t blocks = uint64_t((n_list_tiles + t - 1) / t) * n_qblocks;
-    const uint64_t rounds = (blocks + uint64_t(n_cu) - 1) / uint64_t(n_cu);
+    const uint64_t rounds = (blocks + n_slots - 1) / n_slots;
     const uint64_t cost   = rounds * (t + 2);
     if (cost <= best_cost) {
       best_cost       = cost;
@@ -589,7 +624,7 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
   auto run_pass = [&](auto k1, auto k2) {
     // list tiles (two buffers), their norm terms, and the larger of the two passes' per-query areas
     const size_t smem = size_t(2) * kTile * (k_pad * 2 + 16) + 2 * kTile * 4 +
-                        std::max<size_t>(size_t(kQTile) * kTilesPerBlock * 8 * 4, size_t(kQTile) * (1 + kLocalCap) * 4);
+                        std::max<size_t>(size_t(kQTile) * kMinRow * 4, size_t(kQTile) * (1 + kLocalCap) * 4);
     // a generic lambda has one body per pair of argument types, and the kernels of both K_PAD
     // values have the same type: the flag is keyed by K_PAD explicitly
     lds_limit_once(k_pad == 64 ? 0 : 1, k1, k2, smem);
