@@ -270,7 +270,6 @@ constexpr uint32_t kStatSlots = 256;
 void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
                           uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
                           uint32_t* n_samples, unsigned long long* stats, uint32_t lead_probes,
-                          uint32_t* pair_counts, uint32_t n_lists, const uint32_t* list_rank,
                           hipStream_t stream);
 
 /** Everything the scan needs to know about one (query, probe) pair, gathered once so that the
@@ -291,15 +290,16 @@ static_assert(sizeof(pair_desc) == 32, "pair_desc must stay 32 bytes");
  *  of each query's first `lead_probes` probes come first (n_queries * lead_probes records, grouped
  *  by list) and the others after them (grouped by list again); `alive`, when non-null, gets one
  *  byte per pair slot: 1 for the leading pairs, 0 for the others.  `counters` is scratch of
- *  4 * n_lists + 4 words; with `counted` its first half already holds the histogram of the pairs
- *  (launch_chunk_indices with `pair_counts` makes it on the way).  `list_rank` (n_lists words, a
- *  permutation; null: the identity) gives the order of the groups of leading pairs: group of list
- *  l at position list_rank[l]; both launchers must be given the same table. */
+ *  4 * n_lists + 4 words, `sort_scratch` of order_pairs_scratch_bytes() bytes (256-byte aligned;
+ *  null: the order is made with global atomics).  `list_rank` (n_lists words, a permutation; null:
+ *  the identity) gives the order of the groups of leading pairs: group of list l at position
+ *  list_rank[l]. */
+size_t order_pairs_scratch_bytes(uint32_t n_pairs, uint32_t n_probes, uint32_t n_lists, uint32_t lead_probes);
 void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
                         const uint8_t* const* data_ptrs, const int64_t* const* inds_ptrs,
                         const int64_t* ids_base, uint32_t n_pairs, uint32_t n_probes,
-                        uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
-                        pair_desc* desc, uint32_t lead_probes, uint8_t* alive, bool counted, bool natural_order,
+                        uint32_t n_lists, uint32_t* counters, void* sort_scratch, uint32_t* pair_order,
+                        pair_desc* desc, uint32_t lead_probes, uint8_t* alive, bool natural_order,
                         const uint32_t* list_rank, hipStream_t stream);
 
 struct scan_args {

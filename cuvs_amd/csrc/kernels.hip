@@ -419,10 +419,7 @@ __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __res
                                                             uint32_t* __restrict__ chunk_indices,
                                                             uint32_t* __restrict__ n_samples,
                                                             unsigned long long* stats,
-                                                            uint32_t lead_probes,
-                                                            uint32_t* __restrict__ pair_counts,
-                                                            uint32_t n_lists,
-                                                            const uint32_t* __restrict__ rank)
+                                                            uint32_t lead_probes)
 {
   const uint32_t q    = blockIdx.x;
   const uint32_t lane = threadIdx.x;
@@ -434,8 +431,6 @@ __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __res
     if (p < n_probes) {
       const uint32_t label = probes[uint64_t(q) * n_probes + p];
       sz                   = list_sizes[label];
-      // histogram of the pair ordering, while the probe is at hand
-      if (pair_counts != nullptr) { atomicAdd(&pair_counts[pair_bin(label, p, n_probes, lead_probes, n_lists, rank)], 1u); }
     }
     padded_rows += (sz + 31u) & ~31u;
     if (p < lead_probes) { lead_rows += (sz + 31u) & ~31u; }
@@ -521,6 +516,33 @@ __global__ __launch_bounds__(kScanThreads) void exclusive_scan_kernel(const uint
   }
 }
 
+/** Pair i goes to position `pos` of the order: its id, its record, its byte of `alive`. */
+__device__ __forceinline__ void place_pair(uint32_t i, uint32_t pos, uint32_t label,
+                                           const uint32_t* __restrict__ chunk_indices,
+                                           const uint8_t* const* __restrict__ data_ptrs,
+                                           const int64_t* const* __restrict__ inds_ptrs,
+                                           const int64_t* ids_base, uint32_t n_probes, uint32_t lead_probes,
+                                           uint32_t* __restrict__ pair_order, pair_desc* __restrict__ desc,
+                                           uint8_t* __restrict__ alive)
+{
+  pair_order[pos] = i;
+  if (alive != nullptr) { alive[i] = (i % n_probes) < lead_probes ? 1 : 0; }
+  if (desc != nullptr) {
+    const uint32_t q   = i / n_probes;
+    const uint32_t p   = i - q * n_probes;
+    const uint32_t off = p > 0 ? chunk_indices[i - 1] : 0u;
+    pair_desc d;
+    d.data       = data_ptrs[label];
+    d.q          = q;
+    d.slot       = i;
+    d.label      = label;
+    d.sample_off = off;
+    d.n_rows     = chunk_indices[i] - off;
+    d.row_off    = uint32_t(inds_ptrs[label] - ids_base);
+    desc[pos]    = d;
+  }
+}
+
 __global__ void pair_scatter_kernel(const uint32_t* __restrict__ probes,
                                     const uint32_t* __restrict__ chunk_indices,
                                     const uint8_t* const* __restrict__ data_ptrs,
@@ -538,21 +560,247 @@ __global__ void pair_scatter_kernel(const uint32_t* __restrict__ probes,
     const uint32_t pos = cursors != nullptr
                            ? atomicAdd(&cursors[pair_bin(label, i, n_probes, lead_probes, n_lists, rank)], 1u)
                            : i;
-    pair_order[pos]    = i;
-    if (alive != nullptr) { alive[i] = (i % n_probes) < lead_probes ? 1 : 0; }
-    if (desc != nullptr) {
-      const uint32_t q   = i / n_probes;
-      const uint32_t p   = i - q * n_probes;
-      const uint32_t off = p > 0 ? chunk_indices[i - 1] : 0u;
-      pair_desc d;
-      d.data       = data_ptrs[label];
-      d.q          = q;
-      d.slot       = i;
-      d.label      = label;
-      d.sample_off = off;
-      d.n_rows     = chunk_indices[i] - off;
-      d.row_off    = uint32_t(inds_ptrs[label] - ids_base);
-      desc[pos]    = d;
+    place_pair(i, pos, label, chunk_indices, data_ptrs, inds_ptrs, ids_base, n_probes, lead_probes, pair_order, desc,
+               alive);
+  }
+}
+
+/*
+ * The pair order as a two-level counting sort.  A global atomic per pair (one for the histogram,
+ * one for the position) costs about 60 ns of memory-side atomic throughput at 640,000 pairs; here
+ * every count is an LDS atomic.  Level one splits the bins (lists) into at most kOrderBuckets
+ * buckets of 2^shift consecutive bins: blocks of kOrderThreads threads count their chunk of pairs
+ * per bucket (pair_bucket_count_kernel); every block then finds its range inside every bucket from
+ * the table of (bucket, block) counts and moves (list, pair) records there
+ * (pair_bucket_move_kernel).  Level two takes one block per bucket: it counts the bucket's records
+ * per bin in LDS, scans, and places every pair (pair_bucket_finish_kernel).  The loops request
+ * kOrderUnroll pairs' worth of loads at a time: every pair is a chain of dependent loads
+ * (probe -> rank, record -> list pointers), and a block has few pairs per thread.
+ */
+constexpr uint32_t kOrderBuckets = 512;
+constexpr uint32_t kOrderThreads = 1024;
+constexpr uint32_t kOrderUnroll  = 4;
+constexpr uint32_t kOrderChunk   = kOrderThreads * kOrderUnroll;  // pairs per block
+constexpr uint32_t kOrderFineMax = 8192;  // bins per bucket (LDS words of the last kernel)
+
+__global__ __launch_bounds__(kOrderThreads) void pair_bucket_count_kernel(
+  const uint32_t* __restrict__ probes, uint32_t n_pairs, uint32_t n_probes, uint32_t lead_probes,
+  uint32_t n_lists, const uint32_t* __restrict__ rank, uint32_t shift, uint32_t* __restrict__ block_counts)
+{
+  __shared__ uint32_t hist[kOrderBuckets];
+  const uint32_t tid = threadIdx.x;
+  if (tid < kOrderBuckets) { hist[tid] = 0; }
+  __syncthreads();
+  const uint32_t i0 = blockIdx.x * kOrderChunk;
+  const uint32_t i1 = i0 + kOrderChunk < n_pairs ? i0 + kOrderChunk : n_pairs;
+  {
+    const uint32_t base = i0 + tid;
+    uint32_t label[kOrderUnroll], bin[kOrderUnroll];
+#pragma unroll
+    for (uint32_t u = 0; u < kOrderUnroll; u++) {
+      const uint32_t i = base + u * kOrderThreads;
+      label[u]         = i < i1 ? probes[i] : 0u;
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < kOrderUnroll; u++) {
+      bin[u] = pair_bin(label[u], base + u * kOrderThreads, n_probes, lead_probes, n_lists, rank);
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < kOrderUnroll; u++) {
+      if (base + u * kOrderThreads < i1) { atomicAdd(&hist[bin[u] >> shift], 1u); }
+    }
+  }
+  __syncthreads();
+  if (tid < kOrderBuckets) { block_counts[blockIdx.x * kOrderBuckets + tid] = hist[tid]; }
+}
+
+/** A record of the first level: what the last kernel needs to know of a pair, gathered while the
+ *  pairs are still in their natural order (the chunk indices of consecutive pairs are neighbours). */
+struct order_record {
+  uint32_t label, pair, sample_off, n_rows;
+};
+
+/** Moves the block's pairs to their buckets.  The block orders its records by bucket in LDS first,
+ *  so that every bucket receives a run of consecutive records from consecutive lanes.  Also writes
+ *  the byte of `alive` of every pair and, from block 0, where every bucket starts. */
+__global__ __launch_bounds__(kOrderThreads) void pair_bucket_move_kernel(
+  const uint32_t* __restrict__ probes, const uint32_t* __restrict__ chunk_indices, uint32_t n_pairs,
+  uint32_t n_probes, uint32_t lead_probes, uint32_t n_lists, const uint32_t* __restrict__ rank,
+  uint32_t shift, uint32_t n_buckets, const uint32_t* __restrict__ block_counts,
+  uint32_t* __restrict__ bucket_start, order_record* __restrict__ records, uint8_t* __restrict__ alive)
+{
+  __shared__ uint32_t hist[kOrderBuckets];    // the block's pairs per bucket, then their local offsets
+  __shared__ uint32_t gbase[kOrderBuckets];   // pairs of the blocks before this one, then the block's global range
+  __shared__ uint32_t totals[kOrderBuckets];  // pairs of all blocks
+  __shared__ uint32_t wave_sums[2][kOrderBuckets / 64];
+  __shared__ order_record staged[kOrderChunk];
+  __shared__ uint16_t staged_bucket[kOrderChunk];
+  const uint32_t tid = threadIdx.x;
+  if (tid < kOrderBuckets) { hist[tid] = 0; }
+  // the table is [block][bucket]: thread (bucket, half) sums every other row of its column in
+  // registers (LDS atomics here cost more than everything else in this kernel)
+  {
+    static_assert(kOrderThreads == 2 * kOrderBuckets, "two threads per bucket");
+    const uint32_t bkt = tid % kOrderBuckets, half = tid / kOrderBuckets;
+    uint32_t total = 0, before = 0;
+#pragma unroll 8
+    for (uint32_t k = half; k < gridDim.x; k += 2) {
+      const uint32_t c = block_counts[k * kOrderBuckets + bkt];
+      total += c;
+      before += k < blockIdx.x ? c : 0u;
+    }
+    if (half == 1) {
+      totals[bkt] = total;
+      gbase[bkt]  = before;
+    }
+    __syncthreads();
+    if (half == 0) {
+      totals[bkt] += total;
+      gbase[bkt] += before;
+    }
+  }
+  const uint32_t i0 = blockIdx.x * kOrderChunk;
+  const uint32_t i1 = i0 + kOrderChunk < n_pairs ? i0 + kOrderChunk : n_pairs;
+  order_record rec[kOrderUnroll];
+  uint32_t bucket[kOrderUnroll], local[kOrderUnroll];
+#pragma unroll
+  for (uint32_t u = 0; u < kOrderUnroll; u++) {
+    const uint32_t i = i0 + tid + u * kOrderThreads;
+    const bool in    = i < i1;
+    rec[u].label     = in ? probes[i] : 0u;
+    rec[u].pair      = i;
+    const uint32_t incl = in ? chunk_indices[i] : 0u;
+    rec[u].sample_off   = in && (i % n_probes) != 0 ? chunk_indices[i - 1] : 0u;
+    rec[u].n_rows       = incl - rec[u].sample_off;
+    if (in && alive != nullptr) { alive[i] = (i % n_probes) < lead_probes ? 1 : 0; }
+  }
+#pragma unroll
+  for (uint32_t u = 0; u < kOrderUnroll; u++) {
+    bucket[u] = pair_bin(rec[u].label, rec[u].pair, n_probes, lead_probes, n_lists, rank) >> shift;
+  }
+#pragma unroll
+  for (uint32_t u = 0; u < kOrderUnroll; u++) {
+    local[u] = i0 + tid + u * kOrderThreads < i1 ? atomicAdd(&hist[bucket[u]], 1u) : 0u;
+  }
+  __syncthreads();
+  // exclusive scans over the buckets: of the block's counts (local offsets) and of the totals
+  // (bucket starts; plus the blocks before this one: the block's range in the bucket)
+  uint32_t mine = 0, total = 0;
+  if (tid < kOrderBuckets) {
+    mine  = hist[tid];
+    total = totals[tid];
+    const uint32_t incl_m = wave_inclusive_scan(mine);
+    const uint32_t incl_t = wave_inclusive_scan(total);
+    if ((tid & 63u) == 63u) {
+      wave_sums[0][tid >> 6] = incl_m;
+      wave_sums[1][tid >> 6] = incl_t;
+    }
+    mine  = incl_m - mine;
+    total = incl_t - total;
+  }
+  __syncthreads();
+  if (tid < kOrderBuckets) {
+    for (uint32_t w = 0; w < (tid >> 6); w++) {
+      mine += wave_sums[0][w];
+      total += wave_sums[1][w];
+    }
+    hist[tid] = mine;
+    if (blockIdx.x == 0 && tid < n_buckets) { bucket_start[tid] = total; }
+    gbase[tid] += total;
+  }
+  __syncthreads();
+#pragma unroll
+  for (uint32_t u = 0; u < kOrderUnroll; u++) {
+    if (i0 + tid + u * kOrderThreads < i1) {
+      const uint32_t at = hist[bucket[u]] + local[u];
+      staged[at]        = rec[u];
+      staged_bucket[at] = uint16_t(bucket[u]);
+    }
+  }
+  __syncthreads();
+  for (uint32_t at = tid; at < i1 - i0; at += kOrderThreads) {
+    const uint32_t b              = staged_bucket[at];
+    records[gbase[b] + at - hist[b]] = staged[at];
+  }
+}
+
+__global__ __launch_bounds__(kOrderThreads) void pair_bucket_finish_kernel(
+  const order_record* __restrict__ records, const uint32_t* __restrict__ bucket_start, uint32_t n_buckets,
+  uint32_t n_pairs, uint32_t shift, uint32_t n_lists, const uint32_t* __restrict__ rank,
+  const uint8_t* const* __restrict__ data_ptrs, const int64_t* const* __restrict__ inds_ptrs,
+  const int64_t* ids_base, uint32_t n_probes, uint32_t lead_probes, uint32_t* __restrict__ pair_order,
+  pair_desc* __restrict__ desc)
+{
+  extern __shared__ __align__(16) uint32_t fine[];  // 2^shift counts, then cursors
+  __shared__ uint32_t wave_sums[kOrderThreads / 64];
+  constexpr uint32_t U  = 4;
+  const uint32_t tid    = threadIdx.x;
+  const uint32_t b      = blockIdx.x;
+  const uint32_t n_fine = 1u << shift;
+  const uint32_t begin  = bucket_start[b];
+  const uint32_t end    = b + 1 < n_buckets ? bucket_start[b + 1] : n_pairs;
+  for (uint32_t f = tid; f < n_fine; f += kOrderThreads) { fine[f] = 0; }
+  __syncthreads();
+  for (uint32_t base = begin + tid; base < end; base += kOrderThreads * U) {
+    uint32_t label[U], pair[U], bin[U];
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) {
+      const uint32_t e = base + u * kOrderThreads;
+      label[u]         = e < end ? records[e].label : 0u;
+      pair[u]          = e < end ? records[e].pair : 0u;
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) { bin[u] = pair_bin(label[u], pair[u], n_probes, lead_probes, n_lists, rank); }
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) {
+      if (base + u * kOrderThreads < end) { atomicAdd(&fine[bin[u] & (n_fine - 1u)], 1u); }
+    }
+  }
+  __syncthreads();
+  // exclusive scan of the counts: every thread owns a run of consecutive bins
+  const uint32_t per = (n_fine + kOrderThreads - 1) / kOrderThreads;
+  const uint32_t f0  = tid * per;
+  uint32_t sum       = 0;
+  for (uint32_t f = f0; f < f0 + per && f < n_fine; f++) { sum += fine[f]; }
+  const uint32_t incl = wave_inclusive_scan(sum);
+  if ((tid & 63u) == 63u) { wave_sums[tid >> 6] = incl; }
+  __syncthreads();
+  uint32_t run = begin + incl - sum;
+  for (uint32_t w = 0; w < (tid >> 6); w++) { run += wave_sums[w]; }
+  for (uint32_t f = f0; f < f0 + per && f < n_fine; f++) {
+    const uint32_t c = fine[f];
+    fine[f]          = run;
+    run += c;
+  }
+  __syncthreads();
+  for (uint32_t base = begin + tid; base < end; base += kOrderThreads * U) {
+    order_record r[U];
+    uint32_t bin[U];
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) {
+      const uint32_t e = base + u * kOrderThreads;
+      r[u]             = e < end ? records[e] : order_record{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) { bin[u] = pair_bin(r[u].label, r[u].pair, n_probes, lead_probes, n_lists, rank); }
+    pair_desc d[U];
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) {
+      d[u].data       = data_ptrs[r[u].label];
+      d[u].q          = r[u].pair / n_probes;
+      d[u].slot       = r[u].pair;
+      d[u].label      = r[u].label;
+      d[u].sample_off = r[u].sample_off;
+      d[u].n_rows     = r[u].n_rows;
+      d[u].row_off    = uint32_t(inds_ptrs[r[u].label] - ids_base);
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) {
+      if (base + u * kOrderThreads < end) {
+        const uint32_t pos = atomicAdd(&fine[bin[u] & (n_fine - 1u)], 1u);
+        pair_order[pos]    = r[u].pair;
+        if (desc != nullptr) { desc[pos] = d[u]; }
+      }
     }
   }
 }
@@ -1220,25 +1468,47 @@ void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries,
 void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
                           uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
                           uint32_t* n_samples, unsigned long long* stats, uint32_t lead_probes,
-                          uint32_t* pair_counts, uint32_t n_lists, const uint32_t* list_rank,
                           hipStream_t stream)
 {
   if (n_queries == 0) { return; }
-  if (pair_counts != nullptr) {
-    launch_fill_u32(pair_counts, 0, lead_probes < n_probes ? 2 * n_lists : n_lists, stream);
-  }
   chunk_indices_kernel<<<n_queries, 64, 0, stream>>>(list_sizes, probes, n_probes, row_chunk_bytes,
-                                                     chunk_indices, n_samples, stats, lead_probes,
-                                                     pair_counts, n_lists, list_rank);
+                                                     chunk_indices, n_samples, stats, lead_probes);
   CUVS_LAUNCH_CHECK();
+}
+
+namespace {
+struct order_shape {
+  uint32_t n_bins, shift, n_buckets, chunk, n_blocks;
+  bool sorted;  // the two-level sort takes it (otherwise: global atomics)
+};
+order_shape shape_order(uint32_t n_pairs, uint32_t n_probes, uint32_t n_lists, uint32_t lead_probes)
+{
+  order_shape o{};
+  o.n_bins = lead_probes < n_probes ? 2 * n_lists : n_lists;
+  while (((o.n_bins + (1u << o.shift) - 1) >> o.shift) > kOrderBuckets) { o.shift++; }
+  o.n_buckets = (o.n_bins + (1u << o.shift) - 1) >> o.shift;
+  // every block reads the table of blocks x buckets counts: beyond 1024 blocks (4 M pairs) that
+  // costs more than the atomics it saves
+  o.chunk    = kOrderChunk;
+  o.n_blocks = (n_pairs + o.chunk - 1) / o.chunk;
+  o.sorted   = (1u << o.shift) <= kOrderFineMax && o.n_blocks <= 1024;
+  return o;
+}
+}  // namespace
+
+size_t order_pairs_scratch_bytes(uint32_t n_pairs, uint32_t n_probes, uint32_t n_lists, uint32_t lead_probes)
+{
+  const order_shape o = shape_order(n_pairs, n_probes, n_lists, lead_probes);
+  const size_t words  = size_t(kOrderBuckets) * o.n_blocks + kOrderBuckets;
+  return ((words * 4 + 255) & ~size_t(255)) + size_t(n_pairs) * sizeof(order_record) + 256;
 }
 
 void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
                         const uint8_t* const* data_ptrs, const int64_t* const* inds_ptrs,
                         const int64_t* ids_base, uint32_t n_pairs, uint32_t n_probes,
-                        uint32_t n_lists, uint32_t* counters, uint32_t* pair_order,
-                        pair_desc* desc, uint32_t lead_probes, uint8_t* alive, bool counted,
-                        bool natural_order, const uint32_t* list_rank, hipStream_t stream)
+                        uint32_t n_lists, uint32_t* counters, void* sort_scratch, uint32_t* pair_order,
+                        pair_desc* desc, uint32_t lead_probes, uint8_t* alive, bool natural_order,
+                        const uint32_t* list_rank, hipStream_t stream)
 {
   if (n_pairs == 0) { return; }
   if (natural_order) {
@@ -1249,25 +1519,41 @@ void launch_order_pairs(const uint32_t* probes, const uint32_t* chunk_indices,
     CUVS_LAUNCH_CHECK();
     return;
   }
-  const uint32_t n_bins = lead_probes < n_probes ? 2 * n_lists : n_lists;
-  uint32_t* counts      = counters;
-  uint32_t* cursors     = counters + n_bins;
-  if (!counted) {
-    launch_fill_u32(counts, 0, n_bins, stream);
-    pair_histogram_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(probes, n_pairs, n_probes,
-                                                                        lead_probes, n_lists, list_rank, counts);
+  const order_shape o = shape_order(n_pairs, n_probes, n_lists, lead_probes);
+  if (o.sorted && sort_scratch != nullptr) {
+    const uint32_t n_words = kOrderBuckets * o.n_blocks;
+    uint32_t* block_counts = static_cast<uint32_t*>(sort_scratch);
+    uint32_t* bucket_start = block_counts + n_words;
+    order_record* records = reinterpret_cast<order_record*>(static_cast<char*>(sort_scratch) +
+                                                            ((size_t(n_words + kOrderBuckets) * 4 + 255) & ~size_t(255)));
+    pair_bucket_count_kernel<<<o.n_blocks, kOrderThreads, 0, stream>>>(probes, n_pairs, n_probes, lead_probes, n_lists,
+                                                                      list_rank, o.shift, block_counts);
     CUVS_LAUNCH_CHECK();
+    pair_bucket_move_kernel<<<o.n_blocks, kOrderThreads, 0, stream>>>(probes, chunk_indices, n_pairs, n_probes,
+                                                                     lead_probes, n_lists, list_rank, o.shift, o.n_buckets,
+                                                                     block_counts, bucket_start, records, alive);
+    CUVS_LAUNCH_CHECK();
+    pair_bucket_finish_kernel<<<o.n_buckets, kOrderThreads, size_t(4) << o.shift, stream>>>(
+      records, bucket_start, o.n_buckets, n_pairs, o.shift, n_lists, list_rank, data_ptrs, inds_ptrs, ids_base, n_probes,
+      lead_probes, pair_order, desc);
+    CUVS_LAUNCH_CHECK();
+    return;
   }
-  {
-    const size_t smem = size_t(kScanTile + kScanThreads) * 4;
-    static const int attr_set = [&] {
-      CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(exclusive_scan_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
-      return 1;
-    }();
-    (void)attr_set;
-    exclusive_scan_kernel<<<1, kScanThreads, smem, stream>>>(counts, n_bins, cursors);
-  }
+  // more bins than the two levels take: a global atomic per pair for the histogram, one for its position
+  const size_t scan_smem    = size_t(kScanTile + kScanThreads) * 4;
+  static const int attr_set = [&] {
+    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(exclusive_scan_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(scan_smem)));
+    return 1;
+  }();
+  (void)attr_set;
+  uint32_t* counts  = counters;
+  uint32_t* cursors = counters + o.n_bins;
+  launch_fill_u32(counts, 0, o.n_bins, stream);
+  pair_histogram_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(probes, n_pairs, n_probes, lead_probes, n_lists,
+                                                                      list_rank, counts);
+  CUVS_LAUNCH_CHECK();
+  exclusive_scan_kernel<<<1, kScanThreads, scan_smem, stream>>>(counts, o.n_bins, cursors);
   CUVS_LAUNCH_CHECK();
   pair_scatter_kernel<<<blocks_for(n_pairs, 256), 256, 0, stream>>>(
     probes, chunk_indices, data_ptrs, inds_ptrs, ids_base, n_pairs, n_probes, lead_probes, n_lists,

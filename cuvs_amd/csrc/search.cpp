@@ -94,9 +94,9 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
   const size_t P = p.n_probes;
   p.per_query_bytes = size_t(ix.dim) * 4 + size_t(ix.dim_ext) * 4 + size_t(ix.n_lists) * 4 +
                       size_t(ix.rot_dim) * 4 +
-                      P * 4 * 3 + P * (2 * sizeof(detail::pair_desc) + 1) + 16 +
+                      P * 4 * 3 + P * (2 * sizeof(detail::pair_desc) + 1) + 16 + P * 17 +
                       (p.fused ? P * k * 8 * 4 : size_t(p.max_samples) * 4);
-  p.fixed_bytes = a256(size_t(ix.n_lists) * 16 + 16) + a256(size_t(ix.dim_ext) * 128 * 4) + a256(detail::kSelectSlackBytes) + 16 * 256;
+  p.fixed_bytes = a256(size_t(ix.n_lists) * 16 + 16) + 3 * 256 + size_t(512) * 8 + a256(size_t(ix.dim_ext) * 128 * 4) + a256(detail::kSelectSlackBytes) + 16 * 256;
   if (ix.coarse_fast_ok) {
     // buffers of the two-precision probe selection (the batch must fit with them)
     p.per_query_bytes += size_t(detail::coarse_fast_k_pad(ix.dim)) * 2 + size_t(detail::coarse_fast_groups(ix.n_lists)) * 4 +
@@ -443,6 +443,8 @@ void search(cuvs::resources const& res_c,
     observe_screen = early_stop && capture == hipStreamCaptureStatusNone;
   }
   const uint32_t lead          = early_stop ? kLeadProbes : P;
+  void* sort_scratch = few_pairs ? nullptr
+                                 : res.workspace_alloc(detail::order_pairs_scratch_bytes(Qb * P, P, ix.n_lists, lead));
   detail::pair_desc* survivors = nullptr;
   uint8_t* alive               = nullptr;
   uint32_t* n_survivors        = nullptr;
@@ -493,11 +495,10 @@ void search(cuvs::resources const& res_c,
     detail::launch_rotate(qf, ix.rotation_t.as<float>(), nq, ix.dim, ix.rot_dim,
                           ix.rotation_is_identity, cosine, params.coarse_search_dtype, rot_q, s);
     detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
-                                 ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead,
-                                 few_pairs ? nullptr : counters, ix.n_lists, list_rank, s);
+                                 ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead, s);
     detail::launch_order_pairs(probes, chunk, ix.data_ptrs.as<const uint8_t*>(),
                                ix.inds_ptrs.as<const int64_t*>(), ix.ids_arena.as<int64_t>(), nq * P, P,
-                               ix.n_lists, counters, order, desc, lead, alive, true, few_pairs, list_rank, s);
+                               ix.n_lists, counters, sort_scratch, order, desc, lead, alive, few_pairs, list_rank, s);
     if (pl.fused) { detail::launch_fill_u32(kth, 0xFFFFFFFFu, nq, s); }
     mark(2);
 
