@@ -412,6 +412,7 @@ struct merge_args {
   float scaling;
   const unsigned long long* in_keys;  // fused
   const uint8_t* alive;               // fused: per pair slot, 0 = no keys were written (or null: all)
+  uint8_t* redo;                      // with alive: scratch, a byte per query (null: one kernel does all)
   const float* in_scores;             // non-fused
   const uint32_t* n_samples;
   const uint32_t* probes;

@@ -11,6 +11,7 @@
  * element in ascending index order; lookup-table entries are built in fp32 and rounded once.
  */
 #include "device_utils.cuh"
+#include "scan_wave_select.cuh"
 
 #include <algorithm>
 
@@ -1061,13 +1062,123 @@ __global__ __launch_bounds__(64) void kth_bound_kernel(const unsigned long long*
   }
 }
 
+/** Output row r of query q from its r-th best key: the sample number inside the query's probed
+ *  lists back to a list and a row (find_chunk_ix, cpp/src/neighbors/ivf_common.cuh:94-110), the
+ *  distance in the metric's final form.  `chunk` and `probes` are the query's rows. */
+__device__ __forceinline__ void write_neighbor(const merge_args& a, uint32_t q, uint32_t r, unsigned long long key,
+                                               const uint32_t* chunk, const uint32_t* probes)
+{
+  int64_t id = INT64_MAX;  // kOutOfBoundsRecord
+  float d    = FLT_MAX;
+  if (key != kInvalidKey) {
+    uint32_t sample = uint32_t(key);
+    d               = unorder_f32(uint32_t(key >> 32));
+    uint32_t lo = 0, hi = a.n_probes;
+    do {
+      const uint32_t mid = (lo + hi) >> 1;
+      if (chunk[mid] <= sample) {
+        lo = mid + 1;
+      } else {
+        hi = mid;
+      }
+    } while (lo < hi);
+    if (lo < a.n_probes) {
+      if (lo > 0) { sample -= chunk[lo - 1]; }
+      id = a.inds_ptrs[probes[lo]][sample];
+    }
+  }
+  a.neighbors[uint64_t(q) * a.k + r] = id;
+  a.distances[uint64_t(q) * a.k + r] = postprocess_distance(d, a.metric, a.scaling);
+}
+
+/**
+ * The merge after an early stop, one wave per query: most pairs were dropped by the screen and
+ * wrote no keys, a handful is left (a.alive).  The wave lists the live pairs, packs their valid
+ * keys into LDS (a pair's block of keys is mostly padding), keeps the k smallest by the wave's
+ * radix selection, ranks those against each other (keys are distinct: the sample number is part of
+ * the key) and writes them out; the query's chunk indices and probes sit in LDS for the search
+ * from sample number to list.  A query with more than kLiveSmall valid keys is left to
+ * merge_redo_kernel (a.redo[q] = 1).
+ */
+constexpr uint32_t kLiveSmall = 512;
+__global__ __launch_bounds__(64) void merge_live_kernel(merge_args a)
+{
+  extern __shared__ __align__(16) unsigned char dyn_smem[];
+  unsigned long long* small_keys = reinterpret_cast<unsigned long long*>(dyn_smem);  // [kLiveSmall]
+  unsigned long long* out        = small_keys + kLiveSmall;                          // [k]
+  uint32_t* chunk                = reinterpret_cast<uint32_t*>(out + a.k);           // [n_probes]
+  uint32_t* probes               = chunk + a.n_probes;                               // [n_probes]
+  uint16_t* live                 = reinterpret_cast<uint16_t*>(probes + a.n_probes);  // [n_probes]
+  const uint32_t q    = blockIdx.x;
+  const uint32_t lane = threadIdx.x;
+  const uint32_t kpp  = a.keys_per_pair;
+  const unsigned long long* keys = a.in_keys + uint64_t(q) * a.n_probes * kpp;
+  const uint8_t* alive           = a.alive + uint64_t(q) * a.n_probes;
+  uint32_t n_live                = 0;
+  for (uint32_t p0 = 0; p0 < a.n_probes; p0 += 64) {
+    const uint32_t p = p0 + lane;
+    bool al          = false;
+    if (p < a.n_probes) {
+      al        = alive[p] != 0;
+      chunk[p]  = a.chunk_indices[uint64_t(q) * a.n_probes + p];
+      probes[p] = a.probes[uint64_t(q) * a.n_probes + p];
+    }
+    const unsigned long long mask = __builtin_amdgcn_ballot_w64(al);
+    if (al) { live[n_live + __builtin_amdgcn_mbcnt_hi(uint32_t(mask >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(mask), 0u))] = uint16_t(p); }
+    n_live += uint32_t(__popcll(mask));
+  }
+  __syncthreads();
+  // the valid keys of the live pairs, packed; lanes walk a pair's keys, pair after pair
+  const uint32_t n_keys = n_live * kpp;
+  uint32_t n_valid      = 0;
+  constexpr uint32_t U  = 4;  // keys a lane requests at a time: a query with many live pairs is a chain of loads
+  for (uint32_t i0 = 0; i0 < n_keys && n_valid <= kLiveSmall; i0 += 64 * U) {
+    unsigned long long key[U];
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) {
+      const uint32_t i = i0 + u * 64 + lane;
+      key[u]           = kInvalidKey;
+      if (i < n_keys) {
+        const uint32_t pair = i / kpp;
+        key[u]              = keys[uint32_t(live[pair]) * kpp + (i - pair * kpp)];
+      }
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < U; u++) {
+      const bool valid              = key[u] != kInvalidKey;
+      const unsigned long long mask = __builtin_amdgcn_ballot_w64(valid);
+      const uint32_t at = n_valid + __builtin_amdgcn_mbcnt_hi(uint32_t(mask >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(mask), 0u));
+      if (valid && at < kLiveSmall) { small_keys[at] = key[u]; }
+      n_valid += uint32_t(__popcll(mask));
+    }
+  }
+  if (lane == 0) { a.redo[q] = n_valid > kLiveSmall ? 1 : 0; }
+  if (n_valid > kLiveSmall) { return; }
+  for (uint32_t r = lane; r < a.k; r += 64) { out[r] = kInvalidKey; }
+  __syncthreads();
+  uint32_t m = n_valid;
+  if (n_valid > a.k) {
+    wave_select_keys<int(kLiveSmall / 64)>((LDS_AS unsigned long long*)small_keys, lane, n_valid, a.k);
+    m = a.k;
+  }
+  __syncthreads();
+  for (uint32_t i = lane; i < m; i += 64) {
+    const unsigned long long key = small_keys[i];
+    uint32_t rank                = 0;
+    for (uint32_t j = 0; j < m; j++) { rank += small_keys[j] < key ? 1u : 0u; }
+    out[rank] = key;
+  }
+  __syncthreads();
+  for (uint32_t r = lane; r < a.k; r += 64) { write_neighbor(a, q, r, out[r], chunk, probes); }
+}
+
 constexpr uint32_t kMergeMaxProbes = 8192;  // with the alive list: slots are kept as 16-bit numbers
-__global__ __launch_bounds__(kBlock) void merge_kernel(merge_args a, uint32_t out_cap)
+/** The k best of query q, by the whole block. */
+__device__ void merge_query(const merge_args& a, uint32_t out_cap, uint32_t q)
 {
   extern __shared__ __align__(16) unsigned char dyn_smem[];
   __shared__ select_smem sm;
   unsigned long long* out = reinterpret_cast<unsigned long long*>(dyn_smem);
-  const uint32_t q        = blockIdx.x;
   uint32_t n;
   if (a.fused) {
     n                              = a.n_probes * a.keys_per_pair;
@@ -1124,30 +1235,26 @@ __global__ __launch_bounds__(kBlock) void merge_kernel(merge_args a, uint32_t ou
   }
   const uint32_t* chunk  = a.chunk_indices + uint64_t(q) * a.n_probes;
   const uint32_t* probes = a.probes + uint64_t(q) * a.n_probes;
-  for (uint32_t r = threadIdx.x; r < a.k; r += kBlock) {
-    const unsigned long long key = out[r];
-    int64_t id                   = INT64_MAX;  // kOutOfBoundsRecord
-    float d                      = FLT_MAX;
-    if (key != kInvalidKey) {
-      uint32_t sample = uint32_t(key);
-      d               = unorder_f32(uint32_t(key >> 32));
-      // find_chunk_ix (cpp/src/neighbors/ivf_common.cuh:94-110)
-      uint32_t lo = 0, hi = a.n_probes;
-      do {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (chunk[mid] <= sample) {
-          lo = mid + 1;
-        } else {
-          hi = mid;
-        }
-      } while (lo < hi);
-      if (lo < a.n_probes) {
-        if (lo > 0) { sample -= chunk[lo - 1]; }
-        id = a.inds_ptrs[probes[lo]][sample];
-      }
-    }
-    a.neighbors[uint64_t(q) * a.k + r] = id;
-    a.distances[uint64_t(q) * a.k + r] = postprocess_distance(d, a.metric, a.scaling);
+  for (uint32_t r = threadIdx.x; r < a.k; r += kBlock) { write_neighbor(a, q, r, out[r], chunk, probes); }
+}
+
+__global__ __launch_bounds__(kBlock) void merge_kernel(merge_args a, uint32_t out_cap) { merge_query(a, out_cap, blockIdx.x); }
+
+/** The queries merge_live_kernel left over (a.redo), normally none: a block looks at kBlock queries'
+ *  flags and merges the flagged ones one after the other. */
+__global__ __launch_bounds__(kBlock) void merge_redo_kernel(merge_args a, uint32_t out_cap)
+{
+  __shared__ uint32_t todo[kBlock];
+  __shared__ uint32_t n_todo;
+  if (threadIdx.x == 0) { n_todo = 0; }
+  __syncthreads();
+  const uint32_t q = blockIdx.x * kBlock + threadIdx.x;
+  if (q < a.n_queries && a.redo[q] != 0) { todo[atomicAdd(&n_todo, 1u)] = q; }
+  __syncthreads();
+  const uint32_t n = n_todo;
+  for (uint32_t i = 0; i < n; i++) {
+    merge_query(a, out_cap, todo[i]);
+    __syncthreads();
   }
 }
 
@@ -1695,6 +1802,19 @@ void launch_merge(const merge_args& a, hipStream_t stream)
   if (smem > 32 * 1024) {
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(merge_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(merge_redo_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+  }
+  if (a.fused && a.alive != nullptr && a.redo != nullptr) {
+    // one wave per query for the queries with few live keys; the block-wide merge for the others
+    const size_t live_smem = size_t(kLiveSmall) * 8 + size_t(a.k) * 8 + size_t(a.n_probes) * 10;
+    if (live_smem <= 64 * 1024) {
+      merge_live_kernel<<<a.n_queries, 64, live_smem, stream>>>(a);
+      CUVS_LAUNCH_CHECK();
+      merge_redo_kernel<<<blocks_for(a.n_queries, kBlock), kBlock, smem, stream>>>(a, out_cap);
+      CUVS_LAUNCH_CHECK();
+      return;
+    }
   }
   merge_kernel<<<a.n_queries, kBlock, smem, stream>>>(a, out_cap);
   CUVS_LAUNCH_CHECK();

@@ -94,9 +94,9 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
   const size_t P = p.n_probes;
   p.per_query_bytes = size_t(ix.dim) * 4 + size_t(ix.dim_ext) * 4 + size_t(ix.n_lists) * 4 +
                       size_t(ix.rot_dim) * 4 +
-                      P * 4 * 3 + P * (2 * sizeof(detail::pair_desc) + 1) + 16 + P * 17 +
+                      P * 4 * 3 + P * (2 * sizeof(detail::pair_desc) + 1) + 17 + P * 17 +
                       (p.fused ? P * k * 8 * 4 : size_t(p.max_samples) * 4);
-  p.fixed_bytes = a256(size_t(ix.n_lists) * 16 + 16) + 3 * 256 + size_t(512) * 8 + a256(size_t(ix.dim_ext) * 128 * 4) + a256(detail::kSelectSlackBytes) + 16 * 256;
+  p.fixed_bytes = a256(size_t(ix.n_lists) * 16 + 16) + 3 * 256 + size_t(512) * 8 + a256(size_t(ix.dim_ext) * 128 * 4) + a256(detail::kSelectSlackBytes) + 20 * 256;
   if (ix.coarse_fast_ok) {
     // buffers of the two-precision probe selection (the batch must fit with them)
     p.per_query_bytes += size_t(detail::coarse_fast_k_pad(ix.dim)) * 2 + size_t(detail::coarse_fast_groups(ix.n_lists)) * 4 +
@@ -448,10 +448,12 @@ void search(cuvs::resources const& res_c,
   detail::pair_desc* survivors = nullptr;
   uint8_t* alive               = nullptr;
   uint32_t* n_survivors        = nullptr;
+  uint8_t* merge_redo          = nullptr;
   if (early_stop) {
     survivors   = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));
     alive       = static_cast<uint8_t*>(res.workspace_alloc(size_t(Qb) * P));
     n_survivors = static_cast<uint32_t*>(res.workspace_alloc(256));
+    merge_redo  = static_cast<uint8_t*>(res.workspace_alloc(size_t(Qb)));
   }
   if (pl.fused) {
     keys = static_cast<unsigned long long*>(res.workspace_alloc(size_t(Qb) * P * kpp * 8));
@@ -571,6 +573,7 @@ void search(cuvs::resources const& res_c,
     ma.scaling       = scaling_factor(type);
     ma.in_keys       = keys;
     ma.alive         = alive;
+    ma.redo          = merge_redo;
     ma.in_scores     = all_scores;
     ma.n_samples     = n_samples;
     ma.probes        = probes;
