@@ -11,7 +11,7 @@
  * than n_probes - are then scored by the fp32 path's own arithmetic (one FMA chain over ascending
  * dimensions) and ordered by (score, list).  The probes are bit for bit those of the fp32 path.
  *
- *   pass 1  fp16 scores; per query the minimum of every group of 16 lists      (no score matrix)
+ *   pass 1  fp16 scores; per query the minimum of every group of 32 lists      (no score matrix)
  *   bound   T_q = n_probes-th smallest of those minima (at least n_probes scores are <= T_q),
  *           thr_q = T_q + 2 E_q
  *   pass 2  the same fp16 scores again; lists with score <= thr_q are appended to the query's
@@ -116,8 +116,10 @@ __global__ void pack_centers_kernel(const float* __restrict__ centers, uint32_t 
 
 constexpr uint32_t kGemmThreads = 256;
 constexpr uint32_t kLocalCap    = 32;  // PASS 2: candidates a query may collect between two flushes before its block gives up
-constexpr uint32_t kFlushTiles  = 8;   // list tiles between two flushes: 32 group minima, one 128-byte line of a query's row
-constexpr uint32_t kMinRow      = kFlushTiles * 4u + 4u;  // floats per query in the staged minima (rows 144 bytes apart)
+constexpr uint32_t kGroup       = 32;  // PASS 1: lists per group minimum (one MFMA tile's rows)
+constexpr uint32_t kMinFlushTiles  = 16;  // PASS 1: list tiles between two flushes: 32 group minima, one 128-byte line of a query's row
+constexpr uint32_t kCandFlushTiles = 8;   // PASS 2: list tiles (512 lists) between two flushes of the candidates
+constexpr uint32_t kMinRow      = kMinFlushTiles * 2u + 4u;  // floats per query in the staged minima (rows 144 bytes apart)
 
 /**
  * fp16 scores s' = alpha * (cn * qterm + dot16(c, q)) of a block's 256 queries against a run of
@@ -127,7 +129,7 @@ constexpr uint32_t kMinRow      = kFlushTiles * 4u + 4u;  // floats per query in
  * blocks fit a CU, so that one block's matrix products run under the other's epilogue, staging
  * and barrier.  List tiles stream through two LDS buffers, the next tile's global loads in flight
  * while the current one is multiplied (one barrier per tile).  The norm term is the accumulators'
- * starting value.  PASS 1 keeps, per query, the minimum of every group of 16 lists; PASS 2 collects
+ * starting value.  PASS 1 keeps, per query, the minimum of every group of 32 lists; PASS 2 collects
  * the lists whose score is at or below the query's threshold.  Both results are staged in LDS by
  * the wave that owns the query and written out by that wave every kFlushTiles tiles (the minima
  * as whole 128-byte lines; the candidates with one global atomic per query), without a barrier.
@@ -288,7 +290,9 @@ __global__ __launch_bounds__(kGemmThreads, 2) void coarse_f16_kernel(
           float best = neg_inf;
 #pragma unroll
           for (int r = 0; r < 16; r++) { best = fmaxf(best, acc[i][j][r]); }  // NaN scores are ignored here and never pass the threshold
-          lmin[qloc[j] * kMinRow + (tile % kFlushTiles) * 4u + uint32_t(i) * 2u + half] = alpha * best;
+          // the lane 32 further on holds the tile's other 16 rows of this query
+          best = fmaxf(best, __shfl_xor(best, 32, 64));
+          if (half == 0) { lmin[qloc[j] * kMinRow + (tile % kMinFlushTiles) * 2u + uint32_t(i)] = alpha * best; }
         }
       }
     } else {
@@ -325,20 +329,21 @@ __global__ __launch_bounds__(kGemmThreads, 2) void coarse_f16_kernel(
     }
   };
   // The wave writes out what it has staged for its 64 queries since the last flush (its own LDS
-  // writes, in order: no barrier).  PASS 1: the minima of tiles [first, tile], parts of one
-  // 128-byte line per query, 8 queries an instruction.  PASS 2: a lane per query.
+  // writes, in order: no barrier).  PASS 1: the minima of tiles [first, tile], 16-byte parts (two
+  // tiles each: a block starts at an even tile) of one 128-byte line per query, 8 queries an
+  // instruction.  PASS 2: a lane per query.
   auto flush = [&](uint32_t tile) __attribute__((always_inline)) {
     if (PASS == 1) {
-      const uint32_t slot  = tile % kFlushTiles;
-      const uint32_t line  = tile - slot;                        // first tile of the line
-      const uint32_t lo    = line < t0 ? t0 - line : 0u;         // the block's first part of it
+      const uint32_t slot  = (tile % kMinFlushTiles) >> 1;
+      const uint32_t line  = tile - tile % kMinFlushTiles;       // first tile of the line
+      const uint32_t lo    = line < t0 ? (t0 - line) >> 1 : 0u;  // the block's first part of it
       const uint32_t part  = lane & 7u;
       // (all eight reads first and the stores after them measured 20 % slower for the whole kernel)
 #pragma unroll
       for (uint32_t it = 0; it < 8; it++) {
         const uint32_t ql = wid * 64u + it * 8u + (lane >> 3);
         if (part >= lo && part <= slot && q0 + ql < n_queries) {
-          *reinterpret_cast<float4*>(minima + uint64_t(q0 + ql) * n_groups + (line + part) * 4u) =
+          *reinterpret_cast<float4*>(minima + uint64_t(q0 + ql) * n_groups + line * 2u + part * 4u) =
             *reinterpret_cast<const float4*>(lmin + ql * kMinRow + part * 4u);
         }
       }
@@ -367,7 +372,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void coarse_f16_kernel(
     const uint32_t buf = (tile - t0) & 1u;
     issue(tile + 1u, sx, cx);
     multiply(tile, buf);
-    if ((tile + 1u) % kFlushTiles == 0 || tile + 1u == t1) { flush(tile); }
+    if ((tile + 1u) % (PASS == 1 ? kMinFlushTiles : kCandFlushTiles) == 0 || tile + 1u == t1) { flush(tile); }
     arrived(sx, cx);
     commit(tile + 1u, buf ^ 1u, sx, cx);
     // the barrier orders LDS traffic only (the staged tile); the flushes' global stores stay in
@@ -377,8 +382,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void coarse_f16_kernel(
 }
 
 /** thr[q] = (n_probes-th smallest of the query's group minima) + 2 E_q, rounded up.  One wave per
- *  query: the minima sit in registers as ordered keys (HELD per lane: 16 cover 16,384 lists, 64
- *  cover 65,536; more are re-read every round) and a round of the bitwise search counts with
+ *  query: the minima sit in registers as ordered keys (HELD per lane: 8 cover 16,384 lists, 64
+ *  cover 131,072; more are re-read every round) and a round of the bitwise search counts with
  *  ballots, without LDS or barriers.  One probe (labelling rows during extend) needs no search:
  *  the threshold is the smallest minimum. */
 template <uint32_t HELD>
@@ -456,7 +461,10 @@ __global__ __launch_bounds__(512) void coarse_rescore_kernel(
   unsigned long long* keys  = reinterpret_cast<unsigned long long*>(smem + ((dim * 4u + 15u) & ~15u));
   const uint32_t q   = blockIdx.x;
   const uint32_t tid = threadIdx.x;
-  const uint32_t n   = cand_count[q];
+  // this thread's candidate is requested together with the count that says whether it has one
+  // (tid < the candidate slots of a query: the address is always the query's own row)
+  const uint32_t my_cand = cand[uint64_t(q) * kCandCapF + tid];
+  const uint32_t n       = cand_count[q];
   // one candidate per thread: the block is as wide as the longest candidate list it accepts
   if (n > blockDim.x || n < n_probes) {
     if (tid == 0) { fallback[q] = 1; }
@@ -471,19 +479,21 @@ __global__ __launch_bounds__(512) void coarse_rescore_kernel(
   __syncthreads();
   unsigned long long key = kInvalidKey;
   if (tid < n) {
-    const uint32_t l = cand[uint64_t(q) * kCandCapF + tid];
+    const uint32_t l = my_cand;
     const float* c   = centers + uint64_t(l) * dim_ext;  // rows are 32-byte aligned (dim_ext % 8 == 0)
     float acc        = 0.0f;
-    // The FMA chain is sequential; the loads are not: 32 dimensions of the centre row are requested
-    // together (one latency for eight 16-byte loads), then multiplied in.
-    const uint32_t dim32 = dim & ~31u;
+    // The FMA chain is sequential; the loads are not: 32 dimensions of the centre row (one 128-byte
+    // line) are requested together, then multiplied in.  (64 dimensions at a time measured 30 %
+    // slower: two lines per lane in flight no longer fit the vector cache.)
+    constexpr uint32_t kAhead = 8;
+    const uint32_t dim32 = dim - dim % (4 * kAhead);
     const uint32_t dim4  = dim & ~3u;
-    for (uint32_t d0 = 0; d0 < dim32; d0 += 32) {
-      float4 v[8];
+    for (uint32_t d0 = 0; d0 < dim32; d0 += 4 * kAhead) {
+      float4 v[kAhead];
 #pragma unroll
-      for (uint32_t x = 0; x < 8; x++) { v[x] = *reinterpret_cast<const float4*>(c + d0 + 4 * x); }
+      for (uint32_t x = 0; x < kAhead; x++) { v[x] = *reinterpret_cast<const float4*>(c + d0 + 4 * x); }
 #pragma unroll
-      for (uint32_t x = 0; x < 8; x++) {
+      for (uint32_t x = 0; x < kAhead; x++) {
         const uint32_t d = d0 + 4 * x;
         acc              = fmaf(v[x].x, qf[d], acc);
         acc              = fmaf(v[x].y, qf[d + 1], acc);
@@ -541,7 +551,7 @@ __global__ __launch_bounds__(256) void coarse_exact_rows_kernel(
 }  // namespace
 
 uint32_t coarse_fast_k_pad(uint32_t dim) { return (dim + kSlab - 1) / kSlab * kSlab; }
-uint32_t coarse_fast_groups(uint32_t n_lists) { return coarse_pad(n_lists) / 16u; }
+uint32_t coarse_fast_groups(uint32_t n_lists) { return coarse_pad(n_lists) / kGroup; }
 uint32_t coarse_fast_cand_cap() { return kCandCapF; }
 
 void launch_pack_centers_f16(const float* centers, uint32_t n_lists, uint32_t dim, uint32_t dim_ext,
@@ -570,7 +580,7 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
   const uint32_t q_pad = coarse_pad(a.n_queries);
   const uint32_t l_pad = coarse_pad(a.n_lists);
   const uint32_t k_pad = coarse_fast_k_pad(a.dim);
-  const uint32_t n_groups = l_pad / 16u;
+  const uint32_t n_groups = l_pad / kGroup;
   const float qterm    = a.ip_like ? 0.0f : -0.5f;
   const float alpha    = a.ip_like ? -1.0f : -2.0f;
   // |s - s'| <= |alpha| * [ (2^-11 + 9 (dim + 4) 2^-24) |q| Cmax + sqrt(dim) 2^-25 |q| + (dim + 4) 2^-24 * Nmax / 2 ],
@@ -609,9 +619,10 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
   // those: fewer blocks load the queries).
   const uint64_t n_slots   = uint64_t(device_cu_count()) * 2u;
   const uint32_t n_qblocks = (q_pad + kQTile - 1) / kQTile;
-  uint32_t tiles_per_block = 1;
+  uint32_t tiles_per_block = 2;
   uint64_t best_cost       = ~uint64_t(0);
-  for (uint32_t t = 1; t <= n_list_tiles; t++) {
+  // (even run lengths: the group minima of two tiles share a 16-byte store)
+  for (uint32_t t = 2; t <= n_list_tiles; t += 2) {
     const uint64_t blocks = uint64_t((n_list_tiles + t - 1) / t) * n_qblocks;
     const uint64_t rounds = (blocks + n_slots - 1) / n_slots;
     const uint64_t cost   = rounds * (t + 2);
@@ -631,7 +642,9 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
     k1<<<grid, kGemmThreads, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, q_pad, n_list_tiles, tiles_per_block, alpha,
                                     qterm, a.minima, n_groups, nullptr, nullptr, nullptr);
     CUVS_HIP_TRY(hipGetLastError());
-    if (n_groups <= 16u * 64u) {
+    if (n_groups <= 8u * 64u) {
+      coarse_threshold_kernel<8><<<(a.n_queries + 3) / 4, 256, 0, stream>>>(a.minima, a.n_queries, n_groups, a.n_probes, a.qnorm, e_rel, e_abs, a.thr);
+    } else if (n_groups <= 16u * 64u) {
       coarse_threshold_kernel<16><<<(a.n_queries + 3) / 4, 256, 0, stream>>>(a.minima, a.n_queries, n_groups, a.n_probes, a.qnorm, e_rel, e_abs, a.thr);
     } else {
       coarse_threshold_kernel<64><<<(a.n_queries + 3) / 4, 256, 0, stream>>>(a.minima, a.n_queries, n_groups, a.n_probes, a.qnorm, e_rel, e_abs, a.thr);
