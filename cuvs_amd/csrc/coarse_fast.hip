@@ -57,11 +57,13 @@ __device__ __forceinline__ float map_elem<uint8_t>(uint8_t v) { return float(v) 
 
 /** qh[q][d] = mapped query as binary16 (exact for these element types), zero padded to k_pad
  *  columns and q_pad rows; qnorm[q] = an upper bound of the query's Euclidean norm (of the
- *  unrounded values: float32 queries are the one type that binary16 does not hold exactly). */
+ *  unrounded values: float32 queries are the one type that binary16 does not hold exactly);
+ *  qf[q][d] = the mapped query in fp32 (what the stages after the probe selection read). */
 template <typename T>
 __global__ void pack_queries_kernel(const T* __restrict__ in, uint32_t n_queries, uint32_t dim,
                                     uint32_t k_pad, _Float16* __restrict__ qh, float* __restrict__ qnorm,
-                                    uint32_t* __restrict__ cand_count, uint8_t* __restrict__ fallback)
+                                    uint32_t* __restrict__ cand_count, uint8_t* __restrict__ fallback,
+                                    float* __restrict__ qf)
 {
   const uint32_t q    = blockIdx.x;
   const uint32_t lane = threadIdx.x;
@@ -73,7 +75,10 @@ __global__ void pack_queries_kernel(const T* __restrict__ in, uint32_t n_queries
   float ss            = 0.0f;
   for (uint32_t d = lane; d < k_pad; d += 64) {
     float v = 0.0f;
-    if (q < n_queries && d < dim) { v = map_elem<T>(in[uint64_t(q) * dim + d]); }
+    if (q < n_queries && d < dim) {
+      v = map_elem<T>(in[uint64_t(q) * dim + d]);
+      if (qf != nullptr) { qf[uint64_t(q) * dim + d] = v; }
+    }
     qh[uint64_t(q) * k_pad + d] = _Float16(v);
     ss                          = fmaf(v, v, ss);
   }
@@ -598,16 +603,16 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
 
   switch (a.type) {
     case elem_type::f32:
-      pack_queries_kernel<float><<<q_pad, 64, 0, stream>>>(static_cast<const float*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm, a.cand_count, a.fallback);
+      pack_queries_kernel<float><<<q_pad, 64, 0, stream>>>(static_cast<const float*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm, a.cand_count, a.fallback, a.qf);
       break;
     case elem_type::f16:
-      pack_queries_kernel<_Float16><<<q_pad, 64, 0, stream>>>(static_cast<const _Float16*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm, a.cand_count, a.fallback);
+      pack_queries_kernel<_Float16><<<q_pad, 64, 0, stream>>>(static_cast<const _Float16*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm, a.cand_count, a.fallback, a.qf);
       break;
     case elem_type::i8:
-      pack_queries_kernel<int8_t><<<q_pad, 64, 0, stream>>>(static_cast<const int8_t*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm, a.cand_count, a.fallback);
+      pack_queries_kernel<int8_t><<<q_pad, 64, 0, stream>>>(static_cast<const int8_t*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm, a.cand_count, a.fallback, a.qf);
       break;
     case elem_type::u8:
-      pack_queries_kernel<uint8_t><<<q_pad, 64, 0, stream>>>(static_cast<const uint8_t*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm, a.cand_count, a.fallback);
+      pack_queries_kernel<uint8_t><<<q_pad, 64, 0, stream>>>(static_cast<const uint8_t*>(a.queries), a.n_queries, a.dim, k_pad, a.qh, a.qnorm, a.cand_count, a.fallback, a.qf);
       break;
   }
   CUVS_HIP_TRY(hipGetLastError());

@@ -236,6 +236,7 @@ struct coarse_fast_args {
   const _Float16* ch;      // [coarse_pad(n_lists), k_pad] centres as binary16
   const float* cn;         // [coarse_pad(n_lists)] stored squared norms
   float c_max, n_max;      // largest centre length, largest |stored norm|
+  float* qf;               // [n_queries, dim] out: the mapped queries in fp32 (null: not wanted)
   _Float16* qh;            // [coarse_pad(n_queries), k_pad]
   float* qnorm;            // [coarse_pad(n_queries)]
   float* minima;           // [n_queries, coarse_fast_groups(n_lists)]
@@ -265,12 +266,13 @@ void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries,
 
 /** chunk_indices[q, p] = inclusive prefix sum of list_sizes[probes[q, p]]; n_samples[q] = total.
  *  When `stats` is non-null (kStatSlots x 4 words), query q adds the scanned bytes, the rows and
- *  the bytes of its leading probes to words 0, 1, 2 of slot q % kStatSlots. */
+ *  the bytes of its leading probes to words 0, 1, 2 of slot q % kStatSlots.  `query_max`
+ *  (n_queries words) is filled with 0xFFFFFFFF and `zero_word` (one word) with 0 when given. */
 constexpr uint32_t kStatSlots = 256;
 void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
                           uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
                           uint32_t* n_samples, unsigned long long* stats, uint32_t lead_probes,
-                          hipStream_t stream);
+                          uint32_t* query_max, uint32_t* zero_word, hipStream_t stream);
 
 /** Everything the scan needs to know about one (query, probe) pair, gathered once so that the
  *  scan kernel reads one 32-byte record instead of chasing four dependent pointers. */

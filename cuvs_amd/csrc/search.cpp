@@ -218,9 +218,9 @@ void run_coarse(const cuvs::resources& res, const search_params& params, const i
   hipStream_t s     = res.stream();
   const bool ip     = ix.metric == detail::DistanceType::InnerProduct ||
                   ix.metric == detail::DistanceType::CosineExpanded;
-  detail::launch_map_queries(queries, type, uint64_t(nq) * ix.dim, b.qf, s);
   if (b.qh != nullptr) {
     detail::coarse_fast_args a{};
+    a.qf         = b.qf;  // the packing kernel maps the queries on its way
     a.queries    = queries;
     a.type       = type;
     a.n_queries  = nq;
@@ -246,6 +246,7 @@ void run_coarse(const cuvs::resources& res, const search_params& params, const i
     detail::launch_coarse_fast(a, s);
     return;
   }
+  detail::launch_map_queries(queries, type, uint64_t(nq) * ix.dim, b.qf, s);
   if (params.coarse_search_dtype == CUDA_R_8I) {
     // ivf_pq_search.cuh:170-256
     detail::launch_coarse_scores_i8(b.qf, ix.centers_i8.as<uint32_t>(), nq, ix.n_lists, ix.dim, ip,
@@ -494,20 +495,25 @@ void search(cuvs::resources const& res_c,
     mark(1);
     cuvs::tracing::range worker_scope("ivf_pq::search-worker(n_queries = %u, n_probes = %u, k = %u, dim = %u)", nq, P,
                                       k, ix.dim);
-    detail::launch_rotate(qf, ix.rotation_t.as<float>(), nq, ix.dim, ix.rot_dim,
-                          ix.rotation_is_identity, cosine, params.coarse_search_dtype, rot_q, s);
+    // an identity rotation of fp32 operands leaves the mapped queries as they are
+    const bool rotate = !(ix.rotation_is_identity && ix.rot_dim == ix.dim && !cosine &&
+                          params.coarse_search_dtype == CUDA_R_32F);
+    if (rotate) {
+      detail::launch_rotate(qf, ix.rotation_t.as<float>(), nq, ix.dim, ix.rot_dim,
+                            ix.rotation_is_identity, cosine, params.coarse_search_dtype, rot_q, s);
+    }
     detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
-                                 ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead, s);
+                                 ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead,
+                                 pl.fused ? kth : nullptr, n_survivors, s);
     detail::launch_order_pairs(probes, chunk, ix.data_ptrs.as<const uint8_t*>(),
                                ix.inds_ptrs.as<const int64_t*>(), ix.ids_arena.as<int64_t>(), nq * P, P,
                                ix.n_lists, counters, sort_scratch, order, desc, lead, alive, few_pairs, list_rank, s);
-    if (pl.fused) { detail::launch_fill_u32(kth, 0xFFFFFFFFu, nq, s); }
     mark(2);
 
     {
     cuvs::tracing::range scan_scope("ivf_pq::search-worker::scan");
     sa.n_queries     = nq;
-    sa.rot_q         = rot_q;
+    sa.rot_q         = rotate ? rot_q : qf;
     sa.probes        = probes;
     sa.chunk_indices = chunk;
     sa.pair_order    = order;
@@ -527,7 +533,6 @@ void search(cuvs::resources const& res_c,
       detail::launch_kth_bound(keys, nq, uint64_t(P) * kpp, lead * kpp, k, kth, s);
       mark(5);
       // 2. every other pair on its first chunk only
-      detail::launch_fill_u32(n_survivors, 0, 1, s);
       detail::launch_scan_screen(sa, desc + size_t(nq) * lead, nq * (P - lead), survivors, n_survivors,
                                  alive, s);
       if (observe_screen) {
