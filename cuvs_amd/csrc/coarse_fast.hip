@@ -453,8 +453,14 @@ __global__ __launch_bounds__(256) void coarse_threshold_kernel(
   }
 }
 
-/** Exact fp32 score of every candidate by the fp32 path's arithmetic, then the n_probes best in
- *  ascending (score, list) order.  One block of 256 threads per query. */
+/** Exact fp32 score of every candidate by the fp32 path's arithmetic (one FMA chain over ascending
+ *  dimensions, then the norm term), then the n_probes best in ascending (score, list) order.  One
+ *  block per query, a lane per candidate.  A lane reading its own centre row costs a vector-cache
+ *  lookup per lane and 16 bytes; here the 64 rows of a wave come in 32 dimensions at a time with
+ *  whole 128-byte lines per 8 lanes, pass through the wave's own LDS area (rows 144 bytes apart),
+ *  and every lane reads its row back; the next 32 dimensions are on their way meanwhile.  Nothing
+ *  but the final ranking crosses waves. */
+constexpr uint32_t kRescoreRow = 36;  // floats between the staged rows of a wave
 template <typename T>
 __global__ __launch_bounds__(512) void coarse_rescore_kernel(
   const T* __restrict__ queries, const float* __restrict__ centers, uint32_t dim, uint32_t dim_ext,
@@ -463,9 +469,12 @@ __global__ __launch_bounds__(512) void coarse_rescore_kernel(
 {
   extern __shared__ __align__(16) unsigned char smem[];
   float* qf                 = reinterpret_cast<float*>(smem);  // [dim]
-  unsigned long long* keys  = reinterpret_cast<unsigned long long*>(smem + ((dim * 4u + 15u) & ~15u));
-  const uint32_t q   = blockIdx.x;
-  const uint32_t tid = threadIdx.x;
+  unsigned long long* keys  = reinterpret_cast<unsigned long long*>(smem + ((dim * 4u + 15u) & ~15u));  // [threads]
+  uint32_t* lcand           = reinterpret_cast<uint32_t*>(keys + blockDim.x);                           // [threads]
+  float* stage_all          = reinterpret_cast<float*>(lcand + blockDim.x);  // [waves][64][kRescoreRow]
+  const uint32_t q    = blockIdx.x;
+  const uint32_t tid  = threadIdx.x;
+  const uint32_t lane = tid & 63u;
   // this thread's candidate is requested together with the count that says whether it has one
   // (tid < the candidate slots of a query: the address is always the query's own row)
   const uint32_t my_cand = cand[uint64_t(q) * kCandCapF + tid];
@@ -481,42 +490,64 @@ __global__ __launch_bounds__(512) void coarse_rescore_kernel(
   const uint32_t n_active = (n + 63u) & ~63u;
   if (tid >= n_active) { return; }
   for (uint32_t d = tid; d < dim; d += n_active) { qf[d] = map_elem<T>(queries[uint64_t(q) * dim + d]); }
+  lcand[tid] = tid < n ? my_cand : 0u;  // idle lanes of the last wave shadow list 0
   __syncthreads();
+  float* stage = stage_all + (tid >> 6) * (64u * kRescoreRow);
+  // lane -> (row, 16-byte piece) of the wave's k-th staging instruction: rows 8k .. 8k + 7
+  const uint32_t piece = lane & 7u;
+  const float* src[8];
+#pragma unroll
+  for (uint32_t k = 0; k < 8; k++) {
+    src[k] = centers + uint64_t(lcand[(tid & ~63u) + k * 8u + (lane >> 3)]) * dim_ext + piece * 4u;
+  }
+  const float norm_term = centers[uint64_t(lcand[tid]) * dim_ext + dim];
+  // two rounds of 32 dimensions are in flight while a third is multiplied
+  float4 in[2][8];
+  auto request = [&](uint32_t d0, float4(&dst)[8]) __attribute__((always_inline)) {
+#pragma unroll
+    for (uint32_t k = 0; k < 8; k++) {
+      // a piece past the padded row is not read (rows are dim_ext floats, a multiple of 8)
+      dst[k] = d0 + piece * 4u < dim_ext ? *reinterpret_cast<const float4*>(src[k] + d0) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+  };
+  float acc = 0.0f;
+  auto round = [&](uint32_t d0, float4(&cur)[8]) __attribute__((always_inline)) {
+#pragma unroll
+    for (uint32_t k = 0; k < 8; k++) {
+      *reinterpret_cast<float4*>(stage + (k * 8u + (lane >> 3)) * kRescoreRow + piece * 4u) = cur[k];
+    }
+    if (d0 + 64 < dim) { request(d0 + 64, cur); }
+    // the wave's own LDS writes, in order, before its reads of other lanes' words
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const float* row  = stage + lane * kRescoreRow;
+    const uint32_t nd = dim - d0 < 32u ? dim - d0 : 32u;
+    if (nd == 32u) {
+#pragma unroll
+      for (uint32_t x = 0; x < 8; x++) {
+        const float4 v   = *reinterpret_cast<const float4*>(row + 4 * x);
+        const uint32_t d = d0 + 4 * x;
+        acc              = fmaf(v.x, qf[d], acc);
+        acc              = fmaf(v.y, qf[d + 1], acc);
+        acc              = fmaf(v.z, qf[d + 2], acc);
+        acc              = fmaf(v.w, qf[d + 3], acc);
+      }
+    } else {
+      for (uint32_t x = 0; x < nd; x++) { acc = fmaf(row[x], qf[d0 + x], acc); }
+    }
+    // ... and the reads before the next round's writes
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  };
+  request(0, in[0]);
+  if (32 < dim) { request(32, in[1]); }
+  for (uint32_t d0 = 0; d0 < dim; d0 += 64) {
+    round(d0, in[0]);
+    if (d0 + 32 < dim) { round(d0 + 32, in[1]); }
+  }
   unsigned long long key = kInvalidKey;
   if (tid < n) {
-    const uint32_t l = my_cand;
-    const float* c   = centers + uint64_t(l) * dim_ext;  // rows are 32-byte aligned (dim_ext % 8 == 0)
-    float acc        = 0.0f;
-    // The FMA chain is sequential; the loads are not: 32 dimensions of the centre row (one 128-byte
-    // line) are requested together, then multiplied in.  (64 dimensions at a time measured 30 %
-    // slower: two lines per lane in flight no longer fit the vector cache.)
-    constexpr uint32_t kAhead = 8;
-    const uint32_t dim32 = dim - dim % (4 * kAhead);
-    const uint32_t dim4  = dim & ~3u;
-    for (uint32_t d0 = 0; d0 < dim32; d0 += 4 * kAhead) {
-      float4 v[kAhead];
-#pragma unroll
-      for (uint32_t x = 0; x < kAhead; x++) { v[x] = *reinterpret_cast<const float4*>(c + d0 + 4 * x); }
-#pragma unroll
-      for (uint32_t x = 0; x < kAhead; x++) {
-        const uint32_t d = d0 + 4 * x;
-        acc              = fmaf(v[x].x, qf[d], acc);
-        acc              = fmaf(v[x].y, qf[d + 1], acc);
-        acc              = fmaf(v[x].z, qf[d + 2], acc);
-        acc              = fmaf(v[x].w, qf[d + 3], acc);
-      }
-    }
-    for (uint32_t d = dim32; d < dim4; d += 4) {
-      const float4 v = *reinterpret_cast<const float4*>(c + d);
-      acc            = fmaf(v.x, qf[d], acc);
-      acc            = fmaf(v.y, qf[d + 1], acc);
-      acc            = fmaf(v.z, qf[d + 2], acc);
-      acc            = fmaf(v.w, qf[d + 3], acc);
-    }
-    for (uint32_t d = dim4; d < dim; d++) { acc = fmaf(c[d], qf[d], acc); }
-    acc           = fmaf(c[dim], qterm, acc);
+    acc           = fmaf(norm_term, qterm, acc);
     const float s = alpha * acc;
-    key = (s != s) ? kInvalidKey : ((static_cast<unsigned long long>(order_f32(s)) << 32) | l);
+    key = (s != s) ? kInvalidKey : ((static_cast<unsigned long long>(order_f32(s)) << 32) | my_cand);
   }
   keys[tid] = key;
   __syncthreads();
@@ -666,10 +697,22 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
     run_pass(coarse_f16_kernel<1, 128>, coarse_f16_kernel<2, 128>);
   }
   // up to 128 probes about 1.4 x 128 candidates pass the threshold: 256 threads; 512 beyond
-  const uint32_t rthreads = a.n_probes <= 128 ? 256u : 512u;
-  const size_t rsmem      = ((size_t(a.dim) * 4 + 15) & ~size_t(15)) + size_t(rthreads) * 8;
+  // about 1.15 x n_probes candidates pass the threshold: 128 threads up to 64 probes, 256 up to
+  // 128, 512 beyond (a query with more candidates than threads takes the plain path)
+  const uint32_t rthreads = a.n_probes <= 64 ? 128u : (a.n_probes <= 128 ? 256u : 512u);
+  const size_t rsmem      = ((size_t(a.dim) * 4 + 15) & ~size_t(15)) + size_t(rthreads) * 12 +
+                       size_t(rthreads) * kRescoreRow * 4;
   const size_t xsmem = size_t(a.dim) * 4;
-  CUVS_EXPECTS(rsmem <= 48 * 1024, "dim (%u) is too large for the two-precision probe selection", a.dim);
+  CUVS_EXPECTS(rsmem <= 96 * 1024, "dim (%u) is too large for the two-precision probe selection", a.dim);
+  if (rsmem > 48 * 1024) {
+    static std::once_flag big_lds;
+    std::call_once(big_lds, [&] {
+      CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(coarse_rescore_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+      CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(coarse_rescore_kernel<_Float16>), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+      CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(coarse_rescore_kernel<int8_t>), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+      CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(coarse_rescore_kernel<uint8_t>), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+    });
+  }
   switch (a.type) {
     case elem_type::f32:
       coarse_rescore_kernel<float><<<a.n_queries, rthreads, rsmem, stream>>>(static_cast<const float*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);

@@ -449,6 +449,47 @@ def test_screen_turns_itself_off_where_it_does_not_pay(orc):
     H.compare_results(nb2.cpu().numpy(), d2.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
 
 
+def test_merge_after_early_stop_with_many_live_keys(orc):
+    """Unclustered rows and k = 64 with the screen forced on: nearly every pair survives and brings
+    dozens of valid keys, far more than the one-wave merge takes (512 per query), so the queries go
+    through its leftover launch; clustered queries of the same batch size stay in the wave merge.
+    Both return the oracle's results."""
+    from cuvs_amd.resources import Resources
+    rng = np.random.default_rng(23)
+    allrows = rng.standard_normal((30200, 128)).astype(np.float32)
+    x, q = allrows[:30000], allrows[30000:]
+    model = H.train(x, 100, 64, 8, iters=4)
+    index = G.build_gpu_index(model, x, 64, 8, "sqeuclidean", "subspace")
+    ix, _ = G.read_back(orc, index, model, 128, 64, 8, "sqeuclidean", "subspace")
+    res = Resources()
+    res.enable_profiling(True)
+    res.set_search_tuning(early_stop="on")
+    for k in (64, 10):
+        sp = ivf_pq.SearchParams(n_probes=32, lut_dtype=R_16F)
+        want_nb, want_d = orc.search(ix, q, k, 32, lut_dtype=ORC_DT[R_16F])
+        d, nb = ivf_pq.search(sp, index, G.to_dev(q), k, resources=res)
+        res.sync()
+        prof = ivf_pq.get_search_profile(res)
+        assert prof["n_screened_pairs"] == q.shape[0] * 31
+        assert prof["n_surviving_pairs"] > 0.7 * prof["n_screened_pairs"]
+        H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
+
+
+def test_pair_order_beyond_the_sorted_range():
+    """More than 4 M (query, probe) pairs in one internal batch: the pair order falls back from the
+    two-level counting sort to global atomics.  Same neighbours as the same queries in batches that
+    the sort takes."""
+    import datasets as testing
+    allrows = testing.gaussian_mixture(40000 + 70000, 32, 64, 0.2, seed=91, device="cuda")
+    data, queries = allrows[:40000], allrows[40000:]
+    index = ivf_pq.build(ivf_pq.IndexParams(n_lists=256, pq_dim=16, kmeans_trainset_fraction=0.5), data)
+    big = ivf_pq.SearchParams(n_probes=64, lut_dtype=R_16F, max_internal_batch_size=70000)
+    small = ivf_pq.SearchParams(n_probes=64, lut_dtype=R_16F, max_internal_batch_size=8192)
+    d1, nb1 = ivf_pq.search(big, index, queries, 5)
+    d2, nb2 = ivf_pq.search(small, index, queries, 5)
+    assert torch.equal(nb1, nb2) and torch.equal(d1, d2)
+
+
 @pytest.mark.parametrize("kind", ["subspace", "cluster"])
 def test_early_stop_pq_len_4(orc, kind):
     """Four dimensions per subspace: 16-byte codebook entries in the table-free screen (shared by
