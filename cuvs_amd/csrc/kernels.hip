@@ -1106,7 +1106,8 @@ __device__ __forceinline__ void write_neighbor(const merge_args& a, uint32_t q, 
  * from sample number to list.  A query with more than kLiveSmall valid keys is left to
  * merge_redo_kernel (a.redo[q] = 1).
  */
-constexpr uint32_t kLiveSmall = 512;
+constexpr uint32_t kLiveSmall = 1024;
+constexpr uint32_t kRedoQueries = 16;  // queries whose flags a block of merge_redo_kernel looks at
 __global__ __launch_bounds__(64) void merge_live_kernel(merge_args a)
 {
   extern __shared__ __align__(16) unsigned char dyn_smem[];
@@ -1164,7 +1165,11 @@ __global__ __launch_bounds__(64) void merge_live_kernel(merge_args a)
   __syncthreads();
   uint32_t m = n_valid;
   if (n_valid > a.k) {
-    wave_select_keys<int(kLiveSmall / 64)>((LDS_AS unsigned long long*)small_keys, lane, n_valid, a.k);
+    if (n_valid <= kLiveSmall / 2) {
+      wave_select_keys<int(kLiveSmall / 128)>((LDS_AS unsigned long long*)small_keys, lane, n_valid, a.k);
+    } else {
+      wave_select_keys<int(kLiveSmall / 64)>((LDS_AS unsigned long long*)small_keys, lane, n_valid, a.k);
+    }
     m = a.k;
   }
   __syncthreads();
@@ -1246,16 +1251,16 @@ __device__ void merge_query(const merge_args& a, uint32_t out_cap, uint32_t q)
 
 __global__ __launch_bounds__(kBlock) void merge_kernel(merge_args a, uint32_t out_cap) { merge_query(a, out_cap, blockIdx.x); }
 
-/** The queries merge_live_kernel left over (a.redo), normally none: a block looks at kBlock queries'
- *  flags and merges the flagged ones one after the other. */
+/** The queries merge_live_kernel left over (a.redo), normally none: a block looks at the flags of
+ *  kRedoQueries queries and merges the flagged ones one after the other. */
 __global__ __launch_bounds__(kBlock) void merge_redo_kernel(merge_args a, uint32_t out_cap)
 {
-  __shared__ uint32_t todo[kBlock];
+  __shared__ uint32_t todo[kRedoQueries];
   __shared__ uint32_t n_todo;
   if (threadIdx.x == 0) { n_todo = 0; }
   __syncthreads();
-  const uint32_t q = blockIdx.x * kBlock + threadIdx.x;
-  if (q < a.n_queries && a.redo[q] != 0) { todo[atomicAdd(&n_todo, 1u)] = q; }
+  const uint32_t q = blockIdx.x * kRedoQueries + threadIdx.x;
+  if (threadIdx.x < kRedoQueries && q < a.n_queries && a.redo[q] != 0) { todo[atomicAdd(&n_todo, 1u)] = q; }
   __syncthreads();
   const uint32_t n = n_todo;
   for (uint32_t i = 0; i < n; i++) {
@@ -1812,13 +1817,15 @@ void launch_merge(const merge_args& a, hipStream_t stream)
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(merge_redo_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
   }
-  if (a.fused && a.alive != nullptr && a.redo != nullptr) {
+  // a pair hands over up to four times k keys: beyond k = 64 a handful of live pairs is already
+  // more than the one-wave merge takes
+  if (a.fused && a.alive != nullptr && a.redo != nullptr && a.k <= 64) {
     // one wave per query for the queries with few live keys; the block-wide merge for the others
     const size_t live_smem = size_t(kLiveSmall) * 8 + size_t(a.k) * 8 + size_t(a.n_probes) * 10;
     if (live_smem <= 64 * 1024) {
       merge_live_kernel<<<a.n_queries, 64, live_smem, stream>>>(a);
       CUVS_LAUNCH_CHECK();
-      merge_redo_kernel<<<blocks_for(a.n_queries, kBlock), kBlock, smem, stream>>>(a, out_cap);
+      merge_redo_kernel<<<blocks_for(a.n_queries, kRedoQueries), kBlock, smem, stream>>>(a, out_cap);
       CUVS_LAUNCH_CHECK();
       return;
     }

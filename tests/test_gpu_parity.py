@@ -451,7 +451,7 @@ def test_screen_turns_itself_off_where_it_does_not_pay(orc):
 
 def test_merge_after_early_stop_with_many_live_keys(orc):
     """Unclustered rows and k = 64 with the screen forced on: nearly every pair survives and brings
-    dozens of valid keys, far more than the one-wave merge takes (512 per query), so the queries go
+    dozens of valid keys, far more than the one-wave merge takes (1024 per query), so the queries go
     through its leftover launch; clustered queries of the same batch size stay in the wave merge.
     Both return the oracle's results."""
     from cuvs_amd.resources import Resources
