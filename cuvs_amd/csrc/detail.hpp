@@ -162,6 +162,16 @@ struct index_impl {
    *  touches half the cache lines the interleaved arena would, in whole lines.  Rebuilt whenever
    *  the arena changes; empty for other code widths or 2^32 and more row slots. */
   device_buffer lead_plane;
+  /** 5 - 7 bit codes: the lists once more with a byte per code, in the layout of an 8-bit index
+   *  (n_chunks8 = ceil(pq_dim / 16) chunks a row), their pointer table, and the codebooks padded to
+   *  256 entries.  A search whose 256-entry table fits the byte-wide kernels then runs on these as
+   *  if the index had 8-bit codes (same table entries for the codes that occur, same order of
+   *  summation: same results), early stop included; the packed lists stay what every other
+   *  function reads and writes.  Costs 8 / pq_bits times the packed lists' memory; not kept with
+   *  conservative_memory_allocation.  Rebuilt with the lead plane. */
+  device_buffer codes8_arena, data_ptrs8, pq_centers8;
+  uint32_t n_chunks8 = 0;
+  bool wide() const { return codes8_arena.bytes != 0; }
   std::vector<uint32_t> h_list_sizes;
   std::vector<uint64_t> h_row_offsets;  // [n_lists + 1], in rows, multiples of 32
   device_buffer list_sizes, data_ptrs, inds_ptrs;
@@ -176,7 +186,8 @@ struct index_impl {
   /** Recompute pointer tables, device sizes and the sorted prefix sums from the host vectors
    *  (role of ivf::detail::recompute_internal_state, cpp/src/neighbors/ivf_common.cuh:255-290). */
   void recompute_internal_state(hipStream_t stream);
-  /** Refill `lead_plane` from the codes arena (after the arena's contents changed). */
+  /** Refill `lead_plane` and the byte-wide copy of narrower codes from the codes arena (after the
+   *  arena's contents changed). */
   void rebuild_lead_plane(hipStream_t stream);
 };
 
@@ -364,6 +375,10 @@ void launch_train_codebooks(const float* res, uint32_t rot_dim, uint32_t pq_dim,
                             uint32_t n_iters, uint32_t seed, float* pq_centers, hipStream_t stream);
 
 /** plane[slot] = first eight bytes of row slot `slot` of an arena of 8-bit codes. */
+/** The packed codes of `n_slots` row slots as bytes in the 8-bit layout; codebook rows padded to 256 entries. */
+void launch_widen_codes(const uint8_t* packed, uint8_t* wide, uint64_t n_slots, uint32_t pq_dim,
+                        uint32_t pq_bits, uint32_t n_chunks, uint32_t n_chunks8, hipStream_t stream);
+void launch_pad_codebooks(const float* src, float* dst, uint64_t n_rows, uint32_t book_size, hipStream_t stream);
 void launch_build_lead_plane(const uint8_t* arena, uint64_t* plane, uint64_t n_slots,
                              uint32_t n_chunks, hipStream_t stream);
 constexpr uint64_t kLeadPlaneSlack = 512;  // slots past the last list that look-ahead loads of whole tiles may read

@@ -151,13 +151,44 @@ void index_impl::refresh_coarse(hipStream_t stream)
 void index_impl::rebuild_lead_plane(hipStream_t stream)
 {
   const uint64_t n_slots = h_row_offsets.empty() ? 0 : h_row_offsets[n_lists];
-  if (pq_bits != 8 || n_slots == 0 || n_slots + kLeadPlaneSlack > 0xFFFFFFFFull) {
+  // narrower codes, a byte each
+  const bool widen = pq_bits >= 5 && pq_bits < 8 && n_slots != 0 && !conservative_memory_allocation;
+  if (widen) {
+    n_chunks8                = (pq_dim + 15u) / 16u;
+    const uint64_t gb8       = uint64_t(n_chunks8) * kIndexGroupSize * kIndexGroupVecLen;
+    const uint64_t n_groups  = n_slots / kIndexGroupSize;
+    // two groups of slack: the scan kernels read whole 64-row tiles past a list's last group
+    device_buffer wide_codes((n_groups + 2) * gb8);
+    CUVS_HIP_TRY(hipMemsetAsync(wide_codes.ptr, 0, wide_codes.bytes, stream));
+    launch_widen_codes(codes_arena.as<uint8_t>(), wide_codes.as<uint8_t>(), n_slots, pq_dim, pq_bits, n_chunks,
+                       n_chunks8, stream);
+    std::vector<uint8_t*> dptr(n_lists);
+    for (uint32_t l = 0; l < n_lists; l++) {
+      dptr[l] = wide_codes.as<uint8_t>() + (h_row_offsets[l] / kIndexGroupSize) * gb8;
+    }
+    device_buffer ptrs(sizeof(void*) * n_lists);
+    CUVS_HIP_TRY(hipMemcpyAsync(ptrs.ptr, dptr.data(), ptrs.bytes, hipMemcpyHostToDevice, stream));
+    const uint64_t book_rows = pq_centers.bytes / (sizeof(float) * book_size);
+    device_buffer books(book_rows * 256 * sizeof(float));
+    launch_pad_codebooks(pq_centers.as<float>(), books.as<float>(), book_rows, book_size, stream);
+    CUVS_HIP_TRY(hipStreamSynchronize(stream));  // `dptr` goes out of scope; the old buffers are released
+    codes8_arena = std::move(wide_codes);
+    data_ptrs8   = std::move(ptrs);
+    pq_centers8  = std::move(books);
+  } else {
+    codes8_arena = device_buffer();
+    data_ptrs8   = device_buffer();
+    pq_centers8  = device_buffer();
+    n_chunks8    = 0;
+  }
+  if ((pq_bits != 8 && !widen) || n_slots == 0 || n_slots + kLeadPlaneSlack > 0xFFFFFFFFull) {
     lead_plane = device_buffer();
     return;
   }
   device_buffer plane((n_slots + kLeadPlaneSlack) * sizeof(uint64_t));
   CUVS_HIP_TRY(hipMemsetAsync(plane.ptr, 0, plane.bytes, stream));
-  launch_build_lead_plane(codes_arena.as<uint8_t>(), plane.as<uint64_t>(), n_slots, n_chunks, stream);
+  launch_build_lead_plane(widen ? codes8_arena.as<uint8_t>() : codes_arena.as<uint8_t>(), plane.as<uint64_t>(), n_slots,
+                          widen ? n_chunks8 : n_chunks, stream);
   CUVS_HIP_TRY(hipStreamSynchronize(stream));  // the old plane is released on assignment
   lead_plane = std::move(plane);
 }
@@ -297,13 +328,13 @@ index<int64_t> clone(cuvs::resources const& res, const index<int64_t>& source)
   copy(dst.centers_i8, src.centers_i8);
   copy(dst.codes_arena, src.codes_arena);
   copy(dst.ids_arena, src.ids_arena);
-  copy(dst.lead_plane, src.lead_plane);
   dst.h_list_sizes  = src.h_list_sizes;
   dst.h_row_offsets = src.h_row_offsets;
   dst.list_sizes.allocate(sizeof(uint32_t) * dst.n_lists);
   dst.data_ptrs.allocate(sizeof(void*) * dst.n_lists);
   dst.inds_ptrs.allocate(sizeof(void*) * dst.n_lists);
   dst.recompute_internal_state(stream);  // the tables point into the copy's own arenas; synchronises
+  dst.rebuild_lead_plane(stream);
   return out;
 }
 

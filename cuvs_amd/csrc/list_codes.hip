@@ -148,7 +148,61 @@ __global__ void unmap_rows_kernel(const float* __restrict__ in, uint64_t n, T* _
 
 inline uint32_t blocks_for(uint64_t n, uint32_t block) { return uint32_t((n + block - 1) / block); }
 
+/** One thread per (row slot, 16-code chunk): the codes of the packed row as bytes, in the layout of
+ *  an 8-bit index (chunk c of row i at (i / 32) * n_chunks8 * 512 + c * 512 + (i % 32) * 16). */
+__global__ __launch_bounds__(kRowBlock) void widen_codes_kernel(const uint8_t* __restrict__ packed,
+                                                                uint8_t* __restrict__ wide, uint64_t n_slots,
+                                                                uint32_t pq_dim, uint32_t pq_bits,
+                                                                uint32_t n_chunks, uint32_t n_chunks8)
+{
+  const uint64_t t = uint64_t(blockIdx.x) * kRowBlock + threadIdx.x;
+  if (t >= n_slots * n_chunks8) { return; }
+  const uint64_t i    = t / n_chunks8;
+  const uint32_t c8   = uint32_t(t - i * n_chunks8);
+  const uint32_t cpc  = 128u / pq_bits;
+  const uint8_t* row0 = packed + (i >> 5) * n_chunks * 512u + (i & 31u) * 16u;
+  uint32_t w[4]       = {0, 0, 0, 0};
+#pragma unroll
+  for (uint32_t x = 0; x < 16; x++) {
+    const uint32_t j = c8 * 16u + x;
+    if (j < pq_dim) { w[x >> 2] |= stored_code(row0, j, cpc, pq_bits) << ((x & 3u) * 8u); }
+  }
+  *reinterpret_cast<uint4*>(wide + (i >> 5) * n_chunks8 * 512u + uint64_t(c8) * 512u + (i & 31u) * 16u) =
+    make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+/** dst[row][e] = e < book_size ? src[row][e] : 0 for 256 entries a row. */
+__global__ void pad_codebooks_kernel(const float* __restrict__ src, float* __restrict__ dst, uint64_t n_rows,
+                                     uint32_t book_size)
+{
+  const uint64_t t = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (t >= n_rows * 256u) { return; }
+  const uint64_t row = t >> 8;
+  const uint32_t e   = uint32_t(t & 255u);
+  dst[t]             = e < book_size ? src[row * book_size + e] : 0.0f;
+}
+
 }  // namespace
+
+void launch_widen_codes(const uint8_t* packed, uint8_t* wide, uint64_t n_slots, uint32_t pq_dim,
+                        uint32_t pq_bits, uint32_t n_chunks, uint32_t n_chunks8, hipStream_t stream)
+{
+  if (n_slots == 0) { return; }
+  const uint64_t blocks = (n_slots * n_chunks8 + kRowBlock - 1) / kRowBlock;
+  CUVS_EXPECTS(blocks <= 0x7FFFFFFFull, "too many row slots for one launch");
+  widen_codes_kernel<<<uint32_t(blocks), kRowBlock, 0, stream>>>(packed, wide, n_slots, pq_dim, pq_bits, n_chunks,
+                                                                n_chunks8);
+  CUVS_HIP_TRY(hipGetLastError());
+}
+
+void launch_pad_codebooks(const float* src, float* dst, uint64_t n_rows, uint32_t book_size, hipStream_t stream)
+{
+  if (n_rows == 0) { return; }
+  const uint64_t blocks = (n_rows * 256u + 255u) / 256u;
+  CUVS_EXPECTS(blocks <= 0x7FFFFFFFull, "too many codebook rows for one launch");
+  pad_codebooks_kernel<<<uint32_t(blocks), 256, 0, stream>>>(src, dst, n_rows, book_size);
+  CUVS_HIP_TRY(hipGetLastError());
+}
 
 void launch_unpack_codes(const uint8_t* list_data, uint32_t n_rows, uint32_t offset,
                          const uint32_t* rows, uint32_t pq_dim, uint32_t pq_bits, uint8_t* out,

@@ -371,10 +371,23 @@ void search(cuvs::resources const& res_c,
   sa.list_sizes   = ix.list_sizes.as<uint32_t>();
   sa.filter_bits  = filter_bits;
   sa.filter_nbits = filter_nbits;
+  if (ix.pq_bits != 8) { sa.lead_plane = nullptr; }
+  if (ix.wide() && !res.tuning.generic_scan) {
+    // 5 - 7 bit codes: the byte-wide copy of the lists, if one of the 8-bit kernels takes the shape
+    detail::scan_args w = sa;
+    w.pq_bits    = 8;
+    w.pq_centers = ix.pq_centers8.as<float>();
+    w.data_ptrs  = ix.data_ptrs8.as<const uint8_t*>();
+    w.lead_plane = ix.lead_plane.bytes != 0 ? ix.lead_plane.as<uint64_t>() : nullptr;
+    if (detail::scan_lds_bytes(w) <= kMaxLds &&
+        (detail::scan_stream_keys_per_pair(w) != 0 || detail::scan_fast_supported(w))) {
+      sa = w;
+    }
+  }
   // a table too large for LDS goes to global memory (8-bit codes, generic kernel)
   const bool global_lut = detail::scan_lds_bytes(sa) > kMaxLds;
   if (global_lut) {
-    CUVS_EXPECTS(ix.pq_bits == 8,
+    CUVS_EXPECTS(sa.pq_bits == 8,
                  "the lookup table (pq_dim = %u, pq_bits = %u, lut_dtype = %d) needs %zu bytes of LDS, "
                  "more than the %zu available; use a smaller lut_dtype",
                  ix.pq_dim, ix.pq_bits, int(params.lut_dtype), detail::scan_lds_bytes(sa), kMaxLds);
@@ -505,7 +518,7 @@ void search(cuvs::resources const& res_c,
     detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
                                  ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead,
                                  pl.fused ? kth : nullptr, n_survivors, s);
-    detail::launch_order_pairs(probes, chunk, ix.data_ptrs.as<const uint8_t*>(),
+    detail::launch_order_pairs(probes, chunk, sa.data_ptrs,
                                ix.inds_ptrs.as<const int64_t*>(), ix.ids_arena.as<int64_t>(), nq * P, P,
                                ix.n_lists, counters, sort_scratch, order, desc, lead, alive, few_pairs, list_rank, s);
     mark(2);

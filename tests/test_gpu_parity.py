@@ -942,6 +942,43 @@ def test_five_to_seven_bit_codes_filter_and_long_lists(orc):
         H.compare_results(nb2, d2, want_nb2, want_d2, 2e-3, exact=True)
 
 
+def test_byte_wide_copy_of_narrow_codes_follows_the_lists():
+    """5 - 7 bit codes are searched on a byte-per-code copy of the lists.  The copy is an
+    acceleration only: the generic kernel on the packed lists (search tuning), an index built with
+    conservative_memory_allocation (no copy) and the default path return the same neighbours and
+    distances, before and after the lists grow, and the early stop runs on these widths too."""
+    import datasets as testing
+    from cuvs_amd.resources import Resources
+    allrows = testing.gaussian_mixture(60000 + 2000, 128, 96, 0.15, seed=123, device="cuda")
+    data, queries = allrows[:60000], allrows[60000:]
+    first, second = data[:40000], data[40000:]
+    ids2 = torch.arange(40000, 60000, dtype=torch.int64, device="cuda")
+    for bits in (5, 6, 7):
+        kw = dict(n_lists=128, pq_dim=64, pq_bits=bits)
+        ids1 = torch.arange(40000, dtype=torch.int64, device="cuda")
+        trained = ivf_pq.build(ivf_pq.IndexParams(kmeans_trainset_fraction=0.5, add_data_on_build=False, **kw), first)
+        model = (trained.pq_centers, trained.centers_padded, trained.centers_rot, trained.rotation_matrix)
+        index = ivf_pq.extend(ivf_pq.build_precomputed(ivf_pq.IndexParams(**kw), 128, *model), first, ids1)
+        lean = ivf_pq.extend(ivf_pq.build_precomputed(
+            ivf_pq.IndexParams(conservative_memory_allocation=True, **kw), 128, *model), first, ids1)
+        plain, tuned = Resources(), Resources()
+        plain.enable_profiling(True)
+        tuned.set_search_tuning(generic_scan=True)
+        sp = ivf_pq.SearchParams(n_probes=20, lut_dtype=R_16F)
+        for step in range(2):
+            d, nb = ivf_pq.search(sp, index, queries, 10, resources=plain)
+            plain.sync()
+            assert ivf_pq.get_search_profile(plain)["n_screened_pairs"] == queries.shape[0] * 19, bits
+            d2, nb2 = ivf_pq.search(sp, index, queries, 10, resources=tuned)
+            d3, nb3 = ivf_pq.search(sp, lean, queries, 10)
+            assert torch.equal(nb, nb2) and torch.equal(d, d2), (bits, step, "generic kernel")
+            assert torch.equal(nb, nb3) and torch.equal(d, d3), (bits, step, "no copy")
+            if step == 0:
+                index = ivf_pq.extend(index, second, ids2)
+                lean = ivf_pq.extend(lean, second, ids2)
+        assert int(nb.max()) >= 40000  # the rows added later are found
+
+
 def test_four_bit_block_kernel_filter_and_long_lists(orc):
     """Lists of several thousand rows (more than one pruning segment of the candidate buffer) and a
     bitset filter."""
