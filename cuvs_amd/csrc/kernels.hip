@@ -172,16 +172,16 @@ __global__ __launch_bounds__(kBlock) void select_probes_kernel(const float* __re
 /*
  * Probe selection with the score row held in registers (n_probes <= 256).
  *
- * A block takes one query and walks its row in segments of 256 x 64 scores, thread t holding
- * scores t, t + 256, ... of the segment as ordered 32-bit keys.  Bound: the smallest score of each
+ * A block takes one query and walks its row in segments of 256 x PER scores (PER = 4, 16 or 64 by
+ * the row's length: a short row is not padded to 16,384 loads), thread t holding scores t,
+ * t + 256, ... of the segment as ordered 32-bit keys.  Bound: the smallest score of each
  * thread gives 256 distinct elements, so the n_probes-th smallest of those minima has at least
  * n_probes elements at or below it - and, for scores in no particular order, only a few more.
  * Everything at or below the bound (and the best of the earlier segments) is collected into a small
  * LDS list and sorted by (score, list id); one pass over HBM, no histogram atomics.  If the list
  * overflows (adversarially ordered rows) the block falls back to the radix selection.
  */
-constexpr uint32_t kSelPerThread = 64;
-constexpr uint32_t kSelCap       = 1024;
+constexpr uint32_t kSelCap = 1024;
 
 /** Ascending bitonic sort of one 32-bit key per lane across the wave. */
 __device__ __forceinline__ uint32_t wave_sort_u32(uint32_t v, uint32_t lane)
@@ -201,6 +201,7 @@ __device__ __forceinline__ uint32_t wave_sort_u32(uint32_t v, uint32_t lane)
   return v;
 }
 
+template <uint32_t kSelPerThread>
 __global__ __launch_bounds__(kBlock, 3) void select_probes_fast_kernel(const float* __restrict__ scores,
                                                                      uint32_t n_lists,
                                                                      uint32_t n_probes,
@@ -1551,7 +1552,13 @@ void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_li
 {
   if (n_queries == 0) { return; }
   if (n_probes <= kBlock) {
-    select_probes_fast_kernel<<<n_queries, kBlock, 0, stream>>>(scores, n_lists, n_probes, probes, only);
+    if (n_lists <= 4u * kBlock) {
+      select_probes_fast_kernel<4><<<n_queries, kBlock, 0, stream>>>(scores, n_lists, n_probes, probes, only);
+    } else if (n_lists <= 16u * kBlock) {
+      select_probes_fast_kernel<16><<<n_queries, kBlock, 0, stream>>>(scores, n_lists, n_probes, probes, only);
+    } else {
+      select_probes_fast_kernel<64><<<n_queries, kBlock, 0, stream>>>(scores, n_lists, n_probes, probes, only);
+    }
     CUVS_LAUNCH_CHECK();
     return;
   }
