@@ -205,6 +205,117 @@ __device__ uint32_t block_select_sorted(KeyFn key_of, uint32_t n, uint32_t k,
   return cnt < k ? cnt : k;
 }
 
+/**
+ * The same result for at most kBlock * kMinimaPer keys and k <= kBlock, in one pass over the keys:
+ * thread t holds keys t, t + kBlock, ... in registers; the k-th smallest of the kBlock per-thread
+ * minima (by the keys' high words) is at or above the k-th smallest key, and for keys in no
+ * particular order only a few more than k lie at or below it; those are collected in LDS (the
+ * histogram area of `sm`) and ranked.  Returns false, with nothing written, when more than 1024
+ * keys pass the bound (keys in an adversarial order, or k close to the number of threads' worth of
+ * valid keys): the caller then selects by radix passes.
+ */
+constexpr uint32_t kMinimaPer = 16;
+template <typename KeyFn>
+__device__ bool block_select_by_minima(KeyFn key_of, uint32_t n, uint32_t k, unsigned long long* out,
+                                       uint32_t out_cap, select_smem& sm)
+{
+  static_assert(sizeof(sm.hist) >= 1024 * sizeof(unsigned long long), "candidate area");
+  constexpr uint32_t kCap = 1024;
+  __shared__ uint32_t mins[kBlock];
+  __shared__ uint32_t s_bound, s_count;
+  unsigned long long* cand = reinterpret_cast<unsigned long long*>(sm.hist);
+  const uint32_t tid  = threadIdx.x;
+  const uint32_t lane = tid & 63u;
+  const uint32_t wid  = tid >> 6;
+  unsigned long long key[kMinimaPer];
+#pragma unroll
+  for (uint32_t j = 0; j < kMinimaPer; j++) {
+    const uint32_t i = j * kBlock + tid;
+    key[j]           = i < n ? key_of(i) : kInvalidKey;
+  }
+  uint32_t mine = 0xFFFFFFFFu;
+#pragma unroll
+  for (uint32_t j = 0; j < kMinimaPer; j++) {
+    const uint32_t hi = uint32_t(key[j] >> 32);
+    mine              = hi < mine ? hi : mine;
+  }
+  if (tid == 0) {
+    s_bound = 0xFFFFFFFFu;
+    s_count = 0;
+  }
+  // ascending bitonic sort of the wave's 64 minima
+  uint32_t v = mine;
+#pragma unroll
+  for (uint32_t size = 2; size <= 64; size <<= 1) {
+#pragma unroll
+    for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+      const uint32_t other = __shfl_xor(v, int(stride), 64);
+      const bool ascending = (lane & size) == 0 || size == 64;
+      const bool low_half  = (lane & stride) == 0;
+      const uint32_t lo    = v < other ? v : other;
+      const uint32_t hi    = v < other ? other : v;
+      v                    = (low_half == ascending) ? lo : hi;
+    }
+  }
+  mins[tid] = v;
+  __syncthreads();
+  // rank of (v, wid, lane) among all minima: `<=` against earlier waves' lists
+  uint32_t rank = lane;
+#pragma unroll
+  for (uint32_t w = 0; w < kBlock / 64; w++) {
+    if (w == wid) { continue; }
+    const uint32_t* list = mins + w * 64u;
+    uint32_t lo = 0, hi = 64;
+#pragma unroll
+    for (int step = 0; step < 6; step++) {
+      const uint32_t mid = (lo + hi) >> 1;
+      const uint32_t m   = list[mid];
+      const bool before  = w < wid ? m <= v : m < v;
+      lo                 = before ? mid + 1u : lo;
+      hi                 = before ? hi : mid;
+    }
+    rank += lo;
+  }
+  if (rank == k - 1u) { s_bound = v; }
+  __syncthreads();
+  const uint32_t bound = s_bound;
+  if (mine <= bound) {
+#pragma unroll
+    for (uint32_t j = 0; j < kMinimaPer; j++) {
+      if (key[j] != kInvalidKey && uint32_t(key[j] >> 32) <= bound) {
+        const uint32_t pos = atomicAdd(&s_count, 1u);
+        if (pos < kCap) { cand[pos] = key[j]; }
+      }
+    }
+  }
+  __syncthreads();
+  const uint32_t total = s_count;
+  __syncthreads();  // everybody has read the count before a later call resets it
+  if (total > kCap) { return false; }
+  if (total <= kBlock) {
+    // few candidates: place each by counting the smaller ones (keys are distinct)
+    unsigned long long mykey = kInvalidKey;
+    uint32_t pos             = 0;
+    if (tid < total) {
+      mykey = cand[tid];
+      for (uint32_t x = 0; x < total; x++) { pos += cand[x] < mykey ? 1u : 0u; }
+    }
+    for (uint32_t r = tid; r < out_cap; r += kBlock) { out[r] = kInvalidKey; }
+    __syncthreads();
+    if (tid < total && pos < out_cap) { out[pos] = mykey; }
+    __syncthreads();
+  } else {
+    uint32_t n_sort = 1;
+    while (n_sort < total) { n_sort <<= 1; }
+    for (uint32_t i = total + tid; i < n_sort; i += kBlock) { cand[i] = kInvalidKey; }
+    __syncthreads();
+    block_bitonic_sort(cand, n_sort);
+    for (uint32_t r = tid; r < out_cap; r += kBlock) { out[r] = r < total ? cand[r] : kInvalidKey; }
+    __syncthreads();
+  }
+  return true;
+}
+
 /* ---------------------------------------------------------------------------------------- */
 /* lookup-table element types                                                                */
 /* ---------------------------------------------------------------------------------------- */

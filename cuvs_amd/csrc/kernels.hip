@@ -1196,7 +1196,10 @@ __device__ void merge_query(const merge_args& a, uint32_t out_cap, uint32_t q)
     n                              = a.n_probes * a.keys_per_pair;
     const unsigned long long* keys = a.in_keys + uint64_t(q) * n;
     if (a.alive == nullptr) {
-      block_select_sorted([keys](uint32_t i) { return keys[i]; }, n, a.k, out, out_cap, sm);
+      auto key_of = [keys](uint32_t i) { return keys[i]; };
+      if (!(n <= kBlock * kMinimaPer && a.k <= kBlock && block_select_by_minima(key_of, n, a.k, out, out_cap, sm))) {
+        block_select_sorted(key_of, n, a.k, out, out_cap, sm);
+      }
     } else {
       // pairs that the screen dropped wrote no keys: gather the slots that did, select among those
       __shared__ uint16_t live_slots[kMergeMaxProbes];
@@ -1229,9 +1232,11 @@ __device__ void merge_query(const merge_args& a, uint32_t out_cap, uint32_t q)
         }
         __syncthreads();
       } else {
-        block_select_sorted(
-          [keys, kpp](uint32_t i) { return keys[uint32_t(live_slots[i / kpp]) * kpp + i % kpp]; },
-          n_keys, a.k, out, out_cap, sm);
+        auto key_of = [keys, kpp](uint32_t i) { return keys[uint32_t(live_slots[i / kpp]) * kpp + i % kpp]; };
+        if (!(n_keys <= kBlock * kMinimaPer && a.k <= kBlock &&
+              block_select_by_minima(key_of, n_keys, a.k, out, out_cap, sm))) {
+          block_select_sorted(key_of, n_keys, a.k, out, out_cap, sm);
+        }
       }
     }
   } else {
