@@ -249,7 +249,7 @@ def main():
                  else "scan_nibble_pack_kernel" if (nibble and args.internal == "f16" and pq_dim % 128 == 0
                                                     and pq_dim <= 512 and k <= 64 and args.lut != "f32")
                  else "scan_nibble_kernel" if nibble
-                 else "scan_kernel" if (pq_bits not in (5, 6, 7, 8) or (pq_dim, pq_len) not in ((64, 2), (48, 2), (32, 4)))
+                 else "scan_kernel" if (pq_bits not in (5, 6, 7, 8) or (pq_dim, pq_len) not in ((64, 2), (48, 2), (32, 4), (32, 2)))
                  else "scan_stream_kernel" if (args.lut != "f32" and k <= 128) else "scan_fast_kernel")
     if first_call_screened and not early_stop:
         log("the screen kept most pairs on the first search: it is off for the searches after it")

@@ -727,7 +727,7 @@ uint32_t scan_stream_keys_per_pair(const scan_args& a)
   if (a.rot_dim != a.pq_dim * a.pq_len) { return 0; }
   if (a.lut_dtype != CUDA_R_16F && a.lut_dtype != CUDA_R_8U) { return 0; }
   const bool shape = (a.pq_dim == 64 && a.pq_len == 2) || (a.pq_dim == 48 && a.pq_len == 2) ||
-                     (a.pq_dim == 32 && a.pq_len == 4);
+                     (a.pq_dim == 32 && a.pq_len == 4) || (a.pq_dim == 32 && a.pq_len == 2);
   return shape ? kStreamWG * a.k : 0;
 }
 
@@ -737,6 +737,7 @@ bool launch_scan_stream(const scan_args& a, hipStream_t stream)
   if (a.pq_dim == 64 && a.pq_len == 2) { return launch_stream_kind<4, 2>(a, stream); }
   if (a.pq_dim == 48 && a.pq_len == 2) { return launch_stream_kind<3, 2>(a, stream); }
   if (a.pq_dim == 32 && a.pq_len == 4) { return launch_stream_kind<2, 4>(a, stream); }
+  if (a.pq_dim == 32 && a.pq_len == 2) { return launch_stream_kind<2, 2>(a, stream); }
   return false;
 }
 

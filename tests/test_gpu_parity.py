@@ -311,9 +311,9 @@ def test_getters_round_trip(orc):
     assert int(index.list_sizes.sum().item()) == 800
 
 
-# --- shapes served by the persistent 8-bit scan kernel (pq_dim x pq_len in {64x2, 48x2, 32x4}) ---
+# --- shapes served by the persistent 8-bit scan kernel (pq_dim x pq_len in {64x2, 48x2, 32x4, 32x2}) ---
 
-@pytest.mark.parametrize("dim,pq_dim", [(128, 64), (96, 48), (128, 32)])
+@pytest.mark.parametrize("dim,pq_dim", [(128, 64), (96, 48), (128, 32), (64, 32)])
 @pytest.mark.parametrize("lut,internal,rtol", [(R_32F, R_32F, 1e-5), (R_16F, R_32F, 2e-3),
                                                (R_8U, R_32F, 2e-3), (R_16F, R_16F, 2e-3),
                                                (R_8U, R_16F, 2e-3)])
