@@ -121,6 +121,26 @@ void finish_edit(cuvs::resources const& res, index_impl& ix)
 
 namespace codepacker {
 
+void unpack(cuvs::resources const& res, const uint8_t* list_data, uint32_t pq_bits, uint32_t offset,
+            device_matrix_view<uint8_t> codes)
+{
+  CUVS_EXPECTS(pq_bits >= 4 && pq_bits <= 8, "pq_bits must be within [4, 8], got %u", pq_bits);
+  CUVS_EXPECTS(list_data != nullptr || codes.extent(0) == 0, "list_data is null");
+  if (codes.extent(0) == 0) { return; }
+  detail::launch_unpack_codes(list_data, uint32_t(codes.extent(0)), offset, nullptr, uint32_t(codes.extent(1)),
+                              pq_bits, codes.data_handle(), res.stream());
+}
+
+void pack(cuvs::resources const& res, device_matrix_view<const uint8_t> codes, uint32_t pq_bits,
+          uint32_t offset, uint8_t* list_data)
+{
+  CUVS_EXPECTS(pq_bits >= 4 && pq_bits <= 8, "pq_bits must be within [4, 8], got %u", pq_bits);
+  CUVS_EXPECTS(list_data != nullptr || codes.extent(0) == 0, "list_data is null");
+  if (codes.extent(0) == 0) { return; }
+  detail::launch_pack_codes(list_data, codes.data_handle(), false, uint32_t(codes.extent(0)), offset,
+                            uint32_t(codes.extent(1)), pq_bits, res.stream());
+}
+
 void unpack_list_data(cuvs::resources const& res, const index<int64_t>& idx,
                       device_matrix_view<uint8_t> out_codes, uint32_t label, uint32_t offset)
 {

@@ -264,6 +264,24 @@ void deserialize(cuvs::resources const& res, const std::string& filename, index<
 namespace helpers {
 namespace codepacker {
 
+/** ivf_pq.hpp:2597 -- codes of rows offset .. offset + codes.extent(0) - 1 of a bare list buffer
+ *  (interleaved groups of 32 rows, as `index::lists()[label]->data` in the reference; here a
+ *  pointer: the extents follow from pq_dim = codes.extent(1) and pq_bits), one code per byte. */
+void unpack(cuvs::resources const& res,
+            const uint8_t* list_data,
+            uint32_t pq_bits,
+            uint32_t offset,
+            device_matrix_view<uint8_t> codes);
+
+/** ivf_pq.hpp:2669 -- writes `codes` [n_rows, pq_dim], one code per byte, into the rows from
+ *  `offset` on of a bare list buffer.  A buffer that belongs to an index is better written through
+ *  pack_list_data, which also refreshes what the index derives from its lists. */
+void pack(cuvs::resources const& res,
+          device_matrix_view<const uint8_t> codes,
+          uint32_t pq_bits,
+          uint32_t offset,
+          uint8_t* list_data);
+
 /** ivf_pq.hpp:2818 -- codes of rows offset .. offset + out_codes.extent(0) - 1 of list `label`, one
  *  code per byte: out_codes is [n_take, pq_dim]. */
 void unpack_list_data(cuvs::resources const& res,

@@ -165,6 +165,25 @@ void run(uint32_t pq_bits, ivf_pq::codebook_gen kind, uint32_t pq_dim_asked, con
   res.sync();
   REQUIRE(to_host(d_part, size_t(20) * pq_dim) ==
           std::vector<uint8_t>(codes.begin() + 37 * pq_dim, codes.begin() + 57 * pq_dim));
+  {
+    // the same through the bare-buffer calls: reading the index's own list buffer, and a round trip
+    // through a scratch buffer of four groups of 32 rows
+    auto ptrs = to_host(index.data_ptrs(), n_lists);
+    packer::unpack(res, ptrs[label], pq_bits, 37, make_device_matrix_view(d_part, 20, pq_dim));
+    res.sync();
+    REQUIRE(to_host(d_part, size_t(20) * pq_dim) ==
+            std::vector<uint8_t>(codes.begin() + 37 * pq_dim, codes.begin() + 57 * pq_dim));
+    const uint32_t cpc = 128 / pq_bits, n_chunks = (pq_dim + cpc - 1) / cpc;
+    auto* d_buf = device_array<uint8_t>(size_t(4) * n_chunks * 512);
+    REQUIRE(hipMemset(d_buf, 0, size_t(4) * n_chunks * 512) == hipSuccess);
+    packer::pack(res, make_device_matrix_view<const uint8_t>(d_codes, 60, pq_dim), pq_bits, 50, d_buf);
+    auto* d_back = device_array<uint8_t>(size_t(60) * pq_dim);
+    packer::unpack(res, d_buf, pq_bits, 50, make_device_matrix_view(d_back, 60, pq_dim));
+    res.sync();
+    REQUIRE(to_host(d_back, size_t(60) * pq_dim) == std::vector<uint8_t>(codes.begin(), codes.begin() + 60 * pq_dim));
+    REQUIRE(throws([&] { packer::unpack(res, d_buf, 9, 0, make_device_matrix_view(d_back, 4, pq_dim)); }));
+    REQUIRE(hipFree(d_buf) == hipSuccess && hipFree(d_back) == hipSuccess);
+  }
   const std::vector<uint32_t> picks = {3, 0, n - 1, 33, 32, 3};
   uint32_t* d_picks = to_device(picks);
   packer::unpack_list_data(res, index, make_device_vector_view<const uint32_t>(d_picks, picks.size()),
