@@ -447,13 +447,14 @@ void search(cuvs::resources const& res_c,
   if (early_stop && res.tuning.early_stop == 0 && ix.feedback.host != nullptr) {
     auto& fb = ix.feedback;
     std::lock_guard<std::mutex> guard(fb.mu);
-    fb.collect();
+    // while a stream captures, an event query invalidates the capture: the verdict stays as it is
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    CUVS_HIP_TRY(hipStreamIsCapturing(s, &capture));
+    if (capture == hipStreamCaptureStatusNone) { fb.collect(); }
     if (fb.off && fb.probes == P && fb.k == k) {
       fb.plain_searches += 1;
       if (fb.plain_searches % detail::screen_feedback::kScreenRecheck != 0) { early_stop = false; }
     }
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    CUVS_HIP_TRY(hipStreamIsCapturing(s, &capture));
     observe_screen = early_stop && capture == hipStreamCaptureStatusNone;
   }
   const uint32_t lead          = early_stop ? kLeadProbes : P;
