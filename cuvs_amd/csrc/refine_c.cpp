@@ -39,12 +39,14 @@ extern "C" cuvsError_t cuvsRefine(cuvsResources_t res,
     const auto& candidates = candidates_t->dl_tensor;
     const auto& indices    = indices_t->dl_tensor;
     const auto& distances  = distances_t->dl_tensor;
-    // the reference also takes all-host tensors and refines on the CPU; this library has no CPU
-    // path, so every tensor must be reachable from the device (pinned host memory is)
-    CUVS_EXPECTS(is_dlpack_device_compatible(dataset) && is_dlpack_device_compatible(queries) &&
-                   is_dlpack_device_compatible(candidates) && is_dlpack_device_compatible(indices) &&
-                   is_dlpack_device_compatible(distances),
-                 "Tensors must all be accessible from the device");
+    // all matrices on the device (or reachable from it: pinned, managed), or all in plain host
+    // memory; the latter are staged through the device, a batch of queries at a time
+    const bool on_device = is_dlpack_device_compatible(dataset);
+    CUVS_EXPECTS(on_device == is_dlpack_device_compatible(queries) &&
+                   on_device == is_dlpack_device_compatible(candidates) &&
+                   on_device == is_dlpack_device_compatible(indices) &&
+                   on_device == is_dlpack_device_compatible(distances),
+                 "Tensors must either all be on device memory, or all on host memory");
     CUVS_EXPECTS(candidates.dtype.code == kDLInt && candidates.dtype.bits == 64,
                  "candidates should be of type int64_t");
     CUVS_EXPECTS(indices.dtype.code == kDLInt && indices.dtype.bits == 64,
@@ -71,11 +73,18 @@ extern "C" cuvsError_t cuvsRefine(cuvsResources_t res,
                  "Number of columns in output indices and distances matrices must be equal to k");
     CUVS_EXPECTS(queries.shape[1] == dataset.shape[1],
                  "Number of columns must be equal for dataset and queries");
-    cuvs::neighbors::refine(*res_of(res), tensor_data(dataset_t), tensor_data(queries_t), t,
-                            dataset.shape[0], n_queries, dataset.shape[1],
-                            static_cast<const int64_t*>(tensor_data(candidates_t)), candidates.shape[1],
-                            static_cast<int64_t*>(tensor_data(indices_t)),
-                            static_cast<float*>(tensor_data(distances_t)), indices.shape[1],
-                            cuvs::distance::DistanceType(int(metric)));
+    const auto type_of_metric = cuvs::distance::DistanceType(int(metric));
+    const auto* cand          = static_cast<const int64_t*>(tensor_data(candidates_t));
+    auto* out_idx             = static_cast<int64_t*>(tensor_data(indices_t));
+    auto* out_dist            = static_cast<float*>(tensor_data(distances_t));
+    if (on_device) {
+      cuvs::neighbors::refine(*res_of(res), tensor_data(dataset_t), tensor_data(queries_t), t, dataset.shape[0],
+                              n_queries, dataset.shape[1], cand, candidates.shape[1], out_idx, out_dist,
+                              indices.shape[1], type_of_metric);
+    } else {
+      cuvs::neighbors::refine_host(*res_of(res), tensor_data(dataset_t), tensor_data(queries_t), t,
+                                   dataset.shape[0], n_queries, dataset.shape[1], cand, candidates.shape[1],
+                                   out_idx, out_dist, indices.shape[1], type_of_metric);
+    }
   });
 }

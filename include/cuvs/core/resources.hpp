@@ -46,6 +46,22 @@ device_matrix_view<T> make_device_matrix_view(T* data, int64_t rows, int64_t col
   return device_matrix_view<T>{data, rows, cols};
 }
 
+/** Non-owning row-major 2-D view of host memory (role of raft::host_matrix_view<T, int64_t, row_major>). */
+template <typename T>
+struct host_matrix_view {
+  T* data      = nullptr;
+  int64_t rows = 0;
+  int64_t cols = 0;
+  T* data_handle() const { return data; }
+  int64_t extent(int i) const { return i == 0 ? rows : cols; }
+};
+
+template <typename T>
+host_matrix_view<T> make_host_matrix_view(T* data, int64_t rows, int64_t cols)
+{
+  return host_matrix_view<T>{data, rows, cols};
+}
+
 /** Non-owning 1-D view (role of raft::device_vector_view<T, uint32_t>). */
 template <typename T>
 struct device_vector_view {

@@ -19,9 +19,11 @@ extern "C" {
  *
  * dataset [n_rows, dim] and queries [n_queries, dim] of one element type (float32, float16, int8,
  * uint8), candidates int64 [n_queries, n_candidates], indices int64 [n_queries, k], distances
- * float32 [n_queries, k], k <= n_candidates.  All tensors must be accessible from the device
- * (device, managed or pinned host memory).  Candidate ids outside [0, n_rows) are skipped; rows of
- * the output that cannot be filled hold id -1 and the largest float.
+ * float32 [n_queries, k], k <= n_candidates.  The tensors are either all accessible from the
+ * device (device, managed or pinned host memory) or all in plain host memory (kDLCPU); host
+ * matrices are staged through the device, a batch of queries at a time, and the call returns when
+ * the outputs are complete.  Candidate ids outside [0, n_rows) are skipped; rows of the output
+ * that cannot be filled hold id -1 and the largest float.
  */
 CUVS_EXPORT cuvsError_t cuvsRefine(cuvsResources_t res,
                                    DLManagedTensor* dataset,

@@ -25,11 +25,30 @@ void refine(cuvs::resources const& res,
             device_matrix_view<float> distances,
             cuvs::distance::DistanceType metric = cuvs::distance::DistanceType::L2Unexpanded);
 
+/** The same on matrices in host memory (cuVS refine.hpp:287-293 and the overloads for half, int8_t
+ *  and uint8_t that follow it).  The reference computes these on the CPU; here the candidate rows
+ *  are gathered into pinned memory, a batch of queries at a time, and the device kernel above
+ *  ranks them: same results as the device overload.  Returns when the outputs are complete. */
+template <typename T>
+void refine(cuvs::resources const& res,
+            host_matrix_view<const T> dataset,
+            host_matrix_view<const T> queries,
+            host_matrix_view<const int64_t> neighbor_candidates,
+            host_matrix_view<int64_t> indices,
+            host_matrix_view<float> distances,
+            cuvs::distance::DistanceType metric = cuvs::distance::DistanceType::L2Unexpanded);
+
 /** Type-erased entry point behind the C API. */
 void refine(cuvs::resources const& res, const void* dataset, const void* queries,
             ivf_pq::elem_type type, int64_t n_rows, int64_t n_queries, int64_t dim,
             const int64_t* candidates, int64_t n_candidates, int64_t* indices, float* distances,
             int64_t k, cuvs::distance::DistanceType metric);
+
+/** Type-erased entry point for matrices in host memory. */
+void refine_host(cuvs::resources const& res, const void* dataset, const void* queries,
+                 ivf_pq::elem_type type, int64_t n_rows, int64_t n_queries, int64_t dim,
+                 const int64_t* candidates, int64_t n_candidates, int64_t* indices, float* distances,
+                 int64_t k, cuvs::distance::DistanceType metric);
 
 }  // namespace cuvs::neighbors
 

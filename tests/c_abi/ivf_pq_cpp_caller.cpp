@@ -95,6 +95,19 @@ int main()
   }
   if (self < n_queries * 95 / 100) { std::fprintf(stderr, "%d of %ld rows found themselves\n", self, long(n_queries)); return 1; }
 
+  // the overload for matrices in host memory: same rows, same distances
+  {
+    const auto cand = to_host(d_nb, n_queries * k_wide);
+    std::vector<int64_t> h_nb(n_queries * k);
+    std::vector<float> h_dist(n_queries * k);
+    refine<float>(res, cuvs::make_host_matrix_view<const float>(data.data(), n_rows, dim),
+                  cuvs::make_host_matrix_view<const float>(data.data(), n_queries, dim),
+                  cuvs::make_host_matrix_view<const int64_t>(cand.data(), n_queries, k_wide),
+                  cuvs::make_host_matrix_view(h_nb.data(), n_queries, k),
+                  cuvs::make_host_matrix_view(h_dist.data(), n_queries, k));
+    if (h_nb != nb || h_dist != dist) { std::fprintf(stderr, "host refine differs from device refine\n"); return 1; }
+  }
+
   // the same rows as two half-indexes under one model: merged answers = the whole index's answers
   ivf_pq::index_params empty = ip;
   empty.add_data_on_build    = false;

@@ -717,6 +717,63 @@ def test_refine_after_search_raises_recall(orc):
     np.testing.assert_allclose(d.cpu().numpy(), want_d, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.int8, np.uint8])
+@pytest.mark.parametrize("metric", ["sqeuclidean", "euclidean", "inner_product"])
+def test_refine_of_host_matrices_is_the_device_result(orc, dtype, metric):
+    """Matrices in plain host memory (the reference refines those on the CPU): staged through the
+    device, same rows and distances as the device overload, and the oracle's."""
+    from cuvs_amd import refine
+    rng = np.random.default_rng(15)
+    n, dim, nq, nc, k = 3000, 100, 70, 64, 10
+    data = H.make_data(n, dim, dtype, 31)
+    q = H.make_data(nq, dim, dtype, 32)
+    cand = rng.integers(0, n, (nq, nc)).astype(np.int64)
+    cand[0, :6] = [-1, n, -5, n + 1, 2 ** 40, -2 ** 40]
+    cand[1, :] = n
+    cand[2, 1:] = cand[2, 0]  # one row sixty-four times: ties go by position in both overloads
+    d_dev, ids_dev = refine(G.to_dev(data), G.to_dev(q), G.to_dev(cand), k, metric=metric)
+    d, ids = refine(data, q, cand, k, metric=metric)
+    assert isinstance(d, np.ndarray) and isinstance(ids, np.ndarray)
+    assert np.array_equal(ids, ids_dev.cpu().numpy())
+    assert np.array_equal(d.view(np.uint32), d_dev.cpu().numpy().view(np.uint32))
+    # CPU tensors take the same way, into outputs the caller made
+    out_i = torch.full((nq, k), -7, dtype=torch.int64)
+    out_d = torch.zeros((nq, k), dtype=torch.float32)
+    refine(torch.from_numpy(data), torch.from_numpy(q), torch.from_numpy(cand), metric=metric,
+           indices=out_i, distances=out_d)
+    assert np.array_equal(out_i.numpy(), ids) and np.array_equal(out_d.numpy(), d)
+    code = {"sqeuclidean": 0, "euclidean": 1, "inner_product": 6}[metric]
+    want_ids, want_d = orc.refine(data, q, cand, k, code)
+    np.testing.assert_allclose(d, want_d, rtol=1e-5, atol=1e-6)
+    assert (ids[1] == -1).all()
+
+
+def test_refine_of_host_matrices_in_several_batches(orc):
+    """More candidate rows than one staging batch holds (256 MiB): the batches join up."""
+    from cuvs_amd import refine
+    rng = np.random.default_rng(16)
+    n, dim, nq, nc, k = 5000, 1024, 2500, 40, 5   # 2500 x 40 x 4 KiB = 390 MiB of candidate rows
+    data = rng.standard_normal((n, dim), dtype=np.float32)
+    q = rng.standard_normal((nq, dim), dtype=np.float32)
+    cand = rng.integers(0, n, (nq, nc)).astype(np.int64)
+    d, ids = refine(data, q, cand, k)
+    d_dev, ids_dev = refine(G.to_dev(data), G.to_dev(q), G.to_dev(cand), k)
+    assert np.array_equal(ids, ids_dev.cpu().numpy())
+    assert np.array_equal(d.view(np.uint32), d_dev.cpu().numpy().view(np.uint32))
+
+
+def test_refine_refuses_a_mix_of_host_and_device_matrices(orc):
+    from cuvs_amd import refine
+    data = np.zeros((10, 4), dtype=np.float32)
+    q = np.zeros((3, 4), dtype=np.float32)
+    cand = np.zeros((3, 5), dtype=np.int64)
+    with pytest.raises(CuvsError, match="either all be on device memory, or all on host memory"):
+        refine(G.to_dev(data), q, cand, 2, indices=np.zeros((3, 2), np.int64),
+               distances=np.zeros((3, 2), np.float32))
+    with pytest.raises(CuvsError, match="either all be on device memory, or all on host memory"):
+        refine(data, q, G.to_dev(cand), 2)
+
+
 def test_refine_validation(orc):
     from cuvs_amd import refine
     data = G.to_dev(np.zeros((10, 4), dtype=np.float32))
