@@ -141,6 +141,26 @@ void pack(cuvs::resources const& res, device_matrix_view<const uint8_t> codes, u
                             uint32_t(codes.extent(1)), pq_bits, res.stream());
 }
 
+void unpack_contiguous(cuvs::resources const& res, const uint8_t* list_data, uint32_t pq_bits, uint32_t offset,
+                       uint32_t n_rows, uint32_t pq_dim, uint8_t* codes)
+{
+  CUVS_EXPECTS(pq_bits >= 4 && pq_bits <= 8, "pq_bits must be within [4, 8], got %u", pq_bits);
+  CUVS_EXPECTS(pq_dim > 0, "pq_dim must be positive");
+  if (n_rows == 0) { return; }
+  CUVS_EXPECTS(list_data != nullptr && codes != nullptr, "list_data and codes must not be null");
+  detail::launch_unpack_contiguous(list_data, n_rows, offset, pq_dim, pq_bits, codes, res.stream());
+}
+
+void pack_contiguous(cuvs::resources const& res, const uint8_t* codes, uint32_t n_rows, uint32_t pq_dim,
+                     uint32_t pq_bits, uint32_t offset, uint8_t* list_data)
+{
+  CUVS_EXPECTS(pq_bits >= 4 && pq_bits <= 8, "pq_bits must be within [4, 8], got %u", pq_bits);
+  CUVS_EXPECTS(pq_dim > 0, "pq_dim must be positive");
+  if (n_rows == 0) { return; }
+  CUVS_EXPECTS(list_data != nullptr && codes != nullptr, "list_data and codes must not be null");
+  detail::launch_pack_codes(list_data, codes, true, n_rows, offset, pq_dim, pq_bits, res.stream());
+}
+
 void unpack_list_data(cuvs::resources const& res, const index<int64_t>& idx,
                       device_matrix_view<uint8_t> out_codes, uint32_t label, uint32_t offset)
 {

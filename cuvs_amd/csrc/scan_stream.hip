@@ -131,7 +131,7 @@ __device__ __forceinline__ uint16_t table_entry(float score)
 #define ST_HEAD "v_mov_b32 %[acc], 0\n\t" ST_ISSUE(0, c0, c1, va) ST_ISSUE(1, c2, c3, vb)
 /* a chunk that is not the last: its two groups are added, groups o + 2 and o + 3 issued */
 #define ST_CHUNK(o0, o1, o2, o3, c4, c5, c6, c7, ADD, CHECK)  \
-  ST_WAIT8 ADD(va) ST_ISSUE(o2, c4, c5, va)                   \
+  ST_WAIT8 ADD(va) CHECK ST_ISSUE(o2, c4, c5, va)             \
   ST_WAIT8 ADD(vb) CHECK ST_ISSUE(o3, c6, c7, vb)
 #define ST_TAIL(ADD) ST_WAIT8 ADD(va) ST_WAIT0 ADD(vb) ".Ltile_done%=:\n\t" ST_WAIT0
 #define ST_BODY_2(ADD, CHECK) ST_HEAD ST_CHUNK(0, 1, 2, 3, c4, c5, c6, c7, ADD, CHECK) ST_TAIL(ADD)

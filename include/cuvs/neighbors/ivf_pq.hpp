@@ -282,6 +282,26 @@ void pack(cuvs::resources const& res,
           uint32_t offset,
           uint8_t* list_data);
 
+/** ivf_pq.hpp:2637 -- the same rows of a bare list buffer as bit strings: row r of `codes` holds
+ *  ceildiv(pq_dim * pq_bits, 8) bytes, code j in bits [j * pq_bits, (j + 1) * pq_bits). */
+void unpack_contiguous(cuvs::resources const& res,
+                       const uint8_t* list_data,
+                       uint32_t pq_bits,
+                       uint32_t offset,
+                       uint32_t n_rows,
+                       uint32_t pq_dim,
+                       uint8_t* codes);
+
+/** ivf_pq.hpp:2705 -- writes `n_rows` bit strings of that form into the rows from `offset` on of a
+ *  bare list buffer. */
+void pack_contiguous(cuvs::resources const& res,
+                     const uint8_t* codes,
+                     uint32_t n_rows,
+                     uint32_t pq_dim,
+                     uint32_t pq_bits,
+                     uint32_t offset,
+                     uint8_t* list_data);
+
 /** ivf_pq.hpp:2818 -- codes of rows offset .. offset + out_codes.extent(0) - 1 of list `label`, one
  *  code per byte: out_codes is [n_take, pq_dim]. */
 void unpack_list_data(cuvs::resources const& res,

@@ -198,6 +198,30 @@ void run(uint32_t pq_bits, ivf_pq::codebook_gen kind, uint32_t pq_dim_asked, con
   res.sync();
   const auto flat = to_host(d_flat, size_t(n) * row_bytes);
   REQUIRE(flat == contiguous_rows(codes, n, pq_dim, pq_bits));
+  {
+    // bit strings through the bare-buffer calls: the index's own list buffer read from row 37 on,
+    // and rows 5 .. 64 of a scratch buffer written and read back
+    auto ptrs = to_host(index.data_ptrs(), n_lists);
+    auto* d_rows = device_array<uint8_t>(size_t(60) * row_bytes);
+    packer::unpack_contiguous(res, ptrs[label], pq_bits, 37, 20, pq_dim, d_rows);
+    res.sync();
+    REQUIRE(to_host(d_rows, size_t(20) * row_bytes) ==
+            std::vector<uint8_t>(flat.begin() + 37 * row_bytes, flat.begin() + 57 * row_bytes));
+    const uint32_t cpc = 128 / pq_bits, n_chunks = (pq_dim + cpc - 1) / cpc;
+    auto* d_buf = device_array<uint8_t>(size_t(3) * n_chunks * 512);
+    REQUIRE(hipMemset(d_buf, 0, size_t(3) * n_chunks * 512) == hipSuccess);
+    packer::pack_contiguous(res, d_flat, 60, pq_dim, pq_bits, 5, d_buf);
+    packer::unpack_contiguous(res, d_buf, pq_bits, 5, 60, pq_dim, d_rows);
+    res.sync();
+    REQUIRE(to_host(d_rows, size_t(60) * row_bytes) == std::vector<uint8_t>(flat.begin(), flat.begin() + 60 * row_bytes));
+    // and the byte-per-code reading of the same buffer agrees
+    auto* d_back = device_array<uint8_t>(size_t(60) * pq_dim);
+    packer::unpack(res, d_buf, pq_bits, 5, make_device_matrix_view(d_back, 60, pq_dim));
+    res.sync();
+    REQUIRE(to_host(d_back, size_t(60) * pq_dim) == std::vector<uint8_t>(codes.begin(), codes.begin() + 60 * pq_dim));
+    REQUIRE(throws([&] { packer::pack_contiguous(res, d_flat, 4, pq_dim, 3, 0, d_buf); }));
+    REQUIRE(hipFree(d_buf) == hipSuccess && hipFree(d_back) == hipSuccess && hipFree(d_rows) == hipSuccess);
+  }
 
   /* check_packing: erase the list, put the rows back from their codes: the same bytes */
   int64_t* d_ids = to_device(before.ids);

@@ -1029,7 +1029,11 @@ def test_byte_wide_copy_of_narrow_codes_follows_the_lists():
             d2, nb2 = ivf_pq.search(sp, index, queries, 10, resources=tuned)
             d3, nb3 = ivf_pq.search(sp, lean, queries, 10)
             assert torch.equal(nb, nb2) and torch.equal(d, d2), (bits, step, "generic kernel")
-            assert torch.equal(nb, nb3) and torch.equal(d, d3), (bits, step, "no copy")
+            # another index object: rows take their places inside a list in the order the encoding
+            # blocks finish, so two rows at exactly the same distance may swap ranks
+            assert torch.equal(d, d3), (bits, step, "no copy")
+            tied = (d == d.roll(1, dims=1)) | (d == d.roll(-1, dims=1))
+            assert bool(((nb == nb3) | tied).all()), (bits, step, "no copy")
             if step == 0:
                 index = ivf_pq.extend(index, second, ids2)
                 lean = ivf_pq.extend(lean, second, ids2)
