@@ -299,6 +299,8 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
  * lookups as it has entries.  Here the block keeps the first 8 subspaces' codebooks in LDS once,
  * and a lane computes the table entry its row's code selects on the spot: the same subtractions,
  * FMAs and rounding to the table's type, so the partial sums are the ones the table kernels form.
+ * Only the subspaces that every tile looks at (the first FIRST) get a table of the wave's own, and
+ * only for a list long enough to repay it.
  * Nothing is shared between the waves of a block after the codebooks are loaded: each wave walks
  * its own sequence of pairs, with the next pair's record, first codes, bound and query-minus-centre
  * terms in flight while it scans the current one.
@@ -332,6 +334,8 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   auto* book      = reinterpret_cast<LDS_AS vec_t*>(uintptr_t(kScreenLdsBase));
   const float one = opaque_one_s();
   constexpr uint32_t off_pending = kScreenLdsBase + SUB * 256u * PQ_LEN * 4u;
+  constexpr uint32_t off_mini    = off_pending + (kDirectThreads / 64u) * kSurvivorBatchBytes;
+  constexpr uint32_t kMiniTiles  = 6;
 
   const uint32_t tid  = threadIdx.x;
   const uint32_t lane = tid & 63u;
@@ -351,6 +355,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   uint32_t p = blockIdx.x * WPB + wid;
   if (p >= n_pairs) { return; }
   auto* pending = reinterpret_cast<LDS_AS uint32_t*>(uintptr_t(off_pending + wid * kSurvivorBatchBytes));
+  auto* mini    = reinterpret_cast<LDS_AS lut_t*>(uintptr_t(off_mini + wid * uint32_t(FIRST) * 256u * uint32_t(sizeof(lut_t))));
   uint32_t n_pending = 0;
 
   // A record is fetched two pairs ahead with a vector load (index hidden from the uniformity
@@ -425,8 +430,27 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
       bool in_play             = false;
       const uint32_t full_tiles         = n_rows >> 6;
       const unsigned long long tail_rows = (1ull << (n_rows & 63u)) - 1ull;
+      // A list of kMiniTiles tiles or more gets the table of its first FIRST subspaces after all
+      // (the subspaces every tile looks at): 4 * FIRST entries a lane, computed as below, against
+      // FIRST entries a lane and tile.  The wave reads what it wrote itself: LDS serves a wave's
+      // requests in order, no barrier.
+      const bool tabled = n_tiles >= kMiniTiles;
+      if (tabled) {
+#pragma unroll
+        for (uint32_t e = 0; e < uint32_t(FIRST) * 4u; e++) {
+          const vec_t b = book[e * 64u + lane];
+          float score   = 0.0f;
+#pragma unroll
+          for (int t = 0; t < PQ_LEN; t++) {
+            float df = diff[(e >> 2) * PQ_LEN + t];
+            df -= b[t];
+            score = fmaf(df, df, score);
+          }
+          mini[e * 64u + lane] = traits::encode(score);
+        }
+      }
       // sums the leading codes `cur` of the rows of tile `tile`
-      auto sum_tile = [&](const u32x2& cur, uint32_t tile) __attribute__((always_inline)) {
+      auto sum_tile = [&](auto use_table, const u32x2& cur, uint32_t tile) __attribute__((always_inline)) {
         // lanes past the list's end count only in its last, partial tile
         const unsigned long long rows = tile < full_tiles ? ~0ull : tail_rows;
         const uint32_t w[2]           = {cur.x, cur.y};
@@ -435,22 +459,27 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
 #pragma unroll
           for (int kk = first; kk < last; kk++) {
             const uint32_t c = (w[kk >> 2] >> ((kk & 3) * 8)) & 0xffu;
-            const vec_t b    = book[kk * 256 + c];
-            float score      = 0.0f;
+            lut_t v;
+            if (decltype(use_table)::value && kk < FIRST) {
+              v = mini[kk * 256 + c];
+            } else {
+              const vec_t b = book[kk * 256 + c];
+              float score   = 0.0f;
 #pragma unroll
-            for (int t = 0; t < PQ_LEN; t++) {
-              float df;
-              if (kk < 4) {
-                df = diff[(kk & 3) * PQ_LEN + t];
-              } else {
-                int held = __float_as_int(dv0);
-                asm volatile("" : "+v"(held));  // keeps the broadcast inside the rare branch
-                df = __int_as_float(__builtin_amdgcn_readlane(held, kk * PQ_LEN + t));
+              for (int t = 0; t < PQ_LEN; t++) {
+                float df;
+                if (kk < 4) {
+                  df = diff[(kk & 3) * PQ_LEN + t];
+                } else {
+                  int held = __float_as_int(dv0);
+                  asm volatile("" : "+v"(held));  // keeps the broadcast inside the rare branch
+                  df = __int_as_float(__builtin_amdgcn_readlane(held, kk * PQ_LEN + t));
+                }
+                df -= b[t];
+                score = fmaf(df, df, score);
               }
-              df -= b[t];
-              score = fmaf(df, df, score);
+              v = traits::encode(score);
             }
-            const lut_t v = traits::encode(score);
             if (OUT_HALF) {
               acc = acc_t(acc + traits::to_half(v));
             } else if (LUT == LUT_F16) {
@@ -479,17 +508,24 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
       // is unrolled by three so that none is copied while its load is outstanding.  Loads are
       // unconditional (they may run up to three tiles past the list, into the plane's slack or the
       // next lists), so the waits in the loop count outstanding loads instead of draining them.
-      u32x2 r0 = lead0, r1 = next0, r2;
-      for (uint32_t tile = 0; tile < n_tiles; tile += 3u) {
-        r2 = lead_codes(d0, tile + 2u);
-        sum_tile(r0, tile);
-        if (in_play || tile + 1u >= n_tiles) { break; }
-        r0 = lead_codes(d0, tile + 3u);
-        sum_tile(r1, tile + 1u);
-        if (in_play || tile + 2u >= n_tiles) { break; }
-        r1 = lead_codes(d0, tile + 4u);
-        sum_tile(r2, tile + 2u);
-        if (in_play) { break; }
+      auto walk = [&](auto use_table) __attribute__((always_inline)) {
+        u32x2 r0 = lead0, r1 = next0, r2;
+        for (uint32_t tile = 0; tile < n_tiles; tile += 3u) {
+          r2 = lead_codes(d0, tile + 2u);
+          sum_tile(use_table, r0, tile);
+          if (in_play || tile + 1u >= n_tiles) { break; }
+          r0 = lead_codes(d0, tile + 3u);
+          sum_tile(use_table, r1, tile + 1u);
+          if (in_play || tile + 2u >= n_tiles) { break; }
+          r1 = lead_codes(d0, tile + 4u);
+          sum_tile(use_table, r2, tile + 2u);
+          if (in_play) { break; }
+        }
+      };
+      if (tabled) {
+        walk(std::true_type{});
+      } else {
+        walk(std::false_type{});
       }
       if (in_play) { push_survivor(pending, n_pending, lane, d0, survivors, n_survivors, alive); }
     }
@@ -513,7 +549,8 @@ void launch_screen_direct_first(const scan_args& a, const pair_desc* desc, uint3
 {
   auto kernel       = scan_screen_direct_kernel<PQ_LEN, LUT, OUT_HALF, FIRST>;
   const size_t smem = kScreenLdsBase + size_t(kDirectSubs) * 256 * PQ_LEN * 4 +
-                      size_t(kDirectThreads / 64u) * kSurvivorBatchBytes;
+                      size_t(kDirectThreads / 64u) * kSurvivorBatchBytes +
+                      size_t(kDirectThreads / 64u) * FIRST * 256 * sizeof(typename lut_traits<LUT>::storage);
   // persistent blocks: exactly as many as are resident at once (per instance)
   static const int per_cu = prepare_persistent_kernel(kernel, kDirectThreads, smem, smem);
   const int n_cu          = device_cu_count();

@@ -109,14 +109,28 @@ __device__ __forceinline__ uint16_t table_entry(float score)
   ST_SDWA(a4, cb, 0) ST_SDWA(a5, cb, 1) ST_SDWA(a6, cb, 2) ST_SDWA(a7, cb, 3)                      \
   ST_READ(V##0, a0, o, 0) ST_READ(V##1, a1, o, 1) ST_READ(V##2, a2, o, 2) ST_READ(V##3, a3, o, 3)  \
   ST_READ(V##4, a4, o, 4) ST_READ(V##5, a5, o, 5) ST_READ(V##6, a6, o, 6) ST_READ(V##7, a7, o, 7)
+/* the two halves of a group: one code dword each */
+#define ST_ISSUE_LO(o, ca, V)                                                                      \
+  ST_SDWA(a0, ca, 0) ST_SDWA(a1, ca, 1) ST_SDWA(a2, ca, 2) ST_SDWA(a3, ca, 3)                      \
+  ST_READ(V##0, a0, o, 0) ST_READ(V##1, a1, o, 1) ST_READ(V##2, a2, o, 2) ST_READ(V##3, a3, o, 3)
+#define ST_ISSUE_HI(o, cb, V)                                                                      \
+  ST_SDWA(a4, cb, 0) ST_SDWA(a5, cb, 1) ST_SDWA(a6, cb, 2) ST_SDWA(a7, cb, 3)                      \
+  ST_READ(V##4, a4, o, 4) ST_READ(V##5, a5, o, 5) ST_READ(V##6, a6, o, 6) ST_READ(V##7, a7, o, 7)
+#define ST_WAIT4 "s_waitcnt lgkmcnt(4)\n\t"
 #define ST_WAIT8 "s_waitcnt lgkmcnt(8)\n\t"
 #define ST_WAIT0 "s_waitcnt lgkmcnt(0)\n\t"
 /* fp32 sums: entry * scale + sum in one instruction that widens the binary16 entry (exact product) */
 #define ST_ADD_F32_1(v) "v_fma_mix_f32 %[acc], %[" #v "], %[one], %[acc] op_sel_hi:[1,0,0]\n\t"
 #define ST_ADD_F16_1(v) "v_add_f16_e32 %[acc], %[acc], %[" #v "]\n\t"
 #define ST_ADD8(ADD1, V) ADD1(V##0) ADD1(V##1) ADD1(V##2) ADD1(V##3) ADD1(V##4) ADD1(V##5) ADD1(V##6) ADD1(V##7)
+#define ST_ADD4_LO(ADD1, V) ADD1(V##0) ADD1(V##1) ADD1(V##2) ADD1(V##3)
+#define ST_ADD4_HI(ADD1, V) ADD1(V##4) ADD1(V##5) ADD1(V##6) ADD1(V##7)
 #define ST_ADD_F32(V) ST_ADD8(ST_ADD_F32_1, V)
 #define ST_ADD_F16(V) ST_ADD8(ST_ADD_F16_1, V)
+#define ST_ADD_F32_LO(V) ST_ADD4_LO(ST_ADD_F32_1, V)
+#define ST_ADD_F32_HI(V) ST_ADD4_HI(ST_ADD_F32_1, V)
+#define ST_ADD_F16_LO(V) ST_ADD4_LO(ST_ADD_F16_1, V)
+#define ST_ADD_F16_HI(V) ST_ADD4_HI(ST_ADD_F16_1, V)
 /* rows in play whose sum is not past the bound; none: leave */
 #define ST_CHECK_F32                                 \
   "v_cmp_ge_u32_e32 vcc, %[stop], %[acc]\n\t"        \
@@ -128,17 +142,23 @@ __device__ __forceinline__ uint16_t table_entry(float score)
   "s_and_b64 %[tmp], vcc, %[valid]\n\t"              \
   "s_cbranch_scc0 .Ltile_done%=\n\t"
 #define ST_NO_CHECK ""
-#define ST_HEAD "v_mov_b32 %[acc], 0\n\t" ST_ISSUE(0, c0, c1, va) ST_ISSUE(1, c2, c3, vb)
+/* The first chunk starts with half as many lookups in flight and looks at the bound after four
+ * subspaces already: most tiles that cannot win are known by then, and leave with eight lookups
+ * issued. */
+#define ST_FIRST(ADD, CHECK)                                                    \
+  "v_mov_b32 %[acc], 0\n\t" ST_ISSUE_LO(0, c0, va) ST_ISSUE_HI(0, c1, va)       \
+  ST_WAIT4 ADD##_LO(va) CHECK ST_ISSUE(1, c2, c3, vb)                           \
+  ST_WAIT8 ADD##_HI(va) CHECK ST_ISSUE(2, c4, c5, va)                           \
+  ST_WAIT8 ADD(vb) CHECK ST_ISSUE(3, c6, c7, vb)
 /* a chunk that is not the last: its two groups are added, groups o + 2 and o + 3 issued */
 #define ST_CHUNK(o0, o1, o2, o3, c4, c5, c6, c7, ADD, CHECK)  \
   ST_WAIT8 ADD(va) CHECK ST_ISSUE(o2, c4, c5, va)             \
   ST_WAIT8 ADD(vb) CHECK ST_ISSUE(o3, c6, c7, vb)
 #define ST_TAIL(ADD) ST_WAIT8 ADD(va) ST_WAIT0 ADD(vb) ".Ltile_done%=:\n\t" ST_WAIT0
-#define ST_BODY_2(ADD, CHECK) ST_HEAD ST_CHUNK(0, 1, 2, 3, c4, c5, c6, c7, ADD, CHECK) ST_TAIL(ADD)
-#define ST_BODY_3(ADD, CHECK) \
-  ST_HEAD ST_CHUNK(0, 1, 2, 3, c4, c5, c6, c7, ADD, CHECK) ST_CHUNK(2, 3, 4, 5, c8, c9, c10, c11, ADD, CHECK) ST_TAIL(ADD)
-#define ST_BODY_4(ADD, CHECK)                                                                                     \
-  ST_HEAD ST_CHUNK(0, 1, 2, 3, c4, c5, c6, c7, ADD, CHECK) ST_CHUNK(2, 3, 4, 5, c8, c9, c10, c11, ADD, CHECK)     \
+#define ST_BODY_2(ADD, CHECK) ST_FIRST(ADD, CHECK) ST_TAIL(ADD)
+#define ST_BODY_3(ADD, CHECK) ST_FIRST(ADD, CHECK) ST_CHUNK(2, 3, 4, 5, c8, c9, c10, c11, ADD, CHECK) ST_TAIL(ADD)
+#define ST_BODY_4(ADD, CHECK)                                                            \
+  ST_FIRST(ADD, CHECK) ST_CHUNK(2, 3, 4, 5, c8, c9, c10, c11, ADD, CHECK)                \
   ST_CHUNK(4, 5, 6, 7, c12, c13, c14, c15, ADD, CHECK) ST_TAIL(ADD)
 
 #define ST_OUTPUTS                                                                                              \
