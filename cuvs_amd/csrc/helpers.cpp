@@ -320,6 +320,31 @@ void erase_list(cuvs::resources const& res, index<int64_t>* idx, uint32_t label)
   finish_edit(res, ix);
 }
 
+void resize_list(cuvs::resources const& res, index<int64_t>* idx, uint32_t label, uint32_t new_used_size)
+{
+  index_impl& ix      = checked(idx, label);
+  const uint32_t old  = ix.h_list_sizes[label];
+  if (new_used_size == old) { return; }
+  hipStream_t s = res.stream();
+  // the move copies as many rows of each list as the device-side sizes say: min(old, new) of this one
+  if (new_used_size < old) { detail::launch_fill_u32(ix.list_sizes.as<uint32_t>() + label, new_used_size, 1, s); }
+  std::vector<uint32_t> sizes(ix.h_list_sizes);
+  ix.h_list_sizes[label] = std::min(old, new_used_size);
+  sizes[label]           = new_used_size;
+  detail::relayout_lists(res, ix, sizes);
+  // the move copies whole groups of 32 rows: what a smaller size leaves behind in the last group
+  // is cleared, so that slots past a list's end hold zero codes as everywhere else
+  const uint32_t n_pad = round_up_u32(new_used_size, kIndexGroupSize) - new_used_size;
+  if (new_used_size < old && n_pad != 0) {
+    device_buffer zeros(size_t(n_pad) * ix.pq_dim);
+    CUVS_HIP_TRY(hipMemsetAsync(zeros.ptr, 0, zeros.bytes, s));
+    detail::launch_pack_codes(list_codes(ix, label), zeros.as<uint8_t>(), false, n_pad, new_used_size, ix.pq_dim,
+                              ix.pq_bits, s);
+    CUVS_HIP_TRY(hipStreamSynchronize(s));  // `zeros` goes out of scope
+  }
+  finish_edit(res, ix);
+}
+
 void reset_index(cuvs::resources const& res, index<int64_t>* idx)
 {
   CUVS_EXPECTS(idx != nullptr && idx->impl() != nullptr, "index must not be null");

@@ -385,6 +385,13 @@ void extend_list(cuvs::resources const& res,
 
 }  // namespace codepacker
 
+/** ivf_pq.hpp:3362-3366 -- list `label` holds `new_used_size` rows from now on: its first
+ *  min(old, new) rows keep their codes and ids, rows added by a larger size hold zero codes and
+ *  the id of an empty slot until they are written (pack_list_data; extend_list_with_codes does both
+ *  steps).  The reference resizes a list object (`index.lists()[label]`) given its spec and old
+ *  size; the lists of this index share one allocation, so the call names the index and the list. */
+void resize_list(cuvs::resources const& res, index<int64_t>* idx, uint32_t label, uint32_t new_used_size);
+
 /** ivf_pq.hpp:3144 -- list `label` becomes empty. */
 void erase_list(cuvs::resources const& res, index<int64_t>* idx, uint32_t label);
 

@@ -251,6 +251,30 @@ void run(uint32_t pq_bits, ivf_pq::codebook_gen kind, uint32_t pq_dim_asked, con
   }
   packer::pack_list_data(res, &index, make_device_matrix_view<const uint8_t>(d_codes + 10 * pq_dim, 3, pq_dim), label, 10);
   REQUIRE(snapshot(index, label).bytes == before.bytes);
+  // the list resized by hand: 40 more rows (empty slots until written), then the old size again
+  ivf_pq::helpers::resize_list(res, &index, label, n + 40);
+  REQUIRE(index.size() == n_rows + 40 && to_host(index.list_sizes(), n_lists)[label] == n + 40);
+  {
+    const auto grown = snapshot(index, label);
+    REQUIRE(std::equal(before.ids.begin(), before.ids.end(), grown.ids.begin()));
+    for (uint32_t i = n; i < n + 40; i++) { REQUIRE(grown.ids[i] == -1); }
+    packer::unpack_list_data(res, index, make_device_matrix_view(d_codes, n, pq_dim), label, 0);
+    res.sync();
+    REQUIRE(to_host(d_codes, size_t(n) * pq_dim) == codes);
+    // written like any other rows of the list
+    packer::pack_list_data(res, &index, make_device_matrix_view<const uint8_t>(d_codes, 40, pq_dim), label, n);
+    packer::unpack_list_data(res, index, make_device_matrix_view(d_part, 20, pq_dim), label, n + 20);
+    res.sync();
+    REQUIRE(to_host(d_part, size_t(20) * pq_dim) ==
+            std::vector<uint8_t>(codes.begin() + 20 * pq_dim, codes.begin() + 40 * pq_dim));
+  }
+  ivf_pq::helpers::resize_list(res, &index, label, n);
+  REQUIRE(index.size() == n_rows);
+  after = snapshot(index, label);
+  REQUIRE(after.size == n && after.ids == before.ids && after.bytes == before.bytes);
+  again = search_all(res, index, d_data, n_queries, k);
+  REQUIRE(again.ids == before_search.ids && again.dist == before_search.dist);
+  REQUIRE(throws([&] { ivf_pq::helpers::resize_list(res, &index, n_lists, 1); }));
   // the same from bit-contiguous rows, in two parts: the second fits the padding or moves the lists
   ivf_pq::helpers::erase_list(res, &index, label);
   const uint32_t first_part = n - 7;
