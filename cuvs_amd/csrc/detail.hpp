@@ -442,6 +442,9 @@ void launch_merge(const merge_args& a, hipStream_t stream);
 
 /** Exact re-ranking of candidates (refine.hip): ids and distances of the k best candidates of every
  *  query, ascending distance (descending similarity with `ip`). */
+/** Ids between the two widths the refinement's interfaces take. */
+void launch_widen_ids(const uint32_t* in, int64_t* out, uint64_t n, hipStream_t stream);
+void launch_narrow_ids(const int64_t* in, uint32_t* out, uint64_t n, hipStream_t stream);
 void launch_refine(const void* dataset, const void* queries, elem_type type,
                    const int64_t* candidates, int64_t n_rows, uint32_t n_queries, uint32_t dim,
                    uint32_t n_candidates, uint32_t k, bool ip, bool sqrt_out, int64_t* indices,

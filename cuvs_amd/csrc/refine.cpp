@@ -242,6 +242,60 @@ void refine(cuvs::resources const& res,
               indices.extent(1), metric);
 }
 
+namespace {
+template <typename View32, typename ViewOut32>
+void check_u32_views(int64_t n_queries, const View32& cand, const ViewOut32& indices, int64_t dist_rows,
+                     int64_t dist_cols, int64_t q_cols, int64_t d_cols)
+{
+  CUVS_EXPECTS(indices.extent(0) == n_queries && dist_rows == n_queries && cand.extent(0) == n_queries,
+               "Number of rows in output indices, distances and candidates matrices must be equal "
+               "with the number of rows in search matrix.");
+  CUVS_EXPECTS(indices.extent(1) == dist_cols,
+               "Number of columns in output indices and distances matrices must be equal to k");
+  CUVS_EXPECTS(q_cols == d_cols, "Number of columns must be equal for dataset and queries");
+}
+}  // namespace
+
+void refine(cuvs::resources const& res,
+            device_matrix_view<const float> dataset,
+            device_matrix_view<const float> queries,
+            device_matrix_view<const uint32_t> neighbor_candidates,
+            device_matrix_view<uint32_t> indices,
+            device_matrix_view<float> distances,
+            cuvs::distance::DistanceType metric)
+{
+  const int64_t nq = queries.extent(0), nc = neighbor_candidates.extent(1), k = indices.extent(1);
+  check_u32_views(nq, neighbor_candidates, indices, distances.extent(0), distances.extent(1), queries.extent(1),
+                  dataset.extent(1));
+  CUVS_EXPECTS(nq >= 0 && nc >= 0 && k >= 0, "refine: invalid matrix extents");
+  cuvs::device_buffer wide_cand(size_t(nq) * nc * 8 + 8), wide_idx(size_t(nq) * k * 8 + 8);
+  hipStream_t s = res.stream();
+  ivf_pq::detail::launch_widen_ids(neighbor_candidates.data_handle(), wide_cand.as<int64_t>(), uint64_t(nq) * nc, s);
+  refine(res, dataset.data_handle(), queries.data_handle(), ivf_pq::elem_type::f32, dataset.extent(0), nq,
+         dataset.extent(1), wide_cand.as<int64_t>(), nc, wide_idx.as<int64_t>(), distances.data_handle(), k, metric);
+  ivf_pq::detail::launch_narrow_ids(wide_idx.as<int64_t>(), indices.data_handle(), uint64_t(nq) * k, s);
+  CUVS_HIP_TRY(hipStreamSynchronize(s));  // the wide copies go out of scope
+}
+
+void refine(cuvs::resources const& res,
+            host_matrix_view<const float> dataset,
+            host_matrix_view<const float> queries,
+            host_matrix_view<const uint32_t> neighbor_candidates,
+            host_matrix_view<uint32_t> indices,
+            host_matrix_view<float> distances,
+            cuvs::distance::DistanceType metric)
+{
+  const int64_t nq = queries.extent(0), nc = neighbor_candidates.extent(1), k = indices.extent(1);
+  check_u32_views(nq, neighbor_candidates, indices, distances.extent(0), distances.extent(1), queries.extent(1),
+                  dataset.extent(1));
+  CUVS_EXPECTS(nq >= 0 && nc >= 0 && k >= 0, "refine: invalid matrix extents");
+  std::vector<int64_t> wide_cand(size_t(nq) * nc + 1), wide_idx(size_t(nq) * k + 1);
+  for (size_t i = 0; i < size_t(nq) * nc; i++) { wide_cand[i] = int64_t(neighbor_candidates.data_handle()[i]); }
+  refine_host(res, dataset.data_handle(), queries.data_handle(), ivf_pq::elem_type::f32, dataset.extent(0), nq,
+              dataset.extent(1), wide_cand.data(), nc, wide_idx.data(), distances.data_handle(), k, metric);
+  for (size_t i = 0; i < size_t(nq) * k; i++) { indices.data_handle()[i] = uint32_t(wide_idx[i]); }
+}
+
 #define INSTANTIATE_REFINE(T)                                                                  \
   template void refine<T>(cuvs::resources const&, device_matrix_view<const T>,                \
                           device_matrix_view<const T>, device_matrix_view<const int64_t>,     \

@@ -125,6 +125,33 @@ void launch_refine_typed(const void* dataset, const void* queries, const int64_t
 
 }  // namespace
 
+namespace {
+__global__ void widen_ids_kernel(const uint32_t* __restrict__ in, int64_t* __restrict__ out, uint64_t n)
+{
+  const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) { out[i] = int64_t(in[i]); }
+}
+__global__ void narrow_ids_kernel(const int64_t* __restrict__ in, uint32_t* __restrict__ out, uint64_t n)
+{
+  const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) { out[i] = uint32_t(in[i]); }  // the id of an unfilled slot, -1, becomes 0xFFFFFFFF
+}
+}  // namespace
+
+void launch_widen_ids(const uint32_t* in, int64_t* out, uint64_t n, hipStream_t stream)
+{
+  if (n == 0) { return; }
+  widen_ids_kernel<<<uint32_t((n + 255) / 256), 256, 0, stream>>>(in, out, n);
+  CUVS_HIP_TRY(hipGetLastError());
+}
+
+void launch_narrow_ids(const int64_t* in, uint32_t* out, uint64_t n, hipStream_t stream)
+{
+  if (n == 0) { return; }
+  narrow_ids_kernel<<<uint32_t((n + 255) / 256), 256, 0, stream>>>(in, out, n);
+  CUVS_HIP_TRY(hipGetLastError());
+}
+
 void launch_refine(const void* dataset, const void* queries, elem_type type,
                    const int64_t* candidates, int64_t n_rows, uint32_t n_queries, uint32_t dim,
                    uint32_t n_candidates, uint32_t k, bool ip, bool sqrt_out, int64_t* indices,

@@ -38,6 +38,23 @@ void refine(cuvs::resources const& res,
             host_matrix_view<float> distances,
             cuvs::distance::DistanceType metric = cuvs::distance::DistanceType::L2Unexpanded);
 
+/** refine.hpp:107-113 and 332-338: float rows with 32-bit ids, on the device and in host memory
+ *  (an output slot that cannot be filled holds 0xFFFFFFFF). */
+void refine(cuvs::resources const& res,
+            device_matrix_view<const float> dataset,
+            device_matrix_view<const float> queries,
+            device_matrix_view<const uint32_t> neighbor_candidates,
+            device_matrix_view<uint32_t> indices,
+            device_matrix_view<float> distances,
+            cuvs::distance::DistanceType metric = cuvs::distance::DistanceType::L2Unexpanded);
+void refine(cuvs::resources const& res,
+            host_matrix_view<const float> dataset,
+            host_matrix_view<const float> queries,
+            host_matrix_view<const uint32_t> neighbor_candidates,
+            host_matrix_view<uint32_t> indices,
+            host_matrix_view<float> distances,
+            cuvs::distance::DistanceType metric = cuvs::distance::DistanceType::L2Unexpanded);
+
 /** Type-erased entry point behind the C API. */
 void refine(cuvs::resources const& res, const void* dataset, const void* queries,
             ivf_pq::elem_type type, int64_t n_rows, int64_t n_queries, int64_t dim,

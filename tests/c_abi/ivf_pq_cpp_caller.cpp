@@ -106,6 +106,23 @@ int main()
                   cuvs::make_host_matrix_view(h_nb.data(), n_queries, k),
                   cuvs::make_host_matrix_view(h_dist.data(), n_queries, k));
     if (h_nb != nb || h_dist != dist) { std::fprintf(stderr, "host refine differs from device refine\n"); return 1; }
+    // and the overloads with 32-bit ids, on the device and in host memory
+    std::vector<uint32_t> cand32(cand.begin(), cand.end()), h_nb32(n_queries * k);
+    refine(res, cuvs::make_host_matrix_view<const float>(data.data(), n_rows, dim),
+           cuvs::make_host_matrix_view<const float>(data.data(), n_queries, dim),
+           cuvs::make_host_matrix_view<const uint32_t>(cand32.data(), n_queries, k_wide),
+           cuvs::make_host_matrix_view(h_nb32.data(), n_queries, k), cuvs::make_host_matrix_view(h_dist.data(), n_queries, k));
+    uint32_t* d_cand32 = to_device(cand32);
+    auto* d_nb32       = device_array<uint32_t>(n_queries * k);
+    refine(res, cuvs::make_device_matrix_view<const float>(d_data, n_rows, dim), q_view,
+           cuvs::make_device_matrix_view<const uint32_t>(d_cand32, n_queries, k_wide),
+           cuvs::make_device_matrix_view(d_nb32, n_queries, k), cuvs::make_device_matrix_view(d_ref_dist, n_queries, k));
+    res.sync();
+    const auto nb32 = to_host(d_nb32, n_queries * k);
+    for (int64_t i = 0; i < n_queries * k; i++) {
+      if (int64_t(nb32[i]) != nb[i] || int64_t(h_nb32[i]) != nb[i]) { std::fprintf(stderr, "32-bit refine differs at %ld\n", long(i)); return 1; }
+    }
+    if (h_dist != dist || to_host(d_ref_dist, n_queries * k) != dist) { std::fprintf(stderr, "32-bit refine distances differ\n"); return 1; }
   }
 
   // the same rows as two half-indexes under one model: merged answers = the whole index's answers
