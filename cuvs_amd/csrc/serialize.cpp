@@ -177,10 +177,18 @@ void read_array(std::istream& is, const std::string& what, size_t item_size, uin
 
 void serialize(cuvs::resources const& res, const std::string& filename, const index<int64_t>& idx)
 {
-  const auto& ix = *idx.impl();
-  CUVS_EXPECTS(ix.centers.ptr != nullptr, "ivf_pq::serialize: the index holds no model");
   std::ofstream os(filename, std::ios::out | std::ios::binary);
   CUVS_EXPECTS(bool(os), "Cannot open file %s", filename.c_str());
+  serialize(res, os, idx);
+  os.close();
+  CUVS_EXPECTS(bool(os), "Error writing output %s", filename.c_str());
+}
+
+void serialize(cuvs::resources const& res, std::ostream& os, const index<int64_t>& idx)
+{
+  const auto& ix = *idx.impl();
+  CUVS_EXPECTS(ix.centers.ptr != nullptr, "ivf_pq::serialize: the index holds no model");
+  CUVS_EXPECTS(bool(os), "ivf_pq::serialize: the output stream is not writable");
   hipStream_t s = res.stream();
 
   write_scalar<int32_t>(os, "<i4", kSerializationVersion);
@@ -229,8 +237,7 @@ void serialize(cuvs::resources const& res, const std::string& filename, const in
                 codes.data() + (ix.h_row_offsets[l] / kIndexGroupSize) * gb, groups * gb);
     write_array(os, "<i8", {size}, ids.data() + ix.h_row_offsets[l], uint64_t(size) * sizeof(int64_t));
   }
-  os.close();
-  CUVS_EXPECTS(bool(os), "Error writing output %s", filename.c_str());
+  CUVS_EXPECTS(bool(os), "ivf_pq::serialize: error writing to the output stream");
 }
 
 void deserialize(cuvs::resources const& res, const std::string& filename, index<int64_t>* idx)
@@ -238,6 +245,13 @@ void deserialize(cuvs::resources const& res, const std::string& filename, index<
   CUVS_EXPECTS(idx != nullptr, "index must not be null");
   std::ifstream is(filename, std::ios::in | std::ios::binary);
   CUVS_EXPECTS(bool(is), "Cannot open file %s", filename.c_str());
+  deserialize(res, is, idx);
+}
+
+void deserialize(cuvs::resources const& res, std::istream& is, index<int64_t>* idx)
+{
+  CUVS_EXPECTS(idx != nullptr, "index must not be null");
+  CUVS_EXPECTS(bool(is), "ivf_pq::deserialize: the input stream is not readable");
 
   const int ver = read_scalar<int32_t>(is, "version");
   CUVS_EXPECTS(ver == kSerializationVersion, "serialization version mismatch %d vs. %d", ver,

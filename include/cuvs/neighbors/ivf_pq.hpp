@@ -13,6 +13,7 @@
 
 #include <cstdint>
 #include <memory>
+#include <iosfwd>
 #include <string>
 
 // The library is built with hidden visibility; what this header declares is its C++ interface
@@ -254,6 +255,10 @@ void unpack_contiguous_list_data(cuvs::resources const& res,
 
 void serialize(cuvs::resources const& res, const std::string& filename, const index<int64_t>& idx);
 void deserialize(cuvs::resources const& res, const std::string& filename, index<int64_t>* idx);
+/** The same format on a stream (cuVS ivf_pq.hpp:2034-2036, 2084-2086): several indexes, or an index
+ *  and what a caller keeps beside it, can share one file. */
+void serialize(cuvs::resources const& res, std::ostream& os, const index<int64_t>& idx);
+void deserialize(cuvs::resources const& res, std::istream& is, index<int64_t>* idx);
 
 /**
  * Reading and editing single lists of an index (cuVS: namespace ivf_pq::helpers,

@@ -16,6 +16,7 @@
 
 #include <cstdio>
 #include <random>
+#include <sstream>
 #include <vector>
 
 namespace {
@@ -169,6 +170,29 @@ int main()
     // ids may swap only between equal distances
     const bool tie = (i % k > 0 && whole_d[i] == whole_d[i - 1]) || (i % k < k - 1 && whole_d[i] == whole_d[i + 1]);
     if (merged_nb[i] != whole_nb[i] && !tie) { std::fprintf(stderr, "merged ids differ at %ld\n", long(i)); return 1; }
+  }
+
+  // the two halves written to one stream and read back from it: each answers as before
+  {
+    std::stringstream both(std::ios::in | std::ios::out | std::ios::binary);
+    ivf_pq::serialize(res, both, lo);
+    ivf_pq::serialize(res, both, hi);
+    ivf_pq::index<int64_t> lo2, hi2;
+    ivf_pq::deserialize(res, both, &lo2);
+    ivf_pq::deserialize(res, both, &hi2);
+    if (lo2.size() != lo.size() || hi2.size() != hi.size()) { std::fprintf(stderr, "sizes after the stream differ\n"); return 1; }
+    auto* d_nb2   = device_array<int64_t>(2 * n_queries * k);
+    auto* d_dist2 = device_array<float>(2 * n_queries * k);
+    ivf_pq::search<float>(res, sp, lo2, q_view, cuvs::make_device_matrix_view(d_nb2, n_queries, k),
+                          cuvs::make_device_matrix_view(d_dist2, n_queries, k));
+    ivf_pq::search<float>(res, sp, hi2, q_view, cuvs::make_device_matrix_view(d_nb2 + n_queries * k, n_queries, k),
+                          cuvs::make_device_matrix_view(d_dist2 + n_queries * k, n_queries, k));
+    res.sync();
+    if (to_host(d_nb2, 2 * n_queries * k) != to_host(d_parts_nb, 2 * n_queries * k) ||
+        to_host(d_dist2, 2 * n_queries * k) != to_host(d_parts_dist, 2 * n_queries * k)) {
+      std::fprintf(stderr, "indexes read back from a stream answer differently\n");
+      return 1;
+    }
   }
 
   // an invalid call throws cuvs::logic_error with a message
