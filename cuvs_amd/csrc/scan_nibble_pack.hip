@@ -63,76 +63,120 @@ static_assert(kPackCandBase + kPackMaxPairs * kPackWaveCap * 8u <= kPackTableBas
   NP_RD(V##a0, aa0, j, 0) NP_RD(V##a1, aa1, j, 1) NP_RD(V##a2, aa2, j, 2) NP_RD(V##a3, aa3, j, 3)          \
   NP_RD(V##b0, ab0, j, 0) NP_RD(V##b1, ab1, j, 1) NP_RD(V##b2, ab2, j, 2) NP_RD(V##b3, ab3, j, 3)
 /* the two rows' sums are separate chains of adds: one proceeds while the other's result is on its way */
-#define NP_ADD4(V)                                      \
-  "v_add_f16_e32 %[accA], %[accA], %[" #V "a0]\n\t"     \
-  "v_add_f16_e32 %[accB], %[accB], %[" #V "b0]\n\t"     \
-  "v_add_f16_e32 %[accA], %[accA], %[" #V "a1]\n\t"     \
-  "v_add_f16_e32 %[accB], %[accB], %[" #V "b1]\n\t"     \
-  "v_add_f16_e32 %[accA], %[accA], %[" #V "a2]\n\t"     \
-  "v_add_f16_e32 %[accB], %[accB], %[" #V "b2]\n\t"     \
-  "v_add_f16_e32 %[accA], %[accA], %[" #V "a3]\n\t"     \
-  "v_add_f16_e32 %[accB], %[accB], %[" #V "b3]\n\t"
+#define NP_ADD_H(acc, v) "v_add_f16_e32 %[" #acc "], %[" #acc "], %[" #v "]\n\t"
+/* fp32 sums: the binary16 entry is widened inside a multiply-add by its factor (an exact product) */
+#define NP_ADD_F(acc, v) "v_fma_mix_f32 %[" #acc "], %[" #v "], %[one], %[" #acc "] op_sel_hi:[1,0,0]\n\t"
+#define NP_ADD4(ADD1, V)                                                              \
+  ADD1(accA, V##a0) ADD1(accB, V##b0) ADD1(accA, V##a1) ADD1(accB, V##b1)             \
+  ADD1(accA, V##a2) ADD1(accB, V##b2) ADD1(accA, V##a3) ADD1(accB, V##b3)
+/* L2 sums only grow: when no row in play of either half is at or below the bound any more, the
+ * step ends (the reads on their way are awaited and dropped).  Sums as the bits of a float. */
+#define NP_CHECK_F                                     \
+  "v_cmp_ge_u32_e32 vcc, %[stop], %[accA]\n\t"         \
+  "s_and_b64 %[tmpA], vcc, %[validA]\n\t"              \
+  "v_cmp_ge_u32_e32 vcc, %[stop], %[accB]\n\t"         \
+  "s_and_b64 %[tmpB], vcc, %[validB]\n\t"              \
+  "s_or_b64 %[tmpA], %[tmpA], %[tmpB]\n\t"             \
+  "s_cbranch_scc0 .Lstep_done%=\n\t"
+#define NP_CHECK_H                                     \
+  "v_cvt_f32_f16_e32 %[chkA], %[accA]\n\t"             \
+  "v_cvt_f32_f16_e32 %[chkB], %[accB]\n\t"             \
+  "v_cmp_ge_u32_e32 vcc, %[stop], %[chkA]\n\t"         \
+  "s_and_b64 %[tmpA], vcc, %[validA]\n\t"              \
+  "v_cmp_ge_u32_e32 vcc, %[stop], %[chkB]\n\t"         \
+  "s_and_b64 %[tmpB], vcc, %[validB]\n\t"              \
+  "s_or_b64 %[tmpA], %[tmpA], %[tmpB]\n\t"             \
+  "s_cbranch_scc0 .Lstep_done%=\n\t"
+#define NP_NO_CHECK ""
 #define NP_W15 "s_waitcnt lgkmcnt(15)\n\t"  /* of 24 reads in flight: the oldest group of eight has landed */
 #define NP_W8 "s_waitcnt lgkmcnt(8)\n\t"
 #define NP_W0 "s_waitcnt lgkmcnt(0)\n\t"
 /* The sixteen groups of a step: three are in flight (sets x, y, z in turn) while the oldest is added;
  * the masked copies of code word d are made before its first group (2 d) is issued. */
-#define NP_BODY \
+#define NP_BODY(A, CHECK) \
   NP_MASKS(ca0, cb0) NP_ISSUE(0, x, 0, 1) NP_ISSUE(1, y, 2, 3) NP_MASKS(ca1, cb1) NP_ISSUE(2, z, 0, 1) \
-  NP_W15 NP_ADD4(x) NP_ISSUE(3, x, 2, 3) \
-  NP_W15 NP_ADD4(y) NP_MASKS(ca2, cb2) NP_ISSUE(4, y, 0, 1) \
-  NP_W15 NP_ADD4(z) NP_ISSUE(5, z, 2, 3) \
-  NP_W15 NP_ADD4(x) NP_MASKS(ca3, cb3) NP_ISSUE(6, x, 0, 1) \
-  NP_W15 NP_ADD4(y) NP_ISSUE(7, y, 2, 3) \
-  NP_W15 NP_ADD4(z) NP_MASKS(ca4, cb4) NP_ISSUE(8, z, 0, 1) \
-  NP_W15 NP_ADD4(x) NP_ISSUE(9, x, 2, 3) \
-  NP_W15 NP_ADD4(y) NP_MASKS(ca5, cb5) NP_ISSUE(10, y, 0, 1) \
-  NP_W15 NP_ADD4(z) NP_ISSUE(11, z, 2, 3) \
-  NP_W15 NP_ADD4(x) NP_MASKS(ca6, cb6) NP_ISSUE(12, x, 0, 1) \
-  NP_W15 NP_ADD4(y) NP_ISSUE(13, y, 2, 3) \
-  NP_W15 NP_ADD4(z) NP_MASKS(ca7, cb7) NP_ISSUE(14, z, 0, 1) \
-  NP_W15 NP_ADD4(x) NP_ISSUE(15, x, 2, 3) \
-  NP_W15 NP_ADD4(y) \
-  NP_W8 NP_ADD4(z) \
-  NP_W0 NP_ADD4(x)
+  NP_W15 NP_ADD4(A, x) NP_ISSUE(3, x, 2, 3) \
+  NP_W15 NP_ADD4(A, y) CHECK NP_MASKS(ca2, cb2) NP_ISSUE(4, y, 0, 1) \
+  NP_W15 NP_ADD4(A, z) NP_ISSUE(5, z, 2, 3) \
+  NP_W15 NP_ADD4(A, x) CHECK NP_MASKS(ca3, cb3) NP_ISSUE(6, x, 0, 1) \
+  NP_W15 NP_ADD4(A, y) NP_ISSUE(7, y, 2, 3) \
+  NP_W15 NP_ADD4(A, z) NP_MASKS(ca4, cb4) NP_ISSUE(8, z, 0, 1) \
+  NP_W15 NP_ADD4(A, x) NP_ISSUE(9, x, 2, 3) \
+  NP_W15 NP_ADD4(A, y) CHECK NP_MASKS(ca5, cb5) NP_ISSUE(10, y, 0, 1) \
+  NP_W15 NP_ADD4(A, z) NP_ISSUE(11, z, 2, 3) \
+  NP_W15 NP_ADD4(A, x) NP_MASKS(ca6, cb6) NP_ISSUE(12, x, 0, 1) \
+  NP_W15 NP_ADD4(A, y) NP_ISSUE(13, y, 2, 3) \
+  NP_W15 NP_ADD4(A, z) CHECK NP_MASKS(ca7, cb7) NP_ISSUE(14, z, 0, 1) \
+  NP_W15 NP_ADD4(A, x) NP_ISSUE(15, x, 2, 3) \
+  NP_W15 NP_ADD4(A, y) \
+  NP_W8 NP_ADD4(A, z) \
+  NP_W0 NP_ADD4(A, x) \
+  ".Lstep_done%=:\n\t" NP_W0
 
-/** acc_a, acc_b (binary16 sums of rows A and B, in the low halves) plus the entries that the codes
- *  of one step select, in subspace order.  a / b: the step's two chunks of rows A and B; aa / ab:
- *  address registers holding the address of the step's part of the table in their upper three
- *  bytes (the routine writes their lowest bytes only). */
+#define NP_OUTPUTS                                                                                              \
+  [accA] "+v"(acc_a), [accB] "+v"(acc_b), [aa0] "+v"(aa[0]), [aa1] "+v"(aa[1]), [aa2] "+v"(aa[2]),             \
+    [aa3] "+v"(aa[3]), [ab0] "+v"(ab[0]), [ab1] "+v"(ab[1]), [ab2] "+v"(ab[2]), [ab3] "+v"(ab[3]),             \
+    [xa0] "=&v"(xa[0]), [xa1] "=&v"(xa[1]), [xa2] "=&v"(xa[2]), [xa3] "=&v"(xa[3]), [xb0] "=&v"(xb[0]),        \
+    [xb1] "=&v"(xb[1]), [xb2] "=&v"(xb[2]), [xb3] "=&v"(xb[3]), [ya0] "=&v"(ya[0]), [ya1] "=&v"(ya[1]),        \
+    [ya2] "=&v"(ya[2]), [ya3] "=&v"(ya[3]), [yb0] "=&v"(yb[0]), [yb1] "=&v"(yb[1]), [yb2] "=&v"(yb[2]),        \
+    [yb3] "=&v"(yb[3]), [za0] "=&v"(za[0]), [za1] "=&v"(za[1]), [za2] "=&v"(za[2]), [za3] "=&v"(za[3]),        \
+    [zb0] "=&v"(zb[0]), [zb1] "=&v"(zb[1]), [zb2] "=&v"(zb[2]), [zb3] "=&v"(zb[3]), [evA] "=&v"(evA),          \
+    [odA] "=&v"(odA), [evB] "=&v"(evB), [odB] "=&v"(odB), [chkA] "=&v"(chkA), [chkB] "=&v"(chkB),              \
+    [tmpA] "=&s"(tmpA), [tmpB] "=&s"(tmpB)
+#define NP_INPUTS                                                                                               \
+  [one_u] "v"(one_u), [one] "v"(one), [stop] "s"(stop), [validA] "s"(valid_a), [validB] "s"(valid_b),          \
+    [ca0] "v"(a[0].x), [ca1] "v"(a[0].y), [ca2] "v"(a[0].z), [ca3] "v"(a[0].w), [ca4] "v"(a[1].x),             \
+    [ca5] "v"(a[1].y), [ca6] "v"(a[1].z), [ca7] "v"(a[1].w), [cb0] "v"(b[0].x), [cb1] "v"(b[0].y),             \
+    [cb2] "v"(b[0].z), [cb3] "v"(b[0].w), [cb4] "v"(b[1].x), [cb5] "v"(b[1].y), [cb6] "v"(b[1].z),             \
+    [cb7] "v"(b[1].w)
+
+/** acc_a, acc_b (sums of rows A and B: binary16 numbers in the low halves, or the bits of floats)
+ *  plus the entries that the codes of one step select, in subspace order.  a / b: the step's two
+ *  chunks of rows A and B; aa / ab: address registers holding the address of the step's part of
+ *  the table in their upper three bytes (the routine writes their lowest bytes only).  CHECK: the
+ *  step ends after 8, 16, 32 or 48 subspaces when no row of valid_a / valid_b has a sum whose bits
+ *  (as a float's) are at most `stop`. */
+template <bool HALF, bool CHECK>
 __device__ __forceinline__ void nibble_pack_step(uint32_t& acc_a, uint32_t& acc_b, const u32x4 (&a)[2],
                                                  const u32x4 (&b)[2], uint32_t (&aa)[4], uint32_t (&ab)[4],
-                                                 uint32_t one_u)
+                                                 uint32_t one_u, float one, uint32_t stop,
+                                                 unsigned long long valid_a, unsigned long long valid_b)
 {
-  uint32_t xa[4], xb[4], ya[4], yb[4], za[4], zb[4], evA, odA, evB, odB;
-  asm volatile(NP_BODY
-               : [accA] "+v"(acc_a), [accB] "+v"(acc_b), [aa0] "+v"(aa[0]), [aa1] "+v"(aa[1]), [aa2] "+v"(aa[2]),
-                 [aa3] "+v"(aa[3]), [ab0] "+v"(ab[0]), [ab1] "+v"(ab[1]), [ab2] "+v"(ab[2]), [ab3] "+v"(ab[3]),
-                 [xa0] "=&v"(xa[0]), [xa1] "=&v"(xa[1]), [xa2] "=&v"(xa[2]), [xa3] "=&v"(xa[3]), [xb0] "=&v"(xb[0]),
-                 [xb1] "=&v"(xb[1]), [xb2] "=&v"(xb[2]), [xb3] "=&v"(xb[3]), [ya0] "=&v"(ya[0]), [ya1] "=&v"(ya[1]),
-                 [ya2] "=&v"(ya[2]), [ya3] "=&v"(ya[3]), [yb0] "=&v"(yb[0]), [yb1] "=&v"(yb[1]), [yb2] "=&v"(yb[2]),
-                 [yb3] "=&v"(yb[3]), [za0] "=&v"(za[0]), [za1] "=&v"(za[1]), [za2] "=&v"(za[2]), [za3] "=&v"(za[3]),
-                 [zb0] "=&v"(zb[0]), [zb1] "=&v"(zb[1]), [zb2] "=&v"(zb[2]), [zb3] "=&v"(zb[3]), [evA] "=&v"(evA), [odA] "=&v"(odA), [evB] "=&v"(evB), [odB] "=&v"(odB)
-               : [one_u] "v"(one_u), [ca0] "v"(a[0].x), [ca1] "v"(a[0].y), [ca2] "v"(a[0].z), [ca3] "v"(a[0].w),
-                 [ca4] "v"(a[1].x), [ca5] "v"(a[1].y), [ca6] "v"(a[1].z), [ca7] "v"(a[1].w), [cb0] "v"(b[0].x),
-                 [cb1] "v"(b[0].y), [cb2] "v"(b[0].z), [cb3] "v"(b[0].w), [cb4] "v"(b[1].x), [cb5] "v"(b[1].y),
-                 [cb6] "v"(b[1].z), [cb7] "v"(b[1].w)
-               : "memory");
+  uint32_t xa[4], xb[4], ya[4], yb[4], za[4], zb[4], evA, odA, evB, odB, chkA, chkB;
+  unsigned long long tmpA, tmpB;
+#define NP_EMIT(ADD1, CHK)                                                                                      \
+  asm volatile(NP_BODY(ADD1, CHK)                                                                               \
+               : NP_OUTPUTS                                                                                     \
+               : NP_INPUTS                                                                                      \
+               : "vcc", "scc", "memory")
+  if constexpr (HALF && CHECK) {
+    NP_EMIT(NP_ADD_H, NP_CHECK_H);
+  } else if constexpr (HALF) {
+    NP_EMIT(NP_ADD_H, NP_NO_CHECK);
+  } else if constexpr (CHECK) {
+    NP_EMIT(NP_ADD_F, NP_CHECK_F);
+  } else {
+    NP_EMIT(NP_ADD_F, NP_NO_CHECK);
+  }
+#undef NP_EMIT
 }
 
-/** decode(encode(score)) as binary16, for the table type chosen at run time. */
-template <bool IP>
+/** decode(encode(score)) as binary16, for the table type chosen at run time.  For fp32 sums an
+ *  8-bit entry is decoded as a float, whose top binade binary16 does not reach: the table holds
+ *  half of it (exact: a power of two) and the add multiplies by two. */
+template <bool IP, bool HALF>
 __device__ __forceinline__ _Float16 pack_entry(float score, int lut_dtype)
 {
   if (lut_dtype == CUDA_R_8U) {
     using traits = lut_traits<IP ? LUT_FP8S : LUT_FP8U>;
+    if constexpr (!HALF) { return _Float16(traits::to_float(traits::encode(score)) * 0.5f); }
     return traits::to_half(traits::encode(score));
   }
   using traits = lut_traits<LUT_F16>;
   return traits::to_half(traits::encode(score));
 }
 
-template <bool IP, int PQ_LEN, int NOWN>  // NOWN = pq_dim / 64: subspaces a builder thread owns
+template <bool IP, int PQ_LEN, int NOWN, bool HALF>  // NOWN = pq_dim / 64: subspaces a builder thread owns
 __global__ __launch_bounds__(kPackThreads) void scan_nibble_pack_kernel(scan_args a, uint32_t pairs_per_it)
 {
   const uint32_t tid  = threadIdx.x;
@@ -150,7 +194,7 @@ __global__ __launch_bounds__(kPackThreads) void scan_nibble_pack_kernel(scan_arg
 
   const uint32_t rot         = a.rot_dim;
   const uint32_t nch         = a.pq_dim >> 5;  // 16-byte chunks per row
-  const uint32_t n_steps     = nch >> 1;       // even (pq_dim is a multiple of 128)
+  const uint32_t n_steps     = nch >> 1;       // steps of 64 subspaces (an even number for inner products)
   const uint32_t table_bytes = a.pq_dim * 32u;
 
   /* ---- builder state: entry e of subspaces sg, sg + 64, ... ---- */
@@ -171,6 +215,12 @@ __global__ __launch_bounds__(kPackThreads) void scan_nibble_pack_kernel(scan_arg
   auto* my_cand = reinterpret_cast<LDS_AS unsigned long long*>(uintptr_t(kPackCandBase)) + wid * kPackWaveCap;
   uint32_t one_u = 1u;
   asm volatile("" : "+v"(one_u));
+  float one = a.lut_dtype == CUDA_R_8U ? 2.0f : 1.0f;  // factor of the entries (fp32 sums)
+  asm volatile("" : "+v"(one));
+  // a sum as a float: the binary16 number in the low half, or the register's bits
+  auto sum_of = [](uint32_t acc) {
+    return HALF ? float(__builtin_bit_cast(_Float16, uint16_t(acc))) : __uint_as_float(acc);
+  };
 
   for (uint32_t it = 0; it < n_it; it++) {
     const uint32_t first = (lb + it * grid) * G;  // first pair of the iteration
@@ -236,7 +286,7 @@ __global__ __launch_bounds__(kPackThreads) void scan_nibble_pack_kernel(scan_arg
               score = fmaf(-qd, pqc, score);
             }
           }
-          mine[i * 64 * 16] = pack_entry<IP>(score, a.lut_dtype);
+          mine[i * 64 * 16] = pack_entry<IP, HALF>(score, a.lut_dtype);
         }
       }
     }
@@ -302,83 +352,121 @@ __global__ __launch_bounds__(kPackThreads) void scan_nibble_pack_kernel(scan_arg
         u32x4 cur_a[2], cur_b[2], nxt_a[2], nxt_b[2];
         load_step(lane < n_rows ? lane : 0u, 0u, cur_a);
         load_step(lane + 64u < n_rows ? lane + 64u : 0u, 0u, cur_b);
-        for (uint32_t tile = 0; tile < n_tiles; tile++) {
-          const uint32_t row_a = tile * 128u + lane;
-          const uint32_t row_b = row_a + 64u;
-          const bool valid_a   = in_play(row_a);
-          const bool valid_b   = in_play(row_b);
-#pragma unroll
-          for (int i = 0; i < 4; i++) {
-            aa[i] = table;
-            ab[i] = table;
-            asm volatile("" : "+v"(aa[i]), "+v"(ab[i]));
-          }
-          uint32_t acc_a = 0, acc_b = 0;  // binary16 zeros
-          bool stopped = false;
-          // L2 sums only grow: rows past the bound after a step stay past it (compute_score's early stop)
-          auto all_past = [&]() {
-            if constexpr (IP) {
-              return false;
-            } else {
-              const float sa_ = float(__builtin_bit_cast(_Float16, uint16_t(acc_a)));
-              const float sb_ = float(__builtin_bit_cast(_Float16, uint16_t(acc_b)));
-              return __builtin_amdgcn_ballot_w64((valid_a && !(sa_ > thr_f)) || (valid_b && !(sb_ > thr_f))) == 0ull;
-            }
-          };
-          for (uint32_t step = 0; step < n_steps; step += 2) {
-            // the step after this one: of the same rows, or the first of the next tile's (past the
-            // end: row 0 again); requested without a condition
+        if constexpr (!IP) {
+          // L2: most tiles end inside their first step (no row can still win), so what is worth having
+          // on its way is the next tile's first step, not this tile's next one.  The two buffers
+          // swap roles from tile to tile; a tile whose rows stay in play fetches its later steps
+          // when it gets there.
+          auto l2_tile = [&](uint32_t tile, u32x4 (&pa)[2], u32x4 (&pb)[2], u32x4 (&qa)[2], u32x4 (&qb)[2]) {
+            const uint32_t row_a = tile * 128u + lane;
+            const uint32_t row_b = row_a + 64u;
+            const bool valid_a   = in_play(row_a);
+            const bool valid_b   = in_play(row_b);
             {
-              const uint32_t ra = row_a < n_rows ? row_a : 0u;
-              const uint32_t rb = row_b < n_rows ? row_b : 0u;
-              load_step(ra, step + 1u, nxt_a);
-              load_step(rb, step + 1u, nxt_b);
-            }
-            nibble_pack_step(acc_a, acc_b, cur_a, cur_b, aa, ab, one_u);
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-              aa[i] += kPackStepBytes;
-              ab[i] += kPackStepBytes;
-            }
-            if (all_past()) {
-              stopped = true;
-              break;
-            }
-            {
-              const bool more   = step + 2u < n_steps;
-              const uint32_t na = more ? row_a : row_a + 128u;
-              const uint32_t nb = more ? row_b : row_b + 128u;
-              load_step(na < n_rows ? na : 0u, more ? step + 2u : 0u, cur_a);
-              load_step(nb < n_rows ? nb : 0u, more ? step + 2u : 0u, cur_b);
-            }
-            nibble_pack_step(acc_a, acc_b, nxt_a, nxt_b, aa, ab, one_u);
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-              aa[i] += kPackStepBytes;
-              ab[i] += kPackStepBytes;
-            }
-            if (step + 2u < n_steps && all_past()) {
-              stopped = true;
-              break;
-            }
-          }
-          if (stopped) {
-            // the codes on their way are of this tile: the next tile's first step is fetched afresh
-            if (tile + 1u < n_tiles) {
+              // requested without a condition (past the end: row 0 again)
               const uint32_t na = row_a + 128u, nb = row_b + 128u;
-              load_step(na < n_rows ? na : 0u, 0u, cur_a);
-              load_step(nb < n_rows ? nb : 0u, 0u, cur_b);
+              load_step(na < n_rows ? na : 0u, 0u, qa);
+              load_step(nb < n_rows ? nb : 0u, 0u, qb);
             }
-            continue;  // every row in play is past the bound
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+              aa[i] = table;
+              ab[i] = table;
+              asm volatile("" : "+v"(aa[i]), "+v"(ab[i]));
+            }
+            uint32_t acc_a = 0, acc_b = 0;  // zeros of either type
+            // inside a step the bound is compared as bits (sums are not negative: past the bound =
+            // past its bits); between steps as numbers
+            const uint32_t stop_bits        = thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u;
+            const unsigned long long mask_a = __builtin_amdgcn_ballot_w64(valid_a);
+            const unsigned long long mask_b = __builtin_amdgcn_ballot_w64(valid_b);
+            auto all_past = [&]() {
+              return __builtin_amdgcn_ballot_w64((valid_a && !(sum_of(acc_a) > thr_f)) ||
+                                                 (valid_b && !(sum_of(acc_b) > thr_f))) == 0ull;
+            };
+            nibble_pack_step<HALF, true>(acc_a, acc_b, pa, pb, aa, ab, one_u, one, stop_bits, mask_a, mask_b);
+            bool stopped = all_past();
+            for (uint32_t step = 1; step < n_steps && !stopped; step++) {
+              load_step(row_a < n_rows ? row_a : 0u, step, pa);
+              load_step(row_b < n_rows ? row_b : 0u, step, pb);
+#pragma unroll
+              for (int i = 0; i < 4; i++) {
+                aa[i] += kPackStepBytes;
+                ab[i] += kPackStepBytes;
+              }
+              nibble_pack_step<HALF, true>(acc_a, acc_b, pa, pb, aa, ab, one_u, one, stop_bits, mask_a, mask_b);
+              stopped = step + 1u < n_steps && all_past();
+            }
+            if (stopped) { return; }  // every row in play is past the bound
+            take(sum_of(acc_a), valid_a, row_a);
+            take(sum_of(acc_b), valid_b, row_b);
+          };
+          for (uint32_t tile = 0; tile < n_tiles; tile += 2u) {
+            l2_tile(tile, cur_a, cur_b, nxt_a, nxt_b);
+            if (tile + 1u < n_tiles) { l2_tile(tile + 1u, nxt_a, nxt_b, cur_a, cur_b); }
           }
-          _Float16 ha = __builtin_bit_cast(_Float16, uint16_t(acc_a));
-          _Float16 hb = __builtin_bit_cast(_Float16, uint16_t(acc_b));
-          if (cosine) {
-            ha = _Float16(ha + _Float16(1));
-            hb = _Float16(hb + _Float16(1));
+        } else {
+          for (uint32_t tile = 0; tile < n_tiles; tile++) {
+            const uint32_t row_a = tile * 128u + lane;
+            const uint32_t row_b = row_a + 64u;
+            const bool valid_a   = in_play(row_a);
+            const bool valid_b   = in_play(row_b);
+  #pragma unroll
+            for (int i = 0; i < 4; i++) {
+              aa[i] = table;
+              ab[i] = table;
+              asm volatile("" : "+v"(aa[i]), "+v"(ab[i]));
+            }
+            uint32_t acc_a = 0, acc_b = 0;  // zeros of either type
+            for (uint32_t step = 0; step < n_steps; step += 2) {
+              // the step after this one: of the same rows, or the first of the next tile's (past the
+              // end: row 0 again); requested without a condition
+              {
+                const uint32_t ra = row_a < n_rows ? row_a : 0u;
+                const uint32_t rb = row_b < n_rows ? row_b : 0u;
+                load_step(ra, step + 1u, nxt_a);
+                load_step(rb, step + 1u, nxt_b);
+              }
+              nibble_pack_step<HALF, false>(acc_a, acc_b, cur_a, cur_b, aa, ab, one_u, one, 0u, 0ull, 0ull);
+  #pragma unroll
+              for (int i = 0; i < 4; i++) {
+                aa[i] += kPackStepBytes;
+                ab[i] += kPackStepBytes;
+              }
+              {
+                const bool more   = step + 2u < n_steps;
+                const uint32_t na = more ? row_a : row_a + 128u;
+                const uint32_t nb = more ? row_b : row_b + 128u;
+                load_step(na < n_rows ? na : 0u, more ? step + 2u : 0u, cur_a);
+                load_step(nb < n_rows ? nb : 0u, more ? step + 2u : 0u, cur_b);
+              }
+              nibble_pack_step<HALF, false>(acc_a, acc_b, nxt_a, nxt_b, aa, ab, one_u, one, 0u, 0ull, 0ull);
+  #pragma unroll
+              for (int i = 0; i < 4; i++) {
+                aa[i] += kPackStepBytes;
+                ab[i] += kPackStepBytes;
+              }
+            }
+            if constexpr (HALF) {
+              _Float16 ha = __builtin_bit_cast(_Float16, uint16_t(acc_a));
+              _Float16 hb = __builtin_bit_cast(_Float16, uint16_t(acc_b));
+              if (cosine) {
+                ha = _Float16(ha + _Float16(1));
+                hb = _Float16(hb + _Float16(1));
+              }
+              take(float(ha), valid_a, row_a);
+              take(float(hb), valid_b, row_b);
+            } else {
+              float fa = __uint_as_float(acc_a);
+              float fb = __uint_as_float(acc_b);
+              if (cosine) {
+                fa += 1.0f;
+                fb += 1.0f;
+              }
+              take(fa, valid_a, row_a);
+              take(fb, valid_b, row_b);
+            }
           }
-          take(float(ha), valid_a, row_a);
-          take(float(hb), valid_b, row_b);
         }
         if (wcount >= a.k) {
           const uint32_t kth = wcount <= 64u ? wave_select_keys<1>(my_cand, lane, wcount, a.k)
@@ -399,10 +487,10 @@ uint32_t pack_pairs_per_iteration(const scan_args& a)
   return fit < kPackMaxPairs ? fit : kPackMaxPairs;
 }
 
-template <bool IP, int PQ_LEN, int NOWN>
-void launch_pack_instance(const scan_args& a, hipStream_t stream)
+template <bool IP, int PQ_LEN, int NOWN, bool HALF>
+void launch_pack_sums(const scan_args& a, hipStream_t stream)
 {
-  auto kernel = scan_nibble_pack_kernel<IP, PQ_LEN, NOWN>;
+  auto kernel = scan_nibble_pack_kernel<IP, PQ_LEN, NOWN, HALF>;
   // per instance: the whole LDS of a CU belongs to the one resident block
   static const int attr_set = [&] {
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -421,6 +509,16 @@ void launch_pack_instance(const scan_args& a, hipStream_t stream)
   CUVS_HIP_TRY(hipGetLastError());
 }
 
+template <bool IP, int PQ_LEN, int NOWN>
+void launch_pack_instance(const scan_args& a, hipStream_t stream)
+{
+  if (a.out_half) {
+    launch_pack_sums<IP, PQ_LEN, NOWN, true>(a, stream);
+  } else {
+    launch_pack_sums<IP, PQ_LEN, NOWN, false>(a, stream);
+  }
+}
+
 template <bool IP, int PQ_LEN>
 void launch_pack_width(const scan_args& a, hipStream_t stream)
 {
@@ -429,7 +527,18 @@ void launch_pack_width(const scan_args& a, hipStream_t stream)
     case 4: launch_pack_instance<IP, PQ_LEN, 4>(a, stream); break;
     case 6: launch_pack_instance<IP, PQ_LEN, 6>(a, stream); break;
     case 8: launch_pack_instance<IP, PQ_LEN, 8>(a, stream); break;
-    default: break;
+    default:
+      // an odd number of steps: the L2 tile loop takes them one by one
+      if constexpr (!IP) {
+        switch (a.pq_dim >> 6) {
+          case 1: launch_pack_instance<IP, PQ_LEN, 1>(a, stream); break;
+          case 3: launch_pack_instance<IP, PQ_LEN, 3>(a, stream); break;
+          case 5: launch_pack_instance<IP, PQ_LEN, 5>(a, stream); break;
+          case 7: launch_pack_instance<IP, PQ_LEN, 7>(a, stream); break;
+          default: break;
+        }
+      }
+      break;
   }
 }
 
@@ -445,8 +554,10 @@ void launch_pack_len(const scan_args& a, hipStream_t stream)
 
 bool scan_nibble_pack_supported(const scan_args& a)
 {
-  if (!a.fused || a.pq_bits != 4 || !a.out_half || a.k > kPackMaxK) { return false; }
-  if (a.pq_dim % 128u != 0 || a.pq_dim > 512u || a.rot_dim != a.pq_dim * a.pq_len) { return false; }
+  if (!a.fused || a.pq_bits != 4 || a.k > kPackMaxK) { return false; }
+  const bool ip = a.metric == int(DistanceType::InnerProduct) || a.metric == int(DistanceType::CosineExpanded);
+  // steps of 64 subspaces: in pairs for inner products (one step's codes arrive while the other's are summed)
+  if (a.pq_dim % (ip ? 128u : 64u) != 0 || a.pq_dim > 512u || a.rot_dim != a.pq_dim * a.pq_len) { return false; }
   if (a.pq_len != 1 && a.pq_len != 2 && a.pq_len != 4) { return false; }
   return a.lut_dtype == CUDA_R_16F || a.lut_dtype == CUDA_R_8U;
 }

@@ -919,18 +919,21 @@ def test_four_bit_block_kernel_matches_oracle(orc, lut, internal, dim, pq_dim, m
 
 
 @pytest.mark.parametrize("lut", [R_16F, R_8U])
+@pytest.mark.parametrize("internal", [R_16F, R_32F])
 @pytest.mark.parametrize("dim,pq_dim,metric,kind", [
     (256, 128, "sqeuclidean", "subspace"),   # two steps, pq_len 2, early stop inside a tile
     (128, 128, "inner_product", "subspace"), # pq_len 1
     (512, 128, "cosine", "cluster"),         # pq_len 4, per-cluster codebooks
     (512, 256, "euclidean", "subspace"),     # four steps
+    (128, 64, "sqeuclidean", "subspace"),    # a single step (L2 takes any number of them)
+    (192, 192, "euclidean", "cluster"),      # three steps, pq_len 1, per-cluster codebooks
 ])
-def test_four_bit_two_rows_per_lane_kernel_matches_oracle(orc, lut, dim, pq_dim, metric, kind):
-    """binary16 sums, pq_dim a multiple of 128, k <= 64: the kernel that scores two rows per lane
-    with packed adds, one wave per pair."""
+def test_four_bit_two_rows_per_lane_kernel_matches_oracle(orc, lut, internal, dim, pq_dim, metric, kind):
+    """pq_dim a multiple of 128, k <= 64, binary16 tables (sums of either type): the kernel that
+    scores two rows per lane, one wave per pair, with the bound looked at inside a step."""
     data, model, queries, index, ix, _ = _nibble_case(orc, dim, pq_dim, metric, kind)
     for k, n_probes in ((1, 3), (10, 8), (64, 24)):
-        nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, k, n_probes, lut=lut, internal=R_16F)
+        nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, k, n_probes, lut=lut, internal=internal)
         H.compare_results(nb, d, want_nb, want_d, 2e-3, exact=(metric != "euclidean"))
 
 
