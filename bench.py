@@ -246,8 +246,9 @@ def main():
     nibble = pq_bits == 4 and pq_dim % 32 == 0 and pq_len in (1, 2, 4) and (pq_dim // 16) * pq_len <= 48
     fused = k <= 256  # beyond that every score is stored and selected afterwards (generic kernel)
     full_name = ("scan_kernel" if not fused
-                 else "scan_nibble_pack_kernel" if (nibble and args.internal == "f16" and pq_dim % 128 == 0
-                                                    and pq_dim <= 512 and k <= 64 and args.lut != "f32")
+                 else "scan_nibble_pack_kernel" if (nibble and pq_dim <= 512 and k <= 64 and args.lut != "f32"
+                                                    and pq_dim % (128 if args.metric in ("inner_product", "cosine")
+                                                                  else 64) == 0)
                  else "scan_nibble_kernel" if nibble
                  else "scan_kernel" if (pq_bits not in (5, 6, 7, 8) or (pq_dim, pq_len) not in ((64, 2), (48, 2), (32, 4), (32, 2)))
                  else "scan_stream_kernel" if (args.lut != "f32" and k <= 128) else "scan_fast_kernel")

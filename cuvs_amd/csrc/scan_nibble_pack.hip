@@ -1,5 +1,5 @@
 /*
- * CU-wide LUT + code-scan kernel for 4-bit codes with binary16 sums (the sub-byte path of the
+ * CU-wide LUT + code-scan kernel for 4-bit codes with binary16 tables (the sub-byte path of the
  * reference's compute_similarity kernel, cpp/src/neighbors/ivf_pq/detail/jit_lto_kernels/
  * compute_score_impl.cuh:13-79 with PqBits = 4; tables as in create_lut_impl.cuh:16-79).
  *
@@ -7,8 +7,9 @@
  * 32-byte window), so the scan is bound by the vector instructions around the lookups, and the
  * kernel is built to need few of them:
  *
- *   - a lane scores two rows at a time, 64 apart: two independent chains of binary16 adds, so that
- *     one row's add is issued while the other's result is on its way.  Each row's entries are added
+ *   - a lane scores two rows at a time, 64 apart: two independent chains of adds (binary16, or fp32
+ *     through a multiply-add that widens the entry), so that one row's add is issued while the
+ *     other's result is on its way.  Each row's entries are added
  *     one by one in subspace order, as the reference adds them.  (The two sums cannot share a
  *     register and a packed add: a 16-bit LDS read into one half of a register clears the other
  *     half on this hardware, whose register files are ECC protected.);
@@ -18,11 +19,14 @@
  *     byte (the nibbles of a code word are spread over the bytes of two masked copies first: three
  *     instructions per eight codes); the subspace's offset is the read's immediate;
  *   - a step of two 16-byte chunks per row (64 subspaces, 128 lookups) is one block of assembly
- *     with three groups of eight reads in flight while the oldest is added.
+ *     with three groups of eight reads in flight while the oldest is added; an L2 scan looks at the
+ *     query's bound after 8, 16, 32 and 48 subspaces and ends the step when none of the 128 rows can
+ *     still win (early stop of compute_score in the reference), and has the next tile's first step
+ *     on its way rather than this tile's next one.
  *
- * One persistent 1024-thread block per CU.  An iteration takes up to twelve (query, probe) pairs:
+ * One persistent 1024-thread block per CU.  An iteration takes up to fifteen (query, probe) pairs:
  * all sixteen waves build the pairs' tables (a thread owns one codebook entry of every 64th
- * subspace and keeps those codebook components in registers), then each of the first twelve waves
+ * subspace and keeps those codebook components in registers), then each of the first fifteen waves
  * scans one pair against its table, with a candidate buffer and bound of its own, and writes the
  * pair's <= k best.  One wave per pair leaves no rows idle in a list's last tile but the last one's.
  */
@@ -35,10 +39,10 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t kPackThreads   = 1024;
-constexpr uint32_t kPackMaxPairs  = 12;    // pairs of an iteration: one scanner wave each
+constexpr uint32_t kPackMaxPairs  = 15;    // pairs of an iteration: one scanner wave each
 constexpr uint32_t kPackMaxK      = 64;
 constexpr uint32_t kPackWaveCap   = 128;   // candidate keys a wave buffers: k kept ones and one tile's
-constexpr uint32_t kPackCandBase  = 256;   // twelve buffers of 1 KB
+constexpr uint32_t kPackCandBase  = 256;   // fifteen buffers of 1 KB
 constexpr uint32_t kPackTableBase = 16384; // tables: pq_dim * 32 bytes each, 256-byte aligned
 constexpr uint32_t kPackLdsBytes  = 160 * 1024;
 constexpr uint32_t kPackStepBytes = 64 * 32;  // table bytes of the 64 subspaces of a step
