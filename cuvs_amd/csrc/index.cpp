@@ -181,7 +181,10 @@ void index_impl::rebuild_lead_plane(hipStream_t stream)
     pq_centers8  = device_buffer();
     n_chunks8    = 0;
   }
-  if ((pq_bits != 8 && !widen) || n_slots == 0 || n_slots + kLeadPlaneSlack > 0xFFFFFFFFull) {
+  // byte codes (as stored or widened), and nibble codes unless memory is to be spared: the plane
+  // is what lets an L2 search of either width screen pairs without scanning them
+  const bool plane_codes = pq_bits == 8 || widen || (pq_bits == 4 && !conservative_memory_allocation);
+  if (!plane_codes || n_slots == 0 || n_slots + kLeadPlaneSlack > 0xFFFFFFFFull) {
     lead_plane = device_buffer();
     return;
   }

@@ -311,6 +311,10 @@ constexpr uint32_t kDirectSubs    = 8;
 template <int PQ_LEN>
 struct book_vec;
 template <>
+struct book_vec<1> {
+  typedef float type __attribute__((ext_vector_type(1)));
+};
+template <>
 struct book_vec<2> {
   typedef float type __attribute__((ext_vector_type(2)));
 };
@@ -319,7 +323,7 @@ struct book_vec<4> {
   typedef float type __attribute__((ext_vector_type(4)));
 };
 
-template <int PQ_LEN, int LUT, bool OUT_HALF, int FIRST>
+template <int PQ_LEN, int LUT, bool OUT_HALF, int FIRST, int BITS>
 __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   scan_args a, const pair_desc* __restrict__ desc, uint32_t n_pairs, uint32_t group_bytes,
   pair_desc* __restrict__ survivors, uint32_t* __restrict__ n_survivors, uint8_t* __restrict__ alive)
@@ -328,12 +332,17 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   using lut_t  = typename traits::storage;
   using acc_t  = typename std::conditional<OUT_HALF, _Float16, float>::type;
   using vec_t  = typename book_vec<PQ_LEN>::type;
-  constexpr uint32_t SUB   = kDirectSubs;
+  // the eight leading code bytes of a row: 8 subspaces of 256 entries, or 16 of 16 (4-bit codes)
+  static_assert(BITS == 8 || BITS == 4, "byte or nibble codes");
+  constexpr uint32_t SUB   = BITS == 8 ? kDirectSubs : 2u * kDirectSubs;
+  constexpr uint32_t BOOK  = 1u << BITS;
+  constexpr int MID        = BITS == 8 ? 4 : 8;  // the second look at the bound
   constexpr uint32_t NDIFF = SUB * PQ_LEN;
   static_assert(NDIFF <= 64, "one lane per leading rotated dimension");
+  static_assert(FIRST <= 4 && FIRST <= MID, "the first subspaces' terms sit in scalar registers");
   auto* book      = reinterpret_cast<LDS_AS vec_t*>(uintptr_t(kScreenLdsBase));
   const float one = opaque_one_s();
-  constexpr uint32_t off_pending = kScreenLdsBase + SUB * 256u * PQ_LEN * 4u;
+  constexpr uint32_t off_pending = kScreenLdsBase + SUB * BOOK * PQ_LEN * 4u;
   constexpr uint32_t off_mini    = off_pending + (kDirectThreads / 64u) * kSurvivorBatchBytes;
   constexpr uint32_t kMiniTiles  = 6;
 
@@ -344,10 +353,10 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   const uint32_t total   = gridDim.x * WPB;
   if (blockIdx.x * WPB >= n_pairs) { return; }
 
-  for (uint32_t e = tid; e < SUB * 256u; e += kDirectThreads) {
+  for (uint32_t e = tid; e < SUB * BOOK; e += kDirectThreads) {
     vec_t v;
 #pragma unroll
-    for (int t = 0; t < PQ_LEN; t++) { v[t] = a.pq_centers[((e >> 8) * PQ_LEN + t) * 256u + (e & 255u)]; }
+    for (int t = 0; t < PQ_LEN; t++) { v[t] = a.pq_centers[((e / BOOK) * PQ_LEN + t) * BOOK + (e % BOOK)]; }
     book[e] = v;
   }
   lds_barrier_s();
@@ -434,7 +443,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
       // (the subspaces every tile looks at): 4 * FIRST entries a lane, computed as below, against
       // FIRST entries a lane and tile.  The wave reads what it wrote itself: LDS serves a wave's
       // requests in order, no barrier.
-      const bool tabled = n_tiles >= kMiniTiles;
+      const bool tabled = BITS == 8 && n_tiles >= kMiniTiles;
       if (tabled) {
 #pragma unroll
         for (uint32_t e = 0; e < uint32_t(FIRST) * 4u; e++) {
@@ -458,12 +467,12 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
         auto add_codes = [&](int first, int last) __attribute__((always_inline)) {
 #pragma unroll
           for (int kk = first; kk < last; kk++) {
-            const uint32_t c = (w[kk >> 2] >> ((kk & 3) * 8)) & 0xffu;
+            const uint32_t c = BITS == 8 ? (w[kk >> 2] >> ((kk & 3) * 8)) & 0xffu : (w[kk >> 3] >> ((kk & 7) * 4)) & 0xfu;
             lut_t v;
             if (decltype(use_table)::value && kk < FIRST) {
               v = mini[kk * 256 + c];
             } else {
-              const vec_t b = book[kk * 256 + c];
+              const vec_t b = book[kk * int(BOOK) + c];
               float score   = 0.0f;
 #pragma unroll
               for (int t = 0; t < PQ_LEN; t++) {
@@ -494,12 +503,12 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
         };
         add_codes(0, FIRST);
         in_play = any_in_play();
-        if (FIRST < 4 && in_play) {
-          add_codes(FIRST, 4);
+        if (FIRST < MID && in_play) {
+          add_codes(FIRST, MID);
           in_play = any_in_play();
         }
         if (in_play) {
-          add_codes(4, int(SUB));
+          add_codes(MID, int(SUB));
           in_play = any_in_play();
         }
       };
@@ -542,13 +551,15 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   if (n_pending != 0) { flush_survivors(pending, n_pending, lane, survivors, n_survivors); }
 }
 
-template <int PQ_LEN, int LUT, bool OUT_HALF, int FIRST>
+template <int PQ_LEN, int LUT, bool OUT_HALF, int FIRST, int BITS>
 void launch_screen_direct_first(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
                                 pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
                                 hipStream_t stream)
 {
-  auto kernel       = scan_screen_direct_kernel<PQ_LEN, LUT, OUT_HALF, FIRST>;
-  const size_t smem = kScreenLdsBase + size_t(kDirectSubs) * 256 * PQ_LEN * 4 +
+  auto kernel       = scan_screen_direct_kernel<PQ_LEN, LUT, OUT_HALF, FIRST, BITS>;
+  // codebooks of the leading subspaces (8 x 256 or 16 x 16 entries), a batch of survivors per wave,
+  // and (byte codes) a wave's table of the first subspaces
+  const size_t smem = kScreenLdsBase + size_t(kDirectSubs) * (BITS == 8 ? 256 : 32) * PQ_LEN * 4 +
                       size_t(kDirectThreads / 64u) * kSurvivorBatchBytes +
                       size_t(kDirectThreads / 64u) * FIRST * 256 * sizeof(typename lut_traits<LUT>::storage);
   // persistent blocks: exactly as many as are resident at once (per instance)
@@ -568,7 +579,11 @@ template <int PQ_LEN, int LUT, bool OUT_HALF>
 void launch_screen_direct(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
                           pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive, hipStream_t stream)
 {
-  launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, kScreenFirstCheck>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+  if (a.pq_bits == 4) {
+    launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, 4, 4>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+    return;
+  }
+  launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, kScreenFirstCheck, 8>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
 }
 
 template <int SUBS, int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER>
@@ -640,8 +655,13 @@ uint32_t scan_screen_bytes_per_row(bool per_cluster, bool lead_plane)
 bool scan_screen_supported(const scan_args& a)
 {
   const bool l2 = a.metric == int(DistanceType::L2Expanded) || a.metric == int(DistanceType::L2SqrtExpanded);
-  if (!l2 || !a.fused || a.pq_bits != 8 || a.pq_dim < 32) { return false; }
+  if (!l2 || !a.fused || (a.pq_bits != 8 && a.pq_bits != 4) || a.pq_dim < 32) { return false; }
   if (a.lut_dtype == CUDA_R_32F && a.out_half) { return false; }
+  if (a.pq_bits == 4) {
+    // nibble codes: only the table-free kernel on the plane of leading code bytes reads them
+    return !a.per_cluster && a.lead_plane != nullptr && a.lut_dtype != CUDA_R_32F &&
+           (a.pq_len == 1 || a.pq_len == 2 || a.pq_len == 4);
+  }
   return a.pq_len == 2 || a.pq_len == 4;
 }
 
@@ -651,7 +671,9 @@ void launch_scan_screen(const scan_args& a, const pair_desc* desc, uint32_t n_pa
 {
   CUVS_EXPECTS(scan_screen_supported(a), "the screening pass does not cover these search arguments");
   if (n_pairs == 0) { return; }
-  if (a.pq_len == 2) {
+  if (a.pq_len == 1) {
+    launch_screen_types<1, false>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+  } else if (a.pq_len == 2) {
     if (a.per_cluster) {
       launch_screen_types<2, true>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
     } else {

@@ -371,7 +371,7 @@ void search(cuvs::resources const& res_c,
   sa.list_sizes   = ix.list_sizes.as<uint32_t>();
   sa.filter_bits  = filter_bits;
   sa.filter_nbits = filter_nbits;
-  if (ix.pq_bits != 8) { sa.lead_plane = nullptr; }
+  if (ix.pq_bits != 8 && ix.pq_bits != 4) { sa.lead_plane = nullptr; }
   if (ix.wide() && !res.tuning.generic_scan) {
     // 5 - 7 bit codes: the byte-wide copy of the lists, if one of the 8-bit kernels takes the shape
     detail::scan_args w = sa;
@@ -441,6 +441,8 @@ void search(cuvs::resources const& res_c,
   const bool few_pairs       = uint64_t(Qb) * P <= kFewPairs;
   bool early_stop = fast_scan && !few_pairs && P > kLeadProbes && P <= 8192 &&
                     detail::scan_screen_supported(sa) && res.tuning.early_stop != 1;
+  // nibble codes: the leading and the surviving pairs go to the wave-per-pair kernel
+  if (sa.pq_bits == 4 && !detail::scan_nibble_pack_supported(sa)) { early_stop = false; }
   // In the automatic mode the index remembers whether the screen pays on its data: where it kept
   // most pairs the last time it ran with these parameters, this search scans plainly.
   bool observe_screen = false;
@@ -540,7 +542,9 @@ void search(cuvs::resources const& res_c,
     if (early_stop) {
       // 1. the leading probes' lists in full: candidates and a first bound per query
       auto full_scan = [&] {
-        return quad_kpp != 0 ? detail::launch_scan_stream(sa, s) : detail::launch_scan_fast(sa, s);
+        return quad_kpp != 0   ? detail::launch_scan_stream(sa, s)
+               : sa.pq_bits == 4 ? detail::launch_scan_nibble_pack(sa, s)
+                                 : detail::launch_scan_fast(sa, s);
       };
       sa.n_pairs = nq * lead;
       CUVS_EXPECTS(full_scan(), "scan kernel launch failed");

@@ -514,6 +514,39 @@ def test_early_stop_pq_len_4(orc, kind):
         H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
 
 
+@pytest.mark.parametrize("lut,internal", [(R_16F, R_32F), (R_8U, R_32F), (R_16F, R_16F), (R_8U, R_16F)])
+@pytest.mark.parametrize("dim,pq_dim", [(128, 64), (128, 128), (256, 64), (192, 192)])
+def test_early_stop_with_four_bit_codes(orc, lut, internal, dim, pq_dim):
+    """4-bit codes, L2: the leading pairs and the survivors of the screen go to the wave-per-pair
+    kernel, the screen sums the 16 subspaces of the leading 8 code bytes (pq_len 2, 1, 4, 1; one,
+    two, one and three steps of 64 subspaces a row).  Same results as the oracle and as the single
+    launch."""
+    import datasets as testing
+    from cuvs_amd.resources import Resources
+    allrows = testing.gaussian_mixture(24200, dim, 64, 0.15, seed=79).numpy()
+    x, q = allrows[:24000], allrows[24000:]
+    model = H.train(x, 120, pq_dim, 4, iters=6)
+    index = G.build_gpu_index(model, x, pq_dim, 4, "sqeuclidean", "subspace")
+    ix, _ = G.read_back(orc, index, model, dim, pq_dim, 4, "sqeuclidean", "subspace")
+    res = Resources()
+    res.enable_profiling(True)
+    sp = ivf_pq.SearchParams(n_probes=40, lut_dtype=lut, internal_distance_dtype=internal)
+    for k in (1, 10, 64):
+        d, nb = ivf_pq.search(sp, index, G.to_dev(q), k, resources=res)
+        res.sync()
+        prof = ivf_pq.get_search_profile(res)
+        assert prof["n_screened_pairs"] == q.shape[0] * 39
+        assert 0 < prof["n_surviving_pairs"] < prof["n_screened_pairs"]
+        want_nb, want_d = orc.search(ix, q, k, 40, lut_dtype=ORC_DT[lut], internal_distance_dtype=ORC_DT[internal])
+        H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
+        res.set_search_tuning(early_stop="off")
+        d2, nb2 = ivf_pq.search(sp, index, G.to_dev(q), k, resources=res)
+        res.sync()
+        assert ivf_pq.get_search_profile(res)["n_screened_pairs"] == 0
+        res.set_search_tuning(early_stop="auto")
+        assert torch.equal(nb, nb2) and torch.equal(d, d2)
+
+
 def test_early_stop_with_filter_and_small_lists(orc):
     """A filter can leave the leading list with fewer than k rows (no bound: nothing is dropped),
     and the screen ignores the filter (it may keep a pair whose rows in play are all filtered)."""
