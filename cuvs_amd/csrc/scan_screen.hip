@@ -443,15 +443,22 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
       // (the subspaces every tile looks at): 4 * FIRST entries a lane, computed as below, against
       // FIRST entries a lane and tile.  The wave reads what it wrote itself: LDS serves a wave's
       // requests in order, no barrier.
-      const bool tabled = BITS == 8 && n_tiles >= kMiniTiles;
+      // (Nibble codes: 16 entries a subspace, one entry a lane for the first four: always.)
+      const bool tabled = BITS == 4 || n_tiles >= kMiniTiles;
       if (tabled) {
 #pragma unroll
-        for (uint32_t e = 0; e < uint32_t(FIRST) * 4u; e++) {
+        for (uint32_t e = 0; e < uint32_t(FIRST) * BOOK / 64u; e++) {
           const vec_t b = book[e * 64u + lane];
           float score   = 0.0f;
 #pragma unroll
           for (int t = 0; t < PQ_LEN; t++) {
-            float df = diff[(e >> 2) * PQ_LEN + t];
+            float df;
+            if constexpr (BITS == 8) {
+              df = diff[(e >> 2) * PQ_LEN + t];  // 256 entries: four rounds a subspace
+            } else {
+              // the lane's entry belongs to subspace lane / 16, whose terms sit in lanes of `dv0`
+              df = __shfl(dv0, int((lane >> 4) * uint32_t(PQ_LEN) + uint32_t(t)), 64);
+            }
             df -= b[t];
             score = fmaf(df, df, score);
           }
@@ -470,7 +477,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
             const uint32_t c = BITS == 8 ? (w[kk >> 2] >> ((kk & 3) * 8)) & 0xffu : (w[kk >> 3] >> ((kk & 7) * 4)) & 0xfu;
             lut_t v;
             if (decltype(use_table)::value && kk < FIRST) {
-              v = mini[kk * 256 + c];
+              v = mini[kk * int(BOOK) + c];
             } else {
               const vec_t b = book[kk * int(BOOK) + c];
               float score   = 0.0f;
