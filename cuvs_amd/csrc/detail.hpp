@@ -341,7 +341,10 @@ struct scan_args {
   unsigned long long* out_keys;   // fused: [n_queries, n_probes, k]
   float* out_scores;              // non-fused: [n_queries, max_samples]
   void* global_lut;               // generic kernel: table scratch when it does not fit LDS, or null
-  const uint64_t* lead_plane;     // first eight code bytes of every row slot (8-bit codes), or null
+  const uint64_t* lead_plane;     // first eight code bytes of every row slot (8- and 4-bit codes), or null
+  int rare_exits;                 // few tiles of this launch are expected to end early (the leading and the
+                                  // surviving pairs of an early stop): the wave-per-pair kernel then has a
+                                  // tile's next step on its way instead of the next tile's first one
 };
 /** LDS bytes the scan kernel needs for these arguments (without the table when `global_lut` is
  *  set), the bytes of one lookup table, and the number of blocks (= table slices) the generic

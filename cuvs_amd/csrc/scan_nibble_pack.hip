@@ -405,9 +405,82 @@ __global__ __launch_bounds__(kPackThreads) void scan_nibble_pack_kernel(scan_arg
             take(sum_of(acc_a), valid_a, row_a);
             take(sum_of(acc_b), valid_b, row_b);
           };
-          for (uint32_t tile = 0; tile < n_tiles; tile += 2u) {
-            l2_tile(tile, cur_a, cur_b, nxt_a, nxt_b);
-            if (tile + 1u < n_tiles) { l2_tile(tile + 1u, nxt_a, nxt_b, cur_a, cur_b); }
+          if (a.rare_exits == 0 || (n_steps & 1u) != 0u) {
+            for (uint32_t tile = 0; tile < n_tiles; tile += 2u) {
+              l2_tile(tile, cur_a, cur_b, nxt_a, nxt_b);
+              if (tile + 1u < n_tiles) { l2_tile(tile + 1u, nxt_a, nxt_b, cur_a, cur_b); }
+            }
+          } else {
+            // Pairs whose rows mostly stay under the bound (no bound yet, or the survivors of the
+            // screen): a tile's next step is what should be on its way, as for inner products, and a
+            // tile that does end early fetches the next one's first step afresh.
+            for (uint32_t tile = 0; tile < n_tiles; tile++) {
+              const uint32_t row_a = tile * 128u + lane;
+              const uint32_t row_b = row_a + 64u;
+              const bool valid_a   = in_play(row_a);
+              const bool valid_b   = in_play(row_b);
+#pragma unroll
+              for (int i = 0; i < 4; i++) {
+                aa[i] = table;
+                ab[i] = table;
+                asm volatile("" : "+v"(aa[i]), "+v"(ab[i]));
+              }
+              uint32_t acc_a = 0, acc_b = 0;
+              bool stopped   = false;
+              const uint32_t stop_bits        = thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u;
+              const unsigned long long mask_a = __builtin_amdgcn_ballot_w64(valid_a);
+              const unsigned long long mask_b = __builtin_amdgcn_ballot_w64(valid_b);
+              auto all_past = [&]() {
+                return __builtin_amdgcn_ballot_w64((valid_a && !(sum_of(acc_a) > thr_f)) ||
+                                                   (valid_b && !(sum_of(acc_b) > thr_f))) == 0ull;
+              };
+              for (uint32_t step = 0; step < n_steps; step += 2) {
+                {
+                  const uint32_t ra = row_a < n_rows ? row_a : 0u;
+                  const uint32_t rb = row_b < n_rows ? row_b : 0u;
+                  load_step(ra, step + 1u, nxt_a);
+                  load_step(rb, step + 1u, nxt_b);
+                }
+                nibble_pack_step<HALF, true>(acc_a, acc_b, cur_a, cur_b, aa, ab, one_u, one, stop_bits, mask_a, mask_b);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                  aa[i] += kPackStepBytes;
+                  ab[i] += kPackStepBytes;
+                }
+                if (all_past()) {
+                  stopped = true;
+                  break;
+                }
+                {
+                  const bool more   = step + 2u < n_steps;
+                  const uint32_t na = more ? row_a : row_a + 128u;
+                  const uint32_t nb = more ? row_b : row_b + 128u;
+                  load_step(na < n_rows ? na : 0u, more ? step + 2u : 0u, cur_a);
+                  load_step(nb < n_rows ? nb : 0u, more ? step + 2u : 0u, cur_b);
+                }
+                nibble_pack_step<HALF, true>(acc_a, acc_b, nxt_a, nxt_b, aa, ab, one_u, one, stop_bits, mask_a, mask_b);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                  aa[i] += kPackStepBytes;
+                  ab[i] += kPackStepBytes;
+                }
+                if (step + 2u < n_steps && all_past()) {
+                  stopped = true;
+                  break;
+                }
+              }
+              if (stopped) {
+                // the codes on their way are of this tile: the next tile's first step is fetched afresh
+                if (tile + 1u < n_tiles) {
+                  const uint32_t na = row_a + 128u, nb = row_b + 128u;
+                  load_step(na < n_rows ? na : 0u, 0u, cur_a);
+                  load_step(nb < n_rows ? nb : 0u, 0u, cur_b);
+                }
+                continue;  // every row in play is past the bound
+              }
+              take(sum_of(acc_a), valid_a, row_a);
+              take(sum_of(acc_b), valid_b, row_b);
+            }
           }
         } else {
           for (uint32_t tile = 0; tile < n_tiles; tile++) {

@@ -546,7 +546,8 @@ void search(cuvs::resources const& res_c,
                : sa.pq_bits == 4 ? detail::launch_scan_nibble_pack(sa, s)
                                  : detail::launch_scan_fast(sa, s);
       };
-      sa.n_pairs = nq * lead;
+      sa.n_pairs    = nq * lead;
+      sa.rare_exits = 1;  // no bound yet here, and the screen's survivors mostly stay under theirs
       CUVS_EXPECTS(full_scan(), "scan kernel launch failed");
       detail::launch_kth_bound(keys, nq, uint64_t(P) * kpp, lead * kpp, k, kth, s);
       mark(5);
