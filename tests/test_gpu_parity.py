@@ -547,6 +547,34 @@ def test_early_stop_with_four_bit_codes(orc, lut, internal, dim, pq_dim):
         assert torch.equal(nb, nb2) and torch.equal(d, d2)
 
 
+def test_four_bit_index_without_the_plane_of_leading_codes(orc):
+    """conservative_memory_allocation: a 4-bit index keeps no plane of leading code bytes, and an L2
+    search is then one scan launch with the same results."""
+    import datasets as testing
+    from cuvs_amd.resources import Resources
+    allrows = testing.gaussian_mixture(24200, 128, 64, 0.15, seed=80, device="cuda")
+    x, q = allrows[:24000], allrows[24000:]
+    kw = dict(n_lists=120, pq_dim=64, pq_bits=4)
+    trained = ivf_pq.build(ivf_pq.IndexParams(add_data_on_build=False, **kw), x)
+    model = (trained.pq_centers, trained.centers_padded, trained.centers_rot, trained.rotation_matrix)
+    ids = torch.arange(24000, dtype=torch.int64, device="cuda")
+    index = ivf_pq.extend(ivf_pq.build_precomputed(ivf_pq.IndexParams(**kw), 128, *model), x, ids)
+    lean = ivf_pq.extend(ivf_pq.build_precomputed(
+        ivf_pq.IndexParams(conservative_memory_allocation=True, **kw), 128, *model), x, ids)
+    res = Resources()
+    res.enable_profiling(True)
+    sp = ivf_pq.SearchParams(n_probes=40, lut_dtype=R_16F)
+    d, nb = ivf_pq.search(sp, index, q, 10, resources=res)
+    res.sync()
+    assert ivf_pq.get_search_profile(res)["n_screened_pairs"] == q.shape[0] * 39
+    d2, nb2 = ivf_pq.search(sp, lean, q, 10, resources=res)
+    res.sync()
+    assert ivf_pq.get_search_profile(res)["n_screened_pairs"] == 0
+    assert torch.equal(d, d2)
+    tied = (d == d.roll(1, dims=1)) | (d == d.roll(-1, dims=1))  # another index object: rows may swap places
+    assert bool(((nb == nb2) | tied).all())
+
+
 def test_early_stop_with_filter_and_small_lists(orc):
     """A filter can leave the leading list with fewer than k rows (no bound: nothing is dropped),
     and the screen ignores the filter (it may keep a pair whose rows in play are all filtered)."""
