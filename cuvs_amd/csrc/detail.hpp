@@ -157,10 +157,12 @@ struct index_impl {
   bool rotation_is_identity = false;
 
   device_buffer codes_arena, ids_arena;
-  /** 8-bit codes: the first eight code bytes of every row slot, packed (8 bytes per row next to the
-   *  arena's n_chunks * 16): the early-stop screen decides on these alone, and reading them here
-   *  touches half the cache lines the interleaved arena would, in whole lines.  Rebuilt whenever
-   *  the arena changes; empty for other code widths or 2^32 and more row slots. */
+  /** 8-bit codes (also the byte-wide copy of narrower ones) and 4-bit codes: the first eight code
+   *  bytes of every row slot, packed (8 bytes per row next to the arena's n_chunks * 16): the
+   *  early-stop screen decides on these alone, and reading them here touches half the cache lines
+   *  the interleaved arena would, in whole lines.  Rebuilt whenever the arena changes; empty for
+   *  other code widths, for 4-bit codes with conservative_memory_allocation, or with 2^32 and more
+   *  row slots. */
   device_buffer lead_plane;
   /** 5 - 7 bit codes: the lists once more with a byte per code, in the layout of an 8-bit index
    *  (n_chunks8 = ceil(pq_dim / 16) chunks a row), their pointer table, and the codebooks padded to

@@ -1,5 +1,5 @@
 /*
- * Screening pass of the L2 early stop (8-bit codes).
+ * Screening pass of the L2 early stop (8-bit codes; 4-bit codes through the table-free kernel).
  *
  * A row's score is a sum of non-negative table entries taken in subspace order, so the partial sum
  * over the first S subspaces is a lower bound of its final score, and it is exactly the
@@ -10,7 +10,8 @@
  * list at once).  For clustered data this removes most (query, probe) pairs for an eighth of the
  * table-building and gather work, and only the survivors go through the full scan.  S = 8 by
  * default (the first half of each row's first 16-byte chunk): on the benchmark data as many pairs
- * are dropped as with 16, and with 4 three times as many survive.
+ * are dropped as with 16, and with 4 three times as many survive.  The same 8 bytes of a row of
+ * 4-bit codes hold 16 subspaces of 16 entries.
  *
  * Organisation: persistent 256-thread blocks, several per CU so that the table-building phase of
  * one block overlaps the gather phase of another.  A block takes G = 4 pairs per iteration; thread
