@@ -5,6 +5,7 @@
 #pragma once
 
 #include "device_utils.cuh"
+#include "scan_wave_select.cuh"
 
 namespace cuvs::neighbors::ivf_pq::detail {
 
@@ -36,7 +37,8 @@ __device__ __forceinline__ void lds_barrier()
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-/** Keep the k smallest keys of cand[0..count) sorted at the front; publish the k-th score.
+/** Keep the k smallest keys of cand[0..count) at the front (in no particular order beyond 64
+ *  candidates); publish the k-th score.
  *  `cnt` is the candidate count every thread read between two barriers; returns after a barrier.
  *  No-op when cnt < k. */
 __device__ __forceinline__ void block_prune(LDS_AS unsigned long long* cand, LDS_AS fast_tail* tail,
@@ -60,6 +62,45 @@ __device__ __forceinline__ void block_prune(LDS_AS unsigned long long* cand, LDS
       if (tid < cnt && rank < k) { cand[rank] = key; }
       if (tid < cnt && rank == k - 1u) { tail->thr = hi; }
       if (tid == 0) { tail->count = k; }
+    }
+    lds_barrier();
+    return;
+  }
+  if (cnt <= 1024u) {
+    // one wave keeps the k smallest by radix selection on its registers (no order among them)
+    if (tid < 64u) {
+      const uint32_t kth = cnt <= 256u   ? wave_select_keys<4>(cand, tid, cnt, k)
+                           : cnt <= 512u ? wave_select_keys<8>(cand, tid, cnt, k)
+                                         : wave_select_keys<16>(cand, tid, cnt, k);
+      if (tid == 0) {
+        tail->count = k;
+        tail->thr   = kth;
+      }
+    }
+    lds_barrier();
+    return;
+  }
+  if (cnt <= 2048u && k <= 256u) {
+    // two waves take a half each, then one of them what the halves kept
+    const uint32_t second = cnt - 1024u;
+    if (tid < 64u) {
+      wave_select_keys<16>(cand, tid, 1024u, k);
+    } else if (tid < 128u && second > k) {
+      wave_select_keys<16>(cand + 1024, tid - 64u, second, k);
+    }
+    lds_barrier();
+    const uint32_t kept = second < k ? second : k;
+    unsigned long long moved = kInvalidKey;
+    if (tid < kept) { moved = cand[1024u + tid]; }  // kept <= 256 = the block's threads
+    lds_barrier();
+    if (tid < kept) { cand[k + tid] = moved; }
+    lds_barrier();
+    if (tid < 64u) {
+      const uint32_t kth = wave_select_keys<8>(cand, tid, k + kept, k);
+      if (tid == 0) {
+        tail->count = k;
+        tail->thr   = kth;
+      }
     }
     lds_barrier();
     return;
