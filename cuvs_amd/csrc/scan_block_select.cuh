@@ -20,7 +20,7 @@ namespace {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte chunk of codes
 constexpr uint32_t kLdsBase = 16;
 
-constexpr uint32_t kFastCap      = 2048;                // candidate keys held per block
+constexpr uint32_t kFastCap      = 1536;                // candidate keys held per block (with a 64 KB fp32 table, two blocks still share a CU)
 constexpr uint32_t kFastMaxK     = 256;                 // largest k the buffer arithmetic allows
 constexpr uint32_t kFastSegIters = (kFastCap - kFastMaxK) / kBlock;  // row iterations per prune
 
