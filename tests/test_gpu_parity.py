@@ -1104,6 +1104,17 @@ def test_byte_wide_copy_of_narrow_codes_follows_the_lists():
         assert int(nb.max()) >= 40000  # the rows added later are found
 
 
+@pytest.mark.parametrize("lut", [R_32F, R_16F])
+def test_block_per_pair_kernel_prunes_long_lists(orc, lut):
+    """Lists of 5,000 rows scanned by the block-per-pair kernel (fp32 tables; k above the CU-wide
+    kernel's limit): its candidate buffer fills to 1,280 and more keys several times a list and is
+    pruned by the waves' radix selection, in one piece up to 1,024 keys and in two halves beyond."""
+    data, model, queries, index, ix, _ = _case(orc, 20000, 128, 4, 64, 8, n_queries=32)
+    for k, n_probes in ((256, 3), (100, 4), (10, 2)):
+        nb, d, want_nb, want_d = _search_both(orc, index, ix, queries, k, n_probes, lut=lut)
+        H.compare_results(nb, d, want_nb, want_d, 1e-5 if lut == R_32F else 2e-3, exact=True)
+
+
 def test_four_bit_block_kernel_filter_and_long_lists(orc):
     """Lists of several thousand rows (more than one pruning segment of the candidate buffer) and a
     bitset filter."""
