@@ -399,6 +399,10 @@ bool launch_scan_nibble(const scan_args& a, hipStream_t stream);
 /** 4-bit codes with binary16 sums, two rows per lane and one wave per pair (pq_dim a multiple of 128
  *  up to 512, k <= 64, fp16 or 8-bit tables; scan_nibble_pack.hip).  k keys per pair. */
 bool scan_nibble_pack_supported(const scan_args& a);
+/** Table-free wave-per-pair scan for fp32 tables (8-bit codes, L2, per-subspace codebooks, pq_len 2,
+ *  k <= 64): what the leading and the surviving pairs of an early stop take. */
+bool scan_direct_supported(const scan_args& a);
+bool launch_scan_direct(const scan_args& a, hipStream_t stream);
 bool launch_scan_nibble_pack(const scan_args& a, hipStream_t stream);
 /** CU-wide kernel for 8-bit codes, k <= 128 and fp16 / 8-bit tables (scan_stream.hip).  It writes
  *  several candidate groups per pair: scan_stream_keys_per_pair() is the number of keys the output

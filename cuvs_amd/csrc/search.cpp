@@ -542,9 +542,10 @@ void search(cuvs::resources const& res_c,
     if (early_stop) {
       // 1. the leading probes' lists in full: candidates and a first bound per query
       auto full_scan = [&] {
-        return quad_kpp != 0   ? detail::launch_scan_stream(sa, s)
-               : sa.pq_bits == 4 ? detail::launch_scan_nibble_pack(sa, s)
-                                 : detail::launch_scan_fast(sa, s);
+        return quad_kpp != 0                       ? detail::launch_scan_stream(sa, s)
+               : sa.pq_bits == 4                     ? detail::launch_scan_nibble_pack(sa, s)
+               : detail::scan_direct_supported(sa) ? detail::launch_scan_direct(sa, s)
+                                                     : detail::launch_scan_fast(sa, s);
       };
       sa.n_pairs    = nq * lead;
       sa.rare_exits = 1;  // no bound yet here, and the screen's survivors mostly stay under theirs
