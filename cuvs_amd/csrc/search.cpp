@@ -428,7 +428,8 @@ void search(cuvs::resources const& res_c,
   const bool generic_only  = res.tuning.generic_scan || global_lut;
   const uint32_t quad_kpp  = generic_only ? 0u : detail::scan_stream_keys_per_pair(sa);
   const bool nibble_scan   = !generic_only && detail::scan_nibble_supported(sa);
-  const bool fast_scan     = !generic_only && (quad_kpp != 0 || detail::scan_fast_supported(sa) || nibble_scan);
+  const bool fast_scan     = !generic_only && (quad_kpp != 0 || detail::scan_fast_supported(sa) || nibble_scan ||
+                                               detail::scan_direct_supported(sa));
   const uint32_t kpp       = quad_kpp != 0 ? quad_kpp : k;  // candidate keys stored per pair
   if (fast_scan) {
     desc = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));
@@ -580,7 +581,8 @@ void search(cuvs::resources const& res_c,
       const bool launched = fast_scan && (quad_kpp != 0   ? detail::launch_scan_stream(sa, s)
                                           : nibble_scan ? (detail::launch_scan_nibble_pack(sa, s) ||
                                                            detail::launch_scan_nibble(sa, s))
-                                                        : detail::launch_scan_fast(sa, s));
+                                                        : (detail::launch_scan_fast(sa, s) ||
+                                                           detail::launch_scan_direct(sa, s)));
       if (!launched) { detail::launch_scan(sa, s); }
     }
     }

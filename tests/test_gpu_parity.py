@@ -575,6 +575,44 @@ def test_four_bit_index_without_the_plane_of_leading_codes(orc):
     assert bool(((nb == nb2) | tied).all())
 
 
+@pytest.mark.parametrize("dim,pq_dim", [(128, 64), (96, 48), (64, 32)])
+def test_early_stop_with_fp32_tables(orc, dim, pq_dim):
+    """fp32 tables (the reference's default lut_dtype): the leading and the surviving pairs go to
+    the table-free wave-per-pair kernel (four, three and two chunks a row), with and without a
+    bitset filter; same results as the oracle and as the single launch of the block-per-pair kernel."""
+    import datasets as testing
+    from cuvs_amd.resources import Resources
+    allrows = testing.gaussian_mixture(24300, dim, 64, 0.15, seed=81).numpy()
+    x, q = allrows[:24000], allrows[24000:]
+    model = H.train(x, 120, pq_dim, 8, iters=6)
+    index = G.build_gpu_index(model, x, pq_dim, 8, "euclidean", "subspace")
+    ix, _ = G.read_back(orc, index, model, dim, pq_dim, 8, "euclidean", "subspace")
+    n = x.shape[0]
+    keep = np.ones(n, dtype=bool)
+    keep[::3] = False
+    bits = np.packbits(keep, bitorder="little")
+    bits = np.concatenate([bits, np.zeros((-bits.size) % 4, dtype=np.uint8)]).view(np.uint32)
+    res = Resources()
+    res.enable_profiling(True)
+    sp = ivf_pq.SearchParams(n_probes=30)  # lut_dtype and internal_distance_dtype at their defaults
+    for k, filtered in ((1, False), (10, False), (64, False), (10, True), (64, True)):
+        kw = dict(filter_bitset=G.to_dev(bits.view(np.int32)), filter_nbits=n) if filtered else {}
+        okw = dict(filter_bitset=bits, filter_nbits=n) if filtered else {}
+        d, nb = ivf_pq.search(sp, index, G.to_dev(q), k, resources=res, **kw)
+        res.sync()
+        prof = ivf_pq.get_search_profile(res)
+        assert prof["n_screened_pairs"] == q.shape[0] * 29
+        assert 0 < prof["n_surviving_pairs"] < prof["n_screened_pairs"]
+        want_nb, want_d = orc.search(ix, q, k, 30, **okw)
+        H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 1e-5, exact=False)
+        res.set_search_tuning(early_stop="off")
+        d2, nb2 = ivf_pq.search(sp, index, G.to_dev(q), k, resources=res, **kw)
+        res.sync()
+        assert ivf_pq.get_search_profile(res)["n_screened_pairs"] == 0
+        res.set_search_tuning(early_stop="auto")
+        assert torch.equal(nb, nb2) and torch.equal(d, d2)
+
+
 def test_early_stop_with_filter_and_small_lists(orc):
     """A filter can leave the leading list with fewer than k rows (no bound: nothing is dropped),
     and the screen ignores the filter (it may keep a pair whose rows in play are all filtered)."""
