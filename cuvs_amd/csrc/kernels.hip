@@ -848,9 +848,13 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(scan_args a)
   scan_smem_tail* tail = reinterpret_cast<scan_smem_tail*>(cand + (FUSED ? kCandCap : 0));
 
   const uint32_t tid = threadIdx.x;
-  // one pair per block; with a global table a bounded grid walks over the pairs
-  for (uint32_t pb = blockIdx.x; pb < a.n_queries * a.n_probes; pb += gridDim.x) {
-  const uint32_t pair = a.pair_order != nullptr ? a.pair_order[pb] : pb;
+  // one pair per block; with a global table, or a number of pairs only the device knows, a bounded
+  // grid walks over the pairs.  A subset of the pairs (the leading or the surviving ones of an early
+  // stop) comes as a list of records.
+  const uint32_t n_work = a.subset != 0 ? (a.n_pairs_dev != nullptr ? *a.n_pairs_dev : a.n_pairs)
+                                        : a.n_queries * a.n_probes;
+  for (uint32_t pb = blockIdx.x; pb < n_work; pb += gridDim.x) {
+  const uint32_t pair = a.subset != 0 ? a.desc[pb].slot : a.pair_order != nullptr ? a.pair_order[pb] : pb;
   const uint32_t q    = pair / a.n_probes;
   const uint32_t p    = pair - q * a.n_probes;
   const uint32_t label = a.probes[uint64_t(q) * a.n_probes + p];
@@ -1763,7 +1767,13 @@ void launch_scan_instance(const scan_args& a, hipStream_t stream)
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
   }
-  kernel<<<a.n_queries * a.n_probes, kBlock, smem, stream>>>(a);
+  uint32_t grid = a.n_queries * a.n_probes;
+  if (a.subset != 0) {
+    // a count known to the device only: as many blocks as keep the chip busy, each walking on
+    grid = a.n_pairs_dev != nullptr ? std::min(grid, uint32_t(device_cu_count()) * 16u) : a.n_pairs;
+    if (grid == 0) { return; }
+  }
+  kernel<<<grid, kBlock, smem, stream>>>(a);
   CUVS_LAUNCH_CHECK();
 }
 

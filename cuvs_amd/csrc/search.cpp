@@ -431,7 +431,10 @@ void search(cuvs::resources const& res_c,
   const bool fast_scan     = !generic_only && (quad_kpp != 0 || detail::scan_fast_supported(sa) || nibble_scan ||
                                                detail::scan_direct_supported(sa));
   const uint32_t kpp       = quad_kpp != 0 ? quad_kpp : k;  // candidate keys stored per pair
-  if (fast_scan) {
+  // byte codes of a shape no specialised kernel takes (pq_dim beyond 64): the generic kernel scans
+  // the leading and the surviving pairs of an early stop as a subset of the pairs
+  const bool generic_subset = !generic_only && !fast_scan && sa.pq_bits == 8 && sa.fused;
+  if (fast_scan || generic_subset) {
     desc = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));
   }
   // L2 early stop: lists of the leading probes in full, the others screened on their first chunk
@@ -440,7 +443,7 @@ void search(cuvs::resources const& res_c,
   // they save (the reference skips the grouping when lists are rarely shared,
   // expected_probe_coresidency, ivf_pq_search.cuh:353-373).
   const bool few_pairs       = uint64_t(Qb) * P <= kFewPairs;
-  bool early_stop = fast_scan && !few_pairs && P > kLeadProbes && P <= 8192 &&
+  bool early_stop = (fast_scan || generic_subset) && !few_pairs && P > kLeadProbes && P <= 8192 &&
                     detail::scan_screen_supported(sa) && res.tuning.early_stop != 1;
   // nibble codes: the leading and the surviving pairs go to the wave-per-pair kernel
   if (sa.pq_bits == 4 && !detail::scan_nibble_pack_supported(sa)) { early_stop = false; }
@@ -543,6 +546,12 @@ void search(cuvs::resources const& res_c,
     if (early_stop) {
       // 1. the leading probes' lists in full: candidates and a first bound per query
       auto full_scan = [&] {
+        if (generic_subset) {
+          sa.subset = 1;
+          detail::launch_scan(sa, s);
+          sa.subset = 0;
+          return true;
+        }
         return quad_kpp != 0                       ? detail::launch_scan_stream(sa, s)
                : sa.pq_bits == 4                     ? detail::launch_scan_nibble_pack(sa, s)
                : detail::scan_direct_supported(sa) ? detail::launch_scan_direct(sa, s)
