@@ -613,6 +613,39 @@ def test_early_stop_with_fp32_tables(orc, dim, pq_dim):
         assert torch.equal(nb, nb2) and torch.equal(d, d2)
 
 
+@pytest.mark.parametrize("lut,internal", [(R_32F, R_32F), (R_16F, R_32F), (R_8U, R_16F)])
+@pytest.mark.parametrize("dim,pq_dim,kind", [(256, 128, "subspace"), (192, 96, "subspace"), (384, 96, "cluster")])
+def test_early_stop_with_more_than_64_subspaces(orc, lut, internal, dim, pq_dim, kind):
+    """Byte codes of a shape no specialised kernel takes (pq_dim 128, 96; pq_len 2, 4; both codebook
+    kinds): the generic kernel scans the leading and the surviving pairs of the early stop as a
+    subset of the pairs.  Same results as the oracle and as its single launch over all pairs."""
+    import datasets as testing
+    from cuvs_amd.resources import Resources
+    allrows = testing.gaussian_mixture(16200, dim, 48, 0.15, seed=82).numpy()
+    x, q = allrows[:16000], allrows[16000:]
+    model = H.train(x, 80, pq_dim, 8, codebook_kind=kind, iters=5)
+    index = G.build_gpu_index(model, x, pq_dim, 8, "sqeuclidean", kind)
+    ix, _ = G.read_back(orc, index, model, dim, pq_dim, 8, "sqeuclidean", kind)
+    res = Resources()
+    res.enable_profiling(True)
+    sp = ivf_pq.SearchParams(n_probes=24, lut_dtype=lut, internal_distance_dtype=internal)
+    for k in (10, 100):
+        d, nb = ivf_pq.search(sp, index, G.to_dev(q), k, resources=res)
+        res.sync()
+        prof = ivf_pq.get_search_profile(res)
+        assert prof["n_screened_pairs"] == q.shape[0] * 23
+        assert 0 < prof["n_surviving_pairs"] < prof["n_screened_pairs"]
+        want_nb, want_d = orc.search(ix, q, k, 24, lut_dtype=ORC_DT[lut], internal_distance_dtype=ORC_DT[internal])
+        H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 1e-5 if lut == R_32F else 2e-3,
+                          exact=True)
+        res.set_search_tuning(early_stop="off")
+        d2, nb2 = ivf_pq.search(sp, index, G.to_dev(q), k, resources=res)
+        res.sync()
+        assert ivf_pq.get_search_profile(res)["n_screened_pairs"] == 0
+        res.set_search_tuning(early_stop="auto")
+        assert torch.equal(nb, nb2) and torch.equal(d, d2)
+
+
 def test_early_stop_with_filter_and_small_lists(orc):
     """A filter can leave the leading list with fewer than k rows (no bound: nothing is dropped),
     and the screen ignores the filter (it may keep a pair whose rows in play are all filtered)."""
