@@ -819,6 +819,16 @@ __global__ __launch_bounds__(kOrderThreads) void pair_bucket_finish_kernel(
 
 constexpr uint32_t kCandCap = 1024;  // per-block candidate buffer (keys), >= k + kBlock
 
+/** One wave keeps the k smallest of the n <= kCandCap keys of the block's buffer at its front (in no
+ *  particular order) by radix selection on its registers; returns the k-th smallest's high word. */
+__device__ __forceinline__ uint32_t keep_smallest_keys(unsigned long long* cand, uint32_t lane, uint32_t n, uint32_t k)
+{
+  auto* buf = (LDS_AS unsigned long long*)cand;
+  return n <= 256u ? wave_select_keys<4>(buf, lane, n, k)
+         : n <= 512u ? wave_select_keys<8>(buf, lane, n, k)
+                     : wave_select_keys<16>(buf, lane, n, k);
+}
+
 struct scan_smem_tail {
   uint32_t count;
   uint32_t thr;
@@ -997,13 +1007,13 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(scan_args a)
       const uint32_t cnt = tail->count;
       __syncthreads();  // every thread has read the count before anyone appends again
       if (cnt > kCandCap - kBlock) {
-        // prune: keep the k smallest candidates, tighten the threshold
-        for (uint32_t t = cnt + tid; t < kCandCap; t += kBlock) { cand[t] = kInvalidKey; }
-        __syncthreads();
-        block_bitonic_sort(cand, kCandCap);
-        if (tid == 0) {
-          tail->count = cnt < a.k ? cnt : a.k;
-          if (cnt >= a.k) { tail->thr = uint32_t(cand[a.k - 1] >> 32); }
+        // prune: keep the k smallest candidates (k <= kCandCap - kBlock < cnt), tighten the threshold
+        if (tid < 64u) {
+          const uint32_t kth = keep_smallest_keys(cand, tid, cnt, a.k);
+          if (tid == 0) {
+            tail->count = a.k;
+            tail->thr   = kth;
+          }
         }
         __syncthreads();
         const uint32_t t2 = tail->thr;
@@ -1021,13 +1031,12 @@ __global__ __launch_bounds__(kBlock) void scan_kernel(scan_args a)
     __syncthreads();
     uint32_t cnt = tail->count;
     if (cnt >= a.k) {
-      uint32_t n2 = 1;
-      while (n2 < cnt) { n2 <<= 1; }
-      for (uint32_t t = cnt + tid; t < n2; t += kBlock) { cand[t] = kInvalidKey; }
+      if (tid < 64u) {
+        const uint32_t kth = keep_smallest_keys(cand, tid, cnt, a.k);
+        if (tid == 0) { atomicMin(&a.query_kth[q], kth); }
+      }
       __syncthreads();
-      block_bitonic_sort(cand, n2);
       cnt = a.k;
-      if (tid == 0) { atomicMin(&a.query_kth[q], uint32_t(cand[a.k - 1] >> 32)); }
     }
     unsigned long long* out = a.out_keys + (uint64_t(q) * a.n_probes + p) * a.k;
     for (uint32_t r = tid; r < a.k; r += kBlock) { out[r] = r < cnt ? cand[r] : kInvalidKey; }
