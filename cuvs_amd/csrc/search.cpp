@@ -433,7 +433,10 @@ void search(cuvs::resources const& res_c,
   const uint32_t kpp       = quad_kpp != 0 ? quad_kpp : k;  // candidate keys stored per pair
   // byte codes of a shape no specialised kernel takes (pq_dim beyond 64): the generic kernel scans
   // the leading and the surviving pairs of an early stop as a subset of the pairs
-  const bool generic_subset = !generic_only && !fast_scan && sa.pq_bits == 8 && sa.fused;
+  // (also nibble codes outside the wave-per-pair kernel's shapes)
+  const bool generic_subset = !generic_only && sa.fused &&
+                              ((!fast_scan && (sa.pq_bits == 8 || sa.pq_bits == 4)) ||
+                               (sa.pq_bits == 4 && !detail::scan_nibble_pack_supported(sa)));
   if (fast_scan || generic_subset) {
     desc = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));
   }
@@ -445,8 +448,6 @@ void search(cuvs::resources const& res_c,
   const bool few_pairs       = uint64_t(Qb) * P <= kFewPairs;
   bool early_stop = (fast_scan || generic_subset) && !few_pairs && P > kLeadProbes && P <= 8192 &&
                     detail::scan_screen_supported(sa) && res.tuning.early_stop != 1;
-  // nibble codes: the leading and the surviving pairs go to the wave-per-pair kernel
-  if (sa.pq_bits == 4 && !detail::scan_nibble_pack_supported(sa)) { early_stop = false; }
   // In the automatic mode the index remembers whether the screen pays on its data: where it kept
   // most pairs the last time it ran with these parameters, this search scans plainly.
   bool observe_screen = false;
