@@ -515,12 +515,13 @@ def test_early_stop_pq_len_4(orc, kind):
 
 
 @pytest.mark.parametrize("lut,internal", [(R_16F, R_32F), (R_8U, R_32F), (R_16F, R_16F), (R_8U, R_16F)])
-@pytest.mark.parametrize("dim,pq_dim", [(128, 64), (128, 128), (256, 64), (192, 192)])
+@pytest.mark.parametrize("dim,pq_dim", [(128, 64), (128, 128), (256, 64), (192, 192), (64, 32)])
 def test_early_stop_with_four_bit_codes(orc, lut, internal, dim, pq_dim):
     """4-bit codes, L2: the leading pairs and the survivors of the screen go to the wave-per-pair
     kernel, the screen sums the 16 subspaces of the leading 8 code bytes (pq_len 2, 1, 4, 1; one,
-    two, one and three steps of 64 subspaces a row).  Same results as the oracle and as the single
-    launch."""
+    two, one and three steps of 64 subspaces a row).  Outside that kernel's shapes (pq_dim 32; k
+    above 64) the generic kernel scans those pairs as a subset.  Same results as the oracle and as
+    the single launch."""
     import datasets as testing
     from cuvs_amd.resources import Resources
     allrows = testing.gaussian_mixture(24200, dim, 64, 0.15, seed=79).numpy()
@@ -531,12 +532,12 @@ def test_early_stop_with_four_bit_codes(orc, lut, internal, dim, pq_dim):
     res = Resources()
     res.enable_profiling(True)
     sp = ivf_pq.SearchParams(n_probes=40, lut_dtype=lut, internal_distance_dtype=internal)
-    for k in (1, 10, 64):
+    for k in (1, 10, 64, 100):
         d, nb = ivf_pq.search(sp, index, G.to_dev(q), k, resources=res)
         res.sync()
         prof = ivf_pq.get_search_profile(res)
         assert prof["n_screened_pairs"] == q.shape[0] * 39
-        assert 0 < prof["n_surviving_pairs"] < prof["n_screened_pairs"]
+        assert 0 < prof["n_surviving_pairs"] <= prof["n_screened_pairs"]
         want_nb, want_d = orc.search(ix, q, k, 40, lut_dtype=ORC_DT[lut], internal_distance_dtype=ORC_DT[internal])
         H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
         res.set_search_tuning(early_stop="off")
