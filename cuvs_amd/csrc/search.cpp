@@ -434,7 +434,8 @@ void search(cuvs::resources const& res_c,
   // byte codes of a shape no specialised kernel takes (pq_dim beyond 64): the generic kernel scans
   // the leading and the surviving pairs of an early stop as a subset of the pairs
   // (also nibble codes outside the wave-per-pair kernel's shapes)
-  const bool generic_subset = !generic_only && sa.fused &&
+  // (a table in global memory included: the generic kernel's bounded grid walks the subset as well)
+  const bool generic_subset = !res.tuning.generic_scan && sa.fused &&
                               ((!fast_scan && (sa.pq_bits == 8 || sa.pq_bits == 4)) ||
                                (sa.pq_bits == 4 && !detail::scan_nibble_pack_supported(sa)));
   if (fast_scan || generic_subset) {
@@ -458,7 +459,10 @@ void search(cuvs::resources const& res_c,
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     CUVS_HIP_TRY(hipStreamIsCapturing(s, &capture));
     if (capture == hipStreamCaptureStatusNone) { fb.collect(); }
-    if (fb.off && fb.probes == P && fb.k == k) {
+    // (The generic kernel keeps the three launches even then: what the leading pairs give it is a
+    // bound from its first row on, which its exits after every chunk of a long row live on; the
+    // screen is a small fraction of its time.)
+    if (fb.off && fb.probes == P && fb.k == k && !generic_subset) {
       fb.plain_searches += 1;
       if (fb.plain_searches % detail::screen_feedback::kScreenRecheck != 0) { early_stop = false; }
     }
