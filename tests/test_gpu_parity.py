@@ -647,6 +647,31 @@ def test_early_stop_with_more_than_64_subspaces(orc, lut, internal, dim, pq_dim,
         assert torch.equal(nb, nb2) and torch.equal(d, d2)
 
 
+def test_early_stop_with_the_table_in_global_memory(orc):
+    """768 dimensions at pq_dim 384: an fp16 table of 196 KB does not fit LDS and lives in global
+    memory; the generic kernel still scans the leading and the surviving pairs as a subset."""
+    import datasets as testing
+    from cuvs_amd.resources import Resources
+    allrows = testing.gaussian_mixture(12150, 768, 32, 0.15, seed=83).numpy()
+    x, q = allrows[:12000], allrows[12000:]
+    model = H.train(x, 40, 384, 8, iters=4)
+    index = G.build_gpu_index(model, x, 384, 8, "sqeuclidean", "subspace")
+    ix, _ = G.read_back(orc, index, model, 768, 384, 8, "sqeuclidean", "subspace")
+    res = Resources()
+    res.enable_profiling(True)
+    sp = ivf_pq.SearchParams(n_probes=12, lut_dtype=R_16F)
+    d, nb = ivf_pq.search(sp, index, G.to_dev(q), 10, resources=res)
+    res.sync()
+    assert ivf_pq.get_search_profile(res)["n_screened_pairs"] == q.shape[0] * 11
+    want_nb, want_d = orc.search(ix, q, 10, 12, lut_dtype=ORC_DT[R_16F])
+    H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
+    res.set_search_tuning(early_stop="off")
+    d2, nb2 = ivf_pq.search(sp, index, G.to_dev(q), 10, resources=res)
+    res.sync()
+    assert ivf_pq.get_search_profile(res)["n_screened_pairs"] == 0
+    assert torch.equal(nb, nb2) and torch.equal(d, d2)
+
+
 def test_early_stop_with_filter_and_small_lists(orc):
     """A filter can leave the leading list with fewer than k rows (no bound: nothing is dropped),
     and the screen ignores the filter (it may keep a pair whose rows in play are all filtered)."""
