@@ -242,16 +242,10 @@ def main():
     mean = lambda pr, f: float(np.mean([p[f] for p in pr]))
     scan_bytes = float(stage["scan_bytes"])  # all probed lists in full, summed on the device from the probe lists
     early_stop = stage["n_screened_pairs"] > 0
-    pq_len = dim // pq_dim
-    nibble = pq_bits == 4 and pq_dim % 32 == 0 and pq_len in (1, 2, 4) and (pq_dim // 16) * pq_len <= 48
-    fused = k <= 256  # beyond that every score is stored and selected afterwards (generic kernel)
-    full_name = ("scan_kernel" if not fused
-                 else "scan_nibble_pack_kernel" if (nibble and pq_dim <= 512 and k <= 64 and args.lut != "f32"
-                                                    and pq_dim % (128 if args.metric in ("inner_product", "cosine")
-                                                                  else 64) == 0)
-                 else "scan_nibble_kernel" if nibble
-                 else "scan_kernel" if (pq_bits not in (5, 6, 7, 8) or (pq_dim, pq_len) not in ((64, 2), (48, 2), (32, 4), (32, 2)))
-                 else "scan_stream_kernel" if (args.lut != "f32" and k <= 128) else "scan_fast_kernel")
+    # the kernel that scans pairs in full, as the library reports it
+    KERNELS = {0: "scan_kernel", 1: "scan_stream_kernel", 2: "scan_fast_kernel", 3: "scan_direct_kernel",
+               4: "scan_nibble_kernel", 5: "scan_nibble_pack_kernel", 6: "scan_slab_kernel"}
+    full_name = KERNELS[stage["scan_kernel"]]
     if first_call_screened and not early_stop:
         log("the screen kept most pairs on the first search: it is off for the searches after it")
     default_path = {"early_stop": bool(early_stop), "screen_switched_itself_off": bool(first_call_screened and not early_stop),
@@ -291,6 +285,7 @@ def main():
         same_ids = bool((full_ids == gpu_ids).all()) if args.refine_ratio <= 1 else None
     else:
         full_ms_per_step, full_prof, same_ids = ms_per_step, prof, None
+    full_name = KERNELS[full_prof[-1]["scan_kernel"]]
     full_launches = max(full_prof[-1]["n_scan_launches"], 1)
     kernel_ms = mean(full_prof, "scan_ms") / full_launches
     kernel_bytes = float(full_prof[-1]["scan_bytes"]) / full_launches

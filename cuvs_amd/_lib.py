@@ -72,7 +72,7 @@ class SearchProfileStruct(C.Structure):
                 ("rotate_ms", C.c_float), ("scan_ms", C.c_float), ("merge_ms", C.c_float),
                 ("total_ms", C.c_float), ("scan_bytes", C.c_uint64), ("scan_rows", C.c_uint64),
                 ("lead_scan_ms", C.c_float), ("screen_ms", C.c_float),
-                ("survivor_scan_ms", C.c_float), ("reserved_", C.c_float),
+                ("survivor_scan_ms", C.c_float), ("scan_kernel", C.c_uint32),
                 ("lead_bytes", C.c_uint64), ("screen_bytes", C.c_uint64),
                 ("survivor_bytes", C.c_uint64), ("n_screened_pairs", C.c_uint64),
                 ("n_surviving_pairs", C.c_uint64)]

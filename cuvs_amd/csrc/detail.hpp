@@ -410,6 +410,10 @@ bool launch_scan_nibble_pack(const scan_args& a, hipStream_t stream);
  *  buffer must hold per (query, probe) pair, 0 when the arguments are outside what it covers. */
 uint32_t scan_stream_keys_per_pair(const scan_args& a);
 bool launch_scan_stream(const scan_args& a, hipStream_t stream);
+/** The same organisation with the table of a pair taken in slabs of 64 subspaces (scan_slab.cuh):
+ *  8-bit codes, pq_dim a multiple of 32, pq_len 1, 2, 3, 4 or 8, k <= 128, fp16 / 8-bit tables. */
+uint32_t scan_slab_keys_per_pair(const scan_args& a);
+bool launch_scan_slab(const scan_args& a, hipStream_t stream);
 
 /**
  * Early termination for L2 metrics, as compute_score's early stop in the reference

@@ -675,7 +675,7 @@ cuvsError_t cuvsAmdIvfPqGetSearchProfile(cuvsResources_t res, cuvsAmdIvfPqSearch
     profile->lead_scan_ms      = p.lead_scan_ms;
     profile->screen_ms         = p.screen_ms;
     profile->survivor_scan_ms  = p.survivor_scan_ms;
-    profile->reserved_         = 0;
+    profile->scan_kernel       = p.scan_kernel;
     profile->lead_bytes        = p.lead_bytes;
     profile->screen_bytes      = p.screen_bytes;
     profile->survivor_bytes    = p.survivor_bytes;

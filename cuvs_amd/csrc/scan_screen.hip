@@ -320,8 +320,16 @@ struct book_vec<2> {
   typedef float type __attribute__((ext_vector_type(2)));
 };
 template <>
+struct book_vec<3> {
+  typedef float type __attribute__((ext_vector_type(4)));  // the fourth component is not used
+};
+template <>
 struct book_vec<4> {
   typedef float type __attribute__((ext_vector_type(4)));
+};
+template <>
+struct book_vec<8> {
+  typedef float type __attribute__((ext_vector_type(8)));
 };
 
 template <int PQ_LEN, int LUT, bool OUT_HALF, int FIRST, int BITS>
@@ -343,7 +351,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   static_assert(FIRST <= 4 && FIRST <= MID, "the first subspaces' terms sit in scalar registers");
   auto* book      = reinterpret_cast<LDS_AS vec_t*>(uintptr_t(kScreenLdsBase));
   const float one = opaque_one_s();
-  constexpr uint32_t off_pending = kScreenLdsBase + SUB * BOOK * PQ_LEN * 4u;
+  constexpr uint32_t off_pending = kScreenLdsBase + SUB * BOOK * uint32_t(sizeof(vec_t));
   constexpr uint32_t off_mini    = off_pending + (kDirectThreads / 64u) * kSurvivorBatchBytes;
   constexpr uint32_t kMiniTiles  = 6;
 
@@ -355,7 +363,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   if (blockIdx.x * WPB >= n_pairs) { return; }
 
   for (uint32_t e = tid; e < SUB * BOOK; e += kDirectThreads) {
-    vec_t v;
+    vec_t v = {};
 #pragma unroll
     for (int t = 0; t < PQ_LEN; t++) { v[t] = a.pq_centers[((e / BOOK) * PQ_LEN + t) * BOOK + (e % BOOK)]; }
     book[e] = v;
@@ -567,7 +575,7 @@ void launch_screen_direct_first(const scan_args& a, const pair_desc* desc, uint3
   auto kernel       = scan_screen_direct_kernel<PQ_LEN, LUT, OUT_HALF, FIRST, BITS>;
   // codebooks of the leading subspaces (8 x 256 or 16 x 16 entries), a batch of survivors per wave,
   // and (byte codes) a wave's table of the first subspaces
-  const size_t smem = kScreenLdsBase + size_t(kDirectSubs) * (BITS == 8 ? 256 : 32) * PQ_LEN * 4 +
+  const size_t smem = kScreenLdsBase + size_t(kDirectSubs) * (BITS == 8 ? 256 : 32) * sizeof(typename book_vec<PQ_LEN>::type) +
                       size_t(kDirectThreads / 64u) * kSurvivorBatchBytes +
                       size_t(kDirectThreads / 64u) * FIRST * 256 * sizeof(typename lut_traits<LUT>::storage);
   // persistent blocks: exactly as many as are resident at once (per instance)
@@ -587,9 +595,11 @@ template <int PQ_LEN, int LUT, bool OUT_HALF>
 void launch_screen_direct(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
                           pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive, hipStream_t stream)
 {
-  if (a.pq_bits == 4) {
-    launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, 4, 4>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
-    return;
+  if constexpr (PQ_LEN == 1 || PQ_LEN == 2 || PQ_LEN == 4) {
+    if (a.pq_bits == 4) {
+      launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, 4, 4>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+      return;
+    }
   }
   launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, kScreenFirstCheck, 8>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
 }
@@ -670,7 +680,7 @@ bool scan_screen_supported(const scan_args& a)
     return !a.per_cluster && a.lead_plane != nullptr && a.lut_dtype != CUDA_R_32F &&
            (a.pq_len == 1 || a.pq_len == 2 || a.pq_len == 4);
   }
-  return a.pq_len == 2 || a.pq_len == 4;
+  return a.pq_len == 1 || a.pq_len == 2 || a.pq_len == 3 || a.pq_len == 4 || a.pq_len == 8;
 }
 
 void launch_scan_screen(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
@@ -679,20 +689,20 @@ void launch_scan_screen(const scan_args& a, const pair_desc* desc, uint32_t n_pa
 {
   CUVS_EXPECTS(scan_screen_supported(a), "the screening pass does not cover these search arguments");
   if (n_pairs == 0) { return; }
-  if (a.pq_len == 1) {
-    launch_screen_types<1, false>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
-  } else if (a.pq_len == 2) {
+  auto by_kind = [&](auto len) {
+    constexpr int PQ_LEN = decltype(len)::value;
     if (a.per_cluster) {
-      launch_screen_types<2, true>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+      launch_screen_types<PQ_LEN, true>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
     } else {
-      launch_screen_types<2, false>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+      launch_screen_types<PQ_LEN, false>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
     }
-  } else {
-    if (a.per_cluster) {
-      launch_screen_types<4, true>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
-    } else {
-      launch_screen_types<4, false>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
-    }
+  };
+  switch (a.pq_len) {
+    case 1: by_kind(std::integral_constant<int, 1>{}); break;
+    case 2: by_kind(std::integral_constant<int, 2>{}); break;
+    case 3: by_kind(std::integral_constant<int, 3>{}); break;
+    case 4: by_kind(std::integral_constant<int, 4>{}); break;
+    default: by_kind(std::integral_constant<int, 8>{}); break;
   }
 }
 

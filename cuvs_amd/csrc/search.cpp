@@ -379,13 +379,19 @@ void search(cuvs::resources const& res_c,
     w.pq_centers = ix.pq_centers8.as<float>();
     w.data_ptrs  = ix.data_ptrs8.as<const uint8_t*>();
     w.lead_plane = ix.lead_plane.bytes != 0 ? ix.lead_plane.as<uint64_t>() : nullptr;
-    if (detail::scan_lds_bytes(w) <= kMaxLds &&
-        (detail::scan_stream_keys_per_pair(w) != 0 || detail::scan_fast_supported(w))) {
+    if ((detail::scan_lds_bytes(w) <= kMaxLds &&
+         (detail::scan_stream_keys_per_pair(w) != 0 || detail::scan_fast_supported(w))) ||
+        detail::scan_slab_keys_per_pair(w) != 0) {
       sa = w;
     }
   }
+  // the CU-wide kernels: a pair's whole table in LDS for the shapes scan_stream.hip has, else (any
+  // pq_dim that is a multiple of 32) the table in slabs
+  sa.fused = pl.fused;
+  const uint32_t stream_kpp = res.tuning.generic_scan ? 0u : detail::scan_stream_keys_per_pair(sa);
+  const uint32_t slab_kpp   = res.tuning.generic_scan || stream_kpp != 0 ? 0u : detail::scan_slab_keys_per_pair(sa);
   // a table too large for LDS goes to global memory (8-bit codes, generic kernel)
-  const bool global_lut = detail::scan_lds_bytes(sa) > kMaxLds;
+  const bool global_lut = slab_kpp == 0 && detail::scan_lds_bytes(sa) > kMaxLds;
   if (global_lut) {
     CUVS_EXPECTS(sa.pq_bits == 8,
                  "the lookup table (pq_dim = %u, pq_bits = %u, lut_dtype = %d) needs %zu bytes of LDS, "
@@ -426,7 +432,7 @@ void search(cuvs::resources const& res_c,
   sa.fused                 = pl.fused;
   if (global_lut) { sa.global_lut = res.workspace_alloc(global_lut_bytes); }
   const bool generic_only  = res.tuning.generic_scan || global_lut;
-  const uint32_t quad_kpp  = generic_only ? 0u : detail::scan_stream_keys_per_pair(sa);
+  const uint32_t quad_kpp  = generic_only ? 0u : (stream_kpp != 0 ? stream_kpp : slab_kpp);
   const bool nibble_scan   = !generic_only && detail::scan_nibble_supported(sa);
   const bool fast_scan     = !generic_only && (quad_kpp != 0 || detail::scan_fast_supported(sa) || nibble_scan ||
                                                detail::scan_direct_supported(sa));
@@ -548,23 +554,42 @@ void search(cuvs::resources const& res_c,
     sa.desc        = desc;
     sa.n_pairs     = nq * P;
     sa.n_pairs_dev = nullptr;
+    // the kernel that scans pairs in full (the launchers return false for arguments they do not
+    // cover); which one it was goes into the profile
+    uint32_t scan_kernel_id = cuvs::scan_kernel_generic;
+    auto full_scan = [&](bool subset) {
+      if (subset && generic_subset) {
+        sa.subset = 1;
+        detail::launch_scan(sa, s);
+        sa.subset      = 0;
+        scan_kernel_id = cuvs::scan_kernel_generic;
+        return;
+      }
+      if (fast_scan) {
+        if (slab_kpp != 0) {
+          if (detail::launch_scan_slab(sa, s)) { scan_kernel_id = cuvs::scan_kernel_slab; return; }
+        } else if (quad_kpp != 0) {
+          if (detail::launch_scan_stream(sa, s)) { scan_kernel_id = cuvs::scan_kernel_stream; return; }
+        } else if (sa.pq_bits == 4) {
+          if (detail::launch_scan_nibble_pack(sa, s)) { scan_kernel_id = cuvs::scan_kernel_nibble_pack; return; }
+          if (!subset && detail::launch_scan_nibble(sa, s)) { scan_kernel_id = cuvs::scan_kernel_nibble; return; }
+        } else if (subset) {
+          if (detail::scan_direct_supported(sa) && detail::launch_scan_direct(sa, s)) { scan_kernel_id = cuvs::scan_kernel_direct; return; }
+          if (detail::launch_scan_fast(sa, s)) { scan_kernel_id = cuvs::scan_kernel_fast; return; }
+        } else {
+          if (detail::launch_scan_fast(sa, s)) { scan_kernel_id = cuvs::scan_kernel_fast; return; }
+          if (detail::launch_scan_direct(sa, s)) { scan_kernel_id = cuvs::scan_kernel_direct; return; }
+        }
+      }
+      CUVS_EXPECTS(!subset, "scan kernel launch failed");
+      detail::launch_scan(sa, s);
+      scan_kernel_id = cuvs::scan_kernel_generic;
+    };
     if (early_stop) {
       // 1. the leading probes' lists in full: candidates and a first bound per query
-      auto full_scan = [&] {
-        if (generic_subset) {
-          sa.subset = 1;
-          detail::launch_scan(sa, s);
-          sa.subset = 0;
-          return true;
-        }
-        return quad_kpp != 0                       ? detail::launch_scan_stream(sa, s)
-               : sa.pq_bits == 4                     ? detail::launch_scan_nibble_pack(sa, s)
-               : detail::scan_direct_supported(sa) ? detail::launch_scan_direct(sa, s)
-                                                     : detail::launch_scan_fast(sa, s);
-      };
       sa.n_pairs    = nq * lead;
       sa.rare_exits = 1;  // no bound yet here, and the screen's survivors mostly stay under theirs
-      CUVS_EXPECTS(full_scan(), "scan kernel launch failed");
+      full_scan(true);
       detail::launch_kth_bound(keys, nq, uint64_t(P) * kpp, lead * kpp, k, kth, s);
       mark(5);
       // 2. every other pair on its first chunk only
@@ -590,15 +615,11 @@ void search(cuvs::resources const& res_c,
       sa.desc        = survivors;
       sa.n_pairs     = 0;
       sa.n_pairs_dev = n_survivors;
-      CUVS_EXPECTS(full_scan(), "scan kernel launch failed");
+      full_scan(true);
     } else {
-      const bool launched = fast_scan && (quad_kpp != 0   ? detail::launch_scan_stream(sa, s)
-                                          : nibble_scan ? (detail::launch_scan_nibble_pack(sa, s) ||
-                                                           detail::launch_scan_nibble(sa, s))
-                                                        : (detail::launch_scan_fast(sa, s) ||
-                                                           detail::launch_scan_direct(sa, s)));
-      if (!launched) { detail::launch_scan(sa, s); }
+      full_scan(false);
     }
+    if (prof) { res.last_profile.scan_kernel = scan_kernel_id; }
     }
     mark(3);
 

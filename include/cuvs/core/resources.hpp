@@ -78,6 +78,17 @@ device_vector_view<T> make_device_vector_view(T* data, int64_t size)
 }
 
 /** Per-stage timing of a search (filled when profiling is enabled on the resources). */
+/** The kernel that scanned the pairs of a search in full (search_profile::scan_kernel). */
+enum scan_kernel_id : uint32_t {
+  scan_kernel_generic     = 0,
+  scan_kernel_stream      = 1,
+  scan_kernel_fast        = 2,
+  scan_kernel_direct      = 3,
+  scan_kernel_nibble      = 4,
+  scan_kernel_nibble_pack = 5,
+  scan_kernel_slab        = 6,
+};
+
 struct search_profile {
   uint32_t n_queries       = 0;
   uint32_t n_probes        = 0;
@@ -94,6 +105,7 @@ struct search_profile {
   float lead_scan_ms         = 0;
   float screen_ms            = 0;
   float survivor_scan_ms     = 0;
+  uint32_t scan_kernel       = 0;  // scan_kernel_id of the last batch
   uint64_t lead_bytes        = 0;
   uint64_t screen_bytes      = 0;
   uint64_t survivor_bytes    = 0;

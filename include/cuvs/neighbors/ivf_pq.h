@@ -257,7 +257,9 @@ typedef struct {
   float lead_scan_ms;      /* full scan of each query's leading probes + bound per query */
   float screen_ms;         /* first-chunk screening of all other pairs */
   float survivor_scan_ms;  /* full scan of the pairs the screen kept */
-  float reserved_;
+  uint32_t scan_kernel;    /* which kernel scanned pairs in full: 0 scan_kernel (generic), 1 scan_stream_kernel,
+                              2 scan_fast_kernel, 3 scan_direct_kernel, 4 scan_nibble_kernel,
+                              5 scan_nibble_pack_kernel, 6 scan_slab_kernel */
   uint64_t lead_bytes;     /* scan_bytes share of the leading pairs */
   uint64_t screen_bytes;   /* sum over screened pairs of round_up(list size, 32) * bytes read per row (8) */
   uint64_t survivor_bytes; /* scan_bytes share of the pairs the screen kept */
