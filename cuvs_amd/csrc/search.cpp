@@ -465,10 +465,11 @@ void search(cuvs::resources const& res_c,
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     CUVS_HIP_TRY(hipStreamIsCapturing(s, &capture));
     if (capture == hipStreamCaptureStatusNone) { fb.collect(); }
-    // (The generic kernel keeps the three launches even then: what the leading pairs give it is a
-    // bound from its first row on, which its exits after every chunk of a long row live on; the
-    // screen is a small fraction of its time.)
-    if (fb.off && fb.probes == P && fb.k == k && !generic_subset) {
+    // (The generic kernel and the slab kernel on rows of several slabs keep the three launches even
+    // then: what the leading pairs give them is a bound from a pair's first row on, which their
+    // exits inside a long row live on; the screen of 8 bytes a row is a small fraction of their time.)
+    const bool long_rows = slab_kpp != 0 && sa.pq_dim > 64;
+    if (fb.off && fb.probes == P && fb.k == k && !generic_subset && !long_rows) {
       fb.plain_searches += 1;
       if (fb.plain_searches % detail::screen_feedback::kScreenRecheck != 0) { early_stop = false; }
     }

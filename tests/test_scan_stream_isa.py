@@ -1,4 +1,4 @@
-"""The table lookups of scan_stream.hip and scan_nibble_pack.hip are issued and waited for in
+"""The table lookups of scan_stream.hip, scan_slab_len*.hip and scan_nibble_pack.hip are issued and waited for in
 inline assembly, so that the adds of one group overlap the reads of the next.  From the compiler's
 point of view a read's destination register holds its value as soon as the read is issued; nothing
 stops it from copying or reusing that register before the data has arrived.  Both files therefore
@@ -15,7 +15,8 @@ import subprocess
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-SOURCES = {"scan_stream.hip": 48 * 32, "scan_nibble_pack.hip": 128 * 24}  # file: inline reads at least expected
+# file: inline reads at least expected
+SOURCES = {"scan_stream.hip": 48 * 32, "scan_nibble_pack.hip": 128 * 24, "scan_slab_len2.hip": 64 * 32 * 4}
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 
