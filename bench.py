@@ -96,6 +96,9 @@ def main():
                     help="fix the library's choice of the L2 early stop for the whole run (profiling runs)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-sweep", action="store_true",
+                    help="skip the `sweep` entries (other search parameters and workloads, 5 steps each) that the "
+                         "default run appends to its JSON line")
     ap.add_argument("--with-cpu", action="store_true", help="time the CPU oracle also with --config")
     ap.add_argument("--config", type=int, default=2, choices=sorted(CONFIGS))
     ap.add_argument("--metric", default="sqeuclidean", choices=["sqeuclidean", "euclidean", "inner_product", "cosine"])
@@ -351,7 +354,123 @@ def main():
                                            pq_bits, P, k, log)
         out["config"]["oracle_recall_on_sample"] = out["cpu_baseline"].pop("oracle_recall")
         out["config"]["gpu_recall_on_sample"] = out["cpu_baseline"].pop("gpu_recall")
+    default_run = args.config == 2 and (n, dim, pq_dim, pq_bits, nq, n_lists, P, k) == (
+        10_000_000, 128, 64, 8, 10_000, 16384, 64, 10) and args.refine_ratio <= 1
+    if default_run and not args.no_sweep:
+        out["sweep"] = sweep(args, res, index, data, queries, log)
     print(json.dumps(out), flush=True)
+
+
+def measure_variant(res, index, queries, truth, k, P, lut, internal, steps, warmup, workload):
+    """One sweep entry: the default path's time per batch and recall, and the code-scan kernel of
+    the same batch with the early stop off (every probed list streamed in full) against the HBM
+    peak, as `roofline` does for the headline."""
+    import numpy as np
+    import torch
+
+    import datasets as testing
+    from cuvs_amd import ivf_pq
+
+    lut_np = {"f32": np.float32, "f16": np.float16, "fp8": np.uint8}[lut]
+    int_np = {"f32": np.float32, "f16": np.float16}[internal]
+    nq = queries.shape[0]
+    sp = ivf_pq.SearchParams(n_probes=P, lut_dtype=lut_np, internal_distance_dtype=int_np,
+                             max_internal_batch_size=max(nq, 1))
+    neighbors = torch.empty((nq, k), dtype=torch.int64, device="cuda")
+    distances = torch.empty((nq, k), dtype=torch.float32, device="cuda")
+
+    def step():
+        ivf_pq.search(sp, index, queries, k, neighbors=neighbors, distances=distances, resources=res)
+
+    def timed():
+        for _ in range(warmup):
+            step()
+        res.sync()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        res.sync()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
+    res.set_search_tuning(early_stop="auto")
+    step()  # the first search with new parameters is the one the screen's feedback observes
+    res.sync()
+    ms = timed()
+    ids = neighbors.cpu().numpy().copy()
+    res.enable_profiling(True)
+    step()
+    default_prof = ivf_pq.get_search_profile(res)
+    res.set_search_tuning(early_stop="off")
+    prof = []
+    for _ in range(steps):
+        step()
+        prof.append(ivf_pq.get_search_profile(res))
+    res.enable_profiling(False)
+    res.set_search_tuning(early_stop="auto")
+    same = bool((neighbors.cpu().numpy() == ids).all())
+    launches = max(prof[-1]["n_scan_launches"], 1)
+    kernel_ms = float(np.mean([p_["scan_ms"] for p_ in prof])) / launches
+    kernel_bytes = float(prof[-1]["scan_bytes"]) / launches
+    achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9
+    kernels = {0: "scan_kernel", 1: "scan_stream_kernel", 2: "scan_fast_kernel", 3: "scan_direct_kernel",
+               4: "scan_nibble_kernel", 5: "scan_nibble_pack_kernel", 6: "scan_slab_kernel"}
+    return {"workload": workload, "ms_per_step": ms, "qps": nq / ms * 1e3,
+            "recall": testing.recall(ids, truth), "early_stop_on_default_path": default_prof["n_screened_pairs"] > 0,
+            "kernel": kernels[prof[-1]["scan_kernel"]], "kernel_ms": kernel_ms,
+            "algorithmic_bytes": kernel_bytes, "achieved_GBs": achieved, "frac": achieved / HBM_PEAK_GBS,
+            "ids_identical_to_default_path": same}
+
+
+def sweep(args, res, index, data, queries, log):
+    """Other search parameters on the headline index, and two other workloads, 5 steps each: the
+    figures that do not depend on how well the headline rows cluster."""
+    import torch
+
+    import datasets as testing
+    from cuvs_amd import ivf_pq
+
+    steps, warmup = 5, 2
+    entries = []
+
+    def add(res_, index_, queries_, truth_, k, P, lut, internal, workload):
+        e = measure_variant(res_, index_, queries_, truth_, k, P, lut, internal, steps, warmup, workload)
+        log(f"sweep: {workload}: {e['ms_per_step']:.2f} ms per batch, recall {e['recall']:.4f}; {e['kernel']} "
+            f"{e['kernel_ms']:.3f} ms for {e['algorithmic_bytes'] / 1e9:.2f} GB = {e['frac']:.3f} of HBM peak")
+        entries.append(e)
+
+    truth10 = testing.exact_knn(data, queries, 10, metric=args.metric).cpu().numpy()
+    truth100 = testing.exact_knn(data, queries, 100, metric=args.metric).cpu().numpy()
+    head = "configs[2] (10M x 128 u8, 16384 lists, pq_dim 64)"
+    add(res, index, queries, truth10, 10, 64, "fp8", "f32", head + ", k=10, n_probes=64, fp8 table")
+    add(res, index, queries, truth100, 100, 64, "f16", "f32", head + ", k=100, n_probes=64, fp16 table")
+    add(res, index, queries, truth10, 10, 128, "f16", "f32", head + ", k=10, n_probes=128, fp16 table")
+    add(res, index, queries, truth10, 10, 64, "f32", "f32",
+        head + ", k=10, n_probes=64, fp32 table (the reference's default lut_dtype)")
+
+    def other(dataset, rows, dim, lists, pq_dim, P, lut, workload):
+        nq = queries.shape[0]
+        allrows = make_rows(dataset, rows + nq, dim, "cuda")
+        x, q = allrows[:rows], allrows[rows:].contiguous()
+        params = ivf_pq.IndexParams(n_lists=lists, metric="sqeuclidean", pq_bits=8, pq_dim=pq_dim,
+                                    kmeans_trainset_fraction=min(1.0, max(lists * 32, 200_000) / rows))
+        ix = ivf_pq.build(params, x, resources=res)
+        res.sync()
+        truth = testing.exact_knn(x, q, 10, metric="sqeuclidean").cpu().numpy()
+        add(res, ix, q, truth, 10, P, lut, "f32", workload)
+        del ix, x, q, allrows
+        torch.cuda.empty_cache()
+
+    other("unit_mixture_f32", 1_000_000, 96, 1024, 48, 32, "f16",
+          "configs[1] (1M x 96 f32 unit vectors, 1024 lists, pq_dim 48), k=10, n_probes=32, fp16 table")
+    other("sift_u8", 2_000_000, 256, 2048, 128, 32, "f16",
+          "2M x 256 u8 (sift_u8), 2048 lists, pq_dim 128 (the reference's default pq_dim for 256 dimensions), "
+          "k=10, n_probes=32, fp16 table")
+    other("sift_u8", 1_000_000, 768, 1024, 384, 32, "f16",
+          "1M x 768 u8 (sift_u8), 1024 lists, pq_dim 384 (the reference's default pq_dim for 768 dimensions), "
+          "k=10, n_probes=32, fp16 table")
+    return entries
 
 
 def cpu_baseline(args, index, model, queries, truth, gpu_ids, dim, pq_dim, pq_bits, P, k, log):

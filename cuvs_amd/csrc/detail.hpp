@@ -10,6 +10,7 @@
 
 #include "memory.hpp"
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -122,9 +123,17 @@ struct screen_feedback {
   bool pending      = false;
   uint64_t pending_pairs  = 0;  // pairs that search screened
   uint32_t pending_probes = 0, pending_k = 0;
-  bool off          = false;    // verdict, for searches with these parameters:
-  uint32_t probes = 0, k = 0;
-  uint32_t plain_searches = 0;  // since the verdict
+  /** Verdicts by (n_probes, k), the most recently used first: callers that alternate between a few
+   *  parameter sets each keep theirs. */
+  struct verdict {
+    uint32_t probes = 0, k = 0;    // 0: unused entry
+    bool off                = false;
+    uint32_t plain_searches = 0;   // since the verdict
+  };
+  static constexpr int kVerdicts = 8;
+  verdict verdicts[kVerdicts];
+  /** The entry of (probes, k), moved to the front; null when there is none. */
+  verdict* find(uint32_t probes, uint32_t k);
   /** The pinned word and the event (allocates; called when an index is made, never by a search). */
   void create();
   /** Folds in an observation that has landed.  Call with `mu` held. */
@@ -136,6 +145,10 @@ struct screen_feedback {
 };
 
 struct index_impl {
+  index_impl();
+  ~index_impl();
+  index_impl(const index_impl&)            = delete;
+  index_impl& operator=(const index_impl&) = delete;
   DistanceType metric        = DistanceType::L2Expanded;
   codebook_gen codebook_kind = codebook_gen::PER_SUBSPACE;
   bool conservative_memory_allocation = false;
@@ -191,7 +204,16 @@ struct index_impl {
   /** Refill `lead_plane` and the byte-wide copy of narrower codes from the codes arena (after the
    *  arena's contents changed). */
   void rebuild_lead_plane(hipStream_t stream);
+  /** Set when list memory was written through a bare pointer (codepacker::pack on a buffer of this
+   *  index): what the index derives from its lists is then refreshed by the next search, under
+   *  `derived_mu`. */
+  mutable std::atomic<bool> derived_stale{false};
+  mutable std::mutex derived_mu;
 };
+
+/** Tells the index whose codes arena holds `list_data` (if any) that its lists were written behind
+ *  its back. */
+void mark_lists_written(const void* list_data);
 
 void init_index(index_impl& ix, const index_params& params, uint32_t dim);
 

@@ -139,6 +139,7 @@ void pack(cuvs::resources const& res, device_matrix_view<const uint8_t> codes, u
   if (codes.extent(0) == 0) { return; }
   detail::launch_pack_codes(list_data, codes.data_handle(), false, uint32_t(codes.extent(0)), offset,
                             uint32_t(codes.extent(1)), pq_bits, res.stream());
+  detail::mark_lists_written(list_data);
 }
 
 void unpack_contiguous(cuvs::resources const& res, const uint8_t* list_data, uint32_t pq_bits, uint32_t offset,
@@ -159,6 +160,7 @@ void pack_contiguous(cuvs::resources const& res, const uint8_t* codes, uint32_t 
   if (n_rows == 0) { return; }
   CUVS_EXPECTS(list_data != nullptr && codes != nullptr, "list_data and codes must not be null");
   detail::launch_pack_codes(list_data, codes, true, n_rows, offset, pq_dim, pq_bits, res.stream());
+  detail::mark_lists_written(list_data);
 }
 
 void unpack_list_data(cuvs::resources const& res, const index<int64_t>& idx,

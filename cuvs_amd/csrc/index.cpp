@@ -14,6 +14,43 @@ namespace cuvs::neighbors::ivf_pq {
 
 namespace detail {
 
+/* Every live index, so that a write through a bare list pointer finds the index it belongs to. */
+namespace {
+std::mutex& registry_mutex()
+{
+  static std::mutex m;
+  return m;
+}
+std::vector<index_impl*>& registry()
+{
+  static std::vector<index_impl*> all;
+  return all;
+}
+}  // namespace
+
+index_impl::index_impl()
+{
+  std::lock_guard<std::mutex> guard(registry_mutex());
+  registry().push_back(this);
+}
+
+index_impl::~index_impl()
+{
+  std::lock_guard<std::mutex> guard(registry_mutex());
+  auto& all = registry();
+  all.erase(std::remove(all.begin(), all.end(), this), all.end());
+}
+
+void mark_lists_written(const void* list_data)
+{
+  const auto p = reinterpret_cast<uintptr_t>(list_data);
+  std::lock_guard<std::mutex> guard(registry_mutex());
+  for (index_impl* ix : registry()) {
+    const auto begin = reinterpret_cast<uintptr_t>(ix->codes_arena.ptr);
+    if (begin != 0 && p >= begin && p < begin + ix->codes_arena.bytes) { ix->derived_stale.store(true); }
+  }
+}
+
 void screen_feedback::create()
 {
   if (host != nullptr) { return; }
@@ -27,10 +64,29 @@ void screen_feedback::collect()
   if (!pending || hipEventQuery(landed) != hipSuccess) { return; }
   pending = false;
   if (pending_pairs == 0) { return; }
-  off            = double(host[0]) > kKeepLimit * double(pending_pairs);
-  probes         = pending_probes;
-  k              = pending_k;
-  plain_searches = 0;
+  verdict* v = find(pending_probes, pending_k);
+  if (v == nullptr) {
+    // a new parameter set takes the place of the one used longest ago
+    for (int i = kVerdicts - 1; i > 0; i--) { verdicts[i] = verdicts[i - 1]; }
+    v         = &verdicts[0];
+    v->probes = pending_probes;
+    v->k      = pending_k;
+  }
+  v->off            = double(host[0]) > kKeepLimit * double(pending_pairs);
+  v->plain_searches = 0;
+}
+
+screen_feedback::verdict* screen_feedback::find(uint32_t probes, uint32_t k)
+{
+  for (int i = 0; i < kVerdicts; i++) {
+    if (verdicts[i].probes == probes && verdicts[i].k == k && probes != 0) {
+      const verdict hit = verdicts[i];
+      for (int j = i; j > 0; j--) { verdicts[j] = verdicts[j - 1]; }
+      verdicts[0] = hit;
+      return &verdicts[0];
+    }
+  }
+  return nullptr;
 }
 
 screen_feedback::~screen_feedback()
@@ -150,6 +206,7 @@ void index_impl::refresh_coarse(hipStream_t stream)
 
 void index_impl::rebuild_lead_plane(hipStream_t stream)
 {
+  derived_stale.store(false);  // whatever was written so far is seen by the kernels below
   const uint64_t n_slots = h_row_offsets.empty() ? 0 : h_row_offsets[n_lists];
   // narrower codes, a byte each
   const bool widen = pq_bits >= 5 && pq_bits < 8 && n_slots != 0 && !conservative_memory_allocation;

@@ -116,6 +116,10 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
   }
   // keep the pair count of a batch within uint32 indexing
   while (b > 1 && b * P >= (size_t(1) << 31)) { b /= 2; }
+  // batches of equal size: 10,000 queries at a limit of 4096 run as 3 x 3334, not 4096 + 4096 + 1808
+  // (a short last batch leaves most of the persistent grids' last round idle)
+  const size_t n_batches = (size_t(n_queries) + b - 1) / b;
+  b                      = (size_t(n_queries) + n_batches - 1) / n_batches;
   p.batch = uint32_t(b);
   return p;
 }
@@ -342,6 +346,13 @@ void search(cuvs::resources const& res_c,
                  device_accessible(distances),
                "all pointers must be accessible from the device.");
 
+  if (ix.derived_stale.load()) {
+    // list memory was written through a bare pointer (codepacker::pack on one of the index's list
+    // buffers): the copies the kernels read instead of the lists follow before anything is searched
+    std::lock_guard<std::mutex> guard(ix.derived_mu);
+    if (ix.derived_stale.load()) { const_cast<index_impl&>(ix).rebuild_lead_plane(res.stream()); }
+  }
+
   const uint32_t k  = uint32_t(k64);
   cuvs::tracing::range search_scope("ivf_pq::search(n_queries = %u, n_probes = %u, k = %u, dim = %u)",
                                     uint32_t(n_queries), params.n_probes, k, ix.dim);
@@ -464,14 +475,22 @@ void search(cuvs::resources const& res_c,
     // while a stream captures, an event query invalidates the capture: the verdict stays as it is
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     CUVS_HIP_TRY(hipStreamIsCapturing(s, &capture));
-    if (capture == hipStreamCaptureStatusNone) { fb.collect(); }
+    // (another thread's capture in the global mode would be invalidated by the query as well: the
+    // query runs with this thread's capture mode relaxed)
+    if (capture == hipStreamCaptureStatusNone) {
+      hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+      CUVS_HIP_TRY(hipThreadExchangeStreamCaptureMode(&mode));
+      fb.collect();
+      CUVS_HIP_TRY(hipThreadExchangeStreamCaptureMode(&mode));
+    }
     // (The generic kernel and the slab kernel on rows of several slabs keep the three launches even
     // then: what the leading pairs give them is a bound from a pair's first row on, which their
     // exits inside a long row live on; the screen of 8 bytes a row is a small fraction of their time.)
     const bool long_rows = slab_kpp != 0 && sa.pq_dim > 64;
-    if (fb.off && fb.probes == P && fb.k == k && !generic_subset && !long_rows) {
-      fb.plain_searches += 1;
-      if (fb.plain_searches % detail::screen_feedback::kScreenRecheck != 0) { early_stop = false; }
+    auto* verdict = fb.find(P, k);
+    if (verdict != nullptr && verdict->off && !generic_subset && !long_rows) {
+      verdict->plain_searches += 1;
+      if (verdict->plain_searches % detail::screen_feedback::kScreenRecheck != 0) { early_stop = false; }
     }
     observe_screen = early_stop && capture == hipStreamCaptureStatusNone;
   }
@@ -601,7 +620,10 @@ void search(cuvs::resources const& res_c,
         observe_screen = false;
         auto& fb       = ix.feedback;
         std::lock_guard<std::mutex> guard(fb.mu);
+        hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+        CUVS_HIP_TRY(hipThreadExchangeStreamCaptureMode(&mode));
         fb.collect();
+        CUVS_HIP_TRY(hipThreadExchangeStreamCaptureMode(&mode));
         if (!fb.pending) {
           CUVS_HIP_TRY(hipMemcpyAsync(fb.host, n_survivors, 4, hipMemcpyDeviceToHost, s));
           CUVS_HIP_TRY(hipEventRecord(fb.landed, s));

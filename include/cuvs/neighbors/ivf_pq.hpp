@@ -279,8 +279,11 @@ void unpack(cuvs::resources const& res,
             device_matrix_view<uint8_t> codes);
 
 /** ivf_pq.hpp:2669 -- writes `codes` [n_rows, pq_dim], one code per byte, into the rows from
- *  `offset` on of a bare list buffer.  A buffer that belongs to an index is better written through
- *  pack_list_data, which also refreshes what the index derives from its lists. */
+ *  `offset` on of a bare list buffer.  The buffer may be one of an index's own lists
+ *  (`index::data_ptrs()[label]`): the index notices, and its next search first refreshes the copies
+ *  of leading and widened codes it keeps next to the lists (as pack_list_data does at once).  List
+ *  memory written by any other means (a kernel of the caller's) MUST be followed by
+ *  helpers::recompute_internal_state before the index is searched again. */
 void pack(cuvs::resources const& res,
           device_matrix_view<const uint8_t> codes,
           uint32_t pq_bits,
@@ -298,7 +301,7 @@ void unpack_contiguous(cuvs::resources const& res,
                        uint8_t* codes);
 
 /** ivf_pq.hpp:2705 -- writes `n_rows` bit strings of that form into the rows from `offset` on of a
- *  bare list buffer. */
+ *  bare list buffer (one of an index's own lists included, as for `pack`). */
 void pack_contiguous(cuvs::resources const& res,
                      const uint8_t* codes,
                      uint32_t n_rows,
@@ -427,7 +430,9 @@ void make_rotation_matrix(cuvs::resources const& res,
                           device_matrix_view<float> rotation_matrix,
                           bool force_random_rotation);
 
-/** ivf_pq.hpp:3265 -- rebuilds the tables derived from the list sizes and addresses. */
+/** ivf_pq.hpp:3265 -- rebuilds the tables derived from the list sizes and addresses, and the copies
+ *  of leading / widened codes the searches read: to be called after list memory was written
+ *  directly. */
 void recompute_internal_state(cuvs::resources const& res, index<int64_t>* idx);
 
 }  // namespace helpers
