@@ -10,10 +10,8 @@
  * is x >> 1 for uint8 and x for int8 elements), 1 - m in column `dim`, then -128 (L2) or 0 (inner
  * product, cosine).  The score is alpha times the integer dot product, alpha = -2 (L2) or -1.
  *
- * The reference pads the query rows to round_up(dim + 1, 8) columns and passes that as the leading
- * dimension of the centre matrix too, so its GEMM reads the centres at the wrong stride whenever
- * the two paddings differ; here both sides use the centres' padding, which is the scheme its
- * comments describe and the same arithmetic wherever the reference's is self-consistent.
+ * The query rows are padded to the same dim_ext_int8 columns: the reference's driver takes the row
+ * length of the int8 centre matrix as `dim_ext` for this mode (ivf_pq_search.cuh:929-931).
  *
  * Scores leave this file as floats whose order (as the selection kernels see it through
  * order_f32) is the order of the int32 scores, so that the probe selection is shared with the

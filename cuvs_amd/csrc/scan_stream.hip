@@ -7,10 +7,11 @@
  *
  *   - 8 of the 16 waves build lookup tables, the other 8 scan codes with them, at the same time:
  *     while the scanners work through the two (query, probe) pairs of iteration i, the builders
- *     make the two tables of iteration i + 1 in the other half of a double buffer.  One block
- *     barrier per iteration is the only synchronisation.  On every SIMD two waves of each kind
- *     share the issue slots, so the vector work of the table build fills the cycles in which the
- *     scanners wait for their LDS gathers and code loads;
+ *     compute the entries of the two tables of iteration i + 1 into registers, and write them into
+ *     the one set of tables between the two block barriers that end an iteration (LDS writes that
+ *     mix with the scanners' gathers cost several times what they cost alone).  On every SIMD two
+ *     waves of each kind share the issue slots, so the vector work of the table build fills the
+ *     cycles in which the scanners wait for their LDS gathers and code loads;
  *   - a builder thread owns two neighbouring codebook entries of a quarter of the subspaces and keeps
  *     those codebook components in registers for the whole kernel; the two table entries of a
  *     subspace go out as one 32-bit write (the scanners spend their registers on code

@@ -275,13 +275,9 @@ void coarse_scores_f16(const orc_index& ix, const float* qf, float* scores)
  * the columns past it -128 (L2) or 0 (inner product, cosine).  Scores are int32: alpha times the
  * dot product, alpha = -2 (L2) or -1.
  *
- * The reference lays the query rows out with dim_ext = round_up(dim + 1, 8) columns and hands the
- * centre matrix (dim_ext_int8 columns a row) to the GEMM with that same leading dimension, so
- * whenever the two paddings differ its GEMM reads the centre rows at the wrong stride; its own
- * test asks a recall of 0.1 of this variant (cpp/tests/neighbors/ann_ivf_pq.cuh:1040-1046).  This
- * restatement uses the centre matrix's padding on both sides, which is what the comment in
- * ivf_pq_index.cu describes and equals the reference's arithmetic where the paddings agree
- * (dim % 16 in 7..14).  Parity unpinned for the other dims. */
+ * Both operands have dim_ext_int8 columns in the reference as well: its driver takes the row
+ * length of the int8 centre matrix as `dim_ext` whenever coarse_search_dtype is CUDA_R_8I
+ * (ivf_pq_search.cuh:929-931), and select_clusters pads the query rows to it. */
 inline uint32_t dim_ext_int8_of(uint32_t dim) { return round_up(dim + 2, 16); }
 
 inline int8_t clamp_to_int8(float v)

@@ -243,20 +243,25 @@ void run(uint32_t pq_bits, ivf_pq::codebook_gen kind, uint32_t pq_dim_asked, con
   {
     // The same kind of edit through a bare pointer into the index's own list buffer: searches read
     // copies of the lists' leading codes (and of 5 - 7-bit codes a byte each), which have to follow.
-    auto ptrs = to_host(index.data_ptrs(), n_lists);
-    packer::pack(res, make_device_matrix_view<const uint8_t>(d_codes + 20 * pq_dim, 20, pq_dim), pq_bits, 0, const_cast<uint8_t*>(ptrs[label]));
+    // (every row of the list takes the codes of the row after it: the queries that are rows of this
+    // list find other neighbours then)
+    auto ptrs       = to_host(index.data_ptrs(), n_lists);
+    uint8_t* own    = const_cast<uint8_t*>(ptrs[label]);
+    packer::pack(res, make_device_matrix_view<const uint8_t>(d_codes + pq_dim, n - 1, pq_dim), pq_bits, 0, own);
+    packer::pack(res, make_device_matrix_view<const uint8_t>(d_codes, 1, pq_dim), pq_bits, n - 1, own);
     const auto bare = search_all(res, index, d_data, n_queries, k);
-    packer::pack_list_data(res, &index, make_device_matrix_view<const uint8_t>(d_codes, 20, pq_dim), label, 0);
+    packer::pack_list_data(res, &index, make_device_matrix_view<const uint8_t>(d_codes, n, pq_dim), label, 0);
     REQUIRE(snapshot(index, label).bytes == before.bytes);
-    packer::pack_list_data(res, &index, make_device_matrix_view<const uint8_t>(d_codes + 20 * pq_dim, 20, pq_dim), label, 0);
+    packer::pack_list_data(res, &index, make_device_matrix_view<const uint8_t>(d_codes + pq_dim, n - 1, pq_dim), label, 0);
+    packer::pack_list_data(res, &index, make_device_matrix_view<const uint8_t>(d_codes, 1, pq_dim), label, n - 1);
     const auto proper = search_all(res, index, d_data, n_queries, k);
     REQUIRE(bare.ids == proper.ids && bare.dist == proper.dist);
+    REQUIRE(!(proper.ids == before_search.ids && proper.dist == before_search.dist));  // the edit is visible at all
     // bit strings the same way, back to the original rows
-    packer::pack_contiguous(res, d_flat, 20, pq_dim, pq_bits, 0, const_cast<uint8_t*>(ptrs[label]));
+    packer::pack_contiguous(res, d_flat, n, pq_dim, pq_bits, 0, own);
     const auto restored = search_all(res, index, d_data, n_queries, k);
     REQUIRE(restored.ids == before_search.ids && restored.dist == before_search.dist);
     REQUIRE(snapshot(index, label).bytes == before.bytes);
-    REQUIRE(!(proper.ids == before_search.ids && proper.dist == before_search.dist));  // the edit was visible at all
   }
   // rows written somewhere else do change the list, and exactly those rows
   packer::pack_list_data(res, &index, make_device_matrix_view<const uint8_t>(d_codes + 5 * pq_dim, 3, pq_dim), label, 10);
