@@ -70,7 +70,14 @@ struct slab_kernel {
   static constexpr float kEntryScale = LUT == LUT_F16 ? 1.0f : 2.0f;
   static constexpr int TERMS = IP ? 2 : 1;
   static constexpr int FPS   = PQ_LEN * TERMS;  // staged floats per subspace
-  static_assert(NCH_LAST == 2 || NCH_LAST == 4, "pq_dim is a multiple of 32");
+  // a table of 16-bit entries takes 64 subspaces (four 16-byte chunks of a row) in its 32 KB, one
+  // of fp32 entries 32
+  static constexpr bool WIDE     = LUT == LUT_F32;
+  static constexpr int SCH       = WIDE ? 2 : 4;         // chunks of a whole slab
+  static constexpr uint32_t SUBS = 16u * SCH;            // its subspaces
+  static constexpr uint32_t SUB_BYTES = WIDE ? 1024u : 512u;  // bytes of a subspace's 256 entries
+  static_assert((NCH_LAST == 2 || NCH_LAST == 4) && NCH_LAST <= SCH, "pq_dim is a multiple of 32");
+  static_assert(!(WIDE && OUT_HALF), "fp32 entries are summed in fp32");
   static_assert(kSlabSubs * FPS * 4u <= kSlabStageSlot, "staged terms of a slab must fit their slot");
   // staging elements (pair, dimension of the slab) per builder thread
   static constexpr uint32_t E = (G * kSlabSubs * PQ_LEN + 511u) / 512u;
@@ -160,17 +167,17 @@ struct slab_kernel {
     __device__ __forceinline__ bool valid() const { return (flags & 8u) != 0u; }
     __device__ __forceinline__ uint32_t slab() const { return flags >> 4; }
   };
-  /** Runs fn(NCH) for the slab's chunk count: 4, or NCH_LAST in a last slab. */
+  /** Runs fn(NCH) for the slab's chunk count: SCH, or NCH_LAST in a last slab. */
   template <typename Fn>
   static __device__ __forceinline__ void for_chunks(bool last, Fn fn)
   {
-    if constexpr (NCH_LAST == 4) {
-      fn(std::integral_constant<int, 4>{});
+    if constexpr (NCH_LAST == SCH) {
+      fn(std::integral_constant<int, SCH>{});
     } else {
       if (last) {
         fn(std::integral_constant<int, NCH_LAST>{});
       } else {
-        fn(std::integral_constant<int, 4>{});
+        fn(std::integral_constant<int, SCH>{});
       }
     }
   }
@@ -206,7 +213,7 @@ struct slab_kernel {
   __device__ __forceinline__ void fetch_terms(const quad_info& info, uint32_t bt, staged& f) const
   {
     constexpr uint32_t DIMS = 16u * NCH * PQ_LEN;  // rotated dimensions of the slab
-    const uint32_t d0       = f.slab() * (kSlabSubs * PQ_LEN);
+    const uint32_t d0       = f.slab() * (SUBS * PQ_LEN);
 #pragma unroll
     for (uint32_t x = 0; x < E; x++) {
       const uint32_t idx = bt + 512u * x;
@@ -272,7 +279,7 @@ struct slab_kernel {
     constexpr int QM = 4 * NCH;  // subspaces of a builder thread
     constexpr int NG = QM / GB;
     static_assert(QM % GB == 0, "whole groups");
-    const uint32_t j_first = f.slab() * kSlabSubs + quarter * uint32_t(QM);
+    const uint32_t j_first = f.slab() * SUBS + quarter * uint32_t(QM);
     book_group bk[2];
     if constexpr (!PER_CLUSTER) { bk[0] = load_books(j_first, code); }
     // per-cluster codebooks: the components of the thread's two codes in the books of the two lists,
@@ -335,7 +342,12 @@ struct slab_kernel {
               }
             }
           }
-          entries[g][jj] = pack_entries(score[0], score[1]);
+          if constexpr (WIDE) {
+            entries[g][2 * jj]     = __float_as_uint(score[0]);
+            entries[g][2 * jj + 1] = __float_as_uint(score[1]);
+          } else {
+            entries[g][jj] = pack_entries(score[0], score[1]);
+          }
         }
       }
       // the requests stay where they are written: one group ahead of the arithmetic, no further
@@ -343,13 +355,27 @@ struct slab_kernel {
     }
   }
 
+  /** ds_write_b64 at addr + IMM: the fp32 entries of two neighbouring codes of one subspace. */
+  template <int IMM>
+  __device__ __forceinline__ static void entries_write_wide(uint32_t addr, uint32_t e0, uint32_t e1)
+  {
+    static_assert(IMM >= 0 && IMM < 65536, "the write's offset field has 16 bits");
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 two = {e0, e1};
+    asm volatile("ds_write_b64 %0, %1 offset:%2" : : "v"(addr), "v"(two), "n"(IMM) : "memory");
+  }
+
   /** ... and from the registers into the tables, while no scanner reads:
-   *  entry (j, code) of a slab's table at base + j * 512 + code * 2. */
+   *  entry (j, code) of a slab's table at base + j * SUB_BYTES + code * (2 or 4). */
   template <int NCH, int jj = 0>
   __device__ __forceinline__ static void write_entries(uint32_t waddr, const uint32_t (&entries)[16])
   {
     if constexpr (jj < 4 * NCH) {
-      entries_write<jj * 512>(waddr, entries[jj]);
+      if constexpr (WIDE) {
+        entries_write_wide<jj * 1024>(waddr, entries[2 * jj], entries[2 * jj + 1]);
+      } else {
+        entries_write<jj * 512>(waddr, entries[jj]);
+      }
       write_entries<NCH, jj + 1>(waddr, entries);
     }
   }
@@ -360,7 +386,7 @@ struct slab_kernel {
 #pragma unroll
     for (uint32_t g = 0; g < G; g++) {
       if (!f.live(g)) { continue; }  // uniform
-      write_entries<NCH>(slab_table_base(g) + quarter * uint32_t(4 * NCH) * 512u + code * 2u, entries[g]);
+      write_entries<NCH>(slab_table_base(g) + quarter * uint32_t(4 * NCH) * SUB_BYTES + code * (WIDE ? 4u : 2u), entries[g]);
     }
   }
 
@@ -461,12 +487,12 @@ struct slab_kernel {
     return rows;
   }
 
-  /** Chunk 4 s of `row`; chunk m of the slab is 32 vectors further on each. */
+  /** Chunk SCH * s of `row`; chunk m of the slab is 32 vectors further on each. */
   __device__ __forceinline__ const GLOBAL_AS u32x4* row_ptr(const uint8_t* list_data, uint32_t row, uint32_t s) const
   {
     return reinterpret_cast<const GLOBAL_AS u32x4*>(reinterpret_cast<uintptr_t>(list_data) +
                                                     uint64_t(row >> 5) * (nch_total * 512u) + uint64_t(row & 31u) * 16u +
-                                                    uint64_t(s) * (4u * 512u));
+                                                    uint64_t(s) * (uint32_t(SCH) * 512u));
   }
   template <int NCH>
   __device__ __forceinline__ static void load_tile(const GLOBAL_AS u32x4* ptr, u32x4 (&dst)[4])
@@ -499,7 +525,7 @@ struct slab_kernel {
     // sums of the pair's rows between slabs: row r of the row block at word r
     auto* part         = reinterpret_cast<LDS_AS uint32_t*>(uintptr_t(kSlabPartBase + uint32_t(GI) * kSlabRows * 4u)) + lane;
     const float one    = opaque_float(kEntryScale);
-    uint32_t one_u     = 1u;
+    uint32_t one_u     = WIDE ? 2u : 1u;  // a code shifted by this is its entry's offset in a subspace's table
     asm volatile("" : "+v"(one_u));
 
     // address registers of the lookups: the window of the group's table in the high halves
@@ -582,7 +608,7 @@ struct slab_kernel {
           if (s != 0u) { start = *my_part; }
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // see ST_FIRST
           const uint32_t sum_bits =
-            stream_tile_sum<NCH, OUT_HALF, !IP, IMMG>(now, addr, one_u, one, stop_bits, in_play, start);
+            stream_tile_sum<NCH, OUT_HALF, !IP, IMMG, WIDE>(now, addr, one_u, one, stop_bits, in_play, start);
           if constexpr (!LAST) {
             bool keep = true;
             if constexpr (!IP) {
@@ -647,7 +673,7 @@ struct slab_kernel {
         if (last) {
           run_tiles(std::integral_constant<int, NCH_LAST>{}, std::true_type{});
         } else {
-          run_tiles(std::integral_constant<int, 4>{}, std::false_type{});
+          run_tiles(std::integral_constant<int, SCH>{}, std::false_type{});
         }
       }
 
@@ -702,7 +728,7 @@ __global__ __launch_bounds__(kSlabThreads) void scan_slab_kernel(scan_args a)
   if (lb >= n_quads) { return; }  // whole block, before any barrier
   const uint32_t nch_total = a.pq_dim >> 4;
   body k{a, n_pairs, n_quads, grid, lb, (n_quads - lb + grid - 1u) / grid, tid & 63u,
-         (wid & 3u) | ((wid >> 3) << 2), (a.pq_dim + kSlabSubs - 1u) / kSlabSubs, nch_total};
+         (wid & 3u) | ((wid >> 3) << 2), (a.pq_dim + body::SUBS - 1u) / body::SUBS, nch_total};
   // waves 0-3 and 8-11 build, 4-7 and 12-15 scan: two of each kind on every SIMD
   if (((wid >> 2) & 1u) == 0u) {
     k.run_builder();
@@ -735,7 +761,8 @@ void launch_slab_instance(const scan_args& a, hipStream_t stream)
     if (grid > n_quads) { grid = n_quads; }
     if (grid == 0) { return; }
   }
-  const uint32_t lds = a.pq_dim > kSlabSubs ? kSlabLdsBytes : kSlabLdsOneSlab;
+  constexpr uint32_t subs = LUT == LUT_F32 ? 32u : 64u;  // of a slab
+  const uint32_t lds      = a.pq_dim > subs ? kSlabLdsBytes : kSlabLdsOneSlab;
   kernel<<<grid, kSlabThreads, lds, stream>>>(a);
   CUVS_HIP_TRY(hipGetLastError());
 }
@@ -768,6 +795,25 @@ bool launch_slab_types(const scan_args& a, hipStream_t s)
 template <int PQ_LEN>
 bool launch_slab_len(const scan_args& a, hipStream_t s)
 {
+  if (a.lut_dtype == CUDA_R_32F) {
+    // fp32 entries: slabs of 32 subspaces, all of them whole; fp32 sums
+    if (a.out_half) { return false; }
+    const bool ip = a.metric == int(DistanceType::InnerProduct) || a.metric == int(DistanceType::CosineExpanded);
+    if (a.per_cluster) {
+      if (ip) {
+        launch_slab_instance<2, PQ_LEN, LUT_F32, false, true, true>(a, s);
+      } else {
+        launch_slab_instance<2, PQ_LEN, LUT_F32, false, true, false>(a, s);
+      }
+    } else {
+      if (ip) {
+        launch_slab_instance<2, PQ_LEN, LUT_F32, false, false, true>(a, s);
+      } else {
+        launch_slab_instance<2, PQ_LEN, LUT_F32, false, false, false>(a, s);
+      }
+    }
+    return true;
+  }
   const bool half_last = (a.pq_dim & 63u) != 0u;  // a last slab of 32 subspaces
   if (a.per_cluster) {
     return half_last ? launch_slab_types<2, PQ_LEN, true>(a, s) : launch_slab_types<4, PQ_LEN, true>(a, s);

@@ -16,7 +16,7 @@ uint32_t scan_slab_keys_per_pair(const scan_args& a)
 {
   if (!a.fused || a.pq_bits != 8 || a.k > kSlabMaxK) { return 0; }
   if (a.rot_dim != a.pq_dim * a.pq_len) { return 0; }
-  if (a.lut_dtype != CUDA_R_16F && a.lut_dtype != CUDA_R_8U) { return 0; }
+  if (a.lut_dtype != CUDA_R_16F && a.lut_dtype != CUDA_R_8U && !(a.lut_dtype == CUDA_R_32F && !a.out_half)) { return 0; }
   if (a.pq_dim < 32 || a.pq_dim % 32 != 0) { return 0; }
   const bool len = a.pq_len == 1 || a.pq_len == 2 || a.pq_len == 3 || a.pq_len == 4 || a.pq_len == 8;
   return len ? kSlabWG * a.k : 0;

@@ -63,35 +63,42 @@ __device__ __forceinline__ uint16_t table_entry(float score)
 #define ST_SDWA(a, c, sel)                                                                                   \
   "v_lshlrev_b32_sdwa %[" #a "], %[one_u], %[" #c "] dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD " \
   "src1_sel:BYTE_" #sel "\n\t"
-#define ST_READ(v, a, o, i) "ds_read_u16 %[" #v "], %[" #a "] offset:%[immg]+" #o "*4096+" #i "*512\n\t"
+/* the read of subspace 8 o + i: 16-bit entries 512 bytes a subspace, or (RD32) fp32 entries 1 KB a subspace */
+#define ST_RD16(v, a, o, i) "ds_read_u16 %[" #v "], %[" #a "] offset:%[immg]+" #o "*4096+" #i "*512\n\t"
+#define ST_RD32(v, a, o, i) "ds_read_b32 %[" #v "], %[" #a "] offset:%[immg]+" #o "*8192+" #i "*1024\n\t"
 /* group o: subspaces 8 o .. 8 o + 7, code dwords ca, cb, entries into V0 .. V7 */
-#define ST_ISSUE(o, ca, cb, V)                                                                     \
+#define ST_ISSUE(RD, o, ca, cb, V)                                                                 \
   ST_SDWA(a0, ca, 0) ST_SDWA(a1, ca, 1) ST_SDWA(a2, ca, 2) ST_SDWA(a3, ca, 3)                      \
   ST_SDWA(a4, cb, 0) ST_SDWA(a5, cb, 1) ST_SDWA(a6, cb, 2) ST_SDWA(a7, cb, 3)                      \
-  ST_READ(V##0, a0, o, 0) ST_READ(V##1, a1, o, 1) ST_READ(V##2, a2, o, 2) ST_READ(V##3, a3, o, 3)  \
-  ST_READ(V##4, a4, o, 4) ST_READ(V##5, a5, o, 5) ST_READ(V##6, a6, o, 6) ST_READ(V##7, a7, o, 7)
+  RD(V##0, a0, o, 0) RD(V##1, a1, o, 1) RD(V##2, a2, o, 2) RD(V##3, a3, o, 3)                      \
+  RD(V##4, a4, o, 4) RD(V##5, a5, o, 5) RD(V##6, a6, o, 6) RD(V##7, a7, o, 7)
 /* the two halves of a group: one code dword each */
-#define ST_ISSUE_LO(o, ca, V)                                                                      \
+#define ST_ISSUE_LO(RD, o, ca, V)                                                                  \
   ST_SDWA(a0, ca, 0) ST_SDWA(a1, ca, 1) ST_SDWA(a2, ca, 2) ST_SDWA(a3, ca, 3)                      \
-  ST_READ(V##0, a0, o, 0) ST_READ(V##1, a1, o, 1) ST_READ(V##2, a2, o, 2) ST_READ(V##3, a3, o, 3)
-#define ST_ISSUE_HI(o, cb, V)                                                                      \
+  RD(V##0, a0, o, 0) RD(V##1, a1, o, 1) RD(V##2, a2, o, 2) RD(V##3, a3, o, 3)
+#define ST_ISSUE_HI(RD, o, cb, V)                                                                  \
   ST_SDWA(a4, cb, 0) ST_SDWA(a5, cb, 1) ST_SDWA(a6, cb, 2) ST_SDWA(a7, cb, 3)                      \
-  ST_READ(V##4, a4, o, 4) ST_READ(V##5, a5, o, 5) ST_READ(V##6, a6, o, 6) ST_READ(V##7, a7, o, 7)
+  RD(V##4, a4, o, 4) RD(V##5, a5, o, 5) RD(V##6, a6, o, 6) RD(V##7, a7, o, 7)
 #define ST_WAIT4 "s_waitcnt lgkmcnt(4)\n\t"
 #define ST_WAIT8 "s_waitcnt lgkmcnt(8)\n\t"
 #define ST_WAIT0 "s_waitcnt lgkmcnt(0)\n\t"
 /* fp32 sums: entry * scale + sum in one instruction that widens the binary16 entry (exact product) */
 #define ST_ADD_F32_1(v) "v_fma_mix_f32 %[acc], %[" #v "], %[one], %[acc] op_sel_hi:[1,0,0]\n\t"
 #define ST_ADD_F16_1(v) "v_add_f16_e32 %[acc], %[acc], %[" #v "]\n\t"
+/* fp32 entries */
+#define ST_ADD_W32_1(v) "v_add_f32_e32 %[acc], %[acc], %[" #v "]\n\t"
 #define ST_ADD8(ADD1, V) ADD1(V##0) ADD1(V##1) ADD1(V##2) ADD1(V##3) ADD1(V##4) ADD1(V##5) ADD1(V##6) ADD1(V##7)
 #define ST_ADD4_LO(ADD1, V) ADD1(V##0) ADD1(V##1) ADD1(V##2) ADD1(V##3)
 #define ST_ADD4_HI(ADD1, V) ADD1(V##4) ADD1(V##5) ADD1(V##6) ADD1(V##7)
 #define ST_ADD_F32(V) ST_ADD8(ST_ADD_F32_1, V)
 #define ST_ADD_F16(V) ST_ADD8(ST_ADD_F16_1, V)
+#define ST_ADD_W32(V) ST_ADD8(ST_ADD_W32_1, V)
 #define ST_ADD_F32_LO(V) ST_ADD4_LO(ST_ADD_F32_1, V)
 #define ST_ADD_F32_HI(V) ST_ADD4_HI(ST_ADD_F32_1, V)
 #define ST_ADD_F16_LO(V) ST_ADD4_LO(ST_ADD_F16_1, V)
 #define ST_ADD_F16_HI(V) ST_ADD4_HI(ST_ADD_F16_1, V)
+#define ST_ADD_W32_LO(V) ST_ADD4_LO(ST_ADD_W32_1, V)
+#define ST_ADD_W32_HI(V) ST_ADD4_HI(ST_ADD_W32_1, V)
 /* rows in play whose sum is not past the bound; none: leave */
 #define ST_CHECK_F32                                 \
   "v_cmp_ge_u32_e32 vcc, %[stop], %[acc]\n\t"        \
@@ -108,21 +115,22 @@ __device__ __forceinline__ uint16_t table_entry(float score)
  * issued.  The sum starts from the value the caller put into the accumulator.  The waits count
  * this block's own reads: nothing else that counts on lgkmcnt and may complete out of order (a
  * scalar load) may be in flight when the block starts. */
-#define ST_FIRST(ADD, CHECK)                                                    \
-  ST_ISSUE_LO(0, c0, va) ST_ISSUE_HI(0, c1, va)                                 \
-  ST_WAIT4 ADD##_LO(va) CHECK ST_ISSUE(1, c2, c3, vb)                           \
-  ST_WAIT8 ADD##_HI(va) CHECK ST_ISSUE(2, c4, c5, va)                           \
-  ST_WAIT8 ADD(vb) CHECK ST_ISSUE(3, c6, c7, vb)
+#define ST_FIRST(RD, ADD, CHECK)                                                \
+  ST_ISSUE_LO(RD, 0, c0, va) ST_ISSUE_HI(RD, 0, c1, va)                         \
+  ST_WAIT4 ADD##_LO(va) CHECK ST_ISSUE(RD, 1, c2, c3, vb)                       \
+  ST_WAIT8 ADD##_HI(va) CHECK ST_ISSUE(RD, 2, c4, c5, va)                       \
+  ST_WAIT8 ADD(vb) CHECK ST_ISSUE(RD, 3, c6, c7, vb)
 /* a chunk that is not the last: its two groups are added, groups o + 2 and o + 3 issued */
-#define ST_CHUNK(o0, o1, o2, o3, c4, c5, c6, c7, ADD, CHECK)  \
-  ST_WAIT8 ADD(va) CHECK ST_ISSUE(o2, c4, c5, va)             \
-  ST_WAIT8 ADD(vb) CHECK ST_ISSUE(o3, c6, c7, vb)
+#define ST_CHUNK(RD, o0, o1, o2, o3, c4, c5, c6, c7, ADD, CHECK)  \
+  ST_WAIT8 ADD(va) CHECK ST_ISSUE(RD, o2, c4, c5, va)             \
+  ST_WAIT8 ADD(vb) CHECK ST_ISSUE(RD, o3, c6, c7, vb)
 #define ST_TAIL(ADD) ST_WAIT8 ADD(va) ST_WAIT0 ADD(vb) ".Ltile_done%=:\n\t" ST_WAIT0
-#define ST_BODY_2(ADD, CHECK) ST_FIRST(ADD, CHECK) ST_TAIL(ADD)
-#define ST_BODY_3(ADD, CHECK) ST_FIRST(ADD, CHECK) ST_CHUNK(2, 3, 4, 5, c8, c9, c10, c11, ADD, CHECK) ST_TAIL(ADD)
-#define ST_BODY_4(ADD, CHECK)                                                            \
-  ST_FIRST(ADD, CHECK) ST_CHUNK(2, 3, 4, 5, c8, c9, c10, c11, ADD, CHECK)                \
-  ST_CHUNK(4, 5, 6, 7, c12, c13, c14, c15, ADD, CHECK) ST_TAIL(ADD)
+#define ST_BODY_2(RD, ADD, CHECK) ST_FIRST(RD, ADD, CHECK) ST_TAIL(ADD)
+#define ST_BODY_3(RD, ADD, CHECK) \
+  ST_FIRST(RD, ADD, CHECK) ST_CHUNK(RD, 2, 3, 4, 5, c8, c9, c10, c11, ADD, CHECK) ST_TAIL(ADD)
+#define ST_BODY_4(RD, ADD, CHECK)                                                            \
+  ST_FIRST(RD, ADD, CHECK) ST_CHUNK(RD, 2, 3, 4, 5, c8, c9, c10, c11, ADD, CHECK)            \
+  ST_CHUNK(RD, 4, 5, 6, 7, c12, c13, c14, c15, ADD, CHECK) ST_TAIL(ADD)
 
 #define ST_OUTPUTS                                                                                              \
   [acc] "+v"(acc), [chk] "=&v"(chk), [tmp] "=&s"(tmp), [a0] "+v"(ad[0]), [a1] "+v"(ad[1]), [a2] "+v"(ad[2]),     \
@@ -146,26 +154,32 @@ __device__ __forceinline__ uint16_t table_entry(float score)
  *  summed.  CHECK: end the tile when no row of `valid` has a sum whose bits are at most `stop`.
  *  IMMG: offset of the table inside its 64 KB window, which the high halves of the address
  *  registers `ad` name (the routine changes their low halves only); `one` is the factor of the
- *  entries (fp32 sums), one_u the integer 1. */
-template <int NCH, bool HALF, bool CHECK, int IMMG, int NCUR>
+ *  entries (fp32 sums), one_u the integer 1.  WIDE: the table holds fp32 entries, 1 KB a subspace,
+ *  added as they are; one_u is then 2 (the shift that turns a code into its entry's offset). */
+template <int NCH, bool HALF, bool CHECK, int IMMG, bool WIDE = false, int NCUR = NCH>
 __device__ __forceinline__ uint32_t stream_tile_sum(const u32x4 (&cur)[NCUR], uint32_t (&ad)[8], uint32_t one_u, float one,
                                                     uint32_t stop, unsigned long long valid, uint32_t start = 0u)
 {
   static_assert(NCH >= 2 && NCH <= 4 && NCH <= NCUR, "two to four chunks of sixteen subspaces");
-  static_assert(IMMG >= 0 && IMMG + (NCH * 16 - 1) * 512 < 65536, "the read's offset field has 16 bits");
+  static_assert(IMMG >= 0 && IMMG + (NCH * 16 - 1) * (WIDE ? 1024 : 512) < 65536, "the read's offset field has 16 bits");
+  static_assert(!(WIDE && HALF), "fp32 entries are summed in fp32");
   uint32_t acc = start, chk, va[8], vb[8];
   unsigned long long tmp;
-#define ST_EMIT(BODY, ADD, CHK, ...) \
-  asm volatile(BODY(ADD, CHK) : ST_OUTPUTS : ST_COMMON_INPUTS, __VA_ARGS__ : "vcc", "scc", "memory")
+#define ST_EMIT(BODY, RD, ADD, CHK, ...) \
+  asm volatile(BODY(RD, ADD, CHK) : ST_OUTPUTS : ST_COMMON_INPUTS, __VA_ARGS__ : "vcc", "scc", "memory")
 #define ST_EMIT_KIND(BODY, ...)                                              \
-  if constexpr (!HALF && CHECK) {                                            \
-    ST_EMIT(BODY, ST_ADD_F32, ST_CHECK_F32, __VA_ARGS__);                    \
+  if constexpr (WIDE && CHECK) {                                             \
+    ST_EMIT(BODY, ST_RD32, ST_ADD_W32, ST_CHECK_F32, __VA_ARGS__);           \
+  } else if constexpr (WIDE && !CHECK) {                                     \
+    ST_EMIT(BODY, ST_RD32, ST_ADD_W32, ST_NO_CHECK, __VA_ARGS__);            \
+  } else if constexpr (!HALF && CHECK) {                                     \
+    ST_EMIT(BODY, ST_RD16, ST_ADD_F32, ST_CHECK_F32, __VA_ARGS__);           \
   } else if constexpr (!HALF && !CHECK) {                                    \
-    ST_EMIT(BODY, ST_ADD_F32, ST_NO_CHECK, __VA_ARGS__);                     \
+    ST_EMIT(BODY, ST_RD16, ST_ADD_F32, ST_NO_CHECK, __VA_ARGS__);            \
   } else if constexpr (HALF && CHECK) {                                      \
-    ST_EMIT(BODY, ST_ADD_F16, ST_CHECK_F16, __VA_ARGS__);                    \
+    ST_EMIT(BODY, ST_RD16, ST_ADD_F16, ST_CHECK_F16, __VA_ARGS__);           \
   } else {                                                                   \
-    ST_EMIT(BODY, ST_ADD_F16, ST_NO_CHECK, __VA_ARGS__);                     \
+    ST_EMIT(BODY, ST_RD16, ST_ADD_F16, ST_NO_CHECK, __VA_ARGS__);            \
   }
   if constexpr (NCH == 2) {
     ST_EMIT_KIND(ST_BODY_2, ST_CODES_2)

@@ -400,7 +400,10 @@ void search(cuvs::resources const& res_c,
   // pq_dim that is a multiple of 32) the table in slabs
   sa.fused = pl.fused;
   const uint32_t stream_kpp = res.tuning.generic_scan ? 0u : detail::scan_stream_keys_per_pair(sa);
-  const uint32_t slab_kpp   = res.tuning.generic_scan || stream_kpp != 0 ? 0u : detail::scan_slab_keys_per_pair(sa);
+  // fp32 tables: the table-free kernel where it has the shape (it also beats a table in slabs on
+  // the lists of a few hundred rows its shapes come with), else the slab kernel
+  const bool direct_scan    = !res.tuning.generic_scan && detail::scan_direct_supported(sa);
+  const uint32_t slab_kpp   = res.tuning.generic_scan || stream_kpp != 0 || direct_scan ? 0u : detail::scan_slab_keys_per_pair(sa);
   // a table too large for LDS goes to global memory (8-bit codes, generic kernel)
   const bool global_lut = slab_kpp == 0 && detail::scan_lds_bytes(sa) > kMaxLds;
   if (global_lut) {
@@ -593,12 +596,9 @@ void search(cuvs::resources const& res_c,
         } else if (sa.pq_bits == 4) {
           if (detail::launch_scan_nibble_pack(sa, s)) { scan_kernel_id = cuvs::scan_kernel_nibble_pack; return; }
           if (!subset && detail::launch_scan_nibble(sa, s)) { scan_kernel_id = cuvs::scan_kernel_nibble; return; }
-        } else if (subset) {
-          if (detail::scan_direct_supported(sa) && detail::launch_scan_direct(sa, s)) { scan_kernel_id = cuvs::scan_kernel_direct; return; }
-          if (detail::launch_scan_fast(sa, s)) { scan_kernel_id = cuvs::scan_kernel_fast; return; }
         } else {
+          if (direct_scan && detail::launch_scan_direct(sa, s)) { scan_kernel_id = cuvs::scan_kernel_direct; return; }
           if (detail::launch_scan_fast(sa, s)) { scan_kernel_id = cuvs::scan_kernel_fast; return; }
-          if (detail::launch_scan_direct(sa, s)) { scan_kernel_id = cuvs::scan_kernel_direct; return; }
         }
       }
       CUVS_EXPECTS(!subset, "scan kernel launch failed");

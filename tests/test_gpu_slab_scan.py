@@ -20,7 +20,7 @@ pytestmark = pytest.mark.gpu
 R_32F, R_16F, R_8U = np.float32, np.float16, np.uint8
 ORC_DT = {np.float32: 0, np.float16: 2, np.int8: 3, np.uint8: 8}
 SLAB, GENERIC = 6, 0
-TABLES = [(R_16F, R_32F), (R_8U, R_32F), (R_16F, R_16F), (R_8U, R_16F)]
+TABLES = [(R_32F, R_32F), (R_16F, R_32F), (R_8U, R_32F), (R_16F, R_16F), (R_8U, R_16F)]
 
 
 def _build(orc, n, dim, n_lists, pq_dim, pq_bits=8, dtype=np.float32, metric="sqeuclidean", kind="subspace",
@@ -118,7 +118,7 @@ def test_slab_scan_lists_longer_than_a_row_block(orc, metric):
                                       labels=labels)
     assert ix.list_sizes.max() > 2 * 8192 and ix.list_sizes.min() < 4096
     res = _profiling_resources("off")
-    for lut, internal in [(R_16F, R_32F), (R_8U, R_16F)]:
+    for lut, internal in [(R_32F, R_32F), (R_16F, R_32F), (R_8U, R_16F)]:
         for k in (10, 100):
             _check(orc, res, index, ix, queries, k, 3, lut, internal)
             _check(orc, res, index, ix, queries, k, 2, lut, internal)
@@ -132,7 +132,7 @@ def test_slab_scan_filter_and_empty_lists(orc):
     bits = np.packbits(keep, bitorder="little")
     bits = np.concatenate([bits, np.zeros((-bits.size) % 4, dtype=np.uint8)]).view(np.uint32)
     res = _profiling_resources("off")
-    for lut, internal in [(R_16F, R_32F), (R_8U, R_16F)]:
+    for lut, internal in [(R_32F, R_32F), (R_16F, R_32F), (R_8U, R_16F)]:
         _check(orc, res, index, ix, queries, 20, 6, lut, internal,
                filter_bitset=G.to_dev(bits.view(np.int32)), filter_nbits=n)
         _check(orc, res, index, ix, queries, 30, 2, lut, internal)
@@ -168,7 +168,7 @@ def test_slab_scan_under_the_early_stop(orc, dim, pq_dim, kind):
     index = G.build_gpu_index(model, x, pq_dim, 8, "sqeuclidean", kind)
     ix, _ = G.read_back(orc, index, model, dim, pq_dim, 8, "sqeuclidean", kind)
     res = _profiling_resources("on")
-    for lut, internal in [(R_16F, R_32F), (R_8U, R_16F)]:
+    for lut, internal in [(R_32F, R_32F), (R_16F, R_32F), (R_8U, R_16F)]:
         for k in (10, 100):
             nb, d, prof = _check(orc, res, index, ix, q, k, 24, lut, internal)
             assert prof["n_screened_pairs"] == q.shape[0] * 23
