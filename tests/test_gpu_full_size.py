@@ -236,3 +236,48 @@ def test_20m_f16_per_cluster(orc):
                       want_nb, want_d, 2e-3, exact=True)
     del index, data, allrows
     torch.cuda.empty_cache()
+
+
+# ------------------------------------------------------------------------------------------------
+# The 100M-row configuration itself: 100M x 96 fp16, 50,000 lists, per-cluster codebooks, pq_dim 48,
+# 200 probes (4.8 GB of codes + 0.8 GB of ids on the GPU).  Properties only: a host copy of this index
+# for the oracle would take longer than everything else here (the case above has the oracle sample).
+# ------------------------------------------------------------------------------------------------
+
+def test_100m_f16_per_cluster():
+    n, nq, dim, n_lists = 100_000_000, 10_000, 96, 50_000
+    allrows = testing.gaussian_mixture(n + nq, dim, n_lists, 0.25, seed=1234, device="cuda", dtype=torch.float16)
+    data, queries = allrows[:n], allrows[n:].contiguous()
+    params = ivf_pq.IndexParams(n_lists=n_lists, pq_bits=8, pq_dim=48, codebook_kind="cluster",
+                                kmeans_trainset_fraction=1_600_000 / n)
+    index = ivf_pq.build(params, data)
+    assert len(index) == n
+    sizes = index.list_sizes.cpu().numpy()
+    assert int(sizes.sum()) == n and sizes.max() < 20 * sizes.mean()
+    results = {}
+    for batch in (1, 100, 10_000):
+        q = queries[:batch].contiguous()
+        d, nb = _search(index, q, 10, 200)
+        _well_formed(d, nb, n)
+        results[batch] = (d, nb)
+    # a query's answer depends neither on the batch it arrives in nor on how the batch is split
+    for small in (1, 100):
+        assert torch.equal(results[small][0], results[10_000][0][:small])
+        assert torch.equal(results[small][1], results[10_000][1][:small])
+    d_split, nb_split = _search(index, queries, 10, 200, batch=3000)
+    assert torch.equal(nb_split, results[10_000][1]) and torch.equal(d_split, results[10_000][0])
+    # more probes can only improve every rank; the first k of a longer list are the shorter list
+    d100, _ = _search(index, queries[:2000].contiguous(), 10, 100)
+    _rankwise_no_worse(results[10_000][0][:2000], d100)
+    d40, nb40 = _search(index, queries[:2000].contiguous(), 40, 200)
+    _prefix_of(results[10_000][0][:2000], results[10_000][1][:2000], d40, nb40)
+    # recall against exact search, and exact re-ranking of 40 candidates
+    truth = testing.exact_knn(data, queries[:500], 10).cpu().numpy()
+    rec = testing.recall(results[10_000][1][:500].cpu().numpy(), truth)
+    d_ref, nb_ref = refine(data, queries[:500].contiguous(), nb40[:500].contiguous(), 10)
+    torch.cuda.synchronize()
+    refined = testing.recall(nb_ref.cpu().numpy(), truth)
+    print(f"recall@10 at 200 probes: {rec:.4f}; 40 candidates re-ranked: {refined:.4f}", flush=True)
+    assert rec >= 0.75 and refined >= rec
+    del index, data, allrows
+    torch.cuda.empty_cache()
