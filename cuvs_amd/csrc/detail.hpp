@@ -449,8 +449,12 @@ bool launch_scan_slab(const scan_args& a, hipStream_t stream);
 bool scan_screen_supported(const scan_args& a);
 /** Bytes of each row the screen reads (8 or 16). */
 uint32_t scan_screen_bytes_per_row(bool per_cluster, bool lead_plane);
+/** Inner-product and cosine searches are screened on a proven lower bound of what the subspaces
+ *  past the leading ones can still add; the bound's per-query part lives in `scratch`
+ *  (scan_screen_scratch_bytes() bytes for the batch, 0 for L2 metrics; rewritten by every launch). */
+size_t scan_screen_scratch_bytes(const scan_args& a, uint32_t n_queries);
 void launch_scan_screen(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
-                        pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
+                        pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive, void* scratch,
                         hipStream_t stream);
 /** query_kth[q] = min(query_kth[q], score of the k-th smallest valid key among the first `n_keys`
  *  keys of query q's candidate block (`keys_per_query` keys apart)). */

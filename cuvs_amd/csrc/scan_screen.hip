@@ -22,6 +22,8 @@
 #include "device_utils.cuh"
 
 #include <algorithm>
+#include <cfloat>
+#include <cmath>
 #include <cstddef>
 #include <cstdlib>
 
@@ -308,6 +310,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
  */
 constexpr uint32_t kDirectThreads = 512;
 constexpr uint32_t kDirectSubs    = 8;
+constexpr uint32_t kIpRounds      = 12;  // the inner-product screen keeps a value per 64 subspaces: pq_dim <= 768
 
 template <int PQ_LEN>
 struct book_vec;
@@ -661,6 +664,360 @@ void launch_screen_types(const scan_args& a, const pair_desc* desc, uint32_t n_p
   }
 }
 
+
+/* ---------------------------------------------------------------------------------------------
+ * Screening for inner-product and cosine searches (per-subspace codebooks, the plane of leading
+ * codes; 8- and 4-bit codes).
+ *
+ * Table entries of these metrics have either sign, so a partial sum bounds nothing by itself.  What
+ * does: entry (j, code) is LutT(x) with x = -(sum_t c_t q_t) - (sum_t q_t b_t[code]) over the
+ * subspace's dimensions, whose second term depends on the query and the code alone.  With
+ * U_j(q) = max over codes of that term (ip_query_bounds_kernel, once per query) every entry of
+ * subspace j of a pair is at least m_j = LutT(-(sum_t c_t q_t) - U_j - rounding slack), because the
+ * table's rounding is monotone.  A row whose sum over the first S subspaces is p then ends at or
+ * above p + sum_{j >= S} m_j - (rounding of the remaining additions), and a pair none of whose rows
+ * can still reach the query's k-th best score is dropped, exactly as under L2.  Rows are only ever
+ * dropped on a proven bound, so the results are those of the full scan.
+ *
+ * fp32 sums: the rounding of the M additions is bounded analytically (a few 2^-24 of the sum of the
+ * entries' magnitudes).  binary16 sums: the error bound of hundreds of half-precision additions
+ * would be useless, but rounded addition is monotone in both operands, so the sum of a
+ * hypothetical row that takes the minimum m_j in every remaining subspace, added in the scan's own
+ * order and type, is a lower bound of every real row that starts from at least the same partial
+ * sum.  The wave evaluates that chain for 64 starting values at once (a lane each) and takes the
+ * smallest one that ends above the bound as the threshold for the rows' partial sums.
+ * --------------------------------------------------------------------------------------------- */
+
+/** out[q][j] = (U, W): the largest sum_t q_t b_t[code] over the codes of subspace j, and the largest
+ *  sum_t |q_t b_t[code]| (what bounds the rounding of an entry's evaluation). */
+__global__ __launch_bounds__(256) void ip_query_bounds_kernel(const float* __restrict__ rot_q,
+                                                              const float* __restrict__ pq_centers, uint32_t pq_dim,
+                                                              uint32_t pq_len, uint32_t book, uint32_t rot_dim,
+                                                              float2* __restrict__ out)
+{
+  __shared__ float s_u[4], s_w[4];
+  const uint32_t q    = blockIdx.x;
+  const uint32_t tid  = threadIdx.x;
+  const uint32_t per  = 256u / book;        // subspaces per pass: 1 (256 codes) or 16 (16 codes)
+  const uint32_t code = tid % book;
+  const float* qrow   = rot_q + uint64_t(q) * rot_dim;
+  for (uint32_t j0 = 0; j0 < pq_dim; j0 += per) {
+    const uint32_t j = j0 + tid / book;
+    float dot = -FLT_MAX, mag = 0.0f;
+    if (j < pq_dim) {
+      dot = 0.0f;
+      for (uint32_t t = 0; t < pq_len; t++) {
+        const float prod = qrow[j * pq_len + t] * pq_centers[(uint64_t(j) * pq_len + t) * book + code];
+        dot += prod;
+        mag += fabsf(prod);
+      }
+    }
+    // maxima over the `book` lanes of a subspace
+    for (uint32_t m = (book < 64u ? book : 64u) >> 1; m >= 1u; m >>= 1) {
+      dot = fmaxf(dot, __shfl_xor(dot, int(m), 64));
+      mag = fmaxf(mag, __shfl_xor(mag, int(m), 64));
+    }
+    if (book == 256u) {
+      if ((tid & 63u) == 0u) {
+        s_u[tid >> 6] = dot;
+        s_w[tid >> 6] = mag;
+      }
+      __syncthreads();
+      if (tid == 0 && j < pq_dim) {
+        out[uint64_t(q) * pq_dim + j] = make_float2(fmaxf(fmaxf(s_u[0], s_u[1]), fmaxf(s_u[2], s_u[3])),
+                                                    fmaxf(fmaxf(s_w[0], s_w[1]), fmaxf(s_w[2], s_w[3])));
+      }
+      __syncthreads();
+    } else if (code == 0u && j < pq_dim) {
+      out[uint64_t(q) * pq_dim + j] = make_float2(dot, mag);
+    }
+  }
+}
+
+__device__ __forceinline__ float wave_sum_f32(float v)
+{
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) { v += __shfl_xor(v, m, 64); }
+  return v;
+}
+
+/** The product as its own rounded fp32 number (the table's term c q is rounded before it is
+ *  subtracted: the compiler must not fuse it into the subtraction). */
+__device__ __forceinline__ float rounded_product(float x, float y)
+{
+  float p = x * y;
+  asm volatile("" : "+v"(p));
+  return p;
+}
+
+template <int PQ_LEN, int LUT, bool OUT_HALF, int BITS>
+__global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_ip_kernel(
+  scan_args a, const pair_desc* __restrict__ desc, uint32_t n_pairs, const float2* __restrict__ qbounds,
+  pair_desc* __restrict__ survivors, uint32_t* __restrict__ n_survivors, uint8_t* __restrict__ alive)
+{
+  using traits = lut_traits<LUT>;
+  using lut_t  = typename traits::storage;
+  using acc_t  = typename std::conditional<OUT_HALF, _Float16, float>::type;
+  using vec_t  = typename book_vec<PQ_LEN>::type;
+  static_assert(BITS == 8 || BITS == 4, "byte or nibble codes");
+  constexpr uint32_t SUB  = BITS == 8 ? kDirectSubs : 2u * kDirectSubs;  // subspaces in a row's 8 leading bytes
+  constexpr uint32_t BOOK = 1u << BITS;
+  constexpr int FIRST     = BITS == 8 ? 2 : 4;
+  constexpr int MID       = BITS == 8 ? 4 : 8;
+  static_assert(SUB * PQ_LEN <= 64, "the leading subspaces' terms sit in the lanes of a register per component");
+  auto* book      = reinterpret_cast<LDS_AS vec_t*>(uintptr_t(kScreenLdsBase));
+  const float one = opaque_one_s();
+  constexpr uint32_t off_pending = kScreenLdsBase + SUB * BOOK * uint32_t(sizeof(vec_t));
+
+  const uint32_t tid  = threadIdx.x;
+  const uint32_t lane = tid & 63u;
+  const uint32_t wid  = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr uint32_t WPB = kDirectThreads / 64u;
+  const uint32_t total   = gridDim.x * WPB;
+  if (blockIdx.x * WPB >= n_pairs) { return; }
+  for (uint32_t e = tid; e < SUB * BOOK; e += kDirectThreads) {
+    vec_t v = {};
+#pragma unroll
+    for (int t = 0; t < PQ_LEN; t++) { v[t] = a.pq_centers[((e / BOOK) * PQ_LEN + t) * BOOK + (e % BOOK)]; }
+    book[e] = v;
+  }
+  lds_barrier_s();
+  auto* pending      = reinterpret_cast<LDS_AS uint32_t*>(uintptr_t(off_pending + wid * kSurvivorBatchBytes));
+  uint32_t n_pending = 0;
+  const auto* plane  = reinterpret_cast<const GLOBAL_AS u32x2*>(reinterpret_cast<uintptr_t>(a.lead_plane));
+  const bool cosine  = a.metric == int(DistanceType::CosineExpanded);
+  const uint32_t M   = a.pq_dim;
+
+  /** The entry as the scan adds it, widened to the type of the sums. */
+  auto widen = [&](float x) -> float {
+    const lut_t e = traits::encode(x);
+    return OUT_HALF ? float(traits::to_half(e)) : traits::to_float(e);
+  };
+
+  for (uint32_t p = blockIdx.x * WPB + wid; p < n_pairs; p += total) {
+    pair_desc d = desc[p];
+    {
+      const uint64_t ptr = reinterpret_cast<uint64_t>(d.data);
+      const uint32_t hi  = uint32_t(__builtin_amdgcn_readfirstlane(uint32_t(ptr >> 32)));
+      const uint32_t lo  = uint32_t(__builtin_amdgcn_readfirstlane(uint32_t(ptr)));
+      d.data       = reinterpret_cast<const uint8_t*>((uint64_t(hi) << 32) | uint64_t(lo));
+      d.q          = uint32_t(__builtin_amdgcn_readfirstlane(d.q));
+      d.slot       = uint32_t(__builtin_amdgcn_readfirstlane(d.slot));
+      d.label      = uint32_t(__builtin_amdgcn_readfirstlane(d.label));
+      d.sample_off = uint32_t(__builtin_amdgcn_readfirstlane(d.sample_off));
+      d.n_rows     = uint32_t(__builtin_amdgcn_readfirstlane(d.n_rows));
+      d.row_off    = uint32_t(__builtin_amdgcn_readfirstlane(d.row_off));
+    }
+    const uint32_t n_rows = d.n_rows;
+    if (n_rows == 0) { continue; }
+    const uint32_t thr = uint32_t(__builtin_amdgcn_readfirstlane(a.query_kth[d.q]));
+    // no bound yet (fewer than k candidates so far): nothing can be dropped
+    const bool bounded = thr < 0xFF800000u;
+    const float thr_f  = bounded ? unorder_f32(thr) : __uint_as_float(0x7F800000u);
+
+    /* ---- the least each subspace can add: lane l takes subspaces l, l + 64, ... ---- */
+    const float* qrow  = a.rot_q + uint64_t(d.q) * a.rot_dim;
+    const float* crow  = a.centers_rot + uint64_t(d.label) * a.rot_dim;
+    const float2* brow = qbounds + uint64_t(d.q) * M;
+    float q0[PQ_LEN], tc0[PQ_LEN];  // terms of subspace `lane` (the leading subspaces are lanes 0 .. SUB - 1)
+    float lows[kIpRounds];          // least entry of subspace r * 64 + lane (0 past the last subspace)
+    float low_sum = 0.0f, mag_sum = 0.0f;
+#pragma unroll
+    for (uint32_t r = 0; r < kIpRounds; r++) {
+      lows[r] = 0.0f;
+      if (r * 64u >= M) { continue; }  // uniform
+      const uint32_t j = r * 64u + lane;
+      float low = 0.0f, mag = 0.0f;
+      float qv[PQ_LEN], tcv[PQ_LEN];
+#pragma unroll
+      for (int t = 0; t < PQ_LEN; t++) {
+        qv[t]  = 0.0f;
+        tcv[t] = 0.0f;
+      }
+      if (j < M) {
+        float t_sum = 0.0f, t_abs = 0.0f;
+#pragma unroll
+        for (int t = 0; t < PQ_LEN; t++) {
+          qv[t]  = qrow[j * PQ_LEN + t];
+          tcv[t] = rounded_product(crow[j * PQ_LEN + t], qv[t]);
+          t_sum += tcv[t];
+          t_abs += fabsf(tcv[t]);
+        }
+        const float2 uw = brow[j];
+        mag             = t_abs + uw.y;
+        // below every entry's fp32 value: the exact minimum less 2^-20 of the magnitudes (the
+        // evaluation of an entry makes 2 pq_len roundings of at most 2^-24 of them each)
+        const float x = -t_sum - uw.x - mag * 0x1.0p-20f;
+        low           = widen(x);
+        // the table's rounding may enlarge a magnitude (8-bit entries by up to an eighth)
+        mag = fmaxf(mag, fabsf(low)) * 1.25f;
+      }
+      if (r == 0) {
+#pragma unroll
+        for (int t = 0; t < PQ_LEN; t++) {
+          q0[t]  = qv[t];
+          tc0[t] = tcv[t];
+        }
+      }
+      lows[r] = low;
+      low_sum += low;
+      mag_sum += mag;
+    }
+
+    /* ---- thresholds of the rows' partial sums after FIRST, MID and SUB subspaces: a row whose sum
+     * is above stop[c] (binary16 sums: at or above it) after at[c] subspaces is out ---- */
+    float stop[3]   = {__uint_as_float(0x7F800000u), __uint_as_float(0x7F800000u), __uint_as_float(0x7F800000u)};
+    const int at[3] = {FIRST, MID, int(SUB)};
+    if (bounded) {
+      const float all = wave_sum_f32(low_sum);
+      float rest[3];  // what the subspaces from at[c] on add at least
+#pragma unroll
+      for (int c = 0; c < 3; c++) {
+        rest[c] = all - wave_sum_f32(lane < uint32_t(at[c]) ? lows[0] : 0.0f) + (cosine ? 1.0f : 0.0f);
+      }
+      if constexpr (!OUT_HALF) {
+        // rounding of the scan's additions, of the sums above and of the expression below
+        const float slack = float(M + 2u) * 0x1.0p-22f * (wave_sum_f32(mag_sum) + 1.0f);
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+          stop[c] = thr_f - rest[c] + slack + (fabsf(thr_f) + fabsf(rest[c]) + 1.0f) * 0x1.0p-21f;
+        }
+      } else {
+        // binary16 sums.  The chain of a hypothetical row that adds the least entry of every
+        // subspace from at[c] on, in the scan's order and type: 21 lanes per checkpoint start it
+        // from values around thr - rest[c], four units in the last place apart; the smallest start
+        // that ends above the bound is the checkpoint's threshold.
+        const uint32_t grp = lane >= 42u ? 2u : (lane >= 21u ? 1u : 0u);
+        const float mid    = thr_f - (grp == 0 ? rest[0] : (grp == 1 ? rest[1] : rest[2]));
+        int expo           = 0;
+        (void)frexpf(mid, &expo);  // |mid| in [2^(expo-1), 2^expo)
+        expo               = expo < -13 ? -13 : expo;
+        const float step   = ldexpf(1.0f, expo - 11 + 2);  // four ulps of binary16 at mid's magnitude
+        _Float16 x         = _Float16(mid + (float(lane - grp * 21u) - 13.0f) * step);
+        const _Float16 start = x;
+        const uint32_t from  = grp == 0 ? uint32_t(FIRST) : (grp == 1 ? uint32_t(MID) : SUB);  // the lane's first subspace
+#pragma unroll
+        for (uint32_t r = 0; r < kIpRounds; r++) {
+          if (r * 64u >= M) { continue; }  // uniform
+          const uint32_t lowbits = uint32_t(__builtin_bit_cast(uint16_t, _Float16(lows[r])));  // exact: a binary16 number
+#pragma unroll
+          for (int l = 0; l < 64; l++) {
+            if (r == 0 && l < FIRST) { continue; }
+            const _Float16 add = __builtin_bit_cast(_Float16, uint16_t(__builtin_amdgcn_readlane(int(lowbits), l)));
+            if (r == 0 && l < int(SUB)) {
+              x = _Float16(x + (uint32_t(l) >= from ? add : _Float16(0)));
+            } else {
+              x = _Float16(x + add);
+            }
+          }
+        }
+        if (cosine) { x = _Float16(x + _Float16(1)); }
+        // a chain is monotone in its starting value: the lanes of a group that end above the bound are an upper range
+        const unsigned long long over = __builtin_amdgcn_ballot_w64(float(x) > thr_f);
+        const uint32_t startbits      = uint32_t(__builtin_bit_cast(uint16_t, start));
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+          const unsigned long long mine = over & (c == 0 ? 0x1FFFFFull : (c == 1 ? 0x1FFFFFull << 21 : ~0ull << 42));
+          if (mine != 0ull) {
+            stop[c] = float(__builtin_bit_cast(_Float16, uint16_t(__builtin_amdgcn_readlane(int(startbits), __builtin_ctzll(mine)))));
+          }
+        }
+      }
+    }
+
+    /* ---- the rows' leading codes ---- */
+    const uint32_t n_tiles = (n_rows + 63u) >> 6;
+    bool in_play           = false;
+    u32x2 cur              = plane[uint64_t(d.row_off) + lane];
+    for (uint32_t tile = 0; tile < n_tiles && !in_play; tile++) {
+      // (the plane carries slack past the last list: the load needs no condition)
+      const u32x2 ahead = plane[uint64_t(d.row_off) + (tile + 1u) * 64u + lane];
+      const unsigned long long rows =
+        tile * 64u + 64u <= n_rows ? ~0ull : (1ull << (n_rows & 63u)) - 1ull;
+      const uint32_t w[2] = {cur.x, cur.y};
+      acc_t acc           = acc_t(0);
+      auto add_codes = [&](int first, int last) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kk = first; kk < last; kk++) {
+          const uint32_t c = BITS == 8 ? (w[kk >> 2] >> ((kk & 3) * 8)) & 0xffu : (w[kk >> 3] >> ((kk & 7) * 4)) & 0xfu;
+          const vec_t b    = book[kk * int(BOOK) + c];
+          float score      = 0.0f;
+#pragma unroll
+          for (int t = 0; t < PQ_LEN; t++) {
+            const float tc = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tc0[t]), kk));
+            const float qv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(q0[t]), kk));
+            score -= tc;
+            score = fmaf(-qv, b[t], score);
+          }
+          const lut_t v = traits::encode(score);
+          if (OUT_HALF) {
+            acc = acc_t(acc + traits::to_half(v));
+          } else if (LUT == LUT_F16) {
+            acc = acc_t(fmaf(traits::to_float(v), one, float(acc)));
+          } else {
+            acc = acc_t(acc + traits::to_float(v));
+          }
+        }
+      };
+      // still open: at or below the threshold (binary16 sums: below it)
+      auto open = [&](int c) __attribute__((always_inline)) {
+        const bool mine = OUT_HALF ? float(acc) < stop[c] : float(acc) <= stop[c];
+        return (__builtin_amdgcn_ballot_w64(mine) & rows) != 0ull;
+      };
+      add_codes(0, FIRST);
+      in_play = open(0);
+      if (in_play) {
+        add_codes(FIRST, MID);
+        in_play = open(1);
+      }
+      if (in_play) {
+        add_codes(MID, int(SUB));
+        in_play = open(2);
+      }
+      cur = ahead;
+    }
+    if (in_play) { push_survivor(pending, n_pending, lane, d, survivors, n_survivors, alive); }
+  }
+  if (n_pending != 0) { flush_survivors(pending, n_pending, lane, survivors, n_survivors); }
+}
+
+template <int PQ_LEN, int LUT, bool OUT_HALF, int BITS>
+void launch_screen_ip_instance(const scan_args& a, const pair_desc* desc, uint32_t n_pairs, const float2* qbounds,
+                               pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive, hipStream_t stream)
+{
+  auto kernel       = scan_screen_ip_kernel<PQ_LEN, LUT, OUT_HALF, BITS>;
+  const size_t smem = kScreenLdsBase + size_t(kDirectSubs) * (BITS == 8 ? 256 : 32) * sizeof(typename book_vec<PQ_LEN>::type) +
+                      size_t(kDirectThreads / 64u) * kSurvivorBatchBytes;
+  static const int per_cu = prepare_persistent_kernel(kernel, kDirectThreads, smem, smem);
+  constexpr uint32_t wpb = kDirectThreads / 64u;
+  uint32_t grid          = uint32_t(device_cu_count()) * uint32_t(per_cu);
+  const uint32_t needed  = (n_pairs + wpb - 1u) / wpb;
+  if (grid > needed) { grid = needed; }
+  kernel<<<grid, kDirectThreads, smem, stream>>>(a, desc, n_pairs, qbounds, survivors, n_survivors, alive);
+  CUVS_HIP_TRY(hipGetLastError());
+}
+
+template <int PQ_LEN, int BITS>
+void launch_screen_ip_types(const scan_args& a, const pair_desc* desc, uint32_t n_pairs, const float2* qbounds,
+                            pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive, hipStream_t s)
+{
+  if (!a.out_half) {
+    if (a.lut_dtype == CUDA_R_32F) {
+      launch_screen_ip_instance<PQ_LEN, LUT_F32, false, BITS>(a, desc, n_pairs, qbounds, survivors, n_survivors, alive, s);
+    } else if (a.lut_dtype == CUDA_R_16F) {
+      launch_screen_ip_instance<PQ_LEN, LUT_F16, false, BITS>(a, desc, n_pairs, qbounds, survivors, n_survivors, alive, s);
+    } else {
+      launch_screen_ip_instance<PQ_LEN, LUT_FP8S, false, BITS>(a, desc, n_pairs, qbounds, survivors, n_survivors, alive, s);
+    }
+  } else {
+    if (a.lut_dtype == CUDA_R_16F) {
+      launch_screen_ip_instance<PQ_LEN, LUT_F16, true, BITS>(a, desc, n_pairs, qbounds, survivors, n_survivors, alive, s);
+    } else {
+      launch_screen_ip_instance<PQ_LEN, LUT_FP8S, true, BITS>(a, desc, n_pairs, qbounds, survivors, n_survivors, alive, s);
+    }
+  }
+}
+
 }  // namespace
 
 uint32_t scan_screen_bytes_per_row(bool per_cluster, bool lead_plane)
@@ -670,8 +1027,20 @@ uint32_t scan_screen_bytes_per_row(bool per_cluster, bool lead_plane)
   return kScreenSubs <= 8 ? 8u : 16u;
 }
 
+bool scan_screen_ip(const scan_args& a)
+{
+  const bool ip = a.metric == int(DistanceType::InnerProduct) || a.metric == int(DistanceType::CosineExpanded);
+  if (!ip || !a.fused || (a.pq_bits != 8 && a.pq_bits != 4) || a.pq_dim < 32) { return false; }
+  if (a.lut_dtype == CUDA_R_32F && a.out_half) { return false; }
+  // per-subspace codebooks (the bound's query part is per query then) and the plane of leading codes
+  if (a.per_cluster || a.lead_plane == nullptr || a.rot_dim != a.pq_dim * a.pq_len) { return false; }
+  if (a.pq_dim > 64u * kIpRounds) { return false; }
+  return a.pq_len == 1 || a.pq_len == 2 || a.pq_len == 4;
+}
+
 bool scan_screen_supported(const scan_args& a)
 {
+  if (scan_screen_ip(a)) { return true; }
   const bool l2 = a.metric == int(DistanceType::L2Expanded) || a.metric == int(DistanceType::L2SqrtExpanded);
   if (!l2 || !a.fused || (a.pq_bits != 8 && a.pq_bits != 4) || a.pq_dim < 32) { return false; }
   if (a.lut_dtype == CUDA_R_32F && a.out_half) { return false; }
@@ -683,12 +1052,38 @@ bool scan_screen_supported(const scan_args& a)
   return a.pq_len == 1 || a.pq_len == 2 || a.pq_len == 3 || a.pq_len == 4 || a.pq_len == 8;
 }
 
+size_t scan_screen_scratch_bytes(const scan_args& a, uint32_t n_queries)
+{
+  return scan_screen_ip(a) ? size_t(n_queries) * a.pq_dim * sizeof(float2) : 0;
+}
+
 void launch_scan_screen(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
-                        pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
+                        pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive, void* scratch,
                         hipStream_t stream)
 {
   CUVS_EXPECTS(scan_screen_supported(a), "the screening pass does not cover these search arguments");
   if (n_pairs == 0) { return; }
+  if (scan_screen_ip(a)) {
+    CUVS_EXPECTS(scratch != nullptr, "the screen of an inner-product search needs its scratch buffer");
+    auto* qbounds = static_cast<float2*>(scratch);
+    ip_query_bounds_kernel<<<a.n_queries, 256, 0, stream>>>(a.rot_q, a.pq_centers, a.pq_dim, a.pq_len, 1u << a.pq_bits,
+                                                          a.rot_dim, qbounds);
+    CUVS_HIP_TRY(hipGetLastError());
+    auto by_bits = [&](auto len) {
+      constexpr int PQ_LEN = decltype(len)::value;
+      if (a.pq_bits == 8) {
+        launch_screen_ip_types<PQ_LEN, 8>(a, desc, n_pairs, qbounds, survivors, n_survivors, alive, stream);
+      } else {
+        launch_screen_ip_types<PQ_LEN, 4>(a, desc, n_pairs, qbounds, survivors, n_survivors, alive, stream);
+      }
+    };
+    switch (a.pq_len) {
+      case 1: by_bits(std::integral_constant<int, 1>{}); break;
+      case 2: by_bits(std::integral_constant<int, 2>{}); break;
+      default: by_bits(std::integral_constant<int, 4>{}); break;
+    }
+    return;
+  }
   auto by_kind = [&](auto len) {
     constexpr int PQ_LEN = decltype(len)::value;
     if (a.per_cluster) {

@@ -418,8 +418,10 @@ void search(cuvs::resources const& res_c,
   /* workspace carve-up for one batch */
   res.reset_workspace();
   const bool fast_coarse = coarse_fast_applies(res, params, ix, P);
+  const size_t screen_scratch_bytes = a256(detail::scan_screen_scratch_bytes(sa, Qb));
   const size_t workspace_bytes = pl.fixed_bytes + size_t(Qb) * (pl.per_query_bytes + 64) + 16 * 256 +
-                                 global_lut_bytes + (fast_coarse ? coarse_fast_bytes(ix, Qb) : 0);
+                                 global_lut_bytes + (fast_coarse ? coarse_fast_bytes(ix, Qb) : 0) +
+                                 screen_scratch_bytes;
   CUVS_EXPECTS(!res.workspace_borrowed() || workspace_bytes <= res.workspace_capacity(),
                "a batch of %u queries (n_probes = %u, k = %u, n_lists = %u) needs %zu bytes of workspace; "
                "the fixed workspace of this call holds %zu: pass fewer queries per call or lower "
@@ -504,11 +506,13 @@ void search(cuvs::resources const& res_c,
   uint8_t* alive               = nullptr;
   uint32_t* n_survivors        = nullptr;
   uint8_t* merge_redo          = nullptr;
+  void* screen_scratch         = nullptr;
   if (early_stop) {
     survivors   = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));
     alive       = static_cast<uint8_t*>(res.workspace_alloc(size_t(Qb) * P));
     n_survivors = static_cast<uint32_t*>(res.workspace_alloc(256));
     merge_redo  = static_cast<uint8_t*>(res.workspace_alloc(size_t(Qb)));
+    if (screen_scratch_bytes != 0) { screen_scratch = res.workspace_alloc(screen_scratch_bytes); }
   }
   if (pl.fused) {
     keys = static_cast<unsigned long long*>(res.workspace_alloc(size_t(Qb) * P * kpp * 8));
@@ -614,7 +618,7 @@ void search(cuvs::resources const& res_c,
       mark(5);
       // 2. every other pair on its first chunk only
       detail::launch_scan_screen(sa, desc + size_t(nq) * lead, nq * (P - lead), survivors, n_survivors,
-                                 alive, s);
+                                 alive, screen_scratch, s);
       if (observe_screen) {
         // the survivor count follows the search to the host, for the searches after this one
         observe_screen = false;
