@@ -477,7 +477,9 @@ struct merge_args {
   const int64_t* const* inds_ptrs;
   int64_t* neighbors;  // [n_queries, k]
   float* distances;    // [n_queries, k]
+  unsigned long long* out_scratch;  // k beyond kMergeLdsK: [n_queries, next_pow2(k)] keys (else null)
 };
+constexpr uint32_t kMergeLdsK = 8192;  // the selection's output of up to this many keys sits in LDS
 void launch_merge(const merge_args& a, hipStream_t stream);
 
 /** Exact re-ranking of candidates (refine.hip): ids and distances of the k best candidates of every

@@ -1203,7 +1203,8 @@ __device__ void merge_query(const merge_args& a, uint32_t out_cap, uint32_t q)
 {
   extern __shared__ __align__(16) unsigned char dyn_smem[];
   __shared__ select_smem sm;
-  unsigned long long* out = reinterpret_cast<unsigned long long*>(dyn_smem);
+  unsigned long long* out = a.out_scratch != nullptr ? a.out_scratch + uint64_t(q) * out_cap
+                                                     : reinterpret_cast<unsigned long long*>(dyn_smem);
   uint32_t n;
   if (a.fused) {
     n                              = a.n_probes * a.keys_per_pair;
@@ -1840,7 +1841,7 @@ void launch_merge(const merge_args& a, hipStream_t stream)
 {
   if (a.n_queries == 0) { return; }
   const uint32_t out_cap = next_pow2(a.k);
-  const size_t smem      = size_t(out_cap) * 8;
+  const size_t smem      = a.out_scratch != nullptr ? 0 : size_t(out_cap) * 8;
   CUVS_EXPECTS(smem <= 96 * 1024, "k (%u) is too large for the merge kernel", a.k);
   if (smem > 32 * 1024) {
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(merge_kernel),

@@ -16,7 +16,6 @@ namespace cuvs::neighbors::ivf_pq::detail {
 
 namespace {
 
-constexpr uint32_t kRefineMaxCandidates = 4096;
 
 template <typename T>
 struct refine_acc {
@@ -39,14 +38,18 @@ __global__ __launch_bounds__(kBlock) void refine_kernel(const T* __restrict__ da
                                                          uint32_t n_candidates, uint32_t k,
                                                          uint32_t out_cap, int sqrt_out,
                                                          int64_t* __restrict__ indices,
-                                                         float* __restrict__ distances)
+                                                         float* __restrict__ distances,
+                                                         unsigned long long* __restrict__ scratch)
 {
   using acc_t = typename refine_acc<T>::type;
   extern __shared__ __align__(16) unsigned char dyn_smem[];
   __shared__ select_smem sm;
-  auto* keys = reinterpret_cast<unsigned long long*>(dyn_smem);                  // [n_candidates]
-  auto* out  = keys + n_candidates;                                              // [out_cap]
-  auto* sq   = reinterpret_cast<acc_t*>(out + out_cap);                          // [dim]
+  // keys [n_candidates] and the selection's output [out_cap]: in LDS, or (more candidates than LDS
+  // holds) in the block's part of a global scratch buffer
+  auto* keys = scratch != nullptr ? scratch + uint64_t(blockIdx.x) * (uint64_t(n_candidates) + out_cap)
+                                  : reinterpret_cast<unsigned long long*>(dyn_smem);
+  auto* out  = keys + n_candidates;
+  auto* sq   = scratch != nullptr ? reinterpret_cast<acc_t*>(dyn_smem) : reinterpret_cast<acc_t*>(out + out_cap);  // [dim]
   const uint32_t tid  = threadIdx.x;
   const uint32_t lane = tid & 63u;
   const uint32_t wid  = tid >> 6;
@@ -102,9 +105,15 @@ void launch_refine_typed(const void* dataset, const void* queries, const int64_t
                          hipStream_t stream)
 {
   const uint32_t out_cap = next_pow2(k);
-  const size_t smem      = size_t(n_candidates) * 8 + size_t(out_cap) * 8 + size_t(dim) * 4;
-  CUVS_EXPECTS(smem <= 150 * 1024, "refine: n_candidates (%u), k (%u) and dim (%u) need %zu bytes of LDS",
-               n_candidates, k, dim, smem);
+  size_t smem            = size_t(n_candidates) * 8 + size_t(out_cap) * 8 + size_t(dim) * 4;
+  // more than LDS holds: the keys live in a scratch buffer for the duration of the call
+  device_buffer scratch;
+  if (smem > 150 * 1024) {
+    scratch.allocate(size_t(n_queries) * (size_t(n_candidates) + out_cap) * 8);
+    smem = size_t(dim) * 4;
+    CUVS_EXPECTS(smem <= 150 * 1024, "refine: dim (%u) is too large", dim);
+  }
+  auto* d_scratch = scratch.as<unsigned long long>();
   auto launch = [&](auto kernel) {
     if (smem > 32 * 1024) {
       CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -113,8 +122,10 @@ void launch_refine_typed(const void* dataset, const void* queries, const int64_t
     kernel<<<n_queries, kBlock, smem, stream>>>(static_cast<const T*>(dataset),
                                                 static_cast<const T*>(queries), candidates, n_rows,
                                                 dim, n_candidates, k, out_cap, sqrt_out ? 1 : 0,
-                                                indices, distances);
+                                                indices, distances, d_scratch);
     CUVS_HIP_TRY(hipGetLastError());
+    // the buffer goes back when this function returns: the kernel must be through with it
+    if (d_scratch != nullptr) { CUVS_HIP_TRY(hipStreamSynchronize(stream)); }
   };
   if (ip) {
     launch(refine_kernel<T, true>);
@@ -158,8 +169,6 @@ void launch_refine(const void* dataset, const void* queries, elem_type type,
                    float* distances, hipStream_t stream)
 {
   if (n_queries == 0) { return; }
-  CUVS_EXPECTS(n_candidates <= kRefineMaxCandidates, "refine: at most %u candidates per query (got %u)",
-               kRefineMaxCandidates, n_candidates);
   switch (type) {
     case elem_type::f32:
       launch_refine_typed<float>(dataset, queries, candidates, n_rows, n_queries, dim, n_candidates, k, ip, sqrt_out, indices, distances, stream);

@@ -38,7 +38,6 @@ namespace {
 using detail::index_impl;
 
 constexpr uint32_t kMaxFusedK = 256;   // larger k dumps all scores and selects afterwards
-constexpr uint32_t kMaxK      = 8192;  // bound of the per-query selection buffer in LDS
 constexpr size_t kMaxLds      = 160 * 1024;
 constexpr uint32_t kFewPairs  = 1024;  // (query, probe) pairs of a batch below which they are scanned in one plain launch
 
@@ -95,7 +94,8 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
   p.per_query_bytes = size_t(ix.dim) * 4 + size_t(ix.dim_ext) * 4 + size_t(ix.n_lists) * 4 +
                       size_t(ix.rot_dim) * 4 +
                       P * 4 * 3 + P * (2 * sizeof(detail::pair_desc) + 1) + 17 + P * 17 +
-                      (p.fused ? P * k * 8 * 4 : size_t(p.max_samples) * 4);
+                      (p.fused ? P * k * 8 * 4 : size_t(p.max_samples) * 4) +
+                      (k > detail::kMergeLdsK ? size_t(next_pow2(k)) * 8 : 0);
   p.fixed_bytes = a256(size_t(ix.n_lists) * 16 + 16) + 3 * 256 + size_t(512) * 8 + a256(size_t(ix.dim_ext) * 128 * 4) + a256(detail::kSelectSlackBytes) + 20 * 256;
   if (ix.coarse_fast_ok) {
     // buffers of the two-precision probe selection (the batch must fit with them)
@@ -148,8 +148,6 @@ void validate(const search_params& params, const index_impl& ix, int64_t k)
   CUVS_EXPECTS(params.coarse_search_dtype == CUDA_R_32F || params.coarse_search_dtype == CUDA_R_16F ||
                  params.coarse_search_dtype == CUDA_R_8I,
                "Unsupported coarse_search_dtype (only CUDA_R_32F, CUDA_R_16F, and CUDA_R_8I are supported)");
-  CUVS_EXPECTS(k <= kMaxK, "parameter `k` (%lld) must not exceed %u", static_cast<long long>(k),
-               kMaxK);
 }
 
 /** Probes per query whose lists are scanned in full before the others are screened against the
@@ -514,6 +512,11 @@ void search(cuvs::resources const& res_c,
     merge_redo  = static_cast<uint8_t*>(res.workspace_alloc(size_t(Qb)));
     if (screen_scratch_bytes != 0) { screen_scratch = res.workspace_alloc(screen_scratch_bytes); }
   }
+  // k beyond what the merge's LDS holds: its selection writes into global memory
+  unsigned long long* merge_scratch = nullptr;
+  if (k > detail::kMergeLdsK) {
+    merge_scratch = static_cast<unsigned long long*>(res.workspace_alloc(size_t(Qb) * next_pow2(k) * 8));
+  }
   if (pl.fused) {
     keys = static_cast<unsigned long long*>(res.workspace_alloc(size_t(Qb) * P * kpp * 8));
   } else {
@@ -670,6 +673,7 @@ void search(cuvs::resources const& res_c,
     ma.inds_ptrs     = ix.inds_ptrs.as<const int64_t*>();
     ma.neighbors     = neighbors + q0 * k;
     ma.distances     = distances + q0 * k;
+    ma.out_scratch   = merge_scratch;
     detail::launch_merge(ma, s);
     mark(4);
 
