@@ -108,12 +108,6 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
   b        = std::max<size_t>(b, 1);
   b        = std::min<size_t>(b, std::max<uint32_t>(params.max_internal_batch_size, 1u));
   b        = std::min<size_t>(b, n_queries);
-  if (res.workspace_borrowed()) {
-    // a fixed workspace does not shrink the batch behind the caller's back: one internal batch
-    // (n_queries, or max_internal_batch_size of them) has to fit, or the call is refused
-    const size_t want = std::min<size_t>(n_queries, std::max<uint32_t>(params.max_internal_batch_size, 1u));
-    b                 = want;
-  }
   // keep the pair count of a batch within uint32 indexing
   while (b > 1 && b * P >= (size_t(1) << 31)) { b /= 2; }
   // batches of equal size: 10,000 queries at a limit of 4096 run as 3 x 3334, not 4096 + 4096 + 1808
@@ -356,7 +350,7 @@ void search(cuvs::resources const& res_c,
                                     uint32_t(n_queries), params.n_probes, k, ix.dim);
   const plan pl     = make_plan(res, params, ix, uint32_t(n_queries), k);
   const uint32_t P  = pl.n_probes;
-  const uint32_t Qb = pl.batch;
+  uint32_t Qb       = pl.batch;
   hipStream_t s     = res.stream();
 
   detail::scan_args sa{};
@@ -416,15 +410,25 @@ void search(cuvs::resources const& res_c,
   /* workspace carve-up for one batch */
   res.reset_workspace();
   const bool fast_coarse = coarse_fast_applies(res, params, ix, P);
+  auto bytes_for = [&](uint32_t batch) {
+    return pl.fixed_bytes + size_t(batch) * (pl.per_query_bytes + 64) + 16 * 256 + global_lut_bytes +
+           (fast_coarse ? coarse_fast_bytes(ix, batch) : 0) + a256(detail::scan_screen_scratch_bytes(sa, batch));
+  };
+  if (res.workspace_borrowed()) {
+    // a fixed workspace: the largest internal batch that fits it (results do not depend on how the
+    // queries are batched); only a single query that does not fit is refused
+    while (Qb > 1 && bytes_for(Qb) > res.workspace_capacity()) { Qb -= (Qb + 7) / 8; }
+    if (Qb > 1) {
+      const uint32_t n_batches = uint32_t((n_queries + Qb - 1) / Qb);
+      Qb                       = uint32_t((n_queries + n_batches - 1) / n_batches);
+    }
+  }
   const size_t screen_scratch_bytes = a256(detail::scan_screen_scratch_bytes(sa, Qb));
-  const size_t workspace_bytes = pl.fixed_bytes + size_t(Qb) * (pl.per_query_bytes + 64) + 16 * 256 +
-                                 global_lut_bytes + (fast_coarse ? coarse_fast_bytes(ix, Qb) : 0) +
-                                 screen_scratch_bytes;
+  const size_t workspace_bytes      = bytes_for(Qb);
   CUVS_EXPECTS(!res.workspace_borrowed() || workspace_bytes <= res.workspace_capacity(),
-               "a batch of %u queries (n_probes = %u, k = %u, n_lists = %u) needs %zu bytes of workspace; "
-               "the fixed workspace of this call holds %zu: pass fewer queries per call or lower "
-               "max_internal_batch_size",
-               Qb, P, k, ix.n_lists, workspace_bytes, res.workspace_capacity());
+               "one query (n_probes = %u, k = %u, n_lists = %u) needs %zu bytes of workspace; the fixed "
+               "workspace of this call holds %zu",
+               P, k, ix.n_lists, workspace_bytes, res.workspace_capacity());
   res.reserve_workspace(workspace_bytes);
   auto* qt        = static_cast<float*>(
     res.workspace_alloc(size_t(ix.dim_ext) * detail::coarse_pad(Qb) * 4));

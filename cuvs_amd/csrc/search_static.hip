@@ -10,10 +10,12 @@
  * code object: every GPU the library is loaded on holds its own copy from load to process exit.
  * The kernels are the ones cuvsIvfPqSearch launches and get their buffers as arguments as there.
  *
- * Consequences of the one array per GPU: calls that overlap on one GPU (from several host threads
- * or on several streams) race on it; the array keeps the previous call's contents, and the
- * search initialises every counter, bound and flag it reads (as it must on the cached workspace,
- * which is reused the same way).
+ * Consequences of the one array per GPU: calls on different streams of one GPU take turns (each
+ * waits for an event recorded behind the call before it), but calls issued from several host
+ * threads at once, and captured calls replayed side by side, race on it; the array keeps the
+ * previous call's contents, and the search initialises every counter, bound and flag it reads (as
+ * it must on the cached workspace, which is reused the same way).  A call larger than the array
+ * runs in internal batches that fit; only a single query that does not fit is refused.
  */
 #include <hip/hip_runtime.h>
 
@@ -30,6 +32,10 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 std::mutex scratch_mutex;
 void* scratch_ptr[kMaxDevices] = {};
+// recorded behind every call on a device: the next call's stream waits for it, so that calls on
+// different streams or handles take turns on the one array (not under stream capture: a captured
+// call is ordered by its graph's launches, and two graphs that hold such calls must not overlap)
+hipEvent_t scratch_free[kMaxDevices] = {};
 
 /** Device address of the current device's copy of `scratch` (looked up once per device). */
 void* static_scratch()
@@ -61,9 +67,29 @@ extern "C" cuvsError_t cuvsAmdIvfPqSearchNoAlloc(cuvsResources_t res,
     cuvs::resources* caller = cuvs::core::res_of(res);
     // a handle of this call's own: the caller's stream, the static array as the whole workspace
     cuvs::resources local;
-    local.set_stream(caller->stream());
+    hipStream_t stream = caller->stream();
+    local.set_stream(stream);
+    local.tuning = caller->tuning;
     local.borrow_workspace(static_scratch(), kStaticScratchBytes);
+    int device = 0;
+    CUVS_HIP_TRY(hipGetDevice(&device));
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    CUVS_HIP_TRY(hipStreamIsCapturing(stream, &capture));
+    hipEvent_t turn = nullptr;
+    if (capture == hipStreamCaptureStatusNone) {
+      std::lock_guard<std::mutex> lock(scratch_mutex);
+      if (scratch_free[device] == nullptr) {
+        CUVS_HIP_TRY(hipEventCreateWithFlags(&scratch_free[device], hipEventDisableTiming));
+      } else {
+        CUVS_HIP_TRY(hipStreamWaitEvent(stream, scratch_free[device], 0));
+      }
+      turn = scratch_free[device];
+    }
     cuvs::core::ivf_pq_search_tensors(local, search_params, index, queries, neighbors, distances,
                                       nullptr, 0);
+    if (turn != nullptr) {
+      std::lock_guard<std::mutex> lock(scratch_mutex);
+      CUVS_HIP_TRY(hipEventRecord(turn, stream));
+    }
   });
 }

@@ -1,7 +1,8 @@
 """cuvsAmdIvfPqSearchNoAlloc runs the search on a fixed workspace inside the library and makes no
 device allocation.  Its results must equal cuvsIvfPqSearch's bit for bit, also on a second call
-with a smaller input (the workspace keeps the first call's contents), and a search that does not
-fit the workspace must be refused with a message."""
+with a smaller input (the workspace keeps the first call's contents); a search that does not fit
+the workspace runs in internal batches that do, calls on two streams take turns on it, and the call
+can be captured into a HIP graph."""
 import numpy as np
 import pytest
 import torch
@@ -66,7 +67,7 @@ def test_no_device_allocation_is_made():
     assert free_after == free_before
 
 
-def test_a_search_beyond_the_workspace_is_refused():
+def test_a_search_beyond_the_workspace_runs_in_batches_that_fit():
     index, dim = _index()
     res = Resources()
     n_queries = 20000  # x 256 lists x 4 bytes of coarse scores alone is 20 MB; with k = 100 far beyond 32 MiB
@@ -74,13 +75,69 @@ def test_a_search_beyond_the_workspace_is_refused():
     queries = G.to_dev(H.make_data(n_queries, dim, np.float32, 6, n_components=64))
     nb = torch.full((n_queries, 100), -7, dtype=torch.int64, device="cuda")
     d = torch.empty((n_queries, 100), dtype=torch.float32, device="cuda")
-    with pytest.raises(CuvsError, match="bytes of workspace"):
+    ivf_pq.search_no_alloc(sp, index, queries, nb, d, resources=res)
+    res.sync()
+    want_d, want_nb = ivf_pq.search(sp, index, queries, 100, resources=res)
+    res.sync()
+    assert torch.equal(nb, want_nb) and torch.equal(d, want_d)
+
+
+def test_calls_on_two_streams_take_turns():
+    """Two handles on two streams share the one workspace: the second call waits for the first."""
+    index, dim = _index()
+    sp = ivf_pq.SearchParams(n_probes=20, lut_dtype=np.float16)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    handles, outs, qs = [], [], []
+    for i, st in enumerate(streams):
+        with torch.cuda.stream(st):
+            res = Resources()
+            res.use_torch_current_stream()
+            handles.append(res)
+        qs.append(G.to_dev(H.make_data(300, dim, np.float32, 20 + i, n_components=64)))
+        outs.append((torch.empty((300, 10), dtype=torch.int64, device="cuda"),
+                     torch.empty((300, 10), dtype=torch.float32, device="cuda")))
+    torch.cuda.synchronize()
+    for rep in range(5):
+        for i in range(2):
+            ivf_pq.search_no_alloc(sp, index, qs[i], outs[i][0], outs[i][1], resources=handles[i])
+    torch.cuda.synchronize()
+    ref = Resources()
+    for i in range(2):
+        want_d, want_nb = ivf_pq.search(sp, index, qs[i], 10, resources=ref)
+        ref.sync()
+        assert torch.equal(outs[i][0], want_nb) and torch.equal(outs[i][1], want_d)
+
+
+def test_captured_call_replays_like_eager():
+    """The entry point under HIP graph capture (what it is for): replays on new query contents equal
+    eager searches, with eager work and synchronisations between the replays."""
+    index, dim = _index()
+    n_queries = 200
+    pool = G.to_dev(H.make_data(4 * n_queries, dim, np.float32, 31, n_components=64))
+    sp = ivf_pq.SearchParams(n_probes=20, lut_dtype=np.float16)
+    res = Resources()
+    queries = pool[:n_queries].clone()
+    nb = torch.empty((n_queries, 10), dtype=torch.int64, device="cuda")
+    d = torch.empty((n_queries, 10), dtype=torch.float32, device="cuda")
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        res.use_torch_current_stream()
+        for _ in range(2):
+            ivf_pq.search_no_alloc(sp, index, queries, nb, d, resources=res)
+        res.sync()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        res.use_torch_current_stream()
         ivf_pq.search_no_alloc(sp, index, queries, nb, d, resources=res)
-    assert int((nb != -7).sum()) == 0  # nothing ran
-    # the same search in internal batches that fit is served
-    sp_small = ivf_pq.SearchParams(n_probes=64, lut_dtype=np.float16, max_internal_batch_size=100)
-    ivf_pq.search_no_alloc(sp_small, index, queries[:1000], nb[:1000], d[:1000], resources=res)
-    res.sync()
-    want_d, want_nb = ivf_pq.search(sp_small, index, queries[:1000], 100, resources=res)
-    res.sync()
-    assert torch.equal(nb[:1000], want_nb) and torch.equal(d[:1000], want_d)
+    for rep in range(4):
+        fresh = pool[rep * n_queries:(rep + 1) * n_queries].contiguous()
+        queries.copy_(fresh)
+        graph.replay()
+        torch.cuda.synchronize()
+        got_nb, got_d = nb.clone(), d.clone()
+        res.use_torch_current_stream()
+        want_d, want_nb = ivf_pq.search(sp, index, fresh, 10, resources=res)
+        res.sync()
+        torch.cuda.synchronize()
+        assert torch.equal(got_nb, want_nb) and torch.equal(got_d, want_d), rep
