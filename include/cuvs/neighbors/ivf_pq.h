@@ -214,12 +214,14 @@ CUVS_EXPORT cuvsError_t cuvsAmdIvfPqSearchWithBitset(cuvsResources_t res,
  *  arguments, checks and results as cuvsIvfPqSearch (it runs the same kernels on the stream of
  *  `res`), but the workspace between the stages of the search is a fixed array of
  *  CUVS_AMD_NO_ALLOC_WORKSPACE_BYTES in the library's device image instead of the handle's cached
- *  allocation, and the call makes no hipMalloc / hipFree.  One internal batch
- *  (min(n_queries, max_internal_batch_size) queries) must fit that array, or the call fails with a
- *  message that states the bytes needed: roughly 4 * n_lists + 32 * n_probes * k + 100 * n_probes
- *  + 12 * dim bytes per query (a few hundred queries at 16384 lists, 64 probes, k = 10).  Every
- *  GPU holds one such array: calls that overlap on one GPU race on it.  Profiling
- *  (cuvsAmdIvfPqProfilingEnable) does not apply to this call. */
+ *  allocation, and the call makes no hipMalloc / hipFree.  The queries run in internal batches
+ *  that fit that array (roughly 4 * n_lists + 32 * n_probes * k + 100 * n_probes + 12 * dim bytes
+ *  per query: a few hundred queries a batch at 16384 lists, 64 probes, k = 10; results do not
+ *  depend on the batching); only a single query that does not fit fails, with a message that
+ *  states the bytes needed.  Every GPU holds one such array: calls on different streams take
+ *  turns on it (each waits for an event recorded behind the call before it, except under stream
+ *  capture); calls issued by several host threads at once, and captured calls replayed side by
+ *  side, race on it.  Profiling (cuvsAmdIvfPqProfilingEnable) does not apply to this call. */
 #define CUVS_AMD_NO_ALLOC_WORKSPACE_BYTES ((size_t)32 << 20)
 CUVS_EXPORT cuvsError_t cuvsAmdIvfPqSearchNoAlloc(cuvsResources_t res,
                                                   cuvsIvfPqSearchParams_t search_params,
