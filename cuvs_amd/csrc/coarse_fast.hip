@@ -39,9 +39,6 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr uint32_t kTile    = 64;   // lists per tile
-constexpr uint32_t kQTile   = 256;  // queries per block: 4 waves x 64
-constexpr uint32_t kSlab    = 64;   // the padded dimension is a multiple of this
 constexpr uint32_t kCandCapF = 512;  // candidate slots per query (256 are used up to 128 probes)
 
 template <typename T>
@@ -122,60 +119,79 @@ __global__ void pack_centers_kernel(const float* __restrict__ centers, uint32_t 
 constexpr uint32_t kGemmThreads = 256;
 constexpr uint32_t kLocalCap    = 32;  // PASS 2: candidates a query may collect between two flushes before its block gives up
 constexpr uint32_t kGroup       = 32;  // PASS 1: lists per group minimum (one MFMA tile's rows)
-constexpr uint32_t kMinFlushTiles  = 16;  // PASS 1: list tiles between two flushes: 32 group minima, one 128-byte line of a query's row
-constexpr uint32_t kCandFlushTiles = 8;   // PASS 2: list tiles (512 lists) between two flushes of the candidates
-constexpr uint32_t kMinRow      = kMinFlushTiles * 2u + 4u;  // floats per query in the staged minima (rows 144 bytes apart)
+constexpr uint32_t kMinLine     = 32;  // PASS 1: group minima between two flushes: one 128-byte line of a query's row
+constexpr uint32_t kCandFlushLists = 512;  // PASS 2: lists between two flushes of the candidates
+constexpr uint32_t kMinRow      = kMinLine + 4u;  // floats per query in the staged minima (rows 144 bytes apart)
+
+/** Shape of the GEMM by the padded dimension: MFMA tiles of 32 lists per list tile (NI), MFMA tiles
+ *  of 32 queries per wave (NJ), blocks per CU.  A wave keeps its queries' whole rows in registers
+ *  (K_PAD / 8 registers per query tile), and two buffers of a list tile sit in LDS
+ *  (64 NI (K_PAD + 8) bytes): both shrink as the dimension grows. */
+template <uint32_t K_PAD>
+struct gemm_shape {
+  static constexpr uint32_t NI     = K_PAD <= 256 ? 2 : 1;
+  static constexpr uint32_t NJ     = K_PAD <= 512 ? 2 : 1;
+  static constexpr uint32_t BLOCKS = K_PAD <= 128 ? 2 : 1;
+};
 
 /**
- * fp16 scores s' = alpha * (cn * qterm + dot16(c, q)) of a block's 256 queries against a run of
- * list tiles (64 lists each).  Four waves, one per SIMD, each with 64 of the queries and all 64
- * lists of a tile: four MFMA tiles of v_mfma_f32_32x32x16_f16 (each 16-byte read of the list
- * operand out of LDS feeds two products), the query operand in registers for the whole block.  Two
+ * fp16 scores s' = alpha * (cn * qterm + dot16(c, q)) of a block's queries against a run of list
+ * tiles.  Four waves, one per SIMD, each with 32 NJ of the queries and all 32 NI lists of a tile:
+ * NI x NJ MFMA tiles of v_mfma_f32_32x32x16_f16 (each 16-byte read of the list operand out of LDS
+ * feeds NJ products), the query operand in registers for the whole block.  Up to 128 dimensions two
  * blocks fit a CU, so that one block's matrix products run under the other's epilogue, staging
  * and barrier.  List tiles stream through two LDS buffers, the next tile's global loads in flight
  * while the current one is multiplied (one barrier per tile).  The norm term is the accumulators'
  * starting value.  PASS 1 keeps, per query, the minimum of every group of 32 lists; PASS 2 collects
  * the lists whose score is at or below the query's threshold.  Both results are staged in LDS by
- * the wave that owns the query and written out by that wave every kFlushTiles tiles (the minima
+ * the wave that owns the query and written out by that wave every so many tiles (the minima
  * as whole 128-byte lines; the candidates with one global atomic per query), without a barrier.
  * Both passes execute the same instructions up to the epilogue, so a list's score is the same
- * number in both.  K_PAD = padded dimension (64 or 128).
+ * number in both.  K_PAD = padded dimension.
  */
 template <int PASS, uint32_t K_PAD>
-__global__ __launch_bounds__(kGemmThreads, 2) void coarse_f16_kernel(
+__global__ __launch_bounds__(kGemmThreads, gemm_shape<K_PAD>::BLOCKS) void coarse_f16_kernel(
   const _Float16* __restrict__ ch, const _Float16* __restrict__ qh, const float* __restrict__ cn,
   uint32_t n_lists, uint32_t n_queries, uint32_t q_rows, uint32_t n_list_tiles, uint32_t tiles_per_block, float alpha,
   float qterm, float* __restrict__ minima, uint32_t n_groups, const float* __restrict__ thr,
   uint32_t* __restrict__ cand_count, uint32_t* __restrict__ cand)
 {
+  constexpr uint32_t NI     = gemm_shape<K_PAD>::NI;
+  constexpr uint32_t NJ     = gemm_shape<K_PAD>::NJ;
+  constexpr uint32_t LT     = 32u * NI;          // lists per tile
+  constexpr uint32_t QB     = 4u * 32u * NJ;     // queries per block
+  constexpr uint32_t FLUSH1 = kMinLine / NI;     // PASS 1: list tiles between two flushes
+  constexpr uint32_t FLUSH2 = kCandFlushLists / LT;
   constexpr uint32_t ROWB   = K_PAD * 2u + 16u;  // 16-byte reads of 32 consecutive rows hit all banks
   constexpr uint32_t CHUNKS = K_PAD / 8u;        // 16-byte chunks per row
-  constexpr uint32_t PER_T  = kTile * CHUNKS / kGemmThreads;  // chunks per thread and tile (2 or 4)
+  constexpr uint32_t PER_T  = LT * CHUNKS / kGemmThreads;  // chunks per thread and tile
+  static_assert(LT * CHUNKS % kGemmThreads == 0 && PER_T >= 1 && PER_T <= 16, "a tile's chunks split evenly over the block");
   extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char* sa0 = smem;  // lists [2][64][ROWB], two buffers
-  float* scn         = reinterpret_cast<float*>(smem + 2u * kTile * ROWB);  // [2][64] norm terms
-  uint32_t* lcount   = reinterpret_cast<uint32_t*>(scn + 2u * kTile);       // PASS 2: [256]
-  uint32_t* lcand    = lcount + kQTile;                                     // PASS 2: [256][kLocalCap]
-  float* lmin        = reinterpret_cast<float*>(lcount);  // PASS 1: [256][kMinRow] group minima
+  unsigned char* sa0 = smem;  // lists [2][LT][ROWB], two buffers
+  float* scn         = reinterpret_cast<float*>(smem + 2u * LT * ROWB);  // [2][LT] norm terms
+  uint32_t* lcount   = reinterpret_cast<uint32_t*>(scn + 2u * LT);       // PASS 2: [QB]
+  uint32_t* lcand    = lcount + QB;                                      // PASS 2: [QB][kLocalCap]
+  float* lmin        = reinterpret_cast<float*>(lcount);  // PASS 1: [QB][kMinRow] group minima
   const uint32_t tid  = threadIdx.x;
   const uint32_t lane = tid & 63u;
-  const uint32_t wid  = tid >> 6;  // the wave's quarter of the queries (64)
+  const uint32_t wid  = tid >> 6;  // the wave's quarter of the queries
   const uint32_t half = lane >> 5;
-  const uint32_t q0   = blockIdx.y * kQTile;
+  const uint32_t q0   = blockIdx.y * QB;
   const uint32_t t0   = blockIdx.x * tiles_per_block;
   const uint32_t t1   = t0 + tiles_per_block < n_list_tiles ? t0 + tiles_per_block : n_list_tiles;
   const float neg_inf   = -__uint_as_float(0x7f800000u);
   const float inv_alpha = 1.0f / alpha;
 
-  // this lane's two queries inside the block (columns of the wave's two query tiles); the packed
-  // queries are padded to a multiple of 128 rows, a block's second half may lie beyond them.  The
-  // wave's query operand never changes: it lives in registers.
-  uint32_t qloc[2], q[2];
-  v8h bq[2][K_PAD / 16u];
-  float limit[2] = {0.0f, 0.0f};
+  // this lane's queries inside the block (columns of the wave's query tiles); the packed queries
+  // are padded to a multiple of 128 rows, a block's tail may lie beyond them.  The wave's query
+  // operand never changes: it lives in registers.
+  uint32_t qloc[NJ], q[NJ];
+  v8h bq[NJ][K_PAD / 16u];
+  float limit[NJ];
 #pragma unroll
-  for (int j = 0; j < 2; j++) {
-    qloc[j]             = wid * 64u + uint32_t(j) * 32u + (lane & 31u);
+  for (uint32_t j = 0; j < NJ; j++) {
+    limit[j]            = 0.0f;
+    qloc[j]             = wid * (32u * NJ) + j * 32u + (lane & 31u);
     q[j]                = q0 + qloc[j];
     const uint32_t q_rd = q[j] < q_rows ? q[j] : q_rows - 1u;
 #pragma unroll
@@ -201,19 +217,21 @@ __global__ __launch_bounds__(kGemmThreads, 2) void coarse_f16_kernel(
 #pragma unroll
   for (uint32_t c = 0; c < PER_T; c++) {
     *reinterpret_cast<uint4*>(sa0 + crow[c] * ROWB + cpart[c] * 16u) =
-      *reinterpret_cast<const uint4*>(ch + uint64_t(t0 * kTile + crow[c]) * K_PAD + cpart[c] * 8u);
+      *reinterpret_cast<const uint4*>(ch + uint64_t(t0 * LT + crow[c]) * K_PAD + cpart[c] * 8u);
   }
   // per list: the norm term of the score, and for the padding lists a value no maximum picks
-  if (tid < kTile) {
-    const uint32_t l = t0 * kTile + tid;
+  if (tid < LT) {
+    const uint32_t l = t0 * LT + tid;
     scn[tid]         = l < n_lists ? cn[l] * qterm : neg_inf;
   }
-  if (PASS == 2) { lcount[tid] = 0; }
+  if (PASS == 2) {
+    for (uint32_t x = tid; x < QB; x += kGemmThreads) { lcount[x] = 0; }
+  }
   __syncthreads();
   // Use the query operand once here, so that the compiler's wait for these loads sits here and not
   // inside the loop: there it would also wait for the staged loads below, which it does not count.
 #pragma unroll
-  for (int j = 0; j < 2; j++) {
+  for (uint32_t j = 0; j < NJ; j++) {
 #pragma unroll
     for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) { asm volatile("" : "+v"(bq[j][ks])); }
   }
@@ -231,141 +249,158 @@ __global__ __launch_bounds__(kGemmThreads, 2) void coarse_f16_kernel(
     const uint32_t at = tile < t1 ? tile : t1 - 1u;
 #pragma unroll
     for (uint32_t c = 0; c < PER_T; c++) {
-      const _Float16* src = ch + uint64_t(at * kTile + crow[c]) * K_PAD + cpart[c] * 8u;
+      const _Float16* src = ch + uint64_t(at * LT + crow[c]) * K_PAD + cpart[c] * 8u;
       asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(st[c]) : "v"(src) : "memory");
     }
     // cn has coarse_pad(n_lists) entries: every thread loads one (most of the block a repeat)
-    const float* src = cn + at * kTile + (tid & (kTile - 1u));
+    const float* src = cn + at * LT + (tid & (LT - 1u));
     asm volatile("global_load_dword %0, %1, off" : "=v"(sc) : "v"(src) : "memory");
   };
   auto arrived = [&](u32x4(&st)[PER_T], float& sc) __attribute__((always_inline)) {
-    if constexpr (PER_T == 4) {
-      asm volatile("s_waitcnt vmcnt(0)" : "+v"(st[0]), "+v"(st[1]), "+v"(st[2]), "+v"(st[3]), "+v"(sc) : : "memory");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0)" : "+v"(st[0]), "+v"(st[1]), "+v"(sc) : : "memory");
-    }
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(sc) : : "memory");
+#pragma unroll
+    for (uint32_t c = 0; c < PER_T; c++) { asm volatile("" : "+v"(st[c]) : : "memory"); }
   };
   auto commit = [&](uint32_t tile, uint32_t buf, const u32x4(&st)[PER_T], float sc) __attribute__((always_inline)) {
     const uint32_t at  = tile < t1 ? tile : t1 - 1u;
-    unsigned char* san = sa0 + buf * (kTile * ROWB);
+    unsigned char* san = sa0 + buf * (LT * ROWB);
 #pragma unroll
     for (uint32_t c = 0; c < PER_T; c++) {
       *reinterpret_cast<u32x4*>(san + crow[c] * ROWB + cpart[c] * 16u) = st[c];
     }
-    if (tid < kTile) { scn[buf * kTile + tid] = at * kTile + tid < n_lists ? sc * qterm : neg_inf; }
+    if (tid < LT) { scn[buf * LT + tid] = at * LT + tid < n_lists ? sc * qterm : neg_inf; }
   };
   // products and epilogue of one tile out of LDS buffer `buf`
   auto multiply = [&](uint32_t tile, uint32_t buf) __attribute__((always_inline)) {
-    const unsigned char* sa = sa0 + buf * (kTile * ROWB);
+    const unsigned char* sa = sa0 + buf * (LT * ROWB);
     // element r of an MFMA tile: row (list) (r / 4) * 8 + (lane / 32) * 4 + r % 4, column (query) lane % 32
-    v16f nv[2];  // the norm terms of this lane's rows: where the sums start
+    v16f nv[NI];  // the norm terms of this lane's rows: where the sums start
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
+    for (uint32_t i = 0; i < NI; i++) {
 #pragma unroll
       for (int g = 0; g < 4; g++) {
-        const float4 t = *reinterpret_cast<const float4*>(scn + buf * kTile + uint32_t(i) * 32u + half * 4u + uint32_t(g) * 8u);
+        const float4 t = *reinterpret_cast<const float4*>(scn + buf * LT + i * 32u + half * 4u + uint32_t(g) * 8u);
         nv[i][g * 4 + 0] = t.x;
         nv[i][g * 4 + 1] = t.y;
         nv[i][g * 4 + 2] = t.z;
         nv[i][g * 4 + 3] = t.w;
       }
     }
-    v16f acc[2][2];  // [list tile][query tile]
-#pragma unroll
-    for (uint32_t ks = 0; ks < K_PAD / 16u; ks++) {
+    v16f acc[NI][NJ];  // [list tile][query tile]
+    // The list operand is read DEPTH steps ahead of the product that uses it, and the order is
+    // pinned: left to itself the compiler, short of registers at the larger dimensions, reads each
+    // step into the same registers and waits for it in front of its product (an LDS round trip
+    // per product with nothing else to run on the SIMD).
+    constexpr uint32_t KS    = K_PAD / 16u;
+    constexpr uint32_t DEPTH = KS < 6u ? KS : (NI == 1 ? 6u : 4u);
+    auto read_step = [&](uint32_t ks, v8h(&dst)[NI]) __attribute__((always_inline)) {
       const uint32_t kb = (ks * 16u + half * 8u) * 2u;  // byte offset of this lane's 8 values
-      v8h a[2];
 #pragma unroll
-      for (int i = 0; i < 2; i++) {
-        a[i] = *reinterpret_cast<const v8h*>(sa + (uint32_t(i) * 32u + (lane & 31u)) * ROWB + kb);
+      for (uint32_t i = 0; i < NI; i++) {
+        dst[i] = *reinterpret_cast<const v8h*>(sa + (i * 32u + (lane & 31u)) * ROWB + kb);
       }
+    };
+    v8h a[DEPTH][NI];
 #pragma unroll
-      for (int i = 0; i < 2; i++) {
+    for (uint32_t d = 0; d < DEPTH; d++) { read_step(d, a[d]); }
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], bq[j][ks], ks == 0 ? nv[i] : acc[i][j], 0, 0, 0);
+    for (uint32_t ks = 0; ks < KS; ks++) {
+#pragma unroll
+      for (uint32_t i = 0; i < NI; i++) {
+#pragma unroll
+        for (uint32_t j = 0; j < NJ; j++) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[ks % DEPTH][i], bq[j][ks], ks == 0 ? nv[i] : acc[i][j], 0, 0, 0);
         }
       }
+      __builtin_amdgcn_sched_barrier(0);
+      if (ks + DEPTH < KS) { read_step(ks + DEPTH, a[ks % DEPTH]); }
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (PASS == 1) {
 #pragma unroll
-      for (int j = 0; j < 2; j++) {
+      for (uint32_t j = 0; j < NJ; j++) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (uint32_t i = 0; i < NI; i++) {
           float best = neg_inf;
 #pragma unroll
           for (int r = 0; r < 16; r++) { best = fmaxf(best, acc[i][j][r]); }  // NaN scores are ignored here and never pass the threshold
           // the lane 32 further on holds the tile's other 16 rows of this query
           best = fmaxf(best, __shfl_xor(best, 32, 64));
-          if (half == 0) { lmin[qloc[j] * kMinRow + (tile % kMinFlushTiles) * 2u + uint32_t(i)] = alpha * best; }
+          if (half == 0) { lmin[qloc[j] * kMinRow + (tile % FLUSH1) * NI + i] = alpha * best; }
         }
       }
     } else {
-      // bit (j * 32 + i * 16 + r) of `hits`: that list is a candidate of query j.  The sign of
-      // v - limit is shifted in element by element (two instructions an element), last element
-      // lowest: set bits are misses.  A NaN may land on either side: a NaN candidate sends the
-      // query to the plain path when it is rescored.
-      uint32_t miss[2];
+      // bit (i * 16 + r) of miss[j]: that list is no candidate of query j.  The sign of v - limit is
+      // shifted in element by element (two instructions an element), last element lowest.  A NaN
+      // may land on either side: a NaN candidate sends the query to the plain path when it is
+      // rescored.
+      uint32_t hits[NJ];
+      bool any = false;
 #pragma unroll
-      for (int j = 0; j < 2; j++) {
+      for (uint32_t j = 0; j < NJ; j++) {
         uint32_t m      = 0;
         const float lim = limit[j] * inv_alpha;  // alpha is -1 or -2: exact
 #pragma unroll
-        for (int i = 1; i >= 0; i--) {
+        for (int i = int(NI) - 1; i >= 0; i--) {
 #pragma unroll
           for (int r = 15; r >= 0; r--) { m = __builtin_amdgcn_alignbit(m, __float_as_uint(acc[i][j][r] - lim), 31); }
         }
-        miss[j] = m;
+        hits[j] = NI == 2 ? ~m : (~m) & 0xFFFFu;  // a single list tile fills the low 16 bits only
+        any     = any || hits[j] != 0u;
       }
-      unsigned long long hits = ~((static_cast<unsigned long long>(miss[1]) << 32) | miss[0]);
-      if (hits != 0) {
-        uint32_t slot[2];
-        slot[0] = atomicAdd(&lcount[qloc[0]], uint32_t(__popc(~miss[0])));
-        slot[1] = atomicAdd(&lcount[qloc[1]], uint32_t(__popc(~miss[1])));
-        while (hits != 0) {
-          const uint32_t bit = uint32_t(__builtin_ctzll(hits));
-          hits &= hits - 1u;
-          const uint32_t j   = bit >> 5;
-          const uint32_t row = ((bit >> 4) & 1u) * 32u + half * 4u + ((bit & 15u) >> 2) * 8u + (bit & 3u);
-          const uint32_t s   = j ? slot[1]++ : slot[0]++;
-          if (s < kLocalCap) { lcand[(j ? qloc[1] : qloc[0]) * kLocalCap + s] = tile * kTile + row; }
+      if (any) {
+#pragma unroll
+        for (uint32_t j = 0; j < NJ; j++) {
+          uint32_t h = hits[j];
+          if (h == 0u) { continue; }
+          uint32_t slot = atomicAdd(&lcount[qloc[j]], uint32_t(__popc(h)));
+          while (h != 0u) {
+            const uint32_t bit = uint32_t(__builtin_ctz(h));
+            h &= h - 1u;
+            const uint32_t row = (bit >> 4) * 32u + half * 4u + ((bit & 15u) >> 2) * 8u + (bit & 3u);
+            const uint32_t s   = slot++;
+            if (s < kLocalCap) { lcand[qloc[j] * kLocalCap + s] = tile * LT + row; }
+          }
         }
       }
     }
   };
-  // The wave writes out what it has staged for its 64 queries since the last flush (its own LDS
-  // writes, in order: no barrier).  PASS 1: the minima of tiles [first, tile], 16-byte parts (two
-  // tiles each: a block starts at an even tile) of one 128-byte line per query, 8 queries an
-  // instruction.  PASS 2: a lane per query.
+  // The wave writes out what it has staged for its queries since the last flush (its own LDS
+  // writes, in order: no barrier).  PASS 1: the minima of tiles [first, tile], 16-byte parts (four
+  // minima each: a block starts at a multiple of that many tiles) of one 128-byte line per query,
+  // 8 queries an instruction.  PASS 2: a lane per query.
   auto flush = [&](uint32_t tile) __attribute__((always_inline)) {
     if (PASS == 1) {
-      const uint32_t slot  = (tile % kMinFlushTiles) >> 1;
-      const uint32_t line  = tile - tile % kMinFlushTiles;       // first tile of the line
-      const uint32_t lo    = line < t0 ? (t0 - line) >> 1 : 0u;  // the block's first part of it
-      const uint32_t part  = lane & 7u;
+      constexpr uint32_t TP = 4u / NI;                             // tiles per 16-byte part
+      const uint32_t slot   = (tile % FLUSH1) / TP;                // the last part that has minima
+      const uint32_t line   = tile - tile % FLUSH1;                // first tile of the line
+      const uint32_t lo     = line < t0 ? (t0 - line) / TP : 0u;   // the block's first part of it
+      const uint32_t part   = lane & 7u;
       // (all eight reads first and the stores after them measured 20 % slower for the whole kernel)
 #pragma unroll
-      for (uint32_t it = 0; it < 8; it++) {
-        const uint32_t ql = wid * 64u + it * 8u + (lane >> 3);
+      for (uint32_t it = 0; it < 4u * NJ; it++) {
+        const uint32_t ql = wid * (32u * NJ) + it * 8u + (lane >> 3);
         if (part >= lo && part <= slot && q0 + ql < n_queries) {
-          *reinterpret_cast<float4*>(minima + uint64_t(q0 + ql) * n_groups + line * 2u + part * 4u) =
+          *reinterpret_cast<float4*>(minima + uint64_t(q0 + ql) * n_groups + line * NI + part * 4u) =
             *reinterpret_cast<const float4*>(lmin + ql * kMinRow + part * 4u);
         }
       }
     } else {
-      const uint32_t ql = wid * 64u + lane;
-      const uint32_t n  = lcount[ql];
-      if (n != 0) {
-        lcount[ql] = 0;
-        if (q0 + ql < n_queries) {
-          // more than the block can hold: push the query's count past the limit, it will be redone
-          // by the plain path
-          const uint32_t claim = n <= kLocalCap ? n : kCandCapF + 1u;
-          const uint32_t base  = atomicAdd(&cand_count[q0 + ql], claim);
-          if (n <= kLocalCap) {
-            for (uint32_t e = 0; e < n; e++) {
-              const uint32_t l = lcand[ql * kLocalCap + e];
-              if (base + e < kCandCapF && l < n_lists) { cand[uint64_t(q0 + ql) * kCandCapF + base + e] = l; }
+      if (lane < 32u * NJ) {
+        const uint32_t ql = wid * (32u * NJ) + lane;
+        const uint32_t n  = lcount[ql];
+        if (n != 0) {
+          lcount[ql] = 0;
+          if (q0 + ql < n_queries) {
+            // more than the block can hold: push the query's count past the limit, it will be redone
+            // by the plain path
+            const uint32_t claim = n <= kLocalCap ? n : kCandCapF + 1u;
+            const uint32_t base  = atomicAdd(&cand_count[q0 + ql], claim);
+            if (n <= kLocalCap) {
+              for (uint32_t e = 0; e < n; e++) {
+                const uint32_t l = lcand[ql * kLocalCap + e];
+                if (base + e < kCandCapF && l < n_lists) { cand[uint64_t(q0 + ql) * kCandCapF + base + e] = l; }
+              }
             }
           }
         }
@@ -377,7 +412,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void coarse_f16_kernel(
     const uint32_t buf = (tile - t0) & 1u;
     issue(tile + 1u, sx, cx);
     multiply(tile, buf);
-    if ((tile + 1u) % (PASS == 1 ? kMinFlushTiles : kCandFlushTiles) == 0 || tile + 1u == t1) { flush(tile); }
+    if ((tile + 1u) % (PASS == 1 ? FLUSH1 : FLUSH2) == 0 || tile + 1u == t1) { flush(tile); }
     arrived(sx, cx);
     commit(tile + 1u, buf ^ 1u, sx, cx);
     // the barrier orders LDS traffic only (the staged tile); the flushes' global stores stay in
@@ -586,7 +621,15 @@ __global__ __launch_bounds__(256) void coarse_exact_rows_kernel(
 
 }  // namespace
 
-uint32_t coarse_fast_k_pad(uint32_t dim) { return (dim + kSlab - 1) / kSlab * kSlab; }
+/** The padded dimensions the GEMM has instances for. */
+uint32_t coarse_fast_k_pad(uint32_t dim)
+{
+  for (uint32_t k : {64u, 128u, 256u, 384u, 512u, 768u}) {
+    if (dim <= k) { return k; }
+  }
+  return 1024u;
+}
+uint32_t coarse_fast_max_dim() { return 1024u; }
 uint32_t coarse_fast_groups(uint32_t n_lists) { return coarse_pad(n_lists) / kGroup; }
 uint32_t coarse_fast_cand_cap() { return kCandCapF; }
 
@@ -598,18 +641,6 @@ void launch_pack_centers_f16(const float* centers, uint32_t n_lists, uint32_t di
   pack_centers_kernel<<<l_pad, 64, 0, stream>>>(centers, n_lists, dim, dim_ext, coarse_fast_k_pad(dim), ch, cn, stats);
   CUVS_HIP_TRY(hipGetLastError());
 }
-
-namespace {
-template <typename K1, typename K2>
-void lds_limit_once(int which, K1 k1, K2 k2, size_t smem)
-{
-  static std::once_flag flags[2];
-  std::call_once(flags[which], [&] {
-    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k1), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
-    CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k2), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
-  });
-}
-}  // namespace
 
 void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
 {
@@ -648,33 +679,41 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
   }
   CUVS_HIP_TRY(hipGetLastError());
 
-  // list tiles per block: the queries of a block are loaded once for all of them
-  const uint32_t n_list_tiles = l_pad / kTile;
-  // A block costs about two tile-times of set-up besides its tiles, and the grid runs in rounds of
-  // two blocks per CU: take the run length whose rounds x (tiles + 2) is smallest (the longest of
-  // those: fewer blocks load the queries).
-  const uint64_t n_slots   = uint64_t(device_cu_count()) * 2u;
-  const uint32_t n_qblocks = (q_pad + kQTile - 1) / kQTile;
-  uint32_t tiles_per_block = 2;
-  uint64_t best_cost       = ~uint64_t(0);
-  // (even run lengths: the group minima of two tiles share a 16-byte store)
-  for (uint32_t t = 2; t <= n_list_tiles; t += 2) {
-    const uint64_t blocks = uint64_t((n_list_tiles + t - 1) / t) * n_qblocks;
-    const uint64_t rounds = (blocks + n_slots - 1) / n_slots;
-    const uint64_t cost   = rounds * (t + 2);
-    if (cost <= best_cost) {
-      best_cost       = cost;
-      tiles_per_block = t;
+  auto run_pass = [&](auto kpad) {
+    constexpr uint32_t K_PAD = decltype(kpad)::value;
+    using shape              = gemm_shape<K_PAD>;
+    constexpr uint32_t LT = 32u * shape::NI, QB = 128u * shape::NJ, TP = 4u / shape::NI;
+    auto k1 = coarse_f16_kernel<1, K_PAD>;
+    auto k2 = coarse_f16_kernel<2, K_PAD>;
+    // list tiles per block: the queries of a block are loaded once for all of them
+    const uint32_t n_list_tiles = l_pad / LT;
+    // A block costs about two tile-times of set-up besides its tiles, and the grid runs in rounds of
+    // its blocks per CU: take the run length whose rounds x (tiles + 2) is smallest (the longest of
+    // those: fewer blocks load the queries).
+    const uint64_t n_slots   = uint64_t(device_cu_count()) * shape::BLOCKS;
+    const uint32_t n_qblocks = (q_pad + QB - 1) / QB;
+    uint32_t tiles_per_block = TP;
+    uint64_t best_cost       = ~uint64_t(0);
+    // (run lengths of whole 16-byte parts of the staged minima: four group minima)
+    for (uint32_t t = TP; t <= n_list_tiles; t += TP) {
+      const uint64_t blocks = uint64_t((n_list_tiles + t - 1) / t) * n_qblocks;
+      const uint64_t rounds = (blocks + n_slots - 1) / n_slots;
+      const uint64_t cost   = rounds * (t + 2);
+      if (cost <= best_cost) {
+        best_cost       = cost;
+        tiles_per_block = t;
+      }
     }
-  }
-  dim3 grid((n_list_tiles + tiles_per_block - 1) / tiles_per_block, n_qblocks);
-  auto run_pass = [&](auto k1, auto k2) {
+    dim3 grid((n_list_tiles + tiles_per_block - 1) / tiles_per_block, n_qblocks);
     // list tiles (two buffers), their norm terms, and the larger of the two passes' per-query areas
-    const size_t smem = size_t(2) * kTile * (k_pad * 2 + 16) + 2 * kTile * 4 +
-                        std::max<size_t>(size_t(kQTile) * kMinRow * 4, size_t(kQTile) * (1 + kLocalCap) * 4);
-    // a generic lambda has one body per pair of argument types, and the kernels of both K_PAD
-    // values have the same type: the flag is keyed by K_PAD explicitly
-    lds_limit_once(k_pad == 64 ? 0 : 1, k1, k2, smem);
+    const size_t smem = size_t(2) * LT * (K_PAD * 2 + 16) + 2 * LT * 4 +
+                        std::max<size_t>(size_t(QB) * kMinRow * 4, size_t(QB) * (1 + kLocalCap) * 4);
+    static const int limit_set = [&] {
+      CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k1), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+      CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(k2), hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
+      return 1;
+    }();
+    (void)limit_set;
     k1<<<grid, kGemmThreads, smem, stream>>>(a.ch, a.qh, a.cn, a.n_lists, a.n_queries, q_pad, n_list_tiles, tiles_per_block, alpha,
                                     qterm, a.minima, n_groups, nullptr, nullptr, nullptr);
     CUVS_HIP_TRY(hipGetLastError());
@@ -690,11 +729,15 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
                                     qterm, nullptr, n_groups, a.thr, a.cand_count, a.cand);
     CUVS_HIP_TRY(hipGetLastError());
   };
-  if (k_pad == 64) {
-    run_pass(coarse_f16_kernel<1, 64>, coarse_f16_kernel<2, 64>);
-  } else {
-    CUVS_EXPECTS(k_pad == 128, "the two-precision probe selection takes dim <= 128");
-    run_pass(coarse_f16_kernel<1, 128>, coarse_f16_kernel<2, 128>);
+  switch (k_pad) {
+    case 64: run_pass(std::integral_constant<uint32_t, 64>{}); break;
+    case 128: run_pass(std::integral_constant<uint32_t, 128>{}); break;
+    case 256: run_pass(std::integral_constant<uint32_t, 256>{}); break;
+    case 384: run_pass(std::integral_constant<uint32_t, 384>{}); break;
+    case 512: run_pass(std::integral_constant<uint32_t, 512>{}); break;
+    case 768: run_pass(std::integral_constant<uint32_t, 768>{}); break;
+    case 1024: run_pass(std::integral_constant<uint32_t, 1024>{}); break;
+    default: CUVS_EXPECTS(false, "the two-precision probe selection takes dim <= 1024");
   }
   // up to 128 probes about 1.4 x 128 candidates pass the threshold: 256 threads; 512 beyond
   // about 1.15 x n_probes candidates pass the threshold: 128 threads up to 64 probes, 256 up to

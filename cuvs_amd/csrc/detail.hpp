@@ -283,6 +283,7 @@ struct coarse_fast_args {
   uint32_t* probes;        // [n_queries, n_probes]
 };
 uint32_t coarse_fast_k_pad(uint32_t dim);
+uint32_t coarse_fast_max_dim();
 uint32_t coarse_fast_groups(uint32_t n_lists);
 uint32_t coarse_fast_cand_cap();
 /** stats (3 words, device): bit patterns of the largest |element|, |stored norm| and centre length. */

@@ -180,7 +180,7 @@ bool coarse_fast_applies(const cuvs::resources& res, const search_params& params
 {
   return !res.tuning.plain_coarse && ix.coarse_fast_ok &&
          params.coarse_search_dtype == CUDA_R_32F && n_probes <= detail::coarse_fast_cand_cap() / 2 &&
-         ix.n_lists >= 1024 && ix.n_lists >= 64u * n_probes && ix.dim <= 128;
+         ix.n_lists >= 1024 && ix.n_lists >= 64u * n_probes && ix.dim <= detail::coarse_fast_max_dim();
 }
 
 /** Workspace bytes of the two-precision selection for a batch, and its allocation. */

@@ -968,7 +968,11 @@ def _coarse_model(n_lists, dim, pq_dim, seed, scale=1.0, cluster=True):
 
 
 @pytest.mark.parametrize("metric", ["sqeuclidean", "inner_product", "cosine"])
-@pytest.mark.parametrize("dtype,dim", [(np.float32, 96), (np.float16, 128), (np.int8, 64), (np.uint8, 40)])
+# (dimensions from 129 on run the GEMM shapes of one list tile or one query tile a wave: padded to
+# 256, 384, 512, 768 and 1024)
+@pytest.mark.parametrize("dtype,dim", [(np.float32, 96), (np.float16, 128), (np.int8, 64), (np.uint8, 40),
+                                       (np.float32, 256), (np.float16, 200), (np.float32, 384), (np.int8, 512),
+                                       (np.uint8, 768), (np.float32, 1024), (np.float16, 1000), (np.float32, 640)])
 def test_two_precision_probe_selection_equals_the_fp32_path(orc, metric, dtype, dim):
     n_lists, pq_dim = 4096, dim // 4
     model = _coarse_model(n_lists, dim, pq_dim, 3, scale=(0.5 if dtype in (np.int8, np.uint8) else 1.0))
