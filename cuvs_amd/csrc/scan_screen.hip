@@ -689,48 +689,43 @@ void launch_screen_types(const scan_args& a, const pair_desc* desc, uint32_t n_p
  * --------------------------------------------------------------------------------------------- */
 
 /** out[q][j] = (U, W): the largest sum_t q_t b_t[code] over the codes of subspace j, and the largest
- *  sum_t |q_t b_t[code]| (what bounds the rounding of an entry's evaluation). */
+ *  sum_t |q_t b_t[code]| (what bounds the rounding of an entry's evaluation).  One block per
+ *  query; a wave takes 64 / book subspaces at a time (book / 64 codes a lane when a codebook has
+ *  more than 64 entries), reads their codebook rows as whole lines and reduces with lane
+ *  exchanges: no LDS, no barrier. */
 __global__ __launch_bounds__(256) void ip_query_bounds_kernel(const float* __restrict__ rot_q,
                                                               const float* __restrict__ pq_centers, uint32_t pq_dim,
                                                               uint32_t pq_len, uint32_t book, uint32_t rot_dim,
                                                               float2* __restrict__ out)
 {
-  __shared__ float s_u[4], s_w[4];
-  const uint32_t q    = blockIdx.x;
-  const uint32_t tid  = threadIdx.x;
-  const uint32_t per  = 256u / book;        // subspaces per pass: 1 (256 codes) or 16 (16 codes)
-  const uint32_t code = tid % book;
-  const float* qrow   = rot_q + uint64_t(q) * rot_dim;
-  for (uint32_t j0 = 0; j0 < pq_dim; j0 += per) {
-    const uint32_t j = j0 + tid / book;
-    float dot = -FLT_MAX, mag = 0.0f;
+  const uint32_t q     = blockIdx.x;
+  const uint32_t lane  = threadIdx.x & 63u;
+  const uint32_t wave  = threadIdx.x >> 6;
+  const uint32_t spw   = book < 64u ? 64u / book : 1u;  // subspaces per wave and pass
+  const uint32_t cpl   = book > 64u ? book / 64u : 1u;  // codes per lane
+  const uint32_t width = book < 64u ? book : 64u;       // lanes of one subspace
+  const float* qrow    = rot_q + uint64_t(q) * rot_dim;
+  for (uint32_t j0 = wave * spw; j0 < pq_dim; j0 += 4u * spw) {
+    const uint32_t j = j0 + lane / width;
+    float best = -FLT_MAX, mag = 0.0f;
     if (j < pq_dim) {
-      dot = 0.0f;
-      for (uint32_t t = 0; t < pq_len; t++) {
-        const float prod = qrow[j * pq_len + t] * pq_centers[(uint64_t(j) * pq_len + t) * book + code];
-        dot += prod;
-        mag += fabsf(prod);
+      for (uint32_t c = 0; c < cpl; c++) {
+        const uint32_t code = (lane % width) + c * 64u;
+        float dot = 0.0f, m = 0.0f;
+        for (uint32_t t = 0; t < pq_len; t++) {
+          const float prod = qrow[j * pq_len + t] * pq_centers[(uint64_t(j) * pq_len + t) * book + code];
+          dot += prod;
+          m += fabsf(prod);
+        }
+        best = fmaxf(best, dot);
+        mag  = fmaxf(mag, m);
       }
     }
-    // maxima over the `book` lanes of a subspace
-    for (uint32_t m = (book < 64u ? book : 64u) >> 1; m >= 1u; m >>= 1) {
-      dot = fmaxf(dot, __shfl_xor(dot, int(m), 64));
-      mag = fmaxf(mag, __shfl_xor(mag, int(m), 64));
+    for (uint32_t x = width >> 1; x >= 1u; x >>= 1) {
+      best = fmaxf(best, __shfl_xor(best, int(x), 64));
+      mag  = fmaxf(mag, __shfl_xor(mag, int(x), 64));
     }
-    if (book == 256u) {
-      if ((tid & 63u) == 0u) {
-        s_u[tid >> 6] = dot;
-        s_w[tid >> 6] = mag;
-      }
-      __syncthreads();
-      if (tid == 0 && j < pq_dim) {
-        out[uint64_t(q) * pq_dim + j] = make_float2(fmaxf(fmaxf(s_u[0], s_u[1]), fmaxf(s_u[2], s_u[3])),
-                                                    fmaxf(fmaxf(s_w[0], s_w[1]), fmaxf(s_w[2], s_w[3])));
-      }
-      __syncthreads();
-    } else if (code == 0u && j < pq_dim) {
-      out[uint64_t(q) * pq_dim + j] = make_float2(dot, mag);
-    }
+    if (lane % width == 0u && j < pq_dim) { out[uint64_t(q) * pq_dim + j] = make_float2(best, mag); }
   }
 }
 

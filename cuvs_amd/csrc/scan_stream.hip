@@ -68,6 +68,13 @@ struct stream_kernel {
   // fp32 sums: entry * kEntryScale is added (one instruction: the binary16 entry is widened inside a
   // multiply-add); 8-bit tables hold half the decoded value
   static constexpr float kEntryScale = LUT == LUT_F16 ? 1.0f : 2.0f;
+  // Unsigned 8-bit tables (L2 metrics) keep the entry's 8-bit code itself, a byte an entry: the
+  // scan's reads then fall into 256 bytes a subspace instead of 512 (fewer bank conflicts), the
+  // table's writes are half as many bytes, and the builders skip the decoding; the scanners decode
+  // with one shift-and-add per lookup.
+  static constexpr bool BYTE            = LUT == LUT_FP8U;
+  static constexpr uint32_t SUB_BYTES   = BYTE ? 256u : 512u;  // bytes of a subspace's 256 entries
+  static constexpr uint32_t ENTRY_BYTES = BYTE ? 1u : 2u;
   static_assert(n_diff * 4u <= kStreamStageSlot, "staged terms of a pair must fit their slot");
   static_assert(ROT * G <= 512u, "one builder thread stages one (pair, dimension)");
   static_assert(uint32_t(M) * 512u <= 0x8000u, "a table must fit its 32 KB slot");
@@ -135,12 +142,16 @@ struct stream_kernel {
     bool live[G];
   };
 
-  /** ds_write_b32 at addr + IMM: the entries of two neighbouring codes of one subspace. */
+  /** One LDS write at addr + IMM: the entries of two neighbouring codes of one subspace. */
   template <int IMM>
   __device__ __forceinline__ static void entries_write(uint32_t addr, uint32_t two_entries)
   {
     static_assert(IMM >= 0 && IMM < 65536, "the write's offset field has 16 bits");
-    asm volatile("ds_write_b32 %0, %1 offset:%2" : : "v"(addr), "v"(two_entries), "n"(IMM) : "memory");
+    if constexpr (BYTE) {
+      asm volatile("ds_write_b16 %0, %1 offset:%2" : : "v"(addr), "v"(two_entries), "n"(IMM) : "memory");
+    } else {
+      asm volatile("ds_write_b32 %0, %1 offset:%2" : : "v"(addr), "v"(two_entries), "n"(IMM) : "memory");
+    }
   }
 
   /** The entries of two scores side by side, the first in the low half. */
@@ -155,6 +166,8 @@ struct stream_kernel {
       typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
       const f16x2 h = __builtin_convertvector(f32x2{s0, s1}, f16x2);
       return __builtin_bit_cast(uint32_t, h);
+    } else if constexpr (BYTE) {
+      return uint32_t(traits::encode(s0)) | (uint32_t(traits::encode(s1)) << 8);
     } else {
       return uint32_t(table_entry<LUT, OUT_HALF>(s0)) | (uint32_t(table_entry<LUT, OUT_HALF>(s1)) << 16);
     }
@@ -225,12 +238,12 @@ struct stream_kernel {
     }
   }
 
-  /** The thread's entries of one table go to LDS: entry (j, code) at base + j * 512 + code * 2. */
+  /** The thread's entries of one table go to LDS: entry (j, code) at base + j * SUB_BYTES + code * ENTRY_BYTES. */
   template <int jj = 0>
   __device__ __forceinline__ static void write_entries(uint32_t waddr, const uint32_t (&entries)[QM])
   {
     if constexpr (jj < QM) {
-      entries_write<jj * 512>(waddr, entries[jj]);
+      entries_write<jj * int(SUB_BYTES)>(waddr, entries[jj]);
       write_entries<jj + 1>(waddr, entries);
     }
   }
@@ -321,8 +334,8 @@ struct stream_kernel {
 #pragma unroll
       for (uint32_t g = 0; g < G; g++) {
         if (!f.live[g]) { continue; }  // uniform
-        // entry (j, code) of the table at base + j * 512 + code * 2; j = quarter * QM + jj
-        write_entries<0>(stream_table_base(g) + quarter * uint32_t(QM) * 512u + code * 2u, entries[g]);
+        // entry (j, code) of the table at base + j * SUB_BYTES + code * ENTRY_BYTES; j = quarter * QM + jj
+        write_entries<0>(stream_table_base(g) + quarter * uint32_t(QM) * SUB_BYTES + code * ENTRY_BYTES, entries[g]);
       }
     };
 
@@ -381,8 +394,9 @@ struct stream_kernel {
     const uint32_t sw      = rw;  // scanner wave 0..7
     const uint32_t cap     = stream_wave_cap(a.k);
     auto* my_cand          = reinterpret_cast<LDS_AS unsigned long long*>(uintptr_t(kStreamCandBase)) + sw * cap;
-    const float one        = opaque_float(kEntryScale);
-    uint32_t one_u         = 1u;
+    // (byte entries: the constant of their decoding, and no shift from code to offset)
+    const float one        = opaque_float(BYTE ? __uint_as_float(0x38080000u) : kEntryScale);
+    uint32_t one_u         = BYTE ? 0u : 1u;
     asm volatile("" : "+v"(one_u));
 
     // address registers of the lookups: the window of the group's table in the high halves
@@ -439,7 +453,7 @@ struct stream_kernel {
             }
           }
           const unsigned long long in_play = __builtin_amdgcn_ballot_w64(valid);
-          const uint32_t sum_bits = stream_tile_sum<NCH, OUT_HALF, !IP, IMMG>(now, addr, one_u, one, stop_bits, in_play);
+          const uint32_t sum_bits = stream_tile_sum<NCH, OUT_HALF, !IP, IMMG, false, NCH, BYTE>(now, addr, one_u, one, stop_bits, in_play);
           float score;
           if constexpr (OUT_HALF) {
             score = float(__builtin_bit_cast(_Float16, uint16_t(sum_bits)));

@@ -66,6 +66,8 @@ __device__ __forceinline__ uint16_t table_entry(float score)
 /* the read of subspace 8 o + i: 16-bit entries 512 bytes a subspace, or (RD32) fp32 entries 1 KB a subspace */
 #define ST_RD16(v, a, o, i) "ds_read_u16 %[" #v "], %[" #a "] offset:%[immg]+" #o "*4096+" #i "*512\n\t"
 #define ST_RD32(v, a, o, i) "ds_read_b32 %[" #v "], %[" #a "] offset:%[immg]+" #o "*8192+" #i "*1024\n\t"
+/* (RD8) one-byte entries, 256 bytes a subspace: the 8-bit code of an unsigned 8-bit table entry */
+#define ST_RD8(v, a, o, i) "ds_read_u8 %[" #v "], %[" #a "] offset:%[immg]+" #o "*2048+" #i "*256\n\t"
 /* group o: subspaces 8 o .. 8 o + 7, code dwords ca, cb, entries into V0 .. V7 */
 #define ST_ISSUE(RD, o, ca, cb, V)                                                                 \
   ST_SDWA(a0, ca, 0) ST_SDWA(a1, ca, 1) ST_SDWA(a2, ca, 2) ST_SDWA(a3, ca, 3)                      \
@@ -87,6 +89,11 @@ __device__ __forceinline__ uint16_t table_entry(float score)
 #define ST_ADD_F16_1(v) "v_add_f16_e32 %[acc], %[acc], %[" #v "]\n\t"
 /* fp32 entries */
 #define ST_ADD_W32_1(v) "v_add_f32_e32 %[acc], %[acc], %[" #v "]\n\t"
+/* one-byte entries e of an unsigned 8-bit table: decoded in the register, as the fp32 number with
+ * the bits (e << 20) + 0x38080000 (`one` holds that constant) or the binary16 number with the bits
+ * (e << 7) + 0x40, then added */
+#define ST_ADD_B32_1(v) "v_lshl_add_u32 %[" #v "], %[" #v "], 20, %[one]\n\tv_add_f32_e32 %[acc], %[acc], %[" #v "]\n\t"
+#define ST_ADD_B16_1(v) "v_lshl_add_u32 %[" #v "], %[" #v "], 7, 64\n\tv_add_f16_e32 %[acc], %[acc], %[" #v "]\n\t"
 #define ST_ADD8(ADD1, V) ADD1(V##0) ADD1(V##1) ADD1(V##2) ADD1(V##3) ADD1(V##4) ADD1(V##5) ADD1(V##6) ADD1(V##7)
 #define ST_ADD4_LO(ADD1, V) ADD1(V##0) ADD1(V##1) ADD1(V##2) ADD1(V##3)
 #define ST_ADD4_HI(ADD1, V) ADD1(V##4) ADD1(V##5) ADD1(V##6) ADD1(V##7)
@@ -99,6 +106,12 @@ __device__ __forceinline__ uint16_t table_entry(float score)
 #define ST_ADD_F16_HI(V) ST_ADD4_HI(ST_ADD_F16_1, V)
 #define ST_ADD_W32_LO(V) ST_ADD4_LO(ST_ADD_W32_1, V)
 #define ST_ADD_W32_HI(V) ST_ADD4_HI(ST_ADD_W32_1, V)
+#define ST_ADD_B32(V) ST_ADD8(ST_ADD_B32_1, V)
+#define ST_ADD_B32_LO(V) ST_ADD4_LO(ST_ADD_B32_1, V)
+#define ST_ADD_B32_HI(V) ST_ADD4_HI(ST_ADD_B32_1, V)
+#define ST_ADD_B16(V) ST_ADD8(ST_ADD_B16_1, V)
+#define ST_ADD_B16_LO(V) ST_ADD4_LO(ST_ADD_B16_1, V)
+#define ST_ADD_B16_HI(V) ST_ADD4_HI(ST_ADD_B16_1, V)
 /* rows in play whose sum is not past the bound; none: leave */
 #define ST_CHECK_F32                                 \
   "v_cmp_ge_u32_e32 vcc, %[stop], %[acc]\n\t"        \
@@ -155,20 +168,31 @@ __device__ __forceinline__ uint16_t table_entry(float score)
  *  IMMG: offset of the table inside its 64 KB window, which the high halves of the address
  *  registers `ad` name (the routine changes their low halves only); `one` is the factor of the
  *  entries (fp32 sums), one_u the integer 1.  WIDE: the table holds fp32 entries, 1 KB a subspace,
- *  added as they are; one_u is then 2 (the shift that turns a code into its entry's offset). */
-template <int NCH, bool HALF, bool CHECK, int IMMG, bool WIDE = false, int NCUR = NCH>
+ *  added as they are; one_u is then 2 (the shift that turns a code into its entry's offset).
+ *  BYTE: the table holds the one-byte codes of an unsigned 8-bit table, 256 bytes a subspace,
+ *  decoded after the read; one_u is then 0 and `one` the constant of the fp32 decoding. */
+template <int NCH, bool HALF, bool CHECK, int IMMG, bool WIDE = false, int NCUR = NCH, bool BYTE = false>
 __device__ __forceinline__ uint32_t stream_tile_sum(const u32x4 (&cur)[NCUR], uint32_t (&ad)[8], uint32_t one_u, float one,
                                                     uint32_t stop, unsigned long long valid, uint32_t start = 0u)
 {
   static_assert(NCH >= 2 && NCH <= 4 && NCH <= NCUR, "two to four chunks of sixteen subspaces");
   static_assert(IMMG >= 0 && IMMG + (NCH * 16 - 1) * (WIDE ? 1024 : 512) < 65536, "the read's offset field has 16 bits");
   static_assert(!(WIDE && HALF), "fp32 entries are summed in fp32");
+  static_assert(!(WIDE && BYTE), "one entry size");
   uint32_t acc = start, chk, va[8], vb[8];
   unsigned long long tmp;
 #define ST_EMIT(BODY, RD, ADD, CHK, ...) \
   asm volatile(BODY(RD, ADD, CHK) : ST_OUTPUTS : ST_COMMON_INPUTS, __VA_ARGS__ : "vcc", "scc", "memory")
 #define ST_EMIT_KIND(BODY, ...)                                              \
-  if constexpr (WIDE && CHECK) {                                             \
+  if constexpr (BYTE && !HALF && CHECK) {                                    \
+    ST_EMIT(BODY, ST_RD8, ST_ADD_B32, ST_CHECK_F32, __VA_ARGS__);            \
+  } else if constexpr (BYTE && !HALF && !CHECK) {                            \
+    ST_EMIT(BODY, ST_RD8, ST_ADD_B32, ST_NO_CHECK, __VA_ARGS__);             \
+  } else if constexpr (BYTE && HALF && CHECK) {                              \
+    ST_EMIT(BODY, ST_RD8, ST_ADD_B16, ST_CHECK_F16, __VA_ARGS__);            \
+  } else if constexpr (BYTE && HALF && !CHECK) {                             \
+    ST_EMIT(BODY, ST_RD8, ST_ADD_B16, ST_NO_CHECK, __VA_ARGS__);             \
+  } else if constexpr (WIDE && CHECK) {                                      \
     ST_EMIT(BODY, ST_RD32, ST_ADD_W32, ST_CHECK_F32, __VA_ARGS__);           \
   } else if constexpr (WIDE && !CHECK) {                                     \
     ST_EMIT(BODY, ST_RD32, ST_ADD_W32, ST_NO_CHECK, __VA_ARGS__);            \

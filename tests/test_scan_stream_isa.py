@@ -3,7 +3,7 @@ inline assembly, so that the adds of one group overlap the reads of the next.  F
 point of view a read's destination register holds its value as soon as the read is issued; nothing
 stops it from copying or reusing that register before the data has arrived.  Both files therefore
 keep a whole tile (or step) of lookups in one assembly block.  This test compiles them for gfx950
-and checks the generated code for what that is meant to guarantee: between an inline `ds_read_u16`
+and checks the generated code for what that is meant to guarantee: between an inline `ds_read_u16` / `ds_read_u8`
 and the inline `s_waitcnt` that covers it, no compiler-generated instruction, label or branch
 touches the destination register, and no other inline instruction reads it.
 """
@@ -46,7 +46,7 @@ def check_lookup_windows(asm_text):
         if not line:
             continue
         if in_asm:
-            m = re.match(r"ds_read_u16\s+v(\d+),", line)
+            m = re.match(r"ds_read_u(?:16|8)\s+v(\d+),", line)
             if m:
                 pending.append(int(m.group(1)))
                 n_reads += 1
