@@ -689,43 +689,51 @@ void launch_screen_types(const scan_args& a, const pair_desc* desc, uint32_t n_p
  * --------------------------------------------------------------------------------------------- */
 
 /** out[q][j] = (U, W): the largest sum_t q_t b_t[code] over the codes of subspace j, and the largest
- *  sum_t |q_t b_t[code]| (what bounds the rounding of an entry's evaluation).  One block per
- *  query; a wave takes 64 / book subspaces at a time (book / 64 codes a lane when a codebook has
- *  more than 64 entries), reads their codebook rows as whole lines and reduces with lane
- *  exchanges: no LDS, no barrier. */
+ *  sum_t |q_t b_t[code]| (what bounds the rounding of an entry's evaluation).  A lane per query,
+ *  a block per 256 queries and kBoundSubs subspaces, whose codebooks it stages in LDS: every lane
+ *  reads the same four codes at a time (a broadcast), the maxima need no exchange between lanes. */
+constexpr uint32_t kBoundSubs = 4;
+template <int PQ_LEN>
 __global__ __launch_bounds__(256) void ip_query_bounds_kernel(const float* __restrict__ rot_q,
-                                                              const float* __restrict__ pq_centers, uint32_t pq_dim,
-                                                              uint32_t pq_len, uint32_t book, uint32_t rot_dim,
+                                                              const float* __restrict__ pq_centers, uint32_t n_queries,
+                                                              uint32_t pq_dim, uint32_t book, uint32_t rot_dim,
                                                               float2* __restrict__ out)
 {
-  const uint32_t q     = blockIdx.x;
-  const uint32_t lane  = threadIdx.x & 63u;
-  const uint32_t wave  = threadIdx.x >> 6;
-  const uint32_t spw   = book < 64u ? 64u / book : 1u;  // subspaces per wave and pass
-  const uint32_t cpl   = book > 64u ? book / 64u : 1u;  // codes per lane
-  const uint32_t width = book < 64u ? book : 64u;       // lanes of one subspace
-  const float* qrow    = rot_q + uint64_t(q) * rot_dim;
-  for (uint32_t j0 = wave * spw; j0 < pq_dim; j0 += 4u * spw) {
-    const uint32_t j = j0 + lane / width;
+  __shared__ __align__(16) float s_book[kBoundSubs * PQ_LEN * 256];  // [subspace][component][code]
+  const uint32_t q  = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t qr = q < n_queries ? q : n_queries - 1u;
+  const float* qrow = rot_q + uint64_t(qr) * rot_dim;
+  const uint32_t j0 = blockIdx.y * kBoundSubs;
+  const uint32_t nj = pq_dim - j0 < kBoundSubs ? pq_dim - j0 : kBoundSubs;
+  // the block's codebooks are one contiguous run of nj * PQ_LEN * book floats
+  for (uint32_t x = threadIdx.x; x < nj * PQ_LEN * book; x += 256u) {
+    s_book[x] = pq_centers[uint64_t(j0) * PQ_LEN * book + x];
+  }
+  __syncthreads();
+  for (uint32_t u = 0; u < nj; u++) {
+    const uint32_t j = j0 + u;
+    float qv[PQ_LEN];
+#pragma unroll
+    for (int t = 0; t < PQ_LEN; t++) { qv[t] = qrow[j * PQ_LEN + t]; }
+    const float* bj = s_book + u * PQ_LEN * book;
     float best = -FLT_MAX, mag = 0.0f;
-    if (j < pq_dim) {
-      for (uint32_t c = 0; c < cpl; c++) {
-        const uint32_t code = (lane % width) + c * 64u;
-        float dot = 0.0f, m = 0.0f;
-        for (uint32_t t = 0; t < pq_len; t++) {
-          const float prod = qrow[j * pq_len + t] * pq_centers[(uint64_t(j) * pq_len + t) * book + code];
-          dot += prod;
-          m += fabsf(prod);
+#pragma unroll 4
+    for (uint32_t code = 0; code < book; code += 4) {  // a codebook has 16 entries or more
+      float dot[4] = {0.0f, 0.0f, 0.0f, 0.0f}, m[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int t = 0; t < PQ_LEN; t++) {
+        const float4 bv4 = *reinterpret_cast<const float4*>(bj + uint32_t(t) * book + code);
+        const float bv[4] = {bv4.x, bv4.y, bv4.z, bv4.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          dot[e] = fmaf(qv[t], bv[e], dot[e]);
+          m[e]   = fmaf(fabsf(qv[t]), fabsf(bv[e]), m[e]);
         }
-        best = fmaxf(best, dot);
-        mag  = fmaxf(mag, m);
       }
+      best = fmaxf(fmaxf(best, fmaxf(dot[0], dot[1])), fmaxf(dot[2], dot[3]));
+      mag  = fmaxf(fmaxf(mag, fmaxf(m[0], m[1])), fmaxf(m[2], m[3]));
     }
-    for (uint32_t x = width >> 1; x >= 1u; x >>= 1) {
-      best = fmaxf(best, __shfl_xor(best, int(x), 64));
-      mag  = fmaxf(mag, __shfl_xor(mag, int(x), 64));
-    }
-    if (lane % width == 0u && j < pq_dim) { out[uint64_t(q) * pq_dim + j] = make_float2(best, mag); }
+    if (q < n_queries) { out[uint64_t(q) * pq_dim + j] = make_float2(best, mag); }
   }
 }
 
@@ -1061,8 +1069,15 @@ void launch_scan_screen(const scan_args& a, const pair_desc* desc, uint32_t n_pa
   if (scan_screen_ip(a)) {
     CUVS_EXPECTS(scratch != nullptr, "the screen of an inner-product search needs its scratch buffer");
     auto* qbounds = static_cast<float2*>(scratch);
-    ip_query_bounds_kernel<<<a.n_queries, 256, 0, stream>>>(a.rot_q, a.pq_centers, a.pq_dim, a.pq_len, 1u << a.pq_bits,
-                                                          a.rot_dim, qbounds);
+    {
+      const dim3 grid((a.n_queries + 255u) / 256u, (a.pq_dim + kBoundSubs - 1u) / kBoundSubs);
+      const uint32_t book = 1u << a.pq_bits;
+      switch (a.pq_len) {
+        case 1: ip_query_bounds_kernel<1><<<grid, 256, 0, stream>>>(a.rot_q, a.pq_centers, a.n_queries, a.pq_dim, book, a.rot_dim, qbounds); break;
+        case 2: ip_query_bounds_kernel<2><<<grid, 256, 0, stream>>>(a.rot_q, a.pq_centers, a.n_queries, a.pq_dim, book, a.rot_dim, qbounds); break;
+        default: ip_query_bounds_kernel<4><<<grid, 256, 0, stream>>>(a.rot_q, a.pq_centers, a.n_queries, a.pq_dim, book, a.rot_dim, qbounds); break;
+      }
+    }
     CUVS_HIP_TRY(hipGetLastError());
     auto by_bits = [&](auto len) {
       constexpr int PQ_LEN = decltype(len)::value;
