@@ -771,6 +771,8 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_ip_kernel(
   auto* book      = reinterpret_cast<LDS_AS vec_t*>(uintptr_t(kScreenLdsBase));
   const float one = opaque_one_s();
   constexpr uint32_t off_pending = kScreenLdsBase + SUB * BOOK * uint32_t(sizeof(vec_t));
+  // binary16 sums: the least entries of a pair, a binary16 number a subspace, for the wave's chain
+  constexpr uint32_t off_lows = (off_pending + (kDirectThreads / 64u) * kSurvivorBatchBytes + 15u) & ~15u;
 
   const uint32_t tid  = threadIdx.x;
   const uint32_t lane = tid & 63u;
@@ -786,6 +788,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_ip_kernel(
   }
   lds_barrier_s();
   auto* pending      = reinterpret_cast<LDS_AS uint32_t*>(uintptr_t(off_pending + wid * kSurvivorBatchBytes));
+  auto* my_lows      = reinterpret_cast<LDS_AS uint16_t*>(uintptr_t(off_lows + wid * (kIpRounds * 64u * 2u)));
   uint32_t n_pending = 0;
   const auto* plane  = reinterpret_cast<const GLOBAL_AS u32x2*>(reinterpret_cast<uintptr_t>(a.lead_plane));
   const bool cosine  = a.metric == int(DistanceType::CosineExpanded);
@@ -899,19 +902,35 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_ip_kernel(
         _Float16 x         = _Float16(mid + (float(lane - grp * 21u) - 13.0f) * step);
         const _Float16 start = x;
         const uint32_t from  = grp == 0 ? uint32_t(FIRST) : (grp == 1 ? uint32_t(MID) : SUB);  // the lane's first subspace
+        // The terms go through the wave's LDS area (subspace j at halfword j) and come back eight
+        // at a time, the same eight to every lane: an LDS read per eight additions where a
+        // cross-lane read per addition doubled the chain's vector instructions.  (The wave's own
+        // LDS accesses are performed in order.)
 #pragma unroll
         for (uint32_t r = 0; r < kIpRounds; r++) {
           if (r * 64u >= M) { continue; }  // uniform
-          const uint32_t lowbits = uint32_t(__builtin_bit_cast(uint16_t, _Float16(lows[r])));  // exact: a binary16 number
+          my_lows[r * 64u + lane] = __builtin_bit_cast(uint16_t, _Float16(lows[r]));  // exact: a binary16 number
+        }
+        {
+          // the leading subspaces: a lane's chain starts at its checkpoint
+          const u32x4 w8a = *reinterpret_cast<const LDS_AS u32x4*>(my_lows);
+          const u32x4 w8b = *reinterpret_cast<const LDS_AS u32x4*>(my_lows + 8);
+          const uint32_t wd[8] = {w8a.x, w8a.y, w8a.z, w8a.w, w8b.x, w8b.y, w8b.z, w8b.w};
 #pragma unroll
-          for (int l = 0; l < 64; l++) {
-            if (r == 0 && l < FIRST) { continue; }
-            const _Float16 add = __builtin_bit_cast(_Float16, uint16_t(__builtin_amdgcn_readlane(int(lowbits), l)));
-            if (r == 0 && l < int(SUB)) {
-              x = _Float16(x + (uint32_t(l) >= from ? add : _Float16(0)));
-            } else {
-              x = _Float16(x + add);
-            }
+          for (int l = FIRST; l < int(SUB); l++) {
+            const _Float16 add = __builtin_bit_cast(_Float16, uint16_t(wd[l >> 1] >> ((l & 1) * 16)));
+            x = _Float16(x + (uint32_t(l) >= from ? add : _Float16(0)));
+          }
+        }
+        // (the terms past the last subspace are zero; with four waves a SIMD the wait for a read
+        // is covered: requesting sixteen terms ahead of the additions measured the same)
+        for (uint32_t j = SUB; j < M; j += 8u) {
+          const u32x4 w8 = *reinterpret_cast<const LDS_AS u32x4*>(my_lows + j);
+          const uint32_t wd[4] = {w8.x, w8.y, w8.z, w8.w};
+#pragma unroll
+          for (int l = 0; l < 8; l++) {
+            const _Float16 add = __builtin_bit_cast(_Float16, uint16_t(wd[l >> 1] >> ((l & 1) * 16)));
+            x = _Float16(x + add);
           }
         }
         if (cosine) { x = _Float16(x + _Float16(1)); }
@@ -926,6 +945,23 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_ip_kernel(
           }
         }
       }
+    }
+
+    /* ---- nibble codes: the entries of the first four subspaces, which every tile sums, one a lane
+     * (subspace lane / 16, code lane % 16), in the form the sums take them ---- */
+    float first_entry = 0.0f;
+    if constexpr (BITS == 4) {
+      const int kk   = int(lane >> 4);
+      const vec_t b  = book[lane];  // kk * 16 + code
+      float score    = 0.0f;
+#pragma unroll
+      for (int t = 0; t < PQ_LEN; t++) {
+        const float tc = __shfl(tc0[t], kk, 64);
+        const float qv = __shfl(q0[t], kk, 64);
+        score -= tc;
+        score = fmaf(-qv, b[t], score);
+      }
+      first_entry = widen(score);
     }
 
     /* ---- the rows' leading codes ---- */
@@ -967,7 +1003,18 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_ip_kernel(
         const bool mine = OUT_HALF ? float(acc) < stop[c] : float(acc) <= stop[c];
         return (__builtin_amdgcn_ballot_w64(mine) & rows) != 0ull;
       };
-      add_codes(0, FIRST);
+      if constexpr (BITS == 4) {
+        // a lane exchange per code in place of a codebook gather and the entry's arithmetic
+        static_assert(BITS != 4 || FIRST == 4, "64 entries: four subspaces of sixteen codes");
+#pragma unroll
+        for (int kk = 0; kk < FIRST; kk++) {
+          const uint32_t c  = (w[0] >> (kk * 4)) & 0xfu;
+          const float entry = __int_as_float(__builtin_amdgcn_ds_bpermute(int((uint32_t(kk) * 16u + c) << 2), __float_as_int(first_entry)));
+          acc               = acc_t(acc + acc_t(entry));
+        }
+      } else {
+        add_codes(0, FIRST);
+      }
       in_play = open(0);
       if (in_play) {
         add_codes(FIRST, MID);
@@ -990,7 +1037,8 @@ void launch_screen_ip_instance(const scan_args& a, const pair_desc* desc, uint32
 {
   auto kernel       = scan_screen_ip_kernel<PQ_LEN, LUT, OUT_HALF, BITS>;
   const size_t smem = kScreenLdsBase + size_t(kDirectSubs) * (BITS == 8 ? 256 : 32) * sizeof(typename book_vec<PQ_LEN>::type) +
-                      size_t(kDirectThreads / 64u) * kSurvivorBatchBytes;
+                      size_t(kDirectThreads / 64u) * kSurvivorBatchBytes + 16 +
+                      size_t(kDirectThreads / 64u) * kIpRounds * 64u * 2u;
   static const int per_cu = prepare_persistent_kernel(kernel, kDirectThreads, smem, smem);
   constexpr uint32_t wpb = kDirectThreads / 64u;
   uint32_t grid          = uint32_t(device_cu_count()) * uint32_t(per_cu);

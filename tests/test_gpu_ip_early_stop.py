@@ -65,7 +65,7 @@ TABLES = [(R_32F, R_32F), (R_16F, R_32F), (R_8U, R_32F), (R_16F, R_16F), (R_8U, 
 
 
 @pytest.mark.parametrize("metric", ["inner_product", "cosine"])
-@pytest.mark.parametrize("dim,pq_dim", [(128, 64), (96, 48), (128, 32), (256, 128), (64, 64)])
+@pytest.mark.parametrize("dim,pq_dim", [(128, 64), (96, 48), (128, 32), (256, 128), (64, 64), (72, 36)])
 def test_inner_product_early_stop_byte_codes(orc, metric, dim, pq_dim):
     x, q, index, ix = _case(orc, dim, pq_dim, 8, metric)
     for lut, internal in TABLES:
