@@ -449,7 +449,8 @@ def sweep(args, res, index, data, queries, log):
     add(res, index, queries, truth10, 10, 64, "f32", "f32",
         head + ", k=10, n_probes=64, fp32 table (the reference's default lut_dtype)")
 
-    def other(dataset, rows, dim, lists, pq_dim, P, lut, workload):
+    def other(dataset, rows, dim, lists, pq_dim, P, variants):
+        """variants: (lut, workload) pairs measured on one index"""
         nq = queries.shape[0]
         allrows = make_rows(dataset, rows + nq, dim, "cuda")
         x, q = allrows[:rows], allrows[rows:].contiguous()
@@ -458,18 +459,19 @@ def sweep(args, res, index, data, queries, log):
         ix = ivf_pq.build(params, x, resources=res)
         res.sync()
         truth = testing.exact_knn(x, q, 10, metric="sqeuclidean").cpu().numpy()
-        add(res, ix, q, truth, 10, P, lut, "f32", workload)
+        for lut, workload in variants:
+            add(res, ix, q, truth, 10, P, lut, "f32", workload)
         del ix, x, q, allrows
         torch.cuda.empty_cache()
 
-    other("unit_mixture_f32", 1_000_000, 96, 1024, 48, 32, "f16",
-          "configs[1] (1M x 96 f32 unit vectors, 1024 lists, pq_dim 48), k=10, n_probes=32, fp16 table")
-    other("sift_u8", 2_000_000, 256, 2048, 128, 32, "f16",
-          "2M x 256 u8 (sift_u8), 2048 lists, pq_dim 128 (the reference's default pq_dim for 256 dimensions), "
-          "k=10, n_probes=32, fp16 table")
-    other("sift_u8", 1_000_000, 768, 1024, 384, 32, "f16",
-          "1M x 768 u8 (sift_u8), 1024 lists, pq_dim 384 (the reference's default pq_dim for 768 dimensions), "
-          "k=10, n_probes=32, fp16 table")
+    c1 = "configs[1] (1M x 96 f32 unit vectors, 1024 lists, pq_dim 48), k=10, n_probes=32, "
+    other("unit_mixture_f32", 1_000_000, 96, 1024, 48, 32, [("f16", c1 + "fp16 table"), ("fp8", c1 + "fp8 table")])
+    other("sift_u8", 2_000_000, 256, 2048, 128, 32,
+          [("f16", "2M x 256 u8 (sift_u8), 2048 lists, pq_dim 128 (the reference's default pq_dim for 256 dimensions), "
+            "k=10, n_probes=32, fp16 table")])
+    other("sift_u8", 1_000_000, 768, 1024, 384, 32,
+          [("f16", "1M x 768 u8 (sift_u8), 1024 lists, pq_dim 384 (the reference's default pq_dim for 768 dimensions), "
+            "k=10, n_probes=32, fp16 table")])
     return entries
 
 
