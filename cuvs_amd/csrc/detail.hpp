@@ -204,6 +204,10 @@ struct index_impl {
   /** Refill `lead_plane` and the byte-wide copy of narrower codes from the codes arena (after the
    *  arena's contents changed). */
   void rebuild_lead_plane(hipStream_t stream);
+  /** The same for the rows of one list that were written in place (all of it if a list has moved
+   *  since the copies were made). */
+  void refresh_derived_rows(uint32_t label, hipStream_t stream);
+  std::vector<uint64_t> derived_offsets;  // h_row_offsets at the time the copies were made
   /** Set when list memory was written through a bare pointer (codepacker::pack on a buffer of this
    *  index): what the index derives from its lists is then refreshed by the next search, under
    *  `derived_mu`. */

@@ -111,9 +111,15 @@ uint32_t extend_list_prepare(cuvs::resources const& res, index_impl& ix, const i
   return offset;
 }
 
-void finish_edit(cuvs::resources const& res, index_impl& ix)
+constexpr uint32_t kAllLists = 0xFFFFFFFFu;
+/** The index's derived copies of the list codes follow an edit: of one list, or of everything. */
+void finish_edit(cuvs::resources const& res, index_impl& ix, uint32_t label = kAllLists)
 {
-  ix.rebuild_lead_plane(res.stream());
+  if (label == kAllLists) {
+    ix.rebuild_lead_plane(res.stream());
+  } else {
+    ix.refresh_derived_rows(label, res.stream());
+  }
   CUVS_HIP_TRY(hipStreamSynchronize(res.stream()));
 }
 
@@ -203,7 +209,7 @@ void pack_list_data(cuvs::resources const& res, index<int64_t>* idx,
   expect_range(ix, label, offset, new_codes.extent(0));
   detail::launch_pack_codes(list_codes(ix, label), new_codes.data_handle(), false,
                             uint32_t(new_codes.extent(0)), offset, ix.pq_dim, ix.pq_bits, res.stream());
-  finish_edit(res, ix);
+  finish_edit(res, ix, label);
 }
 
 void pack_contiguous_list_data(cuvs::resources const& res, index<int64_t>* idx, const uint8_t* new_codes,
@@ -215,7 +221,7 @@ void pack_contiguous_list_data(cuvs::resources const& res, index<int64_t>* idx, 
   expect_range(ix, label, offset, n_rows);
   detail::launch_pack_codes(list_codes(ix, label), new_codes, true, n_rows, offset, ix.pq_dim, ix.pq_bits,
                             res.stream());
-  finish_edit(res, ix);
+  finish_edit(res, ix, label);
 }
 
 template <typename T>
@@ -263,7 +269,7 @@ void extend_list_with_codes(cuvs::resources const& res, index<int64_t>* idx,
   const uint32_t offset = extend_list_prepare(res, ix, new_indices.data_handle(), new_codes.extent(0), label);
   detail::launch_pack_codes(list_codes(ix, label), new_codes.data_handle(), false,
                             uint32_t(new_codes.extent(0)), offset, ix.pq_dim, ix.pq_bits, res.stream());
-  finish_edit(res, ix);
+  finish_edit(res, ix, label);
 }
 
 void extend_list_with_contiguous_codes(cuvs::resources const& res, index<int64_t>* idx,
@@ -278,7 +284,7 @@ void extend_list_with_contiguous_codes(cuvs::resources const& res, index<int64_t
   const uint32_t offset = extend_list_prepare(res, ix, new_indices.data_handle(), new_codes.extent(0), label);
   detail::launch_pack_codes(list_codes(ix, label), new_codes.data_handle(), true,
                             uint32_t(new_codes.extent(0)), offset, ix.pq_dim, ix.pq_bits, res.stream());
-  finish_edit(res, ix);
+  finish_edit(res, ix, label);
 }
 
 template <typename T>
@@ -296,7 +302,7 @@ void extend_list(cuvs::resources const& res, index<int64_t>* idx, device_matrix_
   const uint32_t offset = extend_list_prepare(res, ix, new_indices.data_handle(), n, label);
   detail::launch_pack_codes(list_codes(ix, label), codes.as<uint8_t>(), true, uint32_t(n), offset,
                             ix.pq_dim, ix.pq_bits, res.stream());
-  finish_edit(res, ix);
+  finish_edit(res, ix, label);
 }
 
 #define CUVS_INSTANTIATE_EXTEND_LIST(T)                                                                  \

@@ -208,6 +208,15 @@ void index_impl::rebuild_lead_plane(hipStream_t stream)
 {
   derived_stale.store(false);  // whatever was written so far is seen by the kernels below
   const uint64_t n_slots = h_row_offsets.empty() ? 0 : h_row_offsets[n_lists];
+  // Buffers of the right size are written in place; others are released before their successors
+  // are allocated (the copies never exist twice).  Work that still reads them ends first.
+  CUVS_HIP_TRY(hipStreamSynchronize(stream));
+  auto sized = [](device_buffer& b, size_t bytes) {
+    if (b.bytes != bytes) {
+      b = device_buffer();
+      b.allocate(bytes);
+    }
+  };
   // narrower codes, a byte each
   const bool widen = pq_bits >= 5 && pq_bits < 8 && n_slots != 0 && !conservative_memory_allocation;
   if (widen) {
@@ -215,29 +224,27 @@ void index_impl::rebuild_lead_plane(hipStream_t stream)
     const uint64_t gb8       = uint64_t(n_chunks8) * kIndexGroupSize * kIndexGroupVecLen;
     const uint64_t n_groups  = n_slots / kIndexGroupSize;
     // two groups of slack: the scan kernels read whole 64-row tiles past a list's last group
-    device_buffer wide_codes((n_groups + 2) * gb8);
-    CUVS_HIP_TRY(hipMemsetAsync(wide_codes.ptr, 0, wide_codes.bytes, stream));
-    launch_widen_codes(codes_arena.as<uint8_t>(), wide_codes.as<uint8_t>(), n_slots, pq_dim, pq_bits, n_chunks,
+    sized(codes8_arena, (n_groups + 2) * gb8);
+    CUVS_HIP_TRY(hipMemsetAsync(codes8_arena.ptr, 0, codes8_arena.bytes, stream));
+    launch_widen_codes(codes_arena.as<uint8_t>(), codes8_arena.as<uint8_t>(), n_slots, pq_dim, pq_bits, n_chunks,
                        n_chunks8, stream);
     std::vector<uint8_t*> dptr(n_lists);
     for (uint32_t l = 0; l < n_lists; l++) {
-      dptr[l] = wide_codes.as<uint8_t>() + (h_row_offsets[l] / kIndexGroupSize) * gb8;
+      dptr[l] = codes8_arena.as<uint8_t>() + (h_row_offsets[l] / kIndexGroupSize) * gb8;
     }
-    device_buffer ptrs(sizeof(void*) * n_lists);
-    CUVS_HIP_TRY(hipMemcpyAsync(ptrs.ptr, dptr.data(), ptrs.bytes, hipMemcpyHostToDevice, stream));
+    sized(data_ptrs8, sizeof(void*) * n_lists);
+    CUVS_HIP_TRY(hipMemcpyAsync(data_ptrs8.ptr, dptr.data(), data_ptrs8.bytes, hipMemcpyHostToDevice, stream));
     const uint64_t book_rows = pq_centers.bytes / (sizeof(float) * book_size);
-    device_buffer books(book_rows * 256 * sizeof(float));
-    launch_pad_codebooks(pq_centers.as<float>(), books.as<float>(), book_rows, book_size, stream);
-    CUVS_HIP_TRY(hipStreamSynchronize(stream));  // `dptr` goes out of scope; the old buffers are released
-    codes8_arena = std::move(wide_codes);
-    data_ptrs8   = std::move(ptrs);
-    pq_centers8  = std::move(books);
+    sized(pq_centers8, book_rows * 256 * sizeof(float));
+    launch_pad_codebooks(pq_centers.as<float>(), pq_centers8.as<float>(), book_rows, book_size, stream);
+    CUVS_HIP_TRY(hipStreamSynchronize(stream));  // `dptr` goes out of scope
   } else {
     codes8_arena = device_buffer();
     data_ptrs8   = device_buffer();
     pq_centers8  = device_buffer();
     n_chunks8    = 0;
   }
+  derived_offsets = h_row_offsets;
   // byte codes (as stored or widened), and nibble codes unless memory is to be spared: the plane
   // is what lets an L2 search of either width screen pairs without scanning them
   const bool plane_codes = pq_bits == 8 || widen || (pq_bits == 4 && !conservative_memory_allocation);
@@ -245,12 +252,36 @@ void index_impl::rebuild_lead_plane(hipStream_t stream)
     lead_plane = device_buffer();
     return;
   }
-  device_buffer plane((n_slots + kLeadPlaneSlack) * sizeof(uint64_t));
-  CUVS_HIP_TRY(hipMemsetAsync(plane.ptr, 0, plane.bytes, stream));
-  launch_build_lead_plane(widen ? codes8_arena.as<uint8_t>() : codes_arena.as<uint8_t>(), plane.as<uint64_t>(), n_slots,
+  sized(lead_plane, (n_slots + kLeadPlaneSlack) * sizeof(uint64_t));
+  CUVS_HIP_TRY(hipMemsetAsync(lead_plane.ptr, 0, lead_plane.bytes, stream));
+  launch_build_lead_plane(widen ? codes8_arena.as<uint8_t>() : codes_arena.as<uint8_t>(), lead_plane.as<uint64_t>(), n_slots,
                           widen ? n_chunks8 : n_chunks, stream);
-  CUVS_HIP_TRY(hipStreamSynchronize(stream));  // the old plane is released on assignment
-  lead_plane = std::move(plane);
+}
+
+void index_impl::refresh_derived_rows(uint32_t label, hipStream_t stream)
+{
+  // The copies follow the lists where they are now only if no list has moved since they were made
+  // (an edit that outgrows a list's padding moves the arenas); and a write through a bare pointer
+  // may have touched any list.
+  if (derived_stale.load() || derived_offsets != h_row_offsets) {
+    rebuild_lead_plane(stream);
+    return;
+  }
+  const uint64_t begin = h_row_offsets[label], end = h_row_offsets[label + 1];  // whole groups of 32 rows
+  if (begin == end) { return; }
+  const bool widen       = codes8_arena.bytes != 0;
+  const uint64_t gb      = uint64_t(n_chunks) * kIndexGroupSize * kIndexGroupVecLen;
+  const uint64_t gb8     = uint64_t(n_chunks8) * kIndexGroupSize * kIndexGroupVecLen;
+  const uint64_t group   = begin / kIndexGroupSize;
+  const uint8_t* packed  = codes_arena.as<uint8_t>() + group * gb;
+  if (widen) {
+    launch_widen_codes(packed, codes8_arena.as<uint8_t>() + group * gb8, end - begin, pq_dim, pq_bits, n_chunks, n_chunks8,
+                       stream);
+  }
+  if (lead_plane.bytes != 0) {
+    launch_build_lead_plane(widen ? codes8_arena.as<uint8_t>() + group * gb8 : packed, lead_plane.as<uint64_t>() + begin,
+                            end - begin, widen ? n_chunks8 : n_chunks, stream);
+  }
 }
 
 }  // namespace detail
