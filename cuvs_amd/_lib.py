@@ -63,7 +63,7 @@ class IndexStruct(C.Structure):
 
 class SearchTuningStruct(C.Structure):
     _fields_ = [("early_stop", C.c_int32), ("generic_scan", C.c_int32), ("plain_coarse", C.c_int32),
-                ("reserved_", C.c_int32 * 5)]
+                ("serial_batches", C.c_int32), ("reserved_", C.c_int32 * 4)]
 
 
 class SearchProfileStruct(C.Structure):

@@ -646,6 +646,7 @@ cuvsError_t cuvsAmdIvfPqSetSearchTuning(cuvsResources_t res, const cuvsAmdIvfPqS
     t.early_stop   = tuning->early_stop;
     t.generic_scan = tuning->generic_scan != 0;
     t.plain_coarse = tuning->plain_coarse != 0;
+    t.serial_batches = tuning->serial_batches != 0;
   });
 }
 

@@ -11,8 +11,57 @@ resources::resources()
   CUVS_HIP_TRY(hipGetDevice(&device_));
 }
 
+resources* resources::side(int i)
+{
+  if (i < 0 || i >= kMaxSideHandles) { return nullptr; }
+  side_handle& sh = sides_[i];
+  if (sh.handle == nullptr) {
+    hipStream_t st = nullptr;
+    hipEvent_t ev  = nullptr;
+    if (hipStreamCreateWithFlags(&st, hipStreamNonBlocking) != hipSuccess ||
+        hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      if (st != nullptr) { (void)hipStreamDestroy(st); }
+      return nullptr;
+    }
+    sh.stream = st;
+    sh.done   = ev;
+    sh.handle = new resources();
+    sh.handle->set_stream(st);
+  }
+  sh.handle->tuning           = tuning;
+  sh.handle->workspace_limit_ = workspace_limit_;
+  return sh.handle;
+}
+
+void resources::fork_sides(int n)
+{
+  if (fork_event_ == nullptr) { CUVS_HIP_TRY(hipEventCreateWithFlags(&fork_event_, hipEventDisableTiming)); }
+  CUVS_HIP_TRY(hipEventRecord(fork_event_, stream_));
+  for (int i = 0; i < n && i < kMaxSideHandles; i++) {
+    if (sides_[i].handle != nullptr) { CUVS_HIP_TRY(hipStreamWaitEvent(sides_[i].stream, fork_event_, 0)); }
+  }
+}
+
+void resources::join_sides(int n)
+{
+  for (int i = 0; i < n && i < kMaxSideHandles; i++) {
+    if (sides_[i].handle == nullptr) { continue; }
+    CUVS_HIP_TRY(hipEventRecord(sides_[i].done, sides_[i].stream));
+    CUVS_HIP_TRY(hipStreamWaitEvent(stream_, sides_[i].done, 0));
+  }
+}
+
 resources::~resources()
 {
+  for (side_handle& sh : sides_) {
+    if (sh.handle == nullptr) { continue; }
+    (void)hipStreamSynchronize(sh.stream);
+    delete sh.handle;  // its workspace
+    (void)hipEventDestroy(sh.done);
+    (void)hipStreamDestroy(sh.stream);
+  }
+  if (fork_event_ != nullptr) { (void)hipEventDestroy(fork_event_); }
   // a pool of this handle's own returns everything it holds when it goes, right after this body
   if (!(workspace_pooled_ && pool_)) { release_workspace(); }
   for (size_t i = 0; i < retired_.size(); i++) {

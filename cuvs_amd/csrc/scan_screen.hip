@@ -308,6 +308,25 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
  * its own sequence of pairs, with the next pair's record, first codes, bound and query-minus-centre
  * terms in flight while it scans the current one.
  */
+/** The pairs of a wave of the persistent screening kernels: pair first, first + stride, ... below
+ *  end.  Workgroups go to the XCDs in turn, and pairs come in list order: the waves of one XCD take
+ *  one contiguous eighth of the pairs (neighbouring waves neighbouring pairs), so that a list's
+ *  leading codes pass through one XCD's L2 instead of all eight. */
+struct wave_pairs {
+  uint32_t first, stride, end;
+};
+__device__ __forceinline__ wave_pairs screen_wave_pairs(uint32_t n_pairs, uint32_t wid, uint32_t waves_per_block)
+{
+  const uint32_t grid = gridDim.x;
+  if ((grid & 7u) == 0u && n_pairs >= grid * waves_per_block) {
+    const uint32_t chunk = (n_pairs + 7u) >> 3;
+    const uint32_t lo    = (blockIdx.x & 7u) * chunk;
+    const uint32_t hi    = lo + chunk < n_pairs ? lo + chunk : n_pairs;
+    return {lo + (blockIdx.x >> 3) * waves_per_block + wid, (grid >> 3) * waves_per_block, hi};
+  }
+  return {blockIdx.x * waves_per_block + wid, grid * waves_per_block, n_pairs};
+}
+
 constexpr uint32_t kDirectThreads = 512;
 constexpr uint32_t kDirectSubs    = 8;
 constexpr uint32_t kIpRounds      = 12;  // the inner-product screen keeps a value per 64 subspaces: pq_dim <= 768
@@ -362,8 +381,10 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   const uint32_t lane = tid & 63u;
   const uint32_t wid  = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr uint32_t WPB = kDirectThreads / 64u;
-  const uint32_t total   = gridDim.x * WPB;
-  if (blockIdx.x * WPB >= n_pairs) { return; }
+  const wave_pairs mine  = screen_wave_pairs(n_pairs, wid, WPB);
+  const uint32_t total   = mine.stride;
+  const uint32_t p_end   = mine.end;
+  if (mine.first - wid >= p_end) { return; }  // the whole block, before its barrier
 
   for (uint32_t e = tid; e < SUB * BOOK; e += kDirectThreads) {
     vec_t v = {};
@@ -373,8 +394,8 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   }
   lds_barrier_s();
 
-  uint32_t p = blockIdx.x * WPB + wid;
-  if (p >= n_pairs) { return; }
+  uint32_t p = mine.first;
+  if (p >= p_end) { return; }
   auto* pending = reinterpret_cast<LDS_AS uint32_t*>(uintptr_t(off_pending + wid * kSurvivorBatchBytes));
   auto* mini    = reinterpret_cast<LDS_AS lut_t*>(uintptr_t(off_mini + wid * uint32_t(FIRST) * 256u * uint32_t(sizeof(lut_t))));
   uint32_t n_pending = 0;
@@ -383,7 +404,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   // analysis): a scalar load would be waited for by the tile loop's first LDS read, since both
   // count on the same counter, while vector loads return in order behind loads issued earlier.
   auto record = [&](uint32_t idx) -> pair_desc {
-    uint32_t at = idx < n_pairs ? idx : n_pairs - 1u;
+    uint32_t at = idx < p_end ? idx : p_end - 1u;
     asm volatile("" : "+v"(at));
     return desc[at];
   };
@@ -422,7 +443,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   float dv0     = fetch_diff(d0);
 
   for (;;) {
-    const bool has1    = p + total < n_pairs;
+    const bool has1    = p + total < p_end;
     const pair_desc d2 = record(p + 2u * total);
     u32x2 lead1        = lead0;
     u32x2 next1        = next0;
@@ -778,8 +799,8 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_ip_kernel(
   const uint32_t lane = tid & 63u;
   const uint32_t wid  = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr uint32_t WPB = kDirectThreads / 64u;
-  const uint32_t total   = gridDim.x * WPB;
-  if (blockIdx.x * WPB >= n_pairs) { return; }
+  const wave_pairs mine  = screen_wave_pairs(n_pairs, wid, WPB);
+  if (mine.first - wid >= mine.end) { return; }  // the whole block, before its barrier
   for (uint32_t e = tid; e < SUB * BOOK; e += kDirectThreads) {
     vec_t v = {};
 #pragma unroll
@@ -800,7 +821,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_ip_kernel(
     return OUT_HALF ? float(traits::to_half(e)) : traits::to_float(e);
   };
 
-  for (uint32_t p = blockIdx.x * WPB + wid; p < n_pairs; p += total) {
+  for (uint32_t p = mine.first; p < mine.end; p += mine.stride) {
     pair_desc d = desc[p];
     {
       const uint64_t ptr = reinterpret_cast<uint64_t>(d.data);

@@ -38,13 +38,15 @@ class Resources:
     def get_c_obj(self):
         return self._h
 
-    def set_search_tuning(self, early_stop="auto", generic_scan=False, plain_coarse=False):
+    def set_search_tuning(self, early_stop="auto", generic_scan=False, plain_coarse=False, serial_batches=False):
         """cuvsAmdIvfPqSetSearchTuning: fix choices the search otherwise makes by itself (results do
-        not depend on them).  early_stop: "auto", "off" (every probed list streamed in full) or "on"."""
+        not depend on them).  early_stop: "auto", "off" (every probed list streamed in full) or "on";
+        serial_batches: internal batches one after the other instead of side by side."""
         t = SearchTuningStruct()
         t.early_stop = {"auto": 0, "off": 1, "on": 2}[early_stop]
         t.generic_scan = int(bool(generic_scan))
         t.plain_coarse = int(bool(plain_coarse))
+        t.serial_batches = int(bool(serial_batches))
         check(lib().cuvsAmdIvfPqSetSearchTuning(self._h, C.byref(t)))
 
     def enable_profiling(self, on=True):

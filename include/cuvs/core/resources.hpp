@@ -124,6 +124,9 @@ struct search_tuning {
   bool generic_scan = false;
   /** Coarse search by the fp32 contraction and selection instead of the two-precision selection. */
   bool plain_coarse = false;
+  /** The internal batches of a search run one after the other on the handle's stream instead of
+   *  side by side on streams of the handle's own. */
+  bool serial_batches = false;
 };
 
 /**
@@ -181,6 +184,18 @@ class resources {
   void borrow_workspace(void* ptr, size_t bytes);
   bool workspace_borrowed() const { return workspace_borrowed_; }
 
+  /**
+   * Handle number `i` of this handle's own: another stream (default priority) and another cached
+   * workspace, for internal batches of one call that run beside each other.  Created on first
+   * use, destroyed with this handle; null if the stream cannot be made.  fork(): work queued on
+   * the side streams from now on starts after what this handle's stream holds now; join(): this
+   * handle's stream continues after what the side streams hold now.
+   */
+  static constexpr int kMaxSideHandles = 3;
+  resources* side(int i);
+  void fork_sides(int n);
+  void join_sides(int n);
+
   search_tuning tuning;
   bool profiling = false;
   struct profile_state;
@@ -205,6 +220,13 @@ class resources {
   bool workspace_borrowed_ = false;     // workspace_ belongs to the caller of borrow_workspace
   void release_workspace();
   memory::tracker* tracker_ = nullptr;  // track_memory
+  struct side_handle {
+    resources* handle  = nullptr;
+    hipStream_t stream = nullptr;
+    hipEvent_t done    = nullptr;
+  };
+  side_handle sides_[kMaxSideHandles];
+  hipEvent_t fork_event_ = nullptr;
 };
 
 }  // namespace cuvs

@@ -275,12 +275,16 @@ typedef struct {
  *  the others screened on their leading codes, survivors in full) pays; 1 = never, every probed
  *  list is streamed in full by the scan kernel; 2 = whenever the search's parameters allow it.
  *  generic_scan != 0: every search goes through the generic scan kernel.  plain_coarse != 0: coarse
- *  search by the fp32 contraction and selection instead of the two-precision selection. */
+ *  search by the fp32 contraction and selection instead of the two-precision selection.
+ *  serial_batches != 0: the internal batches of a search (max_internal_batch_size) run one after the
+ *  other on the handle's stream; by default up to four of them run side by side on streams of the
+ *  handle's own, each with its own workspace, and the handle's stream continues after all of them. */
 typedef struct {
   int32_t early_stop;
   int32_t generic_scan;
   int32_t plain_coarse;
-  int32_t reserved_[5]; /* zero */
+  int32_t serial_batches;
+  int32_t reserved_[4]; /* zero */
 } cuvsAmdIvfPqSearchTuning;
 CUVS_EXPORT cuvsError_t cuvsAmdIvfPqSetSearchTuning(cuvsResources_t res,
                                                     const cuvsAmdIvfPqSearchTuning* tuning);

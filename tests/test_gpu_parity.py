@@ -13,6 +13,7 @@ import gpu_helpers as G
 import helpers as H
 from cuvs_amd import ivf_pq
 from cuvs_amd._lib import CuvsError
+from cuvs_amd.resources import Resources
 
 pytestmark = pytest.mark.gpu
 
@@ -196,6 +197,46 @@ def test_batching_does_not_change_results(orc):
     b = _search_both(orc, index, ix, queries, 10, 4, max_internal_batch_size=37)
     assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
     H.compare_results(a[0], a[1], a[2], a[3], 1e-5, exact=True)
+
+
+@pytest.mark.parametrize("n_queries,batch", [(301, 37), (1000, 400), (129, 128), (640, 64)])
+def test_batches_side_by_side_equal_batches_in_turn(orc, n_queries, batch):
+    """The internal batches of a call run beside each other on streams of the handle's own (up to
+    four runs of whole batches); switched off on the handle they run one after the other.  Same
+    results either way, and the oracle's; work queued on the handle's stream afterwards sees them
+    (no host synchronisation between the search and the copy that follows it on the same stream);
+    a bitset filter goes to every run."""
+    data, model, queries, index, ix, _ = _case(orc, 4000, 32, 12, 16, 8, n_queries=n_queries)
+    dq = G.to_dev(queries)
+    sp = ivf_pq.SearchParams(n_probes=5, lut_dtype=R_16F, max_internal_batch_size=batch)
+    res = Resources()
+    res.use_torch_current_stream()
+    want_nb, want_d = orc.search(ix, queries, 10, 5, lut_dtype=ORC_DT[R_16F])
+    out = {}
+    for serial in (False, True, False):
+        res.set_search_tuning(serial_batches=serial)
+        d, nb = ivf_pq.search(sp, index, dq, 10, resources=res)
+        nb_copy, d_copy = nb.clone(), d.clone()  # on the same stream, right behind the search
+        torch.cuda.synchronize()
+        H.compare_results(nb_copy.cpu().numpy(), d_copy.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
+        out[serial] = (nb_copy, d_copy)
+    assert torch.equal(out[False][0], out[True][0]) and torch.equal(out[False][1], out[True][1])
+    n = data.shape[0]
+    keep = np.ones(n, dtype=bool)
+    keep[::2] = False
+    bits = np.packbits(keep, bitorder="little")
+    bits = np.concatenate([bits, np.zeros((-bits.size) % 4, dtype=np.uint8)]).view(np.uint32)
+    res.set_search_tuning(serial_batches=False)
+    d, nb = ivf_pq.search(sp, index, dq, 10, resources=res, filter_bitset=G.to_dev(bits.view(np.int32)), filter_nbits=n)
+    torch.cuda.synchronize()
+    want_nb, want_d = orc.search(ix, queries, 10, 5, lut_dtype=ORC_DT[R_16F], filter_bitset=bits, filter_nbits=n)
+    H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
+    # a wrong argument is refused by the first run, before anything is queued on a side stream
+    with pytest.raises(CuvsError):
+        ivf_pq.search(sp, index, G.to_dev(np.zeros((n_queries, 31), dtype=np.float32)), 10, resources=res)
+    d, nb = ivf_pq.search(sp, index, dq, 10, resources=res)
+    torch.cuda.synchronize()
+    assert torch.equal(nb, out[True][0])
 
 
 def test_half_precision_coarse_search(orc):
