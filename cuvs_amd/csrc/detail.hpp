@@ -475,6 +475,7 @@ struct merge_args {
   const unsigned long long* in_keys;  // fused
   const uint8_t* alive;               // fused: per pair slot, 0 = no keys were written (or null: all)
   uint8_t* redo;                      // with alive: scratch, a byte per query (null: one kernel does all)
+  const uint32_t* bound;              // fused: per query, an upper bound of the final k-th key's score word (or null)
   const float* in_scores;             // non-fused
   const uint32_t* n_samples;
   const uint32_t* probes;

@@ -760,6 +760,7 @@ void search_one(cuvs::resources const& res_c,
     ma.in_keys       = keys;
     ma.alive         = alive;
     ma.redo          = merge_redo;
+    ma.bound         = pl.fused ? kth : nullptr;
     ma.in_scores     = all_scores;
     ma.n_samples     = n_samples;
     ma.probes        = probes;
