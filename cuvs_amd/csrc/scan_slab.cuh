@@ -75,7 +75,10 @@ struct slab_kernel {
   static constexpr bool WIDE     = LUT == LUT_F32;
   static constexpr int SCH       = WIDE ? 2 : 4;         // chunks of a whole slab
   static constexpr uint32_t SUBS = 16u * SCH;            // its subspaces
-  static constexpr uint32_t SUB_BYTES = WIDE ? 1024u : 512u;  // bytes of a subspace's 256 entries
+  // unsigned 8-bit tables keep the entry's code itself, a byte an entry, decoded by the scanners
+  // (fewer bank conflicts in 256 bytes a subspace than in 512; see scan_stream.hip)
+  static constexpr bool BYTE     = LUT == LUT_FP8U;
+  static constexpr uint32_t SUB_BYTES = WIDE ? 1024u : (BYTE ? 256u : 512u);  // bytes of a subspace's 256 entries
   static_assert((NCH_LAST == 2 || NCH_LAST == 4) && NCH_LAST <= SCH, "pq_dim is a multiple of 32");
   static_assert(!(WIDE && OUT_HALF), "fp32 entries are summed in fp32");
   static_assert(kSlabSubs * FPS * 4u <= kSlabStageSlot, "staged terms of a slab must fit their slot");
@@ -187,7 +190,11 @@ struct slab_kernel {
   __device__ __forceinline__ static void entries_write(uint32_t addr, uint32_t two_entries)
   {
     static_assert(IMM >= 0 && IMM < 65536, "the write's offset field has 16 bits");
-    asm volatile("ds_write_b32 %0, %1 offset:%2" : : "v"(addr), "v"(two_entries), "n"(IMM) : "memory");
+    if constexpr (BYTE) {
+      asm volatile("ds_write_b16 %0, %1 offset:%2" : : "v"(addr), "v"(two_entries), "n"(IMM) : "memory");
+    } else {
+      asm volatile("ds_write_b32 %0, %1 offset:%2" : : "v"(addr), "v"(two_entries), "n"(IMM) : "memory");
+    }
   }
 
   /** The entries of two scores side by side, the first in the low half. */
@@ -202,6 +209,8 @@ struct slab_kernel {
       typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
       const f16x2 h = __builtin_convertvector(f32x2{s0, s1}, f16x2);
       return __builtin_bit_cast(uint32_t, h);
+    } else if constexpr (BYTE) {
+      return uint32_t(traits::encode(s0)) | (uint32_t(traits::encode(s1)) << 8);
     } else {
       return uint32_t(table_entry<LUT, OUT_HALF>(s0)) | (uint32_t(table_entry<LUT, OUT_HALF>(s1)) << 16);
     }
@@ -374,7 +383,7 @@ struct slab_kernel {
       if constexpr (WIDE) {
         entries_write_wide<jj * 1024>(waddr, entries[2 * jj], entries[2 * jj + 1]);
       } else {
-        entries_write<jj * 512>(waddr, entries[jj]);
+        entries_write<jj * int(SUB_BYTES)>(waddr, entries[jj]);
       }
       write_entries<NCH, jj + 1>(waddr, entries);
     }
@@ -386,7 +395,7 @@ struct slab_kernel {
 #pragma unroll
     for (uint32_t g = 0; g < G; g++) {
       if (!f.live(g)) { continue; }  // uniform
-      write_entries<NCH>(slab_table_base(g) + quarter * uint32_t(4 * NCH) * SUB_BYTES + code * (WIDE ? 4u : 2u), entries[g]);
+      write_entries<NCH>(slab_table_base(g) + quarter * uint32_t(4 * NCH) * SUB_BYTES + code * (WIDE ? 4u : (BYTE ? 1u : 2u)), entries[g]);
     }
   }
 
@@ -524,8 +533,9 @@ struct slab_kernel {
     auto* my_cand      = reinterpret_cast<LDS_AS unsigned long long*>(uintptr_t(kSlabCandBase)) + rw * cap;
     // sums of the pair's rows between slabs: row r of the row block at word r
     auto* part         = reinterpret_cast<LDS_AS uint32_t*>(uintptr_t(kSlabPartBase + uint32_t(GI) * kSlabRows * 4u)) + lane;
-    const float one    = opaque_float(kEntryScale);
-    uint32_t one_u     = WIDE ? 2u : 1u;  // a code shifted by this is its entry's offset in a subspace's table
+    // (byte entries: the constant of their decoding in place of the entries' factor)
+    const float one    = opaque_float(BYTE ? __uint_as_float(0x38080000u) : kEntryScale);
+    uint32_t one_u     = WIDE ? 2u : (BYTE ? 0u : 1u);  // a code shifted by this is its entry's offset in a subspace's table
     asm volatile("" : "+v"(one_u));
 
     // address registers of the lookups: the window of the group's table in the high halves
@@ -608,7 +618,7 @@ struct slab_kernel {
           if (s != 0u) { start = *my_part; }
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // see ST_FIRST
           const uint32_t sum_bits =
-            stream_tile_sum<NCH, OUT_HALF, !IP, IMMG, WIDE>(now, addr, one_u, one, stop_bits, in_play, start);
+            stream_tile_sum<NCH, OUT_HALF, !IP, IMMG, WIDE, BYTE>(now, addr, one_u, one, stop_bits, in_play, start);
           if constexpr (!LAST) {
             bool keep = true;
             if constexpr (!IP) {

@@ -453,7 +453,7 @@ struct stream_kernel {
             }
           }
           const unsigned long long in_play = __builtin_amdgcn_ballot_w64(valid);
-          const uint32_t sum_bits = stream_tile_sum<NCH, OUT_HALF, !IP, IMMG, false, NCH, BYTE>(now, addr, one_u, one, stop_bits, in_play);
+          const uint32_t sum_bits = stream_tile_sum<NCH, OUT_HALF, !IP, IMMG, false, BYTE>(now, addr, one_u, one, stop_bits, in_play);
           float score;
           if constexpr (OUT_HALF) {
             score = float(__builtin_bit_cast(_Float16, uint16_t(sum_bits)));

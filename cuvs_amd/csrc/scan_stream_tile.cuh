@@ -171,7 +171,7 @@ __device__ __forceinline__ uint16_t table_entry(float score)
  *  added as they are; one_u is then 2 (the shift that turns a code into its entry's offset).
  *  BYTE: the table holds the one-byte codes of an unsigned 8-bit table, 256 bytes a subspace,
  *  decoded after the read; one_u is then 0 and `one` the constant of the fp32 decoding. */
-template <int NCH, bool HALF, bool CHECK, int IMMG, bool WIDE = false, int NCUR = NCH, bool BYTE = false>
+template <int NCH, bool HALF, bool CHECK, int IMMG, bool WIDE = false, bool BYTE = false, int NCUR = NCH>
 __device__ __forceinline__ uint32_t stream_tile_sum(const u32x4 (&cur)[NCUR], uint32_t (&ad)[8], uint32_t one_u, float one,
                                                     uint32_t stop, unsigned long long valid, uint32_t start = 0u)
 {
