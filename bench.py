@@ -293,6 +293,12 @@ def main():
     kernel_ms = mean(full_prof, "scan_ms") / full_launches
     kernel_bytes = float(full_prof[-1]["scan_bytes"]) / full_launches
     achieved = kernel_bytes / (kernel_ms * 1e-3) / 1e9
+    default_workload = (args.config == 2 and n == 10_000_000 and dim == 128 and n_lists == 16384 and pq_dim == 64 and
+                        pq_bits == 8 and nq == 10_000 and k == 10 and P == 64 and args.lut == "f16" and
+                        args.internal == "f32" and args.metric == "sqeuclidean" and args.kind == "subspace" and
+                        full_name == "scan_stream_kernel")
+    traffic = 1.67e9 if default_workload else None  # 1.46 GB fetched + 0.21 GB written per launch
+    traffic_source = ("profiles/scan_stream_kernel_configs2_configs1_counters.md" if default_workload else None)
     log(f"code stream in full: {full_name} {kernel_ms:.3f} ms per launch, {kernel_bytes / 1e9:.2f} GB algorithmic "
         f"-> {achieved:.0f} GB/s ({achieved / HBM_PEAK_GBS:.1%} of HBM peak); {full_ms_per_step:.2f} ms per batch = "
         f"{nq / full_ms_per_step * 1e3:,.0f} QPS" + (f"; ids identical to the default path: {same_ids}" if same_ids is not None else ""))
@@ -333,10 +339,13 @@ def main():
                    "refine_ratio": args.refine_ratio,
                    "recall_at_k": gpu_recall},
         # the code-scan kernel streaming every probed list in full: algorithmic bytes as the metric
-        # defines them over the HIP-event time of that one launch; HBM traffic from hardware
-        # counters is not measured by this script (profiles/ holds the counter runs)
+        # defines them over the HIP-event time of that one launch; HBM traffic comes from hardware
+        # counters, which this script does not read: for the default workload it is the figure of
+        # the counter runs kept under profiles/ (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, the factors a
+        # 1 GiB copy reads in the same runs), for any other workload null
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "traffic_source": traffic_source,
                      "kernel": full_name, "kernel_ms": kernel_ms,
                      "algorithmic_bytes_per_launch": kernel_bytes,
                      "path": ("early stop switched off on the handle: every probed list streamed in full"
