@@ -14,14 +14,16 @@ from cuvs_amd.resources import Resources
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("n_queries,n_probes", [(1, 20), (100, 20), (2000, 8)])
-def test_captured_search_replays_like_eager(n_queries, n_probes):
+# (the last case: three internal batches, which an eager call runs side by side on streams of the
+# handle's own and a captured call one after the other on the capturing stream)
+@pytest.mark.parametrize("n_queries,n_probes,batch", [(1, 20, 4096), (100, 20, 4096), (2000, 8, 4096), (2000, 8, 700)])
+def test_captured_search_replays_like_eager(n_queries, n_probes, batch):
     n, dim = 100000, 64
     allrows = testing.gaussian_mixture(n + 4 * n_queries, dim, 100, 0.2, seed=5, device="cuda")
     data, pool = allrows[:n], allrows[n:]
     index = ivf_pq.build(ivf_pq.IndexParams(n_lists=256, pq_dim=32, kmeans_trainset_fraction=0.3), data)
     res = Resources()
-    sp = ivf_pq.SearchParams(n_probes=n_probes, lut_dtype=np.float16)
+    sp = ivf_pq.SearchParams(n_probes=n_probes, lut_dtype=np.float16, max_internal_batch_size=batch)
     queries = pool[:n_queries].clone()
     nb = torch.empty((n_queries, 10), dtype=torch.int64, device="cuda")
     d = torch.empty((n_queries, 10), dtype=torch.float32, device="cuda")
