@@ -372,6 +372,7 @@ struct scan_args {
   void* global_lut;               // generic kernel: table scratch when it does not fit LDS, or null
   const uint64_t* lead_plane;     // first eight code bytes of every row slot (8- and 4-bit codes), or null
   int subset;                     // generic kernel: scan the pairs of desc[0 .. n_pairs) (or *n_pairs_dev) only
+  uint32_t mean_list_rows;        // rows of the index over its lists (which screening kernel pays)
   int rare_exits;                 // few tiles of this launch are expected to end early (the leading and the
                                   // surviving pairs of an early stop): the wave-per-pair kernel then has a
                                   // tile's next step on its way instead of the next tile's first one

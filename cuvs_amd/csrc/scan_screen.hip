@@ -354,7 +354,7 @@ struct book_vec<8> {
   typedef float type __attribute__((ext_vector_type(8)));
 };
 
-template <int PQ_LEN, int LUT, bool OUT_HALF, int FIRST, int BITS>
+template <int PQ_LEN, int LUT, bool OUT_HALF, int FIRST, int BITS, bool PER_CLUSTER = false>
 __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   scan_args a, const pair_desc* __restrict__ desc, uint32_t n_pairs, uint32_t group_bytes,
   pair_desc* __restrict__ survivors, uint32_t* __restrict__ n_survivors, uint8_t* __restrict__ alive)
@@ -371,6 +371,13 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   constexpr uint32_t NDIFF = SUB * PQ_LEN;
   static_assert(NDIFF <= 64, "one lane per leading rotated dimension");
   static_assert(FIRST <= 4 && FIRST <= MID, "the first subspaces' terms sit in scalar registers");
+  // Per-cluster codebooks: one codebook of 256 entries a list, for all of its subspaces.  Each wave
+  // keeps the codebook of its current pair's list in its own eighth of the area that otherwise
+  // holds the eight leading subspaces' codebooks (the same bytes: eight waves a block), fetched a
+  // pair ahead like the pair's other operands (2 KB for two dimensions a subspace, out of L2:
+  // neighbouring waves work on pairs of the same list).
+  static_assert(!PER_CLUSTER || (BITS == 8 && kDirectThreads / 64u == SUB), "a wave's codebook takes one subspace's place");
+  constexpr uint32_t NCB = PER_CLUSTER ? BOOK / 64u : 1u;  // codebook entries a lane fetches
   auto* book      = reinterpret_cast<LDS_AS vec_t*>(uintptr_t(kScreenLdsBase));
   const float one = opaque_one_s();
   constexpr uint32_t off_pending = kScreenLdsBase + SUB * BOOK * uint32_t(sizeof(vec_t));
@@ -386,16 +393,19 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   const uint32_t p_end   = mine.end;
   if (mine.first - wid >= p_end) { return; }  // the whole block, before its barrier
 
-  for (uint32_t e = tid; e < SUB * BOOK; e += kDirectThreads) {
-    vec_t v = {};
+  if constexpr (!PER_CLUSTER) {
+    for (uint32_t e = tid; e < SUB * BOOK; e += kDirectThreads) {
+      vec_t v = {};
 #pragma unroll
-    for (int t = 0; t < PQ_LEN; t++) { v[t] = a.pq_centers[((e / BOOK) * PQ_LEN + t) * BOOK + (e % BOOK)]; }
-    book[e] = v;
+      for (int t = 0; t < PQ_LEN; t++) { v[t] = a.pq_centers[((e / BOOK) * PQ_LEN + t) * BOOK + (e % BOOK)]; }
+      book[e] = v;
+    }
+    lds_barrier_s();
   }
-  lds_barrier_s();
 
   uint32_t p = mine.first;
   if (p >= p_end) { return; }
+  auto* my_book = book + (PER_CLUSTER ? wid * BOOK : 0u);  // per cluster: entry `code` of the pair's list
   auto* pending = reinterpret_cast<LDS_AS uint32_t*>(uintptr_t(off_pending + wid * kSurvivorBatchBytes));
   auto* mini    = reinterpret_cast<LDS_AS lut_t*>(uintptr_t(off_mini + wid * uint32_t(FIRST) * 256u * uint32_t(sizeof(lut_t))));
   uint32_t n_pending = 0;
@@ -434,6 +444,22 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
     return a.rot_q[uint64_t(d.q) * a.rot_dim + dim] - a.centers_rot[uint64_t(d.label) * a.rot_dim + dim];
   };
 
+  // per cluster: entries lane, lane + 64, ... of a pair's list's codebook
+  struct book_part {
+    vec_t v[NCB];
+  };
+  auto fetch_book = [&](const pair_desc& d) -> book_part {
+    book_part b{};
+    if constexpr (PER_CLUSTER) {
+#pragma unroll
+      for (uint32_t c = 0; c < NCB; c++) {
+#pragma unroll
+        for (int t = 0; t < PQ_LEN; t++) { b.v[c][t] = a.pq_centers[(uint64_t(d.label) * PQ_LEN + t) * BOOK + c * 64u + lane]; }
+      }
+    }
+    return b;
+  };
+
   pair_desc d0 = uniform(record(p));
   pair_desc d1 = uniform(record(p + total));
   // leading codes of a pair's tiles 0 and 1 (the plane's slack covers tiles past a list's end)
@@ -441,6 +467,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   u32x2 next0 = lead_codes(d0, 1u);
   uint32_t thr0  = a.query_kth[d0.q];
   float dv0     = fetch_diff(d0);
+  book_part cb0 = fetch_book(d0);
 
   for (;;) {
     const bool has1    = p + total < p_end;
@@ -449,14 +476,21 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
     u32x2 next1        = next0;
     uint32_t thr1      = 0u;
     float dv1          = 0.0f;
+    book_part cb1      = cb0;
     if (has1) {
       lead1 = lead_codes(d1, 0u);
       next1 = lead_codes(d1, 1u);
       thr1  = a.query_kth[d1.q];
       dv1  = fetch_diff(d1);
+      cb1  = fetch_book(d1);
     }
 
     {
+      if constexpr (PER_CLUSTER) {
+        // the pair's codebook into the wave's area (the wave's own LDS accesses are performed in order)
+#pragma unroll
+        for (uint32_t c = 0; c < NCB; c++) { my_book[c * 64u + lane] = cb0.v[c]; }
+      }
       // terms of the first four subspaces, broadcast to scalar registers once per pair; those of
       // subspaces 4..7 are read where the few tiles that get that far need them
       constexpr uint32_t NEAGER = 4 * PQ_LEN;
@@ -481,7 +515,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
       if (tabled) {
 #pragma unroll
         for (uint32_t e = 0; e < uint32_t(FIRST) * BOOK / 64u; e++) {
-          const vec_t b = book[e * 64u + lane];
+          const vec_t b = PER_CLUSTER ? my_book[(e & 3u) * 64u + lane] : book[e * 64u + lane];
           float score   = 0.0f;
 #pragma unroll
           for (int t = 0; t < PQ_LEN; t++) {
@@ -512,7 +546,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
             if (decltype(use_table)::value && kk < FIRST) {
               v = mini[kk * int(BOOK) + c];
             } else {
-              const vec_t b = book[kk * int(BOOK) + c];
+              const vec_t b = PER_CLUSTER ? my_book[c] : book[kk * int(BOOK) + c];
               float score   = 0.0f;
 #pragma unroll
               for (int t = 0; t < PQ_LEN; t++) {
@@ -587,16 +621,17 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
     next0 = next1;
     thr0  = thr1;
     dv0   = dv1;
+    cb0   = cb1;
   }
   if (n_pending != 0) { flush_survivors(pending, n_pending, lane, survivors, n_survivors); }
 }
 
-template <int PQ_LEN, int LUT, bool OUT_HALF, int FIRST, int BITS>
+template <int PQ_LEN, int LUT, bool OUT_HALF, int FIRST, int BITS, bool PER_CLUSTER = false>
 void launch_screen_direct_first(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
                                 pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
                                 hipStream_t stream)
 {
-  auto kernel       = scan_screen_direct_kernel<PQ_LEN, LUT, OUT_HALF, FIRST, BITS>;
+  auto kernel       = scan_screen_direct_kernel<PQ_LEN, LUT, OUT_HALF, FIRST, BITS, PER_CLUSTER>;
   // codebooks of the leading subspaces (8 x 256 or 16 x 16 entries), a batch of survivors per wave,
   // and (byte codes) a wave's table of the first subspaces
   const size_t smem = kScreenLdsBase + size_t(kDirectSubs) * (BITS == 8 ? 256 : 32) * sizeof(typename book_vec<PQ_LEN>::type) +
@@ -615,10 +650,14 @@ void launch_screen_direct_first(const scan_args& a, const pair_desc* desc, uint3
   CUVS_HIP_TRY(hipGetLastError());
 }
 
-template <int PQ_LEN, int LUT, bool OUT_HALF>
+template <int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER = false>
 void launch_screen_direct(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
                           pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive, hipStream_t stream)
 {
+  if constexpr (PER_CLUSTER) {
+    launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, kScreenFirstCheck, 8, true>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+    return;
+  }
   if constexpr (PQ_LEN == 1 || PQ_LEN == 2 || PQ_LEN == 4) {
     if (a.pq_bits == 4) {
       launch_screen_direct_first<PQ_LEN, LUT, OUT_HALF, 4, 4>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
@@ -650,16 +689,21 @@ void launch_screen_sub(const scan_args& a, const pair_desc* desc, uint32_t n_pai
   CUVS_HIP_TRY(hipGetLastError());
 }
 
+constexpr uint32_t kPerClusterDirectRows = 1536;
 template <int PQ_LEN, int LUT, bool OUT_HALF, bool PER_CLUSTER>
 void launch_screen_instance(const scan_args& a, const pair_desc* desc, uint32_t n_pairs,
                             pair_desc* survivors, uint32_t* n_survivors, uint8_t* alive,
                             hipStream_t stream)
 {
-  if constexpr (!PER_CLUSTER) {
-    if (a.lead_plane != nullptr) {
-      launch_screen_direct<PQ_LEN, LUT, OUT_HALF>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
-      return;
-    }
+  // Per-cluster codebooks take the table-free kernel too (a wave then holds its pair's codebook),
+  // but only on lists of moderate length.  What decides is how many rows get past the first
+  // subspaces, each of which costs eight vector instructions here against a lookup there: lists
+  // of 610 / 1,220 / 1,830 rows of the 128-dimensional benchmark rows take 0.44 / 0.71 / 0.95 ms here
+  // and 0.87 / 1.27 ms with a table per pair, but lists of 2,000 rows of which a tenth survives
+  // (100 M rows, 200 probes) 14.8 ms here and 11.0 ms with tables.
+  if (a.lead_plane != nullptr && (!PER_CLUSTER || (a.pq_bits == 8 && a.mean_list_rows < kPerClusterDirectRows))) {
+    launch_screen_direct<PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
+    return;
   }
   launch_screen_sub<kScreenSubs, PQ_LEN, LUT, OUT_HALF, PER_CLUSTER>(a, desc, n_pairs, survivors, n_survivors, alive, stream);
 }

@@ -462,6 +462,7 @@ void search_one(cuvs::resources const& res_c,
   sa.lead_plane   = ix.lead_plane.bytes != 0 ? ix.lead_plane.as<uint64_t>() : nullptr;
   sa.inds_ptrs    = ix.inds_ptrs.as<const int64_t*>();
   sa.list_sizes   = ix.list_sizes.as<uint32_t>();
+  sa.mean_list_rows = uint32_t(std::min<uint64_t>(uint64_t(ix.size) / std::max<uint32_t>(ix.n_lists, 1u), 0xFFFFFFFFull));
   sa.filter_bits  = filter_bits;
   sa.filter_nbits = filter_nbits;
   if (ix.pq_bits != 8 && ix.pq_bits != 4) { sa.lead_plane = nullptr; }
