@@ -171,6 +171,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
     d.q          = uint32_t(__builtin_amdgcn_readfirstlane(d.q));
     d.slot       = uint32_t(__builtin_amdgcn_readfirstlane(d.slot));
     d.n_rows     = uint32_t(__builtin_amdgcn_readfirstlane(d.n_rows));
+    d.row_off    = uint32_t(__builtin_amdgcn_readfirstlane(d.row_off));
     return d;
   };
   // first chunk of row (64 * tile + lane) of a list; the code arena carries two groups of slack
@@ -179,6 +180,19 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   auto chunk_ptr = [&](const uint8_t* list_data, uint32_t tile) {
     return reinterpret_cast<const GLOBAL_AS codes_t*>(reinterpret_cast<uintptr_t>(list_data) +
                                                       uint64_t(tile) * (2u * group_bytes) + lane_off);
+  };
+  // Where the index keeps the plane of leading codes, a tile's eight leading bytes a row are one
+  // contiguous 512-byte load (from the interleaved lists: every other 8 bytes of two groups), and
+  // the plane's slack lets a wave request tiles unconditionally, two ahead of the one it sums.
+  const bool use_plane = SUBS <= 8 && a.lead_plane != nullptr;  // uniform
+  auto codes_of = [&](const pair_desc& d, uint32_t tile) -> codes_t {
+    if constexpr (SUBS <= 8) {
+      if (use_plane) {
+        const auto* plane = reinterpret_cast<const GLOBAL_AS u32x2*>(reinterpret_cast<uintptr_t>(a.lead_plane));
+        return plane[uint64_t(d.row_off) + tile * 64u + lane];
+      }
+    }
+    return *chunk_ptr(d.data, tile);
   };
   // staging element (pair tid / NDIFF, dimension tid % NDIFF) of iteration `it`
   auto fetch_diff = [&](uint32_t it) -> float {
@@ -196,10 +210,11 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   uint32_t it   = blockIdx.x;
   float staged  = fetch_diff(it);
   pair_desc my_d = uniform(record(it, wid));
-  codes_t cur{};
+  codes_t cur{}, cur1{};
   uint32_t thr   = 0xFFFFFFFFu;
   if (my_d.n_rows != 0) {
-    cur = *chunk_ptr(my_d.data, 0u);
+    cur = codes_of(my_d, 0u);
+    if (use_plane) { cur1 = codes_of(my_d, 1u); }
     thr = uint32_t(__builtin_amdgcn_readfirstlane(a.query_kth[my_d.q]));
   }
   if (tid < G * NDIFF) { diff_all[tid] = staged; }
@@ -245,14 +260,13 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
       const uint32_t n_tiles   = (n_rows + 63u) >> 6;
       const uint32_t stop_bits = thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u;
       bool in_play             = false;
-      for (uint32_t tile = 0; tile < n_tiles && !in_play; tile++) {
+      // sums the leading codes `c8` of the rows of tile `tile`
+      auto sum_tile = [&](const codes_t& c8, uint32_t tile) __attribute__((always_inline)) {
         const uint32_t i = tile * 64u + lane;
-        codes_t ahead    = cur;
-        if (tile + 1u < n_tiles) { ahead = *chunk_ptr(my_d.data, tile + 1u); }
-        uint32_t w[4] = {cur.x, cur.y, 0u, 0u};
+        uint32_t w[4] = {c8.x, c8.y, 0u, 0u};
         if constexpr (SUBS > 8) {
-          w[2] = cur.z;
-          w[3] = cur.w;
+          w[2] = c8.z;
+          w[3] = c8.w;
         }
         acc_t acc           = acc_t(0);
         auto add_codes = [&](int first, int last) __attribute__((always_inline)) {
@@ -276,7 +290,28 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
           add_codes(SUBS / 2, SUBS);
           in_play = __ballot(i < n_rows && !(__float_as_uint(float(acc)) > stop_bits)) != 0ull;
         }
-        cur     = ahead;
+      };
+      if (use_plane) {
+        // three registers take turns: two tiles are in flight while one is summed
+        codes_t r0 = cur, r1 = cur1, r2;
+        for (uint32_t tile = 0; tile < n_tiles; tile += 3u) {
+          r2 = codes_of(my_d, tile + 2u);
+          sum_tile(r0, tile);
+          if (in_play || tile + 1u >= n_tiles) { break; }
+          r0 = codes_of(my_d, tile + 3u);
+          sum_tile(r1, tile + 1u);
+          if (in_play || tile + 2u >= n_tiles) { break; }
+          r1 = codes_of(my_d, tile + 4u);
+          sum_tile(r2, tile + 2u);
+          if (in_play) { break; }
+        }
+      } else {
+        for (uint32_t tile = 0; tile < n_tiles && !in_play; tile++) {
+          codes_t ahead = cur;
+          if (tile + 1u < n_tiles) { ahead = *chunk_ptr(my_d.data, tile + 1u); }
+          sum_tile(cur, tile);
+          cur = ahead;
+        }
       }
       if (in_play) { push_survivor(pending, n_pending, lane, my_d, survivors, n_survivors, alive); }
     }
@@ -285,7 +320,8 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
     my_d = nxt_d;
     thr  = 0xFFFFFFFFu;
     if (my_d.n_rows != 0) {
-      cur = *chunk_ptr(my_d.data, 0u);
+      cur = codes_of(my_d, 0u);
+      if (use_plane) { cur1 = codes_of(my_d, 1u); }
       thr = uint32_t(__builtin_amdgcn_readfirstlane(a.query_kth[my_d.q]));
     }
     it = nxt_it;
