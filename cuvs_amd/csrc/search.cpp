@@ -41,7 +41,8 @@ using detail::index_impl;
 
 constexpr uint32_t kMaxFusedK = 256;   // larger k dumps all scores and selects afterwards
 constexpr size_t kMaxLds      = 160 * 1024;
-constexpr uint32_t kFewPairs  = 1024;  // (query, probe) pairs of a batch below which they are scanned in one plain launch
+constexpr uint32_t kFewPairs  = 640;  // (query, probe) pairs of a batch up to which they are scanned in one plain launch
+                                       // (headline index, 64 probes: 8 queries 0.082 ms; 16 queries 0.12 ms against 0.098 ms by the early stop)
 
 /** A pointer is usable by kernels when HIP knows it as device, managed or pinned host memory
  *  (role of utils::check_pointer_residency, detail/ann_utils.cuh). */
