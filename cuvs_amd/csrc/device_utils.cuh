@@ -206,13 +206,13 @@ __device__ uint32_t block_select_sorted(KeyFn key_of, uint32_t n, uint32_t k,
 }
 
 /**
- * The same result for at most kBlock * kMinimaPer keys and k <= kBlock, in one pass over the keys:
- * thread t holds keys t, t + kBlock, ... in registers; the k-th smallest of the kBlock per-thread
- * minima (by the keys' high words) is at or above the k-th smallest key, and for keys in no
- * particular order only a few more than k lie at or below it; those are collected in LDS (the
- * histogram area of `sm`) and ranked.  Returns false, with nothing written, when more than 1024
- * keys pass the bound (keys in an adversarial order, or k close to the number of threads' worth of
- * valid keys): the caller then selects by radix passes.
+ * The same result for k <= kBlock, in one or two passes over the keys: thread t takes keys t,
+ * t + kBlock, ... (up to kMinimaPer of them stay in registers; more are read a second time); the
+ * k-th smallest of the kBlock per-thread minima (by the keys' high words) is at or above the k-th
+ * smallest key, and for keys in no particular order only a few more than k lie at or below it;
+ * those are collected in LDS (the histogram area of `sm`) and ranked.  Returns false, with nothing
+ * written, when more than 1024 keys pass the bound (keys in an adversarial order, or k close to the
+ * number of threads' worth of valid keys): the caller then selects by radix passes.
  */
 constexpr uint32_t kMinimaPer = 16;
 template <typename KeyFn>
@@ -227,17 +227,34 @@ __device__ bool block_select_by_minima(KeyFn key_of, uint32_t n, uint32_t k, uns
   const uint32_t tid  = threadIdx.x;
   const uint32_t lane = tid & 63u;
   const uint32_t wid  = tid >> 6;
+  const bool held = n <= kBlock * kMinimaPer;  // uniform
   unsigned long long key[kMinimaPer];
-#pragma unroll
-  for (uint32_t j = 0; j < kMinimaPer; j++) {
-    const uint32_t i = j * kBlock + tid;
-    key[j]           = i < n ? key_of(i) : kInvalidKey;
-  }
   uint32_t mine = 0xFFFFFFFFu;
+  if (held) {
 #pragma unroll
-  for (uint32_t j = 0; j < kMinimaPer; j++) {
-    const uint32_t hi = uint32_t(key[j] >> 32);
-    mine              = hi < mine ? hi : mine;
+    for (uint32_t j = 0; j < kMinimaPer; j++) {
+      const uint32_t i = j * kBlock + tid;
+      key[j]           = i < n ? key_of(i) : kInvalidKey;
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < kMinimaPer; j++) {
+      const uint32_t hi = uint32_t(key[j] >> 32);
+      mine              = hi < mine ? hi : mine;
+    }
+  } else {
+    // one block may be the only one with this many keys, so what bounds it is the number of
+    // requests it keeps in flight: sixteen per thread here, eight where whole keys come back
+    constexpr uint32_t kAhead = 16;
+    for (uint32_t i0 = tid; i0 < n; i0 += kAhead * kBlock) {
+      uint32_t hi[kAhead];
+#pragma unroll
+      for (uint32_t u = 0; u < kAhead; u++) {
+        const uint32_t i = i0 + u * kBlock;
+        hi[u]            = i < n ? uint32_t(key_of(i) >> 32) : 0xFFFFFFFFu;
+      }
+#pragma unroll
+      for (uint32_t u = 0; u < kAhead; u++) { mine = hi[u] < mine ? hi[u] : mine; }
+    }
   }
   if (tid == 0) {
     s_bound = 0xFFFFFFFFu;
@@ -280,11 +297,30 @@ __device__ bool block_select_by_minima(KeyFn key_of, uint32_t n, uint32_t k, uns
   __syncthreads();
   const uint32_t bound = s_bound;
   if (mine <= bound) {
+    if (held) {
 #pragma unroll
-    for (uint32_t j = 0; j < kMinimaPer; j++) {
-      if (key[j] != kInvalidKey && uint32_t(key[j] >> 32) <= bound) {
-        const uint32_t pos = atomicAdd(&s_count, 1u);
-        if (pos < kCap) { cand[pos] = key[j]; }
+      for (uint32_t j = 0; j < kMinimaPer; j++) {
+        if (key[j] != kInvalidKey && uint32_t(key[j] >> 32) <= bound) {
+          const uint32_t pos = atomicAdd(&s_count, 1u);
+          if (pos < kCap) { cand[pos] = key[j]; }
+        }
+      }
+    } else {
+      constexpr uint32_t kAhead = 8;
+      for (uint32_t i0 = tid; i0 < n; i0 += kAhead * kBlock) {
+        unsigned long long again[kAhead];
+#pragma unroll
+        for (uint32_t u = 0; u < kAhead; u++) {
+          const uint32_t i = i0 + u * kBlock;
+          again[u]         = i < n ? key_of(i) : kInvalidKey;
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < kAhead; u++) {
+          if (again[u] != kInvalidKey && uint32_t(again[u] >> 32) <= bound) {
+            const uint32_t pos = atomicAdd(&s_count, 1u);
+            if (pos < kCap) { cand[pos] = again[u]; }
+          }
+        }
       }
     }
   }

@@ -1221,12 +1221,14 @@ __device__ void merge_query(const merge_args& a, uint32_t out_cap, uint32_t q)
     const unsigned long long* keys = a.in_keys + uint64_t(q) * n;
     if (a.alive == nullptr) {
       auto key_of = [keys](uint32_t i) { return keys[i]; };
-      if (!(n <= kBlock * kMinimaPer && a.k <= kBlock && block_select_by_minima(key_of, n, a.k, out, out_cap, sm))) {
+      if (!(a.k <= kBlock && block_select_by_minima(key_of, n, a.k, out, out_cap, sm))) {
         block_select_sorted(key_of, n, a.k, out, out_cap, sm);
       }
     } else {
       // pairs that the screen dropped wrote no keys: gather the slots that did, select among those
-      __shared__ uint16_t live_slots[kMergeMaxProbes];
+      // (the slot list follows the output area in the launch's LDS: n_probes 16-bit numbers)
+      uint16_t* live_slots =
+        reinterpret_cast<uint16_t*>(dyn_smem + (a.out_scratch != nullptr ? 0u : out_cap * 8u));
       __shared__ uint32_t n_live;
       const uint8_t* alive = a.alive + uint64_t(q) * a.n_probes;
       const uint32_t kpp   = a.keys_per_pair;
@@ -1241,7 +1243,8 @@ __device__ void merge_query(const merge_args& a, uint32_t out_cap, uint32_t q)
       if (n_keys <= kSmall) {
         // a handful of live pairs (the usual case after screening): rank every key against all
         // others in LDS; keys are distinct (the sample number is part of the key)
-        __shared__ unsigned long long small_keys[kSmall];
+        static_assert(sizeof(sm.hist) >= kSmall * sizeof(unsigned long long), "small_keys area");
+        unsigned long long* small_keys = reinterpret_cast<unsigned long long*>(sm.hist);
         for (uint32_t i = threadIdx.x; i < n_keys; i += kBlock) {
           small_keys[i] = keys[uint32_t(live_slots[i / kpp]) * kpp + i % kpp];
         }
@@ -1256,9 +1259,8 @@ __device__ void merge_query(const merge_args& a, uint32_t out_cap, uint32_t q)
         }
         __syncthreads();
       } else {
-        auto key_of = [keys, kpp](uint32_t i) { return keys[uint32_t(live_slots[i / kpp]) * kpp + i % kpp]; };
-        if (!(n_keys <= kBlock * kMinimaPer && a.k <= kBlock &&
-              block_select_by_minima(key_of, n_keys, a.k, out, out_cap, sm))) {
+        auto key_of = [keys, kpp, live_slots](uint32_t i) { return keys[uint32_t(live_slots[i / kpp]) * kpp + i % kpp]; };
+        if (!(a.k <= kBlock && block_select_by_minima(key_of, n_keys, a.k, out, out_cap, sm))) {
           block_select_sorted(key_of, n_keys, a.k, out, out_cap, sm);
         }
       }
@@ -1851,8 +1853,12 @@ void launch_merge(const merge_args& a, hipStream_t stream)
 {
   if (a.n_queries == 0) { return; }
   const uint32_t out_cap = next_pow2(a.k);
-  const size_t smem      = a.out_scratch != nullptr ? 0 : size_t(out_cap) * 8;
-  CUVS_EXPECTS(smem <= 96 * 1024, "k (%u) is too large for the merge kernel", a.k);
+  const size_t out_smem  = a.out_scratch != nullptr ? 0 : size_t(out_cap) * 8;
+  // with the list of live pairs: their slot numbers behind the output area
+  const size_t smem = out_smem + (a.fused && a.alive != nullptr ? (size_t(a.n_probes) * 2 + 15) & ~size_t(15) : 0);
+  CUVS_EXPECTS(out_smem <= 96 * 1024, "k (%u) is too large for the merge kernel", a.k);
+  CUVS_EXPECTS(!(a.fused && a.alive != nullptr) || a.n_probes <= kMergeMaxProbes,
+               "the merge with a list of live pairs takes up to %u probes (%u given)", kMergeMaxProbes, a.n_probes);
   if (smem > 32 * 1024) {
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(merge_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
