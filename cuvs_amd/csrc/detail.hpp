@@ -307,12 +307,13 @@ void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries,
 /** chunk_indices[q, p] = inclusive prefix sum of list_sizes[probes[q, p]]; n_samples[q] = total.
  *  When `stats` is non-null (kStatSlots x 4 words), query q adds the scanned bytes, the rows and
  *  the bytes of its leading probes to words 0, 1, 2 of slot q % kStatSlots.  `query_max`
- *  (n_queries words) is filled with 0xFFFFFFFF and `zero_word` (one word) with 0 when given. */
+ *  (n_queries words) is filled with 0xFFFFFFFF and the `n_zero_words` words at `zero_words` with 0
+ *  when given. */
 constexpr uint32_t kStatSlots = 256;
 void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
                           uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
                           uint32_t* n_samples, unsigned long long* stats, uint32_t lead_probes,
-                          uint32_t* query_max, uint32_t* zero_word, hipStream_t stream);
+                          uint32_t* query_max, uint32_t* zero_words, uint32_t n_zero_words, hipStream_t stream);
 
 /** Everything the scan needs to know about one (query, probe) pair, gathered once so that the
  *  scan kernel reads one 32-byte record instead of chasing four dependent pointers. */
@@ -451,7 +452,18 @@ bool launch_scan_slab(const scan_args& a, hipStream_t stream);
  * subspaces only, sums the first 16-byte chunk of every row of a pair and keeps the pair only if
  * some row is still below the query's bound; surviving records are appended to `survivors`
  * (`n_survivors` counts them) and their slot is marked in `alive`.
+ *
+ * `n_survivors` is the first of kSurvivorWords words.  launch_order_survivors() copies the records
+ * into `ordered` by length class (lists of more 64-row tiles first; its table of counts takes the
+ * words from kSurvivorTable on): the persistent scan kernels hand their blocks the records in turn
+ * and couple the pairs of an iteration, so records in order of length give every block the same
+ * work and an iteration two pairs of the same length.
  */
+constexpr uint32_t kSurvivorClasses = 256;
+constexpr uint32_t kSurvivorTable   = 64;
+constexpr uint32_t kSurvivorWords   = kSurvivorTable + 64 * kSurvivorClasses;
+void launch_order_survivors(const pair_desc* survivors, uint32_t* n_survivors, pair_desc* ordered,
+                            hipStream_t stream);
 bool scan_screen_supported(const scan_args& a);
 /** Bytes of each row the screen reads (8 or 16). */
 uint32_t scan_screen_bytes_per_row(bool per_cluster, bool lead_plane);

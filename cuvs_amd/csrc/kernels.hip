@@ -423,14 +423,17 @@ __global__ __launch_bounds__(64) void chunk_indices_kernel(const uint32_t* __res
                                                             unsigned long long* stats,
                                                             uint32_t lead_probes,
                                                             uint32_t* __restrict__ query_max,
-                                                            uint32_t* __restrict__ zero_word)
+                                                            uint32_t* __restrict__ zero_words,
+                                                            uint32_t n_zero_words)
 {
   const uint32_t q    = blockIdx.x;
   const uint32_t lane = threadIdx.x;
   // start values of the scan that follows, set here to save two launches: every query's bound at
   // its largest, the survivor count at zero
   if (lane == 0 && query_max != nullptr) { query_max[q] = 0xFFFFFFFFu; }
-  if (lane == 0 && q == 0 && zero_word != nullptr) { *zero_word = 0u; }
+  if (q == 0 && zero_words != nullptr) {
+    for (uint32_t w = lane; w < n_zero_words; w += 64u) { zero_words[w] = 0u; }
+  }
   uint32_t carry      = 0;
   unsigned long long padded_rows = 0, lead_rows = 0;
   for (uint32_t p0 = 0; p0 < n_probes; p0 += 64) {
@@ -1624,12 +1627,12 @@ void launch_rotate(const float* qf, const float* rotation_t, uint32_t n_queries,
 void launch_chunk_indices(const uint32_t* list_sizes, const uint32_t* probes, uint32_t n_queries,
                           uint32_t n_probes, uint32_t row_chunk_bytes, uint32_t* chunk_indices,
                           uint32_t* n_samples, unsigned long long* stats, uint32_t lead_probes,
-                          uint32_t* query_max, uint32_t* zero_word, hipStream_t stream)
+                          uint32_t* query_max, uint32_t* zero_words, uint32_t n_zero_words, hipStream_t stream)
 {
   if (n_queries == 0) { return; }
   chunk_indices_kernel<<<n_queries, 64, 0, stream>>>(list_sizes, probes, n_probes, row_chunk_bytes,
                                                      chunk_indices, n_samples, stats, lead_probes, query_max,
-                                                     zero_word);
+                                                     zero_words, n_zero_words);
   CUVS_LAUNCH_CHECK();
 }
 

@@ -70,6 +70,13 @@ constexpr uint32_t kSurvivorBatchBytes = kSurvivorBatch * uint32_t(sizeof(pair_d
 static_assert(kSurvivorBatchBytes == 4 * 64 * 4, "a full batch is four dwords per lane");
 static_assert(offsetof(pair_desc, q) == 8 && offsetof(pair_desc, row_off) == 28, "record layout");
 
+/** Length class of a list of n_rows rows: by its number of 64-row tiles, the longest first. */
+__device__ __forceinline__ uint32_t class_of_rows(uint32_t n_rows)
+{
+  const uint32_t tiles = (n_rows + 63u) >> 6;
+  return tiles >= kSurvivorClasses ? 0u : kSurvivorClasses - 1u - tiles;
+}
+
 __device__ __forceinline__ void flush_survivors(LDS_AS uint32_t* pending, uint32_t n, uint32_t lane,
                                                 pair_desc* __restrict__ survivors,
                                                 uint32_t* __restrict__ n_survivors)
@@ -1188,6 +1195,81 @@ bool scan_screen_ip(const scan_args& a)
   if (a.per_cluster || a.lead_plane == nullptr || a.rot_dim != a.pq_dim * a.pq_len) { return false; }
   if (a.pq_dim > 64u * kIpRounds) { return false; }
   return a.pq_len == 1 || a.pq_len == 2 || a.pq_len == 4;
+}
+
+/*
+ * The surviving records class by class, as a counting sort without global atomics: every block
+ * counts the classes of its contiguous run of records in LDS (order_survivors_count_kernel); every
+ * block then finds where its records of each class go from the table of (block, class) counts and
+ * moves them (order_survivors_move_kernel).  Records that follow each other in the input (the
+ * survivors of one list, as a rule) stay neighbours.
+ */
+constexpr uint32_t kOrderSurvivorThreads = 256;
+constexpr uint32_t kOrderSurvivorBlocks  = 64;
+static_assert(kOrderSurvivorThreads == kSurvivorClasses, "a thread per class in the scans");
+static_assert(kSurvivorTable + kOrderSurvivorBlocks * kSurvivorClasses <= kSurvivorWords, "table of counts");
+
+__global__ __launch_bounds__(kOrderSurvivorThreads) void order_survivors_count_kernel(
+  const pair_desc* __restrict__ survivors, uint32_t* __restrict__ words)
+{
+  __shared__ uint32_t hist[kSurvivorClasses];
+  const uint32_t tid = threadIdx.x;
+  hist[tid]          = 0;
+  __syncthreads();
+  const uint32_t n   = words[0];
+  const uint32_t per = (n + gridDim.x - 1u) / gridDim.x;
+  const uint32_t i0  = blockIdx.x * per;
+  const uint32_t i1  = i0 + per < n ? i0 + per : n;
+  for (uint32_t i = i0 + tid; i < i1; i += kOrderSurvivorThreads) {
+    atomicAdd(&hist[class_of_rows(survivors[i].n_rows)], 1u);
+  }
+  __syncthreads();
+  words[kSurvivorTable + blockIdx.x * kSurvivorClasses + tid] = hist[tid];
+}
+
+__global__ __launch_bounds__(kOrderSurvivorThreads) void order_survivors_move_kernel(
+  const pair_desc* __restrict__ survivors, const uint32_t* __restrict__ words, pair_desc* __restrict__ ordered)
+{
+  __shared__ uint32_t start[kSurvivorClasses];
+  __shared__ uint32_t wave_sums[kOrderSurvivorThreads / 64];
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wid = tid >> 6;
+  // thread = class: records of the class in all blocks, and in the blocks before this one
+  uint32_t total = 0, before = 0;
+#pragma unroll 8
+  for (uint32_t b = 0; b < kOrderSurvivorBlocks; b++) {
+    const uint32_t c = words[kSurvivorTable + b * kSurvivorClasses + tid];
+    total += c;
+    before += b < blockIdx.x ? c : 0u;
+  }
+  const uint32_t incl = wave_inclusive_scan(total);
+  if (lane == 63u) { wave_sums[wid] = incl; }
+  __syncthreads();
+  uint32_t classes_before = 0;
+  for (uint32_t w = 0; w < wid; w++) { classes_before += wave_sums[w]; }
+  start[tid] = classes_before + incl - total + before;
+  __syncthreads();
+  const uint32_t n   = words[0];
+  const uint32_t per = (n + gridDim.x - 1u) / gridDim.x;
+  const uint32_t i0  = blockIdx.x * per;
+  const uint32_t i1  = i0 + per < n ? i0 + per : n;
+  for (uint32_t i = i0 + tid; i < i1; i += kOrderSurvivorThreads) {
+    const u32x4* src = reinterpret_cast<const u32x4*>(survivors + i);
+    const u32x4 lo = src[0], hi = src[1];
+    const uint32_t pos = atomicAdd(&start[class_of_rows(hi.z)], 1u);  // hi.z: n_rows
+    u32x4* dst = reinterpret_cast<u32x4*>(ordered + pos);
+    dst[0]     = lo;
+    dst[1]     = hi;
+  }
+}
+
+void launch_order_survivors(const pair_desc* survivors, uint32_t* n_survivors, pair_desc* ordered,
+                            hipStream_t stream)
+{
+  static_assert(offsetof(pair_desc, n_rows) == 24, "n_rows is the third word of the record's second half");
+  order_survivors_count_kernel<<<kOrderSurvivorBlocks, kOrderSurvivorThreads, 0, stream>>>(survivors, n_survivors);
+  CUVS_HIP_TRY(hipGetLastError());
+  order_survivors_move_kernel<<<kOrderSurvivorBlocks, kOrderSurvivorThreads, 0, stream>>>(survivors, n_survivors, ordered);
+  CUVS_HIP_TRY(hipGetLastError());
 }
 
 bool scan_screen_supported(const scan_args& a)

@@ -504,6 +504,7 @@ void search_one(cuvs::resources const& res_c,
   const bool fast_coarse = coarse_fast_applies(res, params, ix, P);
   auto bytes_for = [&](uint32_t batch) {
     return pl.fixed_bytes + size_t(batch) * (pl.per_query_bytes + 64) + 16 * 256 + global_lut_bytes +
+           a256(detail::kSurvivorWords * sizeof(uint32_t)) +
            (fast_coarse ? coarse_fast_bytes(ix, batch) : 0) + a256(detail::scan_screen_scratch_bytes(sa, batch));
   };
   if (res.workspace_borrowed()) {
@@ -604,7 +605,7 @@ void search_one(cuvs::resources const& res_c,
   if (early_stop) {
     survivors   = static_cast<detail::pair_desc*>(res.workspace_alloc(size_t(Qb) * P * sizeof(detail::pair_desc)));
     alive       = static_cast<uint8_t*>(res.workspace_alloc(size_t(Qb) * P));
-    n_survivors = static_cast<uint32_t*>(res.workspace_alloc(256));
+    n_survivors = static_cast<uint32_t*>(res.workspace_alloc(detail::kSurvivorWords * sizeof(uint32_t)));
     merge_redo  = static_cast<uint8_t*>(res.workspace_alloc(size_t(Qb)));
     if (screen_scratch_bytes != 0) { screen_scratch = res.workspace_alloc(screen_scratch_bytes); }
   }
@@ -661,7 +662,7 @@ void search_one(cuvs::resources const& res_c,
     }
     detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
                                  ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead,
-                                 pl.fused ? kth : nullptr, n_survivors, s);
+                                 pl.fused ? kth : nullptr, n_survivors, 1, s);
     detail::launch_order_pairs(probes, chunk, sa.data_ptrs,
                                ix.inds_ptrs.as<const int64_t*>(), ix.ids_arena.as<int64_t>(), nq * P, P,
                                ix.n_lists, counters, sort_scratch, order, desc, lead, alive, few_pairs, list_rank, s);
@@ -737,8 +738,11 @@ void search_one(cuvs::resources const& res_c,
         }
       }
       mark(6);
-      // 3. the pairs still in play, in full
-      sa.desc        = survivors;
+      // 3. the pairs still in play, in full, from long lists to short ones (the records of the
+      // screened pairs are done with: the ordered ones take their place)
+      detail::pair_desc* ordered = desc + size_t(nq) * lead;
+      detail::launch_order_survivors(survivors, n_survivors, ordered, s);
+      sa.desc        = ordered;
       sa.n_pairs     = 0;
       sa.n_pairs_dev = n_survivors;
       full_scan(true);
