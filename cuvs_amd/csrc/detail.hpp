@@ -129,7 +129,11 @@ struct screen_feedback {
     uint32_t probes = 0, k = 0;    // 0: unused entry
     bool off                = false;
     uint32_t plain_searches = 0;   // since the verdict
+    uint32_t screened_searches = 0;  // with the screen on
   };
+  /** With a verdict for the screen, every kObserveEvery-th screened search is observed (the copy of
+   *  the survivor count is a launch of its own on the search's stream). */
+  static constexpr uint32_t kObserveEvery = 8;
   static constexpr int kVerdicts = 8;
   verdict verdicts[kVerdicts];
   /** The entry of (probes, k), moved to the front; null when there is none. */

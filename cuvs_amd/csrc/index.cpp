@@ -71,6 +71,7 @@ void screen_feedback::collect()
     v         = &verdicts[0];
     v->probes = pending_probes;
     v->k      = pending_k;
+    v->screened_searches = 0;
   }
   v->off            = double(host[0]) > kKeepLimit * double(pending_pairs);
   v->plain_searches = 0;

@@ -593,6 +593,11 @@ void search_one(cuvs::resources const& res_c,
       if (verdict->plain_searches % detail::screen_feedback::kScreenRecheck != 0) { early_stop = false; }
     }
     observe_screen = early_stop && capture == hipStreamCaptureStatusNone;
+    if (observe_screen && verdict != nullptr && !verdict->off) {
+      // (a search that tries the screen again after a verdict against it is always observed)
+      observe_screen = verdict->screened_searches % detail::screen_feedback::kObserveEvery == 0;
+      verdict->screened_searches += 1;
+    }
   }
   const uint32_t lead          = early_stop ? kLeadProbes : P;
   void* sort_scratch = few_pairs ? nullptr
