@@ -256,10 +256,14 @@ void launch_coarse_scores_mfma(const float* qt, const float* ct, uint32_t n_quer
 /** The probe selection reads whole segments of 256 x 64 scores: the score buffer must have this
  *  many readable bytes after its last row. */
 constexpr size_t kSelectSlackBytes = 256 * 64 * 4;
-/** With `only` non-null, queries whose byte there is zero are left alone. */
+/** With `only` non-null, queries whose byte there is zero are left alone.  Beyond kSelectLdsProbes
+ *  probes the selection's output does not fit a block's LDS: `scratch` then has
+ *  select_probes_scratch_bytes(n_queries, n_probes) bytes. */
+constexpr uint32_t kSelectLdsProbes = 8192;
+size_t select_probes_scratch_bytes(uint32_t n_queries, uint32_t n_probes);
 void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_lists,
                           uint32_t n_probes, uint32_t* probes, hipStream_t stream,
-                          const uint8_t* only = nullptr);
+                          const uint8_t* only = nullptr, void* scratch = nullptr);
 
 /* coarse search in 8-bit integers (coarse_i8.hip): 32-bit words of the quantised centre rows,
  * word-major, and scores written as floats that order like the integer scores */

@@ -148,12 +148,14 @@ __global__ __launch_bounds__(kBlock) void select_probes_kernel(const float* __re
                                                                 uint32_t n_probes,
                                                                 uint32_t out_cap,
                                                                 uint32_t* __restrict__ probes,
-                                                                const uint8_t* __restrict__ only)
+                                                                const uint8_t* __restrict__ only,
+                                                                unsigned long long* __restrict__ out_global)
 {
   extern __shared__ __align__(16) unsigned char dyn_smem[];
   __shared__ select_smem sm;
-  unsigned long long* out = reinterpret_cast<unsigned long long*>(dyn_smem);
   const uint32_t q        = blockIdx.x;
+  unsigned long long* out = out_global != nullptr ? out_global + uint64_t(q) * out_cap
+                                                  : reinterpret_cast<unsigned long long*>(dyn_smem);
   if (only != nullptr && !only[q]) { return; }
   const float* row        = scores + uint64_t(q) * n_lists;
   auto key_of             = [row](uint32_t i) -> unsigned long long {
@@ -1581,8 +1583,14 @@ void launch_coarse_scores(const float* qf, const float* centers, uint32_t n_quer
   CUVS_LAUNCH_CHECK();
 }
 
+size_t select_probes_scratch_bytes(uint32_t n_queries, uint32_t n_probes)
+{
+  return n_probes <= kSelectLdsProbes ? 0 : size_t(n_queries) * next_pow2(n_probes) * 8;
+}
+
 void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_lists,
-                          uint32_t n_probes, uint32_t* probes, hipStream_t stream, const uint8_t* only)
+                          uint32_t n_probes, uint32_t* probes, hipStream_t stream, const uint8_t* only,
+                          void* scratch)
 {
   if (n_queries == 0) { return; }
   if (n_probes <= kBlock) {
@@ -1597,13 +1605,15 @@ void launch_select_probes(const float* scores, uint32_t n_queries, uint32_t n_li
     return;
   }
   const uint32_t out_cap = next_pow2(n_probes);
-  const size_t smem      = size_t(out_cap) * 8;
-  CUVS_EXPECTS(smem <= 96 * 1024, "n_probes (%u) is too large for the probe selection kernel", n_probes);
+  const bool in_lds      = n_probes <= kSelectLdsProbes;
+  const size_t smem      = in_lds ? size_t(out_cap) * 8 : 0;
+  CUVS_EXPECTS(in_lds || scratch != nullptr, "n_probes (%u): the probe selection needs its scratch buffer", n_probes);
   if (smem > 32 * 1024) {
     CUVS_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(select_probes_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(smem)));
   }
-  select_probes_kernel<<<n_queries, kBlock, smem, stream>>>(scores, n_lists, n_probes, out_cap, probes, only);
+  select_probes_kernel<<<n_queries, kBlock, smem, stream>>>(scores, n_lists, n_probes, out_cap, probes, only,
+                                                            in_lds ? nullptr : static_cast<unsigned long long*>(scratch));
   CUVS_LAUNCH_CHECK();
 }
 

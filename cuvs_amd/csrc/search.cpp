@@ -98,7 +98,8 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
                       size_t(ix.rot_dim) * 4 +
                       P * 4 * 3 + P * (2 * sizeof(detail::pair_desc) + 1) + 17 + P * 17 +
                       (p.fused ? P * k * 8 * 4 : size_t(p.max_samples) * 4) +
-                      (k > detail::kMergeLdsK ? size_t(next_pow2(k)) * 8 : 0);
+                      (k > detail::kMergeLdsK ? size_t(next_pow2(k)) * 8 : 0) +
+                      detail::select_probes_scratch_bytes(1, uint32_t(P));
   p.fixed_bytes = a256(size_t(ix.n_lists) * 16 + 16) + 3 * 256 + size_t(512) * 8 + a256(size_t(ix.dim_ext) * 128 * 4) + a256(detail::kSelectSlackBytes) + 20 * 256;
   if (ix.coarse_fast_ok) {
     // buffers of the two-precision probe selection (the batch must fit with them)
@@ -164,6 +165,7 @@ struct coarse_buffers {
   float* qf;
   float* scores;
   uint32_t* probes;
+  void* select_scratch = nullptr;  // beyond kSelectLdsProbes probes: where the selection writes
   // two-precision selection (null when it does not apply)
   _Float16* qh      = nullptr;
   float* qnorm      = nullptr;
@@ -250,13 +252,13 @@ void run_coarse(const cuvs::resources& res, const search_params& params, const i
     // ivf_pq_search.cuh:170-256
     detail::launch_coarse_scores_i8(b.qf, ix.centers_i8.as<uint32_t>(), nq, ix.n_lists, ix.dim, ip,
                                     b.scores, s);
-    detail::launch_select_probes(b.scores, nq, ix.n_lists, n_probes, b.probes, s);
+    detail::launch_select_probes(b.scores, nq, ix.n_lists, n_probes, b.probes, s, nullptr, b.select_scratch);
     return;
   }
   detail::launch_map_queries_t(queries, type, nq, ix.dim, ix.dim_ext, ip, b.qt, s);
   detail::launch_coarse_scores_mfma(b.qt, ix.centers_t.as<float>(), nq, ix.n_lists, ix.dim_ext, ip,
                                     params.coarse_search_dtype == CUDA_R_16F, b.scores, s);
-  detail::launch_select_probes(b.scores, nq, ix.n_lists, n_probes, b.probes, s);
+  detail::launch_select_probes(b.scores, nq, ix.n_lists, n_probes, b.probes, s, nullptr, b.select_scratch);
 }
 
 }  // namespace
@@ -536,6 +538,9 @@ void search_one(cuvs::resources const& res_c,
   auto* kth       = static_cast<uint32_t*>(res.workspace_alloc(size_t(Qb) * 4));
   auto* counters  = static_cast<uint32_t*>(res.workspace_alloc(size_t(ix.n_lists) * 16 + 16));
   coarse_buffers cb{qt, qf, scores, probes};
+  if (detail::select_probes_scratch_bytes(Qb, P) != 0) {
+    cb.select_scratch = res.workspace_alloc(detail::select_probes_scratch_bytes(Qb, P));
+  }
   if (fast_coarse) { alloc_coarse_fast(res, ix, Qb, cb); }
   detail::pair_desc* desc = nullptr;
   unsigned long long* keys = nullptr;

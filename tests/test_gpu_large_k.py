@@ -1,7 +1,9 @@
 """k and candidate counts beyond what the selection kernels hold in LDS: the reference's search has
 no limit on k other than the index size (its non-fused path selects over every probed row,
 cpp/src/neighbors/ivf_pq/ivf_pq_search.cuh:637-655), nor has its refinement on the number of
-candidates.  Here the selection's output then lives in a global scratch buffer."""
+candidates.  Here the selection's output then lives in a global scratch buffer.  The same holds for
+the number of probes (the reference takes any n_probes up to n_lists, ivf_pq_search.cuh:932): the
+probe selection keeps up to 8192 probes in LDS and writes to the workspace beyond."""
 import numpy as np
 import pytest
 import torch
@@ -46,3 +48,20 @@ def test_refine_of_more_candidates_than_lds_holds(orc):
     assert differ.mean() < 1e-2
     for q, r in zip(*np.nonzero(differ)):
         assert abs(want_d[q, r] - got_d[q, r]) <= 1e-5 * max(1.0, abs(want_d[q, r]))
+
+
+@pytest.mark.parametrize("n_probes", [8192, 8193, 9000])
+def test_search_with_more_probes_than_the_selection_kernels_lds(orc, n_probes):
+    rng = np.random.default_rng(17)
+    n, dim, n_lists, pq_dim = 60000, 32, 9000, 16
+    data = rng.standard_normal((n, dim)).astype(np.float32)
+    queries = rng.standard_normal((7, dim)).astype(np.float32)
+    model = H.train(data, n_lists, pq_dim, 8, iters=2)
+    index = G.build_gpu_index(model, data, pq_dim, 8)
+    ix, _ = G.read_back(orc, index, model, dim, pq_dim, 8)
+    for k in (10, 300):
+        sp = ivf_pq.SearchParams(n_probes=n_probes, lut_dtype=np.float16)
+        d, nb = ivf_pq.search(sp, index, G.to_dev(queries), k)
+        torch.cuda.synchronize()
+        want_nb, want_d = orc.search(ix, queries, k, n_probes, lut_dtype=2)
+        H.compare_results(nb.cpu().numpy(), d.cpu().numpy(), want_nb, want_d, 2e-3, exact=True)
