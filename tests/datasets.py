@@ -230,6 +230,8 @@ def exact_knn(dataset, queries, k, metric="sqeuclidean", row_chunk=1 << 18, half
     if metric == "cosine":
         qf = torch.nn.functional.normalize(qf, dim=1)
     nq = qf.shape[0]
+    # a chunk's score matrix (and the copies topk makes of it) stays within 4 GiB
+    row_chunk = max(4096, min(row_chunk, (1 << 30) // max(nq, 1)))
     best_d = torch.full((nq, k), float("inf"), device=dev)
     best_i = torch.full((nq, k), -1, dtype=torch.int64, device=dev)
     for s in range(0, dataset.shape[0], row_chunk):
