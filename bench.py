@@ -271,9 +271,14 @@ def main():
             "largely from L2 (pairs run in list order), not the metric's code stream")
         default_path["pairs_screened"] = int(stage["n_screened_pairs"])
         default_path["pairs_surviving"] = int(stage["n_surviving_pairs"])
+        default_path["pairs_dropped_on_their_length"] = int(stage["n_far_pairs"])
+        default_path["launches"]["screen"]["note"] += (
+            "; pairs whose |query - centre| minus the list's radius lies past the query's bound are "
+            "dropped without reading a row, and their rows are counted here all the same")
         log("default path, scan stage: " + ", ".join(f"{n_} {ms:.3f} ms / {b / 1e9:.2f} GB"
                                                      for n_, (_, ms, b) in parts.items())
-            + f"; {stage['n_surviving_pairs']} of {stage['n_screened_pairs']} screened pairs kept; "
+            + f"; {stage['n_surviving_pairs']} of {stage['n_screened_pairs']} screened pairs kept "
+            f"({stage['n_far_pairs']} dropped without reading a row); "
             f"all probed lists in full are {scan_bytes / 1e9:.2f} GB")
 
     # The code stream in full: the same batch with the early stop switched off on the handle.  One

@@ -75,7 +75,7 @@ class SearchProfileStruct(C.Structure):
                 ("survivor_scan_ms", C.c_float), ("scan_kernel", C.c_uint32),
                 ("lead_bytes", C.c_uint64), ("screen_bytes", C.c_uint64),
                 ("survivor_bytes", C.c_uint64), ("n_screened_pairs", C.c_uint64),
-                ("n_surviving_pairs", C.c_uint64)]
+                ("n_surviving_pairs", C.c_uint64), ("n_far_pairs", C.c_uint64)]
 
 
 # every symbol include/cuvs/core/c_api.h and include/cuvs/neighbors/ivf_pq.h declare

@@ -197,6 +197,11 @@ struct index_impl {
   /** Position of every list among all lists by size, largest first (ties by list number): the
    *  order in which the search takes the pairs of each query's leading probe, long lists first. */
   device_buffer list_rank;
+  /** Per list, the largest length of a row's decoded residual (rotated space), rounded up: a row
+   *  of list l is at least |query - centre| - list_radius[l] away from a query, which lets an L2
+   *  search drop a (query, list) pair without reading a row.  Kept with the other copies derived
+   *  from the list codes (rebuild_lead_plane / refresh_derived_rows). */
+  device_buffer list_radius;
   std::vector<int64_t> accum_sorted_sizes;  // [n_lists + 1]
   int64_t size = 0;
   mutable screen_feedback feedback;
@@ -385,6 +390,16 @@ struct scan_args {
   int rare_exits;                 // few tiles of this launch are expected to end early (the leading and the
                                   // surviving pairs of an early stop): the wave-per-pair kernel then has a
                                   // tile's next step on its way instead of the next tile's first one
+  // The screens of an L2 search drop a pair without reading a row when every row of the list is
+  // provably too far: a row's sum of entries is, in exact arithmetic, |r - b|^2 >= (|r| - |b|)^2
+  // for the pair's residual r = rotated query - rotated centre and the row's decoded residual b,
+  // and |b| <= list_radius[list].  prune_keep (below 1) and prune_slack cover what the table's
+  // type and the sums' type can lose against exact arithmetic, prune_cap what a sum is sure to
+  // reach once an entry saturates (8-bit tables): the pair goes if
+  // min((|r| - radius)^2 * prune_keep - prune_slack, prune_cap) is past the query's bound.
+  // prune_keep 0: not used.
+  const float* list_radius;       // [n_lists], or null
+  float prune_keep, prune_slack, prune_cap;
 };
 /** LDS bytes the scan kernel needs for these arguments (without the table when `global_lut` is
  *  set), the bytes of one lookup table, and the number of blocks (= table slices) the generic
@@ -422,6 +437,11 @@ void launch_train_codebooks(const float* res, uint32_t rot_dim, uint32_t pq_dim,
 void launch_widen_codes(const uint8_t* packed, uint8_t* wide, uint64_t n_slots, uint32_t pq_dim,
                         uint32_t pq_bits, uint32_t n_chunks, uint32_t n_chunks8, hipStream_t stream);
 void launch_pad_codebooks(const float* src, float* dst, uint64_t n_rows, uint32_t book_size, hipStream_t stream);
+/** radius[l] for the `n` lists from `first_list` on: an upper bound of the length of the decoded
+ *  residual (the codebook entries of a row's codes, side by side) over the list's rows. */
+void launch_list_radius(const uint8_t* const* data_ptrs, const uint32_t* list_sizes, uint32_t first_list,
+                        uint32_t n, uint32_t pq_dim, uint32_t pq_bits, uint32_t pq_len, const float* pq_centers,
+                        bool per_subspace, float* radius, hipStream_t stream);
 void launch_build_lead_plane(const uint8_t* arena, uint64_t* plane, uint64_t n_slots,
                              uint32_t n_chunks, hipStream_t stream);
 constexpr uint64_t kLeadPlaneSlack = 512;  // slots past the last list that look-ahead loads of whole tiles may read
@@ -468,6 +488,7 @@ bool launch_scan_slab(const scan_args& a, hipStream_t stream);
  * work and an iteration two pairs of the same length.
  */
 constexpr uint32_t kSurvivorClasses = 256;
+constexpr uint32_t kFarPairsWord    = 1;  // the screens count the pairs they drop on their length here
 constexpr uint32_t kSurvivorTable   = 64;
 constexpr uint32_t kSurvivorWords   = kSurvivorTable + 64 * kSurvivorClasses;
 void launch_order_survivors(const pair_desc* survivors, uint32_t* n_survivors, pair_desc* ordered,

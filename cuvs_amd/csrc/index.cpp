@@ -218,6 +218,15 @@ void index_impl::rebuild_lead_plane(hipStream_t stream)
       b.allocate(bytes);
     }
   };
+  // how far a row of each list can lie from the list's centre
+  sized(list_radius, sizeof(float) * n_lists);
+  if (n_slots != 0) {
+    launch_list_radius(data_ptrs.as<const uint8_t*>(), list_sizes.as<uint32_t>(), 0, n_lists, pq_dim, pq_bits, pq_len,
+                       pq_centers.as<float>(), codebook_kind == codebook_gen::PER_SUBSPACE, list_radius.as<float>(),
+                       stream);
+  } else {
+    CUVS_HIP_TRY(hipMemsetAsync(list_radius.ptr, 0, list_radius.bytes, stream));
+  }
   // narrower codes, a byte each
   const bool widen = pq_bits >= 5 && pq_bits < 8 && n_slots != 0 && !conservative_memory_allocation;
   if (widen) {
@@ -269,6 +278,9 @@ void index_impl::refresh_derived_rows(uint32_t label, hipStream_t stream)
     return;
   }
   const uint64_t begin = h_row_offsets[label], end = h_row_offsets[label + 1];  // whole groups of 32 rows
+  launch_list_radius(data_ptrs.as<const uint8_t*>(), list_sizes.as<uint32_t>(), label, 1, pq_dim, pq_bits, pq_len,
+                     pq_centers.as<float>(), codebook_kind == codebook_gen::PER_SUBSPACE, list_radius.as<float>(),
+                     stream);
   if (begin == end) { return; }
   const bool widen       = codes8_arena.bytes != 0;
   const uint64_t gb      = uint64_t(n_chunks) * kIndexGroupSize * kIndexGroupVecLen;

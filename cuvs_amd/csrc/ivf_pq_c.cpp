@@ -682,6 +682,7 @@ cuvsError_t cuvsAmdIvfPqGetSearchProfile(cuvsResources_t res, cuvsAmdIvfPqSearch
     profile->survivor_bytes    = p.survivor_bytes;
     profile->n_screened_pairs  = p.n_screened_pairs;
     profile->n_surviving_pairs = p.n_surviving_pairs;
+    profile->n_far_pairs       = p.n_far_pairs;
   });
 }
 

@@ -171,6 +171,45 @@ __global__ __launch_bounds__(kRowBlock) void widen_codes_kernel(const uint8_t* _
     make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+/** One block per list: the largest squared length of a row's decoded residual. */
+__global__ __launch_bounds__(kRowBlock) void list_radius_kernel(
+  const uint8_t* const* __restrict__ data_ptrs, const uint32_t* __restrict__ list_sizes, uint32_t first_list,
+  uint32_t pq_dim, uint32_t pq_bits, uint32_t pq_len, const float* __restrict__ pq_centers, int per_subspace,
+  float* __restrict__ radius)
+{
+  __shared__ float wave_max[kRowBlock / 64];
+  const uint32_t l        = first_list + blockIdx.x;
+  const uint32_t n_rows   = list_sizes[l];
+  const uint8_t* data     = data_ptrs[l];
+  const uint32_t cpc      = 128u / pq_bits;
+  const uint32_t n_chunks = (pq_dim + cpc - 1u) / cpc;
+  const uint32_t book     = 1u << pq_bits;
+  const float* book_base  = pq_centers + (per_subspace ? 0 : uint64_t(l) * pq_len * book);
+  float best              = 0.0f;
+  for (uint32_t i = threadIdx.x; i < n_rows; i += kRowBlock) {
+    const uint8_t* row0 = data + row_base(i, n_chunks);
+    float s             = 0.0f;
+    for (uint32_t j = 0; j < pq_dim; j++) {
+      const uint32_t code = stored_code(row0, j, cpc, pq_bits);
+      const float* cb     = book_base + (per_subspace ? uint64_t(j) * pq_len * book : 0);
+      for (uint32_t t = 0; t < pq_len; t++) {
+        const float v = cb[uint64_t(t) * book + code];
+        s             = fmaf(v, v, s);
+      }
+    }
+    best = fmaxf(best, s);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) { best = fmaxf(best, __shfl_xor(best, off, 64)); }
+  if ((threadIdx.x & 63u) == 0) { wave_max[threadIdx.x >> 6] = best; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (uint32_t w = 1; w < kRowBlock / 64; w++) { best = fmaxf(best, wave_max[w]); }
+    // rounded up past what the fp32 sum of squares and the root can have lost
+    radius[l] = sqrtf(best) * (1.0f + 1e-5f);
+  }
+}
+
 /** dst[row][e] = e < book_size ? src[row][e] : 0 for 256 entries a row. */
 __global__ void pad_codebooks_kernel(const float* __restrict__ src, float* __restrict__ dst, uint64_t n_rows,
                                      uint32_t book_size)
@@ -192,6 +231,16 @@ void launch_widen_codes(const uint8_t* packed, uint8_t* wide, uint64_t n_slots, 
   CUVS_EXPECTS(blocks <= 0x7FFFFFFFull, "too many row slots for one launch");
   widen_codes_kernel<<<uint32_t(blocks), kRowBlock, 0, stream>>>(packed, wide, n_slots, pq_dim, pq_bits, n_chunks,
                                                                 n_chunks8);
+  CUVS_HIP_TRY(hipGetLastError());
+}
+
+void launch_list_radius(const uint8_t* const* data_ptrs, const uint32_t* list_sizes, uint32_t first_list,
+                        uint32_t n, uint32_t pq_dim, uint32_t pq_bits, uint32_t pq_len, const float* pq_centers,
+                        bool per_subspace, float* radius, hipStream_t stream)
+{
+  if (n == 0) { return; }
+  list_radius_kernel<<<n, kRowBlock, 0, stream>>>(data_ptrs, list_sizes, first_list, pq_dim, pq_bits, pq_len,
+                                                  pq_centers, per_subspace ? 1 : 0, radius);
   CUVS_HIP_TRY(hipGetLastError());
 }
 

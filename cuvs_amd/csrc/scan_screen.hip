@@ -452,6 +452,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   auto* pending = reinterpret_cast<LDS_AS uint32_t*>(uintptr_t(off_pending + wid * kSurvivorBatchBytes));
   auto* mini    = reinterpret_cast<LDS_AS lut_t*>(uintptr_t(off_mini + wid * uint32_t(FIRST) * 256u * uint32_t(sizeof(lut_t))));
   uint32_t n_pending = 0;
+  uint32_t n_far     = 0;  // pairs this wave dropped on their length
 
   // A record is fetched two pairs ahead with a vector load (index hidden from the uniformity
   // analysis): a scalar load would be waited for by the tile loop's first LDS read, since both
@@ -481,10 +482,35 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   auto lead_codes = [&](const pair_desc& d, uint32_t tile) {
     return plane[uint64_t(d.row_off) + tile * 64u + lane];
   };
-  // lane d < NDIFF: (rotated query - rotated centre)[d] of a pair
+  // lane d < rot_dim: (rotated query - rotated centre)[d] of a pair (0 in the lanes past rot_dim)
+  const uint32_t rot_dim = a.rot_dim;
   auto fetch_diff = [&](const pair_desc& d) -> float {
-    const uint32_t dim = lane < NDIFF ? lane : 0u;
-    return a.rot_q[uint64_t(d.q) * a.rot_dim + dim] - a.centers_rot[uint64_t(d.label) * a.rot_dim + dim];
+    const uint32_t dim = lane < rot_dim ? lane : 0u;
+    const float df = a.rot_q[uint64_t(d.q) * rot_dim + dim] - a.centers_rot[uint64_t(d.label) * rot_dim + dim];
+    return lane < rot_dim ? df : 0.0f;
+  };
+  // The pair's whole residual, for its length: dimensions 64 + 64 x + lane as well (rot_dim up to
+  // 64 (1 + kFarDims)), and the radius of its list.  A pair whose rows are all provably past the
+  // query's bound is dropped before its first tile.
+  constexpr uint32_t kFarDims = 3;
+  const bool by_length = a.prune_keep > 0.0f && a.list_radius != nullptr && rot_dim <= 64u * (1u + kFarDims);
+  struct far_part {
+    float v[kFarDims];
+    float radius;
+  };
+  auto fetch_far = [&](const pair_desc& d) -> far_part {
+    far_part f{};
+    if (by_length) {
+#pragma unroll
+      for (uint32_t x = 0; x < kFarDims; x++) {
+        const uint32_t dim = 64u * (x + 1u) + lane;
+        const uint32_t at  = dim < rot_dim ? dim : 0u;
+        const float df = a.rot_q[uint64_t(d.q) * rot_dim + at] - a.centers_rot[uint64_t(d.label) * rot_dim + at];
+        f.v[x]         = dim < rot_dim ? df : 0.0f;
+      }
+      f.radius = a.list_radius[d.label];
+    }
+    return f;
   };
 
   // per cluster: entries lane, lane + 64, ... of a pair's list's codebook
@@ -510,6 +536,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   u32x2 next0 = lead_codes(d0, 1u);
   uint32_t thr0  = a.query_kth[d0.q];
   float dv0     = fetch_diff(d0);
+  far_part far0 = fetch_far(d0);
   book_part cb0 = fetch_book(d0);
 
   for (;;) {
@@ -519,16 +546,35 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
     u32x2 next1        = next0;
     uint32_t thr1      = 0u;
     float dv1          = 0.0f;
+    far_part far1      = far0;
     book_part cb1      = cb0;
     if (has1) {
       lead1 = lead_codes(d1, 0u);
       next1 = lead_codes(d1, 1u);
       thr1  = a.query_kth[d1.q];
       dv1  = fetch_diff(d1);
+      far1 = fetch_far(d1);
       cb1  = fetch_book(d1);
     }
 
-    {
+    // every row of the list at least this far from the query, whatever its codes?
+    bool too_far = false;
+    if (by_length) {
+      float part = dv0 * dv0;
+#pragma unroll
+      for (uint32_t x = 0; x < kFarDims; x++) { part = fmaf(far0.v[x], far0.v[x], part); }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) { part += __shfl_xor(part, off, 64); }
+      const uint32_t thr_now = uint32_t(__builtin_amdgcn_readfirstlane(thr0));
+      const float bound      = __uint_as_float(thr_now >= 0x80000000u ? (thr_now & 0x7fffffffu) : 0u);
+      const float gap        = sqrtf(__int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(part)))) -
+                        __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(far0.radius)));
+      // (an unset bound reads as a NaN here: the comparison fails and the pair is screened)
+      too_far = gap > 0.0f && fminf(gap * gap * a.prune_keep - a.prune_slack, a.prune_cap) > bound;
+      n_far += too_far ? 1u : 0u;
+    }
+
+    if (!too_far) {
       if constexpr (PER_CLUSTER) {
         // the pair's codebook into the wave's area (the wave's own LDS accesses are performed in order)
 #pragma unroll
@@ -664,9 +710,11 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
     next0 = next1;
     thr0  = thr1;
     dv0   = dv1;
+    far0  = far1;
     cb0   = cb1;
   }
   if (n_pending != 0) { flush_survivors(pending, n_pending, lane, survivors, n_survivors); }
+  if (n_far != 0 && lane == 0) { atomicAdd(n_survivors + kFarPairsWord, n_far); }
 }
 
 template <int PQ_LEN, int LUT, bool OUT_HALF, int FIRST, int BITS, bool PER_CLUSTER = false>

@@ -468,6 +468,22 @@ void search_one(cuvs::resources const& res_c,
   sa.mean_list_rows = uint32_t(std::min<uint64_t>(uint64_t(ix.size) / std::max<uint32_t>(ix.n_lists, 1u), 0xFFFFFFFFull));
   sa.filter_bits  = filter_bits;
   sa.filter_nbits = filter_nbits;
+  if ((ix.metric == detail::DistanceType::L2Expanded || ix.metric == detail::DistanceType::L2SqrtExpanded) &&
+      ix.list_radius.bytes == sizeof(float) * ix.n_lists) {
+    // what the computed sum of a row's entries can lose against exact arithmetic: the table's
+    // rounding (binary16 to nearest; the unsigned 8-bit type truncates to 3 fraction bits and
+    // flushes entries below 2^-15, and saturates near 1.2e5), then pq_dim additions if the sums
+    // are binary16 (each rounds by at most 2^-11 of a partial sum that only grows)
+    double lose  = params.lut_dtype == CUDA_R_32F ? 1e-5 : (params.lut_dtype == CUDA_R_16F ? 1.0 / 1024 : 0.07);
+    double slack = params.lut_dtype == CUDA_R_8U ? double(ix.pq_dim) / 16384.0 : double(ix.pq_dim) * 1e-7;
+    if (sa.out_half) { lose += double(ix.pq_dim) / 2048.0 + 1.0 / 1024; }
+    if (lose < 0.5) {
+      sa.list_radius = ix.list_radius.as<float>();
+      sa.prune_keep  = float(1.0 - lose);
+      sa.prune_slack = float(slack);
+      sa.prune_cap   = params.lut_dtype == CUDA_R_8U ? 1.0e5f : std::numeric_limits<float>::infinity();
+    }
+  }
   if (ix.pq_bits != 8 && ix.pq_bits != 4) { sa.lead_plane = nullptr; }
   if (ix.wide() && !res.tuning.generic_scan) {
     // 5 - 7 bit codes: the byte-wide copy of the lists, if one of the 8-bit kernels takes the shape
@@ -672,7 +688,7 @@ void search_one(cuvs::resources const& res_c,
     }
     detail::launch_chunk_indices(ix.list_sizes.as<uint32_t>(), probes, nq, P,
                                  ix.n_chunks * kIndexGroupVecLen, chunk, n_samples, d_stats, lead,
-                                 pl.fused ? kth : nullptr, n_survivors, 1, s);
+                                 pl.fused ? kth : nullptr, n_survivors, 2, s);
     detail::launch_order_pairs(probes, chunk, sa.data_ptrs,
                                ix.inds_ptrs.as<const int64_t*>(), ix.ids_arena.as<int64_t>(), nq * P, P,
                                ix.n_lists, counters, sort_scratch, order, desc, lead, alive, few_pairs, list_rank, s);
@@ -810,8 +826,10 @@ void search_one(cuvs::resources const& res_c,
         lp.screen_ms += screen_ms;
         lp.survivor_scan_ms += surv_ms;
         // which pairs survived: their records are still in the workspace
-        uint32_t n_surv = 0;
-        CUVS_HIP_TRY(hipMemcpy(&n_surv, n_survivors, 4, hipMemcpyDeviceToHost));
+        uint32_t counts[2] = {0, 0};  // survivors, pairs dropped on their length
+        CUVS_HIP_TRY(hipMemcpy(counts, n_survivors, 8, hipMemcpyDeviceToHost));
+        const uint32_t n_surv = counts[0];
+        lp.n_far_pairs += counts[1];
         std::vector<detail::pair_desc> h_surv(n_surv);
         if (n_surv != 0) {
           CUVS_HIP_TRY(hipMemcpy(h_surv.data(), survivors, size_t(n_surv) * sizeof(detail::pair_desc),

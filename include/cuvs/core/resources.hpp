@@ -111,6 +111,7 @@ struct search_profile {
   uint64_t survivor_bytes    = 0;
   uint64_t n_screened_pairs  = 0;
   uint64_t n_surviving_pairs = 0;
+  uint64_t n_far_pairs       = 0;  // screened pairs dropped on the length of their residual alone
 };
 
 /** Choices the search otherwise makes by itself, for measurements and tests that compare the

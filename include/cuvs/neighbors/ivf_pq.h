@@ -267,6 +267,8 @@ typedef struct {
   uint64_t survivor_bytes; /* scan_bytes share of the pairs the screen kept */
   uint64_t n_screened_pairs;
   uint64_t n_surviving_pairs;
+  uint64_t n_far_pairs;    /* screened pairs dropped without reading a row: |query - centre| minus the
+                              list's radius already lies past the query's bound */
 } cuvsAmdIvfPqSearchProfile;
 
 /** Choices the search otherwise makes by itself, fixed on one resources handle: for measurements
