@@ -500,7 +500,8 @@ template <typename T>
 __global__ __launch_bounds__(512) void coarse_rescore_kernel(
   const T* __restrict__ queries, const float* __restrict__ centers, uint32_t dim, uint32_t dim_ext,
   float qterm, float alpha, const uint32_t* __restrict__ cand_count, const uint32_t* __restrict__ cand,
-  uint32_t n_probes, uint32_t* __restrict__ probes, uint8_t* __restrict__ fallback)
+  uint32_t n_probes, uint32_t* __restrict__ probes, uint8_t* __restrict__ fallback,
+  float* __restrict__ probe_scores)
 {
   extern __shared__ __align__(16) unsigned char smem[];
   float* qf                 = reinterpret_cast<float*>(smem);  // [dim]
@@ -593,6 +594,7 @@ __global__ __launch_bounds__(512) void coarse_rescore_kernel(
       fallback[q] = 1;  // a NaN score: let the plain path decide what it means
     } else if (rank < n_probes) {
       probes[uint64_t(q) * n_probes + rank] = uint32_t(key);
+      if (probe_scores != nullptr) { probe_scores[uint64_t(q) * n_probes + rank] = unorder_f32(uint32_t(key >> 32)); }
     }
   }
 }
@@ -758,19 +760,19 @@ void launch_coarse_fast(const coarse_fast_args& a, hipStream_t stream)
   }
   switch (a.type) {
     case elem_type::f32:
-      coarse_rescore_kernel<float><<<a.n_queries, rthreads, rsmem, stream>>>(static_cast<const float*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
+      coarse_rescore_kernel<float><<<a.n_queries, rthreads, rsmem, stream>>>(static_cast<const float*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback, a.probe_scores);
       coarse_exact_rows_kernel<float><<<a.n_queries, 256, xsmem, stream>>>(static_cast<const float*>(a.queries), a.centers, a.n_lists, a.dim, a.dim_ext, qterm, alpha, a.fallback, a.scores);
       break;
     case elem_type::f16:
-      coarse_rescore_kernel<_Float16><<<a.n_queries, rthreads, rsmem, stream>>>(static_cast<const _Float16*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
+      coarse_rescore_kernel<_Float16><<<a.n_queries, rthreads, rsmem, stream>>>(static_cast<const _Float16*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback, a.probe_scores);
       coarse_exact_rows_kernel<_Float16><<<a.n_queries, 256, xsmem, stream>>>(static_cast<const _Float16*>(a.queries), a.centers, a.n_lists, a.dim, a.dim_ext, qterm, alpha, a.fallback, a.scores);
       break;
     case elem_type::i8:
-      coarse_rescore_kernel<int8_t><<<a.n_queries, rthreads, rsmem, stream>>>(static_cast<const int8_t*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
+      coarse_rescore_kernel<int8_t><<<a.n_queries, rthreads, rsmem, stream>>>(static_cast<const int8_t*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback, a.probe_scores);
       coarse_exact_rows_kernel<int8_t><<<a.n_queries, 256, xsmem, stream>>>(static_cast<const int8_t*>(a.queries), a.centers, a.n_lists, a.dim, a.dim_ext, qterm, alpha, a.fallback, a.scores);
       break;
     default:
-      coarse_rescore_kernel<uint8_t><<<a.n_queries, rthreads, rsmem, stream>>>(static_cast<const uint8_t*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback);
+      coarse_rescore_kernel<uint8_t><<<a.n_queries, rthreads, rsmem, stream>>>(static_cast<const uint8_t*>(a.queries), a.centers, a.dim, a.dim_ext, qterm, alpha, a.cand_count, a.cand, a.n_probes, a.probes, a.fallback, a.probe_scores);
       coarse_exact_rows_kernel<uint8_t><<<a.n_queries, 256, xsmem, stream>>>(static_cast<const uint8_t*>(a.queries), a.centers, a.n_lists, a.dim, a.dim_ext, qterm, alpha, a.fallback, a.scores);
       break;
   }

@@ -202,6 +202,12 @@ struct index_impl {
    *  search drop a (query, list) pair without reading a row.  Kept with the other copies derived
    *  from the list codes (rebuild_lead_plane / refresh_derived_rows). */
   device_buffer list_radius;
+  /** Per list (float4): the stored squared norm of the centre, |c_rot|^2 and |R^T c_rot - c|: with
+   *  the probe selection's score they give |rotated query - rotated centre| without a pass over the
+   *  dimensions (scan_far.hip).  Made with list_radius.  rotation_bounded: no row of the rotation
+   *  matrix is longer than 2 (the rounding allowance of that estimate assumes it). */
+  device_buffer center_terms;
+  bool rotation_bounded = false;
   std::vector<int64_t> accum_sorted_sizes;  // [n_lists + 1]
   int64_t size = 0;
   mutable screen_feedback feedback;
@@ -298,6 +304,8 @@ struct coarse_fast_args {
   uint8_t* fallback;       // [round_up(n_queries, 4)]
   float* scores;           // [n_queries, n_lists]: rows of flagged queries only
   uint32_t* probes;        // [n_queries, n_probes]
+  float* probe_scores;     // [n_queries, n_probes] out: the probes' fp32 scores (null: not wanted; not
+                           // written for the flagged queries)
 };
 uint32_t coarse_fast_k_pad(uint32_t dim);
 uint32_t coarse_fast_max_dim();
@@ -400,6 +408,7 @@ struct scan_args {
   // prune_keep 0: not used.
   const float* list_radius;       // [n_lists], or null
   float prune_keep, prune_slack, prune_cap;
+  const uint32_t* screen_pairs_dev;  // screens: when non-null the number of records is read from here
 };
 /** LDS bytes the scan kernel needs for these arguments (without the table when `global_lut` is
  *  set), the bytes of one lookup table, and the number of blocks (= table slices) the generic
@@ -488,11 +497,43 @@ bool launch_scan_slab(const scan_args& a, hipStream_t stream);
  * work and an iteration two pairs of the same length.
  */
 constexpr uint32_t kSurvivorClasses = 256;
-constexpr uint32_t kFarPairsWord    = 1;  // the screens count the pairs they drop on their length here
+constexpr uint32_t kFarPairsWord    = 1;  // pairs dropped on their length alone are counted here
+constexpr uint32_t kKeptPairsWord   = 2;  // launch_far_filter(): records it left for the screen
 constexpr uint32_t kSurvivorTable   = 64;
-constexpr uint32_t kSurvivorWords   = kSurvivorTable + 64 * kSurvivorClasses;
+constexpr uint32_t kFarBlocks       = 256;
+constexpr uint32_t kFarTable        = kSurvivorTable + 64 * kSurvivorClasses;  // its table of block counts
+constexpr uint32_t kSurvivorWords   = kFarTable + kFarBlocks;
 void launch_order_survivors(const pair_desc* survivors, uint32_t* n_survivors, pair_desc* ordered,
                             hipStream_t stream);
+
+/**
+ * Before the screen of an L2 search: the records of the pairs whose lists lie, row for row,
+ * provably past their query's bound are left out (scan_far.hip).  `desc` are the screened pairs'
+ * records, `kept` receives the others in the same order and words[kKeptPairsWord] their number;
+ * words[kFarPairsWord] grows by the number left out.  The probe's fp32 coarse score comes from
+ * `probe_scores` (by pair slot), or from the score matrix `score_rows` where that is null or the
+ * query's byte in `from_rows` is set.  keep / slack / cap as scan_args' prune_*; eps_rel: relative
+ * rounding allowance of the squared length.
+ */
+struct far_args {
+  const pair_desc* desc;
+  uint32_t n_pairs;
+  pair_desc* kept;
+  uint32_t* words;
+  const float* probe_scores;
+  const float* score_rows;
+  uint32_t n_lists;
+  const uint8_t* from_rows;
+  const float4* center_terms;  // per list: stored |c|^2, |c_rot|^2, |R^T c_rot - c|
+  const float* list_radius;
+  float4* qterms;              // scratch, n_queries entries
+  float keep, slack, cap, eps_rel;
+};
+void launch_far_filter(const far_args& f, const float* rot_q, const float* qf, uint32_t rot_dim, uint32_t dim,
+                       const uint32_t* query_kth, uint32_t n_queries, hipStream_t stream);
+void launch_center_terms(const float* centers, const float* centers_rot, const float* rotation, uint32_t n_lists,
+                         uint32_t dim, uint32_t dim_ext, uint32_t rot_dim, bool identity, float4* terms,
+                         hipStream_t stream);
 bool scan_screen_supported(const scan_args& a);
 /** Bytes of each row the screen reads (8 or 16). */
 uint32_t scan_screen_bytes_per_row(bool per_cluster, bool lead_plane);

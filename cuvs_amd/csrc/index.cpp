@@ -227,6 +227,9 @@ void index_impl::rebuild_lead_plane(hipStream_t stream)
   } else {
     CUVS_HIP_TRY(hipMemsetAsync(list_radius.ptr, 0, list_radius.bytes, stream));
   }
+  sized(center_terms, sizeof(float4) * n_lists);
+  launch_center_terms(centers.as<float>(), centers_rot.as<float>(), rotation.as<float>(), n_lists, dim, dim_ext,
+                      rot_dim, rotation_is_identity && rot_dim == dim, center_terms.as<float4>(), stream);
   // narrower codes, a byte each
   const bool widen = pq_bits >= 5 && pq_bits < 8 && n_slots != 0 && !conservative_memory_allocation;
   if (widen) {
@@ -384,6 +387,15 @@ index<int64_t> build(cuvs::resources const& res,
     }
   }
   ix.rotation_is_identity = identity;
+  {
+    double longest = 0.0;
+    for (uint32_t r = 0; r < ix.rot_dim; r++) {
+      double n2 = 0.0;
+      for (uint32_t d = 0; d < ix.dim; d++) { n2 += double(rot[size_t(r) * ix.dim + d]) * rot[size_t(r) * ix.dim + d]; }
+      longest = std::max(longest, n2);
+    }
+    ix.rotation_bounded = longest <= 4.0;  // false for a NaN as well
+  }
   ix.rotation_t.allocate(rot_t.size() * sizeof(float));
   CUVS_HIP_TRY(hipMemcpyAsync(ix.rotation_t.ptr, rot_t.data(), rot_t.size() * sizeof(float),
                               hipMemcpyHostToDevice, stream));
@@ -420,6 +432,7 @@ index<int64_t> clone(cuvs::resources const& res, const index<int64_t>& source)
   dst.n_max                          = src.n_max;
   dst.coarse_fast_ok                 = src.coarse_fast_ok;
   dst.rotation_is_identity           = src.rotation_is_identity;
+  dst.rotation_bounded               = src.rotation_bounded;
   dst.feedback.create();
   copy(dst.centers, src.centers);
   copy(dst.centers_rot, src.centers_rot);

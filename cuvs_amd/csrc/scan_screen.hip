@@ -144,6 +144,7 @@ __global__ __launch_bounds__(kScreenThreads, 4) void scan_screen_kernel(
   const uint32_t tid     = threadIdx.x;
   const uint32_t lane    = tid & 63u;
   const uint32_t wid     = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (a.screen_pairs_dev != nullptr) { n_pairs = uint32_t(__builtin_amdgcn_readfirstlane(*a.screen_pairs_dev)); }
   const uint32_t n_iters = (n_pairs + G - 1u) / G;
   const uint32_t stride  = gridDim.x;
   if (blockIdx.x >= n_iters) { return; }
@@ -431,6 +432,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_direct_kernel(
   const uint32_t lane = tid & 63u;
   const uint32_t wid  = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr uint32_t WPB = kDirectThreads / 64u;
+  if (a.screen_pairs_dev != nullptr) { n_pairs = uint32_t(__builtin_amdgcn_readfirstlane(*a.screen_pairs_dev)); }
   const wave_pairs mine  = screen_wave_pairs(n_pairs, wid, WPB);
   const uint32_t total   = mine.stride;
   const uint32_t p_end   = mine.end;

@@ -96,7 +96,7 @@ plan make_plan(const cuvs::resources& res, const search_params& params, const in
   const size_t P = p.n_probes;
   p.per_query_bytes = size_t(ix.dim) * 4 + size_t(ix.dim_ext) * 4 + size_t(ix.n_lists) * 4 +
                       size_t(ix.rot_dim) * 4 +
-                      P * 4 * 3 + P * (2 * sizeof(detail::pair_desc) + 1) + 17 + P * 17 +
+                      P * 4 * 3 + P * (2 * sizeof(detail::pair_desc) + 1) + 17 + P * 17 + P * 4 + 16 +
                       (p.fused ? P * k * 8 * 4 : size_t(p.max_samples) * 4) +
                       (k > detail::kMergeLdsK ? size_t(next_pow2(k)) * 8 : 0) +
                       detail::select_probes_scratch_bytes(1, uint32_t(P));
@@ -174,6 +174,7 @@ struct coarse_buffers {
   uint32_t* cand_count = nullptr;
   uint32_t* cand    = nullptr;
   uint8_t* fallback = nullptr;
+  float* probe_scores = nullptr;  // wanted by the search: the probes' fp32 scores
 };
 
 /** The two-precision probe selection applies to fp32 coarse search and to shapes where its
@@ -244,6 +245,7 @@ void run_coarse(const cuvs::resources& res, const search_params& params, const i
     a.fallback   = b.fallback;
     a.scores     = b.scores;
     a.probes     = b.probes;
+    a.probe_scores = b.probe_scores;
     detail::launch_coarse_fast(a, s);
     return;
   }
@@ -635,6 +637,15 @@ void search_one(cuvs::resources const& res_c,
     merge_redo  = static_cast<uint8_t*>(res.workspace_alloc(size_t(Qb)));
     if (screen_scratch_bytes != 0) { screen_scratch = res.workspace_alloc(screen_scratch_bytes); }
   }
+  // L2: pairs whose lists lie provably past their query's bound are left out before the screen,
+  // from the probe selection's own fp32 scores (scan_far.hip)
+  const bool far_filter = early_stop && sa.prune_keep > 0.0f && params.coarse_search_dtype == CUDA_R_32F &&
+                          ix.rotation_bounded && ix.center_terms.bytes == sizeof(float4) * ix.n_lists;
+  float4* far_qterms = nullptr;
+  if (far_filter) {
+    far_qterms = static_cast<float4*>(res.workspace_alloc(size_t(Qb) * sizeof(float4)));
+    if (fast_coarse) { cb.probe_scores = static_cast<float*>(res.workspace_alloc(size_t(Qb) * P * 4)); }
+  }
   // k beyond what the merge's LDS holds: its selection writes into global memory
   unsigned long long* merge_scratch = nullptr;
   if (k > detail::kMergeLdsK) {
@@ -674,6 +685,7 @@ void search_one(cuvs::resources const& res_c,
     const void* qptr  = static_cast<const char*>(queries) + size_t(q0) * ix.dim * elem_size(type);
 
     cuvs::tracing::range batch_scope("ivf_pq::search-batch(queries: %u - %u)", uint32_t(q0), uint32_t(q0) + nq);
+    detail::pair_desc* screen_out = survivors;  // where the screen's survivors are, as it appended them
     mark(0);
     run_coarse(res, params, ix, qptr, type, nq, P, cb);
     mark(1);
@@ -743,8 +755,35 @@ void search_one(cuvs::resources const& res_c,
       detail::launch_kth_bound(keys, nq, uint64_t(P) * kpp, lead * kpp, k, kth, s);
       mark(5);
       // 2. every other pair on its first chunk only
-      detail::launch_scan_screen(sa, desc + size_t(nq) * lead, nq * (P - lead), survivors, n_survivors,
-                                 alive, screen_scratch, s);
+      detail::pair_desc* screened = desc + size_t(nq) * lead;
+      const uint32_t n_screened   = nq * (P - lead);
+      if (far_filter) {
+        // the pairs worth screening go to the survivors' buffer, the screen's survivors where the
+        // screened pairs' records were, and the ordered survivors back again
+        detail::far_args f{};
+        f.desc         = screened;
+        f.n_pairs      = n_screened;
+        f.kept         = survivors;
+        f.words        = n_survivors;
+        f.probe_scores = cb.probe_scores;
+        f.score_rows   = scores;
+        f.n_lists      = ix.n_lists;
+        f.from_rows    = cb.probe_scores != nullptr ? cb.fallback : nullptr;
+        f.center_terms = ix.center_terms.as<float4>();
+        f.list_radius  = sa.list_radius;
+        f.qterms       = far_qterms;
+        f.keep         = sa.prune_keep;
+        f.slack        = sa.prune_slack;
+        f.cap          = sa.prune_cap;
+        f.eps_rel      = float(ix.dim + ix.rot_dim + 16) * 1.2e-7f;
+        detail::launch_far_filter(f, sa.rot_q, qf, ix.rot_dim, ix.dim, kth, nq, s);
+        sa.screen_pairs_dev = n_survivors + detail::kKeptPairsWord;
+        detail::launch_scan_screen(sa, survivors, n_screened, screened, n_survivors, alive, screen_scratch, s);
+        sa.screen_pairs_dev = nullptr;
+        screen_out          = screened;
+      } else {
+        detail::launch_scan_screen(sa, screened, n_screened, survivors, n_survivors, alive, screen_scratch, s);
+      }
       if (observe_screen) {
         // the survivor count follows the search to the host, for the searches after this one
         observe_screen = false;
@@ -766,8 +805,8 @@ void search_one(cuvs::resources const& res_c,
       mark(6);
       // 3. the pairs still in play, in full, from long lists to short ones (the records of the
       // screened pairs are done with: the ordered ones take their place)
-      detail::pair_desc* ordered = desc + size_t(nq) * lead;
-      detail::launch_order_survivors(survivors, n_survivors, ordered, s);
+      detail::pair_desc* ordered = far_filter ? survivors : screened;
+      detail::launch_order_survivors(screen_out, n_survivors, ordered, s);
       sa.desc        = ordered;
       sa.n_pairs     = 0;
       sa.n_pairs_dev = n_survivors;
@@ -832,7 +871,7 @@ void search_one(cuvs::resources const& res_c,
         lp.n_far_pairs += counts[1];
         std::vector<detail::pair_desc> h_surv(n_surv);
         if (n_surv != 0) {
-          CUVS_HIP_TRY(hipMemcpy(h_surv.data(), survivors, size_t(n_surv) * sizeof(detail::pair_desc),
+          CUVS_HIP_TRY(hipMemcpy(h_surv.data(), screen_out, size_t(n_surv) * sizeof(detail::pair_desc),
                                  hipMemcpyDeviceToHost));
         }
         const uint64_t row_bytes = uint64_t(ix.n_chunks) * kIndexGroupVecLen;
