@@ -122,6 +122,7 @@ struct screen_feedback {
   hipEvent_t landed = nullptr;  // recorded behind the copy into `host`
   bool pending      = false;
   uint64_t pending_pairs  = 0;  // pairs that search screened
+  bool pending_far        = false;  // that search left far pairs out before the screen
   uint32_t pending_probes = 0, pending_k = 0;
   /** Verdicts by (n_probes, k), the most recently used first: callers that alternate between a few
    *  parameter sets each keep theirs. */
@@ -130,6 +131,10 @@ struct screen_feedback {
     bool off                = false;
     uint32_t plain_searches = 0;   // since the verdict
     uint32_t screened_searches = 0;  // with the screen on
+    // the screening kernel alone does not pay: of the pairs that the bound on their lists'
+    // distance leaves over, it kept most (the early stop then runs without it)
+    bool screen_off           = false;
+    uint32_t unscreened_searches = 0;  // since that verdict
   };
   /** With a verdict for the screen, every kObserveEvery-th screened search is observed (the copy of
    *  the survivor count is a launch of its own on the search's stream). */
@@ -500,7 +505,7 @@ constexpr uint32_t kSurvivorClasses = 256;
 constexpr uint32_t kFarPairsWord    = 1;  // pairs dropped on their length alone are counted here
 constexpr uint32_t kKeptPairsWord   = 2;  // launch_far_filter(): records it left for the screen
 constexpr uint32_t kSurvivorTable   = 64;
-constexpr uint32_t kFarBlocks       = 256;
+constexpr uint32_t kFarBlocks       = 1024;
 constexpr uint32_t kFarTable        = kSurvivorTable + 64 * kSurvivorClasses;  // its table of block counts
 constexpr uint32_t kSurvivorWords   = kFarTable + kFarBlocks;
 void launch_order_survivors(const pair_desc* survivors, uint32_t* n_survivors, pair_desc* ordered,
@@ -509,8 +514,9 @@ void launch_order_survivors(const pair_desc* survivors, uint32_t* n_survivors, p
 /**
  * Before the screen of an L2 search: the records of the pairs whose lists lie, row for row,
  * provably past their query's bound are left out (scan_far.hip).  `desc` are the screened pairs'
- * records, `kept` receives the others in the same order and words[kKeptPairsWord] their number;
- * words[kFarPairsWord] grows by the number left out.  The probe's fp32 coarse score comes from
+ * records, `kept` receives the others in the same order and words[count_word] their number;
+ * words[kFarPairsWord] grows by the number left out.  With `alive` non-null the kept pairs' slots
+ * are marked there (the search then takes them for the survivors without a screen).  The probe's fp32 coarse score comes from
  * `probe_scores` (by pair slot), or from the score matrix `score_rows` where that is null or the
  * query's byte in `from_rows` is set.  keep / slack / cap as scan_args' prune_*; eps_rel: relative
  * rounding allowance of the squared length.
@@ -528,6 +534,8 @@ struct far_args {
   const float* list_radius;
   float4* qterms;              // scratch, n_queries entries
   float keep, slack, cap, eps_rel;
+  uint32_t count_word;         // kKeptPairsWord, or 0 when the kept pairs are the survivors
+  uint8_t* alive;              // or null
 };
 void launch_far_filter(const far_args& f, const float* rot_q, const float* qf, uint32_t rot_dim, uint32_t dim,
                        const uint32_t* query_kth, uint32_t n_queries, hipStream_t stream);

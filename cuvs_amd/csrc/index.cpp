@@ -72,9 +72,14 @@ void screen_feedback::collect()
     v->probes = pending_probes;
     v->k      = pending_k;
     v->screened_searches = 0;
+    v->screen_off        = false;
   }
   v->off            = double(host[0]) > kKeepLimit * double(pending_pairs);
   v->plain_searches = 0;
+  // host[1]: pairs dropped on their lists' distance alone; what the screening kernel was given is the rest
+  const double given = double(pending_pairs) - double(host[1]);
+  v->screen_off          = !v->off && pending_far && double(host[0]) > kKeepLimit * given;
+  v->unscreened_searches = 0;
 }
 
 screen_feedback::verdict* screen_feedback::find(uint32_t probes, uint32_t k)

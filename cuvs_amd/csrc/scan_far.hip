@@ -174,7 +174,7 @@ __global__ __launch_bounds__(kFarThreads) void far_move_kernel(far_args f)
   __syncthreads();
   uint32_t base = s_base;
   if (blockIdx.x == 0 && tid == 0) {
-    f.words[kKeptPairsWord] = s_total;
+    f.words[f.count_word] = s_total;
     atomicAdd(f.words + kFarPairsWord, f.n_pairs - s_total);
   }
   const uint32_t per = (f.n_pairs + gridDim.x - 1u) / gridDim.x;
@@ -203,6 +203,7 @@ __global__ __launch_bounds__(kFarThreads) void far_move_kernel(far_args f)
       u32x4* dst = reinterpret_cast<u32x4*>(f.kept + pos);
       dst[0]     = lo;
       dst[1]     = hi;
+      if (f.alive != nullptr) { f.alive[lo.w] = 1; }  // by slot
     }
     base += all;
     __syncthreads();  // the counts are read before the next round writes them

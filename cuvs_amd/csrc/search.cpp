@@ -591,6 +591,11 @@ void search_one(cuvs::resources const& res_c,
                     detail::scan_screen_supported(sa) && res.tuning.early_stop != 1;
   // In the automatic mode the index remembers whether the screen pays on its data: where it kept
   // most pairs the last time it ran with these parameters, this search scans plainly.
+  // L2: pairs whose lists lie provably past their query's bound are left out before the screen,
+  // from the probe selection's own fp32 scores (scan_far.hip)
+  const bool far_possible = sa.prune_keep > 0.0f && params.coarse_search_dtype == CUDA_R_32F &&
+                            ix.rotation_bounded && ix.center_terms.bytes == sizeof(float4) * ix.n_lists;
+  bool skip_screen    = false;  // what that leaves over is scanned in full without a screening launch
   bool observe_screen = false;
   if (early_stop && res.tuning.early_stop == 0 && ix.feedback.host != nullptr) {
     auto& fb = ix.feedback;
@@ -615,8 +620,13 @@ void search_one(cuvs::resources const& res_c,
       verdict->plain_searches += 1;
       if (verdict->plain_searches % detail::screen_feedback::kScreenRecheck != 0) { early_stop = false; }
     }
-    observe_screen = early_stop && capture == hipStreamCaptureStatusNone;
-    if (observe_screen && verdict != nullptr && !verdict->off) {
+    if (early_stop && far_possible && verdict != nullptr && !verdict->off && verdict->screen_off) {
+      // the screening kernel kept most of what it was given the last time: every 64th search tries it again
+      verdict->unscreened_searches += 1;
+      skip_screen = verdict->unscreened_searches % detail::screen_feedback::kScreenRecheck != 0;
+    }
+    observe_screen = early_stop && !skip_screen && capture == hipStreamCaptureStatusNone;
+    if (observe_screen && verdict != nullptr && !verdict->off && !verdict->screen_off) {
       // (a search that tries the screen again after a verdict against it is always observed)
       observe_screen = verdict->screened_searches % detail::screen_feedback::kObserveEvery == 0;
       verdict->screened_searches += 1;
@@ -637,11 +647,8 @@ void search_one(cuvs::resources const& res_c,
     merge_redo  = static_cast<uint8_t*>(res.workspace_alloc(size_t(Qb)));
     if (screen_scratch_bytes != 0) { screen_scratch = res.workspace_alloc(screen_scratch_bytes); }
   }
-  // L2: pairs whose lists lie provably past their query's bound are left out before the screen,
-  // from the probe selection's own fp32 scores (scan_far.hip)
-  const bool far_filter = early_stop && sa.prune_keep > 0.0f && params.coarse_search_dtype == CUDA_R_32F &&
-                          ix.rotation_bounded && ix.center_terms.bytes == sizeof(float4) * ix.n_lists;
-  float4* far_qterms = nullptr;
+  const bool far_filter = early_stop && far_possible;
+  float4* far_qterms    = nullptr;
   if (far_filter) {
     far_qterms = static_cast<float4*>(res.workspace_alloc(size_t(Qb) * sizeof(float4)));
     if (fast_coarse) { cb.probe_scores = static_cast<float*>(res.workspace_alloc(size_t(Qb) * P * 4)); }
@@ -776,11 +783,19 @@ void search_one(cuvs::resources const& res_c,
         f.slack        = sa.prune_slack;
         f.cap          = sa.prune_cap;
         f.eps_rel      = float(ix.dim + ix.rot_dim + 16) * 1.2e-7f;
+        f.count_word   = skip_screen ? 0u : detail::kKeptPairsWord;
+        f.alive        = skip_screen ? alive : nullptr;
         detail::launch_far_filter(f, sa.rot_q, qf, ix.rot_dim, ix.dim, kth, nq, s);
-        sa.screen_pairs_dev = n_survivors + detail::kKeptPairsWord;
-        detail::launch_scan_screen(sa, survivors, n_screened, screened, n_survivors, alive, screen_scratch, s);
-        sa.screen_pairs_dev = nullptr;
-        screen_out          = screened;
+        if (!skip_screen) {
+          // (the screening kernels' own look at a pair's length would repeat the same test)
+          const float keep    = sa.prune_keep;
+          sa.prune_keep       = 0.0f;
+          sa.screen_pairs_dev = n_survivors + detail::kKeptPairsWord;
+          detail::launch_scan_screen(sa, survivors, n_screened, screened, n_survivors, alive, screen_scratch, s);
+          sa.screen_pairs_dev = nullptr;
+          sa.prune_keep       = keep;
+          screen_out          = screened;
+        }
       } else {
         detail::launch_scan_screen(sa, screened, n_screened, survivors, n_survivors, alive, screen_scratch, s);
       }
@@ -794,7 +809,8 @@ void search_one(cuvs::resources const& res_c,
         fb.collect();
         CUVS_HIP_TRY(hipThreadExchangeStreamCaptureMode(&mode));
         if (!fb.pending) {
-          CUVS_HIP_TRY(hipMemcpyAsync(fb.host, n_survivors, 4, hipMemcpyDeviceToHost, s));
+          CUVS_HIP_TRY(hipMemcpyAsync(fb.host, n_survivors, 8, hipMemcpyDeviceToHost, s));
+          fb.pending_far    = far_filter;
           CUVS_HIP_TRY(hipEventRecord(fb.landed, s));
           fb.pending        = true;
           fb.pending_pairs  = uint64_t(nq) * (P - lead);
@@ -805,7 +821,7 @@ void search_one(cuvs::resources const& res_c,
       mark(6);
       // 3. the pairs still in play, in full, from long lists to short ones (the records of the
       // screened pairs are done with: the ordered ones take their place)
-      detail::pair_desc* ordered = far_filter ? survivors : screened;
+      detail::pair_desc* ordered = screen_out == survivors ? screened : survivors;
       detail::launch_order_survivors(screen_out, n_survivors, ordered, s);
       sa.desc        = ordered;
       sa.n_pairs     = 0;
