@@ -272,6 +272,9 @@ def main():
         default_path["pairs_screened"] = int(stage["n_screened_pairs"])
         default_path["pairs_surviving"] = int(stage["n_surviving_pairs"])
         default_path["pairs_dropped_on_their_length"] = int(stage["n_far_pairs"])
+        if stage["n_far_pairs"]:
+            # the bytes are those of every screened pair; most were never read
+            default_path["launches"]["screen"]["rate_on_those_bytes_GBs"] = None
         default_path["launches"]["screen"]["note"] += (
             "; pairs whose |query - centre| minus the list's radius lies past the query's bound are "
             "dropped without reading a row, and their rows are counted here all the same")
