@@ -123,6 +123,8 @@ __device__ __forceinline__ bool pair_is_far(const far_args& f, uint32_t q, uint3
 }
 
 constexpr uint32_t kFarThreads = 256;
+constexpr uint32_t kFarAhead   = 4;  // records a thread has in flight: every one is a chain of dependent loads
+constexpr uint32_t kFarRound   = kFarThreads * kFarAhead;
 
 /** Kept pairs of every block's contiguous run of records. */
 __global__ __launch_bounds__(kFarThreads) void far_count_kernel(far_args f)
@@ -133,9 +135,21 @@ __global__ __launch_bounds__(kFarThreads) void far_count_kernel(far_args f)
   const uint32_t i0  = blockIdx.x * per;
   const uint32_t i1  = i0 + per < f.n_pairs ? i0 + per : f.n_pairs;
   uint32_t kept      = 0;
-  for (uint32_t i = i0 + tid; i < i1; i += kFarThreads) {
-    const pair_desc* d = f.desc + i;
-    kept += pair_is_far(f, d->q, d->slot, d->label) ? 0u : 1u;
+  for (uint32_t s = i0; s < i1; s += kFarRound) {
+    uint32_t q[kFarAhead], slot[kFarAhead], label[kFarAhead];
+#pragma unroll
+    for (uint32_t u = 0; u < kFarAhead; u++) {
+      const uint32_t i   = s + u * kFarThreads + tid;
+      const pair_desc* d = f.desc + (i < i1 ? i : i1 - 1u);
+      q[u]               = d->q;
+      slot[u]            = d->slot;
+      label[u]           = d->label;
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < kFarAhead; u++) {
+      const bool far = pair_is_far(f, q[u], slot[u], label[u]);
+      kept += (s + u * kFarThreads + tid < i1 && !far) ? 1u : 0u;
+    }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) { kept += __shfl_xor(kept, off, 64); }
@@ -150,7 +164,7 @@ __global__ __launch_bounds__(kFarThreads) void far_count_kernel(far_args f)
 /** The kept records, in their order, behind those of the blocks before. */
 __global__ __launch_bounds__(kFarThreads) void far_move_kernel(far_args f)
 {
-  __shared__ uint32_t wave_counts[kFarThreads / 64];
+  __shared__ uint32_t wave_counts[kFarAhead][kFarThreads / 64];
   __shared__ uint32_t s_base, s_total;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wid = tid >> 6;
   if (wid == 0) {
@@ -180,32 +194,46 @@ __global__ __launch_bounds__(kFarThreads) void far_move_kernel(far_args f)
   const uint32_t per = (f.n_pairs + gridDim.x - 1u) / gridDim.x;
   const uint32_t i0  = blockIdx.x * per;
   const uint32_t i1  = i0 + per < f.n_pairs ? i0 + per : f.n_pairs;
-  for (uint32_t s = i0; s < i1; s += kFarThreads) {  // uniform trip count
-    const uint32_t i = s + tid;
-    u32x4 lo{}, hi{};
-    bool keep = false;
-    if (i < i1) {
-      const u32x4* src = reinterpret_cast<const u32x4*>(f.desc + i);
-      lo               = src[0];
-      hi               = src[1];
-      keep             = !pair_is_far(f, lo.z, lo.w, hi.x);  // q, slot, label
+  for (uint32_t s = i0; s < i1; s += kFarRound) {  // uniform trip count
+    u32x4 lo[kFarAhead], hi[kFarAhead];
+    bool keep[kFarAhead];
+#pragma unroll
+    for (uint32_t u = 0; u < kFarAhead; u++) {
+      const uint32_t i = s + u * kFarThreads + tid;
+      const u32x4* src = reinterpret_cast<const u32x4*>(f.desc + (i < i1 ? i : i1 - 1u));
+      lo[u]            = src[0];
+      hi[u]            = src[1];
     }
-    const unsigned long long votes = __builtin_amdgcn_ballot_w64(keep);
-    if (lane == 0) { wave_counts[wid] = uint32_t(__popcll(votes)); }
+#pragma unroll
+    for (uint32_t u = 0; u < kFarAhead; u++) {
+      const bool far = pair_is_far(f, lo[u].z, lo[u].w, hi[u].x);  // q, slot, label
+      keep[u]        = s + u * kFarThreads + tid < i1 && !far;
+    }
+    unsigned long long votes[kFarAhead];
+#pragma unroll
+    for (uint32_t u = 0; u < kFarAhead; u++) {
+      votes[u] = __builtin_amdgcn_ballot_w64(keep[u]);
+      if (lane == 0) { wave_counts[u][wid] = uint32_t(__popcll(votes[u])); }
+    }
     __syncthreads();
-    uint32_t pos = base + uint32_t(__popcll(votes & ((1ull << lane) - 1ull)));
-    uint32_t all = 0;
-    for (uint32_t w = 0; w < kFarThreads / 64; w++) {
-      pos += w < wid ? wave_counts[w] : 0u;
-      all += wave_counts[w];
+    // records in index order: part u of the round, then wave, then lane
+    uint32_t before = 0;
+#pragma unroll
+    for (uint32_t u = 0; u < kFarAhead; u++) {
+      uint32_t pos = base + before + uint32_t(__popcll(votes[u] & ((1ull << lane) - 1ull)));
+#pragma unroll
+      for (uint32_t w = 0; w < kFarThreads / 64; w++) {
+        pos += w < wid ? wave_counts[u][w] : 0u;
+        before += wave_counts[u][w];
+      }
+      if (keep[u]) {
+        u32x4* dst = reinterpret_cast<u32x4*>(f.kept + pos);
+        dst[0]     = lo[u];
+        dst[1]     = hi[u];
+        if (f.alive != nullptr) { f.alive[lo[u].w] = 1; }  // by slot
+      }
     }
-    if (keep) {
-      u32x4* dst = reinterpret_cast<u32x4*>(f.kept + pos);
-      dst[0]     = lo;
-      dst[1]     = hi;
-      if (f.alive != nullptr) { f.alive[lo.w] = 1; }  // by slot
-    }
-    base += all;
+    base += before;
     __syncthreads();  // the counts are read before the next round writes them
   }
 }
