@@ -519,7 +519,7 @@ void launch_order_survivors(const pair_desc* survivors, uint32_t* n_survivors, p
  * are marked there (the search then takes them for the survivors without a screen).  The probe's fp32 coarse score comes from
  * `probe_scores` (by pair slot), or from the score matrix `score_rows` where that is null or the
  * query's byte in `from_rows` is set.  keep / slack / cap as scan_args' prune_*; eps_rel: relative
- * rounding allowance of the squared length.
+ * rounding allowance of the squared length (L2) or of the score (inner product).
  */
 struct far_args {
   const pair_desc* desc;
@@ -534,6 +534,8 @@ struct far_args {
   const float* list_radius;
   float4* qterms;              // scratch, n_queries entries
   float keep, slack, cap, eps_rel;
+  int ip;                      // inner product: the bound is score - |q| e - |R q| radius, less `tol` of
+  float tol;                   // the entries' summed magnitudes (what the table and the sums may lose)
   uint32_t count_word;         // kKeptPairsWord, or 0 when the kept pairs are the survivors
   uint8_t* alive;              // or null
 };

@@ -15,6 +15,11 @@
  * minus a rounding allowance, from two numbers per query, four per list and the probe's score.
  * The screened pairs whose bound lies past their query's k-th best so far are left out of the
  * record list the screening kernel walks; the others keep their order (the lists' order).
+ *
+ * Inner product: a row's score is -(R q) . c_rot - (R q) . b, at least
+ * -(R q) . c_rot - |R q| radius, and -(R q) . c_rot is the probe selection's score (-q . c) up to
+ * |q| e.  What the computed sum can lose against that is relative to the magnitudes of the table's
+ * entries, whose sum over the subspaces is at most |R q| (|c_rot| + radius).
  */
 #include "device_utils.cuh"
 
@@ -76,7 +81,7 @@ __global__ __launch_bounds__(kTermThreads) void center_terms_kernel(
 __global__ __launch_bounds__(256) void far_query_terms_kernel(const float* __restrict__ rot_q,
                                                               const float* __restrict__ qf, uint32_t rot_dim,
                                                               uint32_t dim, const uint32_t* __restrict__ query_kth,
-                                                              uint32_t n_queries, float4* __restrict__ qterms)
+                                                              uint32_t n_queries, int ip, float4* __restrict__ qterms)
 {
   const uint32_t q    = blockIdx.x * 4u + (threadIdx.x >> 6);
   const uint32_t lane = threadIdx.x & 63u;
@@ -97,9 +102,10 @@ __global__ __launch_bounds__(256) void far_query_terms_kernel(const float* __res
   }
   if (lane == 0) {
     const uint32_t thr = query_kth[q];
-    // ordered score words: non-negative numbers have the top bit set; no bound yet reads as a NaN
-    const float bound = __uint_as_float(thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u);
-    qterms[q]         = make_float4(a, sqrtf(n) * (1.0f + 1e-5f), bound, 0.0f);
+    // ordered score words: non-negative numbers have the top bit set; no bound yet reads as a NaN.
+    // (L2 scores are not negative: a word below that range bounds them at zero, as in the scans.)
+    const float bound = ip ? unorder_f32(thr) : __uint_as_float(thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u);
+    qterms[q]         = make_float4(a, sqrtf(n) * (1.0f + 1e-5f), bound, sqrtf(a) * (1.0f + 1e-5f));
   }
 }
 
@@ -113,6 +119,14 @@ __device__ __forceinline__ bool pair_is_far(const far_args& f, uint32_t q, uint3
     score = f.probe_scores[slot];
   } else {
     score = f.score_rows[uint64_t(q) * f.n_lists + label];
+  }
+  if (f.ip) {
+    const float radius = f.list_radius[label];
+    const float c_len  = sqrtf(ct.y) * (1.0f + 1e-6f);
+    const float mag    = qt.w * (c_len + radius);  // the entries' magnitudes, summed, at most
+    const float lb     = score - qt.y * ct.z - qt.w * radius - f.eps_rel * (fabsf(score) + qt.y * (c_len + ct.z)) -
+                     f.tol * mag;
+    return mag < 6.0e4f && lb > qt.z;  // (a NaN anywhere fails the comparison)
   }
   const float two_dot = ct.x - score;  // 2 q . c
   const float mass    = qt.x + ct.y + fabsf(ct.x) + fabsf(score) + qt.y * qt.y;
@@ -257,7 +271,7 @@ void launch_far_filter(const far_args& f, const float* rot_q, const float* qf, u
                 "record layout");
   if (n_queries == 0) { return; }
   far_query_terms_kernel<<<(n_queries + 3u) / 4u, 256, 0, stream>>>(rot_q, qf, rot_dim, dim, query_kth, n_queries,
-                                                                     f.qterms);
+                                                                     f.ip, f.qterms);
   CUVS_HIP_TRY(hipGetLastError());
   uint32_t grid = (f.n_pairs + 4u * kFarThreads - 1u) / (4u * kFarThreads);
   grid          = grid < 1u ? 1u : (grid > kFarBlocks ? kFarBlocks : grid);

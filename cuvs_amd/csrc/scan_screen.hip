@@ -936,6 +936,7 @@ __global__ __launch_bounds__(kDirectThreads, 2) void scan_screen_ip_kernel(
   const uint32_t lane = tid & 63u;
   const uint32_t wid  = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr uint32_t WPB = kDirectThreads / 64u;
+  if (a.screen_pairs_dev != nullptr) { n_pairs = uint32_t(__builtin_amdgcn_readfirstlane(*a.screen_pairs_dev)); }
   const wave_pairs mine  = screen_wave_pairs(n_pairs, wid, WPB);
   if (mine.first - wid >= mine.end) { return; }  // the whole block, before its barrier
   for (uint32_t e = tid; e < SUB * BOOK; e += kDirectThreads) {

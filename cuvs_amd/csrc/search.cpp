@@ -593,7 +593,14 @@ void search_one(cuvs::resources const& res_c,
   // most pairs the last time it ran with these parameters, this search scans plainly.
   // L2: pairs whose lists lie provably past their query's bound are left out before the screen,
   // from the probe selection's own fp32 scores (scan_far.hip)
-  const bool far_possible = sa.prune_keep > 0.0f && params.coarse_search_dtype == CUDA_R_32F &&
+  // (inner product: the same from the score itself; what the computed sum may lose is then relative
+  // to the entries' magnitudes: the table's rounding (the signed 8-bit type keeps two fraction
+  // bits), fp32 additions, and pq_dim binary16 additions where the sums are binary16)
+  double ip_tol = params.lut_dtype == CUDA_R_32F ? 2e-5 : (params.lut_dtype == CUDA_R_16F ? 1.0 / 1024 + 2e-5 : 0.3);
+  if (sa.out_half) { ip_tol += double(ix.pq_dim) / 2048.0 + 1.0 / 1024; }
+  const bool far_ip = ix.metric == detail::DistanceType::InnerProduct && ip_tol < 0.5 &&
+                      ix.list_radius.bytes == sizeof(float) * ix.n_lists;
+  const bool far_possible = (sa.prune_keep > 0.0f || far_ip) && params.coarse_search_dtype == CUDA_R_32F &&
                             ix.rotation_bounded && ix.center_terms.bytes == sizeof(float4) * ix.n_lists;
   bool skip_screen    = false;  // what that leaves over is scanned in full without a screening launch
   bool observe_screen = false;
@@ -777,7 +784,9 @@ void search_one(cuvs::resources const& res_c,
         f.n_lists      = ix.n_lists;
         f.from_rows    = cb.probe_scores != nullptr ? cb.fallback : nullptr;
         f.center_terms = ix.center_terms.as<float4>();
-        f.list_radius  = sa.list_radius;
+        f.list_radius  = ix.list_radius.as<float>();
+        f.ip           = far_ip ? 1 : 0;
+        f.tol          = float(ip_tol);
         f.qterms       = far_qterms;
         f.keep         = sa.prune_keep;
         f.slack        = sa.prune_slack;

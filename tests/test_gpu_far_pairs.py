@@ -6,6 +6,9 @@ table and sum type, with a random rotation (padded dimensions included), per-clu
 4-bit codes, and with model tensors that do not belong together (rotated centres that are not the
 rotation of the centres, a rotation that is not orthonormal), where the bound has to notice.
 On well separated clusters most pairs must go that way.
+
+Inner-product searches drop pairs on the same two numbers (a row's score is at least the probe
+selection's score minus |query| times the list's radius); the tests run both metrics.
 """
 import numpy as np
 import pytest
@@ -29,7 +32,7 @@ def _rows(n, dim, dtype, seed, sigma=0.05):
     return x.astype(dtype)
 
 
-def _search_all_ways(orc, index, ix, q, k, n_probes, lut, internal, expect_far):
+def _search_all_ways(orc, index, ix, q, k, n_probes, lut, internal, expect_far, some_far=False):
     want_nb, want_d = orc.search(ix, q, k, n_probes, lut_dtype=ORC_DT[lut], internal_distance_dtype=ORC_DT[internal])
     res = Resources()
     res.enable_profiling(True)
@@ -46,20 +49,28 @@ def _search_all_ways(orc, index, ix, q, k, n_probes, lut, internal, expect_far):
     assert far["off"] == 0
     if expect_far:
         assert far["on"] > 0.5 * q.shape[0] * (n_probes - 1), f"only {far['on']} pairs dropped on their lists' distance"
+    if some_far:
+        assert far["on"] > 0
     return far
 
 
 @pytest.mark.parametrize("lut,internal", [(np.float32, np.float32), (np.float16, np.float32), (np.uint8, np.float32),
                                           (np.float16, np.float16), (np.uint8, np.float16)])
 @pytest.mark.parametrize("dtype", [np.float32, np.uint8])
-def test_far_pairs_are_dropped_and_results_stay_exact(orc, lut, internal, dtype):
+@pytest.mark.parametrize("metric", ["sqeuclidean", "inner_product"])
+def test_far_pairs_are_dropped_and_results_stay_exact(orc, lut, internal, dtype, metric):
     n, dim, n_lists, pq_dim = 40000, 64, 192, 32
     allrows = _rows(n + 300, dim, dtype, 7)
     x, q = allrows[:n], allrows[n:]
-    model = H.train(x, n_lists, pq_dim, 8, iters=4)
-    index = G.build_gpu_index(model, x, pq_dim, 8)
-    ix, _ = G.read_back(orc, index, model, dim, pq_dim, 8)
-    _search_all_ways(orc, index, ix, q, 10, 32, lut, internal, expect_far=True)
+    model = H.train(x, n_lists, pq_dim, 8, metric=metric, iters=4)
+    index = G.build_gpu_index(model, x, pq_dim, 8, metric)
+    ix, _ = G.read_back(orc, index, model, dim, pq_dim, 8, metric)
+    l2 = metric == "sqeuclidean"
+    # (inner product with an 8-bit table or binary16 sums: the allowance for their rounding eats most of the bound)
+    far = _search_all_ways(orc, index, ix, q, 10, 32, lut, internal, expect_far=l2,
+                           some_far=not l2 and lut != np.uint8 and internal == np.float32)
+    print(f"{metric} {np.dtype(dtype).name} {np.dtype(lut).name} {np.dtype(internal).name}: {far} of {q.shape[0] * 31}",
+          flush=True)
 
 
 @pytest.mark.parametrize("dim,pq_dim,pq_bits,kind,rotate", [
@@ -83,7 +94,8 @@ def test_far_pairs_with_other_index_shapes(orc, dim, pq_dim, pq_bits, kind, rota
 
 @pytest.mark.parametrize("tamper", ["centers_rot_shifted", "centers_rot_unrelated", "rotation_scaled",
                                     "rotation_long_rows", "norm_column_wrong"])
-def test_model_tensors_that_do_not_belong_together(orc, tamper):
+@pytest.mark.parametrize("metric", ["sqeuclidean", "inner_product"])
+def test_model_tensors_that_do_not_belong_together(orc, tamper, metric):
     """`build(res, params, dim, pq_centers, centers, centers_rot, rotation_matrix)` takes the four
     tensors as they come.  The probe selection uses `centers`, the scan `centers_rot` and the rotated
     query: a bound that took one for the other would drop rows the scan keeps."""
@@ -91,7 +103,7 @@ def test_model_tensors_that_do_not_belong_together(orc, tamper):
     rng = np.random.default_rng(5)
     allrows = _rows(n + 200, dim, np.float32, 13)
     x, q = allrows[:n], allrows[n:]
-    model = H.train(x, n_lists, pq_dim, 8, iters=3, force_random_rotation=True)
+    model = H.train(x, n_lists, pq_dim, 8, metric=metric, iters=3, force_random_rotation=True)
     model = {name: np.array(v, copy=True) for name, v in model.items()}
     if tamper == "centers_rot_shifted":
         model["centers_rot"] += 0.3 * rng.standard_normal(model["centers_rot"].shape).astype(np.float32)
@@ -103,10 +115,10 @@ def test_model_tensors_that_do_not_belong_together(orc, tamper):
         model["rotation_matrix"] *= np.float32(3.0)
     elif tamper == "norm_column_wrong":
         model["centers"][:, dim] *= np.float32(0.5)
-    index = G.build_gpu_index(model, x, pq_dim, 8)
-    ix, _ = G.read_back(orc, index, model, dim, pq_dim, 8)
+    index = G.build_gpu_index(model, x, pq_dim, 8, metric)
+    ix, _ = G.read_back(orc, index, model, dim, pq_dim, 8, metric)
     far = _search_all_ways(orc, index, ix, q, 10, 32, np.float16, np.float32, expect_far=False)
-    print(f"{tamper}: pairs dropped on their lists' distance {far} of {q.shape[0] * 31} screened", flush=True)
+    print(f"{metric} {tamper}: pairs dropped on their lists' distance {far} of {q.shape[0] * 31} screened", flush=True)
 
 
 def test_far_pairs_follow_an_edit_of_a_list(orc):
