@@ -534,13 +534,14 @@ struct far_args {
   const float* list_radius;
   float4* qterms;              // scratch, n_queries entries
   float keep, slack, cap, eps_rel;
-  int ip;                      // inner product: the bound is score - |q| e - |R q| radius, less `tol` of
+  int ip;                      // 1 inner product, 2 cosine: the bound is score - |q| e - |R q| radius, less `tol` of
   float tol;                   // the entries' summed magnitudes (what the table and the sums may lose)
   uint32_t count_word;         // kKeptPairsWord, or 0 when the kept pairs are the survivors
   uint8_t* alive;              // or null
 };
 void launch_far_filter(const far_args& f, const float* rot_q, const float* qf, uint32_t rot_dim, uint32_t dim,
-                       const uint32_t* query_kth, uint32_t n_queries, hipStream_t stream);
+                       const uint32_t* query_kth, uint32_t n_queries, const float* rotation_t, bool identity,
+                       hipStream_t stream);
 void launch_center_terms(const float* centers, const float* centers_rot, const float* rotation, uint32_t n_lists,
                          uint32_t dim, uint32_t dim_ext, uint32_t rot_dim, bool identity, float4* terms,
                          hipStream_t stream);

@@ -19,7 +19,9 @@
  * Inner product: a row's score is -(R q) . c_rot - (R q) . b, at least
  * -(R q) . c_rot - |R q| radius, and -(R q) . c_rot is the probe selection's score (-q . c) up to
  * |q| e.  What the computed sum can lose against that is relative to the magnitudes of the table's
- * entries, whose sum over the subspaces is at most |R q| (|c_rot| + radius).
+ * entries, whose sum over the subspaces is at most |R q| (|c_rot| + radius).  Cosine: the scan's
+ * query is R q / |R q|, so the probe selection's score (of the query as it came) is divided by
+ * |R q| first, and the scans add 1 to a row's sum.
  */
 #include "device_utils.cuh"
 
@@ -77,11 +79,14 @@ __global__ __launch_bounds__(kTermThreads) void center_terms_kernel(
   }
 }
 
-/** One wave per query: |rot_q|^2, |q| (rounded up) and the query's bound as a number. */
+/** One wave per query: |rot_q|^2 (inner product: 1; cosine: 1 / |R q|, what the scan's query was
+ *  divided by), |q| (rounded up), the query's bound as a number, |rot_q| (rounded up). */
 __global__ __launch_bounds__(256) void far_query_terms_kernel(const float* __restrict__ rot_q,
                                                               const float* __restrict__ qf, uint32_t rot_dim,
                                                               uint32_t dim, const uint32_t* __restrict__ query_kth,
-                                                              uint32_t n_queries, int ip, float4* __restrict__ qterms)
+                                                              uint32_t n_queries, int ip,
+                                                              const float* __restrict__ rotation_t, int identity,
+                                                              float4* __restrict__ qterms)
 {
   const uint32_t q    = blockIdx.x * 4u + (threadIdx.x >> 6);
   const uint32_t lane = threadIdx.x & 63u;
@@ -95,17 +100,36 @@ __global__ __launch_bounds__(256) void far_query_terms_kernel(const float* __res
     const float v = qf[uint64_t(q) * dim + d];
     n             = fmaf(v, v, n);
   }
+  float rq = 0.0f;  // cosine: |R q|^2 of the query before it was normalised
+  if (ip == 2 && !identity) {
+    for (uint32_t k = lane; k < rot_dim; k += 64u) {
+      float y = 0.0f;
+      for (uint32_t d = 0; d < dim; d++) { y = fmaf(rotation_t[uint64_t(d) * rot_dim + k], qf[uint64_t(q) * dim + d], y); }
+      rq = fmaf(y, y, rq);
+    }
+  }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     a += __shfl_xor(a, off, 64);
     n += __shfl_xor(n, off, 64);
+    rq += __shfl_xor(rq, off, 64);
   }
   if (lane == 0) {
+    if (ip == 1) { a = 1.0f; }
+    if (ip == 2) { a = 1.0f / sqrtf(identity ? n : rq); }
     const uint32_t thr = query_kth[q];
     // ordered score words: non-negative numbers have the top bit set; no bound yet reads as a NaN.
     // (L2 scores are not negative: a word below that range bounds them at zero, as in the scans.)
     const float bound = ip ? unorder_f32(thr) : __uint_as_float(thr >= 0x80000000u ? (thr & 0x7fffffffu) : 0u);
-    qterms[q]         = make_float4(a, sqrtf(n) * (1.0f + 1e-5f), bound, sqrtf(a) * (1.0f + 1e-5f));
+    float len = 0.0f;  // |rot_q|
+    if (ip != 0) {
+      float l2 = 0.0f;
+      for (uint32_t k = 0; k < rot_dim; k++) { l2 = fmaf(rot_q[uint64_t(q) * rot_dim + k], rot_q[uint64_t(q) * rot_dim + k], l2); }
+      len = sqrtf(l2);
+    } else {
+      len = sqrtf(a);
+    }
+    qterms[q] = make_float4(a, sqrtf(n) * (1.0f + 1e-5f), bound, len * (1.0f + 1e-5f));
   }
 }
 
@@ -124,9 +148,12 @@ __device__ __forceinline__ bool pair_is_far(const far_args& f, uint32_t q, uint3
     const float radius = f.list_radius[label];
     const float c_len  = sqrtf(ct.y) * (1.0f + 1e-6f);
     const float mag    = qt.w * (c_len + radius);  // the entries' magnitudes, summed, at most
-    const float lb     = score - qt.y * ct.z - qt.w * radius - f.eps_rel * (fabsf(score) + qt.y * (c_len + ct.z)) -
-                     f.tol * mag;
-    return mag < 6.0e4f && lb > qt.z;  // (a NaN anywhere fails the comparison)
+    const float sc     = qt.x;                      // 1, or 1 / |R q| (cosine)
+    const float lb     = score * sc - qt.y * ct.z * sc - qt.w * radius -
+                     (f.eps_rel + 2e-5f) * sc * (fabsf(score) + qt.y * (c_len + ct.z)) - f.tol * mag;
+    // cosine: the scans add 1 to a row's sum, in the sums' type (`slack` covers that addition)
+    const float lbv = f.ip == 2 ? 1.0f + lb - f.slack : lb;
+    return mag < 6.0e4f && lbv > qt.z;  // (a NaN anywhere fails the comparison)
   }
   const float two_dot = ct.x - score;  // 2 q . c
   const float mass    = qt.x + ct.y + fabsf(ct.x) + fabsf(score) + qt.y * qt.y;
@@ -265,13 +292,14 @@ void launch_center_terms(const float* centers, const float* centers_rot, const f
 }
 
 void launch_far_filter(const far_args& f, const float* rot_q, const float* qf, uint32_t rot_dim, uint32_t dim,
-                       const uint32_t* query_kth, uint32_t n_queries, hipStream_t stream)
+                       const uint32_t* query_kth, uint32_t n_queries, const float* rotation_t, bool identity,
+                       hipStream_t stream)
 {
   static_assert(offsetof(pair_desc, q) == 8 && offsetof(pair_desc, slot) == 12 && offsetof(pair_desc, label) == 16,
                 "record layout");
   if (n_queries == 0) { return; }
   far_query_terms_kernel<<<(n_queries + 3u) / 4u, 256, 0, stream>>>(rot_q, qf, rot_dim, dim, query_kth, n_queries,
-                                                                     f.ip, f.qterms);
+                                                                     f.ip, rotation_t, identity ? 1 : 0, f.qterms);
   CUVS_HIP_TRY(hipGetLastError());
   uint32_t grid = (f.n_pairs + 4u * kFarThreads - 1u) / (4u * kFarThreads);
   grid          = grid < 1u ? 1u : (grid > kFarBlocks ? kFarBlocks : grid);

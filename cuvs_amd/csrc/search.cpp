@@ -596,9 +596,10 @@ void search_one(cuvs::resources const& res_c,
   // (inner product: the same from the score itself; what the computed sum may lose is then relative
   // to the entries' magnitudes: the table's rounding (the signed 8-bit type keeps two fraction
   // bits), fp32 additions, and pq_dim binary16 additions where the sums are binary16)
+  const bool cosine_metric = ix.metric == detail::DistanceType::CosineExpanded;
   double ip_tol = params.lut_dtype == CUDA_R_32F ? 2e-5 : (params.lut_dtype == CUDA_R_16F ? 1.0 / 1024 + 2e-5 : 0.3);
   if (sa.out_half) { ip_tol += double(ix.pq_dim) / 2048.0 + 1.0 / 1024; }
-  const bool far_ip = ix.metric == detail::DistanceType::InnerProduct && ip_tol < 0.5 &&
+  const bool far_ip = (ix.metric == detail::DistanceType::InnerProduct || cosine_metric) && ip_tol < 0.5 &&
                       ix.list_radius.bytes == sizeof(float) * ix.n_lists;
   const bool far_possible = (sa.prune_keep > 0.0f || far_ip) && params.coarse_search_dtype == CUDA_R_32F &&
                             ix.rotation_bounded && ix.center_terms.bytes == sizeof(float4) * ix.n_lists;
@@ -785,16 +786,17 @@ void search_one(cuvs::resources const& res_c,
         f.from_rows    = cb.probe_scores != nullptr ? cb.fallback : nullptr;
         f.center_terms = ix.center_terms.as<float4>();
         f.list_radius  = ix.list_radius.as<float>();
-        f.ip           = far_ip ? 1 : 0;
+        f.ip           = far_ip ? (cosine_metric ? 2 : 1) : 0;
         f.tol          = float(ip_tol);
         f.qterms       = far_qterms;
         f.keep         = sa.prune_keep;
-        f.slack        = sa.prune_slack;
+        f.slack        = cosine_metric ? (sa.out_half ? 2e-3f : 2e-6f) : sa.prune_slack;
         f.cap          = sa.prune_cap;
         f.eps_rel      = float(ix.dim + ix.rot_dim + 16) * 1.2e-7f;
         f.count_word   = skip_screen ? 0u : detail::kKeptPairsWord;
         f.alive        = skip_screen ? alive : nullptr;
-        detail::launch_far_filter(f, sa.rot_q, qf, ix.rot_dim, ix.dim, kth, nq, s);
+        detail::launch_far_filter(f, sa.rot_q, qf, ix.rot_dim, ix.dim, kth, nq, ix.rotation_t.as<float>(),
+                                  ix.rotation_is_identity && ix.rot_dim == ix.dim, s);
         if (!skip_screen) {
           // (the screening kernels' own look at a pair's length would repeat the same test)
           const float keep    = sa.prune_keep;

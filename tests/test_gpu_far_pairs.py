@@ -7,8 +7,9 @@ table and sum type, with a random rotation (padded dimensions included), per-clu
 rotation of the centres, a rotation that is not orthonormal), where the bound has to notice.
 On well separated clusters most pairs must go that way.
 
-Inner-product searches drop pairs on the same two numbers (a row's score is at least the probe
-selection's score minus |query| times the list's radius); the tests run both metrics.
+Inner-product and cosine searches drop pairs on the same two numbers (a row's score is at least the
+probe selection's score minus |query| times the list's radius; cosine divides the score by the
+length of the rotated query first); the tests run all three metrics.
 """
 import numpy as np
 import pytest
@@ -57,7 +58,7 @@ def _search_all_ways(orc, index, ix, q, k, n_probes, lut, internal, expect_far, 
 @pytest.mark.parametrize("lut,internal", [(np.float32, np.float32), (np.float16, np.float32), (np.uint8, np.float32),
                                           (np.float16, np.float16), (np.uint8, np.float16)])
 @pytest.mark.parametrize("dtype", [np.float32, np.uint8])
-@pytest.mark.parametrize("metric", ["sqeuclidean", "inner_product"])
+@pytest.mark.parametrize("metric", ["sqeuclidean", "inner_product", "cosine"])
 def test_far_pairs_are_dropped_and_results_stay_exact(orc, lut, internal, dtype, metric):
     n, dim, n_lists, pq_dim = 40000, 64, 192, 32
     allrows = _rows(n + 300, dim, dtype, 7)
@@ -94,7 +95,7 @@ def test_far_pairs_with_other_index_shapes(orc, dim, pq_dim, pq_bits, kind, rota
 
 @pytest.mark.parametrize("tamper", ["centers_rot_shifted", "centers_rot_unrelated", "rotation_scaled",
                                     "rotation_long_rows", "norm_column_wrong"])
-@pytest.mark.parametrize("metric", ["sqeuclidean", "inner_product"])
+@pytest.mark.parametrize("metric", ["sqeuclidean", "inner_product", "cosine"])
 def test_model_tensors_that_do_not_belong_together(orc, tamper, metric):
     """`build(res, params, dim, pq_centers, centers, centers_rot, rotation_matrix)` takes the four
     tensors as they come.  The probe selection uses `centers`, the scan `centers_rot` and the rotated
