@@ -275,6 +275,9 @@ def main():
         if stage["n_far_pairs"]:
             # the bytes are those of every screened pair; most were never read
             default_path["launches"]["screen"]["rate_on_those_bytes_GBs"] = None
+            default_path["launches"]["screen"]["kernel"] = (
+                "far_query_terms_kernel, far_count_kernel, far_move_kernel; then " + screen_name +
+                " over the pairs they leave, unless the index has found that it keeps most of them")
         default_path["launches"]["screen"]["note"] += (
             "; pairs whose |query - centre| minus the list's radius lies past the query's bound are "
             "dropped without reading a row, and their rows are counted here all the same")
