@@ -538,6 +538,8 @@ struct far_args {
   float tol;                   // the entries' summed magnitudes (what the table and the sums may lose)
   uint32_t count_word;         // kKeptPairsWord, or 0 when the kept pairs are the survivors
   uint8_t* alive;              // or null
+  int unordered;               // the kept records' order does not matter and words[count_word] is zero:
+                               // one pass, the blocks claim their records' places as they come
 };
 void launch_far_filter(const far_args& f, const float* rot_q, const float* qf, uint32_t rot_dim, uint32_t dim,
                        const uint32_t* query_kth, uint32_t n_queries, const float* rotation_t, bool identity,

@@ -138,9 +138,12 @@ __device__ __forceinline__ bool pair_is_far(const far_args& f, uint32_t q, uint3
 {
   const float4 qt = f.qterms[q];
   const float4 ct = f.center_terms[label];
+  // (the score by slot and the query's flag are requested together: the flag is rarely set)
   float score;
-  if (f.probe_scores != nullptr && (f.from_rows == nullptr || f.from_rows[q] == 0)) {
-    score = f.probe_scores[slot];
+  if (f.probe_scores != nullptr) {
+    const uint8_t rows = f.from_rows != nullptr ? f.from_rows[q] : uint8_t(0);
+    score              = f.probe_scores[slot];
+    if (rows != 0) { score = f.score_rows[uint64_t(q) * f.n_lists + label]; }
   } else {
     score = f.score_rows[uint64_t(q) * f.n_lists + label];
   }
@@ -202,13 +205,17 @@ __global__ __launch_bounds__(kFarThreads) void far_count_kernel(far_args f)
   }
 }
 
-/** The kept records, in their order, behind those of the blocks before. */
+/** The kept records, in their order, behind those of the blocks before.  CLAIM: no counting pass
+ *  went before; a block claims the places of every round's kept records with one atomic add on the
+ *  count (zero before the launch), so the blocks' runs follow each other in no particular order
+ *  (for a list that is put in order of length next anyway). */
+template <bool CLAIM>
 __global__ __launch_bounds__(kFarThreads) void far_move_kernel(far_args f)
 {
   __shared__ uint32_t wave_counts[kFarAhead][kFarThreads / 64];
   __shared__ uint32_t s_base, s_total;
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wid = tid >> 6;
-  if (wid == 0) {
+  if (!CLAIM && wid == 0) {
     // blocks before this one, and all of them (the grid has at most kFarBlocks blocks)
     uint32_t before = 0, total = 0;
     for (uint32_t b = lane; b < gridDim.x; b += 64u) {
@@ -227,8 +234,8 @@ __global__ __launch_bounds__(kFarThreads) void far_move_kernel(far_args f)
     }
   }
   __syncthreads();
-  uint32_t base = s_base;
-  if (blockIdx.x == 0 && tid == 0) {
+  uint32_t base = CLAIM ? 0u : s_base;
+  if (!CLAIM && blockIdx.x == 0 && tid == 0) {
     f.words[f.count_word] = s_total;
     atomicAdd(f.words + kFarPairsWord, f.n_pairs - s_total);
   }
@@ -257,6 +264,21 @@ __global__ __launch_bounds__(kFarThreads) void far_move_kernel(far_args f)
       if (lane == 0) { wave_counts[u][wid] = uint32_t(__popcll(votes[u])); }
     }
     __syncthreads();
+    if constexpr (CLAIM) {
+      if (tid == 0) {
+        uint32_t all = 0;
+#pragma unroll
+        for (uint32_t u = 0; u < kFarAhead; u++) {
+#pragma unroll
+          for (uint32_t w = 0; w < kFarThreads / 64; w++) { all += wave_counts[u][w]; }
+        }
+        const uint32_t in_round = (i1 - s < kFarRound ? i1 - s : kFarRound);
+        s_base = atomicAdd(f.words + f.count_word, all);
+        if (in_round != all) { atomicAdd(f.words + kFarPairsWord, in_round - all); }
+      }
+      __syncthreads();
+      base = s_base;
+    }
     // records in index order: part u of the round, then wave, then lane
     uint32_t before = 0;
 #pragma unroll
@@ -303,9 +325,14 @@ void launch_far_filter(const far_args& f, const float* rot_q, const float* qf, u
   CUVS_HIP_TRY(hipGetLastError());
   uint32_t grid = (f.n_pairs + 4u * kFarThreads - 1u) / (4u * kFarThreads);
   grid          = grid < 1u ? 1u : (grid > kFarBlocks ? kFarBlocks : grid);
+  if (f.unordered) {
+    far_move_kernel<true><<<grid, kFarThreads, 0, stream>>>(f);
+    CUVS_HIP_TRY(hipGetLastError());
+    return;
+  }
   far_count_kernel<<<grid, kFarThreads, 0, stream>>>(f);
   CUVS_HIP_TRY(hipGetLastError());
-  far_move_kernel<<<grid, kFarThreads, 0, stream>>>(f);
+  far_move_kernel<false><<<grid, kFarThreads, 0, stream>>>(f);
   CUVS_HIP_TRY(hipGetLastError());
 }
 

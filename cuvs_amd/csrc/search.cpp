@@ -795,6 +795,7 @@ void search_one(cuvs::resources const& res_c,
         f.eps_rel      = float(ix.dim + ix.rot_dim + 16) * 1.2e-7f;
         f.count_word   = skip_screen ? 0u : detail::kKeptPairsWord;
         f.alive        = skip_screen ? alive : nullptr;
+        f.unordered    = skip_screen ? 1 : 0;  // (the survivors are put in order of length next)
         detail::launch_far_filter(f, sa.rot_q, qf, ix.rot_dim, ix.dim, kth, nq, ix.rotation_t.as<float>(),
                                   ix.rotation_is_identity && ix.rot_dim == ix.dim, s);
         if (!skip_screen) {
