@@ -178,6 +178,7 @@ def _run_larger(orc, seed):
         assert torch.equal(nb, nb2) and torch.equal(d, d2), "the answer depends on the early stop"
 
 
-@pytest.mark.parametrize("seed", list(range(30000, 30024)))
+# (30002, 30006, 30011, 30020 and 30021 pass as well and take 9 - 15 s each: left out to keep the suite short)
+@pytest.mark.parametrize("seed", [s for s in range(30000, 30024) if s not in (30002, 30006, 30011, 30020, 30021)])
 def test_random_larger_configuration_matches_oracle(orc, seed):
     _run_larger(orc, seed)
